@@ -1,0 +1,73 @@
+"""ctypes binding of libcandle_hip_quant.so (the C ABI declared in include/candle_hip_quant.h).
+
+The library must be built first (``python -m candle_amd.build`` or ``__graft_entry__.build()``);
+loading fails loudly when it is missing — there is no CPU or PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcandle_hip_quant.so")
+
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_vp = ctypes.c_void_p
+
+# name -> (restype, argtypes); mirrors include/candle_hip_quant.h one to one
+SIGNATURES = {
+    "cq_status_string": (ctypes.c_char_p, [_int]),
+    "cq_block_size": (_i64, [_int]),
+    "cq_type_size": (_i64, [_int]),
+    "cq_storage_bytes": (_i64, [_int, _i64]),
+    "cq_dequantize": (_int, [_int, _vp, _vp, _i64, _int, _vp]),
+    "cq_quantize": (_int, [_int, _vp, _vp, _i64, _vp]),
+    "cq_act_scratch_bytes": (_i64, [_int, _i64, _i64]),
+    "cq_quantize_act": (_int, [_int, _vp, _int, _vp, _i64, _i64, _vp]),
+    "cq_matvec": (_int, [_int, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
+    "cq_matmul": (_int, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "cq_qmatmul_workspace_bytes": (_i64, [_int, _i64, _i64, _i64]),
+    "cq_qmatmul_forward": (_int, [_int, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "cq_indexed_moe_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _i64]),
+    "cq_indexed_moe_forward": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "cq_moe_gemm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _int]),
+    "cq_moe_gemm_gguf": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
+}
+
+_lib = None
+
+
+class CqError(RuntimeError):
+    """A C-ABI entry point returned a non-zero status."""
+
+    def __init__(self, fn: str, status: int, text: str):
+        super().__init__(f"{fn} failed: {text} (status {status})")
+        self.fn = fn
+        self.status = status
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build the HIP extension first (python -m candle_amd.build). "
+                "There is no fallback path."
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def status_string(status: int) -> str:
+    return lib().cq_status_string(status).decode()
+
+
+def check(fn: str, status: int) -> None:
+    if status != 0:
+        raise CqError(fn, status, status_string(status))

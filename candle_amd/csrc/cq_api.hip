@@ -1,0 +1,241 @@
+// extern "C" boundary of the library: argument validation and dispatch to the kernel launchers.
+// Declarations and the reference interfaces they replace are in include/candle_hip_quant.h.
+#include "cq_device.h"
+#include "cq_launch.h"
+
+namespace {
+
+inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+inline bool matmul_weight_dtype(int dt) {
+    return dt == CQ_Q4_0 || dt == CQ_Q8_0 || dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K;
+}
+
+inline bool block_dtype(int dt) { return matmul_weight_dtype(dt) || dt == CQ_Q8K; }
+
+inline bool float_dtype(int dt) { return dt == CQ_F32 || dt == CQ_F16 || dt == CQ_BF16; }
+
+inline int64_t float_size(int dt) { return dt == CQ_F32 ? 4 : 2; }
+
+// shared checks of the (w_dtype, k, n, rows) tuple of the matmul-family entry points
+inline int check_mm_shape(int w_dtype, int64_t k, int64_t n, int64_t rows) {
+    if (!matmul_weight_dtype(w_dtype)) return CQ_ERR_DTYPE;
+    if (k <= 0 || n < 0 || rows < 0) return CQ_ERR_SHAPE;
+    if (k % cq_block_size(w_dtype) != 0) return CQ_ERR_SHAPE;
+    if (k > (1 << 24) || n > 0x7fffffffLL || rows > 0x7fffffffLL) return CQ_ERR_RANGE;
+    return CQ_OK;
+}
+
+inline int check_weight_ptr(int w_dtype, const void *w) {
+    if (!w) return CQ_ERR_NULL;
+    if (!aligned(w, (w_dtype == CQ_Q4K || w_dtype == CQ_Q5K) ? 16 : 2)) return CQ_ERR_ALIGN;
+    return CQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *cq_status_string(int status) {
+    switch (status) {
+        case CQ_OK: return "ok";
+        case CQ_ERR_DTYPE: return "dtype not supported by this entry point";
+        case CQ_ERR_SHAPE: return "invalid shape (k must be a positive multiple of the block size, sizes must be non-negative)";
+        case CQ_ERR_ALIGN: return "pointer alignment requirement not met";
+        case CQ_ERR_NULL: return "required pointer is NULL";
+        case CQ_ERR_WORKSPACE: return "workspace too small";
+        case CQ_ERR_RANGE: return "size exceeds what this entry point supports";
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "unknown status";
+}
+
+int64_t cq_block_size(int dtype) {
+    switch (dtype) {
+        case CQ_F32: case CQ_F16: case CQ_BF16: return 1;
+        case CQ_Q4_0: case CQ_Q4_1: case CQ_Q5_0: case CQ_Q5_1: case CQ_Q8_0: case CQ_Q8_1: return 32;
+        case CQ_Q2K: case CQ_Q3K: case CQ_Q4K: case CQ_Q5K: case CQ_Q6K: case CQ_Q8K: return 256;
+    }
+    return 0;
+}
+
+int64_t cq_type_size(int dtype) {
+    switch (dtype) {
+        case CQ_F32: return 4;
+        case CQ_F16: case CQ_BF16: return 2;
+        case CQ_Q4_0: return 18;
+        case CQ_Q4_1: return 20;
+        case CQ_Q5_0: return 22;
+        case CQ_Q5_1: return 24;
+        case CQ_Q8_0: return 34;
+        case CQ_Q8_1: return 36;
+        case CQ_Q2K: return 84;
+        case CQ_Q3K: return 110;
+        case CQ_Q4K: return 144;
+        case CQ_Q5K: return 176;
+        case CQ_Q6K: return 210;
+        case CQ_Q8K: return 292;
+    }
+    return 0;
+}
+
+int64_t cq_storage_bytes(int dtype, int64_t elem_count) {
+    int64_t bs = cq_block_size(dtype);
+    if (bs == 0 || elem_count < 0 || elem_count % bs != 0) return -1;
+    return elem_count / bs * cq_type_size(dtype);
+}
+
+int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem_count, int out_dtype, void *stream) {
+    if (!block_dtype(dtype)) return CQ_ERR_DTYPE;
+    if (out_dtype != CQ_F32 && out_dtype != CQ_F16) return CQ_ERR_DTYPE;
+    if (elem_count < 0 || elem_count % cq_block_size(dtype) != 0) return CQ_ERR_SHAPE;
+    if (elem_count == 0) return CQ_OK;
+    if (!blocks_dev || !out_dev) return CQ_ERR_NULL;
+    if (!aligned(blocks_dev, 2) || !aligned(out_dev, 16)) return CQ_ERR_ALIGN;
+    return cq_dequantize_launch(dtype, blocks_dev, out_dev, elem_count, out_dtype, (hipStream_t)stream);
+}
+
+int cq_quantize(int dtype, const float *x_dev, void *blocks_dev, int64_t elem_count, void *stream) {
+    if (!block_dtype(dtype)) return CQ_ERR_DTYPE;
+    if (elem_count < 0 || elem_count % cq_block_size(dtype) != 0) return CQ_ERR_SHAPE;
+    if (elem_count == 0) return CQ_OK;
+    if (!x_dev || !blocks_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 4) || !aligned(blocks_dev, 2)) return CQ_ERR_ALIGN;
+    return cq_quantize_launch(dtype, x_dev, blocks_dev, elem_count, (hipStream_t)stream);
+}
+
+int64_t cq_act_scratch_bytes(int w_dtype, int64_t k, int64_t rows) {
+    if (!block_dtype(w_dtype) || k <= 0 || rows < 0 || k % cq_block_size(w_dtype) != 0) return -1;
+    return cq_act_layout(w_dtype, k, rows).total;
+}
+
+int cq_quantize_act(int w_dtype, const void *x_dev, int x_dtype, void *scratch_dev, int64_t k, int64_t rows, void *stream) {
+    if (!block_dtype(w_dtype) || !float_dtype(x_dtype)) return CQ_ERR_DTYPE;
+    if (k <= 0 || rows < 0 || k % cq_block_size(w_dtype) != 0) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    if (!x_dev || !scratch_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(scratch_dev, 256)) return CQ_ERR_ALIGN;
+    return cq_quantize_act_launch(w_dtype, x_dev, x_dtype, scratch_dev, k, rows, (hipStream_t)stream);
+}
+
+int cq_matvec(int w_dtype, const void *w_dev, const void *act_scratch_dev, void *dst_dev, int dst_dtype,
+              int64_t k, int64_t n, int64_t rows, int64_t stride_dst, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, rows);
+    if (rc) return rc;
+    if (!float_dtype(dst_dtype)) return CQ_ERR_DTYPE;
+    if (rows > CQ_MATVEC_MAX_ROWS) return CQ_ERR_RANGE;
+    if (stride_dst < n) return CQ_ERR_SHAPE;
+    if (n == 0 || rows == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!act_scratch_dev || !dst_dev) return CQ_ERR_NULL;
+    if (!aligned(act_scratch_dev, 256) || !aligned(dst_dev, float_size(dst_dtype))) return CQ_ERR_ALIGN;
+    return cq_matvec_launch(w_dtype, w_dev, act_scratch_dev, dst_dev, dst_dtype, k, n, rows, stride_dst, (hipStream_t)stream);
+}
+
+int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float *dst_dev,
+              int64_t k, int64_t n, int64_t rows, int64_t stride_dst, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, rows);
+    if (rc) return rc;
+    if (stride_dst < n) return CQ_ERR_SHAPE;
+    if (n == 0 || rows == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!act_scratch_dev || !dst_dev) return CQ_ERR_NULL;
+    if (!aligned(act_scratch_dev, 256) || !aligned(dst_dev, 4)) return CQ_ERR_ALIGN;
+    return cq_matmul_launch(w_dtype, w_dev, act_scratch_dev, dst_dev, k, n, rows, stride_dst, (hipStream_t)stream);
+}
+
+int64_t cq_qmatmul_workspace_bytes(int w_dtype, int64_t m, int64_t k, int64_t n) {
+    if (check_mm_shape(w_dtype, k, n, m)) return -1;
+    int64_t bytes = cq_act_layout(w_dtype, k, m).total;
+    // the MFMA path writes f32 and converts afterwards when the caller wants f16 / bf16
+    if (m > CQ_MATVEC_MAX_ROWS) bytes += cq_align256(m * n * 4);
+    return bytes;
+}
+
+int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_dtype, void *dst_dev, int dst_dtype,
+                       int64_t m, int64_t k, int64_t n, void *workspace_dev, int64_t workspace_bytes, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, m);
+    if (rc) return rc;
+    if (!float_dtype(x_dtype) || !float_dtype(dst_dtype)) return CQ_ERR_DTYPE;
+    if (m == 0 || n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!x_dev || !dst_dev || !workspace_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(workspace_dev, 256) || !aligned(dst_dev, float_size(dst_dtype))) return CQ_ERR_ALIGN;
+    if (workspace_bytes < cq_qmatmul_workspace_bytes(w_dtype, m, k, n)) return CQ_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
+    if (m <= CQ_MATVEC_MAX_ROWS)
+        return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, dst_dtype, k, n, m, n, s);
+    if (dst_dtype == CQ_F32)
+        return cq_matmul_launch(w_dtype, w_dev, workspace_dev, (float *)dst_dev, k, n, m, n, s);
+    float *tmp = (float *)((uint8_t *)workspace_dev + cq_act_layout(w_dtype, k, m).total);
+    if ((rc = cq_matmul_launch(w_dtype, w_dev, workspace_dev, tmp, k, n, m, n, s))) return rc;
+    return cq_convert_f32_launch(tmp, dst_dev, dst_dtype, m * n, s);
+}
+
+int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk,
+                                       int64_t input_dim1) {
+    if (check_mm_shape(w_dtype, k, n, batch) || num_experts <= 0 || topk <= 0) return -1;
+    if (input_dim1 != 1 && input_dim1 != topk) return -1;
+    return cq_moe_workspace_bytes_impl(w_dtype, num_experts, batch * topk, batch * input_dim1, k);
+}
+
+int cq_indexed_moe_forward(int w_dtype, const void *w_dev, const float *x_dev, const uint32_t *ids_dev, float *out_dev,
+                           int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk, int64_t input_dim1,
+                           void *workspace_dev, int64_t workspace_bytes, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, batch);
+    if (rc) return rc;
+    if (num_experts <= 0 || topk <= 0) return CQ_ERR_SHAPE;
+    if (input_dim1 != 1 && input_dim1 != topk) return CQ_ERR_SHAPE;
+    if (num_experts > (1 << 20) || batch * topk > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (batch == 0 || n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!x_dev || !ids_dev || !out_dev || !workspace_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(ids_dev, 4) || !aligned(out_dev, 4) || !aligned(workspace_dev, 256)) return CQ_ERR_ALIGN;
+    if (workspace_bytes < cq_indexed_moe_workspace_bytes(w_dtype, num_experts, n, k, batch, topk, input_dim1)) return CQ_ERR_WORKSPACE;
+    MoeArgs a;
+    a.w_dtype = w_dtype; a.w = w_dev; a.x = x_dev; a.out = out_dev;
+    a.num_experts = num_experts; a.n = n; a.k = k;
+    a.n_pairs = batch * topk; a.x_rows = batch * input_dim1;
+    a.mode = MOE_INDEXED; a.ids_u32 = ids_dev; a.topk = topk; a.input_dim1 = input_dim1;
+    a.sorted_token_ids = nullptr; a.expert_ids = nullptr; a.topk_weights = nullptr;
+    a.prefill = 0;
+    return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
+}
+
+int64_t cq_moe_gemm_workspace_bytes(int w_dtype, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k,
+                                    int has_topk_weights) {
+    if (check_mm_shape(w_dtype, k, n, size_m) || num_experts <= 0 || topk <= 0) return -1;
+    if (!has_topk_weights && size_m % topk != 0) return -1;
+    int64_t x_rows = has_topk_weights ? size_m : size_m / topk;
+    return cq_moe_workspace_bytes_impl(w_dtype, num_experts, size_m, x_rows, k);
+}
+
+int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const int32_t *sorted_token_ids_dev,
+                     const int32_t *expert_ids_dev, const float *topk_weights_dev, float *out_dev,
+                     int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int is_prefill,
+                     void *workspace_dev, int64_t workspace_bytes, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, size_m);
+    if (rc) return rc;
+    if (num_experts <= 0 || topk <= 0) return CQ_ERR_SHAPE;
+    if (!topk_weights_dev && size_m % topk != 0) return CQ_ERR_SHAPE;
+    if (num_experts > (1 << 20)) return CQ_ERR_RANGE;
+    if (size_m == 0 || n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!x_dev || !sorted_token_ids_dev || !expert_ids_dev || !out_dev || !workspace_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(sorted_token_ids_dev, 4) || !aligned(expert_ids_dev, 4) || !aligned(out_dev, 4) ||
+        !aligned(workspace_dev, 256) || (topk_weights_dev && !aligned(topk_weights_dev, 4)))
+        return CQ_ERR_ALIGN;
+    if (workspace_bytes < cq_moe_gemm_workspace_bytes(w_dtype, num_experts, topk, size_m, n, k, topk_weights_dev != nullptr))
+        return CQ_ERR_WORKSPACE;
+    MoeArgs a;
+    a.w_dtype = w_dtype; a.w = w_dev; a.x = x_dev; a.out = out_dev;
+    a.num_experts = num_experts; a.n = n; a.k = k;
+    a.n_pairs = size_m; a.x_rows = topk_weights_dev ? size_m : size_m / topk;
+    a.mode = MOE_SORTED; a.ids_u32 = nullptr; a.topk = topk; a.input_dim1 = 0;
+    a.sorted_token_ids = sorted_token_ids_dev; a.expert_ids = expert_ids_dev; a.topk_weights = topk_weights_dev;
+    a.prefill = is_prefill;
+    return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,100 @@
+// Shared device-side definitions for the gfx950 GGUF quantized-matmul kernels:
+// block geometry, unaligned vector loads, f16 helpers, wave64 reductions and the layout of the
+// quantized-activation scratch buffer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#include "../../include/candle_hip_quant.h"
+
+#define CQ_QK_K 256
+#define CQ_WAVE 64
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// GGUF block sizes in bytes (candle-core/src/quantized/k_quants.rs:77-190).
+template <int DT> struct BlockInfo;
+template <> struct BlockInfo<CQ_Q4_0> { static constexpr int elems = 32, bytes = 18; };
+template <> struct BlockInfo<CQ_Q8_0> { static constexpr int elems = 32, bytes = 34; };
+template <> struct BlockInfo<CQ_Q4K> { static constexpr int elems = 256, bytes = 144; };
+template <> struct BlockInfo<CQ_Q5K> { static constexpr int elems = 256, bytes = 176; };
+template <> struct BlockInfo<CQ_Q6K> { static constexpr int elems = 256, bytes = 210; };
+template <> struct BlockInfo<CQ_Q8K> { static constexpr int elems = 256, bytes = 292; };
+
+__host__ __device__ inline bool cq_is_kquant(int dt) { return dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q8K; }
+__host__ __device__ inline bool cq_is_q0(int dt) { return dt == CQ_Q4_0 || dt == CQ_Q8_0; }
+
+// Global loads from addresses that are only 2-byte aligned (Q6_K, Q8_0 and Q4_0 blocks): gfx950
+// serves these with one global_load_dword[x2|x4].
+template <typename T> __device__ __forceinline__ T ld_u(const void *p) {
+    struct __attribute__((packed, aligned(2))) W { T v; };
+    return reinterpret_cast<const W *>(p)->v;
+}
+template <typename T> __device__ __forceinline__ void st_u(void *p, T v) {
+    struct __attribute__((packed, aligned(2))) W { T v; };
+    reinterpret_cast<W *>(p)->v = v;
+}
+
+// f16 bit pattern -> f32 (exact, subnormals included).
+__device__ __forceinline__ float h2f(uint32_t bits16) {
+    return __half2float(__ushort_as_half((unsigned short)(bits16 & 0xffffu)));
+}
+// f32 -> f16 bit pattern, round to nearest even.
+__device__ __forceinline__ uint16_t f2h_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// wave64 butterfly sum; every lane ends with the total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, CQ_WAVE);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Quantized-activation scratch (written by the act-quant kernels, read by matvec / matmul / MoE).
+//   K-quant weights : int8 qs[rows][k] | float d[rows][k/256] | int16 bsums[rows][k/16]
+//   Q4_0 / Q8_0     : int8 qs[rows][k] | {float d; int32 sum;} ds[rows][k/32]
+// Sections start on 256-byte boundaries.
+// ---------------------------------------------------------------------------------------------
+struct ActLayout {
+    int64_t qs_off, d_off, bs_off, total;
+};
+
+__host__ __device__ inline int64_t cq_align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+__host__ __device__ inline ActLayout cq_act_layout(int w_dtype, int64_t k, int64_t rows) {
+    ActLayout L;
+    L.qs_off = 0;
+    L.d_off = cq_align256(rows * k);
+    if (cq_is_kquant(w_dtype)) {
+        L.bs_off = L.d_off + cq_align256(rows * (k / 256) * 4);
+        L.total = L.bs_off + cq_align256(rows * (k / 16) * 2);
+    } else {
+        L.bs_off = L.d_off;
+        L.total = L.d_off + cq_align256(rows * (k / 32) * 8);
+    }
+    return L;
+}
+
+struct ActView {            // resolved pointers for one scratch buffer
+    const int8_t *qs;       // [rows][k]
+    const float *d;         // K-quants: [rows][k/256];  Q4_0/Q8_0: interleaved {d, sum} pairs [rows][k/32][2]
+    const int16_t *bsums;   // K-quants only: [rows][k/16]
+};
+
+__host__ __device__ inline ActView cq_act_view(const void *scratch, int w_dtype, int64_t k, int64_t rows) {
+    ActLayout L = cq_act_layout(w_dtype, k, rows);
+    const uint8_t *b = (const uint8_t *)scratch;
+    ActView v;
+    v.qs = (const int8_t *)(b + L.qs_off);
+    v.d = (const float *)(b + L.d_off);
+    v.bsums = (const int16_t *)(b + L.bs_off);
+    return v;
+}

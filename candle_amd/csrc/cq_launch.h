@@ -1,0 +1,36 @@
+// Internal launcher interface between the extern "C" layer (cq_api.hip) and the kernel files.
+// Every launcher enqueues on `s`, never synchronizes, and returns 0 or a hipError_t / CQ_ERR_* code.
+#pragma once
+#include "cq_device.h"
+
+int cq_dequantize_launch(int dtype, const void *blocks, void *out, int64_t elems, int out_dtype, hipStream_t s);
+int cq_quantize_launch(int dtype, const float *x, void *blocks, int64_t elems, hipStream_t s);
+int cq_quantize_act_launch(int w_dtype, const void *x, int x_dtype, void *scratch, int64_t k, int64_t rows, hipStream_t s);
+int cq_matvec_launch(int w_dtype, const void *w, const void *scratch, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
+                     int64_t stride_dst, hipStream_t s);
+// same, over an already resolved (possibly row-offset) view of the activation scratch
+int cq_matvec_launch_av(int w_dtype, const void *w, const ActView &av, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
+                        int64_t stride_dst, hipStream_t s);
+int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
+                     int64_t stride_dst, hipStream_t s);
+int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t count, hipStream_t s);
+
+// ---- MoE: both public entry points reduce to "pairs" (expert, activation row, output row, scale) ----
+enum { MOE_INDEXED = 0, MOE_SORTED = 1 };
+struct MoeArgs {
+    int w_dtype;
+    const void *w;           // [num_experts, n, k] blocks
+    const float *x;          // [x_rows, k]
+    float *out;              // [n_pairs, n]
+    int64_t num_experts, n, k, n_pairs, x_rows;
+    int mode;
+    // MOE_INDEXED (QTensor::indexed_moe_forward): pair p = b * topk + t
+    const uint32_t *ids_u32;
+    int64_t topk, input_dim1;
+    // MOE_SORTED (candle_nn::moe::moe_gemm_gguf): pair m of the router-sorted list
+    const int32_t *sorted_token_ids, *expert_ids;
+    const float *topk_weights;
+    int prefill;
+};
+int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k);
+int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s);

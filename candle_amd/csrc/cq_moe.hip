@@ -1,0 +1,226 @@
+// Expert-grouped quantized matmul for gfx950: QTensor::indexed_moe_forward and
+// candle_nn::moe::moe_gemm_gguf behind one kernel pair.
+//
+// Both entry points are lists of "pairs" (expert, activation row, output row, scale):
+//   indexed_moe_forward (candle-core/src/quantized/cuda.rs:505-584, candle-kernels/src/quantized.cu:4670-4760)
+//       pair p = b * topk + t : expert ids[p], activation row (input_dim1 == 1 ? b : p), output row p, scale 1
+//   moe_gemm_gguf (candle-nn/src/moe.rs:169-337, candle-kernels/src/moe/moe_gguf.cu:55-132)
+//       pair m : expert expert_ids[m], tok = sorted_token_ids[m],
+//                activation row (topk_weights ? tok : tok / topk), output row tok, scale topk_weights[tok] or 1
+//
+// Step 1 quantizes the activation rows exactly as the CPU path does.  Step 2 (one workgroup)
+// buckets the pairs by expert with a counting sort, so the input order does not matter (the
+// reference sorts with an unstable sort, candle-core/src/sort.rs:282-297).  Step 3 streams every
+// hit expert's rows once: workgroup (row tile, expert) keeps the decoded weight registers and loops
+// over that expert's pairs — unlike the reference kernels, which re-read the expert's weights for
+// every pair routed to it.
+#include "cq_device.h"
+#include "cq_fmt.h"
+#include "cq_launch.h"
+
+namespace {
+
+struct MoeWorkspace {
+    int64_t act_off, offsets_off, cursor_off, pin_off, pout_off, pscale_off, total;
+};
+
+inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k) {
+    MoeWorkspace w;
+    w.act_off = 0;
+    w.offsets_off = cq_act_layout(w_dtype, k, x_rows).total;
+    w.cursor_off = w.offsets_off + cq_align256((num_experts + 1) * 4);
+    w.pin_off = w.cursor_off + cq_align256(num_experts * 4);
+    w.pout_off = w.pin_off + cq_align256(n_pairs * 4);
+    w.pscale_off = w.pout_off + cq_align256(n_pairs * 4);
+    w.total = w.pscale_off + cq_align256(n_pairs * 4);
+    return w;
+}
+
+struct PairSource {
+    int mode;
+    const uint32_t *ids_u32;
+    const int32_t *sorted_token_ids, *expert_ids;
+    const float *topk_weights;
+    int topk, input_dim1;
+    int n_pairs, num_experts, x_rows;
+};
+
+__device__ __forceinline__ bool pair_decode(const PairSource &ps, int p, int &e, int &in_row, int &out_row, float &scale) {
+    if (ps.mode == MOE_INDEXED) {
+        uint32_t id = ps.ids_u32[p];
+        e = (int)id;
+        in_row = ps.input_dim1 == 1 ? p / ps.topk : p;
+        out_row = p;
+        scale = 1.0f;
+        return id < (uint32_t)ps.num_experts;
+    }
+    e = ps.expert_ids[p];
+    int tok = ps.sorted_token_ids[p];
+    out_row = tok;
+    if (ps.topk_weights) {
+        in_row = tok;
+        // a token id outside the table would read past topk_weights; such pairs are dropped below
+        scale = (tok >= 0 && tok < ps.n_pairs) ? ps.topk_weights[tok] : 0.0f;
+    } else {
+        in_row = tok / ps.topk;
+        scale = 1.0f;
+    }
+    return e >= 0 && e < ps.num_experts && tok >= 0 && tok < ps.n_pairs && in_row < ps.x_rows;
+}
+
+// One workgroup: histogram of experts, exclusive scan, scatter of the pair descriptors.
+// offsets[e] .. offsets[e+1] is expert e's segment of pair_in / pair_out / pair_scale.
+__global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__restrict__ offsets, int *__restrict__ cursor,
+                                                         int *__restrict__ pair_in, int *__restrict__ pair_out,
+                                                         float *__restrict__ pair_scale, float *__restrict__ out, int n) {
+    __shared__ int carry;
+    const int tid = threadIdx.x;
+    const int E = ps.num_experts;
+    for (int e = tid; e < E; e += 1024) cursor[e] = 0;
+    __syncthreads();
+    for (int p = tid; p < ps.n_pairs; p += 1024) {
+        int e, in_row, out_row;
+        float scale;
+        if (pair_decode(ps, p, e, in_row, out_row, scale)) atomicAdd(&cursor[e], 1);
+    }
+    if (tid == 0) carry = 0;
+    __syncthreads();
+    // exclusive scan of the counts, 1024 experts per sweep
+    for (int base = 0; base < E; base += 1024) {
+        int e = base + tid;
+        int c = e < E ? cursor[e] : 0;
+        // inclusive scan inside the workgroup through shared memory
+        __shared__ int buf[1024];
+        buf[tid] = c;
+        __syncthreads();
+        for (int o = 1; o < 1024; o <<= 1) {
+            int v = tid >= o ? buf[tid - o] : 0;
+            __syncthreads();
+            buf[tid] += v;
+            __syncthreads();
+        }
+        int start = carry + buf[tid] - c;
+        if (e < E) {
+            offsets[e] = start;
+            cursor[e] = start;
+        }
+        __syncthreads();
+        if (tid == 1023) carry += buf[1023];
+        __syncthreads();
+    }
+    if (tid == 0) offsets[E] = carry;
+    __syncthreads();
+    for (int p = tid; p < ps.n_pairs; p += 1024) {
+        int e, in_row, out_row;
+        float scale;
+        if (pair_decode(ps, p, e, in_row, out_row, scale)) {
+            int pos = atomicAdd(&cursor[e], 1);
+            pair_in[pos] = in_row;
+            pair_out[pos] = out_row;
+            pair_scale[pos] = scale;
+        } else if (ps.mode == MOE_INDEXED) {
+            for (int c = 0; c < n; c++) out[(int64_t)p * n + c] = 0.0f;   // id out of range: defined output
+        }
+    }
+}
+
+// Workgroup (blockIdx.x = row tile, blockIdx.y = expert); 4 waves x R rows.  Pairs of the expert are
+// taken PB at a time with the decoded weight registers held across them.
+template <int DT, int R, int PB>
+__global__ __launch_bounds__(256) void moe_matvec_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ out,
+                                                         const int *__restrict__ offsets, const int *__restrict__ pair_in,
+                                                         const int *__restrict__ pair_out, const float *__restrict__ pair_scale,
+                                                         int k, int n) {
+    typedef Fmt<DT> F;
+    const int e = blockIdx.y;
+    const int seg0 = offsets[e], seg1 = offsets[e + 1];
+    if (seg0 == seg1) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * R;
+    if (row0 >= n) return;
+    const int nblk = k / BlockInfo<DT>::elems;
+    const int units = nblk * F::UPB;
+    const int64_t row_bytes = (int64_t)nblk * BlockInfo<DT>::bytes;
+    const uint8_t *we = w + (int64_t)e * n * row_bytes;
+
+    for (int s0 = seg0; s0 < seg1; s0 += PB) {
+        int arow[PB];
+#pragma unroll
+        for (int b = 0; b < PB; b++) arow[b] = pair_in[s0 + b < seg1 ? s0 + b : seg1 - 1];
+        float acc[R][PB];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int b = 0; b < PB; b++) acc[r][b] = 0.0f;
+
+        for (int u = lane; u < units; u += CQ_WAVE) {
+            typename F::W wr[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                int64_t row = row0 + r < n ? row0 + r : n - 1;
+                F::load_w(wr[r], we + row * row_bytes, u);
+            }
+            typename F::A ar[PB];
+#pragma unroll
+            for (int b = 0; b < PB; b++) F::load_a(ar[b], av, arow[b], k, u);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                typename F::P p;
+                F::prep(p, wr[r], u);
+#pragma unroll
+                for (int b = 0; b < PB; b++) acc[r][b] = F::dot(p, ar[b], acc[r][b]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int b = 0; b < PB; b++) {
+                float v = wave_sum(acc[r][b]);
+                if (lane == 0 && row0 + r < n && s0 + b < seg1)
+                    out[(int64_t)pair_out[s0 + b] * n + row0 + r] = v * pair_scale[s0 + b];
+            }
+    }
+}
+
+template <int DT>
+int launch_moe_matvec(const MoeArgs &a, const ActView &av, const int *offsets, const int *pin, const int *pout, const float *pscale,
+                      hipStream_t s) {
+    constexpr int R = 2, PB = 4;
+    int64_t tiles = (a.n + 4 * R - 1) / (4 * R);
+    if (tiles > 0x7fffffffLL || a.num_experts > 65535) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL((moe_matvec_kernel<DT, R, PB>), dim3((unsigned)tiles, (unsigned)a.num_experts), dim3(256), 0, s,
+                       (const uint8_t *)a.w, av, a.out, offsets, pin, pout, pscale, (int)a.k, (int)a.n);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k) {
+    return moe_workspace(w_dtype, num_experts, n_pairs, x_rows, k).total;
+}
+
+int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
+    if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
+    MoeWorkspace ws = moe_workspace(a.w_dtype, a.num_experts, a.n_pairs, a.x_rows, a.k);
+    uint8_t *b = (uint8_t *)workspace;
+    int rc = cq_quantize_act_launch(a.w_dtype, a.x, CQ_F32, b + ws.act_off, a.k, a.x_rows, s);
+    if (rc) return rc;
+    int *offsets = (int *)(b + ws.offsets_off), *cursor = (int *)(b + ws.cursor_off);
+    int *pin = (int *)(b + ws.pin_off), *pout = (int *)(b + ws.pout_off);
+    float *pscale = (float *)(b + ws.pscale_off);
+    PairSource ps;
+    ps.mode = a.mode; ps.ids_u32 = a.ids_u32; ps.sorted_token_ids = a.sorted_token_ids; ps.expert_ids = a.expert_ids;
+    ps.topk_weights = a.topk_weights; ps.topk = (int)a.topk; ps.input_dim1 = (int)a.input_dim1;
+    ps.n_pairs = (int)a.n_pairs; ps.num_experts = (int)a.num_experts; ps.x_rows = (int)a.x_rows;
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n);
+    if ((rc = (int)hipGetLastError())) return rc;
+    ActView av = cq_act_view(b + ws.act_off, a.w_dtype, a.k, a.x_rows);
+    switch (a.w_dtype) {
+        case CQ_Q4_0: return launch_moe_matvec<CQ_Q4_0>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q8_0: return launch_moe_matvec<CQ_Q8_0>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q4K: return launch_moe_matvec<CQ_Q4K>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q5K: return launch_moe_matvec<CQ_Q5K>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q6K: return launch_moe_matvec<CQ_Q6K>(a, av, offsets, pin, pout, pscale, s);
+    }
+    return CQ_ERR_DTYPE;
+}

@@ -1,0 +1,157 @@
+/*
+ * candle_hip_quant.h — C ABI of the MI355X (gfx950) GGUF quantized-matmul library.
+ *
+ * This is the boundary a `hip` backend of candle-core binds through FFI, in the same way
+ * candle-core binds candle-kernels' statically linked launchers
+ * (candle-kernels/src/ffi.rs:4-631, called from candle-core/src/quantized/fast_mmvq.rs:227-248 and
+ * candle-nn/src/moe.rs:279-317).  Conventions:
+ *
+ *   - plain pointers and sizes only; every pointer named *_dev is a device pointer;
+ *   - the caller owns every buffer; the library never allocates, frees or synchronizes;
+ *     scratch/workspace sizes come from the matching *_bytes() query;
+ *   - everything is enqueued on the caller's stream (`stream` is a hipStream_t passed as void*,
+ *     NULL = the default stream), so calls can be captured into a HIP graph;
+ *   - every entry point returns a status: 0 = ok, negative = argument error (CQ_ERR_*),
+ *     positive = the hipError_t reported by the launch;
+ *   - weights are GGUF blocks exactly as stored on disk, rows contiguous, `n` rows of `k/blk` blocks
+ *     (candle-core/src/quantized/k_quants.rs:77-190); kernels read only [ptr, ptr + size) and never
+ *     rely on the 512-element tail padding the CUDA backend adds
+ *     (candle-core/src/quantized/cuda.rs:624-637,989-1008);
+ *   - activation quantization follows candle's CPU path bit for bit (Q8_K blocks for K-quants,
+ *     Q8_0 blocks for Q4_0/Q8_0: k_quants.rs:2320-2358, 658-687), so results match
+ *     QMatMul::forward on the CPU up to f32 summation order.
+ */
+#ifndef CANDLE_HIP_QUANT_H
+#define CANDLE_HIP_QUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GGUF type codes: GgmlDType::{from_u32,to_u32}, candle-core/src/quantized/mod.rs:300-342 */
+enum cq_dtype {
+    CQ_F32 = 0, CQ_F16 = 1, CQ_Q4_0 = 2, CQ_Q4_1 = 3, CQ_Q5_0 = 6, CQ_Q5_1 = 7, CQ_Q8_0 = 8,
+    CQ_Q8_1 = 9, CQ_Q2K = 10, CQ_Q3K = 11, CQ_Q4K = 12, CQ_Q5K = 13, CQ_Q6K = 14, CQ_Q8K = 15,
+    CQ_BF16 = 30
+};
+
+enum cq_status {
+    CQ_OK = 0,
+    CQ_ERR_DTYPE = -1,      /* dtype not supported by this entry point */
+    CQ_ERR_SHAPE = -2,      /* k not a multiple of the block size, negative sizes, ... */
+    CQ_ERR_ALIGN = -3,      /* a pointer does not meet the stated alignment */
+    CQ_ERR_NULL = -4,       /* a required pointer is NULL */
+    CQ_ERR_WORKSPACE = -5,  /* workspace smaller than the *_bytes() query asks for */
+    CQ_ERR_RANGE = -6       /* a size exceeds what the entry point supports */
+};
+
+/* Human-readable text for a status returned by any entry point. */
+const char *cq_status_string(int status);
+
+/* GgmlDType::block_size / type_size (mod.rs:386-421). 0 for an unknown dtype. */
+int64_t cq_block_size(int dtype);
+int64_t cq_type_size(int dtype);
+/* Bytes of `elem_count` elements stored as `dtype` blocks (QCudaStorage::storage_size_in_bytes,
+ * cuda.rs:880-882, without the tail padding). -1 if elem_count is not a multiple of the block size. */
+int64_t cq_storage_bytes(int dtype, int64_t elem_count);
+
+/* ---------------------------------------------------------------------------------------------
+ * QTensor::dequantize / dequantize_f16 (mod.rs:689-710; CUDA: cuda.rs:105-223,
+ * candle-kernels/src/quantized.cu:780-1156).  Bit-exact with GgmlType::to_float on the CPU; the
+ * f16 result equals the f32 result rounded to nearest even.
+ *   dtype: Q4_0, Q8_0, Q4K, Q5K, Q6K, Q8K.   out_dtype: CQ_F32 or CQ_F16.
+ *   blocks_dev: 2-byte aligned.  out_dev: 16-byte aligned.
+ * ------------------------------------------------------------------------------------------- */
+int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem_count, int out_dtype, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * QTensor::quantize on a device tensor (mod.rs:543-562).  The CUDA backend copies to the host,
+ * runs GgmlType::from_float and copies back (cuda.rs:704-725); here the same arithmetic runs on the
+ * GPU, one thread per block, and produces the same bytes as the CPU from_float.
+ *   dtype: Q4_0, Q8_0, Q4K, Q5K, Q6K, Q8K.   x_dev: f32, 4-byte aligned.  blocks_dev: 2-byte aligned.
+ * ------------------------------------------------------------------------------------------- */
+int cq_quantize(int dtype, const float *x_dev, void *blocks_dev, int64_t elem_count, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Activation quantization, the first half of k_quants::matmul (k_quants.rs:2419-2428): each of
+ * `rows` activation rows of length k is quantized to the weight type's VecDotType — Q8_K for
+ * Q4K/Q5K/Q6K/Q8K, Q8_0 for Q4_0/Q8_0 — with the same results as the CPU from_float.  Replaces the
+ * q8_1 quantize launch of the CUDA backend (cuda.rs:48-103, fast_mmvq.rs:296-303).
+ *
+ * Scratch layout (device-private, 256-byte aligned sections, in this order):
+ *   K-quants : int8 qs[rows][k] | float d[rows][k/256] | int16 bsums[rows][k/16]
+ *   Q4_0/Q8_0: int8 qs[rows][k] | struct { float d (f16-rounded); int32 sum; } ds[rows][k/32]
+ *   x_dtype: CQ_F32, CQ_F16 or CQ_BF16.  x_dev: 16-byte aligned, rows contiguous.  scratch_dev: 256-byte aligned.
+ * ------------------------------------------------------------------------------------------- */
+int64_t cq_act_scratch_bytes(int w_dtype, int64_t k, int64_t rows);
+int cq_quantize_act(int w_dtype, const void *x_dev, int x_dtype, void *scratch_dev, int64_t k, int64_t rows, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Decode matvec over pre-quantized activations:  dst[r, j] = sum_k W[j, k] * x^[r, k]
+ * for r < rows <= CQ_MATVEC_MAX_ROWS.  Counterpart of launch_mmvq_gguf_<t>_<dst>_plain
+ * (candle-kernels/src/ffi.rs:58-631, mmvq_gguf.cu:915-1008).
+ *   w_dev: n rows of k/blk blocks; 16-byte aligned for Q4K/Q5K, 2-byte aligned otherwise.
+ *   act_scratch_dev: written by cq_quantize_act with the same (w_dtype, k, rows).
+ *   dst_dev: f32 / f16 / bf16 (dst_dtype), row stride `stride_dst` elements (>= n).
+ * ------------------------------------------------------------------------------------------- */
+#define CQ_MATVEC_MAX_ROWS 8
+int cq_matvec(int w_dtype, const void *w_dev, const void *act_scratch_dev, void *dst_dev, int dst_dtype,
+              int64_t k, int64_t n, int64_t rows, int64_t stride_dst, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Prefill matmul over pre-quantized activations (any rows >= 1), MFMA tiles with the dequantized
+ * weight tile staged in LDS.  Counterpart of launch_mmq_gguf_<t> (candle-core/src/quantized/
+ * fast_mmq.rs:71-111, candle-kernels/src/mmq_gguf/).  Same buffers as cq_matvec; dst is f32.
+ * ------------------------------------------------------------------------------------------- */
+int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float *dst_dev,
+              int64_t k, int64_t n, int64_t rows, int64_t stride_dst, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * QCudaStorage::fwd (cuda.rs:846-878), the body of CustomOp1::cuda_fwd for QTensor
+ * (mod.rs:1007-1017): quantize the m activation rows, then matvec (m <= CQ_MATVEC_MAX_ROWS) or
+ * MFMA matmul.  x is [m, k] contiguous (f32 / f16 / bf16), dst is [m, n] contiguous in dst_dtype
+ * (CUDA keeps the input dtype: fast_mmvq.rs:161-323).  workspace_dev: 256-byte aligned,
+ * at least cq_qmatmul_workspace_bytes(w_dtype, m, k, n) bytes.
+ * ------------------------------------------------------------------------------------------- */
+int64_t cq_qmatmul_workspace_bytes(int w_dtype, int64_t m, int64_t k, int64_t n);
+int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_dtype, void *dst_dev, int dst_dtype,
+                       int64_t m, int64_t k, int64_t n, void *workspace_dev, int64_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * QTensor::indexed_moe_forward (mod.rs:758-784 -> cuda.rs:505-622 ->
+ * candle-kernels/src/quantized.cu:4670-4845):
+ *   w [num_experts, n, k] blocks, x [batch, input_dim1, k] f32 with input_dim1 == topk or 1,
+ *   ids [batch, topk] u32  ->  out [batch, topk, n] f32,
+ *   out[b, t, :] = W[ids[b, t]] . x[b, input_dim1 == 1 ? 0 : t, :].
+ * Pairs are grouped by expert on the device so each expert's rows are streamed once per call.
+ * An id >= num_experts leaves its output row zero-filled.
+ * ------------------------------------------------------------------------------------------- */
+int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk, int64_t input_dim1);
+int cq_indexed_moe_forward(int w_dtype, const void *w_dev, const float *x_dev, const uint32_t *ids_dev, float *out_dev,
+                           int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk, int64_t input_dim1,
+                           void *workspace_dev, int64_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * candle_nn::moe::moe_gemm_gguf (candle-nn/src/moe.rs:169-337 -> ffi.rs:25-56 ->
+ * candle-kernels/src/moe/moe_gguf.cu:149-216 and moe_wmma_gguf.cu:354-422):
+ *   for m < size_m: tok = sorted_token_ids[m], e = expert_ids[m] (pairs with e outside
+ *   [0, num_experts) are skipped); in_row = topk_weights ? tok : tok / topk;
+ *   out[tok, :] = (topk_weights ? topk_weights[tok] : 1) * W[e] . x[in_row, :]
+ *   x [size_m or size_m/topk, k] f32, out [size_m, n] f32, sorted_token_ids / expert_ids int32 [size_m]
+ *   (both device pointers), topk_weights f32 [size_m] device pointer or NULL.
+ * `is_prefill` selects the MFMA grouped kernel (the reference's WMMA prefill kernel) instead of the
+ * expert-grouped matvec; both give the same values up to f32 summation order.
+ * ------------------------------------------------------------------------------------------- */
+int64_t cq_moe_gemm_workspace_bytes(int w_dtype, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int has_topk_weights);
+int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const int32_t *sorted_token_ids_dev,
+                     const int32_t *expert_ids_dev, const float *topk_weights_dev, float *out_dev,
+                     int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int is_prefill,
+                     void *workspace_dev, int64_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CANDLE_HIP_QUANT_H */

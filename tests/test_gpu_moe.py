@@ -1,0 +1,145 @@
+"""GPU parity for the expert-grouped quantized matmul: QTensor::indexed_moe_forward and
+candle_nn::moe::moe_gemm_gguf, against the CPU oracle's per-pair composition of k_quants::matmul.
+The reference has no tests for these kernels and no CPU implementation (mod.rs:776-782); the
+oracle functions are pinned by brute force in tests/test_oracle_moe.py.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.util import normal, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+TIGHT = 2e-6
+WDTYPES = [oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q4_0]
+NAMES = {oracle.Q4_0: "q4_0", oracle.Q8_0: "q8_0", oracle.Q4K: "q4k", oracle.Q5K: "q5k", oracle.Q6K: "q6k"}
+
+
+def make_experts(dtype, E, n, k, seed):
+    import candle_amd as ca
+    w = normal(seed, (E, n, k), 0.02)
+    blocks = oracle.from_float(dtype, w.reshape(-1))
+    qt = ca.QTensor.new(ca.QStorage.from_data(blocks, "cuda", ca.GgmlDType(dtype)), (E, n, k))
+    return blocks, qt
+
+
+def route(tokens, E, topk, seed):
+    """Router of fused_moe.rs:222-260 on random logits: top-k ids + renormalised softmax weights,
+    then the flattened expert list sorted ascending with the matching token-slot permutation."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    logits = rng.standard_normal((tokens, E)).astype(np.float32)
+    p = np.exp(logits - logits.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    ids = np.argsort(-p, axis=1, kind="stable")[:, :topk].astype(np.uint32)
+    w = np.take_along_axis(p, ids.astype(np.int64), axis=1)
+    w = (w / w.sum(axis=1, keepdims=True)).astype(np.float32)
+    flat = ids.reshape(-1).astype(np.int32)
+    order = np.argsort(flat, kind="stable").astype(np.int32)
+    return ids, w, flat[order], order
+
+
+@pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("input_dim1_is_one", [True, False])
+def test_indexed_moe_forward(dtype, input_dim1_is_one):
+    E, n, k, batch, topk = 8, 48, 512, 5, 3
+    blocks, qt = make_experts(dtype, E, n, k, seed=5)
+    ids, _, _, _ = route(batch, E, topk, seed=6)
+    x = normal(7, (batch, 1 if input_dim1_is_one else topk, k), 1.0)
+    out = qt.indexed_moe_forward(torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda())
+    torch.cuda.synchronize()
+    want = oracle.indexed_moe_forward(dtype, blocks, (E, n, k), x, ids)
+    assert out.shape == (batch, topk, n)
+    err = rel_l2(out.cpu().numpy(), want)
+    assert err <= TOL and err <= TIGHT, err
+
+
+@pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("tokens", [1, 16, 40])
+@pytest.mark.parametrize("is_prefill", [False, True])
+def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
+    """The two call shapes of FusedMoeGGUF::forward (fused_moe.rs:263-294): gate/up without
+    topk_weights on [tokens, k], down with topk_weights on [tokens*topk, k]."""
+    import candle_amd as ca
+    E, n, k, topk = 16, 64, 256, 4
+    blocks, qt = make_experts(dtype, E, n, k, seed=15)
+    ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=16 + tokens)
+    sti = torch.from_numpy(sorted_token_ids).cuda()
+    eid = torch.from_numpy(expert_ids).cuda()
+
+    x = normal(17, (tokens, k), 1.0)
+    got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, None, sti, eid, topk, is_prefill)
+    torch.cuda.synchronize()
+    want = oracle.moe_gemm_gguf(dtype, x, blocks, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+    assert got.shape == (tokens * topk, n)
+    err = rel_l2(got.cpu().numpy(), want)
+    assert err <= TOL and err <= TIGHT, err
+
+    x2 = normal(18, (tokens * topk, k), 1.0)
+    twf = tw.reshape(-1)
+    got2 = ca.moe_gemm_gguf(torch.from_numpy(x2).cuda(), qt, torch.from_numpy(twf).cuda(), sti, eid, topk, is_prefill)
+    torch.cuda.synchronize()
+    want2 = oracle.moe_gemm_gguf(dtype, x2, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
+    err2 = rel_l2(got2.cpu().numpy(), want2)
+    assert err2 <= TOL and err2 <= TIGHT, err2
+
+
+def test_moe_gemm_is_invariant_to_pair_order():
+    # the reference sorts with an unstable sort (candle-core/src/sort.rs:282-297): any order of the pairs
+    # inside an expert segment, and indeed any permutation of the pair list, must give the same output
+    import candle_amd as ca
+    E, n, k, topk, tokens = 16, 64, 256, 4, 24
+    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=25)
+    ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=26)
+    x = torch.from_numpy(normal(27, (tokens, k), 1.0)).cuda()
+    base = ca.moe_gemm_gguf(x, qt, None, torch.from_numpy(sorted_token_ids).cuda(), torch.from_numpy(expert_ids).cuda(), topk, False)
+    perm = np.random.Generator(np.random.PCG64(28)).permutation(expert_ids.size)
+    shuf = ca.moe_gemm_gguf(x, qt, None, torch.from_numpy(sorted_token_ids[perm].copy()).cuda(),
+                            torch.from_numpy(expert_ids[perm].copy()).cuda(), topk, False)
+    torch.cuda.synchronize()
+    assert torch.equal(base, shuf)
+
+
+def test_moe_gemm_skips_invalid_experts():
+    import candle_amd as ca
+    E, n, k, topk, tokens = 4, 32, 256, 2, 3
+    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=35)
+    expert_ids = np.array([0, 1, -1, 2, 7, 3], dtype=np.int32)     # -1 and 7 are outside [0, E)
+    sorted_token_ids = np.arange(6, dtype=np.int32)
+    x = normal(36, (tokens, k), 1.0)
+    out = torch.full((6, n), 123.0, device="cuda")
+    from candle_amd import _lib
+    L = _lib.lib()
+    xs = torch.from_numpy(x).cuda()
+    sti = torch.from_numpy(sorted_token_ids).cuda()
+    eid = torch.from_numpy(expert_ids).cuda()
+    need = L.cq_moe_gemm_workspace_bytes(int(ca.GgmlDType.Q4K), E, topk, 6, n, k, 0)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    _lib.check("cq_moe_gemm_gguf", L.cq_moe_gemm_gguf(int(ca.GgmlDType.Q4K), xs.data_ptr(), qt.device_ptr(), sti.data_ptr(), eid.data_ptr(),
+                                                      None, out.data_ptr(), E, topk, 6, n, k, 0, ws.data_ptr(), need, None))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.all(got[2] == 123.0) and np.all(got[4] == 123.0)          # skipped rows untouched (moe_gguf.cu:91)
+    want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+    keep = [0, 1, 3, 5]
+    assert rel_l2(got[keep], want[keep]) <= TIGHT
+
+
+def test_moe_qwen3_shape_single_token():
+    # BASELINE configs[4] shape: 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K; one token
+    import candle_amd as ca
+    E, topk = 128, 8
+    for (n, k) in ((768, 2048), (2048, 768)):
+        w = torch.from_numpy(normal(45, (E, n, k), 0.02)).cuda()
+        qt = ca.QTensor.quantize(w, ca.GgmlDType.Q4K)
+        blocks = np.frombuffer(qt.data(), dtype=np.uint8)
+        ids, tw, expert_ids, sorted_token_ids = route(1, E, topk, seed=46)
+        x = normal(47, (1, k), 1.0)
+        got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, None, torch.from_numpy(sorted_token_ids).cuda(),
+                               torch.from_numpy(expert_ids).cuda(), topk, False)
+        torch.cuda.synchronize()
+        want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+        err = rel_l2(got.cpu().numpy(), want)
+        assert err <= TOL and err <= TIGHT, err

@@ -1,0 +1,95 @@
+"""CPU-only checks of the host layer: the C-ABI library loads and exports every declared symbol,
+argument validation returns the documented codes before anything touches a GPU, and the Python
+mirror of candle's API keeps candle's sizes and error behaviour."""
+import os
+import re
+
+import pytest
+
+import oracle
+from candle_amd import _lib
+from candle_amd.quantized import GgmlDType, check_shape
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "candle_hip_quant.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib.lib()
+    names = declared_symbols()
+    assert len(names) >= 15
+    for name in names:
+        assert hasattr(L, name), f"{name} declared in include/candle_hip_quant.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), "ctypes signatures out of sync with the header"
+
+
+def test_dtype_sizes_match_reference_and_oracle():
+    # mod.rs:386-421 and the size asserts of k_quants.rs:83-190
+    want = {GgmlDType.Q4_0: (32, 18), GgmlDType.Q4_1: (32, 20), GgmlDType.Q5_0: (32, 22), GgmlDType.Q5_1: (32, 24),
+            GgmlDType.Q8_0: (32, 34), GgmlDType.Q8_1: (32, 36), GgmlDType.Q2K: (256, 84), GgmlDType.Q3K: (256, 110),
+            GgmlDType.Q4K: (256, 144), GgmlDType.Q5K: (256, 176), GgmlDType.Q6K: (256, 210), GgmlDType.Q8K: (256, 292),
+            GgmlDType.F32: (1, 4), GgmlDType.F16: (1, 2), GgmlDType.BF16: (1, 2)}
+    L = _lib.lib()
+    for dt, (bs, ts) in want.items():
+        assert (dt.block_size(), dt.type_size()) == (bs, ts)
+        assert (L.cq_block_size(int(dt)), L.cq_type_size(int(dt))) == (bs, ts)
+    for dt in (oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q8K):
+        assert oracle.block_size(dt) == L.cq_block_size(dt) and oracle.type_size(dt) == L.cq_type_size(dt)
+    assert GgmlDType.from_u32(12) is GgmlDType.Q4K and GgmlDType.Q6K.to_u32() == 14 and GgmlDType.BF16.to_u32() == 30
+    with pytest.raises(ValueError):
+        GgmlDType.from_u32(4)
+    # BASELINE shapes (bytes of a [14336 x 4096] Q4_K tensor etc.)
+    assert L.cq_storage_bytes(12, 14336 * 4096) == 33030144
+    assert L.cq_storage_bytes(14, 4096 * 14336) == 48168960
+    assert L.cq_storage_bytes(8, 4096 * 4096) == 17825792
+    assert L.cq_storage_bytes(12, 100) == -1
+
+
+def test_check_shape_errors():
+    # mod.rs:518-530
+    check_shape((4, 256), 256)
+    with pytest.raises(ValueError, match="scalar tensor cannot be quantized"):
+        check_shape((), 32)
+    with pytest.raises(ValueError, match="divisible by block size"):
+        check_shape((4, 100), 32)
+
+
+def test_argument_validation_codes_without_gpu():
+    L = _lib.lib()
+    Q4K, Q2K, Q8K = 12, 10, 15
+    OK, DTYPE, SHAPE, ALIGN, NULL, WS, RANGE = 0, -1, -2, -3, -4, -5, -6
+    # scratch sizes: K-quants: qs + d + bsums sections, each rounded up to 256 bytes
+    assert L.cq_act_scratch_bytes(Q4K, 4096, 1) == 4096 + 256 + 512
+    assert L.cq_act_scratch_bytes(8, 4096, 2) == 8192 + 2048
+    assert L.cq_act_scratch_bytes(Q4K, 100, 1) == -1
+    assert L.cq_quantize_act(Q4K, None, 0, None, 4096, 0, None) == OK          # zero rows: nothing to do
+    assert L.cq_quantize_act(Q4K, None, 0, None, 4096, 1, None) == NULL
+    assert L.cq_quantize_act(Q4K, 16, 0, 256, 4000, 1, None) == SHAPE
+    assert L.cq_quantize_act(Q4K, 8, 0, 256, 4096, 1, None) == ALIGN           # x must be 16-byte aligned
+    assert L.cq_quantize_act(Q4K, 16, 12, 256, 4096, 1, None) == DTYPE         # activations must be f32/f16/bf16
+    assert L.cq_matvec(Q2K, 16, 256, 16, 0, 256, 4, 1, 4, None) == DTYPE
+    assert L.cq_matvec(Q8K, 16, 256, 16, 0, 256, 4, 1, 4, None) == DTYPE       # Q8K is not a matmul weight type
+    assert L.cq_matvec(Q4K, 16, 256, 16, 0, 256, 4, 9, 4, None) == RANGE       # more than CQ_MATVEC_MAX_ROWS
+    assert L.cq_matvec(Q4K, 16, 256, 16, 0, 256, 4, 1, 3, None) == SHAPE       # stride_dst < n
+    assert L.cq_matvec(Q4K, 8, 256, 16, 0, 256, 4, 1, 4, None) == ALIGN        # Q4_K weights: 16-byte aligned
+    assert L.cq_matvec(Q4K, None, 256, 16, 0, 256, 4, 1, 4, None) == NULL
+    assert L.cq_matvec(Q4K, None, None, None, 0, 256, 0, 1, 0, None) == OK     # n == 0
+    assert L.cq_qmatmul_workspace_bytes(Q4K, 1, 4096, 14336) == 4096 + 256 + 512
+    assert L.cq_qmatmul_forward(Q4K, 16, 16, 0, 16, 0, 1, 4096, 8, 256, 10, None) == WS
+    assert L.cq_indexed_moe_workspace_bytes(Q4K, 8, 16, 256, 2, 4, 3) == -1    # input_dim1 must be topk or 1
+    assert L.cq_moe_gemm_workspace_bytes(Q4K, 8, 4, 6, 16, 256, 0) == -1       # size_m not a multiple of topk
+    assert L.cq_moe_gemm_gguf(Q4K, 16, 16, 4, 4, None, 4, 8, 4, 8, 16, 256, 0, 256, 0, None) == WS
+    assert _lib.status_string(SHAPE).startswith("invalid shape")
+    assert _lib.status_string(OK) == "ok"
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.lib()
