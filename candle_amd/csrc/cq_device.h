@@ -43,8 +43,14 @@ template <typename T> __device__ __forceinline__ void st_u(void *p, T v) {
 __device__ __forceinline__ float h2f(uint32_t bits16) {
     return __half2float(__ushort_as_half((unsigned short)(bits16 & 0xffffu)));
 }
-// f32 -> f16 bit pattern, round to nearest even.
-__device__ __forceinline__ uint16_t f2h_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
+// f32 -> f16 bit pattern, round to nearest even.  The conversion is issued as an opaque
+// v_cvt_f16_f32 on the finished f32 value: left to the compiler, `f16(a * b)` becomes
+// v_fma_mixlo_f16(a, b, +0), which turns a -0.0 product into +0.0.
+__device__ __forceinline__ uint16_t f2h_bits(float f) {
+    uint32_t r;
+    asm("v_cvt_f16_f32 %0, %1" : "=v"(r) : "v"(f));
+    return (uint16_t)(r & 0xffffu);
+}
 
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
