@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF quantized-matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[1], the configuration the metric is quoted on): Q4_K decode matvec,
+weight [14336 x 4096] (1x4096 -> 14336), batch 1, f32 activations ~N(0,1), weights ~N(0,0.02)
+quantized to Q4_K on the device.  One "step" is one pass of the hot path over one activation batch:
+activation quantization + matvec, i.e. QMatMul::forward.  Inputs are resident in HBM when the timed
+region starts.  Steps rotate through a pool of distinct weight tensors larger than the 256 MB
+Infinity Cache, so every step streams its 33 MB of weights from HBM.
+
+The JSON line carries, besides the driver contract fields:
+  roofline      achieved algorithmic GB/s of the dominant kernel (the matvec) from HIP events around
+                back-to-back launches on the launch stream, against the 8 TB/s HBM peak
+  cpu_baseline  the C restatement of candle's CPU path (AVX2 dot products + column-split threads,
+                oracle/cq_oracle_fast.c) timed on this box's host cores on a bounded sample
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+Q4K = 12
+
+
+def algorithmic_bytes(n, k, m, type_size, block):
+    """weights once + f32 activations in + f32 outputs (scratch traffic is not counted)."""
+    return n * (k // block) * type_size + m * k * 4 + m * n * 4
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--n", type=int, default=14336)
+    ap.add_argument("--k", type=int, default=4096)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--pool-mb", type=int, default=1280, help="distinct weight bytes rotated through (MB)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (every configuration of the metric is single-GPU); use --gpus 1")
+
+    import numpy as np
+    import torch
+
+    from candle_amd import _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    n, k, m = args.n, args.k, args.batch
+    wbytes = L.cq_storage_bytes(Q4K, n * k)
+    alg_bytes = algorithmic_bytes(n, k, m, 144, 256)
+
+    # ---- synthetic inputs, resident in HBM --------------------------------------------------
+    pool = max(2, (args.pool_mb * 1000 * 1000 + wbytes - 1) // wbytes)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    weights = []
+    for i in range(pool):
+        wf = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
+        wq = torch.empty(wbytes, dtype=torch.uint8, device=dev)
+        _lib.check("cq_quantize", L.cq_quantize(Q4K, wf.data_ptr(), wq.data_ptr(), n * k, None))
+        weights.append(wq)
+        del wf
+    x = torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32)
+    dst = torch.empty((m, n), dtype=torch.float32, device=dev)
+    ws_bytes = L.cq_qmatmul_workspace_bytes(Q4K, m, k, n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+
+    stream = torch.cuda.Stream(device=dev)
+
+    def step(i, sp):
+        _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(Q4K, weights[i % pool].data_ptr(), x.data_ptr(), 0, dst.data_ptr(), 0,
+                                                              m, k, n, ws.data_ptr(), ws_bytes, sp))
+
+    def matvec_only(i, sp):
+        _lib.check("cq_matvec", L.cq_matvec(Q4K, weights[i % pool].data_ptr(), ws.data_ptr(), dst.data_ptr(), 0, k, n, m, n, sp))
+
+    # The step is a few microseconds of GPU work: capture one rotation over the pool in a HIP graph
+    # so that host launch latency is not what gets measured.
+    def capture(fn):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            fn(0, stream.cuda_stream)          # warm the code path before capture
+            stream.synchronize()
+            with torch.cuda.graph(g, stream=stream):
+                sp = torch.cuda.current_stream().cuda_stream
+                for i in range(pool):
+                    fn(i, sp)
+        return g
+
+    g_step = capture(step)
+    g_mv = capture(matvec_only)
+
+    def run(graph, steps):
+        reps = max(1, (steps + pool - 1) // pool)
+        with torch.cuda.stream(stream):
+            for _ in range(reps):
+                graph.replay()
+        return reps * pool
+
+    # ---- timed region: EXACTLY K steps (rounded up to whole rotations), wall clock ------------
+    run(g_step, args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    done = run(g_step, args.steps)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / done
+    value = alg_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- dominant kernel: back-to-back matvec launches between HIP events on the launch stream ----
+    run(g_mv, args.warmup)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        e0.record(stream)
+        done_mv = run(g_mv, args.steps)
+        e1.record(stream)
+    torch.cuda.synchronize()
+    mv_us = e0.elapsed_time(e1) * 1e3 / done_mv
+    achieved = alg_bytes / (mv_us * 1e-6) / 1e9
+
+    # ---- same kernel with the weights resident in the Infinity Cache (one tensor reused), labelled ----
+    g_res = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        stream.synchronize()
+        with torch.cuda.graph(g_res, stream=stream):
+            sp = torch.cuda.current_stream().cuda_stream
+            for _ in range(pool):
+                matvec_only(0, sp)
+        for _ in range(10):
+            g_res.replay()
+        e0.record(stream)
+        for _ in range(50):
+            g_res.replay()
+        e1.record(stream)
+    torch.cuda.synchronize()
+    res_us = e0.elapsed_time(e1) * 1e3 / (50 * pool)
+
+    out = {
+        "metric": "Q4_K matvec GB/s @4096x14336 (decode, batch %d)" % m,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": done,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8",
+        "data": "synthetic",
+        "config": {"workload": "Q4_K decode matvec 1x%d->%d, weight [%d x %d] Q4_K, batch %d, %d distinct weight tensors rotated (%.2f GB)"
+                               % (k, n, n, k, m, pool, pool * wbytes / 1e9),
+                   "step": "activation quantize (Q8_K) + matvec, captured in a HIP graph", "n": n, "k": k, "batch": m},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "roofline": {"bound": "hbm", "kernel": "matvec_kernel<Q4_K>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "avg_kernel_us": round(mv_us, 3),
+                     "algorithmic_bytes_per_launch": alg_bytes,
+                     "cache_resident_us": round(res_us, 3), "cache_resident_GBps": round(alg_bytes / (res_us * 1e-6) / 1e9, 1)},
+    }
+
+    if not args.no_cpu_baseline:
+        import oracle
+        cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "16")), 16)
+        host_pool = min(pool, 8)
+        hw = [weights[i].cpu().numpy() for i in range(host_pool)]
+        hx = x.cpu().numpy()
+        oracle.matmul_fast(Q4K, hx, hw[0], n, cores)
+        t0 = time.perf_counter()
+        it = 0
+        while time.perf_counter() - t0 < args.cpu_seconds:
+            oracle.matmul_fast(Q4K, hx, hw[it % host_pool], n, cores)
+            it += 1
+        dt = (time.perf_counter() - t0) / it
+        out["cpu_baseline"] = {"value": round(alg_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                               "sample": "%d calls of the same 1x%d->%d Q4_K matvec over %d rotated host weight copies (%.1f s); "
+                                         "C restatement of candle's CPU path: Q8_K activation quantize + AVX2 vec_dot + column split over threads"
+                                         % (it, k, n, host_pool, args.cpu_seconds),
+                               "ms_per_call": round(dt * 1e3, 4)}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

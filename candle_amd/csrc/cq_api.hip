@@ -163,9 +163,9 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     if (!aligned(x_dev, 16) || !aligned(workspace_dev, 256) || !aligned(dst_dev, float_size(dst_dtype))) return CQ_ERR_ALIGN;
     if (workspace_bytes < cq_qmatmul_workspace_bytes(w_dtype, m, k, n)) return CQ_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
+    // decode: one kernel quantizes the activations into LDS and streams W (no scratch traffic)
+    if (m <= CQ_MATVEC_MAX_ROWS) return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
     if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
-    if (m <= CQ_MATVEC_MAX_ROWS)
-        return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, dst_dtype, k, n, m, n, s);
     if (dst_dtype == CQ_F32)
         return cq_matmul_launch(w_dtype, w_dev, workspace_dev, (float *)dst_dev, k, n, m, n, s);
     float *tmp = (float *)((uint8_t *)workspace_dev + cq_act_layout(w_dtype, k, m).total);

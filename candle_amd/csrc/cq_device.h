@@ -56,6 +56,61 @@ __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
 }
 
+// ---- DPP cross-lane helpers (a few cycles each; ds_bpermute-based shuffles cost a round trip through
+// the LDS crossbar per step, which dominates short dependent chains) --------------------------------
+#define CQ_DPP_QUAD_XOR1 0xB1     // quad_perm [1,0,3,2]
+#define CQ_DPP_QUAD_XOR2 0x4E     // quad_perm [2,3,0,1]
+#define CQ_DPP_ROW_SHR(n) (0x110 + (n))
+#define CQ_DPP_ROW_HALF_MIRROR 0x141
+#define CQ_DPP_ROW_BCAST15 0x142
+#define CQ_DPP_ROW_BCAST31 0x143
+
+// max over the wave of a non-negative float, returned in every lane (through a scalar register)
+__device__ __forceinline__ float wave_max_nonneg(float v) {
+#define CQ_MX(ctrl, rmask, bc) v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), ctrl, rmask, 0xf, bc)))
+    CQ_MX(CQ_DPP_ROW_SHR(1), 0xf, false);
+    CQ_MX(CQ_DPP_ROW_SHR(2), 0xf, false);
+    CQ_MX(CQ_DPP_ROW_SHR(4), 0xf, false);
+    CQ_MX(CQ_DPP_ROW_SHR(8), 0xf, false);      // lane 15 of each row: row max
+    CQ_MX(CQ_DPP_ROW_BCAST15, 0xa, false);
+    CQ_MX(CQ_DPP_ROW_BCAST31, 0xc, false);     // lane 63: wave max
+#undef CQ_MX
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// min over the wave of an int, returned in every lane
+__device__ __forceinline__ int wave_min_int(int v) {
+#define CQ_MN(ctrl, rmask) v = min(v, __builtin_amdgcn_update_dpp(v, v, ctrl, rmask, 0xf, false))
+    CQ_MN(CQ_DPP_ROW_SHR(1), 0xf);
+    CQ_MN(CQ_DPP_ROW_SHR(2), 0xf);
+    CQ_MN(CQ_DPP_ROW_SHR(4), 0xf);
+    CQ_MN(CQ_DPP_ROW_SHR(8), 0xf);
+    CQ_MN(CQ_DPP_ROW_BCAST15, 0xa);
+    CQ_MN(CQ_DPP_ROW_BCAST31, 0xc);
+#undef CQ_MN
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
+// sums / maxima over aligned groups of 4 and 8 lanes, result in every lane of the group
+__device__ __forceinline__ int quad_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, CQ_DPP_QUAD_XOR1, 0xf, 0xf, true);
+    v += __builtin_amdgcn_update_dpp(0, v, CQ_DPP_QUAD_XOR2, 0xf, 0xf, true);
+    return v;
+}
+__device__ __forceinline__ int oct_sum(int v) {
+    v = quad_sum(v);
+    v += __builtin_amdgcn_update_dpp(0, v, CQ_DPP_ROW_HALF_MIRROR, 0xf, 0xf, true);
+    return v;
+}
+__device__ __forceinline__ float oct_max(float v) {
+#define CQ_MX(ctrl) v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true)))
+    CQ_MX(CQ_DPP_QUAD_XOR1);
+    CQ_MX(CQ_DPP_QUAD_XOR2);
+    CQ_MX(CQ_DPP_ROW_HALF_MIRROR);
+#undef CQ_MX
+    return v;
+}
+
 // wave64 butterfly sum; every lane ends with the total.
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -102,5 +157,18 @@ __host__ __device__ inline ActView cq_act_view(const void *scratch, int w_dtype,
     v.qs = (const int8_t *)(b + L.qs_off);
     v.d = (const float *)(b + L.d_off);
     v.bsums = (const int16_t *)(b + L.bs_off);
+    return v;
+}
+
+// The same view starting at activation row r0.
+__host__ __device__ inline ActView cq_act_view_rows(const ActView &av, int w_dtype, int64_t k, int64_t r0) {
+    ActView v = av;
+    v.qs = av.qs + r0 * k;
+    if (cq_is_kquant(w_dtype)) {
+        v.d = av.d + r0 * (k / 256);
+        v.bsums = av.bsums + r0 * (k / 16);
+    } else {
+        v.d = av.d + 2 * r0 * (k / 32);
+    }
     return v;
 }

@@ -1,137 +1,152 @@
 // Per-format "unit" decoding shared by the decode matvec and the expert-grouped MoE matvec.
 //
-// A row of W is cut into units — the bytes one lane consumes per step with 128-bit loads:
-//   Q4_K / Q5_K: one 16-byte slice of qs (8 per super-block) + the 16-byte block header
-//   Q6_K       : 16 `l` positions of one 128-element half (3 x 16 bytes, 4 per super-block)
+// A row of W is cut into units — what one lane consumes per step with 128-bit loads:
+//   Q4_K / Q5_K: one 64-element group g of a super-block (32 bytes of qs = two 16-byte loads, the
+//                matching qh bytes for Q5_K) + the 16-byte block header; 4 lanes per super-block
+//   Q6_K       : 16 `l` positions of one 128-element half (3 x 16 bytes); 4 lanes per super-block
 //   Q4_0 / Q8_0: one 32-element block
-// For each format Fmt<DT> gives the raw weight registers (W), the decoded weights (P), the
-// activation registers (A) and the exact integer dot product of one unit.
+// so a wave64 step covers 16 super-blocks (4096 elements) of a K-quant row or 64 blocks (2048
+// elements) of a Q4_0 / Q8_0 row.  For each format Fmt<DT> gives the raw weight registers (W), the
+// activation registers (A) and the dot product of one unit: exact integer arithmetic inside the
+// unit, one f32 scaling at the end, following the CPU vec_dot of
+// candle-core/src/quantized/k_quants.rs (Q4_0 :294-311, Q8_0 :720-738, Q4_K :1460-1540,
+// Q5_K :1714-1801, Q6_K :2035-2092).
 #pragma once
 #include "cq_device.h"
 
 namespace {
 
-// ---------------------------------------------------------------------------------------------
-// Per-format unit: weight registers (W), decoded weights (P), activation registers (A).
-// ---------------------------------------------------------------------------------------------
 template <int DT> struct Fmt;
 
-// ---- shared by Q4_K and Q5_K: 6-bit scale/min pair of sub-blocks 2g and 2g+1 -----------------
-// (vectorised form of get_scale_min_k4, k_quants.rs:1499-1509)
-__device__ __forceinline__ void k4_scales(uint32_t u0, uint32_t u1, uint32_t u2, int g, int &sc_lo, int &sc_hi, int &m_lo, int &m_hi) {
-    uint32_t sc4, m4;
-    if (g < 2) {
-        sc4 = u0 & 0x3f3f3f3fu;
-        m4 = u1 & 0x3f3f3f3fu;
+// Pointers to one quantized activation row (global scratch or its LDS copy).
+struct ActRow {
+    const int8_t *qs;       // [k]
+    const float *d;         // K-quants: [k/256];  Q4_0 / Q8_0: {d, sum} pairs [k/32][2]
+    const int16_t *bsums;   // K-quants: [k/16]
+};
+
+__device__ __forceinline__ ActRow act_row(const int8_t *qs, const float *d, const int16_t *bsums, int w_dtype, int64_t b, int k) {
+    ActRow r;
+    r.qs = qs + b * k;
+    if (cq_is_kquant(w_dtype)) {
+        r.d = d + b * (k >> 8);
+        r.bsums = bsums + b * (k >> 4);
     } else {
-        sc4 = (u2 & 0x0f0f0f0fu) | (((u0 >> 6) & 0x03030303u) << 4);
-        m4 = ((u2 >> 4) & 0x0f0f0f0fu) | (((u1 >> 6) & 0x03030303u) << 4);
+        r.d = d + 2 * b * (k >> 5);
+        r.bsums = bsums;
     }
-    int sh = (g & 1) * 16;
-    sc_lo = (sc4 >> sh) & 0xff;
-    sc_hi = (sc4 >> (sh + 8)) & 0xff;
-    m_lo = (m4 >> sh) & 0xff;
-    m_hi = (m4 >> (sh + 8)) & 0xff;
+    return r;
 }
 
-struct AK45 {   // activations for one Q4_K / Q5_K unit
-    u32x4 lo, hi;
+// ---- Q4_K / Q5_K common parts -------------------------------------------------------------------
+struct AK45 {   // activations of one 64-element group
+    u32x4 a0, a1, a2, a3;   // elements 0..15, 16..31 (sub-block 2g) and 32..47, 48..63 (sub-block 2g+1)
     float d8;
-    int bs_lo, bs_hi;
+    int bs_lo, bs_hi;       // sums of the two 32-element sub-blocks
 };
 
-struct PK45 {   // decoded Q4_K / Q5_K unit
-    uint32_t lo[4], hi[4];
-    float d, dmin;
-    int sc_lo, sc_hi, m_lo, m_hi;
-};
-
-__device__ __forceinline__ void load_act_k45(AK45 &a, const ActView &av, int64_t arow, int k, int u) {
-    int sb = u >> 3, j = u & 7, g = j >> 1, o = 16 * (j & 1);
-    const int8_t *q = av.qs + arow * k + sb * 256 + 64 * g + o;
-    a.lo = *reinterpret_cast<const u32x4 *>(q);
-    a.hi = *reinterpret_cast<const u32x4 *>(q + 32);
-    a.d8 = av.d[arow * (k >> 8) + sb];
-    const int16_t *bs = av.bsums + arow * (k >> 4) + sb * 16 + 4 * g + (j & 1);
-    a.bs_lo = bs[0];
-    a.bs_hi = bs[2];
+__device__ __forceinline__ void load_act_k45(AK45 &a, const ActRow &ar, int u) {
+    const int8_t *q = ar.qs + u * 64;
+    a.a0 = *reinterpret_cast<const u32x4 *>(q);
+    a.a1 = *reinterpret_cast<const u32x4 *>(q + 16);
+    a.a2 = *reinterpret_cast<const u32x4 *>(q + 32);
+    a.a3 = *reinterpret_cast<const u32x4 *>(q + 48);
+    a.d8 = ar.d[u >> 2];
+    u32x2 bs = *reinterpret_cast<const u32x2 *>(ar.bsums + u * 4);   // four 16-element sums
+    a.bs_lo = (int)(int16_t)(bs.x & 0xffff) + (int)(int16_t)(bs.x >> 16);
+    a.bs_hi = (int)(int16_t)(bs.y & 0xffff) + (int)(int16_t)(bs.y >> 16);
 }
 
-__device__ __forceinline__ float dot_k45(const PK45 &p, const AK45 &a, float acc) {
-    int dl = 0, dh = 0;
-    dl = sdot4(p.lo[0], a.lo.x, dl); dl = sdot4(p.lo[1], a.lo.y, dl);
-    dl = sdot4(p.lo[2], a.lo.z, dl); dl = sdot4(p.lo[3], a.lo.w, dl);
-    dh = sdot4(p.hi[0], a.hi.x, dh); dh = sdot4(p.hi[1], a.hi.y, dh);
-    dh = sdot4(p.hi[2], a.hi.z, dh); dh = sdot4(p.hi[3], a.hi.w, dh);
-    int S = p.sc_lo * dl + p.sc_hi * dh;
-    int M = p.m_lo * a.bs_lo + p.m_hi * a.bs_hi;
-    acc = fmaf(p.d * a.d8, (float)S, acc);
-    acc = fmaf(-(p.dmin * a.d8), (float)M, acc);
-    return acc;
+// 6-bit scales / mins of sub-blocks 2g and 2g+1 as bytes [sc_lo, sc_hi, m_lo, m_hi]
+// (get_scale_min_k4, candle-core/src/quantized/utils.rs:50-60, as two byte permutes).
+__device__ __forceinline__ uint32_t k4_scale_min(uint32_t u0, uint32_t u1, uint32_t u2, int g) {
+    // v_perm_b32(hi, lo, sel): selector bytes 0-3 pick from lo, 4-7 from hi
+    const uint32_t sel = (g & 1) ? 0x07060302u : 0x05040100u;        // [lo.b(2p), lo.b(2p+1), hi.b(2p), hi.b(2p+1)]
+    uint32_t A = __builtin_amdgcn_perm(u1, u0, sel);                 // [u0.b, u0.b', u1.b, u1.b']
+    uint32_t B = __builtin_amdgcn_perm(u2 >> 4, u2, sel) & 0x0f0f0f0fu;
+    const uint32_t lo = A & 0x3f3f3f3fu, hi = B | ((A >> 2) & 0x30303030u);
+    const uint32_t m = 0u - (uint32_t)(g >> 1);        // all ones for g >= 2: a bit blend, not a divergent branch
+    return (lo & ~m) | (hi & m);
+}
+
+__device__ __forceinline__ float finish_k45(uint32_t hdr0, uint32_t sm, int dl, int dh, const AK45 &a) {
+    int S = __mul24((int)(sm & 0xff), dl) + __mul24((int)((sm >> 8) & 0xff), dh);
+    int M = __mul24((int)((sm >> 16) & 0xff), a.bs_lo) + __mul24((int)(sm >> 24), a.bs_hi);
+    float d = h2f(hdr0), dmin = h2f(hdr0 >> 16);
+    return a.d8 * (d * (float)S - dmin * (float)M);
 }
 
 template <> struct Fmt<CQ_Q4K> {
-    static constexpr int UPB = 8;
-    struct W { u32x4 hdr, qs; };
-    typedef PK45 P;
+    static constexpr int UE = 64, UPB = 4;
+    struct W { u32x4 hdr, q0, q1; };
     typedef AK45 A;
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *blk = row + (int64_t)(u >> 3) * 144;
+        const uint8_t *blk = row + (u >> 2) * 144;
         w.hdr = *reinterpret_cast<const u32x4 *>(blk);
-        w.qs = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (u & 7));
+        w.q0 = *reinterpret_cast<const u32x4 *>(blk + 16 + 32 * (u & 3));
+        w.q1 = *reinterpret_cast<const u32x4 *>(blk + 32 + 32 * (u & 3));
     }
-    static __device__ __forceinline__ void prep(P &p, const W &w, int u) {
-        p.d = h2f(w.hdr.x);
-        p.dmin = h2f(w.hdr.x >> 16);
-        k4_scales(w.hdr.y, w.hdr.z, w.hdr.w, (u & 7) >> 1, p.sc_lo, p.sc_hi, p.m_lo, p.m_hi);
-        const uint32_t q[4] = {w.qs.x, w.qs.y, w.qs.z, w.qs.w};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            p.lo[i] = q[i] & 0x0f0f0f0fu;
-            p.hi[i] = (q[i] >> 4) & 0x0f0f0f0fu;
-        }
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_k45(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int u) {
+        uint32_t sm = k4_scale_min(w.hdr.y, w.hdr.z, w.hdr.w, u & 3);
+        const uint32_t M4 = 0x0f0f0f0fu;
+        int dl = 0, dh = 0;
+        dl = sdot4(w.q0.x & M4, a.a0.x, dl); dl = sdot4(w.q0.y & M4, a.a0.y, dl);
+        dl = sdot4(w.q0.z & M4, a.a0.z, dl); dl = sdot4(w.q0.w & M4, a.a0.w, dl);
+        dl = sdot4(w.q1.x & M4, a.a1.x, dl); dl = sdot4(w.q1.y & M4, a.a1.y, dl);
+        dl = sdot4(w.q1.z & M4, a.a1.z, dl); dl = sdot4(w.q1.w & M4, a.a1.w, dl);
+        dh = sdot4((w.q0.x >> 4) & M4, a.a2.x, dh); dh = sdot4((w.q0.y >> 4) & M4, a.a2.y, dh);
+        dh = sdot4((w.q0.z >> 4) & M4, a.a2.z, dh); dh = sdot4((w.q0.w >> 4) & M4, a.a2.w, dh);
+        dh = sdot4((w.q1.x >> 4) & M4, a.a3.x, dh); dh = sdot4((w.q1.y >> 4) & M4, a.a3.y, dh);
+        dh = sdot4((w.q1.z >> 4) & M4, a.a3.z, dh); dh = sdot4((w.q1.w >> 4) & M4, a.a3.w, dh);
+        return finish_k45(w.hdr.x, sm, dl, dh, a);
     }
-    static __device__ __forceinline__ void load_a(A &a, const ActView &av, int64_t arow, int k, int u) { load_act_k45(a, av, arow, k, u); }
-    static __device__ __forceinline__ float dot(const P &p, const A &a, float acc) { return dot_k45(p, a, acc); }
 };
 
 template <> struct Fmt<CQ_Q5K> {
-    static constexpr int UPB = 8;
-    struct W { u32x4 hdr, qh, qs; };
-    typedef PK45 P;
+    static constexpr int UE = 64, UPB = 4;
+    struct W { u32x4 hdr, h0, h1, q0, q1; };
     typedef AK45 A;
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *blk = row + (int64_t)(u >> 3) * 176;
-        int j = u & 7;
+        const uint8_t *blk = row + (u >> 2) * 176;
         w.hdr = *reinterpret_cast<const u32x4 *>(blk);
-        w.qh = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (j & 1));
-        w.qs = *reinterpret_cast<const u32x4 *>(blk + 48 + 16 * j);
+        w.h0 = *reinterpret_cast<const u32x4 *>(blk + 16);          // qh[0..15]
+        w.h1 = *reinterpret_cast<const u32x4 *>(blk + 32);          // qh[16..31]
+        w.q0 = *reinterpret_cast<const u32x4 *>(blk + 48 + 32 * (u & 3));
+        w.q1 = *reinterpret_cast<const u32x4 *>(blk + 64 + 32 * (u & 3));
     }
-    static __device__ __forceinline__ void prep(P &p, const W &w, int u) {
-        int g = (u & 7) >> 1;
-        p.d = h2f(w.hdr.x);
-        p.dmin = h2f(w.hdr.x >> 16);
-        k4_scales(w.hdr.y, w.hdr.z, w.hdr.w, g, p.sc_lo, p.sc_hi, p.m_lo, p.m_hi);
-        const uint32_t q[4] = {w.qs.x, w.qs.y, w.qs.z, w.qs.w};
-        const uint32_t h[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_k45(a, ar, u); }
+    // one dword of qs + its qh dword -> unsigned 5-bit values of sub-block 2g (lo) and 2g+1 (hi)
+    static __device__ __forceinline__ void unpack(uint32_t q, uint32_t h, int g, uint32_t &lo, uint32_t &hi) {
+        uint32_t hb = h >> (2 * g);
+        lo = (q & 0x0f0f0f0fu) | ((hb & 0x01010101u) << 4);
+        hi = ((q >> 4) & 0x0f0f0f0fu) | ((hb << 3) & 0x10101010u);
+    }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int u) {
+        const int g = u & 3;
+        uint32_t sm = k4_scale_min(w.hdr.y, w.hdr.z, w.hdr.w, g);
+        const uint32_t q[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
+        const uint32_t h[8] = {w.h0.x, w.h0.y, w.h0.z, w.h0.w, w.h1.x, w.h1.y, w.h1.z, w.h1.w};
+        const uint32_t al[8] = {a.a0.x, a.a0.y, a.a0.z, a.a0.w, a.a1.x, a.a1.y, a.a1.z, a.a1.w};
+        const uint32_t ah[8] = {a.a2.x, a.a2.y, a.a2.z, a.a2.w, a.a3.x, a.a3.y, a.a3.z, a.a3.w};
+        int dl = 0, dh = 0;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            uint32_t hb = h[i] >> (2 * g);
-            p.lo[i] = (q[i] & 0x0f0f0f0fu) | ((hb & 0x01010101u) << 4);
-            p.hi[i] = ((q[i] >> 4) & 0x0f0f0f0fu) | (((hb >> 1) & 0x01010101u) << 4);
+        for (int i = 0; i < 8; i++) {
+            uint32_t lo, hi;
+            unpack(q[i], h[i], g, lo, hi);
+            dl = sdot4(lo, al[i], dl);
+            dh = sdot4(hi, ah[i], dh);
         }
+        return finish_k45(w.hdr.x, sm, dl, dh, a);
     }
-    static __device__ __forceinline__ void load_a(A &a, const ActView &av, int64_t arow, int k, int u) { load_act_k45(a, av, arow, k, u); }
-    static __device__ __forceinline__ float dot(const P &p, const A &a, float acc) { return dot_k45(p, a, acc); }
 };
 
 template <> struct Fmt<CQ_Q6K> {
-    static constexpr int UPB = 4;
+    static constexpr int UE = 64, UPB = 4;
     struct W { u32x4 qa, qb, qh; u32x2 sc; uint32_t d; };
-    struct P { uint32_t q[4][4]; int sc[4]; float d; };
     struct A { u32x4 a[4]; int bs[4]; float d8; };
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *blk = row + (int64_t)(u >> 2) * 210;
+        const uint8_t *blk = row + (u >> 2) * 210;
         int h = (u >> 1) & 1, c = u & 1;
         w.qa = ld_u<u32x4>(blk + 64 * h + 16 * c);          // ql[l], l = 16c..16c+15 of this half
         w.qb = ld_u<u32x4>(blk + 64 * h + 32 + 16 * c);     // ql[l + 32]
@@ -139,48 +154,42 @@ template <> struct Fmt<CQ_Q6K> {
         w.sc = ld_u<u32x2>(blk + 192 + 8 * h);              // the 8 scales of this half
         w.d = ld_u<uint16_t>(blk + 208);
     }
-    static __device__ __forceinline__ void prep(P &p, const W &w, int u) {
-        int c = u & 1;
-        p.d = h2f(w.d);
-        // quarter i of the half uses scale index c + 2i (k_quants.rs:2265-2274)
-        uint32_t s0 = w.sc.x >> (8 * c), s1 = w.sc.y >> (8 * c);
-        p.sc[0] = (int)(int8_t)(s0 & 0xff);
-        p.sc[1] = (int)(int8_t)((s0 >> 16) & 0xff);
-        p.sc[2] = (int)(int8_t)(s1 & 0xff);
-        p.sc[3] = (int)(int8_t)((s1 >> 16) & 0xff);
-        const uint32_t a[4] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w};
-        const uint32_t b[4] = {w.qb.x, w.qb.y, w.qb.z, w.qb.w};
-        const uint32_t h[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {   // unsigned 6-bit values; the -32 is applied through bsums
-            p.q[0][i] = (a[i] & 0x0f0f0f0fu) | ((h[i] & 0x03030303u) << 4);
-            p.q[1][i] = (b[i] & 0x0f0f0f0fu) | (((h[i] >> 2) & 0x03030303u) << 4);
-            p.q[2][i] = ((a[i] >> 4) & 0x0f0f0f0fu) | (((h[i] >> 4) & 0x03030303u) << 4);
-            p.q[3][i] = ((b[i] >> 4) & 0x0f0f0f0fu) | (((h[i] >> 6) & 0x03030303u) << 4);
-        }
-    }
-    static __device__ __forceinline__ void load_a(A &a, const ActView &av, int64_t arow, int k, int u) {
+    // unit (h, c) covers elements 128h + 32i + 16c + [0,16) for the four quarters i (k_quants.rs:2265-2274)
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) {
         int sb = u >> 2, h = (u >> 1) & 1, c = u & 1;
-        const int8_t *q = av.qs + arow * k + sb * 256 + 128 * h + 16 * c;
+        const int8_t *q = ar.qs + sb * 256 + 128 * h + 16 * c;
 #pragma unroll
         for (int i = 0; i < 4; i++) a.a[i] = *reinterpret_cast<const u32x4 *>(q + 32 * i);
         // 16-element sums of quarters 0..3 at index 8h + 2i + c
-        u32x4 bs = *reinterpret_cast<const u32x4 *>(av.bsums + arow * (k >> 4) + sb * 16 + 8 * h);
+        u32x4 bs = *reinterpret_cast<const u32x4 *>(ar.bsums + sb * 16 + 8 * h);
         const uint32_t b4[4] = {bs.x, bs.y, bs.z, bs.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) a.bs[i] = (int)(int16_t)((b4[i] >> (16 * c)) & 0xffff);
-        a.d8 = av.d[arow * (k >> 8) + sb];
+        a.d8 = ar.d[sb];
     }
-    static __device__ __forceinline__ float dot(const P &p, const A &a, float acc) {
-        int S = 0;
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int u) {
+        const int c = u & 1;
+        // quarter i uses scale index c + 2i of the half
+        uint32_t s0 = w.sc.x >> (8 * c), s1 = w.sc.y >> (8 * c);
+        const int sc[4] = {(int)(int8_t)(s0 & 0xff), (int)(int8_t)((s0 >> 16) & 0xff), (int)(int8_t)(s1 & 0xff), (int)(int8_t)((s1 >> 16) & 0xff)};
+        const uint32_t qa[4] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w};
+        const uint32_t qb[4] = {w.qb.x, w.qb.y, w.qb.z, w.qb.w};
+        const uint32_t qh[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
+        // unsigned 6-bit values; the -32 offset is applied through the 16-element sums
+        int dq[4] = {-32 * a.bs[0], -32 * a.bs[1], -32 * a.bs[2], -32 * a.bs[3]};
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int dq = -32 * a.bs[i];
-            dq = sdot4(p.q[i][0], a.a[i].x, dq); dq = sdot4(p.q[i][1], a.a[i].y, dq);
-            dq = sdot4(p.q[i][2], a.a[i].z, dq); dq = sdot4(p.q[i][3], a.a[i].w, dq);
-            S += p.sc[i] * dq;
+        for (int j = 0; j < 4; j++) {
+            const uint32_t A0[4] = {a.a[0].x, a.a[0].y, a.a[0].z, a.a[0].w};
+            const uint32_t A1[4] = {a.a[1].x, a.a[1].y, a.a[1].z, a.a[1].w};
+            const uint32_t A2[4] = {a.a[2].x, a.a[2].y, a.a[2].z, a.a[2].w};
+            const uint32_t A3[4] = {a.a[3].x, a.a[3].y, a.a[3].z, a.a[3].w};
+            dq[0] = sdot4((qa[j] & 0x0f0f0f0fu) | ((qh[j] << 4) & 0x30303030u), A0[j], dq[0]);
+            dq[1] = sdot4((qb[j] & 0x0f0f0f0fu) | ((qh[j] << 2) & 0x30303030u), A1[j], dq[1]);
+            dq[2] = sdot4(((qa[j] >> 4) & 0x0f0f0f0fu) | (qh[j] & 0x30303030u), A2[j], dq[2]);
+            dq[3] = sdot4(((qb[j] >> 4) & 0x0f0f0f0fu) | ((qh[j] >> 2) & 0x30303030u), A3[j], dq[3]);
         }
-        return fmaf(p.d * a.d8, (float)S, acc);
+        int S = __mul24(sc[0], dq[0]) + __mul24(sc[1], dq[1]) + __mul24(sc[2], dq[2]) + __mul24(sc[3], dq[3]);
+        return (h2f(w.d) * a.d8) * (float)S;
     }
 };
 
@@ -191,71 +200,71 @@ struct A0 {
     int s8;
 };
 
-__device__ __forceinline__ void load_act_q0(A0 &a, const ActView &av, int64_t arow, int k, int u) {
-    const int8_t *q = av.qs + arow * k + u * 32;
+__device__ __forceinline__ void load_act_q0(A0 &a, const ActRow &ar, int u) {
+    const int8_t *q = ar.qs + u * 32;
     a.a0 = *reinterpret_cast<const u32x4 *>(q);
     a.a1 = *reinterpret_cast<const u32x4 *>(q + 16);
-    u32x2 ds = *reinterpret_cast<const u32x2 *>(av.d + 2 * (arow * (k >> 5) + u));
+    u32x2 ds = *reinterpret_cast<const u32x2 *>(ar.d + 2 * u);
     a.d8 = __uint_as_float(ds.x);
     a.s8 = (int)ds.y;
 }
 
 template <> struct Fmt<CQ_Q4_0> {
-    static constexpr int UPB = 1;
+    static constexpr int UE = 32, UPB = 1;
     struct W { u32x4 qs; uint32_t d; };
-    struct P { uint32_t lo[4], hi[4]; float d; };
     typedef A0 A;
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *blk = row + (int64_t)u * 18;
+        const uint8_t *blk = row + u * 18;
         w.d = ld_u<uint16_t>(blk);
         w.qs = ld_u<u32x4>(blk + 2);
     }
-    static __device__ __forceinline__ void prep(P &p, const W &w, int) {
-        p.d = h2f(w.d);
-        const uint32_t q[4] = {w.qs.x, w.qs.y, w.qs.z, w.qs.w};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            p.lo[i] = q[i] & 0x0f0f0f0fu;          // elements 4i..4i+3
-            p.hi[i] = (q[i] >> 4) & 0x0f0f0f0fu;   // elements 16+4i..
-        }
-    }
-    static __device__ __forceinline__ void load_a(A &a, const ActView &av, int64_t arow, int k, int u) { load_act_q0(a, av, arow, k, u); }
-    static __device__ __forceinline__ float dot(const P &p, const A &a, float acc) {
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
+        const uint32_t M4 = 0x0f0f0f0fu;
         int s = -8 * a.s8;    // sum((q - 8) * y) = sum(q * y) - 8 * sum(y)
-        s = sdot4(p.lo[0], a.a0.x, s); s = sdot4(p.lo[1], a.a0.y, s);
-        s = sdot4(p.lo[2], a.a0.z, s); s = sdot4(p.lo[3], a.a0.w, s);
-        s = sdot4(p.hi[0], a.a1.x, s); s = sdot4(p.hi[1], a.a1.y, s);
-        s = sdot4(p.hi[2], a.a1.z, s); s = sdot4(p.hi[3], a.a1.w, s);
-        return acc + (float)s * p.d * a.d8;
+        s = sdot4(w.qs.x & M4, a.a0.x, s); s = sdot4(w.qs.y & M4, a.a0.y, s);
+        s = sdot4(w.qs.z & M4, a.a0.z, s); s = sdot4(w.qs.w & M4, a.a0.w, s);
+        s = sdot4((w.qs.x >> 4) & M4, a.a1.x, s); s = sdot4((w.qs.y >> 4) & M4, a.a1.y, s);
+        s = sdot4((w.qs.z >> 4) & M4, a.a1.z, s); s = sdot4((w.qs.w >> 4) & M4, a.a1.w, s);
+        return (float)s * h2f(w.d) * a.d8;
     }
 };
 
 template <> struct Fmt<CQ_Q8_0> {
-    static constexpr int UPB = 1;
+    static constexpr int UE = 32, UPB = 1;
     struct W { u32x4 q0, q1; uint32_t d; };
-    struct P { u32x4 q0, q1; float d; };
     typedef A0 A;
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *blk = row + (int64_t)u * 34;
+        const uint8_t *blk = row + u * 34;
         w.d = ld_u<uint16_t>(blk);
         w.q0 = ld_u<u32x4>(blk + 2);
         w.q1 = ld_u<u32x4>(blk + 18);
     }
-    static __device__ __forceinline__ void prep(P &p, const W &w, int) {
-        p.d = h2f(w.d);
-        p.q0 = w.q0;
-        p.q1 = w.q1;
-    }
-    static __device__ __forceinline__ void load_a(A &a, const ActView &av, int64_t arow, int k, int u) { load_act_q0(a, av, arow, k, u); }
-    static __device__ __forceinline__ float dot(const P &p, const A &a, float acc) {
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
         int s = 0;
-        s = sdot4(p.q0.x, a.a0.x, s); s = sdot4(p.q0.y, a.a0.y, s);
-        s = sdot4(p.q0.z, a.a0.z, s); s = sdot4(p.q0.w, a.a0.w, s);
-        s = sdot4(p.q1.x, a.a1.x, s); s = sdot4(p.q1.y, a.a1.y, s);
-        s = sdot4(p.q1.z, a.a1.z, s); s = sdot4(p.q1.w, a.a1.w, s);
-        return acc + (float)s * p.d * a.d8;
+        s = sdot4(w.q0.x, a.a0.x, s); s = sdot4(w.q0.y, a.a0.y, s);
+        s = sdot4(w.q0.z, a.a0.z, s); s = sdot4(w.q0.w, a.a0.w, s);
+        s = sdot4(w.q1.x, a.a1.x, s); s = sdot4(w.q1.y, a.a1.y, s);
+        s = sdot4(w.q1.z, a.a1.z, s); s = sdot4(w.q1.w, a.a1.w, s);
+        return (float)s * h2f(w.d) * a.d8;
     }
 };
+
+// ---------------------------------------------------------------------------------------------
+// wave64 sum through DPP row shifts and row broadcasts; the total ends up in lane 63.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+#define CQ_DPP(ctrl, rmask, bc) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, rmask, 0xf, bc))
+    v += CQ_DPP(0x111, 0xf, true);     // row_shr:1
+    v += CQ_DPP(0x112, 0xf, true);     // row_shr:2
+    v += CQ_DPP(0x114, 0xf, true);     // row_shr:4
+    v += CQ_DPP(0x118, 0xf, true);     // row_shr:8   -> lane 15 of each row holds the row sum
+    v += CQ_DPP(0x142, 0xa, false);    // row_bcast:15 into rows 1 and 3
+    v += CQ_DPP(0x143, 0xc, false);    // row_bcast:31 into rows 2 and 3 -> lane 63 holds the total
+#undef CQ_DPP
+    return v;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Output conversion (the CUDA backend keeps the activation dtype; the CPU f16 path rounds the f32

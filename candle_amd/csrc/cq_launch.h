@@ -11,6 +11,9 @@ int cq_matvec_launch(int w_dtype, const void *w, const void *scratch, void *dst,
 // same, over an already resolved (possibly row-offset) view of the activation scratch
 int cq_matvec_launch_av(int w_dtype, const void *w, const ActView &av, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
                         int64_t stride_dst, hipStream_t s);
+// QMatMul::forward for <= CQ_MATVEC_MAX_ROWS rows with the activation quantization fused into the matvec kernel
+int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *dst, int dst_dtype, int64_t k, int64_t n,
+                           int64_t rows, int64_t stride_dst, hipStream_t s);
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s);
 int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t count, hipStream_t s);

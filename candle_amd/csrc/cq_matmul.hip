@@ -34,14 +34,7 @@ int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst
     ActView av = cq_act_view(scratch, w_dtype, k, rows);
     for (int64_t r0 = 0; r0 < rows; r0 += CQ_MATVEC_MAX_ROWS) {
         int64_t nb = rows - r0 < CQ_MATVEC_MAX_ROWS ? rows - r0 : CQ_MATVEC_MAX_ROWS;
-        ActView c = av;
-        c.qs = av.qs + r0 * k;
-        if (cq_is_kquant(w_dtype)) {
-            c.d = av.d + r0 * (k / 256);
-            c.bsums = av.bsums + r0 * (k / 16);
-        } else {
-            c.d = av.d + 2 * r0 * (k / 32);
-        }
+        ActView c = cq_act_view_rows(av, w_dtype, k, r0);
         int rc = cq_matvec_launch_av(w_dtype, w, c, dst + r0 * stride_dst, CQ_F32, k, n, nb, stride_dst, s);
         if (rc) return rc;
     }

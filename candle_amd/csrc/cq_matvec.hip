@@ -1,96 +1,295 @@
 // Decode matvec for gfx950:  dst[b, row] = sum_k W[row, k] * x^[b, k]   (b < NB <= 8)
 //
-// W is streamed once from HBM in its GGUF block layout; x^ is the int8-quantized activation scratch
-// written by the act-quant kernels (bit-identical to candle's CPU quantization), so the integer part
-// of every dot product is exact and only the f32 summation order differs from
-// k_quants::matmul (candle-core/src/quantized/k_quants.rs:2375-2492) and its vec_dot kernels
-// (Q4_0 :294-311, Q8_0 :720-738, Q4_K :1460-1540, Q5_K :1714-1801, Q6_K :2035-2092).
+// W is streamed once from HBM in its GGUF block layout; x^ is the int8 quantization of the
+// activations, bit-identical to candle's CPU quantization, so the integer part of every dot product is
+// exact and only the f32 summation order differs from k_quants::matmul
+// (candle-core/src/quantized/k_quants.rs:2375-2492).
 //
-// Work split: a row of W is cut into "units" — the bytes one lane consumes per step with 128-bit
-// loads.  Lane l of a wave takes units l, l+64, ... of R consecutive rows, so the activation
-// registers are reused across the R rows and the weight registers across the NB activation rows.
-//   Q4_K / Q5_K: unit = one 16-byte slice of qs (8 per super-block) + the 16-byte block header
-//   Q6_K       : unit = 16 `l` positions of one 128-element half (3 x 16 bytes, 4 per super-block)
-//   Q4_0 / Q8_0: unit = one 32-element block
-// Packed int8 dot products use v_dot4_i32_i8; wave64 butterflies reduce the per-lane partial sums.
+// One kernel does the whole QMatMul::forward for a decode step:
+//   1. every wave issues the 128-bit loads of its first row of W;
+//   2. the workgroup quantizes the NB activation rows into LDS (Q8_K or Q8_0 blocks, one wave per
+//      256-element span) — or copies an already quantized scratch buffer into LDS;
+//   3. each wave walks its rows (row = first + wave, + waves, ...): lane l takes units l, l+64, ... of
+//      the row (see cq_fmt.h), the next step's weights are in flight while the current one is reduced
+//      with v_dot4_i32_i8, and a DPP wave reduction leaves the row result in lane 63.
+// When a row is a single wave step (K = 4096 for K-quants) the activation registers are loaded from
+// LDS once and reused for every row.
+//
+// The grid is one workgroup of up to 16 waves per CU (256 CUs): waves live long enough to amortize
+// the activation quantization, and all of a CU's weight loads are in flight from the first cycle.
+#include "cq_actquant.h"
 #include "cq_device.h"
 #include "cq_fmt.h"
 #include "cq_launch.h"
 
 namespace {
 
-// ---------------------------------------------------------------------------------------------
-// The kernel: 4 waves per workgroup, each wave owns R consecutive rows.
-// ---------------------------------------------------------------------------------------------
-template <int DT, int NB, int R>
-__global__ __launch_bounds__(256) void matvec_kernel(const uint8_t *__restrict__ w, ActView av, void *__restrict__ dst,
-                                                     int dst_dtype, int k, int n, int64_t stride_dst) {
+constexpr int SRC_SCRATCH = -1;   // activations come pre-quantized (cq_quantize_act); otherwise SRC is the x dtype
+constexpr int64_t LDS_BUDGET = 160 * 1024 - 1024;
+
+struct ActSrc {
+    const void *x;   // fused: [NB, k] activations
+    ActView av;      // pre-quantized: section pointers of the scratch buffer (possibly row-offset)
+};
+
+// Launch geometry, computed once on the host so the kernel prologue is a handful of scalar loads
+// instead of 64-bit divisions and multiplications in front of the first memory access.
+struct QmvGeom {
+    int k, n, rows_per_wg;
+    int units, steps;          // units per row, wave steps per row
+    int lds_d_off, lds_bs_off; // LDS sections (the scratch layout for NB rows)
+    int nw_shift;              // log2(waves per workgroup)
+    int row_bytes;             // bytes of one row of W
+    int dst_dtype;
+    int64_t stride_dst;
+};
+
+template <int DT, int NB, int SRC, bool SINGLE>
+__global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g) {
     typedef Fmt<DT> F;
-    const int lane = threadIdx.x & 63;
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * R;
-    if (row0 >= n) return;
-    const int nblk = k / BlockInfo<DT>::elems;
-    const int units = nblk * F::UPB;
-    const int64_t row_bytes = (int64_t)nblk * BlockInfo<DT>::bytes;
+    constexpr bool FUSED = SRC != SRC_SCRATCH;
+    constexpr int XDT = FUSED ? SRC : CQ_F32;
+    extern __shared__ __align__(16) uint8_t lds[];
+    int8_t *lqs = (int8_t *)lds;
+    float *ld = (float *)(lds + g.lds_d_off);
+    int16_t *lbs = (int16_t *)(lds + g.lds_bs_off);
 
-    float acc[R][NB];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int b = 0; b < NB; b++) acc[r][b] = 0.0f;
+    const int k = g.k, n = g.n, dst_dtype = g.dst_dtype;
+    const int64_t stride_dst = g.stride_dst;
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int lane = tid & 63;
+    const int wv = tid >> 6;
+    const int nwaves = 1 << g.nw_shift;
+    const int units = g.units;
+    const int steps = g.steps;
+    const int row_bytes = g.row_bytes;
+    const int wave_stride = row_bytes << g.nw_shift;
+    const int wg_row0 = blockIdx.x * g.rows_per_wg;
+    const int wg_row1 = min(n, wg_row0 + g.rows_per_wg);
 
-    for (int u = lane; u < units; u += CQ_WAVE) {
-        typename F::W wr[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            int64_t row = row0 + r < n ? row0 + r : n - 1;   // tail rows re-read the last row, never stored
-            F::load_w(wr[r], w + row * row_bytes, u);
-        }
-        typename F::A ar[NB];
-#pragma unroll
-        for (int b = 0; b < NB; b++) F::load_a(ar[b], av, b, k, u);
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            typename F::P p;
-            F::prep(p, wr[r], u);
-#pragma unroll
-            for (int b = 0; b < NB; b++) acc[r][b] = F::dot(p, ar[b], acc[r][b]);
+    // 0. The activation loads go out first.  Vector loads complete in order, so anything issued after
+    //    the weight loads below could only be consumed once the (slow, HBM) weights have arrived.
+    const int total = NB * k;                 // elements of x
+    float xv[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // fused: this wave's first 256-element span
+    const int xbase = wv * 256 + lane * 4;
+    u32x4 c_qs = {0, 0, 0, 0};                // pre-quantized: first round of the scratch -> LDS copy
+    u32x2 c_d = {0, 0};
+    uint32_t c_bs = 0;
+    if (FUSED) {
+        if (xbase < total) cq_load4<XDT>(src.x, xbase, xv);
+    } else {
+        if (tid < (total >> 4)) c_qs = ((const u32x4 *)src.av.qs)[tid];
+        if (cq_is_kquant(DT)) {
+            if (tid < NB * (k >> 8)) c_d.x = __float_as_uint(src.av.d[tid]);
+            if (tid < (NB * (k >> 4)) >> 1) c_bs = ((const uint32_t *)src.av.bsums)[tid];
+        } else {
+            if (tid < NB * (k >> 5)) c_d = ((const u32x2 *)src.av.d)[tid];
         }
     }
 
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            float v = wave_sum(acc[r][b]);
-            if (lane == 0 && row0 + r < n) store_out(dst, dst_dtype, (int64_t)b * stride_dst + row0 + r, v);
+    // 1. first weights in flight.  The load is unconditional (idle waves re-read the last row) so that
+    //    the compiler can wait for the activation load alone and leave these in flight.
+    const int wv_s = __builtin_amdgcn_readfirstlane(wv);
+    int row = wg_row0 + wv_s;
+    // rows this wave owns (the wave count is a power of two: a shift, not an integer division)
+    const int my_rows = row < wg_row1 ? (wg_row1 - row + nwaves - 1) >> g.nw_shift : 0;
+    const uint8_t *wp = w + (int64_t)min(row, n - 1) * (int64_t)row_bytes;
+    const int u0 = min(lane, units - 1);
+    typename F::W wa, wb;
+    F::load_w(wa, wp, u0);
+
+    // 2. activations -> LDS
+    if (FUSED) {
+        // The first span is peeled out of the loop on purpose: its values are already in xv, and as
+        // straight-line code the compiler waits for that one load only (vmcnt = the weight loads still
+        // in flight).  Inside a loop it would wait for everything, i.e. for the weights, and the
+        // quantization latency would no longer hide behind the HBM fetch.
+        const int spans = (total + 255) >> 8;
+        if (wv_s < spans) {
+            if (cq_is_kquant(DT))
+                cq_quantize_q8k_vals(xv, wv_s, lane, lqs, ld, lbs);
+            else
+                cq_quantize_q80_vals(xv, xbase < total, xbase, lane, lqs, ld);
         }
+        for (int span = wv_s + nwaves; span < spans; span += nwaves) {
+            if (cq_is_kquant(DT))
+                cq_quantize_q8k_span<XDT>(src.x, span, lane, lqs, ld, lbs);
+            else
+                cq_quantize_q80_span<XDT>(src.x, span, lane, total, lqs, ld);
+        }
+    } else {
+        if (tid < (total >> 4)) ((u32x4 *)lqs)[tid] = c_qs;
+        for (int i = tid + nthr; i < total >> 4; i += nthr) ((u32x4 *)lqs)[i] = ((const u32x4 *)src.av.qs)[i];
+        if (cq_is_kquant(DT)) {
+            if (tid < NB * (k >> 8)) ld[tid] = __uint_as_float(c_d.x);
+            for (int i = tid + nthr; i < NB * (k >> 8); i += nthr) ld[i] = src.av.d[i];
+            if (tid < (NB * (k >> 4)) >> 1) ((uint32_t *)lbs)[tid] = c_bs;
+            for (int i = tid + nthr; i < (NB * (k >> 4)) >> 1; i += nthr) ((uint32_t *)lbs)[i] = ((const uint32_t *)src.av.bsums)[i];
+        } else {
+            if (tid < NB * (k >> 5)) ((u32x2 *)ld)[tid] = c_d;
+            for (int i = tid + nthr; i < NB * (k >> 5); i += nthr) ((u32x2 *)ld)[i] = ((const u32x2 *)src.av.d)[i];
+        }
+    }
+    __syncthreads();
+    if (my_rows == 0) return;
+
+    ActRow ar[NB];
+#pragma unroll
+    for (int b = 0; b < NB; b++) ar[b] = act_row(lqs, ld, lbs, DT, b, k);
+
+    if (SINGLE) {
+        // A row is one wave step: lane l always works on unit l.  With few activation rows their
+        // registers are loaded from LDS once and reused for every row of W.
+        constexpr bool CACHE = NB <= 2;
+        const bool valid = lane < units;
+        typename F::A areg[NB];
+        if (CACHE) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) F::load_a(areg[b], ar[b], u0);
+        }
+        auto one_row = [&](const typename F::W &cur, int r) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                if (!CACHE) F::load_a(areg[b], ar[b], u0);
+                float v = F::dot(cur, areg[b], u0);
+                v = wave_sum_to_lane63(valid ? v : 0.0f);
+                if (lane == 63) store_out(dst, dst_dtype, (int64_t)b * stride_dst + r, v);
+            }
+        };
+        // ping-pong between wa and wb: the next row's loads are in flight while this one is reduced;
+        // the prefetch past the last row re-reads it instead of branching around the load
+        for (int j = 0; j < my_rows; j += 2) {
+            const uint8_t *p1 = j + 1 < my_rows ? wp + wave_stride : wp;
+            F::load_w(wb, p1, u0);
+            one_row(wa, row);
+            if (j + 1 >= my_rows) break;
+            const uint8_t *p2 = j + 2 < my_rows ? p1 + wave_stride : p1;
+            F::load_w(wa, p2, u0);
+            one_row(wb, row + nwaves);
+            row += 2 * nwaves;
+            wp = p2;
+        }
+    } else {
+        // General walk over (row, step), unrolled by two for the same ping-pong.
+        typename F::A areg[NB];
+        float acc[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) acc[b] = 0.0f;
+        const int total_steps = my_rows * steps;
+        int i = 0;
+        auto one_step = [&](const typename F::W &cur, typename F::W &nxt, int t) {
+            // next (row, step); past the end the last unit is re-read
+            int ni = i + 1;
+            const uint8_t *nwp = wp;
+            if (ni == steps) { ni = 0; nwp = wp + wave_stride; }
+            if (t + 1 >= total_steps) { ni = i; nwp = wp; }
+            F::load_w(nxt, nwp, min(lane + 64 * ni, units - 1));
+            const int u = lane + 64 * i;
+            const bool valid = u < units;
+            const int uc = valid ? u : units - 1;
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                F::load_a(areg[b], ar[b], uc);
+                float v = F::dot(cur, areg[b], uc);
+                acc[b] += valid ? v : 0.0f;
+            }
+            if (i == steps - 1) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    float r = wave_sum_to_lane63(acc[b]);
+                    if (lane == 63) store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, r);
+                    acc[b] = 0.0f;
+                }
+                row += nwaves;
+            }
+            i = ni;
+            wp = nwp;
+        };
+        for (int t = 0; t < total_steps; t += 2) {
+            one_step(wa, wb, t);
+            if (t + 1 >= total_steps) break;
+            one_step(wb, wa, t + 1);
+        }
+    }
 }
 
-template <int DT, int NB>
-int launch_nb(const void *w, const ActView &av, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
-    constexpr int R = NB <= 2 ? 2 : 1;
-    int64_t grid = (n + 4 * R - 1) / (4 * R);
-    if (grid > 0x7fffffffLL) return CQ_ERR_RANGE;
-    hipLaunchKernelGGL((matvec_kernel<DT, NB, R>), dim3((unsigned)grid), dim3(256), 0, s, (const uint8_t *)w, av, dst, dst_dtype,
-                       (int)k, (int)n, stride_dst);
+template <int DT, int NB, int SRC, bool SINGLE>
+int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
+    // waves per workgroup: as many as still leave every wave a row when 256 workgroups are launched
+    int waves = 16;
+    while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
+    int64_t groups = n >= 256 * (int64_t)waves ? 256 : (n + waves - 1) / waves;
+    int64_t rows_per_wg = (n + groups - 1) / groups;
+    groups = (n + rows_per_wg - 1) / rows_per_wg;
+    const ActLayout L = cq_act_layout(DT, k, NB);
+    size_t lds_bytes = (size_t)L.total;
+    QmvGeom g;
+    g.k = (int)k; g.n = (int)n; g.rows_per_wg = (int)rows_per_wg;
+    g.units = (int)(k / Fmt<DT>::UE); g.steps = (g.units + 63) >> 6;
+    g.lds_d_off = (int)L.d_off; g.lds_bs_off = (int)L.bs_off;
+    g.nw_shift = 0;
+    while ((1 << g.nw_shift) < waves) g.nw_shift++;
+    int64_t rb = (k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
+    if (rb > 0x3fffffff) return CQ_ERR_RANGE;
+    g.row_bytes = (int)rb;
+    g.dst_dtype = dst_dtype; g.stride_dst = stride_dst;
+    auto kern = qmv_kernel<DT, NB, SRC, SINGLE>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * waves), lds_bytes, s, (const uint8_t *)w, src, dst, g);
     return (int)hipGetLastError();
 }
 
-template <int DT>
-int launch_dt(const void *w, const ActView &av, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst,
-              hipStream_t s) {
+template <int DT, int NB, int SRC>
+int launch_nb(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
+    if (k / Fmt<DT>::UE <= 64) return launch_cfg<DT, NB, SRC, true>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+    return launch_cfg<DT, NB, SRC, false>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+}
+
+template <int DT, int SRC>
+int launch_rows(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst,
+                hipStream_t s) {
     switch (rows) {
-        case 1: return launch_nb<DT, 1>(w, av, dst, dst_dtype, k, n, stride_dst, s);
-        case 2: return launch_nb<DT, 2>(w, av, dst, dst_dtype, k, n, stride_dst, s);
-        case 3: return launch_nb<DT, 3>(w, av, dst, dst_dtype, k, n, stride_dst, s);
-        case 4: return launch_nb<DT, 4>(w, av, dst, dst_dtype, k, n, stride_dst, s);
-        case 5: return launch_nb<DT, 5>(w, av, dst, dst_dtype, k, n, stride_dst, s);
-        case 6: return launch_nb<DT, 6>(w, av, dst, dst_dtype, k, n, stride_dst, s);
-        case 7: return launch_nb<DT, 7>(w, av, dst, dst_dtype, k, n, stride_dst, s);
-        case 8: return launch_nb<DT, 8>(w, av, dst, dst_dtype, k, n, stride_dst, s);
+        case 1: return launch_nb<DT, 1, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        case 2: return launch_nb<DT, 2, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        case 3: return launch_nb<DT, 3, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        case 4: return launch_nb<DT, 4, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        case 5: return launch_nb<DT, 5, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        case 6: return launch_nb<DT, 6, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        case 7: return launch_nb<DT, 7, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        case 8: return launch_nb<DT, 8, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
     }
     return CQ_ERR_RANGE;
+}
+
+template <int SRC>
+int launch_dt(int w_dtype, const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
+              int64_t stride_dst, hipStream_t s) {
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_rows<CQ_Q4_0, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q8_0: return launch_rows<CQ_Q8_0, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q4K: return launch_rows<CQ_Q4K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q5K: return launch_rows<CQ_Q5K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q6K: return launch_rows<CQ_Q6K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+    }
+    return CQ_ERR_DTYPE;
+}
+
+// Activation rows are processed in groups whose quantized form fits in LDS (always all of them for
+// the shapes of an 8B decoder; a very long k with 8 rows is split, each group streaming W once).
+template <class Launch>
+int for_row_groups(int w_dtype, int64_t k, int64_t rows, Launch launch) {
+    int64_t per_row = cq_act_layout(w_dtype, k, 1).total;
+    if (per_row > LDS_BUDGET) return CQ_ERR_RANGE;
+    int64_t fit = rows;
+    while (fit > 1 && cq_act_layout(w_dtype, k, fit).total > LDS_BUDGET) fit--;
+    for (int64_t r0 = 0; r0 < rows; r0 += fit) {
+        int rc = launch(r0, rows - r0 < fit ? rows - r0 : fit);
+        if (rc) return rc;
+    }
+    return CQ_OK;
 }
 
 }  // namespace
@@ -98,17 +297,35 @@ int launch_dt(const void *w, const ActView &av, void *dst, int dst_dtype, int64_
 int cq_matvec_launch_av(int w_dtype, const void *w, const ActView &av, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
                         int64_t stride_dst, hipStream_t s) {
     if (n == 0 || rows == 0) return CQ_OK;
-    switch (w_dtype) {
-        case CQ_Q4_0: return launch_dt<CQ_Q4_0>(w, av, dst, dst_dtype, k, n, rows, stride_dst, s);
-        case CQ_Q8_0: return launch_dt<CQ_Q8_0>(w, av, dst, dst_dtype, k, n, rows, stride_dst, s);
-        case CQ_Q4K: return launch_dt<CQ_Q4K>(w, av, dst, dst_dtype, k, n, rows, stride_dst, s);
-        case CQ_Q5K: return launch_dt<CQ_Q5K>(w, av, dst, dst_dtype, k, n, rows, stride_dst, s);
-        case CQ_Q6K: return launch_dt<CQ_Q6K>(w, av, dst, dst_dtype, k, n, rows, stride_dst, s);
-    }
-    return CQ_ERR_DTYPE;
+    const int64_t esz = dst_dtype == CQ_F32 ? 4 : 2;
+    return for_row_groups(w_dtype, k, rows, [&](int64_t r0, int64_t nb) {
+        ActSrc src;
+        src.x = nullptr;
+        src.av = cq_act_view_rows(av, w_dtype, k, r0);
+        return launch_dt<SRC_SCRATCH>(w_dtype, w, src, (uint8_t *)dst + r0 * stride_dst * esz, dst_dtype, k, n, nb, stride_dst, s);
+    });
 }
 
 int cq_matvec_launch(int w_dtype, const void *w, const void *scratch, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s) {
     return cq_matvec_launch_av(w_dtype, w, cq_act_view(scratch, w_dtype, k, rows), dst, dst_dtype, k, n, rows, stride_dst, s);
+}
+
+// QMatMul::forward for up to CQ_MATVEC_MAX_ROWS activation rows, activation quantization fused in.
+int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *dst, int dst_dtype, int64_t k, int64_t n,
+                           int64_t rows, int64_t stride_dst, hipStream_t s) {
+    if (n == 0 || rows == 0) return CQ_OK;
+    const int64_t xsz = x_dtype == CQ_F32 ? 4 : 2, esz = dst_dtype == CQ_F32 ? 4 : 2;
+    return for_row_groups(w_dtype, k, rows, [&](int64_t r0, int64_t nb) {
+        ActSrc src;
+        src.x = (const uint8_t *)x + r0 * k * xsz;
+        src.av = ActView{nullptr, nullptr, nullptr};
+        void *d = (uint8_t *)dst + r0 * stride_dst * esz;
+        switch (x_dtype) {
+            case CQ_F32: return launch_dt<CQ_F32>(w_dtype, w, src, d, dst_dtype, k, n, nb, stride_dst, s);
+            case CQ_F16: return launch_dt<CQ_F16>(w_dtype, w, src, d, dst_dtype, k, n, nb, stride_dst, s);
+            case CQ_BF16: return launch_dt<CQ_BF16>(w_dtype, w, src, d, dst_dtype, k, n, nb, stride_dst, s);
+        }
+        return (int)CQ_ERR_DTYPE;
+    });
 }

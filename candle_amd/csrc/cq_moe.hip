@@ -153,6 +153,9 @@ __global__ __launch_bounds__(256) void moe_matvec_kernel(const uint8_t *__restri
 #pragma unroll
             for (int b = 0; b < PB; b++) acc[r][b] = 0.0f;
 
+        ActRow arow_p[PB];
+#pragma unroll
+        for (int b = 0; b < PB; b++) arow_p[b] = act_row(av.qs, av.d, av.bsums, DT, arow[b], k);
         for (int u = lane; u < units; u += CQ_WAVE) {
             typename F::W wr[R];
 #pragma unroll
@@ -162,14 +165,11 @@ __global__ __launch_bounds__(256) void moe_matvec_kernel(const uint8_t *__restri
             }
             typename F::A ar[PB];
 #pragma unroll
-            for (int b = 0; b < PB; b++) F::load_a(ar[b], av, arow[b], k, u);
+            for (int b = 0; b < PB; b++) F::load_a(ar[b], arow_p[b], u);
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                typename F::P p;
-                F::prep(p, wr[r], u);
+            for (int r = 0; r < R; r++)
 #pragma unroll
-                for (int b = 0; b < PB; b++) acc[r][b] = F::dot(p, ar[b], acc[r][b]);
-            }
+                for (int b = 0; b < PB; b++) acc[r][b] += F::dot(wr[r], ar[b], u);
         }
 #pragma unroll
         for (int r = 0; r < R; r++)
