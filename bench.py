@@ -5,20 +5,27 @@
 
 Workload (BASELINE.json configs[1], the configuration the metric is quoted on): Q4_K decode matvec,
 weight [14336 x 4096] (1x4096 -> 14336), batch 1, f32 activations ~N(0,1), weights ~N(0,0.02)
-quantized to Q4_K on the device.  One "step" is one pass of the hot path over one activation batch:
-activation quantization + matvec, i.e. QMatMul::forward.  Inputs are resident in HBM when the timed
-region starts.  Steps rotate through a pool of distinct weight tensors larger than the 256 MB
-Infinity Cache, so every step streams its 33 MB of weights from HBM.
+quantized to Q4_K on the device.  One "step" is one pass of the hot path over one activation batch,
+i.e. one QMatMul::forward: the activation quantization (Q8_K, bit-identical to candle's CPU path) and
+the matvec, which this library runs as ONE kernel.  Inputs are resident in HBM when the timed region
+starts.  Steps rotate through a pool of distinct weight tensors larger than the 256 MB Infinity
+Cache, so every step streams its 33 MB of weights from HBM.
 
 The JSON line carries, besides the driver contract fields:
-  roofline      achieved algorithmic GB/s of the dominant kernel (the matvec) from HIP events around
-                back-to-back launches on the launch stream, against the 8 TB/s HBM peak
+  roofline      achieved algorithmic GB/s of the dominant (only) kernel of the step, from HIP events
+                around back-to-back launches on the launch stream, against the 8 TB/s HBM peak;
+                `traffic` = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE runs
+                (read from the committed summary under profiles/ when present)
   cpu_baseline  the C restatement of candle's CPU path (AVX2 dot products + column-split threads,
                 oracle/cq_oracle_fast.c) timed on this box's host cores on a bounded sample
+
+    python bench.py --pmc-mode     a handful of un-graphed launches of the step kernel plus one plain
+                                   256 MiB device copy, for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -28,11 +35,21 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 Q4K = 12
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "q4k_decode_matvec_1x4096x14336_pmc.txt")
 
 
 def algorithmic_bytes(n, k, m, type_size, block):
     """weights once + f32 activations in + f32 outputs (scratch traffic is not counted)."""
     return n * (k // block) * type_size + m * k * 4 + m * n * 4
+
+
+def committed_traffic():
+    """HBM bytes per launch measured with rocprofv3 --pmc (see the summary file for the commands)."""
+    try:
+        m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", open(TRAFFIC_SUMMARY).read())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def main():
@@ -46,11 +63,12 @@ def main():
     ap.add_argument("--pool-mb", type=int, default=1280, help="distinct weight bytes rotated through (MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--pmc-mode", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the labelled context numbers (cache-resident, pre-quantized)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every configuration of the metric is single-GPU); use --gpus 1")
 
-    import numpy as np
     import torch
 
     from candle_amd import _lib
@@ -66,6 +84,8 @@ def main():
 
     # ---- synthetic inputs, resident in HBM --------------------------------------------------
     pool = max(2, (args.pool_mb * 1000 * 1000 + wbytes - 1) // wbytes)
+    if args.pmc_mode:
+        pool = 8
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     weights = []
@@ -84,15 +104,30 @@ def main():
     stream = torch.cuda.Stream(device=dev)
 
     def step(i, sp):
+        """QMatMul::forward: activation quantization + matvec in one kernel."""
         _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(Q4K, weights[i % pool].data_ptr(), x.data_ptr(), 0, dst.data_ptr(), 0,
                                                               m, k, n, ws.data_ptr(), ws_bytes, sp))
 
-    def matvec_only(i, sp):
+    def matvec_prequantized(i, sp):
         _lib.check("cq_matvec", L.cq_matvec(Q4K, weights[i % pool].data_ptr(), ws.data_ptr(), dst.data_ptr(), 0, k, n, m, n, sp))
+
+    if args.pmc_mode:
+        # plain launches (one dispatch row per kernel in the counter CSV) + a copy of known size
+        with torch.cuda.stream(stream):
+            for i in range(2 * pool):
+                step(i, stream.cuda_stream)
+            a = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+            b = torch.empty_like(a)
+            stream.synchronize()
+            for _ in range(4):
+                b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_mode": True, "copy_bytes": 256 << 20, "step_algorithmic_bytes": alg_bytes}))
+        return
 
     # The step is a few microseconds of GPU work: capture one rotation over the pool in a HIP graph
     # so that host launch latency is not what gets measured.
-    def capture(fn):
+    def capture(fn, same_weight=False):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.stream(stream):
             fn(0, stream.cuda_stream)          # warm the code path before capture
@@ -100,11 +135,8 @@ def main():
             with torch.cuda.graph(g, stream=stream):
                 sp = torch.cuda.current_stream().cuda_stream
                 for i in range(pool):
-                    fn(i, sp)
+                    fn(0 if same_weight else i, sp)
         return g
-
-    g_step = capture(step)
-    g_mv = capture(matvec_only)
 
     def run(graph, steps):
         reps = max(1, (steps + pool - 1) // pool)
@@ -113,7 +145,20 @@ def main():
                 graph.replay()
         return reps * pool
 
-    # ---- timed region: EXACTLY K steps (rounded up to whole rotations), wall clock ------------
+    def event_us(graph, steps):
+        run(graph, args.warmup)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(stream):
+            e0.record(stream)
+            done = run(graph, steps)
+            e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / done
+
+    g_step = capture(step)
+
+    # ---- timed region: K steps (rounded up to whole rotations of the pool), wall clock ------------
     run(g_step, args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -123,34 +168,21 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / done
     value = alg_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- dominant kernel: back-to-back matvec launches between HIP events on the launch stream ----
-    run(g_mv, args.warmup)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with torch.cuda.stream(stream):
-        e0.record(stream)
-        done_mv = run(g_mv, args.steps)
-        e1.record(stream)
-    torch.cuda.synchronize()
-    mv_us = e0.elapsed_time(e1) * 1e3 / done_mv
-    achieved = alg_bytes / (mv_us * 1e-6) / 1e9
-
-    # ---- same kernel with the weights resident in the Infinity Cache (one tensor reused), labelled ----
-    g_res = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(stream):
-        stream.synchronize()
-        with torch.cuda.graph(g_res, stream=stream):
-            sp = torch.cuda.current_stream().cuda_stream
-            for _ in range(pool):
-                matvec_only(0, sp)
-        for _ in range(10):
-            g_res.replay()
-        e0.record(stream)
-        for _ in range(50):
-            g_res.replay()
-        e1.record(stream)
-    torch.cuda.synchronize()
-    res_us = e0.elapsed_time(e1) * 1e3 / (50 * pool)
+    # ---- dominant kernel (the step IS one kernel): HIP events around the same back-to-back launches ----
+    kern_us = event_us(g_step, args.steps)
+    achieved = alg_bytes / (kern_us * 1e-6) / 1e9
+    # context numbers, labelled: the same kernel with the weights resident in the Infinity Cache (one
+    # tensor reused), and the matvec over activations quantized beforehand by cq_quantize_act
+    extra = None
+    if not args.no_extra:
+        resident_us = event_us(capture(step, same_weight=True), args.steps)
+        _lib.check("cq_quantize_act", L.cq_quantize_act(Q4K, x.data_ptr(), 0, ws.data_ptr(), k, m, None))
+        torch.cuda.synchronize()
+        preq_us = event_us(capture(matvec_prequantized), args.steps)
+        extra = {"infinity_cache_resident_us": round(resident_us, 3),
+                 "infinity_cache_resident_GBps": round(alg_bytes / (resident_us * 1e-6) / 1e9, 1),
+                 "prequantized_matvec_us": round(preq_us, 3),
+                 "prequantized_matvec_GBps": round(alg_bytes / (preq_us * 1e-6) / 1e9, 1)}
 
     out = {
         "metric": "Q4_K matvec GB/s @4096x14336 (decode, batch %d)" % m,
@@ -167,12 +199,13 @@ def main():
         "data": "synthetic",
         "config": {"workload": "Q4_K decode matvec 1x%d->%d, weight [%d x %d] Q4_K, batch %d, %d distinct weight tensors rotated (%.2f GB)"
                                % (k, n, n, k, m, pool, pool * wbytes / 1e9),
-                   "step": "activation quantize (Q8_K) + matvec, captured in a HIP graph", "n": n, "k": k, "batch": m},
+                   "step": "QMatMul::forward = Q8_K activation quantization + matvec in one kernel, launches captured in a HIP graph",
+                   "n": n, "k": k, "batch": m},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
-        "roofline": {"bound": "hbm", "kernel": "matvec_kernel<Q4_K>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "avg_kernel_us": round(mv_us, 3),
-                     "algorithmic_bytes_per_launch": alg_bytes,
-                     "cache_resident_us": round(res_us, 3), "cache_resident_GBps": round(alg_bytes / (res_us * 1e-6) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "kernel": "qmv_kernel<Q4_K, NB=1, fused f32 activations>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": committed_traffic(),
+                     "avg_kernel_us": round(kern_us, 3), "algorithmic_bytes_per_launch": alg_bytes},
+        "extra": extra,
     }
 
     if not args.no_cpu_baseline:
