@@ -21,6 +21,10 @@ The JSON line carries, besides the driver contract fields:
 
     python bench.py --pmc-mode     a handful of un-graphed launches of the step kernel plus one plain
                                    256 MiB device copy, for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`
+    python bench.py --workload prefill --wdtype q6k --n 4096 --k 14336 --batch 512
+                                   the prefill matmul (other BASELINE configurations; not the headline line):
+                                   TFLOP/s of QMatMul::forward and of its MFMA kernel against the 2.5 PFLOP/s
+                                   dense f16 peak
 """
 import argparse
 import json
@@ -34,7 +38,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 Q4K = 12
+WDTYPES = {"q4_0": (2, 18, 32), "q8_0": (8, 34, 32), "q4k": (12, 144, 256), "q5k": (13, 176, 256), "q6k": (14, 210, 256)}
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "q4k_decode_matvec_1x4096x14336_pmc.txt")
 
 
@@ -52,11 +58,81 @@ def committed_traffic():
         return None
 
 
+def prefill(args):
+    """QMatMul::forward with more than 8 activation rows: Q8_K / Q8_0 activation quantization kernel + MFMA matmul kernel."""
+    import torch
+
+    from candle_amd import _lib
+
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    dt, ts, bs = WDTYPES[args.wdtype]
+    n, k, m = args.n, args.k, args.batch
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    wbytes = L.cq_storage_bytes(dt, n * k)
+    wf = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
+    wq = torch.empty(wbytes, dtype=torch.uint8, device=dev)
+    _lib.check("cq_quantize", L.cq_quantize(dt, wf.data_ptr(), wq.data_ptr(), n * k, None))
+    del wf
+    x = torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32)
+    dst = torch.empty((m, n), dtype=torch.float32, device=dev)
+    ws_bytes = L.cq_qmatmul_workspace_bytes(dt, m, k, n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.Stream(device=dev)
+    sp = stream.cuda_stream
+
+    def forward():
+        _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(dt, wq.data_ptr(), x.data_ptr(), 0, dst.data_ptr(), 0, m, k, n,
+                                                              ws.data_ptr(), ws_bytes, sp))
+
+    def matmul_only():
+        _lib.check("cq_matmul", L.cq_matmul(dt, wq.data_ptr(), ws.data_ptr(), dst.data_ptr(), k, n, m, n, sp))
+
+    def event_us(fn, steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(stream):
+            for _ in range(args.warmup):
+                fn()
+            e0.record(stream)
+            for _ in range(steps):
+                fn()
+            e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    steps = args.steps
+    with torch.cuda.stream(stream):
+        for _ in range(args.warmup):
+            forward()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        for _ in range(steps):
+            forward()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    flops = 2.0 * m * n * k
+    kern_us = event_us(matmul_only, steps)
+    print(json.dumps({
+        "metric": "%s prefill matmul TFLOP/s @%dx%d, M=%d" % (args.wdtype, n, k, m), "value": round(flops / (ms * 1e-3) / 1e12, 1),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "%s prefill matmul [%d x %d] x [%d x %d]^T" % (args.wdtype, m, k, n, k),
+                   "step": "QMatMul::forward = activation quantization kernel + MFMA matmul kernel", "n": n, "k": k, "batch": m},
+        "roofline": {"bound": "mfma", "kernel": "qmm_kernel<%s>" % args.wdtype, "achieved": round(flops / (kern_us * 1e-6) / 1e12, 1),
+                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (kern_us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "traffic": None, "avg_kernel_us": round(kern_us, 2)},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode")
+    ap.add_argument("--wdtype", choices=sorted(WDTYPES), default="q4k", help="weight format of --workload prefill")
     ap.add_argument("--n", type=int, default=14336)
     ap.add_argument("--k", type=int, default=4096)
     ap.add_argument("--batch", type=int, default=1)
@@ -68,6 +144,12 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every configuration of the metric is single-GPU); use --gpus 1")
+    if args.steps is None:
+        args.steps = 4000 if args.workload == "decode" else 50
+    if args.warmup is None:
+        args.warmup = 400 if args.workload == "decode" else 5
+    if args.workload == "prefill":
+        return prefill(args)
 
     import torch
 

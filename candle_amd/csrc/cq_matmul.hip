@@ -1,8 +1,434 @@
-// Prefill matmul over pre-quantized activations, and the f32 -> f16/bf16 output conversion.
+// Prefill matmul over pre-quantized activations for gfx950 (MFMA), and the f32 -> f16/bf16 output
+// conversion.   dst[m, n] = sum_k x^[m, k] * W^[n, k]
+//
+// Counterpart of candle's tensor-core MMQ path (candle-core/src/quantized/fast_mmq.rs:253-400,
+// candle-kernels/src/mmq_gguf/).  The arithmetic follows the CPU path instead of the CUDA one:
+// activations are the Q8_K / Q8_0 quantization written by cq_quantize_act.
+//
+// K-quants (Q4_K, Q5_K, Q6_K) — integer-exact formulation on the f16 matrix cores:
+//   per 256-element super-block kb      S[m,n] = sum_k q8[m,k] * (sc[n,sub(k)] * q[n,k])
+//   operands are small integers held exactly in f16 (|q8| <= 128, |sc*q| <= 1953 for Q4_K/Q5_K),
+//   products accumulate in f32, and once per super-block
+//       acc[m,n] += d8[m,kb] * ( d[n,kb] * S[m,n] - dmin[n,kb] * M[m,n] ),
+//       M[m,n] = sum_{j<16} bsums16[m,j] * min[n,j/2]          (one extra K=16 MFMA, Q4_K/Q5_K only)
+//   — the same integers the CPU vec_dot sums (k_quants.rs:1460-1540, 1714-1801, 2035-2092).  For Q6_K
+//   the product sc*(q-32) can reach 4096; values above 2048 that are odd round to even in f16
+//   (relative 2^-12 on those elements only).
+// Q4_0 / Q8_0 — both operands carry a per-32 f16 scale, so the dequantized values d*(q-8) and d8*q8
+//   are rounded to f16 (relative 2^-11 per operand) and multiplied at full MFMA rate; the result stays
+//   well inside the 1e-3 tolerance (measured ~2e-4) but is not integer-exact like the decode path.
+//
+// Tiling: workgroup = 4 waves (2 x 2), block tile 128 (m) x 128 (n), wave tile 64 x 64 as 2 x 2
+// v_mfma_f32_32x32x16_f16 tiles.  K advances 64 elements per LDS stage: 256 threads dequantize the
+// 128 x 64 weight tile and convert the 128 x 64 int8 activation tile to f16 in LDS (row stride padded
+// to 144 bytes); the raw bytes of the next stage are loaded into registers before the MFMAs of the
+// current one.
 #include "cq_device.h"
 #include "cq_launch.h"
 
 namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int LDK = BK + 8;            // padded row stride in halves (144 bytes)
+
+// ---- integer bytes -> f16 pairs ------------------------------------------------------------------
+// bytes b0..b3 of `x` (values 0..255) -> two dwords of f16 pairs holding (1024 + b) exactly:
+// the f16 bit pattern 0x6400 | b is 1024 + b for b < 1024.
+__device__ __forceinline__ void bytes_to_h1024(uint32_t x, uint32_t &lo, uint32_t &hi) {
+    lo = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);   // [b0, 0x64, b1, 0x64]
+    hi = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);   // [b2, 0x64, b3, 0x64]
+}
+__device__ __forceinline__ uint32_t pk_fma(uint32_t a, uint32_t b, uint32_t c) {
+    half2v r = __builtin_elementwise_fma(__builtin_bit_cast(half2v, a), __builtin_bit_cast(half2v, b), __builtin_bit_cast(half2v, c));
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t pk_add(uint32_t a, uint32_t b) {
+    half2v r = __builtin_bit_cast(half2v, a) + __builtin_bit_cast(half2v, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t pk_mul(uint32_t a, uint32_t b) {
+    half2v r = __builtin_bit_cast(half2v, a) * __builtin_bit_cast(half2v, b);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t h2_splat(float v) {          // v exactly representable in f16
+    uint32_t h = f2h_bits(v);
+    return h | (h << 16);
+}
+
+// 6-bit scale / min of sub-block j (utils.rs:50-60) from the 12 packed bytes held in three dwords
+__device__ __forceinline__ void k4_sub_scale_min(uint32_t u0, uint32_t u1, uint32_t u2, int j, int &sc, int &mn) {
+    int sh = 8 * (j & 3);
+    if (j < 4) {
+        sc = (u0 >> sh) & 63;
+        mn = (u1 >> sh) & 63;
+    } else {
+        sc = ((u2 >> sh) & 0xF) | (((u0 >> sh) >> 6 & 3) << 4);
+        mn = ((u2 >> sh) >> 4 & 0xF) | (((u1 >> sh) >> 6 & 3) << 4);
+    }
+}
+
+// ---- per-format staging of one (row, 32-element sub-block) of W into 16 dwords of f16 pairs -------
+// raw: what one thread loads for (row n, k-range [kb*256 + 64*g + 32*half, +32)).
+template <int DT> struct Stage;
+
+template <> struct Stage<CQ_Q4K> {
+    static constexpr bool KQ = true, HAS_MIN = true;
+    struct Raw { u32x4 hdr, q0, q1; };
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int) {
+        const uint8_t *blk = row + (int64_t)kb * 144;
+        r.hdr = *reinterpret_cast<const u32x4 *>(blk);
+        r.q0 = *reinterpret_cast<const u32x4 *>(blk + 16 + 32 * g);
+        r.q1 = *reinterpret_cast<const u32x4 *>(blk + 32 + 32 * g);
+    }
+    static __device__ __forceinline__ void header(const Raw &r, float &d, float &dmin, int mins[8]) {
+        d = h2f(r.hdr.x);
+        dmin = h2f(r.hdr.x >> 16);
+#pragma unroll
+        for (int j = 0; j < 8; j++) { int sc; k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, j, sc, mins[j]); }
+    }
+    // 32 values sc*q as f16 pairs, element order = k order
+    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) {
+        int sc, mn;
+        k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g + half, sc, mn);
+        const uint32_t s2 = h2_splat((float)sc), c2 = h2_splat(-1024.0f * (float)sc);
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t v = (half ? (q[i] >> 4) : q[i]) & 0x0f0f0f0fu, lo, hi;
+            bytes_to_h1024(v, lo, hi);
+            out[2 * i] = pk_fma(lo, s2, c2);        // (1024 + q) * sc - 1024 * sc = sc * q, one exact rounding
+            out[2 * i + 1] = pk_fma(hi, s2, c2);
+        }
+    }
+};
+
+template <> struct Stage<CQ_Q5K> {
+    static constexpr bool KQ = true, HAS_MIN = true;
+    struct Raw { u32x4 hdr, h0, h1, q0, q1; };
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int) {
+        const uint8_t *blk = row + (int64_t)kb * 176;
+        r.hdr = *reinterpret_cast<const u32x4 *>(blk);
+        r.h0 = *reinterpret_cast<const u32x4 *>(blk + 16);
+        r.h1 = *reinterpret_cast<const u32x4 *>(blk + 32);
+        r.q0 = *reinterpret_cast<const u32x4 *>(blk + 48 + 32 * g);
+        r.q1 = *reinterpret_cast<const u32x4 *>(blk + 64 + 32 * g);
+    }
+    static __device__ __forceinline__ void header(const Raw &r, float &d, float &dmin, int mins[8]) {
+        d = h2f(r.hdr.x);
+        dmin = h2f(r.hdr.x >> 16);
+#pragma unroll
+        for (int j = 0; j < 8; j++) { int sc; k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, j, sc, mins[j]); }
+    }
+    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) {
+        int sc, mn;
+        k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g + half, sc, mn);
+        const uint32_t s2 = h2_splat((float)sc), c2 = h2_splat(-1024.0f * (float)sc);
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const uint32_t h[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t hb = (h[i] >> (2 * g + half)) & 0x01010101u;
+            uint32_t v = ((half ? (q[i] >> 4) : q[i]) & 0x0f0f0f0fu) | (hb << 4), lo, hi;
+            bytes_to_h1024(v, lo, hi);
+            out[2 * i] = pk_fma(lo, s2, c2);
+            out[2 * i + 1] = pk_fma(hi, s2, c2);
+        }
+    }
+};
+
+template <> struct Stage<CQ_Q6K> {
+    static constexpr bool KQ = true, HAS_MIN = false;
+    // sub-block (g, half) = elements 64g + 32half + [0, 32): half h6 = g >> 1 of the block, quarter = 2*(g&1) + half
+    struct Raw { u32x4 l0, l1, h0, h1; uint32_t sc, d; };
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
+        const uint8_t *blk = row + (int64_t)kb * 210;
+        const int h6 = g >> 1, quarter = 2 * (g & 1) + half;
+        const uint8_t *ql = blk + 64 * h6 + ((quarter & 1) ? 32 : 0);   // ql[l] or ql[l + 32], l = 0..31
+        r.l0 = ld_u<u32x4>(ql);
+        r.l1 = ld_u<u32x4>(ql + 16);
+        r.h0 = ld_u<u32x4>(blk + 128 + 32 * h6);
+        r.h1 = ld_u<u32x4>(blk + 128 + 32 * h6 + 16);
+        // scales of this quarter: index 8*h6 + 2*quarter + {0, 1} (l / 16)
+        r.sc = ld_u<uint16_t>(blk + 192 + 8 * h6 + 2 * quarter);
+        r.d = ld_u<uint16_t>(blk + 208);
+    }
+    static __device__ __forceinline__ void header(const Raw &r, float &d, float &dmin, int mins[8]) {
+        d = h2f(r.d);
+        dmin = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) mins[j] = 0;
+    }
+    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) {
+        const int quarter = 2 * (g & 1) + half;
+        const uint32_t sA = h2_splat((float)(int8_t)(r.sc & 0xff)), sB = h2_splat((float)(int8_t)(r.sc >> 8));
+        const uint32_t off = h2_splat(-1056.0f);                       // -(1024 + 32)
+        const uint32_t ql[8] = {r.l0.x, r.l0.y, r.l0.z, r.l0.w, r.l1.x, r.l1.y, r.l1.z, r.l1.w};
+        const uint32_t qh[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t lo4 = ((quarter >= 2) ? (ql[i] >> 4) : ql[i]) & 0x0f0f0f0fu;
+            uint32_t hi2 = ((qh[i] >> (2 * quarter)) & 0x03030303u) << 4;
+            uint32_t lo, hi;
+            bytes_to_h1024(lo4 | hi2, lo, hi);
+            const uint32_t s2 = i < 4 ? sA : sB;                         // l / 16
+            out[2 * i] = pk_mul(pk_add(lo, off), s2);                    // (q - 32) * sc
+            out[2 * i + 1] = pk_mul(pk_add(hi, off), s2);
+        }
+    }
+};
+
+template <> struct Stage<CQ_Q4_0> {
+    static constexpr bool KQ = false, HAS_MIN = false;
+    struct Raw { u32x4 qs; uint32_t d; };
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
+        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + half) * 18;
+        r.d = ld_u<uint16_t>(blk);
+        r.qs = ld_u<u32x4>(blk + 2);
+    }
+    static __device__ __forceinline__ void header(const Raw &, float &d, float &dmin, int mins[8]) {
+        d = 1.0f; dmin = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) mins[j] = 0;
+    }
+    static __device__ __forceinline__ void convert(const Raw &r, int, int, uint32_t out[16]) {
+        const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1032.0f);   // -(1024 + 8)
+        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t lo, hi;
+            bytes_to_h1024(q[i] & 0x0f0f0f0fu, lo, hi);               // elements 4i..4i+3
+            out[2 * i] = pk_mul(pk_add(lo, off), d2);
+            out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
+            bytes_to_h1024((q[i] >> 4) & 0x0f0f0f0fu, lo, hi);        // elements 16+4i..
+            out[8 + 2 * i] = pk_mul(pk_add(lo, off), d2);
+            out[8 + 2 * i + 1] = pk_mul(pk_add(hi, off), d2);
+        }
+    }
+};
+
+template <> struct Stage<CQ_Q8_0> {
+    static constexpr bool KQ = false, HAS_MIN = false;
+    struct Raw { u32x4 q0, q1; uint32_t d; };
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
+        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + half) * 34;
+        r.d = ld_u<uint16_t>(blk);
+        r.q0 = ld_u<u32x4>(blk + 2);
+        r.q1 = ld_u<u32x4>(blk + 18);
+    }
+    static __device__ __forceinline__ void header(const Raw &, float &d, float &dmin, int mins[8]) {
+        d = 1.0f; dmin = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) mins[j] = 0;
+    }
+    static __device__ __forceinline__ void convert(const Raw &r, int, int, uint32_t out[16]) {
+        const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1152.0f);   // -(1024 + 128)
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t lo, hi;
+            bytes_to_h1024(q[i] ^ 0x80808080u, lo, hi);               // int8 -> biased unsigned
+            out[2 * i] = pk_mul(pk_add(lo, off), d2);
+            out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
+        }
+    }
+};
+
+// 32 int8 activations -> 16 dwords of f16 pairs (exact); scale2 == 0 means "leave as integers"
+__device__ __forceinline__ void act_convert(const u32x4 &a0, const u32x4 &a1, bool scaled, uint32_t scale2, uint32_t out[16]) {
+    const uint32_t off = 0xe480e480u;    // two f16 -1152.0
+    const uint32_t q[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        uint32_t lo, hi;
+        bytes_to_h1024(q[i] ^ 0x80808080u, lo, hi);
+        lo = pk_add(lo, off);
+        hi = pk_add(hi, off);
+        out[2 * i] = scaled ? pk_mul(lo, scale2) : lo;
+        out[2 * i + 1] = scaled ? pk_mul(hi, scale2) : hi;
+    }
+}
+
+__device__ __forceinline__ void lds_write32h(_Float16 *dstrow, const uint32_t v[16]) {
+    u32x4 *p = reinterpret_cast<u32x4 *>(dstrow);
+    p[0] = u32x4{v[0], v[1], v[2], v[3]};
+    p[1] = u32x4{v[4], v[5], v[6], v[7]};
+    p[2] = u32x4{v[8], v[9], v[10], v[11]};
+    p[3] = u32x4{v[12], v[13], v[14], v[15]};
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k, int n, int rows,
+                                                  int64_t stride_dst) {
+    typedef Stage<DT> S;
+    constexpr bool KQ = S::KQ;
+    __shared__ __align__(16) _Float16 As[BM * LDK];
+    __shared__ __align__(16) _Float16 Bs[BN * LDK];
+    __shared__ __align__(16) _Float16 Am[BM * 24];    // bsums16 of the super-block, as f16 (row stride 24 halves)
+    __shared__ __align__(16) _Float16 Bm[BN * 24];    // sub-block mins duplicated per 16-element group
+    __shared__ float sD[BN], sDmin[BN], sD8[BM];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int wm = wv >> 1, wn = wv & 1;
+    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    const int nsb = k >> 8;                                     // 256-element spans
+    const int64_t row_bytes = (int64_t)(k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
+
+    // staging role of this thread: (row r_l of the tile, 32-element half)
+    const int r_l = tid >> 1, half = tid & 1;
+    const int wrow = min(n0 + r_l, n - 1);
+    const int arow = min(m0 + r_l, rows - 1);
+    const bool arow_ok = m0 + r_l < rows;
+    const uint8_t *wrow_p = w + wrow * row_bytes;
+    const int8_t *aq_p = av.qs + (int64_t)arow * k;
+
+    f32x16 acc[2][2], sb[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) { acc[i][j][e] = 0.0f; sb[i][j][e] = 0.0f; }
+
+    typename S::Raw wraw;
+    u32x4 a0, a1;
+    auto load_stage = [&](int kb, int g) {
+        S::load(wraw, wrow_p, kb, g, half);
+        const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
+        a0 = *reinterpret_cast<const u32x4 *>(q);
+        a1 = *reinterpret_cast<const u32x4 *>(q + 16);
+    };
+    load_stage(0, 0);
+
+    for (int kb = 0; kb < nsb; kb++) {
+        for (int g = 0; g < 4; g++) {
+            // ---- write the staged raw data of (kb, g) to LDS as f16 ----
+            uint32_t hv[16];
+            S::convert(wraw, g, half, hv);
+            lds_write32h(Bs + r_l * LDK + 32 * half, hv);
+            uint32_t ascale2 = 0;
+            if (!KQ) {
+                float d8 = av.d[2 * ((int64_t)arow * (k >> 5) + kb * 8 + 2 * g + half)];   // already f16-representable
+                ascale2 = h2_splat(d8);
+            }
+            act_convert(a0, a1, !KQ, ascale2, hv);
+            if (!arow_ok) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) hv[i] = 0;
+            }
+            lds_write32h(As + r_l * LDK + 32 * half, hv);
+            if (KQ && g == 0) {
+                float d, dmin;
+                int mins[8];
+                S::header(wraw, d, dmin, mins);
+                if (half == 0) { sD[r_l] = d; sDmin[r_l] = dmin; sD8[r_l] = arow_ok ? av.d[(int64_t)arow * (k >> 8) + kb] : 0.0f; }
+                if (S::HAS_MIN) {
+                    // Bm[n][j] = min[j/2] for j in 8*half .. 8*half+7 ; Am[m][j] = bsums16[j]
+                    uint32_t mv[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        uint32_t hm = f2h_bits((float)mins[4 * half + i]);
+                        mv[i] = hm | (hm << 16);
+                    }
+                    *reinterpret_cast<u32x4 *>(Bm + r_l * 24 + 8 * half) = u32x4{mv[0], mv[1], mv[2], mv[3]};
+                    u32x4 bs = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
+                    const uint32_t b4[4] = {bs.x, bs.y, bs.z, bs.w};
+                    uint32_t bv[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        uint32_t lo = f2h_bits((float)(int16_t)(b4[i] & 0xffff)), hi = f2h_bits((float)(int16_t)(b4[i] >> 16));
+                        bv[i] = arow_ok ? (lo | (hi << 16)) : 0u;
+                    }
+                    *reinterpret_cast<u32x4 *>(Am + r_l * 24 + 8 * half) = u32x4{bv[0], bv[1], bv[2], bv[3]};
+                }
+            }
+            __syncthreads();
+            // ---- raw bytes of the next stage go in flight while the matrix cores work ----
+            {
+                int ng = g + 1, nkb = kb;
+                if (ng == 4) { ng = 0; nkb = kb + 1; }
+                if (nkb < nsb) load_stage(nkb, ng);
+            }
+            // ---- 4 k-slices of 16: 2 x 2 MFMA tiles per wave ----
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                half8 af[2], bf[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    af[t] = *reinterpret_cast<const half8 *>(As + (wm * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
+                    bf[t] = *reinterpret_cast<const half8 *>(Bs + (wn * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
+                }
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
+            }
+            if (KQ && g == 3) {
+                // ---- end of the super-block: mins term and the f32 scales ----
+                f32x16 mt[2][2];
+                if (S::HAS_MIN) {
+                    half8 am[2], bm[2];
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        am[t] = *reinterpret_cast<const half8 *>(Am + (wm * 64 + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
+                        bm[t] = *reinterpret_cast<const half8 *>(Bm + (wn * 64 + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
+                    }
+#pragma unroll
+                    for (int i = 0; i < 2; i++)
+#pragma unroll
+                        for (int j = 0; j < 2; j++) {
+                            f32x16 z;
+#pragma unroll
+                            for (int e = 0; e < 16; e++) z[e] = 0.0f;
+                            mt[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am[i], bm[j], z, 0, 0, 0);
+                        }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int nl = wn * 64 + j * 32 + (lane & 31);
+                    const float d = sD[nl], dmin = sDmin[nl];
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+#pragma unroll
+                        for (int e = 0; e < 16; e++) {
+                            const int ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                            float t = d * sb[i][j][e];
+                            if (S::HAS_MIN) t = fmaf(-dmin, mt[i][j][e], t);
+                            acc[i][j][e] = fmaf(sD8[ml], t, acc[i][j][e]);
+                            sb[i][j][e] = 0.0f;
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: C layout of the 32x32 tile: column = lane % 32, row = 8*(e/4) + 4*(lane/32) + e%4 ----
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int nn = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int mm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                float v = KQ ? acc[i][j][e] : sb[i][j][e];
+                if (mm < rows && nn < n) dst[(int64_t)mm * stride_dst + nn] = v;
+            }
+        }
+}
+
+template <int DT>
+int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+    dim3 grid((unsigned)((rows + BM - 1) / BM), (unsigned)((n + BN - 1) / BN));
+    if (grid.y > 65535) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL((qmm_kernel<DT>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst);
+    return (int)hipGetLastError();
+}
 
 __global__ __launch_bounds__(256) void convert_f32_kernel(const float *__restrict__ src, void *__restrict__ dst, int dst_dtype, int64_t count) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -28,10 +454,21 @@ int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t co
     return (int)hipGetLastError();
 }
 
-// Row-chunked matvec: every chunk of 8 activation rows streams W once.
+// k is a multiple of 256 for the MFMA kernel (always true for K-quants); Q4_0 / Q8_0 rows whose length
+// is only a multiple of 32, and very small problems, go through the row-chunked matvec instead.
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s) {
     ActView av = cq_act_view(scratch, w_dtype, k, rows);
+    if (k % 256 == 0 && rows > CQ_MATVEC_MAX_ROWS) {
+        switch (w_dtype) {
+            case CQ_Q4_0: return launch_qmm<CQ_Q4_0>(w, av, dst, k, n, rows, stride_dst, s);
+            case CQ_Q8_0: return launch_qmm<CQ_Q8_0>(w, av, dst, k, n, rows, stride_dst, s);
+            case CQ_Q4K: return launch_qmm<CQ_Q4K>(w, av, dst, k, n, rows, stride_dst, s);
+            case CQ_Q5K: return launch_qmm<CQ_Q5K>(w, av, dst, k, n, rows, stride_dst, s);
+            case CQ_Q6K: return launch_qmm<CQ_Q6K>(w, av, dst, k, n, rows, stride_dst, s);
+        }
+        return CQ_ERR_DTYPE;
+    }
     for (int64_t r0 = 0; r0 < rows; r0 += CQ_MATVEC_MAX_ROWS) {
         int64_t nb = rows - r0 < CQ_MATVEC_MAX_ROWS ? rows - r0 : CQ_MATVEC_MAX_ROWS;
         ActView c = cq_act_view_rows(av, w_dtype, k, r0);
