@@ -25,6 +25,9 @@ The JSON line carries, besides the driver contract fields:
                                    the prefill matmul (other BASELINE configurations; not the headline line):
                                    TFLOP/s of QMatMul::forward and of its MFMA kernel against the 2.5 PFLOP/s
                                    dense f16 peak
+    python bench.py --workload decode8b [--steps 256] [--prompt 512]
+                                   the 8B-shape Q4_K_M decoder: prompt and decode tok/s against the weight-streaming
+                                   roofline (8 TB/s / weight bytes per token)
 """
 import argparse
 import json
@@ -126,12 +129,58 @@ def prefill(args):
     }))
 
 
+def decode8b(args):
+    """BASELINE configs[3]: random-init Llama-3-8B-shaped decoder, Q4_K_M mix, 512-token prefill then greedy decode, batch 1."""
+    import torch
+
+    from candle_amd.quantized_llama import Config, ModelWeights
+
+    cfg = Config.llama3_8b()
+    cfg.n_layer = args.layers
+    t0 = time.perf_counter()
+    model = ModelWeights.random_init(cfg, seed=1234)
+    torch.cuda.synchronize()
+    t_init = time.perf_counter() - t0
+    gen = torch.Generator()
+    gen.manual_seed(99)
+    prompt = torch.randint(0, cfg.vocab, (args.prompt,), generator=gen).tolist()
+    n_new = args.steps if args.steps else 256
+    model.generate_greedy(prompt, min(n_new, 8))                      # warm-up: code paths, graph capture
+    res = model.generate_greedy(prompt, n_new)
+    wbytes = model.weight_bytes_per_token()
+    steps = res["decode_steps"]
+    tok_s = steps / res["decode_seconds"]
+    # KV bytes read per decode step, averaged over the positions of the run (f32 cache, K and V)
+    mean_pos = args.prompt + (n_new + 1) / 2.0
+    kv_bytes = 2 * cfg.n_layer * cfg.n_kv_head * cfg.head_dim * 4 * mean_pos
+    roof_tok_s = HBM_PEAK_GBPS * 1e9 / wbytes
+    print(json.dumps({
+        "metric": "8B-shape Q4_K_M decode tok/s (batch 1, greedy)", "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1,
+        "steps": steps, "warmup": 8, "ms_per_step": round(1e3 / tok_s, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8 dot products, f32 glue", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B shape, %d layers, hidden 4096, 32 q / 8 kv heads, head_dim 128, FFN 14336, vocab 128256; "
+                               "attn_v / ffn_down Q6_K, rest and head Q4_K; f32 embedding table; rope theta 500000, rms eps 1e-5; "
+                               "%d random prompt tokens prefilled in one forward, then %d greedy single-token steps replayed from one HIP graph"
+                               % (cfg.n_layer, args.prompt, steps),
+                   "ctx": cfg.ctx, "prompt_tokens": args.prompt},
+        "prompt_tok_s": round(args.prompt / res["prompt_seconds"], 1),
+        "weight_bytes_per_token": wbytes, "kv_bytes_per_token_mean": int(kv_bytes),
+        "roofline": {"bound": "hbm", "kernel": "whole decode step (weights streamed once per token)",
+                     "achieved": round((wbytes + kv_bytes) * tok_s / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round((wbytes + kv_bytes) * tok_s / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "roofline_tok_s_weights_only": round(roof_tok_s, 1), "frac_of_roofline_tok_s": round(tok_s / roof_tok_s, 4)},
+        "init_seconds": round(t_init, 1),
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", choices=["decode", "prefill"], default="decode")
+    ap.add_argument("--workload", choices=["decode", "prefill", "decode8b"], default="decode")
+    ap.add_argument("--layers", type=int, default=32, help="--workload decode8b: number of decoder layers")
+    ap.add_argument("--prompt", type=int, default=512, help="--workload decode8b: prompt tokens")
     ap.add_argument("--wdtype", choices=sorted(WDTYPES), default="q4k", help="weight format of --workload prefill")
     ap.add_argument("--n", type=int, default=14336)
     ap.add_argument("--k", type=int, default=4096)
@@ -144,6 +193,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every configuration of the metric is single-GPU); use --gpus 1")
+    if args.workload == "decode8b":
+        return decode8b(args)
     if args.steps is None:
         args.steps = 4000 if args.workload == "decode" else 50
     if args.warmup is None:

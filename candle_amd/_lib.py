@@ -1,4 +1,5 @@
-"""ctypes binding of libcandle_hip_quant.so (the C ABI declared in include/candle_hip_quant.h).
+"""ctypes binding of libcandle_hip_quant.so (the C ABI declared in include/candle_hip_quant.h and
+include/candle_hip_nn.h).
 
 The library must be built first (``python -m candle_amd.build`` or ``__graft_entry__.build()``);
 loading fails loudly when it is missing — there is no CPU or PyTorch fallback.
@@ -14,8 +15,9 @@ LIB_PATH = os.path.join(_HERE, "libcandle_hip_quant.so")
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
 _vp = ctypes.c_void_p
+_f32 = ctypes.c_float
 
-# name -> (restype, argtypes); mirrors include/candle_hip_quant.h one to one
+# name -> (restype, argtypes); mirrors the two headers under include/ one to one
 SIGNATURES = {
     "cq_status_string": (ctypes.c_char_p, [_int]),
     "cq_block_size": (_i64, [_int]),
@@ -33,6 +35,14 @@ SIGNATURES = {
     "cq_indexed_moe_forward": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_moe_gemm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _int]),
     "cq_moe_gemm_gguf": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
+    # include/candle_hip_nn.h
+    "cq_nn_embedding": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "cq_nn_rms_norm": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
+    "cq_nn_rope_i_kv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "cq_nn_attention_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
+    "cq_nn_attention": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp]),
+    "cq_nn_silu_mul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "cq_nn_argmax": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp]),
 }
 
 _lib = None

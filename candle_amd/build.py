@@ -20,7 +20,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "obj")
 LIB = os.path.join(HERE, "libcandle_hip_quant.so")
 
-SOURCES = ["cq_api.hip", "cq_dequant.hip", "cq_actquant.hip", "cq_matvec.hip", "cq_matmul.hip", "cq_moe.hip", "cq_quantize.hip"]
+SOURCES = ["cq_api.hip", "cq_dequant.hip", "cq_actquant.hip", "cq_matvec.hip", "cq_matmul.hip", "cq_moe.hip", "cq_quantize.hip", "cq_nn.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -32,7 +32,8 @@ FLAGS = [
 
 def _headers_mtime() -> float:
     hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
-    hs.append(os.path.join(os.path.dirname(HERE), "include", "candle_hip_quant.h"))
+    inc = os.path.join(os.path.dirname(HERE), "include")
+    hs += [os.path.join(inc, f) for f in os.listdir(inc) if f.endswith(".h")]
     return max(os.path.getmtime(h) for h in hs)
 
 

@@ -12,8 +12,10 @@
 //       acc[m,n] += d8[m,kb] * ( d[n,kb] * S[m,n] - dmin[n,kb] * M[m,n] ),
 //       M[m,n] = sum_{j<16} bsums16[m,j] * min[n,j/2]          (one extra K=16 MFMA, Q4_K/Q5_K only)
 //   — the same integers the CPU vec_dot sums (k_quants.rs:1460-1540, 1714-1801, 2035-2092).  For Q6_K
-//   the product sc*(q-32) can reach 4096; values above 2048 that are odd round to even in f16
-//   (relative 2^-12 on those elements only).
+//   the product sc*(q-32) can reach 4096, beyond the exact-integer range of f16, so it is fed as two
+//   terms: its f16 rounding and the exact remainder in {-1, 0, 1} (a second MFMA per k-slice).  This
+//   matters: a 1e-4 perturbation of one matmul is amplified to ~1e-2 in a decoder's logits by the
+//   activation quantizers downstream, an exact one is not.
 // Q4_0 / Q8_0 — both operands carry a per-32 f16 scale, so the dequantized values d*(q-8) and d8*q8
 //   are rounded to f16 (relative 2^-11 per operand) and multiplied at full MFMA rate; the result stays
 //   well inside the 1e-3 tolerance (measured ~2e-4) but is not integer-exact like the decode path.
@@ -77,6 +79,7 @@ template <int DT> struct Stage;
 
 template <> struct Stage<CQ_Q4K> {
     static constexpr bool KQ = true, HAS_MIN = true;
+    static constexpr int TERMS = 1;
     struct Raw { u32x4 hdr, q0, q1; };
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int) {
         const uint8_t *blk = row + (int64_t)kb * 144;
@@ -108,6 +111,7 @@ template <> struct Stage<CQ_Q4K> {
 
 template <> struct Stage<CQ_Q5K> {
     static constexpr bool KQ = true, HAS_MIN = true;
+    static constexpr int TERMS = 1;
     struct Raw { u32x4 hdr, h0, h1, q0, q1; };
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int) {
         const uint8_t *blk = row + (int64_t)kb * 176;
@@ -142,6 +146,7 @@ template <> struct Stage<CQ_Q5K> {
 
 template <> struct Stage<CQ_Q6K> {
     static constexpr bool KQ = true, HAS_MIN = false;
+    static constexpr int TERMS = 2;      // sc * (q - 32) reaches 4096: f16 head + exact remainder in {-1, 0, 1}
     // sub-block (g, half) = elements 64g + 32half + [0, 32): half h6 = g >> 1 of the block, quarter = 2*(g&1) + half
     struct Raw { u32x4 l0, l1, h0, h1; uint32_t sc, d; };
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
@@ -162,7 +167,9 @@ template <> struct Stage<CQ_Q6K> {
 #pragma unroll
         for (int j = 0; j < 8; j++) mins[j] = 0;
     }
-    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) {
+    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) { convert2(r, g, half, out, out); }
+    // out = f16(sc * (q - 32)) (rounds odd products above 2048 to even), rem = sc * (q - 32) - out exactly
+    static __device__ __forceinline__ void convert2(const Raw &r, int g, int half, uint32_t out[16], uint32_t rem[16]) {
         const int quarter = 2 * (g & 1) + half;
         const uint32_t sA = h2_splat((float)(int8_t)(r.sc & 0xff)), sB = h2_splat((float)(int8_t)(r.sc >> 8));
         const uint32_t off = h2_splat(-1056.0f);                       // -(1024 + 32)
@@ -175,14 +182,19 @@ template <> struct Stage<CQ_Q6K> {
             uint32_t lo, hi;
             bytes_to_h1024(lo4 | hi2, lo, hi);
             const uint32_t s2 = i < 4 ? sA : sB;                         // l / 16
-            out[2 * i] = pk_mul(pk_add(lo, off), s2);                    // (q - 32) * sc
-            out[2 * i + 1] = pk_mul(pk_add(hi, off), s2);
+            const uint32_t a = pk_add(lo, off), b = pk_add(hi, off);     // q - 32, exact
+            const uint32_t pa = pk_mul(a, s2), pb = pk_mul(b, s2);
+            out[2 * i] = pa;
+            out[2 * i + 1] = pb;
+            rem[2 * i] = pk_fma(a, s2, pa ^ 0x80008000u);                // exact product minus its f16 rounding
+            rem[2 * i + 1] = pk_fma(b, s2, pb ^ 0x80008000u);
         }
     }
 };
 
 template <> struct Stage<CQ_Q4_0> {
     static constexpr bool KQ = false, HAS_MIN = false;
+    static constexpr int TERMS = 1;
     struct Raw { u32x4 qs; uint32_t d; };
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
         const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + half) * 18;
@@ -212,6 +224,7 @@ template <> struct Stage<CQ_Q4_0> {
 
 template <> struct Stage<CQ_Q8_0> {
     static constexpr bool KQ = false, HAS_MIN = false;
+    static constexpr int TERMS = 1;
     struct Raw { u32x4 q0, q1; uint32_t d; };
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
         const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + half) * 34;
@@ -267,6 +280,7 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
     constexpr bool KQ = S::KQ;
     __shared__ __align__(16) _Float16 As[BM * LDK];
     __shared__ __align__(16) _Float16 Bs[BN * LDK];
+    __shared__ __align__(16) _Float16 Bs2[S::TERMS == 2 ? BN * LDK : 8];   // exact remainders of a two-term format
     __shared__ __align__(16) _Float16 Am[BM * 24];    // bsums16 of the super-block, as f16 (row stride 24 halves)
     __shared__ __align__(16) _Float16 Bm[BN * 24];    // sub-block mins duplicated per 16-element group
     __shared__ float sD[BN], sDmin[BN], sD8[BM];
@@ -307,7 +321,13 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
         for (int g = 0; g < 4; g++) {
             // ---- write the staged raw data of (kb, g) to LDS as f16 ----
             uint32_t hv[16];
-            S::convert(wraw, g, half, hv);
+            if constexpr (S::TERMS == 2) {
+                uint32_t hr[16];
+                S::convert2(wraw, g, half, hv, hr);
+                lds_write32h(Bs2 + r_l * LDK + 32 * half, hr);
+            } else {
+                S::convert(wraw, g, half, hv);
+            }
             lds_write32h(Bs + r_l * LDK + 32 * half, hv);
             uint32_t ascale2 = 0;
             if (!KQ) {
@@ -365,6 +385,15 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
                 for (int i = 0; i < 2; i++)
 #pragma unroll
                     for (int j = 0; j < 2; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
+                if constexpr (S::TERMS == 2) {
+#pragma unroll
+                    for (int t = 0; t < 2; t++)
+                        bf[t] = *reinterpret_cast<const half8 *>(Bs2 + (wn * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
+#pragma unroll
+                    for (int i = 0; i < 2; i++)
+#pragma unroll
+                        for (int j = 0; j < 2; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
+                }
             }
             if (KQ && g == 3) {
                 // ---- end of the super-block: mins term and the f32 scales ----

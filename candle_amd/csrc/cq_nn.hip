@@ -1,0 +1,430 @@
+// Decoder glue around the quantized matmuls of candle's quantized llama
+// (candle-transformers/src/models/quantized_llama.rs:191-266, 568-596): embedding lookup, residual add +
+// RMS norm, interleaved rotary embedding + KV-cache append, causal GQA attention over the cache,
+// silu(gate) * up, and greedy argmax.  All f32, like the reference's CPU path.  Token ids and the
+// decode position can be read from device memory so that a whole decode step (including "pick the next
+// token, advance the position") can be captured in a HIP graph and replayed without host round trips.
+#include "cq_device.h"
+#include "../../include/candle_hip_nn.h"
+
+namespace {
+
+__device__ __forceinline__ float block_sum_256(float v, float *red) {     // red: >= 4 floats of LDS
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+// ---- embedding: out[r, :] = table[ids[r], :] (candle_nn::Embedding, index_select) ---------------
+__global__ __launch_bounds__(256) void embedding_kernel(const float *__restrict__ table, const int32_t *__restrict__ ids, float *__restrict__ out,
+                                                        int dim, int64_t vocab) {
+    const int r = blockIdx.x;
+    const int64_t id = ids[r];
+    const bool ok = id >= 0 && id < vocab;
+    const float4 *src = reinterpret_cast<const float4 *>(table + (ok ? id : 0) * dim);
+    float4 *dst = reinterpret_cast<float4 *>(out + (int64_t)r * dim);
+    for (int i = threadIdx.x; i < dim / 4; i += 256) dst[i] = ok ? src[i] : float4{0.f, 0.f, 0.f, 0.f};
+}
+
+// ---- s = x (+ delta); sum_out = s; out = s / sqrt(mean(s^2) + eps) * w  (candle-nn/src/ops.rs:499-510) ----
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float *x, const float *__restrict__ delta, const float *__restrict__ w, float *sum_out,
+                                                       float *__restrict__ out, int dim, float eps) {
+    __shared__ float red[4];
+    const int64_t base = (int64_t)blockIdx.x * dim;
+    const float4 *x4 = reinterpret_cast<const float4 *>(x + base);
+    const float4 *d4 = delta ? reinterpret_cast<const float4 *>(delta + base) : nullptr;
+    float4 *s4 = sum_out ? reinterpret_cast<float4 *>(sum_out + base) : nullptr;
+    const float4 *w4 = reinterpret_cast<const float4 *>(w);
+    float4 *o4 = reinterpret_cast<float4 *>(out + base);
+    const int n4 = dim >> 2;
+    // up to 4 float4 per thread stay in registers (dim <= 4096); longer rows are re-read
+    float4 keep[4];
+    float acc = 0.0f;
+    auto fetch = [&](int i) {
+        float4 v = x4[i];
+        if (d4) {
+            float4 d = d4[i];
+            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        }
+        return v;
+    };
+    auto square = [&](const float4 &v) {
+        acc += v.x * v.x;
+        acc += v.y * v.y;
+        acc += v.z * v.z;
+        acc += v.w * v.w;
+    };
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int i = threadIdx.x + 256 * c;
+        if (i < n4) {
+            keep[c] = fetch(i);
+            if (s4) s4[i] = keep[c];
+            square(keep[c]);
+        }
+    }
+    for (int i = threadIdx.x + 1024; i < n4; i += 256) {
+        const float4 v = fetch(i);
+        if (s4) s4[i] = v;
+        square(v);
+    }
+    const float sum2 = block_sum_256(acc, red);
+    const float m = sqrtf(sum2 / (float)dim + eps);
+    auto emit = [&](int i, const float4 &v) {
+        const float4 a = w4[i];
+        o4[i] = float4{v.x / m * a.x, v.y / m * a.y, v.z / m * a.z, v.w / m * a.w};
+    };
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int i = threadIdx.x + 256 * c;
+        if (i < n4) emit(i, keep[c]);
+    }
+    // x may alias sum_out: each thread re-reads only elements it wrote itself
+    for (int i = threadIdx.x + 1024; i < n4; i += 256) emit(i, s4 ? s4[i] : fetch(i));
+}
+
+// ---- rope_i on q (in place) and k (into the cache), v copied into the cache -------------------------
+// candle-nn/src/rotary_emb.rs:52-70: dst[2i] = x[2i] cos - x[2i+1] sin ; dst[2i+1] = x[2i] sin + x[2i+1] cos,
+// cos/sin rows indexed by the absolute position (quantized_llama.rs:174-189).
+// caches: [n_kv_head][ctx][head_dim]
+__global__ __launch_bounds__(256) void rope_kv_kernel(float *__restrict__ q, const float *__restrict__ k, const float *__restrict__ v,
+                                                      float *__restrict__ k_cache, float *__restrict__ v_cache, const float *__restrict__ cos_t,
+                                                      const float *__restrict__ sin_t, const int32_t *__restrict__ pos_dev, int pos0, int n_head,
+                                                      int n_kv_head, int hd, int ctx, int64_t q_stride, int64_t k_stride, int64_t v_stride) {
+    const int r = blockIdx.x;
+    const int p = pos0 + (pos_dev ? pos_dev[0] : 0) + r;
+    if (p >= ctx) return;
+    const int half = hd >> 1;
+    const float *cs = cos_t + (int64_t)p * half, *sn = sin_t + (int64_t)p * half;
+    float *qr = q + r * q_stride;
+    const float *kr = k + r * k_stride, *vr = v + r * v_stride;
+    for (int i = threadIdx.x; i < n_head * half; i += 256) {
+        const int h = i / half, j = i - h * half;
+        float2 x = *reinterpret_cast<float2 *>(qr + h * hd + 2 * j);
+        const float c = cs[j], s = sn[j];
+        *reinterpret_cast<float2 *>(qr + h * hd + 2 * j) = float2{x.x * c - x.y * s, x.x * s + x.y * c};
+    }
+    for (int i = threadIdx.x; i < n_kv_head * half; i += 256) {
+        const int h = i / half, j = i - h * half;
+        float2 x = *reinterpret_cast<const float2 *>(kr + h * hd + 2 * j);
+        const float c = cs[j], s = sn[j];
+        *reinterpret_cast<float2 *>(k_cache + ((int64_t)h * ctx + p) * hd + 2 * j) = float2{x.x * c - x.y * s, x.x * s + x.y * c};
+        *reinterpret_cast<float2 *>(v_cache + ((int64_t)h * ctx + p) * hd + 2 * j) = *reinterpret_cast<const float2 *>(vr + h * hd + 2 * j);
+    }
+}
+
+// ---- causal attention of `rows` new queries over the cache -------------------------------------------
+// Query row r sits at absolute position p = pos + r and attends keys [0, p] (quantized_llama.rs:246-261:
+// q k^T / sqrt(d), causal mask, softmax_last_dim, . v, with repeat_kv for grouped heads).
+// One workgroup = one kv head x one query row x one split of 256 keys; the G = n_head / n_kv_head query
+// heads that share the kv head are processed together so K and V are read once.
+//   phase 1: thread t owns key j0 + t, dots its 128-float K row against the G query vectors (in LDS)
+//   phase 2: per query head: max, exp, sum over the split
+//   phase 3: lanes own output dims, waves stride over keys, p[j] broadcast from LDS; waves summed via LDS
+// With one split the normalized result is written directly; otherwise (m, l, unnormalized acc) partials
+// go to the workspace and attn_combine_kernel merges them.
+constexpr int ATT_SPLIT = 256;
+
+template <int HD, int G>
+__global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, int64_t q_stride, const float *__restrict__ k_cache,
+                                                   const float *__restrict__ v_cache, float *__restrict__ out, float *__restrict__ part,
+                                                   const int32_t *__restrict__ pos_dev, int pos0, int n_head, int ctx, float scale, int splits) {
+    constexpr int DPL = HD / 64;                  // output dims per lane
+    __shared__ __align__(16) float qs[G * HD];
+    __shared__ float sc[G * ATT_SPLIT];
+    __shared__ float red[4 * G * HD];
+    __shared__ float ml[2 * G];
+    const int kvh = blockIdx.x, r = blockIdx.y, sp = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int kv_len = min(pos0 + (pos_dev ? pos_dev[0] : 0) + r + 1, ctx);
+    const int j0 = sp * ATT_SPLIT;
+    const int cnt = min(kv_len - j0, ATT_SPLIT);      // keys in this split (may be <= 0)
+    const float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
+
+    for (int i = tid; i < G * HD; i += 256) qs[i] = q[r * q_stride + (int64_t)(kvh * G) * HD + i];
+    __syncthreads();
+
+    // ---- phase 1 ----
+    {
+        float acc[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) acc[g] = 0.0f;
+        if (tid < cnt) {
+            const float4 *kr = reinterpret_cast<const float4 *>(kb + (int64_t)(j0 + tid) * HD);
+#pragma unroll 8
+            for (int d = 0; d < HD / 4; d++) {
+                const float4 kk = kr[d];
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    const float4 qq = *reinterpret_cast<const float4 *>(qs + g * HD + 4 * d);
+                    acc[g] += qq.x * kk.x;
+                    acc[g] += qq.y * kk.y;
+                    acc[g] += qq.z * kk.z;
+                    acc[g] += qq.w * kk.w;
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) sc[g * ATT_SPLIT + tid] = tid < cnt ? acc[g] * scale : -INFINITY;
+    }
+    __syncthreads();
+
+    // ---- phase 2: wave w reduces heads g = w, w + 4, ... ----
+    for (int g = wv; g < G; g += 4) {
+        float s[4], m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            s[i] = sc[g * ATT_SPLIT + lane + 64 * i];
+            m = fmaxf(m, s[i]);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        float l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float p = (cnt > 0 && s[i] > -INFINITY) ? __expf(s[i] - m) : 0.0f;
+            sc[g * ATT_SPLIT + lane + 64 * i] = p;
+            l += p;
+        }
+        l = wave_sum(l);
+        if (lane == 0) { ml[2 * g] = m; ml[2 * g + 1] = l; }
+    }
+    __syncthreads();
+
+    // ---- phase 3 ----
+    float o[G][DPL];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int e = 0; e < DPL; e++) o[g][e] = 0.0f;
+    for (int j = wv; j < cnt; j += 4) {
+        float vv[DPL];
+        if (DPL == 2) {
+            const float2 t = *reinterpret_cast<const float2 *>(vb + (int64_t)(j0 + j) * HD + 2 * lane);
+            vv[0] = t.x; vv[DPL - 1] = t.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < DPL; e++) vv[e] = vb[(int64_t)(j0 + j) * HD + DPL * lane + e];
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const float p = sc[g * ATT_SPLIT + j];
+#pragma unroll
+            for (int e = 0; e < DPL; e++) o[g][e] += p * vv[e];
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int e = 0; e < DPL; e++) red[(wv * G + g) * HD + DPL * lane + e] = o[g][e];
+    __syncthreads();
+    for (int i = tid; i < G * HD; i += 256) {
+        const int g = i / HD, d = i - g * HD;
+        const float a = red[(0 * G + g) * HD + d] + red[(1 * G + g) * HD + d] + red[(2 * G + g) * HD + d] + red[(3 * G + g) * HD + d];
+        const int head = kvh * G + g;
+        if (splits == 1) {
+            out[((int64_t)r * n_head + head) * HD + d] = a / ml[2 * g + 1];
+        } else {
+            float *pp = part + (((int64_t)r * n_head + head) * splits + sp) * (HD + 2);
+            pp[2 + d] = a;
+            if (d == 0) { pp[0] = ml[2 * g]; pp[1] = ml[2 * g + 1]; }
+        }
+    }
+}
+
+// merge the splits of one (row, head): out = sum_s e^{m_s - M} acc_s / sum_s e^{m_s - M} l_s
+template <int HD>
+__global__ __launch_bounds__(HD) void attn_combine_kernel(const float *__restrict__ part, float *__restrict__ out, int splits) {
+    const int64_t rh = blockIdx.x;
+    const float *pp = part + rh * splits * (HD + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < splits; s++) M = fmaxf(M, pp[s * (HD + 2) + 1] > 0.0f ? pp[s * (HD + 2)] : -INFINITY);
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < splits; s++) {
+        const float l = pp[s * (HD + 2) + 1];
+        if (l > 0.0f) {
+            const float w = __expf(pp[s * (HD + 2)] - M);
+            num += w * pp[s * (HD + 2) + 2 + threadIdx.x];
+            den += w * l;
+        }
+    }
+    out[rh * HD + threadIdx.x] = num / den;
+}
+
+// ---- out = silu(gate) * up, silu(v) = v / (1 + exp(-v))  (candle-core/src/op.rs Silu; quantized_llama.rs:56-63) ----
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up, float *__restrict__ out, int dim,
+                                                       int64_t gate_stride, int64_t up_stride) {
+    const int r = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= dim / 4) return;
+    const float4 g = reinterpret_cast<const float4 *>(gate + r * gate_stride)[i];
+    const float4 u = reinterpret_cast<const float4 *>(up + r * up_stride)[i];
+    float4 o;
+    o.x = g.x / (1.0f + expf(-g.x)) * u.x;
+    o.y = g.y / (1.0f + expf(-g.y)) * u.y;
+    o.z = g.z / (1.0f + expf(-g.z)) * u.z;
+    o.w = g.w / (1.0f + expf(-g.w)) * u.w;
+    reinterpret_cast<float4 *>(out + (int64_t)r * dim)[i] = o;
+}
+
+// ---- greedy sampling: index of the largest logit, lowest index on ties (Sampling::ArgMax) ----
+// One workgroup.  Optionally appends the token to history[*pos_dev + 1 ...] semantics are the caller's:
+// token_out[0] = idx; if history: history[hist_index] = idx where hist_index = *counter; if counter: *counter += 1.
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, int n, int32_t *__restrict__ token_out,
+                                                      int32_t *__restrict__ history, int32_t *__restrict__ counter, int32_t *__restrict__ pos_dev) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const float v = logits[i];
+        if (v > best || idx == 0x7fffffff) { best = v; idx = i; }      // ascending i per thread: strict > keeps the first
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(idx, o, 64);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = best; bi[threadIdx.x >> 6] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; w++)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        token_out[0] = idx;
+        if (history && counter) history[counter[0]] = idx;
+        if (counter) counter[0] += 1;
+        if (pos_dev) pos_dev[0] += 1;
+    }
+}
+
+inline bool misaligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+template <int HD>
+int launch_attn(int G, dim3 grid, hipStream_t s, const float *q, int64_t q_stride, const float *kc, const float *vc, float *out, float *part,
+                const int32_t *pos_dev, int pos0, int n_head, int ctx, float scale, int splits) {
+#define CQ_ATT(GG)                                                                                                                   \
+    case GG:                                                                                                                         \
+        hipLaunchKernelGGL((attn_kernel<HD, GG>), grid, dim3(256), 0, s, q, q_stride, kc, vc, out, part, pos_dev, pos0, n_head, ctx, \
+                           scale, splits);                                                                                           \
+        break;
+    switch (G) {
+        CQ_ATT(1) CQ_ATT(2) CQ_ATT(4) CQ_ATT(8)
+        default: return CQ_ERR_RANGE;
+    }
+#undef CQ_ATT
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" {
+
+int cq_nn_embedding(const float *table_dev, const int32_t *ids_dev, float *out_dev, int64_t rows, int64_t dim, int64_t vocab, void *stream) {
+    if (rows < 0 || dim <= 0 || vocab <= 0 || dim % 4) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    if (!table_dev || !ids_dev || !out_dev) return CQ_ERR_NULL;
+    if (misaligned(table_dev, 16) || misaligned(out_dev, 16)) return CQ_ERR_ALIGN;
+    if (rows > 0x7fffffffLL || dim > 0x7fffffffLL) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL(embedding_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, table_dev, ids_dev, out_dev, (int)dim, vocab);
+    return (int)hipGetLastError();
+}
+
+int cq_nn_rms_norm(const float *x_dev, const float *delta_dev, const float *weight_dev, float *sum_out_dev, float *out_dev, int64_t rows,
+                   int64_t dim, float eps, void *stream) {
+    if (rows < 0 || dim <= 0 || dim % 4) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    if (!x_dev || !weight_dev || !out_dev) return CQ_ERR_NULL;
+    if (misaligned(x_dev, 16) || misaligned(delta_dev, 16) || misaligned(weight_dev, 16) || misaligned(sum_out_dev, 16) || misaligned(out_dev, 16))
+        return CQ_ERR_ALIGN;
+    if (rows > 0x7fffffffLL || dim > (1 << 24)) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, x_dev, delta_dev, weight_dev, sum_out_dev, out_dev,
+                       (int)dim, eps);
+    return (int)hipGetLastError();
+}
+
+int cq_nn_rope_i_kv(float *q_dev, const float *k_dev, const float *v_dev, float *k_cache_dev, float *v_cache_dev, const float *cos_dev,
+                    const float *sin_dev, const int32_t *pos_dev, int64_t pos, int64_t rows, int64_t n_head, int64_t n_kv_head, int64_t head_dim,
+                    int64_t ctx, int64_t q_stride, int64_t k_stride, int64_t v_stride, void *stream) {
+    if (rows < 0 || n_head <= 0 || n_kv_head <= 0 || head_dim <= 0 || head_dim % 2 || ctx <= 0 || pos < 0) return CQ_ERR_SHAPE;
+    if (q_stride < n_head * head_dim || k_stride < n_kv_head * head_dim || v_stride < n_kv_head * head_dim) return CQ_ERR_SHAPE;
+    if (q_stride % 2 || k_stride % 2 || v_stride % 2) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    if (!q_dev || !k_dev || !v_dev || !k_cache_dev || !v_cache_dev || !cos_dev || !sin_dev) return CQ_ERR_NULL;
+    if (misaligned(q_dev, 8) || misaligned(k_dev, 8) || misaligned(v_dev, 8) || misaligned(k_cache_dev, 8) || misaligned(v_cache_dev, 8))
+        return CQ_ERR_ALIGN;
+    if (!pos_dev && pos + rows > ctx) return CQ_ERR_RANGE;
+    if (rows > 0x7fffffffLL || ctx > 0x7fffffffLL) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL(rope_kv_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, q_dev, k_dev, v_dev, k_cache_dev, v_cache_dev,
+                       cos_dev, sin_dev, pos_dev, (int)pos, (int)n_head, (int)n_kv_head, (int)head_dim, (int)ctx, q_stride, k_stride, v_stride);
+    return (int)hipGetLastError();
+}
+
+static int64_t attn_splits(int64_t max_kv_len) { return (max_kv_len + ATT_SPLIT - 1) / ATT_SPLIT; }
+
+int64_t cq_nn_attention_workspace_bytes(int64_t rows, int64_t n_head, int64_t head_dim, int64_t max_kv_len) {
+    if (rows < 0 || n_head <= 0 || head_dim <= 0 || max_kv_len <= 0) return -1;
+    const int64_t splits = attn_splits(max_kv_len);
+    return splits <= 1 ? 0 : rows * n_head * splits * (head_dim + 2) * 4;
+}
+
+int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_dev, const float *v_cache_dev, float *out_dev,
+                    const int32_t *pos_dev, int64_t pos, int64_t rows, int64_t n_head, int64_t n_kv_head, int64_t head_dim, int64_t ctx,
+                    int64_t max_kv_len, float scale, void *workspace_dev, int64_t workspace_bytes, void *stream) {
+    if (rows < 0 || n_head <= 0 || n_kv_head <= 0 || n_head % n_kv_head || ctx <= 0 || pos < 0 || max_kv_len <= 0 || max_kv_len > ctx)
+        return CQ_ERR_SHAPE;
+    if (q_stride < n_head * head_dim) return CQ_ERR_SHAPE;
+    if (head_dim != 64 && head_dim != 128) return CQ_ERR_RANGE;
+    if (rows == 0) return CQ_OK;
+    if (!q_dev || !k_cache_dev || !v_cache_dev || !out_dev) return CQ_ERR_NULL;
+    if (misaligned(k_cache_dev, 16) || misaligned(v_cache_dev, 16)) return CQ_ERR_ALIGN;
+    if (!pos_dev && pos + rows > max_kv_len) return CQ_ERR_RANGE;
+    const int64_t splits = attn_splits(max_kv_len);
+    const int64_t need = cq_nn_attention_workspace_bytes(rows, n_head, head_dim, max_kv_len);
+    if (need > 0 && (!workspace_dev || workspace_bytes < need)) return CQ_ERR_WORKSPACE;
+    if (rows > 65535 || splits > 65535 || ctx > 0x7fffffffLL) return CQ_ERR_RANGE;
+    const int G = (int)(n_head / n_kv_head);
+    dim3 grid((unsigned)n_kv_head, (unsigned)rows, (unsigned)splits);
+    hipStream_t s = (hipStream_t)stream;
+    int rc = head_dim == 128 ? launch_attn<128>(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev, pos_dev,
+                                                (int)pos, (int)n_head, (int)ctx, scale, (int)splits)
+                             : launch_attn<64>(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev, pos_dev,
+                                               (int)pos, (int)n_head, (int)ctx, scale, (int)splits);
+    if (rc) return rc;
+    if (splits > 1) {
+        if (head_dim == 128)
+            hipLaunchKernelGGL((attn_combine_kernel<128>), dim3((unsigned)(rows * n_head)), dim3(128), 0, s, (const float *)workspace_dev, out_dev,
+                               (int)splits);
+        else
+            hipLaunchKernelGGL((attn_combine_kernel<64>), dim3((unsigned)(rows * n_head)), dim3(64), 0, s, (const float *)workspace_dev, out_dev,
+                               (int)splits);
+        return (int)hipGetLastError();
+    }
+    return CQ_OK;
+}
+
+int cq_nn_silu_mul(const float *gate_dev, const float *up_dev, float *out_dev, int64_t rows, int64_t dim, int64_t gate_stride, int64_t up_stride,
+                   void *stream) {
+    if (rows < 0 || dim <= 0 || dim % 4 || gate_stride < dim || up_stride < dim || gate_stride % 4 || up_stride % 4) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    if (!gate_dev || !up_dev || !out_dev) return CQ_ERR_NULL;
+    if (misaligned(gate_dev, 16) || misaligned(up_dev, 16) || misaligned(out_dev, 16)) return CQ_ERR_ALIGN;
+    if (rows > 65535 || dim > 0x7fffffffLL) return CQ_ERR_RANGE;
+    dim3 grid((unsigned)((dim / 4 + 255) / 256), (unsigned)rows);
+    hipLaunchKernelGGL(silu_mul_kernel, grid, dim3(256), 0, (hipStream_t)stream, gate_dev, up_dev, out_dev, (int)dim, gate_stride, up_stride);
+    return (int)hipGetLastError();
+}
+
+int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
+                 void *stream) {
+    if (n <= 0) return CQ_ERR_SHAPE;
+    if (!logits_dev || !token_out_dev) return CQ_ERR_NULL;
+    if (n > 0x7fffffffLL) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits_dev, (int)n, token_out_dev, history_dev, counter_dev,
+                       pos_dev);
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"

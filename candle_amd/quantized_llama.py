@@ -1,0 +1,356 @@
+"""Host-side mirror of candle's quantized llama decoder over the HIP C ABI.
+
+Mirrors candle-transformers/src/models/quantized_llama.rs: ``LayerWeights`` (:150-266), ``Mlp`` (:49-63),
+``ModelWeights::forward`` (:568-596) and ``precomput_freqs_cis`` (:284-300), for the dense (non-MoE) llama
+architecture with interleaved RoPE.  Every computation is a call into libcandle_hip_quant.so
+(quantized matmuls from candle_hip_quant.h, f32 glue from candle_hip_nn.h); PyTorch only provides device
+memory, the stream and HIP-graph capture.
+
+Differences from the reference that do not change results:
+  * the KV cache is preallocated ([n_kv_head, ctx, head_dim] per layer) instead of grown by Tensor::cat;
+  * attention_wq|attention_wk and feed_forward_w1|feed_forward_w3 are stored back to back, so when their
+    formats agree each pair runs as one matmul over the concatenated rows (rows are independent);
+  * a greedy decode step can be captured once in a HIP graph and replayed: the next token and the
+    position live in device memory (``generate_greedy``).
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+import time
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+from .quantized import GgmlDType, QStorage, QTensor
+
+
+@dataclasses.dataclass
+class Config:
+    n_layer: int = 32
+    hidden: int = 4096
+    n_head: int = 32
+    n_kv_head: int = 8
+    head_dim: int = 128
+    ffn: int = 14336
+    vocab: int = 128256
+    rope_theta: float = 500000.0      # llama.rope.freq_base of Llama-3 files (quantized_llama.rs:455-458 reads it)
+    rms_eps: float = 1e-5             # llama.attention.layer_norm_rms_epsilon
+    ctx: int = 2048                   # rows of the cos/sin tables and of the KV cache (MAX_SEQ_LEN in the reference)
+
+    @staticmethod
+    def llama3_8b() -> "Config":
+        return Config()
+
+
+def precomput_freqs_cis(head_dim: int, freq_base: float, max_seq_len: int):
+    """cos/sin tables [max_seq_len, head_dim/2] in f32 (quantized_llama.rs:284-300)."""
+    i = np.arange(0, head_dim, 2, dtype=np.float32)
+    theta = (np.float32(1.0) / np.power(np.float32(freq_base), i / np.float32(head_dim))).astype(np.float32)
+    idx = np.arange(max_seq_len, dtype=np.float32).reshape(-1, 1)
+    idx_theta = (idx * theta.reshape(1, -1)).astype(np.float32)
+    return np.cos(idx_theta).astype(np.float32), np.sin(idx_theta).astype(np.float32)
+
+
+# tensor order inside one layer's slab: pairs that can be fused are adjacent
+_LAYER_ORDER = ("attention_wq", "attention_wk", "attention_wv", "attention_wo", "feed_forward_w1", "feed_forward_w3", "feed_forward_w2")
+
+
+def _layer_shapes(cfg: Config) -> Dict[str, tuple]:
+    qd, kvd = cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim
+    return {"attention_wq": (qd, cfg.hidden), "attention_wk": (kvd, cfg.hidden), "attention_wv": (kvd, cfg.hidden),
+            "attention_wo": (cfg.hidden, qd), "feed_forward_w1": (cfg.ffn, cfg.hidden), "feed_forward_w3": (cfg.ffn, cfg.hidden),
+            "feed_forward_w2": (cfg.hidden, cfg.ffn)}
+
+
+Q4_K_M = {"attention_wq": GgmlDType.Q4K, "attention_wk": GgmlDType.Q4K, "attention_wv": GgmlDType.Q6K, "attention_wo": GgmlDType.Q4K,
+          "feed_forward_w1": GgmlDType.Q4K, "feed_forward_w3": GgmlDType.Q4K, "feed_forward_w2": GgmlDType.Q6K, "output": GgmlDType.Q4K}
+
+
+class _W:
+    """One quantized weight inside the model's slab: device pointer, format, shape."""
+    __slots__ = ("ptr", "dtype", "n", "k", "nbytes")
+
+    def __init__(self, ptr: int, dtype: GgmlDType, n: int, k: int, nbytes: int):
+        self.ptr, self.dtype, self.n, self.k, self.nbytes = ptr, dtype, n, k, nbytes
+
+
+class LayerWeights:
+    def __init__(self):
+        self.w: Dict[str, _W] = {}
+        self.attention_norm: Optional[torch.Tensor] = None
+        self.ffn_norm: Optional[torch.Tensor] = None
+        self.k_cache: Optional[torch.Tensor] = None
+        self.v_cache: Optional[torch.Tensor] = None
+
+
+class ModelWeights:
+    """quantized_llama::ModelWeights for one GPU.  Build with ``random_init`` or ``from_blocks``."""
+
+    def __init__(self, cfg: Config, device="cuda:0"):
+        if cfg.hidden % 256 or cfg.ffn % 256 or (cfg.n_head * cfg.head_dim) % 256:
+            raise ValueError("hidden, ffn and n_head*head_dim must be multiples of 256 (K-quant super-blocks)")
+        if cfg.n_head % cfg.n_kv_head:
+            raise ValueError("n_head must be a multiple of n_kv_head")
+        self.cfg = cfg
+        self.device = torch.device(device)
+        self.L = _lib.lib()
+        self.layers: List[LayerWeights] = []
+        self.tok_embeddings: Optional[torch.Tensor] = None     # f32 [vocab, hidden] (the reference dequantizes token_embd)
+        self.norm: Optional[torch.Tensor] = None
+        self.output: Optional[_W] = None
+        self._slab: Optional[torch.Tensor] = None
+        self._graph = None
+        self._graph_key = None
+
+    # ------------------------------------------------------------------------------------------ construction
+    def _alloc(self, dtypes: Dict[str, GgmlDType]):
+        cfg, L = self.cfg, self.L
+        shapes = _layer_shapes(cfg)
+        total, plan = 0, []
+        for li in range(cfg.n_layer):
+            for name in _LAYER_ORDER:
+                n, k = shapes[name]
+                nb = L.cq_storage_bytes(int(dtypes[name]), n * k)
+                if nb < 0:
+                    raise ValueError(f"{name}: {n}x{k} is not a whole number of {dtypes[name].name} blocks")
+                plan.append((li, name, total, nb, n, k))
+                total += (nb + 255) // 256 * 256
+        nb = L.cq_storage_bytes(int(dtypes["output"]), cfg.vocab * cfg.hidden)
+        plan.append((-1, "output", total, nb, cfg.vocab, cfg.hidden))
+        total += (nb + 255) // 256 * 256
+        self._slab = torch.empty(total, dtype=torch.uint8, device=self.device)
+        base = self._slab.data_ptr()
+        self.layers = [LayerWeights() for _ in range(cfg.n_layer)]
+        for li, name, off, nb, n, k in plan:
+            w = _W(base + off, dtypes[name], n, k, nb)
+            if li < 0:
+                self.output = w
+            else:
+                self.layers[li].w[name] = w
+        f32 = dict(dtype=torch.float32, device=self.device)
+        for lw in self.layers:
+            lw.k_cache = torch.zeros((cfg.n_kv_head, cfg.ctx, cfg.head_dim), **f32)
+            lw.v_cache = torch.zeros((cfg.n_kv_head, cfg.ctx, cfg.head_dim), **f32)
+        cos, sin = precomput_freqs_cis(cfg.head_dim, cfg.rope_theta, cfg.ctx)
+        self.cos = torch.from_numpy(cos).to(self.device)
+        self.sin = torch.from_numpy(sin).to(self.device)
+        self._alloc_activations(max_rows=1)
+        # device-side decode state for graph replay
+        self.token_dev = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self.pos_dev = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self.counter_dev = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self.history_dev = torch.zeros(cfg.ctx, dtype=torch.int32, device=self.device)
+        return plan
+
+    def _alloc_activations(self, max_rows: int):
+        cfg, L = self.cfg, self.L
+        qd, kvd = cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim
+        f32 = dict(dtype=torch.float32, device=self.device)
+        self.max_rows = max_rows
+        self._graph = None                 # a captured step holds the old buffer addresses
+        self.x = torch.empty((max_rows, cfg.hidden), **f32)
+        self.xn = torch.empty((max_rows, cfg.hidden), **f32)
+        self.qk = torch.empty((max_rows, qd + kvd), **f32)
+        self.v = torch.empty((max_rows, kvd), **f32)
+        self.att = torch.empty((max_rows, qd), **f32)
+        self.delta = torch.empty((max_rows, cfg.hidden), **f32)
+        self.gu = torch.empty((max_rows, 2 * cfg.ffn), **f32)
+        self.h = torch.empty((max_rows, cfg.ffn), **f32)
+        self.logits = torch.empty((1, cfg.vocab), **f32)
+        need = 0
+        for (n, k) in list(_layer_shapes(cfg).values()) + [(qd + kvd, cfg.hidden), (2 * cfg.ffn, cfg.hidden)]:
+            for dt in (GgmlDType.Q4K, GgmlDType.Q8_0):      # K-quant and Q*_0 scratch layouts
+                need = max(need, L.cq_qmatmul_workspace_bytes(int(dt), max_rows, k, n))
+        need = max(need, L.cq_qmatmul_workspace_bytes(int(GgmlDType.Q4K), 1, cfg.hidden, cfg.vocab))
+        self.ws = torch.empty(max(need, 256), dtype=torch.uint8, device=self.device)
+        att_ws = L.cq_nn_attention_workspace_bytes(max_rows, cfg.n_head, cfg.head_dim, cfg.ctx)
+        self.att_ws = torch.empty(max(att_ws, 256), dtype=torch.uint8, device=self.device)
+
+    @classmethod
+    def random_init(cls, cfg: Config, seed: int = 0, device="cuda:0", dtypes: Optional[Dict[str, GgmlDType]] = None,
+                    weight_scale: float = 0.02) -> "ModelWeights":
+        """Random-init weights ~N(0, weight_scale) quantized on the device (norm weights = 1, f32 embedding table)."""
+        self = cls(cfg, device)
+        dtypes = dict(Q4_K_M if dtypes is None else dtypes)
+        plan = self._alloc(dtypes)
+        gen = torch.Generator(device=self.device)
+        gen.manual_seed(seed)
+        base = self._slab.data_ptr()
+        for li, name, off, nb, n, k in plan:
+            wf = torch.randn((n, k), generator=gen, device=self.device, dtype=torch.float32) * weight_scale
+            _lib.check("cq_quantize", self.L.cq_quantize(int(dtypes[name]), wf.data_ptr(), base + off, n * k, None))
+            torch.cuda.synchronize(self.device)
+            del wf
+        self.tok_embeddings = torch.randn((cfg.vocab, cfg.hidden), generator=gen, device=self.device, dtype=torch.float32) * weight_scale
+        ones = torch.ones(cfg.hidden, dtype=torch.float32, device=self.device)
+        for lw in self.layers:
+            lw.attention_norm, lw.ffn_norm = ones, ones
+        self.norm = ones
+        return self
+
+    @classmethod
+    def from_blocks(cls, cfg: Config, tensors: dict, device="cuda:0") -> "ModelWeights":
+        """Build from host data: ``tensors[name] = (GgmlDType, block bytes)`` for ``output`` and
+        ``blk.{i}.{attention_wq,...}``, f32 arrays for ``tok_embeddings``, ``norm``, ``blk.{i}.attention_norm``,
+        ``blk.{i}.ffn_norm`` (the tensors ModelWeights::from_gguf reads, quantized_llama.rs:470-540)."""
+        self = cls(cfg, device)
+        dtypes = {name: GgmlDType(tensors[f"blk.0.{name}"][0]) for name in _LAYER_ORDER}
+        dtypes["output"] = GgmlDType(tensors["output"][0])
+        plan = self._alloc(dtypes)
+        for li, name, off, nb, n, k in plan:
+            dt, blocks = tensors["output" if li < 0 else f"blk.{li}.{name}"]
+            if GgmlDType(dt) != dtypes[name]:
+                raise ValueError("every layer must use the same format per tensor role")
+            raw = np.frombuffer(bytes(blocks), dtype=np.uint8)
+            if raw.size != nb:
+                raise ValueError(f"{name}: expected {nb} bytes of blocks, got {raw.size}")
+            self._slab[off:off + nb].copy_(torch.from_numpy(raw.copy()))
+        as_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device)
+        self.tok_embeddings = as_dev(tensors["tok_embeddings"])
+        self.norm = as_dev(tensors["norm"])
+        for i, lw in enumerate(self.layers):
+            lw.attention_norm = as_dev(tensors[f"blk.{i}.attention_norm"])
+            lw.ffn_norm = as_dev(tensors[f"blk.{i}.ffn_norm"])
+        torch.cuda.synchronize(self.device)
+        return self
+
+    def weight_bytes_per_token(self) -> int:
+        """Quantized weight bytes one decode step streams (every matmul weight once)."""
+        return sum(w.nbytes for lw in self.layers for w in lw.w.values()) + self.output.nbytes
+
+    def clear_kv_cache(self):
+        """quantized_llama.rs:558-566 — with a preallocated cache only the position matters."""
+        self.pos_dev.zero_()
+
+    # ------------------------------------------------------------------------------------------ forward
+    def _mm(self, w: _W, n: int, src: torch.Tensor, dst_ptr: int, rows: int, sp):
+        """QMatMul::forward of `rows` f32 rows of `src` with weight rows [w.ptr, +n rows) into dst_ptr."""
+        L = self.L
+        _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(int(w.dtype), w.ptr, src.data_ptr(), 0, dst_ptr, 0, rows, w.k, n,
+                                                              self.ws.data_ptr(), self.ws.numel(), sp))
+
+    def _enqueue(self, ids_ptr: int, rows: int, pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
+        """All kernels of ModelWeights::forward (quantized_llama.rs:568-596) for `rows` new tokens; logits of the last."""
+        cfg, L = self.cfg, self.L
+        qd, kvd = cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim
+        scale = float(np.float32(1.0 / math.sqrt(cfg.head_dim)))
+        ck = _lib.check
+        x, xn, qk, v, att, delta, gu, h = self.x, self.xn, self.qk, self.v, self.att, self.delta, self.gu, self.h
+        ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), rows, cfg.hidden, cfg.vocab, sp))
+        for li, lw in enumerate(self.layers):
+            w = lw.w
+            # x (+= mlp output of the previous layer); xn = attention_norm(x)          :579-583, :590-592
+            ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr(), delta.data_ptr() if li else None, lw.attention_norm.data_ptr(),
+                                                 x.data_ptr() if li else None, xn.data_ptr(), rows, cfg.hidden, cfg.rms_eps, sp))
+            # q, k, v projections                                                         :200-202
+            wq, wk, wv = w["attention_wq"], w["attention_wk"], w["attention_wv"]
+            if wq.dtype == wk.dtype and wk.ptr == wq.ptr + wq.nbytes:
+                self._mm(wq, qd + kvd, xn, qk.data_ptr(), rows, sp)
+                q_ptr, k_ptr, qs, ks = qk.data_ptr(), qk.data_ptr() + 4 * qd, qd + kvd, qd + kvd
+            else:
+                self._mm(wq, qd, xn, qk.data_ptr(), rows, sp)
+                self._mm(wk, kvd, xn, qk.data_ptr() + 4 * rows * qd, rows, sp)
+                q_ptr, k_ptr, qs, ks = qk.data_ptr(), qk.data_ptr() + 4 * rows * qd, qd, kvd
+            self._mm(wv, kvd, xn, v.data_ptr(), rows, sp)
+            # rope on q and k, append k and v to the cache                                :217-233
+            ck("cq_nn_rope_i_kv", L.cq_nn_rope_i_kv(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
+                                                   self.cos.data_ptr(), self.sin.data_ptr(), pos_dev_ptr, pos, rows, cfg.n_head, cfg.n_kv_head,
+                                                   cfg.head_dim, cfg.ctx, qs, ks, kvd, sp))
+            # softmax(q k^T / sqrt(d) + causal mask) v                                    :246-261
+            ck("cq_nn_attention", L.cq_nn_attention(q_ptr, qs, lw.k_cache.data_ptr(), lw.v_cache.data_ptr(), att.data_ptr(), pos_dev_ptr, pos,
+                                                   rows, cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
+                                                   self.att_ws.data_ptr(), self.att_ws.numel(), sp))
+            self._mm(w["attention_wo"], cfg.hidden, att, delta.data_ptr(), rows, sp)    # :264
+            # x += attn; xn = ffn_norm(x)                                                 :584-589
+            ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr(), delta.data_ptr(), lw.ffn_norm.data_ptr(), x.data_ptr(), xn.data_ptr(), rows,
+                                                 cfg.hidden, cfg.rms_eps, sp))
+            # w2(silu(w1 x) * w3 x)                                                       :56-63
+            w1, w3 = w["feed_forward_w1"], w["feed_forward_w3"]
+            if w1.dtype == w3.dtype and w3.ptr == w1.ptr + w1.nbytes:
+                self._mm(w1, 2 * cfg.ffn, xn, gu.data_ptr(), rows, sp)
+                g_ptr, u_ptr, gs = gu.data_ptr(), gu.data_ptr() + 4 * cfg.ffn, 2 * cfg.ffn
+            else:
+                self._mm(w1, cfg.ffn, xn, gu.data_ptr(), rows, sp)
+                self._mm(w3, cfg.ffn, xn, gu.data_ptr() + 4 * rows * cfg.ffn, rows, sp)
+                g_ptr, u_ptr, gs = gu.data_ptr(), gu.data_ptr() + 4 * rows * cfg.ffn, cfg.ffn
+            ck("cq_nn_silu_mul", L.cq_nn_silu_mul(g_ptr, u_ptr, h.data_ptr(), rows, cfg.ffn, gs, gs, sp))
+            self._mm(w["feed_forward_w2"], cfg.hidden, h, delta.data_ptr(), rows, sp)
+        # last token only: x += mlp; final norm; output head                              :593-596
+        last = 4 * (rows - 1) * cfg.hidden
+        ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr() + last, delta.data_ptr() + last, self.norm.data_ptr(), None, xn.data_ptr(), 1,
+                                             cfg.hidden, cfg.rms_eps, sp))
+        self._mm(self.output, cfg.vocab, xn, self.logits.data_ptr(), 1, sp)
+
+    def forward(self, x: torch.Tensor, index_pos: int) -> torch.Tensor:
+        """ModelWeights::forward: token ids [1, seq_len] at positions index_pos.. -> logits [1, vocab] of the last token."""
+        if x.dim() != 2 or x.shape[0] != 1:
+            raise ValueError(f"expected token ids of shape (1, seq_len), got {tuple(x.shape)}")
+        rows = int(x.shape[1])
+        if rows == 0 or index_pos < 0 or index_pos + rows > self.cfg.ctx:
+            raise ValueError(f"positions {index_pos}..{index_pos + rows} outside the context of {self.cfg.ctx}")
+        if rows > self.max_rows:
+            self._alloc_activations(rows)
+        ids = x.to(device=self.device, dtype=torch.int32).contiguous()
+        sp = torch.cuda.current_stream(self.device).cuda_stream
+        self._enqueue(ids.data_ptr(), rows, index_pos, None, index_pos + rows, sp)
+        return self.logits.clone()
+
+    # ------------------------------------------------------------------------------------------ greedy decode
+    def _decode_step_dev(self, max_kv_len: int, sp) -> None:
+        """One greedy step driven entirely from device state: token_dev at position pos_dev -> next token_dev, pos_dev + 1."""
+        self._enqueue(self.token_dev.data_ptr(), 1, 0, self.pos_dev.data_ptr(), max_kv_len, sp)
+        _lib.check("cq_nn_argmax", self.L.cq_nn_argmax(self.logits.data_ptr(), self.cfg.vocab, self.token_dev.data_ptr(),
+                                                       self.history_dev.data_ptr(), self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), sp))
+
+    def generate_greedy(self, prompt: Sequence[int], n_new: int, use_graph: bool = True) -> dict:
+        """The loop of candle-examples/examples/quantized/main.rs:616-690 with temperature <= 0 (Sampling::ArgMax):
+        prefill the prompt in one forward, pick the arg-max token, then n_new - 1 single-token steps.
+        Returns the generated tokens and the wall-clock split prompt / decode, as the example prints them."""
+        cfg = self.cfg
+        prompt = [int(t) for t in prompt]
+        if len(prompt) + n_new > cfg.ctx:
+            raise ValueError("prompt + generated tokens exceed the context")
+        dev = self.device
+        torch.cuda.synchronize(dev)
+        t0 = time.perf_counter()
+        logits = self.forward(torch.tensor([prompt], dtype=torch.int32, device=dev), 0)
+        stream = torch.cuda.current_stream(dev)
+        self.counter_dev.zero_()
+        self.pos_dev.fill_(len(prompt) - 1)       # argmax advances it to the position of the token it emits
+        _lib.check("cq_nn_argmax", self.L.cq_nn_argmax(logits.data_ptr(), cfg.vocab, self.token_dev.data_ptr(), self.history_dev.data_ptr(),
+                                                       self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), stream.cuda_stream))
+        torch.cuda.synchronize(dev)
+        t1 = time.perf_counter()
+        prompt_seconds = t1 - t0
+        steps = n_new - 1
+        max_kv = len(prompt) + n_new
+        if steps > 0:
+            if use_graph:
+                key = max_kv
+                if self._graph is None or self._graph_key != key:
+                    side = torch.cuda.Stream(device=dev)
+                    # capture must not disturb the live decode state: save and restore it around the warm-up run
+                    saved = (self.token_dev.clone(), self.pos_dev.clone(), self.counter_dev.clone())
+                    with torch.cuda.stream(side):
+                        self._decode_step_dev(max_kv, side.cuda_stream)
+                        side.synchronize()
+                        g = torch.cuda.CUDAGraph()
+                        with torch.cuda.graph(g, stream=side):
+                            self._decode_step_dev(max_kv, torch.cuda.current_stream(dev).cuda_stream)
+                    torch.cuda.synchronize(dev)
+                    self.token_dev.copy_(saved[0]); self.pos_dev.copy_(saved[1]); self.counter_dev.copy_(saved[2])
+                    torch.cuda.synchronize(dev)
+                    self._graph, self._graph_key = g, key
+                t1 = time.perf_counter()
+                for _ in range(steps):
+                    self._graph.replay()
+            else:
+                for _ in range(steps):
+                    self._decode_step_dev(max_kv, stream.cuda_stream)
+        torch.cuda.synchronize(dev)
+        t2 = time.perf_counter()
+        tokens = self.history_dev[:n_new].cpu().tolist()
+        return {"tokens": tokens, "prompt_seconds": prompt_seconds, "decode_seconds": t2 - t1, "decode_steps": steps}

@@ -1,0 +1,70 @@
+/*
+ * candle_hip_nn.h — C ABI of the f32 decoder glue that sits between the quantized matmuls of candle's
+ * quantized llama (candle-transformers/src/models/quantized_llama.rs:191-266, 568-596).
+ *
+ * Same library (libcandle_hip_quant.so) and same conventions as candle_hip_quant.h: device pointers,
+ * caller-owned buffers, nothing allocated or synchronized, everything enqueued on `stream`
+ * (a hipStream_t passed as void*), status codes from enum cq_status.
+ *
+ * Position and token arguments exist in two forms so that one decode step can be captured in a HIP
+ * graph and replayed: `pos` is a host integer, `pos_dev` an optional device int32 that is ADDED to it
+ * when not NULL; cq_nn_argmax can write the chosen token and advance the device position itself.
+ */
+#ifndef CANDLE_HIP_NN_H
+#define CANDLE_HIP_NN_H
+
+#include <stdint.h>
+
+#include "candle_hip_quant.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* out[r, :] = table[ids[r], :] — candle_nn::Embedding::forward (candle-nn/src/embedding.rs), used as
+ * tok_embeddings in quantized_llama.rs:577.  table [vocab, dim] f32, dim % 4 == 0, 16-byte aligned.
+ * An id outside [0, vocab) yields a zero row (the reference returns an error from index_select). */
+int cq_nn_embedding(const float *table_dev, const int32_t *ids_dev, float *out_dev, int64_t rows, int64_t dim, int64_t vocab, void *stream);
+
+/* Residual add + RMS norm: s = x (+ delta when delta_dev != NULL); sum_out = s (when sum_out_dev != NULL,
+ * may alias x_dev); out = s / sqrt(mean(s^2) + eps) * weight.
+ * candle_nn::ops::rms_norm CPU kernel (candle-nn/src/ops.rs:499-510) preceded by the `(attn + residual)`
+ * / `(x + residual)` adds of quantized_llama.rs:584-591.  rows x dim, dim % 4 == 0. */
+int cq_nn_rms_norm(const float *x_dev, const float *delta_dev, const float *weight_dev, float *sum_out_dev, float *out_dev, int64_t rows,
+                   int64_t dim, float eps, void *stream);
+
+/* Interleaved rotary embedding of q (in place) and k, and KV-cache append:
+ * candle_nn::rotary_emb::rope_i (candle-nn/src/rotary_emb.rs:52-70) as called from
+ * LayerWeights::apply_rotary_emb (quantized_llama.rs:174-189), followed by the Tensor::cat of
+ * quantized_llama.rs:222-233 done as a write into a preallocated cache.
+ * Row r has absolute position p = pos + *pos_dev + r.  q [rows, n_head*head_dim] (row stride q_stride),
+ * k, v [rows, n_kv_head*head_dim]; caches [n_kv_head, ctx, head_dim]; cos, sin [>= p_max+1, head_dim/2]. */
+int cq_nn_rope_i_kv(float *q_dev, const float *k_dev, const float *v_dev, float *k_cache_dev, float *v_cache_dev, const float *cos_dev,
+                    const float *sin_dev, const int32_t *pos_dev, int64_t pos, int64_t rows, int64_t n_head, int64_t n_kv_head, int64_t head_dim,
+                    int64_t ctx, int64_t q_stride, int64_t k_stride, int64_t v_stride, void *stream);
+
+/* Causal grouped-query attention of `rows` new queries over the cache (quantized_llama.rs:246-261:
+ * repeat_kv, q k^T / sqrt(d), mask, softmax_last_dim, . v, transpose back to [rows, n_head*head_dim]).
+ * Query row r attends keys [0, pos + *pos_dev + r].  max_kv_len bounds pos + *pos_dev + rows and fixes
+ * the launch geometry (keys are processed in splits of 256; more than one split needs the workspace).
+ * head_dim 64 or 128; n_head / n_kv_head in {1, 2, 4, 8}. */
+int64_t cq_nn_attention_workspace_bytes(int64_t rows, int64_t n_head, int64_t head_dim, int64_t max_kv_len);
+int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_dev, const float *v_cache_dev, float *out_dev,
+                    const int32_t *pos_dev, int64_t pos, int64_t rows, int64_t n_head, int64_t n_kv_head, int64_t head_dim, int64_t ctx,
+                    int64_t max_kv_len, float scale, void *workspace_dev, int64_t workspace_bytes, void *stream);
+
+/* out = silu(gate) * up with silu(v) = v / (1 + exp(-v)): Mlp::forward, quantized_llama.rs:56-63
+ * (candle_nn::ops::silu, candle-core/src/op.rs Silu::f32).  gate/up rows may be strided views of one buffer. */
+int cq_nn_silu_mul(const float *gate_dev, const float *up_dev, float *out_dev, int64_t rows, int64_t dim, int64_t gate_stride, int64_t up_stride,
+                   void *stream);
+
+/* Greedy sampling (LogitsProcessor with Sampling::ArgMax, candle-examples/examples/quantized/main.rs:603-604):
+ * token_out[0] = index of the largest logit (lowest index on ties).  Optional bookkeeping for graph replay:
+ * history_dev[*counter_dev] = token; *counter_dev += 1; *pos_dev += 1. */
+int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
+                 void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

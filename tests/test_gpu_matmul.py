@@ -121,10 +121,9 @@ def test_matmul_vs_oracle(dtype, m):
 
 
 def prefill_bound(dtype):
-    """More than 8 rows run on the f16 matrix cores.  Q4_K / Q5_K operands are exact integers there; Q6_K
-    rounds the odd products scale * (q - 32) above 2048 to even; Q4_0 / Q8_0 operands are the dequantized
-    values rounded to f16."""
-    return {oracle.Q4K: TIGHT, oracle.Q5K: TIGHT}.get(dtype, 5e-4)
+    """More than 8 rows run on the f16 matrix cores.  K-quant operands are exact integers there (Q6_K as an
+    f16 head plus an exact remainder term); Q4_0 / Q8_0 operands are the dequantized values rounded to f16."""
+    return {oracle.Q4K: TIGHT, oracle.Q5K: TIGHT, oracle.Q6K: TIGHT}.get(dtype, 5e-4)
 
 
 @pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])

@@ -1,0 +1,178 @@
+"""GPU parity of the f32 decoder glue (include/candle_hip_nn.h) against the numpy restatement of candle's CPU ops.
+
+Tolerances: these are f32 ops whose only difference from the CPU path is summation order and the
+device exp/sqrt/division, so each result is checked to 1e-5 relative L2 (far inside the 1e-3 bar of the matmul path)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import llama_oracle as lo
+from tests.util import normal, rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def L():
+    from candle_amd import _lib
+    return _lib.lib()
+
+
+_ALIVE = []
+
+
+def dev(a, dtype=None):
+    """Host array -> device tensor that stays alive until the end of the test (the C ABI takes raw pointers)."""
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    t = (t if dtype is None else t.to(dtype)).cuda()
+    _ALIVE.append(t)
+    return t
+
+
+@pytest.fixture(autouse=True)
+def _release_device_tensors():
+    yield
+    torch.cuda.synchronize()
+    _ALIVE.clear()
+
+
+def ok(status):
+    assert status == 0, status
+
+
+def test_embedding_rows_and_out_of_range():
+    table = normal(1, (50, 64), 1.0)
+    ids = np.array([0, 49, 7, 7, 50, -1], dtype=np.int32)
+    out = torch.full((6, 64), 9.0, device="cuda")
+    ok(L().cq_nn_embedding(dev(table).data_ptr(), dev(ids).data_ptr(), out.data_ptr(), 6, 64, 50, None))
+    got = out.cpu().numpy()
+    assert np.array_equal(got[:4], table[[0, 49, 7, 7]])
+    assert np.all(got[4:] == 0.0)
+
+
+@pytest.mark.parametrize("dim", [64, 256, 4096, 5120, 14336])
+@pytest.mark.parametrize("with_delta", [False, True])
+def test_rms_norm(dim, with_delta):
+    rows = 3
+    x, d, w = normal(2, (rows, dim), 1.0), normal(3, (rows, dim), 0.5), normal(4, (dim,), 1.0)
+    xs = dev(x)
+    ds = dev(d)
+    out = torch.empty((rows, dim), device="cuda")
+    ok(L().cq_nn_rms_norm(xs.data_ptr(), ds.data_ptr() if with_delta else None, dev(w).data_ptr(), xs.data_ptr() if with_delta else None,
+                          out.data_ptr(), rows, dim, 1e-5, None))
+    torch.cuda.synchronize()
+    s = (x + d).astype(np.float32) if with_delta else x
+    assert rel_l2(out.cpu().numpy(), lo.rms_norm(s, w, 1e-5)) <= TOL
+    assert np.array_equal(xs.cpu().numpy(), s)          # the residual stream was updated in place (or left alone)
+
+
+def test_rms_norm_kat_on_gpu():
+    # candle-nn/tests/ops.rs:55-66 needs dim % 4 == 0 here: pad the 3-wide rows with a zero and rescale the mean
+    data = np.array([[3.0, 1.0, 4.0, 0.0], [1.0, 5.0, 9.0, 0.0]], dtype=np.float32)
+    alpha = np.array([1.0, 2.0, 3.0, 0.0], dtype=np.float32)
+    out = torch.empty((2, 4), device="cuda")
+    # mean over 4 instead of 3 elements: eps' = eps * 4/3 and a factor sqrt(3/4) on the result give the reference's numbers
+    ok(L().cq_nn_rms_norm(dev(data).data_ptr(), None, dev(alpha).data_ptr(), None, out.data_ptr(), 2, 4, 1e-5 * 3 / 4, None))
+    got = out.cpu().numpy()[:, :3] * math.sqrt(3.0 / 4.0)
+    assert (np.round(got.astype(np.float64) * 1e4) / 1e4).tolist() == [[1.019, 0.6794, 4.0762], [0.1674, 1.6744, 4.521]]
+
+
+@pytest.mark.parametrize("rows,pos", [(1, 0), (1, 37), (5, 3)])
+def test_rope_i_and_cache_append(rows, pos):
+    H, KV, D, ctx = 4, 2, 64, 48
+    cos, sin = lo.precomput_freqs_cis(D, 10000.0, ctx)
+    q, k, v = normal(5, (rows, H * D), 1.0), normal(6, (rows, KV * D), 1.0), normal(7, (rows, KV * D), 1.0)
+    qd, kc, vc = dev(q), torch.zeros((KV, ctx, D), device="cuda"), torch.zeros((KV, ctx, D), device="cuda")
+    posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    # half of the position from the host argument, half from device memory
+    ok(L().cq_nn_rope_i_kv(qd.data_ptr(), dev(k).data_ptr(), dev(v).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(),
+                           dev(sin).data_ptr(), posd.data_ptr(), 0, rows, H, KV, D, ctx, H * D, KV * D, KV * D, None))
+    torch.cuda.synchronize()
+    c, s = cos[pos:pos + rows], sin[pos:pos + rows]
+    want_q = lo.rope_i(q.reshape(rows, H, D).transpose(1, 0, 2)[None], c, s)[0].transpose(1, 0, 2).reshape(rows, H * D)
+    want_k = lo.rope_i(k.reshape(rows, KV, D).transpose(1, 0, 2)[None], c, s)[0]         # [KV, rows, D]
+    assert np.allclose(qd.cpu().numpy(), want_q, rtol=1e-6, atol=1e-6)
+    assert np.allclose(kc.cpu().numpy()[:, pos:pos + rows], want_k, rtol=1e-6, atol=1e-6)
+    assert np.array_equal(vc.cpu().numpy()[:, pos:pos + rows], v.reshape(rows, KV, D).transpose(1, 0, 2))
+    untouched = np.ones(ctx, dtype=bool)
+    untouched[pos:pos + rows] = False
+    assert np.all(kc.cpu().numpy()[:, untouched] == 0.0) and np.all(vc.cpu().numpy()[:, untouched] == 0.0)
+
+
+def attention_oracle(q, kc, vc, pos, H, KV, D):
+    rows = q.shape[0]
+    out = np.empty((rows, H * D), dtype=np.float32)
+    scale = np.float32(1.0 / math.sqrt(D))
+    for r in range(rows):
+        kv_len = pos + r + 1
+        for h in range(H):
+            kvh = h // (H // KV)
+            att = (kc[kvh, :kv_len] @ q[r, h * D:(h + 1) * D]).astype(np.float32) * scale
+            p = lo.softmax_last_dim(att)
+            out[r, h * D:(h + 1) * D] = p @ vc[kvh, :kv_len]
+    return out
+
+
+@pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (4, 4, 128), (8, 2, 128)])
+@pytest.mark.parametrize("rows,pos,ctx", [(1, 0, 32), (1, 199, 256), (1, 600, 1024), (7, 250, 512), (3, 0, 16)])
+def test_attention(H, KV, D, rows, pos, ctx):
+    q = normal(8, (rows, H * D), 1.0)
+    kc, vc = normal(9, (KV, ctx, D), 1.0), normal(10, (KV, ctx, D), 1.0)
+    out = torch.empty((rows, H * D), device="cuda")
+    lib = L()
+    for max_kv in sorted({pos + rows, ctx}):              # exact bound and a looser one (empty trailing splits)
+        wsb = lib.cq_nn_attention_workspace_bytes(rows, H, D, max_kv)
+        ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+        ok(lib.cq_nn_attention(dev(q).data_ptr(), H * D, dev(kc).data_ptr(), dev(vc).data_ptr(), out.data_ptr(), None, pos, rows, H, KV, D,
+                               ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None))
+        torch.cuda.synchronize()
+        assert rel_l2(out.cpu().numpy(), attention_oracle(q, kc, vc, pos, H, KV, D)) <= TOL
+
+
+def test_attention_single_key_returns_value():
+    H, KV, D, ctx = 4, 2, 64, 8
+    q, kc, vc = normal(11, (1, H * D), 5.0), normal(12, (KV, ctx, D), 1.0), normal(13, (KV, ctx, D), 1.0)
+    out = torch.empty((1, H * D), device="cuda")
+    ok(L().cq_nn_attention(dev(q).data_ptr(), H * D, dev(kc).data_ptr(), dev(vc).data_ptr(), out.data_ptr(), None, 0, 1, H, KV, D, ctx, 1,
+                           0.125, None, 0, None))
+    got = out.cpu().numpy().reshape(H, D)
+    for h in range(H):
+        assert np.array_equal(got[h], vc[h // 2, 0])
+
+
+def test_silu_mul_strided_views():
+    rows, dim = 3, 1024
+    gu = normal(14, (rows, 2 * dim), 2.0)
+    g = dev(gu)
+    out = torch.empty((rows, dim), device="cuda")
+    ok(L().cq_nn_silu_mul(g.data_ptr(), g.data_ptr() + 4 * dim, out.data_ptr(), rows, dim, 2 * dim, 2 * dim, None))
+    want = lo.silu(gu[:, :dim]) * gu[:, dim:]
+    assert rel_l2(out.cpu().numpy(), want) <= TOL
+
+
+def test_argmax_first_of_ties_and_bookkeeping():
+    n = 128256
+    logits = normal(15, (n,), 1.0)
+    logits[[777, 90000]] = 50.0                      # a tie: the lower index wins
+    tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    hist = torch.full((8,), -1, dtype=torch.int32, device="cuda")
+    cnt = torch.tensor([2], dtype=torch.int32, device="cuda")
+    pos = torch.tensor([41], dtype=torch.int32, device="cuda")
+    ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), hist.data_ptr(), cnt.data_ptr(), pos.data_ptr(), None))
+    assert tok.item() == 777 and hist.cpu().tolist() == [-1, -1, 777, -1, -1, -1, -1, -1] and cnt.item() == 3 and pos.item() == 42
+    logits[5] = 60.0
+    ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), None, None, None, None))
+    assert tok.item() == 5 == int(np.argmax(logits))
+
+
+def test_argument_validation():
+    lib = L()
+    assert lib.cq_nn_rms_norm(16, None, 16, None, 16, 1, 6, 1e-5, None) == -2          # dim % 4
+    assert lib.cq_nn_rms_norm(None, None, 16, None, 16, 1, 8, 1e-5, None) == -4
+    assert lib.cq_nn_attention(16, 384, 16, 16, 16, None, 0, 1, 4, 2, 96, 8, 1, 0.1, None, 0, None) == -6   # head_dim 96
+    assert lib.cq_nn_attention(16, 256, 16, 16, 16, None, 0, 1, 4, 3, 64, 8, 1, 0.1, None, 0, None) == -2   # heads not divisible
+    assert lib.cq_nn_attention(16, 256, 16, 16, 16, None, 0, 1, 4, 2, 64, 1024, 600, 0.1, None, 0, None) == -5   # splits need a workspace
+    assert lib.cq_nn_silu_mul(16, 16, 16, 1, 8, 4, 8, None) == -2
+    assert lib.cq_nn_rope_i_kv(16, 16, 16, 16, 16, 16, 16, None, 7, 2, 4, 2, 64, 8, 256, 128, 128, None) == -6   # pos + rows > ctx
