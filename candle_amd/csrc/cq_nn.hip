@@ -118,21 +118,35 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float *__restrict__ q, con
 // ---- causal attention of `rows` new queries over the cache -------------------------------------------
 // Query row r sits at absolute position p = pos + r and attends keys [0, p] (quantized_llama.rs:246-261:
 // q k^T / sqrt(d), causal mask, softmax_last_dim, . v, with repeat_kv for grouped heads).
-// One workgroup = one kv head x one query row x one split of 256 keys; the G = n_head / n_kv_head query
+// One workgroup = one kv head x one query row x one split of 128 keys; the G = n_head / n_kv_head query
 // heads that share the kv head are processed together so K and V are read once.
-//   phase 1: thread t owns key j0 + t, dots its 128-float K row against the G query vectors (in LDS)
+//   phase 1: 16 lanes share one key (each holds HD/16 consecutive dims of it and of the G queries), a wave
+//            covers 4 keys per step, the workgroup 16; all K loads of the split are issued before any use;
+//            16-lane DPP sums give the scores
 //   phase 2: per query head: max, exp, sum over the split
-//   phase 3: lanes own output dims, waves stride over keys, p[j] broadcast from LDS; waves summed via LDS
+//   phase 3: lanes own output dims, each wave takes 8 keys per step (loads first, then FMAs), p[j] broadcast
+//            from LDS; waves summed via LDS
 // With one split the normalized result is written directly; otherwise (m, l, unnormalized acc) partials
 // go to the workspace and attn_combine_kernel merges them.
-constexpr int ATT_SPLIT = 256;
+constexpr int ATT_SPLIT = 128;
+
+__device__ __forceinline__ float row16_sum(float v) {      // sum over each aligned group of 16 lanes, in every lane
+#define CQ_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
+    CQ_ADD(CQ_DPP_QUAD_XOR1);
+    CQ_ADD(CQ_DPP_QUAD_XOR2);
+    CQ_ADD(CQ_DPP_ROW_HALF_MIRROR);
+    CQ_ADD(0x140);                                          // row_mirror
+#undef CQ_ADD
+    return v;
+}
 
 template <int HD, int G>
 __global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, int64_t q_stride, const float *__restrict__ k_cache,
                                                    const float *__restrict__ v_cache, float *__restrict__ out, float *__restrict__ part,
                                                    const int32_t *__restrict__ pos_dev, int pos0, int n_head, int ctx, float scale, int splits) {
-    constexpr int DPL = HD / 64;                  // output dims per lane
-    __shared__ __align__(16) float qs[G * HD];
+    constexpr int DPL = HD / 64;                  // output dims per lane (phase 3)
+    constexpr int EPL = HD / 16;                  // dims per lane (phase 1): 16 lanes per key
+    constexpr int IT = ATT_SPLIT / 16;            // phase-1 steps: 16 keys per workgroup step
     __shared__ float sc[G * ATT_SPLIT];
     __shared__ float red[4 * G * HD];
     __shared__ float ml[2 * G];
@@ -142,40 +156,51 @@ __global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, 
     const int j0 = sp * ATT_SPLIT;
     const int cnt = min(kv_len - j0, ATT_SPLIT);      // keys in this split (may be <= 0)
     const float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
-
-    for (int i = tid; i < G * HD; i += 256) qs[i] = q[r * q_stride + (int64_t)(kvh * G) * HD + i];
-    __syncthreads();
+    const int last = max(cnt - 1, 0);                 // loads of masked keys are redirected to a valid row
 
     // ---- phase 1 ----
     {
-        float acc[G];
+        const int sub = lane & 15, kq = lane >> 4;
+        f32x4 kd[IT][EPL / 4];
 #pragma unroll
-        for (int g = 0; g < G; g++) acc[g] = 0.0f;
-        if (tid < cnt) {
-            const float4 *kr = reinterpret_cast<const float4 *>(kb + (int64_t)(j0 + tid) * HD);
-#pragma unroll 8
-            for (int d = 0; d < HD / 4; d++) {
-                const float4 kk = kr[d];
+        for (int it = 0; it < IT; it++) {
+            const int key = min(it * 16 + wv * 4 + kq, last);
+            const f32x4 *kr = reinterpret_cast<const f32x4 *>(kb + (int64_t)(j0 + key) * HD + EPL * sub);
 #pragma unroll
-                for (int g = 0; g < G; g++) {
-                    const float4 qq = *reinterpret_cast<const float4 *>(qs + g * HD + 4 * d);
-                    acc[g] += qq.x * kk.x;
-                    acc[g] += qq.y * kk.y;
-                    acc[g] += qq.z * kk.z;
-                    acc[g] += qq.w * kk.w;
-                }
-            }
+            for (int c = 0; c < EPL / 4; c++) kd[it][c] = kr[c];
+        }
+        f32x4 qf[G][EPL / 4];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const f32x4 *qr = reinterpret_cast<const f32x4 *>(q + r * q_stride + (int64_t)(kvh * G + g) * HD + EPL * sub);
+#pragma unroll
+            for (int c = 0; c < EPL / 4; c++) qf[g][c] = qr[c];
         }
 #pragma unroll
-        for (int g = 0; g < G; g++) sc[g * ATT_SPLIT + tid] = tid < cnt ? acc[g] * scale : -INFINITY;
+        for (int it = 0; it < IT; it++) {
+            const int key = it * 16 + wv * 4 + kq;
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                float a = 0.0f;
+#pragma unroll
+                for (int c = 0; c < EPL / 4; c++) {
+                    a += qf[g][c].x * kd[it][c].x;
+                    a += qf[g][c].y * kd[it][c].y;
+                    a += qf[g][c].z * kd[it][c].z;
+                    a += qf[g][c].w * kd[it][c].w;
+                }
+                a = row16_sum(a);
+                if (sub == 0) sc[g * ATT_SPLIT + key] = key < cnt ? a * scale : -INFINITY;
+            }
+        }
     }
     __syncthreads();
 
     // ---- phase 2: wave w reduces heads g = w, w + 4, ... ----
     for (int g = wv; g < G; g += 4) {
-        float s[4], m = -INFINITY;
+        float s[ATT_SPLIT / 64], m = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < ATT_SPLIT / 64; i++) {
             s[i] = sc[g * ATT_SPLIT + lane + 64 * i];
             m = fmaxf(m, s[i]);
         }
@@ -183,7 +208,7 @@ __global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, 
         for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
         float l = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < ATT_SPLIT / 64; i++) {
             const float p = (cnt > 0 && s[i] > -INFINITY) ? __expf(s[i] - m) : 0.0f;
             sc[g * ATT_SPLIT + lane + 64 * i] = p;
             l += p;
@@ -199,20 +224,28 @@ __global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, 
     for (int g = 0; g < G; g++)
 #pragma unroll
         for (int e = 0; e < DPL; e++) o[g][e] = 0.0f;
-    for (int j = wv; j < cnt; j += 4) {
-        float vv[DPL];
-        if (DPL == 2) {
-            const float2 t = *reinterpret_cast<const float2 *>(vb + (int64_t)(j0 + j) * HD + 2 * lane);
-            vv[0] = t.x; vv[DPL - 1] = t.y;
-        } else {
+    for (int jb = 0; jb < cnt; jb += 32) {
+        float vv[8][DPL];
 #pragma unroll
-            for (int e = 0; e < DPL; e++) vv[e] = vb[(int64_t)(j0 + j) * HD + DPL * lane + e];
+        for (int u = 0; u < 8; u++) {
+            const int j = min(jb + wv + 4 * u, last);
+            if (DPL == 2) {
+                const float2 t = *reinterpret_cast<const float2 *>(vb + (int64_t)(j0 + j) * HD + 2 * lane);
+                vv[u][0] = t.x; vv[u][DPL - 1] = t.y;
+            } else {
+#pragma unroll
+                for (int e = 0; e < DPL; e++) vv[u][e] = vb[(int64_t)(j0 + j) * HD + DPL * lane + e];
+            }
         }
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            const float p = sc[g * ATT_SPLIT + j];
+        for (int u = 0; u < 8; u++) {
+            const int j = jb + wv + 4 * u;                // < ATT_SPLIT; entries at or beyond cnt hold p = 0
 #pragma unroll
-            for (int e = 0; e < DPL; e++) o[g][e] += p * vv[e];
+            for (int g = 0; g < G; g++) {
+                const float p = sc[g * ATT_SPLIT + j];
+#pragma unroll
+                for (int e = 0; e < DPL; e++) o[g][e] += p * vv[u][e];
+            }
         }
     }
 #pragma unroll

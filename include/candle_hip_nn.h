@@ -46,7 +46,7 @@ int cq_nn_rope_i_kv(float *q_dev, const float *k_dev, const float *v_dev, float 
 /* Causal grouped-query attention of `rows` new queries over the cache (quantized_llama.rs:246-261:
  * repeat_kv, q k^T / sqrt(d), mask, softmax_last_dim, . v, transpose back to [rows, n_head*head_dim]).
  * Query row r attends keys [0, pos + *pos_dev + r].  max_kv_len bounds pos + *pos_dev + rows and fixes
- * the launch geometry (keys are processed in splits of 256; more than one split needs the workspace).
+ * the launch geometry (keys are processed in splits of 128; more than one split needs the workspace).
  * head_dim 64 or 128; n_head / n_kv_head in {1, 2, 4, 8}. */
 int64_t cq_nn_attention_workspace_bytes(int64_t rows, int64_t n_head, int64_t head_dim, int64_t max_kv_len);
 int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_dev, const float *v_cache_dev, float *out_dev,
