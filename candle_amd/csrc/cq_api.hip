@@ -2,6 +2,7 @@
 // Declarations and the reference interfaces they replace are in include/candle_hip_quant.h.
 #include "cq_device.h"
 #include "cq_launch.h"
+#include "../../include/candle_hip_nn.h"
 
 namespace {
 
@@ -236,6 +237,29 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
     a.sorted_token_ids = sorted_token_ids_dev; a.expert_ids = expert_ids_dev; a.topk_weights = topk_weights_dev;
     a.prefill = is_prefill;
     return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
+}
+
+// ---- single-row decoder fusions, declared in include/candle_hip_nn.h ----
+int cq_nn_qmatmul_norm(int w_dtype, const void *w_dev, const float *x_dev, const float *sumsq_partials_dev, const float *norm_weight_dev,
+                       float eps, float *dst_dev, int64_t k, int64_t n, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, 1);
+    if (rc) return rc;
+    if (n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!x_dev || !sumsq_partials_dev || !norm_weight_dev || !dst_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(norm_weight_dev, 16) || !aligned(sumsq_partials_dev, 4) || !aligned(dst_dev, 4)) return CQ_ERR_ALIGN;
+    return cq_matvec_norm_launch(w_dtype, w_dev, x_dev, sumsq_partials_dev, norm_weight_dev, eps, dst_dev, k, n, (hipStream_t)stream);
+}
+
+int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
+                           float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, 1);
+    if (rc) return rc;
+    if (n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!x_dev || !residual_dev || !sumsq_partials_out_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(up_dev, 16) || !aligned(residual_dev, 4) || !aligned(sumsq_partials_out_dev, 4)) return CQ_ERR_ALIGN;
+    return cq_matvec_residual_launch(w_dtype, w_dev, x_dev, up_dev, residual_dev, sumsq_partials_out_dev, k, n, (hipStream_t)stream);
 }
 
 }  // extern "C"

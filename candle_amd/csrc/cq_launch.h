@@ -14,6 +14,11 @@ int cq_matvec_launch_av(int w_dtype, const void *w, const ActView &av, void *dst
 // QMatMul::forward for <= CQ_MATVEC_MAX_ROWS rows with the activation quantization fused into the matvec kernel
 int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *dst, int dst_dtype, int64_t k, int64_t n,
                            int64_t rows, int64_t stride_dst, hipStream_t s);
+// single-row decoder fusions (see the Fuse struct in cq_matvec.hip); partial-sum buffers hold 256 floats
+int cq_matvec_norm_launch(int w_dtype, const void *w, const float *x, const float *partials, const float *norm_weight, float eps, float *dst,
+                          int64_t k, int64_t n, hipStream_t s);
+int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const float *up, float *residual, float *partials_out, int64_t k,
+                              int64_t n, hipStream_t s);
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s);
 int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t count, hipStream_t s);

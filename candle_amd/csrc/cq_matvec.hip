@@ -32,6 +32,23 @@ struct ActSrc {
     ActView av;      // pre-quantized: section pointers of the scratch buffer (possibly row-offset)
 };
 
+// Decoder fusions around a single-row f32 matvec (none of them changes what the plain kernel does):
+//   PRO_NORM  the activation row is rms_norm(x) * norm_weight; sum(x^2) arrives as CQ_NN_PARTIALS partial sums
+//             written by the producer of x, so no workgroup-wide reduction is needed before quantizing
+//   PRO_SILU  the activation row is silu(x) * up
+//   EPI_RESID the result is added to a residual row in place of being stored, and the workgroup leaves
+//             its partial sum of residual^2 for the next PRO_NORM consumer
+enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2 };
+enum { EPI_NONE = 0, EPI_RESID = 1 };
+constexpr int NPART = 256;   // == CQ_NN_PARTIALS
+struct Fuse {
+    const float *aux;        // PRO_NORM: norm weight [k];  PRO_SILU: up [k]
+    const float *part_in;    // PRO_NORM: [NPART]
+    float eps;
+    float *resid;            // EPI_RESID: [n], updated in place
+    float *part_out;         // EPI_RESID: [NPART]
+};
+
 // Launch geometry, computed once on the host so the kernel prologue is a handful of scalar loads
 // instead of 64-bit divisions and multiplications in front of the first memory access.
 struct QmvGeom {
@@ -40,13 +57,27 @@ struct QmvGeom {
     int lds_d_off, lds_bs_off; // LDS sections (the scratch layout for NB rows)
     int nw_shift;              // log2(waves per workgroup)
     int row_bytes;             // bytes of one row of W
+    int lds_red_off;           // EPI_RESID: 16 floats behind the activation sections
     int dst_dtype;
     int64_t stride_dst;
 };
 
-template <int DT, int NB, int SRC, bool SINGLE>
-__global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g) {
+// the lane's four activation values of one 256-element span after the prologue op
+template <int PRO>
+__device__ __forceinline__ void pro_apply(float v[4], const float a[4], float m) {
+    if (PRO == PRO_NORM) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = v[i] / m * a[i];                   // candle-nn/src/ops.rs:507-509
+    } else if (PRO == PRO_SILU) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] = v[i] / (1.0f + expf(-v[i])) * a[i];   // Silu::f32, then * up
+    }
+}
+
+template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE>
+__global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g, Fuse fz) {
     typedef Fmt<DT> F;
+    static_assert((PRO == PRO_NONE && EPI == EPI_NONE) || (NB == 1 && SRC == CQ_F32), "fusions are for one f32 row");
     constexpr bool FUSED = SRC != SRC_SCRATCH;
     constexpr int XDT = FUSED ? SRC : CQ_F32;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -75,8 +106,15 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
     u32x4 c_qs = {0, 0, 0, 0};                // pre-quantized: first round of the scratch -> LDS copy
     u32x2 c_d = {0, 0};
     uint32_t c_bs = 0;
+    float av4[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // PRO: norm weight / up values of the same span
+    float pp[NPART / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (FUSED) {
         if (xbase < total) cq_load4<XDT>(src.x, xbase, xv);
+        if (PRO != PRO_NONE && xbase < total) cq_load4<CQ_F32>(fz.aux, xbase, av4);
+        if (PRO == PRO_NORM) {
+#pragma unroll
+            for (int i = 0; i < NPART / 64; i++) pp[i] = fz.part_in[lane + 64 * i];
+        }
     } else {
         if (tid < (total >> 4)) c_qs = ((const u32x4 *)src.av.qs)[tid];
         if (cq_is_kquant(DT)) {
@@ -105,6 +143,13 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
         // in flight).  Inside a loop it would wait for everything, i.e. for the weights, and the
         // quantization latency would no longer hide behind the HBM fetch.
         const int spans = (total + 255) >> 8;
+        float pm = 1.0f;
+        if (PRO == PRO_NORM) {
+            // fixed summation order: the same bits in every wave, workgroup and replay
+            const float sum2 = wave_sum((pp[0] + pp[1]) + (pp[2] + pp[3]));
+            pm = sqrtf(sum2 / (float)k + fz.eps);
+        }
+        pro_apply<PRO>(xv, av4, pm);
         if (wv_s < spans) {
             if (cq_is_kquant(DT))
                 cq_quantize_q8k_vals(xv, wv_s, lane, lqs, ld, lbs);
@@ -112,10 +157,25 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
                 cq_quantize_q80_vals(xv, xbase < total, xbase, lane, lqs, ld);
         }
         for (int span = wv_s + nwaves; span < spans; span += nwaves) {
-            if (cq_is_kquant(DT))
-                cq_quantize_q8k_span<XDT>(src.x, span, lane, lqs, ld, lbs);
-            else
-                cq_quantize_q80_span<XDT>(src.x, span, lane, total, lqs, ld);
+            if (PRO == PRO_NONE) {
+                if (cq_is_kquant(DT))
+                    cq_quantize_q8k_span<XDT>(src.x, span, lane, lqs, ld, lbs);
+                else
+                    cq_quantize_q80_span<XDT>(src.x, span, lane, total, lqs, ld);
+            } else {
+                const int base = span * 256 + lane * 4;
+                const bool ok = base < total;
+                float v[4] = {0.0f, 0.0f, 0.0f, 0.0f}, a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (ok) {
+                    cq_load4<XDT>(src.x, base, v);
+                    cq_load4<CQ_F32>(fz.aux, base, a);
+                }
+                pro_apply<PRO>(v, a, pm);
+                if (cq_is_kquant(DT))
+                    cq_quantize_q8k_vals(v, span, lane, lqs, ld, lbs);
+                else
+                    cq_quantize_q80_vals(v, ok, base, lane, lqs, ld);
+            }
         }
     } else {
         if (tid < (total >> 4)) ((u32x4 *)lqs)[tid] = c_qs;
@@ -131,7 +191,8 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
         }
     }
     __syncthreads();
-    if (my_rows == 0) return;
+    if (EPI == EPI_NONE && my_rows == 0) return;
+    float ssq = 0.0f;            // EPI_RESID: lane 63 accumulates residual^2 of this wave's rows
 
     ActRow ar[NB];
 #pragma unroll
@@ -147,25 +208,38 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
 #pragma unroll
             for (int b = 0; b < NB; b++) F::load_a(areg[b], ar[b], u0);
         }
-        auto one_row = [&](const typename F::W &cur, int r) {
+        auto one_row = [&](const typename F::W &cur, int r, float res) {
 #pragma unroll
             for (int b = 0; b < NB; b++) {
                 if (!CACHE) F::load_a(areg[b], ar[b], u0);
                 float v = F::dot(cur, areg[b], u0);
                 v = wave_sum_to_lane63(valid ? v : 0.0f);
-                if (lane == 63) store_out(dst, dst_dtype, (int64_t)b * stride_dst + r, v);
+                if (EPI == EPI_RESID) {
+                    if (lane == 63) {
+                        const float sres = res + v;                     // (x + residual), quantized_llama.rs:584,591
+                        fz.resid[r] = sres;
+                        ssq += sres * sres;
+                    }
+                } else if (lane == 63) {
+                    store_out(dst, dst_dtype, (int64_t)b * stride_dst + r, v);
+                }
             }
         };
         // ping-pong between wa and wb: the next row's loads are in flight while this one is reduced;
-        // the prefetch past the last row re-reads it instead of branching around the load
+        // the prefetch past the last row re-reads it instead of branching around the load.  The residual
+        // value of a row travels behind its weights in the same in-order load queue.
+        float ra = 0.0f, rb = 0.0f;
+        if (EPI == EPI_RESID) ra = fz.resid[min(row, n - 1)];
         for (int j = 0; j < my_rows; j += 2) {
             const uint8_t *p1 = j + 1 < my_rows ? wp + wave_stride : wp;
             F::load_w(wb, p1, u0);
-            one_row(wa, row);
+            if (EPI == EPI_RESID) rb = fz.resid[min(row + nwaves, n - 1)];
+            one_row(wa, row, ra);
             if (j + 1 >= my_rows) break;
             const uint8_t *p2 = j + 2 < my_rows ? p1 + wave_stride : p1;
             F::load_w(wa, p2, u0);
-            one_row(wb, row + nwaves);
+            if (EPI == EPI_RESID) ra = fz.resid[min(row + 2 * nwaves, n - 1)];
+            one_row(wb, row + nwaves, rb);
             row += 2 * nwaves;
             wp = p2;
         }
@@ -177,6 +251,8 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
         for (int b = 0; b < NB; b++) acc[b] = 0.0f;
         const int total_steps = my_rows * steps;
         int i = 0;
+        float rcur = 0.0f;
+        if (EPI == EPI_RESID) rcur = fz.resid[min(row, n - 1)];
         auto one_step = [&](const typename F::W &cur, typename F::W &nxt, int t) {
             // next (row, step); past the end the last unit is re-read
             int ni = i + 1;
@@ -197,10 +273,19 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
 #pragma unroll
                 for (int b = 0; b < NB; b++) {
                     float r = wave_sum_to_lane63(acc[b]);
-                    if (lane == 63) store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, r);
+                    if (EPI == EPI_RESID) {
+                        if (lane == 63) {
+                            const float sres = rcur + r;
+                            fz.resid[row] = sres;
+                            ssq += sres * sres;
+                        }
+                    } else if (lane == 63) {
+                        store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, r);
+                    }
                     acc[b] = 0.0f;
                 }
                 row += nwaves;
+                if (EPI == EPI_RESID) rcur = fz.resid[min(row, n - 1)];   // consumed a whole row of steps later
             }
             i = ni;
             wp = nwp;
@@ -211,10 +296,24 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
             one_step(wb, wa, t + 1);
         }
     }
+    if (EPI == EPI_RESID) {
+        // the workgroup's partial of sum(residual^2), summed in a fixed order; block 0 clears the unused slots
+        float *red = (float *)(lds + g.lds_red_off);
+        if (lane == 63) red[wv] = ssq;
+        __syncthreads();
+        if (tid == 0) {
+            float t = 0.0f;
+            for (int i = 0; i < nwaves; i++) t += red[i];
+            fz.part_out[blockIdx.x] = t;
+        }
+        if (blockIdx.x == 0)
+            for (int i = (int)gridDim.x + tid; i < NPART; i += nthr) fz.part_out[i] = 0.0f;
+    }
 }
 
-template <int DT, int NB, int SRC, bool SINGLE>
-int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
+template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE>
+int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s,
+               const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr}) {
     // waves per workgroup: as many as still leave every wave a row when 256 workgroups are launched
     int waves = 16;
     while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
@@ -222,8 +321,9 @@ int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64
     int64_t rows_per_wg = (n + groups - 1) / groups;
     groups = (n + rows_per_wg - 1) / rows_per_wg;
     const ActLayout L = cq_act_layout(DT, k, NB);
-    size_t lds_bytes = (size_t)L.total;
+    size_t lds_bytes = (size_t)L.total + (EPI == EPI_RESID ? 64 : 0);
     QmvGeom g;
+    g.lds_red_off = (int)L.total;
     g.k = (int)k; g.n = (int)n; g.rows_per_wg = (int)rows_per_wg;
     g.units = (int)(k / Fmt<DT>::UE); g.steps = (g.units + 63) >> 6;
     g.lds_d_off = (int)L.d_off; g.lds_bs_off = (int)L.bs_off;
@@ -233,12 +333,12 @@ int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64
     if (rb > 0x3fffffff) return CQ_ERR_RANGE;
     g.row_bytes = (int)rb;
     g.dst_dtype = dst_dtype; g.stride_dst = stride_dst;
-    auto kern = qmv_kernel<DT, NB, SRC, SINGLE>;
+    auto kern = qmv_kernel<DT, NB, SRC, SINGLE, PRO, EPI>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * waves), lds_bytes, s, (const uint8_t *)w, src, dst, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * waves), lds_bytes, s, (const uint8_t *)w, src, dst, g, fz);
     return (int)hipGetLastError();
 }
 
@@ -328,4 +428,43 @@ int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtyp
         }
         return (int)CQ_ERR_DTYPE;
     });
+}
+
+namespace {
+template <int DT, int PRO, int EPI>
+int launch_fused1(const void *w, const ActSrc &src, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
+    if (cq_act_layout(DT, k, 1).total + 64 > LDS_BUDGET) return CQ_ERR_RANGE;
+    if (k / Fmt<DT>::UE <= 64) return launch_cfg<DT, 1, CQ_F32, true, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
+    return launch_cfg<DT, 1, CQ_F32, false, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
+}
+template <int PRO, int EPI>
+int launch_fused_dt(int w_dtype, const void *w, const ActSrc &src, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_fused1<CQ_Q4_0, PRO, EPI>(w, src, dst, k, n, s, fz);
+        case CQ_Q8_0: return launch_fused1<CQ_Q8_0, PRO, EPI>(w, src, dst, k, n, s, fz);
+        case CQ_Q4K: return launch_fused1<CQ_Q4K, PRO, EPI>(w, src, dst, k, n, s, fz);
+        case CQ_Q5K: return launch_fused1<CQ_Q5K, PRO, EPI>(w, src, dst, k, n, s, fz);
+        case CQ_Q6K: return launch_fused1<CQ_Q6K, PRO, EPI>(w, src, dst, k, n, s, fz);
+    }
+    return CQ_ERR_DTYPE;
+}
+}  // namespace
+
+// dst[n] = W . quantize(rms_norm(x) * norm_weight), sum(x^2) given as 256 partial sums
+int cq_matvec_norm_launch(int w_dtype, const void *w, const float *x, const float *partials, const float *norm_weight, float eps, float *dst,
+                          int64_t k, int64_t n, hipStream_t s) {
+    if (n == 0) return CQ_OK;
+    ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr};
+    return launch_fused_dt<PRO_NORM, EPI_NONE>(w_dtype, w, src, dst, k, n, s, fz);
+}
+
+// residual[n] += W . quantize(up ? silu(x) * up : x); partials_out[256] = partial sums of residual^2
+int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const float *up, float *residual, float *partials_out, int64_t k,
+                              int64_t n, hipStream_t s) {
+    if (n == 0) return CQ_OK;
+    ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{up, nullptr, 0.0f, residual, partials_out};
+    if (up) return launch_fused_dt<PRO_SILU, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
+    return launch_fused_dt<PRO_NONE, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
 }

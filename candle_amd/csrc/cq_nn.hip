@@ -19,13 +19,26 @@ __device__ __forceinline__ float block_sum_256(float v, float *red) {     // red
 
 // ---- embedding: out[r, :] = table[ids[r], :] (candle_nn::Embedding, index_select) ---------------
 __global__ __launch_bounds__(256) void embedding_kernel(const float *__restrict__ table, const int32_t *__restrict__ ids, float *__restrict__ out,
-                                                        int dim, int64_t vocab) {
+                                                        int dim, int64_t vocab, float *__restrict__ partials) {
+    __shared__ float red[4];
     const int r = blockIdx.x;
     const int64_t id = ids[r];
     const bool ok = id >= 0 && id < vocab;
     const float4 *src = reinterpret_cast<const float4 *>(table + (ok ? id : 0) * dim);
     float4 *dst = reinterpret_cast<float4 *>(out + (int64_t)r * dim);
-    for (int i = threadIdx.x; i < dim / 4; i += 256) dst[i] = ok ? src[i] : float4{0.f, 0.f, 0.f, 0.f};
+    float acc = 0.0f;
+    for (int i = threadIdx.x; i < dim / 4; i += 256) {
+        const float4 v = ok ? src[i] : float4{0.f, 0.f, 0.f, 0.f};
+        dst[i] = v;
+        acc += v.x * v.x;
+        acc += v.y * v.y;
+        acc += v.z * v.z;
+        acc += v.w * v.w;
+    }
+    if (partials) {                       // uniform branch
+        const float t = block_sum_256(acc, red);
+        partials[threadIdx.x] = threadIdx.x == 0 ? t : 0.0f;      // 256 threads == CQ_NN_PARTIALS slots
+    }
 }
 
 // ---- s = x (+ delta); sum_out = s; out = s / sqrt(mean(s^2) + eps) * w  (candle-nn/src/ops.rs:499-510) ----
@@ -355,13 +368,16 @@ int launch_attn(int G, dim3 grid, hipStream_t s, const float *q, int64_t q_strid
 
 extern "C" {
 
-int cq_nn_embedding(const float *table_dev, const int32_t *ids_dev, float *out_dev, int64_t rows, int64_t dim, int64_t vocab, void *stream) {
+int cq_nn_embedding(const float *table_dev, const int32_t *ids_dev, float *out_dev, int64_t rows, int64_t dim, int64_t vocab,
+                    float *sumsq_partials_dev, void *stream) {
     if (rows < 0 || dim <= 0 || vocab <= 0 || dim % 4) return CQ_ERR_SHAPE;
+    if (sumsq_partials_dev && rows != 1) return CQ_ERR_SHAPE;
     if (rows == 0) return CQ_OK;
     if (!table_dev || !ids_dev || !out_dev) return CQ_ERR_NULL;
     if (misaligned(table_dev, 16) || misaligned(out_dev, 16)) return CQ_ERR_ALIGN;
     if (rows > 0x7fffffffLL || dim > 0x7fffffffLL) return CQ_ERR_RANGE;
-    hipLaunchKernelGGL(embedding_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, table_dev, ids_dev, out_dev, (int)dim, vocab);
+    hipLaunchKernelGGL(embedding_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, table_dev, ids_dev, out_dev, (int)dim, vocab,
+                       sumsq_partials_dev);
     return (int)hipGetLastError();
 }
 

@@ -104,6 +104,7 @@ class ModelWeights:
         self._slab: Optional[torch.Tensor] = None
         self._graph = None
         self._graph_key = None
+        self.fuse_decode = True      # single-token steps use the fused matvec prologues / epilogues
 
     # ------------------------------------------------------------------------------------------ construction
     def _alloc(self, dtypes: Dict[str, GgmlDType]):
@@ -160,6 +161,7 @@ class ModelWeights:
         self.gu = torch.empty((max_rows, 2 * cfg.ffn), **f32)
         self.h = torch.empty((max_rows, cfg.ffn), **f32)
         self.logits = torch.empty((1, cfg.vocab), **f32)
+        self.partials = torch.zeros(256, **f32)          # CQ_NN_PARTIALS: sum(x^2) of the residual row, in partial sums
         need = 0
         for (n, k) in list(_layer_shapes(cfg).values()) + [(qd + kvd, cfg.hidden), (2 * cfg.ffn, cfg.hidden)]:
             for dt in (GgmlDType.Q4K, GgmlDType.Q8_0):      # K-quant and Q*_0 scratch layouts
@@ -239,7 +241,9 @@ class ModelWeights:
         scale = float(np.float32(1.0 / math.sqrt(cfg.head_dim)))
         ck = _lib.check
         x, xn, qk, v, att, delta, gu, h = self.x, self.xn, self.qk, self.v, self.att, self.delta, self.gu, self.h
-        ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), rows, cfg.hidden, cfg.vocab, sp))
+        if rows == 1 and self.fuse_decode:
+            return self._enqueue_decode_fused(ids_ptr, pos, pos_dev_ptr, max_kv_len, sp)
+        ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), rows, cfg.hidden, cfg.vocab, None, sp))
         for li, lw in enumerate(self.layers):
             w = lw.w
             # x (+= mlp output of the previous layer); xn = attention_norm(x)          :579-583, :590-592
@@ -283,6 +287,52 @@ class ModelWeights:
         ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr() + last, delta.data_ptr() + last, self.norm.data_ptr(), None, xn.data_ptr(), 1,
                                              cfg.hidden, cfg.rms_eps, sp))
         self._mm(self.output, cfg.vocab, xn, self.logits.data_ptr(), 1, sp)
+
+    def _enqueue_decode_fused(self, ids_ptr: int, pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
+        """The same single-token step with the glue folded into the matvec kernels: the residual add is the
+        epilogue of attention_wo / feed_forward_w2 (which also leaves sum(x^2) as partial sums), rms_norm and
+        silu(w1 x) * w3 x are the prologues of the matvecs that consume them."""
+        cfg, L = self.cfg, self.L
+        qd, kvd = cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim
+        scale = float(np.float32(1.0 / math.sqrt(cfg.head_dim)))
+        ck = _lib.check
+        x, qk, v, att, gu, part = self.x, self.qk, self.v, self.att, self.gu, self.partials
+        ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), 1, cfg.hidden, cfg.vocab,
+                                                part.data_ptr(), sp))
+
+        def norm_mm(w: _W, n: int, norm_w: torch.Tensor, dst_ptr: int):
+            ck("cq_nn_qmatmul_norm", L.cq_nn_qmatmul_norm(int(w.dtype), w.ptr, x.data_ptr(), part.data_ptr(), norm_w.data_ptr(), cfg.rms_eps,
+                                                          dst_ptr, w.k, n, sp))
+
+        def resid_mm(w: _W, src_ptr: int, up_ptr: Optional[int]):
+            ck("cq_nn_qmatmul_residual", L.cq_nn_qmatmul_residual(int(w.dtype), w.ptr, src_ptr, up_ptr, x.data_ptr(), part.data_ptr(), w.k,
+                                                                  cfg.hidden, sp))
+
+        for lw in self.layers:
+            w = lw.w
+            wq, wk, wv = w["attention_wq"], w["attention_wk"], w["attention_wv"]
+            if wq.dtype == wk.dtype and wk.ptr == wq.ptr + wq.nbytes:
+                norm_mm(wq, qd + kvd, lw.attention_norm, qk.data_ptr())
+            else:
+                norm_mm(wq, qd, lw.attention_norm, qk.data_ptr())
+                norm_mm(wk, kvd, lw.attention_norm, qk.data_ptr() + 4 * qd)
+            norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
+            q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
+            ck("cq_nn_rope_i_kv", L.cq_nn_rope_i_kv(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
+                                                   self.cos.data_ptr(), self.sin.data_ptr(), pos_dev_ptr, pos, 1, cfg.n_head, cfg.n_kv_head,
+                                                   cfg.head_dim, cfg.ctx, qd + kvd, qd + kvd, kvd, sp))
+            ck("cq_nn_attention", L.cq_nn_attention(q_ptr, qd + kvd, lw.k_cache.data_ptr(), lw.v_cache.data_ptr(), att.data_ptr(), pos_dev_ptr, pos,
+                                                   1, cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
+                                                   self.att_ws.data_ptr(), self.att_ws.numel(), sp))
+            resid_mm(w["attention_wo"], att.data_ptr(), None)
+            w1, w3 = w["feed_forward_w1"], w["feed_forward_w3"]
+            if w1.dtype == w3.dtype and w3.ptr == w1.ptr + w1.nbytes:
+                norm_mm(w1, 2 * cfg.ffn, lw.ffn_norm, gu.data_ptr())
+            else:
+                norm_mm(w1, cfg.ffn, lw.ffn_norm, gu.data_ptr())
+                norm_mm(w3, cfg.ffn, lw.ffn_norm, gu.data_ptr() + 4 * cfg.ffn)
+            resid_mm(w["feed_forward_w2"], gu.data_ptr(), gu.data_ptr() + 4 * cfg.ffn)
+        norm_mm(self.output, cfg.vocab, self.norm, self.logits.data_ptr())
 
     def forward(self, x: torch.Tensor, index_pos: int) -> torch.Tensor:
         """ModelWeights::forward: token ids [1, seq_len] at positions index_pos.. -> logits [1, vocab] of the last token."""

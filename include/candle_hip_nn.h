@@ -21,10 +21,16 @@
 extern "C" {
 #endif
 
+/* Number of floats in a "sum of squares" partials buffer: a producer of a residual row leaves sum(row^2) as
+ * this many partial sums (unused slots zero), the fused rms-norm consumer adds them in a fixed order. */
+#define CQ_NN_PARTIALS 256
+
 /* out[r, :] = table[ids[r], :] — candle_nn::Embedding::forward (candle-nn/src/embedding.rs), used as
  * tok_embeddings in quantized_llama.rs:577.  table [vocab, dim] f32, dim % 4 == 0, 16-byte aligned.
- * An id outside [0, vocab) yields a zero row (the reference returns an error from index_select). */
-int cq_nn_embedding(const float *table_dev, const int32_t *ids_dev, float *out_dev, int64_t rows, int64_t dim, int64_t vocab, void *stream);
+ * An id outside [0, vocab) yields a zero row (the reference returns an error from index_select).
+ * sumsq_partials_dev (optional, rows == 1 only): receives sum(out[0, :]^2) as CQ_NN_PARTIALS partials. */
+int cq_nn_embedding(const float *table_dev, const int32_t *ids_dev, float *out_dev, int64_t rows, int64_t dim, int64_t vocab,
+                    float *sumsq_partials_dev, void *stream);
 
 /* Residual add + RMS norm: s = x (+ delta when delta_dev != NULL); sum_out = s (when sum_out_dev != NULL,
  * may alias x_dev); out = s / sqrt(mean(s^2) + eps) * weight.
@@ -57,6 +63,19 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
  * (candle_nn::ops::silu, candle-core/src/op.rs Silu::f32).  gate/up rows may be strided views of one buffer. */
 int cq_nn_silu_mul(const float *gate_dev, const float *up_dev, float *out_dev, int64_t rows, int64_t dim, int64_t gate_stride, int64_t up_stride,
                    void *stream);
+
+/* Single-row (decode) fusions of the glue into the quantized matvec kernel.  No counterpart in the reference,
+ * which runs these as separate tensor ops; results equal the unfused sequence up to f32 summation order.
+ *
+ * cq_nn_qmatmul_norm:      dst[n] = QMatMul(w).forward(rms_norm(x, norm_weight, eps)) for one row x[k]
+ *                          (quantized_llama.rs:581-582 / :588-589 / :593-596); sum(x^2) is read from sumsq_partials.
+ * cq_nn_qmatmul_residual:  residual[n] += QMatMul(w).forward(up ? silu(x) * up : x) for one row x[k]
+ *                          (attention_wo + residual add :264,:584, or Mlp :56-63 + residual add :590-591);
+ *                          sumsq_partials_out receives sum(residual^2) of the updated row. */
+int cq_nn_qmatmul_norm(int w_dtype, const void *w_dev, const float *x_dev, const float *sumsq_partials_dev, const float *norm_weight_dev,
+                       float eps, float *dst_dev, int64_t k, int64_t n, void *stream);
+int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
+                           float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream);
 
 /* Greedy sampling (LogitsProcessor with Sampling::ArgMax, candle-examples/examples/quantized/main.rs:603-604):
  * token_out[0] = index of the largest logit (lowest index on ties).  Optional bookkeeping for graph replay:

@@ -78,6 +78,13 @@ def test_generate_greedy_graph_equals_eager_equals_oracle():
     b = model.generate_greedy(prompt, n_new, use_graph=True)["tokens"]
     c = model.generate_greedy(prompt, n_new, use_graph=True)["tokens"]      # replays the cached graph from a fresh state
     assert a == b == c and len(a) == n_new
+    # the same steps with every glue op as its own kernel (no fused matvec prologues / epilogues)
+    model.fuse_decode = False
+    assert model.generate_greedy(prompt, n_new, use_graph=False)["tokens"] == a
+    l_unfused = model.forward(torch.tensor([[7]], dtype=torch.int32), 20).cpu().numpy()
+    model.fuse_decode = True
+    l_fused = model.forward(torch.tensor([[7]], dtype=torch.int32), 20).cpu().numpy()
+    assert rel_l2(l_fused, l_unfused) <= 1e-4
     ref = lo.LlamaOracle(cfg, t)
     logits = ref.forward(prompt, 0)
     want = []

@@ -46,7 +46,7 @@ def test_embedding_rows_and_out_of_range():
     table = normal(1, (50, 64), 1.0)
     ids = np.array([0, 49, 7, 7, 50, -1], dtype=np.int32)
     out = torch.full((6, 64), 9.0, device="cuda")
-    ok(L().cq_nn_embedding(dev(table).data_ptr(), dev(ids).data_ptr(), out.data_ptr(), 6, 64, 50, None))
+    ok(L().cq_nn_embedding(dev(table).data_ptr(), dev(ids).data_ptr(), out.data_ptr(), 6, 64, 50, None, None))
     got = out.cpu().numpy()
     assert np.array_equal(got[:4], table[[0, 49, 7, 7]])
     assert np.all(got[4:] == 0.0)
@@ -165,6 +165,66 @@ def test_argmax_first_of_ties_and_bookkeeping():
     logits[5] = 60.0
     ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), None, None, None, None))
     assert tok.item() == 5 == int(np.argmax(logits))
+
+
+FUSE_DTYPES = [2, 8, 12, 13, 14]      # Q4_0, Q8_0, Q4_K, Q5_K, Q6_K
+
+
+@pytest.mark.parametrize("dtype", FUSE_DTYPES)
+@pytest.mark.parametrize("n,k", [(203, 4096), (64, 256), (1024, 14336), (5000, 1024)])
+def test_fused_norm_matvec_and_residual_chain(dtype, n, k):
+    """embedding -> (rms_norm + matvec) and (matvec + residual add) -> (rms_norm + matvec) against the unfused
+    CPU sequence: rms_norm, quantized matmul, add.  Single row, like a decode step."""
+    import oracle
+    lib = L()
+    table = normal(20, (7, k), 1.0)
+    nw = (1.0 + 0.1 * normal(21, (k,), 1.0)).astype(np.float32)
+    w1 = oracle.from_float(dtype, normal(22, (n, k), 0.05).reshape(-1))
+    w1d = dev(w1)
+    ids = dev(np.array([3], dtype=np.int32))
+    x = torch.empty((1, k), device="cuda")
+    part = torch.full((256,), 7.0, device="cuda")
+    ok(lib.cq_nn_embedding(dev(table).data_ptr(), ids.data_ptr(), x.data_ptr(), 1, k, 7, part.data_ptr(), None))
+    p = part.cpu().numpy()
+    assert np.isclose(p.sum(), float((table[3].astype(np.float64) ** 2).sum()), rtol=1e-5) and np.all(p[1:] == 0.0)
+    y = torch.empty((1, n), device="cuda")
+    ok(lib.cq_nn_qmatmul_norm(dtype, w1d.data_ptr(), x.data_ptr(), part.data_ptr(), dev(nw).data_ptr(), 1e-5, y.data_ptr(), k, n, None))
+    xn = lo.rms_norm(table[3:4], nw, 1e-5)
+    want = oracle.matmul(dtype, xn, w1, n)
+    assert rel_l2(y.cpu().numpy(), want) <= 1e-3
+    # second stage: residual[k] += W2[k x n] . y   (n must be a whole number of blocks for W2)
+    if n % 256 == 0:
+        w2 = oracle.from_float(dtype, normal(23, (k, n), 0.05).reshape(-1))
+        res0 = table[3:4].copy()
+        res = dev(res0)
+        part2 = torch.full((256,), 9.0, device="cuda")
+        ok(lib.cq_nn_qmatmul_residual(dtype, dev(w2).data_ptr(), y.data_ptr(), None, res.data_ptr(), part2.data_ptr(), n, k, None))
+        want_res = res0 + oracle.matmul(dtype, y.cpu().numpy(), w2, k)
+        got_res = res.cpu().numpy()
+        assert rel_l2(got_res, want_res) <= 1e-5
+        assert np.isclose(part2.cpu().numpy().astype(np.float64).sum(), float((got_res.astype(np.float64) ** 2).sum()), rtol=1e-5)
+        # and the partial sums drive the next fused norm
+        y2 = torch.empty((1, n), device="cuda")
+        ok(lib.cq_nn_qmatmul_norm(dtype, w1d.data_ptr(), res.data_ptr(), part2.data_ptr(), dev(nw).data_ptr(), 1e-5, y2.data_ptr(), k, n, None))
+        want2 = oracle.matmul(dtype, lo.rms_norm(got_res, nw, 1e-5), w1, n)
+        assert rel_l2(y2.cpu().numpy(), want2) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [12, 14, 8])
+def test_fused_silu_mul_matvec_residual(dtype):
+    import oracle
+    k, n = 14336, 4096
+    gu = normal(24, (1, 2 * k), 1.5)
+    w = oracle.from_float(dtype, normal(25, (n, k), 0.02).reshape(-1))
+    res0 = normal(26, (1, n), 1.0)
+    g, res = dev(gu), dev(res0)
+    part = torch.empty((256,), device="cuda")
+    ok(L().cq_nn_qmatmul_residual(dtype, dev(w).data_ptr(), g.data_ptr(), g.data_ptr() + 4 * k, res.data_ptr(), part.data_ptr(), k, n, None))
+    h = (lo.silu(gu[:, :k]) * gu[:, k:]).astype(np.float32)
+    want = res0 + oracle.matmul_fast(dtype, h, w, n, 8)
+    # expf on the device differs from the host's by an ulp here and there; the quantizer can turn that into a
+    # one-step difference of a single int8 value
+    assert rel_l2(res.cpu().numpy(), want) <= 1e-4
 
 
 def test_argument_validation():
