@@ -74,7 +74,7 @@ __device__ __forceinline__ void pro_apply(float v[4], const float a[4], float m)
     }
 }
 
-template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE>
+template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
 __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g, Fuse fz) {
     typedef Fmt<DT> F;
     static_assert((PRO == PRO_NONE && EPI == EPI_NONE) || (NB == 1 && SRC == CQ_F32), "fusions are for one f32 row");
@@ -101,16 +101,26 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
     // 0. The activation loads go out first.  Vector loads complete in order, so anything issued after
     //    the weight loads below could only be consumed once the (slow, HBM) weights have arrived.
     const int total = NB * k;                 // elements of x
-    float xv[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // fused: this wave's first 256-element span
+    // fused: this wave's first XS 256-element spans (span wv, wv + nwaves, ...) are loaded up front; with
+    // long rows (PRE) that is normally all of them, so no load -> use round trip is left in the prologue
+    constexpr int XS = PRE ? 4 : 1;
+    float xv[XS][4], av4[XS][4];              // av4: PRO: norm weight / up values of the same spans
+#pragma unroll
+    for (int j = 0; j < XS; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) { xv[j][e] = 0.0f; av4[j][e] = 0.0f; }
     const int xbase = wv * 256 + lane * 4;
+    const int xstep = 256 << g.nw_shift;
     u32x4 c_qs = {0, 0, 0, 0};                // pre-quantized: first round of the scratch -> LDS copy
     u32x2 c_d = {0, 0};
     uint32_t c_bs = 0;
-    float av4[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // PRO: norm weight / up values of the same span
     float pp[NPART / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (FUSED) {
-        if (xbase < total) cq_load4<XDT>(src.x, xbase, xv);
-        if (PRO != PRO_NONE && xbase < total) cq_load4<CQ_F32>(fz.aux, xbase, av4);
+#pragma unroll
+        for (int j = 0; j < XS; j++) {
+            if (xbase + j * xstep < total) cq_load4<XDT>(src.x, xbase + j * xstep, xv[j]);
+            if (PRO != PRO_NONE && xbase + j * xstep < total) cq_load4<CQ_F32>(fz.aux, xbase + j * xstep, av4[j]);
+        }
         if (PRO == PRO_NORM) {
 #pragma unroll
             for (int i = 0; i < NPART / 64; i++) pp[i] = fz.part_in[lane + 64 * i];
@@ -134,7 +144,15 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
     const uint8_t *wp = w + (int64_t)min(row, n - 1) * (int64_t)row_bytes;
     const int u0 = min(lane, units - 1);
     typename F::W wa, wb;
-    F::load_w(wa, wp, u0);
+    // PRE (rows of 2..4 wave steps, e.g. K = 14336): all steps of the wave's first row are issued here, so the
+    // whole first row streams in behind the activation prologue instead of one step of it
+    typename F::W pre[PRE ? 4 : 1];
+    if (PRE) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) F::load_w(pre[i], wp, min(lane + 64 * i, units - 1));
+    } else {
+        F::load_w(wa, wp, u0);
+    }
 
     // 2. activations -> LDS
     if (FUSED) {
@@ -149,14 +167,18 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
             const float sum2 = wave_sum((pp[0] + pp[1]) + (pp[2] + pp[3]));
             pm = sqrtf(sum2 / (float)k + fz.eps);
         }
-        pro_apply<PRO>(xv, av4, pm);
-        if (wv_s < spans) {
-            if (cq_is_kquant(DT))
-                cq_quantize_q8k_vals(xv, wv_s, lane, lqs, ld, lbs);
-            else
-                cq_quantize_q80_vals(xv, xbase < total, xbase, lane, lqs, ld);
+#pragma unroll
+        for (int j = 0; j < XS; j++) {
+            const int span = wv_s + (j << g.nw_shift);
+            pro_apply<PRO>(xv[j], av4[j], pm);
+            if (span < spans) {
+                if (cq_is_kquant(DT))
+                    cq_quantize_q8k_vals(xv[j], span, lane, lqs, ld, lbs);
+                else
+                    cq_quantize_q80_vals(xv[j], xbase + j * xstep < total, xbase + j * xstep, lane, lqs, ld);
+            }
         }
-        for (int span = wv_s + nwaves; span < spans; span += nwaves) {
+        for (int span = wv_s + XS * nwaves; span < spans; span += nwaves) {
             if (PRO == PRO_NONE) {
                 if (cq_is_kquant(DT))
                     cq_quantize_q8k_span<XDT>(src.x, span, lane, lqs, ld, lbs);
@@ -249,18 +271,30 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
         float acc[NB];
 #pragma unroll
         for (int b = 0; b < NB; b++) acc[b] = 0.0f;
-        const int total_steps = my_rows * steps;
+        int total_steps = my_rows * steps;
         int i = 0;
         float rcur = 0.0f;
         if (EPI == EPI_RESID) rcur = fz.resid[min(row, n - 1)];
-        auto one_step = [&](const typename F::W &cur, typename F::W &nxt, int t) {
-            // next (row, step); past the end the last unit is re-read
-            int ni = i + 1;
-            const uint8_t *nwp = wp;
-            if (ni == steps) { ni = 0; nwp = wp + wave_stride; }
-            if (t + 1 >= total_steps) { ni = i; nwp = wp; }
-            F::load_w(nxt, nwp, min(lane + 64 * ni, units - 1));
-            const int u = lane + 64 * i;
+        auto finish_row = [&]() {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                float r = wave_sum_to_lane63(acc[b]);
+                if (EPI == EPI_RESID) {
+                    if (lane == 63) {
+                        const float sres = rcur + r;
+                        fz.resid[row] = sres;
+                        ssq += sres * sres;
+                    }
+                } else if (lane == 63) {
+                    store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, r);
+                }
+                acc[b] = 0.0f;
+            }
+            row += nwaves;
+            if (EPI == EPI_RESID) rcur = fz.resid[min(row, n - 1)];   // consumed a whole row of steps later
+        };
+        auto accumulate = [&](const typename F::W &cur, int step) {
+            const int u = lane + 64 * step;
             const bool valid = u < units;
             const int uc = valid ? u : units - 1;
 #pragma unroll
@@ -269,24 +303,29 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
                 float v = F::dot(cur, areg[b], uc);
                 acc[b] += valid ? v : 0.0f;
             }
-            if (i == steps - 1) {
+        };
+        if (PRE) {
+            if (my_rows > 0) {
 #pragma unroll
-                for (int b = 0; b < NB; b++) {
-                    float r = wave_sum_to_lane63(acc[b]);
-                    if (EPI == EPI_RESID) {
-                        if (lane == 63) {
-                            const float sres = rcur + r;
-                            fz.resid[row] = sres;
-                            ssq += sres * sres;
-                        }
-                    } else if (lane == 63) {
-                        store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, r);
-                    }
-                    acc[b] = 0.0f;
-                }
-                row += nwaves;
-                if (EPI == EPI_RESID) rcur = fz.resid[min(row, n - 1)];   // consumed a whole row of steps later
+                for (int st = 0; st < 4; st++)
+                    if (st < steps) accumulate(pre[st], st);
+                finish_row();
+                wp += wave_stride;
+                total_steps -= steps;
+                if (total_steps > 0) F::load_w(wa, wp, u0);
+            } else {
+                total_steps = 0;
             }
+        }
+        auto one_step = [&](const typename F::W &cur, typename F::W &nxt, int t) {
+            // next (row, step); past the end the last unit is re-read
+            int ni = i + 1;
+            const uint8_t *nwp = wp;
+            if (ni == steps) { ni = 0; nwp = wp + wave_stride; }
+            if (t + 1 >= total_steps) { ni = i; nwp = wp; }
+            F::load_w(nxt, nwp, min(lane + 64 * ni, units - 1));
+            accumulate(cur, i);
+            if (i == steps - 1) finish_row();
             i = ni;
             wp = nwp;
         };
@@ -311,7 +350,7 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
     }
 }
 
-template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE>
+template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
 int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s,
                const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr}) {
     // waves per workgroup: as many as still leave every wave a row when 256 workgroups are launched
@@ -333,7 +372,7 @@ int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64
     if (rb > 0x3fffffff) return CQ_ERR_RANGE;
     g.row_bytes = (int)rb;
     g.dst_dtype = dst_dtype; g.stride_dst = stride_dst;
-    auto kern = qmv_kernel<DT, NB, SRC, SINGLE, PRO, EPI>;
+    auto kern = qmv_kernel<DT, NB, SRC, SINGLE, PRO, EPI, PRE>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
@@ -345,6 +384,8 @@ int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64
 template <int DT, int NB, int SRC>
 int launch_nb(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
     if (k / Fmt<DT>::UE <= 64) return launch_cfg<DT, NB, SRC, true>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+    if (NB == 1 && k / Fmt<DT>::UE <= 256)
+        return launch_cfg<DT, NB, SRC, false, PRO_NONE, EPI_NONE, NB == 1>(w, src, dst, dst_dtype, k, n, stride_dst, s);
     return launch_cfg<DT, NB, SRC, false>(w, src, dst, dst_dtype, k, n, stride_dst, s);
 }
 
@@ -435,6 +476,7 @@ template <int DT, int PRO, int EPI>
 int launch_fused1(const void *w, const ActSrc &src, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
     if (cq_act_layout(DT, k, 1).total + 64 > LDS_BUDGET) return CQ_ERR_RANGE;
     if (k / Fmt<DT>::UE <= 64) return launch_cfg<DT, 1, CQ_F32, true, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
+    if (k / Fmt<DT>::UE <= 256) return launch_cfg<DT, 1, CQ_F32, false, PRO, EPI, true>(w, src, dst, CQ_F32, k, n, n, s, fz);
     return launch_cfg<DT, 1, CQ_F32, false, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
 }
 template <int PRO, int EPI>

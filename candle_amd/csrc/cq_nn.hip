@@ -299,6 +299,191 @@ __global__ __launch_bounds__(HD) void attn_combine_kernel(const float *__restric
     out[rh * HD + threadIdx.x] = num / den;
 }
 
+// ---- one decode step of attention (one new token) ------------------------------------------------------
+// rope_i on q and on the new k, append of the new k / v to the cache, attention over keys [0, p].  Same
+// arithmetic as rope_kv_kernel + attn_kernel; what changes is where it runs:
+//   * q is rotated in registers; the workgroup whose split contains position p takes the new key and value
+//     from the projection outputs instead of the cache, rotates the key, uses both, and writes them to the cache;
+//   * a workgroup is 16 waves over one split of 128 keys, so a wave scores 8 keys and accumulates 8 values, and
+//     every K and V row is requested before anything is consumed (one memory round trip);
+//   * the result is left as per-split partials { acc[HD], m, l, 0, 0 } (stride HD + 4 floats, 16-byte aligned
+//     rows); attn_merge_kernel, or the prologue of the attention_wo matvec, merges them.
+constexpr int ATTD_WAVES = 16;
+constexpr int ATTD_MAX_SPLITS = 16;
+
+template <int HD, int G>
+__global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
+                                                                      const float *__restrict__ v_new, float *k_cache, float *v_cache,
+                                                                      const float *__restrict__ cos_t, const float *__restrict__ sin_t,
+                                                                      float *__restrict__ part, const int32_t *__restrict__ pos_dev, int pos0,
+                                                                      int ctx, float scale, int splits) {
+    constexpr int NW = ATTD_WAVES;
+    constexpr int DPL = HD / 64, EPL = HD / 16, IT = ATT_SPLIT / (4 * NW), VU = ATT_SPLIT / NW;
+    __shared__ float sc[G * ATT_SPLIT];
+    __shared__ float red[NW * G * HD];
+    __shared__ float ml[2 * G];
+    const int kvh = blockIdx.x, sp = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int p = min(pos0 + (pos_dev ? pos_dev[0] : 0), ctx - 1);
+    const int kv_len = p + 1;
+    const int j0 = sp * ATT_SPLIT;
+    const int cnt = min(kv_len - j0, ATT_SPLIT);
+    const int last = max(cnt - 1, 0);
+    float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
+    const int sub = lane & 15, kq = lane >> 4;
+
+    // ---- every load of the kernel, issued before any use ----
+    f32x4 kd[IT][EPL / 4];
+#pragma unroll
+    for (int it = 0; it < IT; it++) {
+        const int key = min((it * NW + wv) * 4 + kq, last);
+        const float *src = (j0 + key == p) ? k_new + kvh * HD + EPL * sub : kb + (int64_t)(j0 + key) * HD + EPL * sub;
+#pragma unroll
+        for (int c = 0; c < EPL / 4; c++) kd[it][c] = reinterpret_cast<const f32x4 *>(src)[c];
+    }
+    float vv[VU][DPL];
+#pragma unroll
+    for (int u = 0; u < VU; u++) {
+        const int j = min(wv + NW * u, last);
+        const float *src = (j0 + j == p) ? v_new + kvh * HD + DPL * lane : vb + (int64_t)(j0 + j) * HD + DPL * lane;
+        if (DPL == 2) {
+            const float2 t = *reinterpret_cast<const float2 *>(src);
+            vv[u][0] = t.x; vv[u][DPL - 1] = t.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < DPL; e++) vv[u][e] = src[e];
+        }
+    }
+    f32x4 qf[G][EPL / 4];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const f32x4 *qr = reinterpret_cast<const f32x4 *>(q + (int64_t)(kvh * G + g) * HD + EPL * sub);
+#pragma unroll
+        for (int c = 0; c < EPL / 4; c++) qf[g][c] = qr[c];
+    }
+    // cos / sin of position p for this lane's EPL/2 pairs
+    float cs[EPL / 2], sn[EPL / 2];
+#pragma unroll
+    for (int c = 0; c < EPL / 2; c++) {
+        cs[c] = cos_t[(int64_t)p * (HD / 2) + (EPL / 2) * sub + c];
+        sn[c] = sin_t[(int64_t)p * (HD / 2) + (EPL / 2) * sub + c];
+    }
+    auto rope4 = [&](f32x4 &v, int c) {       // two interleaved pairs (rotary_emb.rs:52-70)
+        const float a = v.x * cs[2 * c] - v.y * sn[2 * c], b = v.x * sn[2 * c] + v.y * cs[2 * c];
+        const float e = v.z * cs[2 * c + 1] - v.w * sn[2 * c + 1], f = v.z * sn[2 * c + 1] + v.w * cs[2 * c + 1];
+        v = f32x4{a, b, e, f};
+    };
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int c = 0; c < EPL / 4; c++) rope4(qf[g][c], c);
+
+    // ---- phase 1: scores; the lanes holding the new key rotate it and append it to the cache ----
+#pragma unroll
+    for (int it = 0; it < IT; it++) {
+        const int key = (it * NW + wv) * 4 + kq;
+        if (j0 + key == p) {
+#pragma unroll
+            for (int c = 0; c < EPL / 4; c++) {
+                rope4(kd[it][c], c);
+                reinterpret_cast<f32x4 *>(kb + (int64_t)p * HD + EPL * sub)[c] = kd[it][c];
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float a = 0.0f;
+#pragma unroll
+            for (int c = 0; c < EPL / 4; c++) {
+                a += qf[g][c].x * kd[it][c].x;
+                a += qf[g][c].y * kd[it][c].y;
+                a += qf[g][c].z * kd[it][c].z;
+                a += qf[g][c].w * kd[it][c].w;
+            }
+            a = row16_sum(a);
+            if (sub == 0) sc[g * ATT_SPLIT + key] = key < cnt ? a * scale : -INFINITY;
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 2: wave g handles query head g ----
+    if (wv < G) {
+        const int g = wv;
+        float s[ATT_SPLIT / 64], m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < ATT_SPLIT / 64; i++) {
+            s[i] = sc[g * ATT_SPLIT + lane + 64 * i];
+            m = fmaxf(m, s[i]);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        float l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < ATT_SPLIT / 64; i++) {
+            const float pr = (cnt > 0 && s[i] > -INFINITY) ? __expf(s[i] - m) : 0.0f;
+            sc[g * ATT_SPLIT + lane + 64 * i] = pr;
+            l += pr;
+        }
+        l = wave_sum(l);
+        if (lane == 0) { ml[2 * g] = m; ml[2 * g + 1] = l; }
+    }
+    __syncthreads();
+
+    // ---- phase 3: p . v from registers; the wave holding the new value appends it ----
+    float o[G][DPL];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int e = 0; e < DPL; e++) o[g][e] = 0.0f;
+#pragma unroll
+    for (int u = 0; u < VU; u++) {
+        const int j = wv + NW * u;                    // < ATT_SPLIT; entries at or beyond cnt hold p = 0
+        if (j0 + j == p) {
+#pragma unroll
+            for (int e = 0; e < DPL; e++) vb[(int64_t)p * HD + DPL * lane + e] = vv[u][e];
+        }
+        if (j < cnt) {                                // wave-uniform
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float pr = sc[g * ATT_SPLIT + j];
+#pragma unroll
+                for (int e = 0; e < DPL; e++) o[g][e] += pr * vv[u][e];
+            }
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int e = 0; e < DPL; e++) red[(wv * G + g) * HD + DPL * lane + e] = o[g][e];
+    __syncthreads();
+    for (int i = tid; i < G * HD; i += 64 * NW) {
+        const int g = i / HD, d = i - g * HD;
+        float a = 0.0f;
+#pragma unroll
+        for (int w2 = 0; w2 < NW; w2++) a += red[(w2 * G + g) * HD + d];
+        float *pp = part + ((int64_t)(kvh * G + g) * splits + sp) * (HD + 4);
+        pp[d] = a;
+        if (d < 4) pp[HD + d] = d == 0 ? ml[2 * g] : d == 1 ? ml[2 * g + 1] : 0.0f;
+    }
+}
+
+// merge the { acc[HD], m, l } partials of one head: out = sum_s e^{m_s - M} acc_s / sum_s e^{m_s - M} l_s
+template <int HD>
+__global__ __launch_bounds__(HD) void attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int splits) {
+    const float *pp = part + (int64_t)blockIdx.x * splits * (HD + 4);
+    float M = -INFINITY;
+    for (int s = 0; s < splits; s++) M = fmaxf(M, pp[s * (HD + 4) + HD + 1] > 0.0f ? pp[s * (HD + 4) + HD] : -INFINITY);
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < splits; s++) {
+        const float l = pp[s * (HD + 4) + HD + 1];
+        if (l > 0.0f) {
+            const float w = __expf(pp[s * (HD + 4) + HD] - M);
+            num += w * pp[s * (HD + 4) + threadIdx.x];
+            den += w * l;
+        }
+    }
+    out[(int64_t)blockIdx.x * HD + threadIdx.x] = num / den;
+}
+
 // ---- out = silu(gate) * up, silu(v) = v / (1 + exp(-v))  (candle-core/src/op.rs Silu; quantized_llama.rs:56-63) ----
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up, float *__restrict__ out, int dim,
                                                        int64_t gate_stride, int64_t up_stride) {
@@ -452,6 +637,65 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
         return (int)hipGetLastError();
     }
     return CQ_OK;
+}
+
+int64_t cq_nn_attention_decode_workspace_bytes(int64_t n_head, int64_t head_dim, int64_t max_kv_len) {
+    if (n_head <= 0 || head_dim <= 0 || max_kv_len <= 0) return -1;
+    return n_head * attn_splits(max_kv_len) * (head_dim + 4) * 4;
+}
+
+int64_t cq_nn_attention_decode_splits(int64_t max_kv_len) {
+    if (max_kv_len <= 0) return -1;
+    const int64_t s = attn_splits(max_kv_len);
+    return s <= ATTD_MAX_SPLITS ? s : -1;
+}
+
+int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const float *v_new_dev, float *k_cache_dev, float *v_cache_dev,
+                           const float *cos_dev, const float *sin_dev, float *out_dev, const int32_t *pos_dev, int64_t pos, int64_t n_head,
+                           int64_t n_kv_head, int64_t head_dim, int64_t ctx, int64_t max_kv_len, float scale, void *partials_dev,
+                           int64_t partials_bytes, void *stream) {
+    if (n_head <= 0 || n_kv_head <= 0 || n_head % n_kv_head || ctx <= 0 || pos < 0 || max_kv_len <= 0 || max_kv_len > ctx) return CQ_ERR_SHAPE;
+    if (head_dim != 64 && head_dim != 128) return CQ_ERR_RANGE;
+    if (!q_dev || !k_new_dev || !v_new_dev || !k_cache_dev || !v_cache_dev || !cos_dev || !sin_dev || !partials_dev) return CQ_ERR_NULL;
+    if (misaligned(q_dev, 16) || misaligned(k_new_dev, 16) || misaligned(v_new_dev, 16) || misaligned(k_cache_dev, 16) ||
+        misaligned(v_cache_dev, 16) || misaligned(partials_dev, 16))
+        return CQ_ERR_ALIGN;
+    if (!pos_dev && pos + 1 > max_kv_len) return CQ_ERR_RANGE;
+    if (partials_bytes < cq_nn_attention_decode_workspace_bytes(n_head, head_dim, max_kv_len)) return CQ_ERR_WORKSPACE;
+    const int64_t splits = attn_splits(max_kv_len);
+    if (splits > ATTD_MAX_SPLITS || ctx > 0x7fffffffLL) return CQ_ERR_RANGE;
+    const int G = (int)(n_head / n_kv_head);
+    float *part = (float *)partials_dev;
+    dim3 grid((unsigned)n_kv_head, (unsigned)splits);
+    hipStream_t s = (hipStream_t)stream;
+#define CQ_ATTD(HH, GG)                                                                                                                   \
+    hipLaunchKernelGGL((attn_decode_kernel<HH, GG>), grid, dim3(64 * ATTD_WAVES), 0, s, q_dev, k_new_dev, v_new_dev, k_cache_dev, v_cache_dev, \
+                       cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits)
+    if (head_dim == 128) {
+        switch (G) {
+            case 1: CQ_ATTD(128, 1); break;
+            case 2: CQ_ATTD(128, 2); break;
+            case 4: CQ_ATTD(128, 4); break;
+            case 8: CQ_ATTD(128, 8); break;
+            default: return CQ_ERR_RANGE;
+        }
+    } else {
+        switch (G) {
+            case 1: CQ_ATTD(64, 1); break;
+            case 2: CQ_ATTD(64, 2); break;
+            case 4: CQ_ATTD(64, 4); break;
+            case 8: CQ_ATTD(64, 8); break;
+            default: return CQ_ERR_RANGE;
+        }
+    }
+#undef CQ_ATTD
+    int rc = (int)hipGetLastError();
+    if (rc || !out_dev) return rc;
+    if (head_dim == 128)
+        hipLaunchKernelGGL((attn_merge_kernel<128>), dim3((unsigned)n_head), dim3(128), 0, s, (const float *)part, out_dev, (int)splits);
+    else
+        hipLaunchKernelGGL((attn_merge_kernel<64>), dim3((unsigned)n_head), dim3(64), 0, s, (const float *)part, out_dev, (int)splits);
+    return (int)hipGetLastError();
 }
 
 int cq_nn_silu_mul(const float *gate_dev, const float *up_dev, float *out_dev, int64_t rows, int64_t dim, int64_t gate_stride, int64_t up_stride,

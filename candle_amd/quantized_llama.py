@@ -170,6 +170,9 @@ class ModelWeights:
         self.ws = torch.empty(max(need, 256), dtype=torch.uint8, device=self.device)
         att_ws = L.cq_nn_attention_workspace_bytes(max_rows, cfg.n_head, cfg.head_dim, cfg.ctx)
         self.att_ws = torch.empty(max(att_ws, 256), dtype=torch.uint8, device=self.device)
+        # single-token attention: per-split partials
+        attd = L.cq_nn_attention_decode_workspace_bytes(cfg.n_head, cfg.head_dim, min(cfg.ctx, 2048))
+        self.attd_ws = torch.zeros(attd, dtype=torch.uint8, device=self.device)
 
     @classmethod
     def random_init(cls, cfg: Config, seed: int = 0, device="cuda:0", dtypes: Optional[Dict[str, GgmlDType]] = None,
@@ -241,7 +244,7 @@ class ModelWeights:
         scale = float(np.float32(1.0 / math.sqrt(cfg.head_dim)))
         ck = _lib.check
         x, xn, qk, v, att, delta, gu, h = self.x, self.xn, self.qk, self.v, self.att, self.delta, self.gu, self.h
-        if rows == 1 and self.fuse_decode:
+        if rows == 1 and self.fuse_decode and self.L.cq_nn_attention_decode_splits(max_kv_len) > 0:
             return self._enqueue_decode_fused(ids_ptr, pos, pos_dev_ptr, max_kv_len, sp)
         ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), rows, cfg.hidden, cfg.vocab, None, sp))
         for li, lw in enumerate(self.layers):
@@ -318,12 +321,11 @@ class ModelWeights:
                 norm_mm(wk, kvd, lw.attention_norm, qk.data_ptr() + 4 * qd)
             norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
             q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
-            ck("cq_nn_rope_i_kv", L.cq_nn_rope_i_kv(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
-                                                   self.cos.data_ptr(), self.sin.data_ptr(), pos_dev_ptr, pos, 1, cfg.n_head, cfg.n_kv_head,
-                                                   cfg.head_dim, cfg.ctx, qd + kvd, qd + kvd, kvd, sp))
-            ck("cq_nn_attention", L.cq_nn_attention(q_ptr, qd + kvd, lw.k_cache.data_ptr(), lw.v_cache.data_ptr(), att.data_ptr(), pos_dev_ptr, pos,
-                                                   1, cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
-                                                   self.att_ws.data_ptr(), self.att_ws.numel(), sp))
+            # rope, cache append, attention and the merge of the key splits in one kernel          :217-261
+            ck("cq_nn_attention_decode", L.cq_nn_attention_decode(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
+                                                                  self.cos.data_ptr(), self.sin.data_ptr(), att.data_ptr(), pos_dev_ptr, pos,
+                                                                  cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
+                                                                  self.attd_ws.data_ptr(), self.attd_ws.numel(), sp))
             resid_mm(w["attention_wo"], att.data_ptr(), None)
             w1, w3 = w["feed_forward_w1"], w["feed_forward_w3"]
             if w1.dtype == w3.dtype and w3.ptr == w1.ptr + w1.nbytes:

@@ -59,6 +59,21 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
                     const int32_t *pos_dev, int64_t pos, int64_t rows, int64_t n_head, int64_t n_kv_head, int64_t head_dim, int64_t ctx,
                     int64_t max_kv_len, float scale, void *workspace_dev, int64_t workspace_bytes, void *stream);
 
+/* One decode step (a single new token at position p = pos + *pos_dev) of the three calls above:
+ * rope_i on q and on the new k, append of the new k and v to the cache at p, attention of the rotated q over keys
+ * [0, p].  q [n_head*head_dim], k_new / v_new [n_kv_head*head_dim] are the raw projection outputs (16-byte aligned;
+ * q is not modified).  The result is left in partials_dev as per-split records { acc[head_dim], m, l, 0, 0 } for
+ * every head ([n_head][splits][head_dim + 4] floats, splits = cq_nn_attention_decode_splits(max_kv_len), at most 16,
+ * i.e. max_kv_len <= 2048; -1 beyond).  When out_dev != NULL a second small kernel merges them into
+ * out_dev [n_head*head_dim]; with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn.
+ * No counterpart in the reference, which runs these as separate tensor ops (quantized_llama.rs:217-261). */
+int64_t cq_nn_attention_decode_workspace_bytes(int64_t n_head, int64_t head_dim, int64_t max_kv_len);
+int64_t cq_nn_attention_decode_splits(int64_t max_kv_len);
+int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const float *v_new_dev, float *k_cache_dev, float *v_cache_dev,
+                           const float *cos_dev, const float *sin_dev, float *out_dev, const int32_t *pos_dev, int64_t pos, int64_t n_head,
+                           int64_t n_kv_head, int64_t head_dim, int64_t ctx, int64_t max_kv_len, float scale, void *partials_dev,
+                           int64_t partials_bytes, void *stream);
+
 /* out = silu(gate) * up with silu(v) = v / (1 + exp(-v)): Mlp::forward, quantized_llama.rs:56-63
  * (candle_nn::ops::silu, candle-core/src/op.rs Silu::f32).  gate/up rows may be strided views of one buffer. */
 int cq_nn_silu_mul(const float *gate_dev, const float *up_dev, float *out_dev, int64_t rows, int64_t dim, int64_t gate_stride, int64_t up_stride,

@@ -142,6 +142,38 @@ def test_attention_single_key_returns_value():
         assert np.array_equal(got[h], vc[h // 2, 0])
 
 
+@pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (32, 8, 128)])
+@pytest.mark.parametrize("pos,ctx,max_kv", [(0, 16, 1), (5, 64, 64), (127, 256, 200), (128, 256, 256), (300, 1024, 301), (600, 1024, 1024)])
+def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
+    """rope + cache append + attention over 128-key splits (+ merge kernel) == the separate calls == the CPU ops;
+    called twice in a row on fresh caches."""
+    lib = L()
+    cos, sin = lo.precomput_freqs_cis(D, 500000.0, ctx)
+    q, k, v = normal(30, (1, H * D), 1.0), normal(31, (1, KV * D), 1.0), normal(32, (1, KV * D), 1.0)
+    kc0, vc0 = normal(33, (KV, ctx, D), 1.0), normal(34, (KV, ctx, D), 1.0)
+    kc0[:, pos:], vc0[:, pos:] = np.nan, np.nan          # nothing at or beyond the new position may be read
+    wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
+    assert lib.cq_nn_attention_decode_splits(max_kv) == (max_kv + 127) // 128 and lib.cq_nn_attention_decode_splits(2049) == -1
+    ws = torch.full((wsb,), 0xff, dtype=torch.uint8, device="cuda")
+    posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    c, s = cos[pos:pos + 1], sin[pos:pos + 1]
+    want_q = lo.rope_i(q.reshape(1, H, D).transpose(1, 0, 2)[None], c, s)[0].transpose(1, 0, 2).reshape(1, H * D)
+    want_k = lo.rope_i(k.reshape(1, KV, D).transpose(1, 0, 2)[None], c, s)[0]
+    kc_ref, vc_ref = kc0.copy(), vc0.copy()
+    kc_ref[:, pos:pos + 1], vc_ref[:, pos:pos + 1] = want_k, v.reshape(1, KV, D).transpose(1, 0, 2)
+    want = attention_oracle(want_q, kc_ref, vc_ref, pos, H, KV, D)
+    for attempt in range(2):
+        kc, vc, out = dev(kc0), dev(vc0), torch.zeros((1, H * D), device="cuda")
+        ok(lib.cq_nn_attention_decode(dev(q).data_ptr(), dev(k).data_ptr(), dev(v).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(),
+                                      dev(sin).data_ptr(), out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv,
+                                      float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None))
+        torch.cuda.synchronize()
+        assert rel_l2(out.cpu().numpy(), want) <= TOL, attempt
+        assert np.allclose(kc.cpu().numpy()[:, pos], want_k[:, 0], rtol=1e-6, atol=1e-6)
+        assert np.array_equal(vc.cpu().numpy()[:, pos], vc_ref[:, pos])
+        assert np.array_equal(kc.cpu().numpy()[:, :pos], kc0[:, :pos])
+
+
 def test_silu_mul_strided_views():
     rows, dim = 3, 1024
     gu = normal(14, (rows, 2 * dim), 2.0)
