@@ -262,4 +262,16 @@ int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, c
     return cq_matvec_residual_launch(w_dtype, w_dev, x_dev, up_dev, residual_dev, sumsq_partials_out_dev, k, n, (hipStream_t)stream);
 }
 
+int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
+                                float *residual_dev, float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, 1);
+    if (rc) return rc;
+    if (n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!attn_partials_dev || !residual_dev || !sumsq_partials_out_dev) return CQ_ERR_NULL;
+    if (!aligned(attn_partials_dev, 16) || !aligned(residual_dev, 4) || !aligned(sumsq_partials_out_dev, 4)) return CQ_ERR_ALIGN;
+    return cq_matvec_residual_attn_launch(w_dtype, w_dev, attn_partials_dev, splits, head_dim, residual_dev, sumsq_partials_out_dev, k, n,
+                                          (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -36,17 +36,21 @@ struct ActSrc {
 //   PRO_NORM  the activation row is rms_norm(x) * norm_weight; sum(x^2) arrives as CQ_NN_PARTIALS partial sums
 //             written by the producer of x, so no workgroup-wide reduction is needed before quantizing
 //   PRO_SILU  the activation row is silu(x) * up
+//   PRO_MERGE the activation row is the attention output, merged on the fly from the per-split partials
+//             { acc[hd], m, l, 0, 0 } the single-token attention kernel leaves (rows of one wave step only)
 //   EPI_RESID the result is added to a residual row in place of being stored, and the workgroup leaves
 //             its partial sum of residual^2 for the next PRO_NORM consumer
-enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2 };
+enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2, PRO_MERGE = 3 };
+constexpr int MAXS = 16;     // attention splits a PRO_MERGE prologue can merge
 enum { EPI_NONE = 0, EPI_RESID = 1 };
 constexpr int NPART = 256;   // == CQ_NN_PARTIALS
 struct Fuse {
-    const float *aux;        // PRO_NORM: norm weight [k];  PRO_SILU: up [k]
+    const float *aux;        // PRO_NORM: norm weight [k];  PRO_SILU: up [k];  PRO_MERGE: partials [k/hd][splits][hd + 4]
     const float *part_in;    // PRO_NORM: [NPART]
     float eps;
     float *resid;            // EPI_RESID: [n], updated in place
     float *part_out;         // EPI_RESID: [NPART]
+    int splits, hd_shift;    // PRO_MERGE
 };
 
 // Launch geometry, computed once on the host so the kernel prologue is a handful of scalar loads
@@ -74,10 +78,48 @@ __device__ __forceinline__ void pro_apply(float v[4], const float a[4], float m)
     }
 }
 
+// PRO_MERGE: the lane's four consecutive elements [base, base + 4) of the attention output, from the partials
+template <int MS> struct MergeRegs { float m[MS], l[MS]; f32x4 a[MS]; };
+template <int MS>
+__device__ __forceinline__ void merge_load(const Fuse &fz, int base, bool ok, MergeRegs<MS> &r) {
+    const int hd = 1 << fz.hd_shift;
+    const float *pp = fz.aux + (int64_t)(base >> fz.hd_shift) * fz.splits * (hd + 4);
+    const int d = base & (hd - 1);
+#pragma unroll
+    for (int sI = 0; sI < MS; sI++) {
+        r.m[sI] = -INFINITY; r.l[sI] = 0.0f; r.a[sI] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (ok && sI < fz.splits) {
+            const float *rec = pp + sI * (hd + 4);
+            r.a[sI] = *reinterpret_cast<const f32x4 *>(rec + d);
+            const float2 t = *reinterpret_cast<const float2 *>(rec + hd);
+            r.m[sI] = t.x; r.l[sI] = t.y;
+        }
+    }
+}
+template <int MS>
+__device__ __forceinline__ void merge_reduce(const MergeRegs<MS> &r, bool ok, float v[4]) {
+    // same operation order as the stand-alone merge kernel: identical bits
+    float M = -INFINITY;
+#pragma unroll
+    for (int sI = 0; sI < MS; sI++) M = fmaxf(M, r.l[sI] > 0.0f ? r.m[sI] : -INFINITY);
+    f32x4 num = {0.0f, 0.0f, 0.0f, 0.0f};
+    float den = 0.0f;
+#pragma unroll
+    for (int sI = 0; sI < MS; sI++) {
+        if (r.l[sI] > 0.0f) {
+            const float wgt = __expf(r.m[sI] - M);
+            num.x += wgt * r.a[sI].x; num.y += wgt * r.a[sI].y; num.z += wgt * r.a[sI].z; num.w += wgt * r.a[sI].w;
+            den += wgt * r.l[sI];
+        }
+    }
+    if (ok) { v[0] = num.x / den; v[1] = num.y / den; v[2] = num.z / den; v[3] = num.w / den; }
+}
+
 template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
 __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g, Fuse fz) {
     typedef Fmt<DT> F;
     static_assert((PRO == PRO_NONE && EPI == EPI_NONE) || (NB == 1 && SRC == CQ_F32), "fusions are for one f32 row");
+    static_assert(PRO != PRO_MERGE || (SINGLE && !PRE), "the merge prologue preloads one span per wave");
     constexpr bool FUSED = SRC != SRC_SCRATCH;
     constexpr int XDT = FUSED ? SRC : CQ_F32;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -115,7 +157,11 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
     u32x2 c_d = {0, 0};
     uint32_t c_bs = 0;
     float pp[NPART / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (FUSED) {
+    constexpr int MS = PRO == PRO_MERGE ? MAXS : 1;
+    MergeRegs<MS> mg;
+    if (FUSED && PRO == PRO_MERGE) {
+        merge_load<MS>(fz, xbase, xbase < total, mg);
+    } else if (FUSED) {
 #pragma unroll
         for (int j = 0; j < XS; j++) {
             if (xbase + j * xstep < total) cq_load4<XDT>(src.x, xbase + j * xstep, xv[j]);
@@ -167,10 +213,11 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
             const float sum2 = wave_sum((pp[0] + pp[1]) + (pp[2] + pp[3]));
             pm = sqrtf(sum2 / (float)k + fz.eps);
         }
+        if (PRO == PRO_MERGE) merge_reduce<MS>(mg, xbase < total, xv[0]);
 #pragma unroll
         for (int j = 0; j < XS; j++) {
             const int span = wv_s + (j << g.nw_shift);
-            pro_apply<PRO>(xv[j], av4[j], pm);
+            if (PRO == PRO_NORM || PRO == PRO_SILU) pro_apply<PRO>(xv[j], av4[j], pm);
             if (span < spans) {
                 if (cq_is_kquant(DT))
                     cq_quantize_q8k_vals(xv[j], span, lane, lqs, ld, lbs);
@@ -188,11 +235,18 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
                 const int base = span * 256 + lane * 4;
                 const bool ok = base < total;
                 float v[4] = {0.0f, 0.0f, 0.0f, 0.0f}, a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (ok) {
-                    cq_load4<XDT>(src.x, base, v);
-                    cq_load4<CQ_F32>(fz.aux, base, a);
+                if (PRO == PRO_MERGE) {
+                    // fewer waves than spans (a short weight matrix): later spans are merged here
+                    MergeRegs<MS> mr;
+                    merge_load<MS>(fz, base, ok, mr);
+                    merge_reduce<MS>(mr, ok, v);
+                } else {
+                    if (ok) {
+                        cq_load4<XDT>(src.x, base, v);
+                        cq_load4<CQ_F32>(fz.aux, base, a);
+                    }
+                    pro_apply<PRO>(v, a, pm);
                 }
-                pro_apply<PRO>(v, a, pm);
                 if (cq_is_kquant(DT))
                     cq_quantize_q8k_vals(v, span, lane, lqs, ld, lbs);
                 else
@@ -352,7 +406,7 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
 
 template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
 int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s,
-               const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr}) {
+               const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0}) {
     // waves per workgroup: as many as still leave every wave a row when 256 workgroups are launched
     int waves = 16;
     while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
@@ -497,7 +551,7 @@ int cq_matvec_norm_launch(int w_dtype, const void *w, const float *x, const floa
                           int64_t k, int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{norm_weight, partials, eps, nullptr, nullptr};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0};
     return launch_fused_dt<PRO_NORM, EPI_NONE>(w_dtype, w, src, dst, k, n, s, fz);
 }
 
@@ -506,7 +560,36 @@ int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const 
                               int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{up, nullptr, 0.0f, residual, partials_out};
+    Fuse fz{up, nullptr, 0.0f, residual, partials_out, 0, 0};
     if (up) return launch_fused_dt<PRO_SILU, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
     return launch_fused_dt<PRO_NONE, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
+}
+
+namespace {
+template <int DT>
+int launch_merge1(const void *w, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
+    if (k / Fmt<DT>::UE > 64) return CQ_ERR_RANGE;          // one wave step per row, one span per wave
+    ActSrc src{nullptr, ActView{nullptr, nullptr, nullptr}};
+    return launch_cfg<DT, 1, CQ_F32, true, PRO_MERGE, EPI_RESID>(w, src, dst, CQ_F32, k, n, n, s, fz);
+}
+}  // namespace
+
+// residual[n] += W . quantize(merge(attention partials)); partials_out[256] = partial sums of residual^2.
+// CQ_ERR_RANGE when the row is longer than one wave step (k > 4096 for K-quants, > 2048 for Q4_0 / Q8_0),
+// when splits > 16, or when head_dim is not a power of two.
+int cq_matvec_residual_attn_launch(int w_dtype, const void *w, const float *attn_partials, int64_t splits, int64_t head_dim, float *residual,
+                                   float *partials_out, int64_t k, int64_t n, hipStream_t s) {
+    if (n == 0) return CQ_OK;
+    if (splits < 1 || splits > MAXS || head_dim < 4 || (head_dim & (head_dim - 1)) || k % head_dim) return CQ_ERR_RANGE;
+    int sh = 0;
+    while ((1 << sh) < head_dim) sh++;
+    Fuse fz{attn_partials, nullptr, 0.0f, residual, partials_out, (int)splits, sh};
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_merge1<CQ_Q4_0>(w, nullptr, k, n, s, fz);
+        case CQ_Q8_0: return launch_merge1<CQ_Q8_0>(w, nullptr, k, n, s, fz);
+        case CQ_Q4K: return launch_merge1<CQ_Q4K>(w, nullptr, k, n, s, fz);
+        case CQ_Q5K: return launch_merge1<CQ_Q5K>(w, nullptr, k, n, s, fz);
+        case CQ_Q6K: return launch_merge1<CQ_Q6K>(w, nullptr, k, n, s, fz);
+    }
+    return CQ_ERR_DTYPE;
 }

@@ -322,11 +322,20 @@ class ModelWeights:
             norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
             q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
             # rope, cache append, attention and the merge of the key splits in one kernel          :217-261
+            wo = w["attention_wo"]
+            merge_in_wo = qd <= (4096 if wo.dtype in (GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K) else 2048) and \
+                (cfg.head_dim & (cfg.head_dim - 1)) == 0
             ck("cq_nn_attention_decode", L.cq_nn_attention_decode(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
-                                                                  self.cos.data_ptr(), self.sin.data_ptr(), att.data_ptr(), pos_dev_ptr, pos,
+                                                                  self.cos.data_ptr(), self.sin.data_ptr(),
+                                                                  None if merge_in_wo else att.data_ptr(), pos_dev_ptr, pos,
                                                                   cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
                                                                   self.attd_ws.data_ptr(), self.attd_ws.numel(), sp))
-            resid_mm(w["attention_wo"], att.data_ptr(), None)
+            if merge_in_wo:
+                ck("cq_nn_qmatmul_residual_attn", L.cq_nn_qmatmul_residual_attn(int(wo.dtype), wo.ptr, self.attd_ws.data_ptr(),
+                                                                                L.cq_nn_attention_decode_splits(max_kv_len), cfg.head_dim,
+                                                                                x.data_ptr(), part.data_ptr(), wo.k, cfg.hidden, sp))
+            else:
+                resid_mm(wo, att.data_ptr(), None)
             w1, w3 = w["feed_forward_w1"], w["feed_forward_w3"]
             if w1.dtype == w3.dtype and w3.ptr == w1.ptr + w1.nbytes:
                 norm_mm(w1, 2 * cfg.ffn, lw.ffn_norm, gu.data_ptr())

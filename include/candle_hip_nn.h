@@ -91,6 +91,12 @@ int cq_nn_qmatmul_norm(int w_dtype, const void *w_dev, const float *x_dev, const
                        float eps, float *dst_dev, int64_t k, int64_t n, void *stream);
 int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
                            float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream);
+/* cq_nn_qmatmul_residual whose input row is the attention output still in the per-split partials of
+ * cq_nn_attention_decode (out_dev == NULL there): the merge of the splits is the matvec's prologue.
+ * CQ_ERR_RANGE (use the merge kernel + cq_nn_qmatmul_residual instead) when k = n_head*head_dim is longer than one
+ * wave step per row (k > 4096 for K-quants, > 2048 for Q4_0 / Q8_0), splits > 16, or head_dim is not a power of 2. */
+int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
+                                float *residual_dev, float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream);
 
 /* Greedy sampling (LogitsProcessor with Sampling::ArgMax, candle-examples/examples/quantized/main.rs:603-604):
  * token_out[0] = index of the largest logit (lowest index on ties).  Optional bookkeeping for graph replay:

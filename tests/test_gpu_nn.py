@@ -174,6 +174,38 @@ def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
         assert np.array_equal(kc.cpu().numpy()[:, :pos], kc0[:, :pos])
 
 
+@pytest.mark.parametrize("dtype", [12, 14, 2])
+@pytest.mark.parametrize("pos,max_kv", [(3, 128), (700, 701), (700, 2048)])
+def test_attention_merge_as_matvec_prologue(dtype, pos, max_kv):
+    """attention partials merged inside the attention_wo matvec == merge kernel followed by the plain fused matvec, bit for bit."""
+    import oracle
+    lib = L()
+    H, KV, D, ctx, hidden = (32, 8, 128, 2048, 512) if dtype != 2 else (16, 4, 128, 2048, 512)
+    k = H * D
+    cos, sin = lo.precomput_freqs_cis(D, 500000.0, ctx)
+    q, kn, vn = normal(40, (1, k), 1.0), normal(41, (1, KV * D), 1.0), normal(42, (1, KV * D), 1.0)
+    kc, vc = dev(normal(43, (KV, ctx, D), 1.0)), dev(normal(44, (KV, ctx, D), 1.0))
+    w = dev(oracle.from_float(dtype, normal(45, (hidden, k), 0.05).reshape(-1)))
+    wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
+    ws = torch.zeros(wsb, dtype=torch.uint8, device="cuda")
+    att = torch.empty((1, k), device="cuda")
+    args = (dev(q).data_ptr(), dev(kn).data_ptr(), dev(vn).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(), dev(sin).data_ptr())
+    tail = (None, pos, H, KV, D, ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None)
+    ok(lib.cq_nn_attention_decode(*args, att.data_ptr(), *tail))
+    res0 = normal(46, (1, hidden), 1.0)
+    r1, r2 = dev(res0), dev(res0)
+    p1, p2 = torch.empty(256, device="cuda"), torch.empty(256, device="cuda")
+    ok(lib.cq_nn_qmatmul_residual(dtype, w.data_ptr(), att.data_ptr(), None, r1.data_ptr(), p1.data_ptr(), k, hidden, None))
+    ok(lib.cq_nn_attention_decode(*args, None, *tail))
+    ok(lib.cq_nn_qmatmul_residual_attn(dtype, w.data_ptr(), ws.data_ptr(), lib.cq_nn_attention_decode_splits(max_kv), D, r2.data_ptr(),
+                                       p2.data_ptr(), k, hidden, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(r1.cpu().numpy(), r2.cpu().numpy()) and np.array_equal(p1.cpu().numpy(), p2.cpu().numpy())
+    assert not np.array_equal(r1.cpu().numpy(), res0)
+    assert lib.cq_nn_qmatmul_residual_attn(12, w.data_ptr(), ws.data_ptr(), 17, D, r2.data_ptr(), p2.data_ptr(), k, hidden, None) == -6
+    assert lib.cq_nn_qmatmul_residual_attn(12, w.data_ptr(), ws.data_ptr(), 2, D, r2.data_ptr(), p2.data_ptr(), 8192, hidden, None) == -6
+
+
 def test_silu_mul_strided_views():
     rows, dim = 3, 1024
     gu = normal(14, (rows, 2 * dim), 2.0)
