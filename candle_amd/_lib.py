@@ -39,6 +39,8 @@ SIGNATURES = {
     "cq_nn_embedding": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "cq_nn_qmatmul_norm": (_int, [_int, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
     "cq_nn_qmatmul_residual": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "cq_nn_qmatmul_norm_swiglu": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
+    "cq_nn_qmatmul_norm_pair": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _vp, _vp, _vp, _vp, _f32, _i64, _vp]),
     "cq_nn_qmatmul_residual_attn": (_int, [_int, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp]),
     "cq_nn_rms_norm": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "cq_nn_rope_i_kv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
@@ -48,7 +50,7 @@ SIGNATURES = {
     "cq_nn_attention_decode_splits": (_i64, [_i64]),
     "cq_nn_attention_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp]),
     "cq_nn_silu_mul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
-    "cq_nn_argmax": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "cq_nn_argmax": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
 }
 
 _lib = None

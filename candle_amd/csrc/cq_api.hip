@@ -262,6 +262,31 @@ int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, c
     return cq_matvec_residual_launch(w_dtype, w_dev, x_dev, up_dev, residual_dev, sumsq_partials_out_dev, k, n, (hipStream_t)stream);
 }
 
+int cq_nn_qmatmul_norm_swiglu(int w_dtype, const void *w1_dev, const void *w3_dev, const float *x_dev, const float *sumsq_partials_dev,
+                              const float *norm_weight_dev, float eps, float *dst_dev, int64_t k, int64_t ffn, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, ffn, 1);
+    if (rc) return rc;
+    if (ffn == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w1_dev)) || (rc = check_weight_ptr(w_dtype, w3_dev))) return rc;
+    if (!x_dev || !sumsq_partials_dev || !norm_weight_dev || !dst_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(norm_weight_dev, 16) || !aligned(sumsq_partials_dev, 4) || !aligned(dst_dev, 4)) return CQ_ERR_ALIGN;
+    return cq_matvec_norm_swiglu_launch(w_dtype, w1_dev, w3_dev, x_dev, sumsq_partials_dev, norm_weight_dev, eps, dst_dev, k, ffn,
+                                        (hipStream_t)stream);
+}
+
+int cq_nn_qmatmul_norm_pair(int w_dtype_a, const void *w_a_dev, int64_t n_a, float *dst_a_dev, int w_dtype_b, const void *w_b_dev, int64_t n_b,
+                            float *dst_b_dev, const float *x_dev, const float *sumsq_partials_dev, const float *norm_weight_dev, float eps,
+                            int64_t k, void *stream) {
+    int rc = check_mm_shape(w_dtype_a, k, n_a, 1);
+    if (rc || (rc = check_mm_shape(w_dtype_b, k, n_b, 1))) return rc;
+    if ((rc = check_weight_ptr(w_dtype_a, w_a_dev)) || (rc = check_weight_ptr(w_dtype_b, w_b_dev))) return rc;
+    if (!x_dev || !sumsq_partials_dev || !norm_weight_dev || !dst_a_dev || !dst_b_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(norm_weight_dev, 16) || !aligned(sumsq_partials_dev, 4) || !aligned(dst_a_dev, 4) || !aligned(dst_b_dev, 4))
+        return CQ_ERR_ALIGN;
+    return cq_matvec_norm_pair_launch(w_dtype_a, w_a_dev, n_a, dst_a_dev, w_dtype_b, w_b_dev, n_b, dst_b_dev, x_dev, sumsq_partials_dev,
+                                      norm_weight_dev, eps, k, (hipStream_t)stream);
+}
+
 int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
                                 float *residual_dev, float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream) {
     int rc = check_mm_shape(w_dtype, k, n, 1);

@@ -21,6 +21,10 @@ int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const 
                               int64_t n, hipStream_t s);
 int cq_matvec_residual_attn_launch(int w_dtype, const void *w, const float *attn_partials, int64_t splits, int64_t head_dim, float *residual,
                                    float *partials_out, int64_t k, int64_t n, hipStream_t s);
+int cq_matvec_norm_swiglu_launch(int w_dtype, const void *w1, const void *w3, const float *x, const float *partials, const float *norm_weight,
+                                 float eps, float *dst, int64_t k, int64_t ffn, hipStream_t s);
+int cq_matvec_norm_pair_launch(int dta, const void *wa, int64_t na, float *dsta, int dtb, const void *wb, int64_t nb, float *dstb, const float *x,
+                               const float *partials, const float *norm_weight, float eps, int64_t k, hipStream_t s);
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s);
 int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t count, hipStream_t s);

@@ -38,11 +38,13 @@ struct ActSrc {
 //   PRO_SILU  the activation row is silu(x) * up
 //   PRO_MERGE the activation row is the attention output, merged on the fly from the per-split partials
 //             { acc[hd], m, l, 0, 0 } the single-token attention kernel leaves (rows of one wave step only)
+//   EPI_SWIGLU a logical row r is the pair (W[r], W[r] + pair_off bytes) = (feed_forward_w1, feed_forward_w3):
+//             dst[r] = silu(W1[r] . x) * (W3[r] . x)   (rows of one wave step only)
 //   EPI_RESID the result is added to a residual row in place of being stored, and the workgroup leaves
 //             its partial sum of residual^2 for the next PRO_NORM consumer
 enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2, PRO_MERGE = 3 };
 constexpr int MAXS = 16;     // attention splits a PRO_MERGE prologue can merge
-enum { EPI_NONE = 0, EPI_RESID = 1 };
+enum { EPI_NONE = 0, EPI_RESID = 1, EPI_SWIGLU = 2 };
 constexpr int NPART = 256;   // == CQ_NN_PARTIALS
 struct Fuse {
     const float *aux;        // PRO_NORM: norm weight [k];  PRO_SILU: up [k];  PRO_MERGE: partials [k/hd][splits][hd + 4]
@@ -51,6 +53,7 @@ struct Fuse {
     float *resid;            // EPI_RESID: [n], updated in place
     float *part_out;         // EPI_RESID: [NPART]
     int splits, hd_shift;    // PRO_MERGE
+    int64_t pair_off;        // EPI_SWIGLU: byte distance from a row of w1 to the same row of w3
 };
 
 // Launch geometry, computed once on the host so the kernel prologue is a handful of scalar loads
@@ -115,11 +118,13 @@ __device__ __forceinline__ void merge_reduce(const MergeRegs<MS> &r, bool ok, fl
     if (ok) { v[0] = num.x / den; v[1] = num.y / den; v[2] = num.z / den; v[3] = num.w / den; }
 }
 
-template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
-__global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g, Fuse fz) {
+template <int DT, int NB, int SRC, bool SINGLE, int PRO, int EPI, bool PRE>
+__device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const ActSrc &src, void *__restrict__ dst, const QmvGeom &g, const Fuse &fz,
+                                         const int block, const int nblocks) {
     typedef Fmt<DT> F;
     static_assert((PRO == PRO_NONE && EPI == EPI_NONE) || (NB == 1 && SRC == CQ_F32), "fusions are for one f32 row");
     static_assert(PRO != PRO_MERGE || (SINGLE && !PRE), "the merge prologue preloads one span per wave");
+    static_assert(EPI != EPI_SWIGLU || SINGLE, "the paired-row epilogue is written for rows of one wave step");
     constexpr bool FUSED = SRC != SRC_SCRATCH;
     constexpr int XDT = FUSED ? SRC : CQ_F32;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -137,7 +142,7 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
     const int steps = g.steps;
     const int row_bytes = g.row_bytes;
     const int wave_stride = row_bytes << g.nw_shift;
-    const int wg_row0 = blockIdx.x * g.rows_per_wg;
+    const int wg_row0 = block * g.rows_per_wg;
     const int wg_row1 = min(n, wg_row0 + g.rows_per_wg);
 
     // 0. The activation loads go out first.  Vector loads complete in order, so anything issued after
@@ -267,7 +272,7 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
         }
     }
     __syncthreads();
-    if (EPI == EPI_NONE && my_rows == 0) return;
+    if (EPI != EPI_RESID && my_rows == 0) return;
     float ssq = 0.0f;            // EPI_RESID: lane 63 accumulates residual^2 of this wave's rows
 
     ActRow ar[NB];
@@ -301,6 +306,22 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
                 }
             }
         };
+        if (EPI == EPI_SWIGLU) {
+            // wa = W1[row] (already in flight), wb = W3[row]; the next W1 row is requested before W3 is reduced
+            for (int j = 0; j < my_rows; j++) {
+                F::load_w(wb, wp + fz.pair_off, u0);
+                float gate = F::dot(wa, areg[0], u0);
+                gate = wave_sum_to_lane63(valid ? gate : 0.0f);
+                const uint8_t *p1 = j + 1 < my_rows ? wp + wave_stride : wp;
+                F::load_w(wa, p1, u0);
+                float up = F::dot(wb, areg[0], u0);
+                up = wave_sum_to_lane63(valid ? up : 0.0f);
+                if (lane == 63) store_out(dst, dst_dtype, row, gate / (1.0f + expf(-gate)) * up);   // Mlp::forward, quantized_llama.rs:56-63
+                row += nwaves;
+                wp = p1;
+            }
+            return;
+        }
         // ping-pong between wa and wb: the next row's loads are in flight while this one is reduced;
         // the prefetch past the last row re-reads it instead of branching around the load.  The residual
         // value of a row travels behind its weights in the same in-order load queue.
@@ -397,25 +418,42 @@ __global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w
         if (tid == 0) {
             float t = 0.0f;
             for (int i = 0; i < nwaves; i++) t += red[i];
-            fz.part_out[blockIdx.x] = t;
+            fz.part_out[block] = t;
         }
-        if (blockIdx.x == 0)
-            for (int i = (int)gridDim.x + tid; i < NPART; i += nthr) fz.part_out[i] = 0.0f;
+        if (block == 0)
+            for (int i = nblocks + tid; i < NPART; i += nthr) fz.part_out[i] = 0.0f;
     }
 }
 
 template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
-int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s,
-               const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0}) {
-    // waves per workgroup: as many as still leave every wave a row when 256 workgroups are launched
-    int waves = 16;
-    while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
-    int64_t groups = n >= 256 * (int64_t)waves ? 256 : (n + waves - 1) / waves;
+__global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g, Fuse fz) {
+    qmv_body<DT, NB, SRC, SINGLE, PRO, EPI, PRE>(w, src, dst, g, fz, blockIdx.x, gridDim.x);
+}
+
+// Two weight tensors of different K-quant formats over the same activation row in one launch (attention_wq|wk and
+// attention_wv of a Q4_K_M file): workgroups [0, blocks_a) take tensor A, the rest tensor B.
+template <int DTA, int DTB, bool SINGLE, int PRO>
+__global__ __launch_bounds__(1024) void qmv2_kernel(const uint8_t *__restrict__ wa, const uint8_t *__restrict__ wb, ActSrc src, void *__restrict__ dsta,
+                                                    void *__restrict__ dstb, QmvGeom ga, QmvGeom gb, Fuse fz, int blocks_a) {
+    if ((int)blockIdx.x < blocks_a)
+        qmv_body<DTA, 1, CQ_F32, SINGLE, PRO, EPI_NONE, false>(wa, src, dsta, ga, fz, blockIdx.x, blocks_a);
+    else
+        qmv_body<DTB, 1, CQ_F32, SINGLE, PRO, EPI_NONE, false>(wb, src, dstb, gb, fz, blockIdx.x - blocks_a, gridDim.x - blocks_a);
+}
+
+// Geometry of one launch.  waves == 0: as many waves per workgroup (a power of two, at most 16) as still leave every
+// wave a row when 256 workgroups are launched; otherwise the given wave count is used.
+template <int DT, int NB>
+int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int64_t stride_dst, int dst_dtype, int extra_lds, size_t &lds_bytes) {
+    if (waves == 0) {
+        waves = 16;
+        while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
+    }
+    groups = n >= 256 * (int64_t)waves ? 256 : (n + waves - 1) / waves;
     int64_t rows_per_wg = (n + groups - 1) / groups;
     groups = (n + rows_per_wg - 1) / rows_per_wg;
     const ActLayout L = cq_act_layout(DT, k, NB);
-    size_t lds_bytes = (size_t)L.total + (EPI == EPI_RESID ? 64 : 0);
-    QmvGeom g;
+    lds_bytes = (size_t)L.total + extra_lds;
     g.lds_red_off = (int)L.total;
     g.k = (int)k; g.n = (int)n; g.rows_per_wg = (int)rows_per_wg;
     g.units = (int)(k / Fmt<DT>::UE); g.steps = (g.units + 63) >> 6;
@@ -426,6 +464,18 @@ int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64
     if (rb > 0x3fffffff) return CQ_ERR_RANGE;
     g.row_bytes = (int)rb;
     g.dst_dtype = dst_dtype; g.stride_dst = stride_dst;
+    return CQ_OK;
+}
+
+template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
+int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s,
+               const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0}) {
+    QmvGeom g;
+    int64_t groups;
+    int waves = 0;
+    size_t lds_bytes;
+    int rc = make_geom<DT, NB>(g, groups, waves, k, n, stride_dst, dst_dtype, EPI == EPI_RESID ? 64 : 0, lds_bytes);
+    if (rc) return rc;
     auto kern = qmv_kernel<DT, NB, SRC, SINGLE, PRO, EPI, PRE>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -551,7 +601,7 @@ int cq_matvec_norm_launch(int w_dtype, const void *w, const float *x, const floa
                           int64_t k, int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0};
     return launch_fused_dt<PRO_NORM, EPI_NONE>(w_dtype, w, src, dst, k, n, s, fz);
 }
 
@@ -560,7 +610,7 @@ int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const 
                               int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{up, nullptr, 0.0f, residual, partials_out, 0, 0};
+    Fuse fz{up, nullptr, 0.0f, residual, partials_out, 0, 0, 0};
     if (up) return launch_fused_dt<PRO_SILU, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
     return launch_fused_dt<PRO_NONE, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
 }
@@ -583,13 +633,96 @@ int cq_matvec_residual_attn_launch(int w_dtype, const void *w, const float *attn
     if (splits < 1 || splits > MAXS || head_dim < 4 || (head_dim & (head_dim - 1)) || k % head_dim) return CQ_ERR_RANGE;
     int sh = 0;
     while ((1 << sh) < head_dim) sh++;
-    Fuse fz{attn_partials, nullptr, 0.0f, residual, partials_out, (int)splits, sh};
+    Fuse fz{attn_partials, nullptr, 0.0f, residual, partials_out, (int)splits, sh, 0};
     switch (w_dtype) {
         case CQ_Q4_0: return launch_merge1<CQ_Q4_0>(w, nullptr, k, n, s, fz);
         case CQ_Q8_0: return launch_merge1<CQ_Q8_0>(w, nullptr, k, n, s, fz);
         case CQ_Q4K: return launch_merge1<CQ_Q4K>(w, nullptr, k, n, s, fz);
         case CQ_Q5K: return launch_merge1<CQ_Q5K>(w, nullptr, k, n, s, fz);
         case CQ_Q6K: return launch_merge1<CQ_Q6K>(w, nullptr, k, n, s, fz);
+    }
+    return CQ_ERR_DTYPE;
+}
+
+namespace {
+template <int DT>
+int launch_swiglu1(const void *w1, int64_t pair_off, const ActSrc &src, float *dst, int64_t k, int64_t ffn, hipStream_t s, Fuse fz) {
+    if (k / Fmt<DT>::UE > 64) return CQ_ERR_RANGE;
+    fz.pair_off = pair_off;
+    return launch_cfg<DT, 1, CQ_F32, true, PRO_NORM, EPI_SWIGLU>(w1, src, dst, CQ_F32, k, ffn, ffn, s, fz);
+}
+
+template <int DTA, int DTB>
+int launch_pair(const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const ActSrc &src, int64_t k, hipStream_t s,
+                const Fuse &fz) {
+    QmvGeom ga, gb;
+    int64_t groups_a, groups_b;
+    size_t lds_a, lds_b;
+    // one block size for both segments: that of the larger tensor
+    int waves = 0;
+    int rc = na >= nb ? make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, 0, lds_a) : make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, 0, lds_b);
+    if (rc) return rc;
+    if ((rc = make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, 0, lds_a))) return rc;
+    if ((rc = make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, 0, lds_b))) return rc;
+    const size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
+    const bool single = k / 64 <= 64;                     // every K-quant unit is 64 elements
+    if (lds_bytes > 48 * 1024) {
+        const void *kp = single ? (const void *)qmv2_kernel<DTA, DTB, true, PRO_NORM> : (const void *)qmv2_kernel<DTA, DTB, false, PRO_NORM>;
+        hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    dim3 grid((unsigned)(groups_a + groups_b)), block(64 * waves);
+    if (single)
+        hipLaunchKernelGGL((qmv2_kernel<DTA, DTB, true, PRO_NORM>), grid, block, lds_bytes, s, (const uint8_t *)wa, (const uint8_t *)wb, src,
+                           (void *)dsta, (void *)dstb, ga, gb, fz, (int)groups_a);
+    else
+        hipLaunchKernelGGL((qmv2_kernel<DTA, DTB, false, PRO_NORM>), grid, block, lds_bytes, s, (const uint8_t *)wa, (const uint8_t *)wb, src,
+                           (void *)dsta, (void *)dstb, ga, gb, fz, (int)groups_a);
+    return (int)hipGetLastError();
+}
+
+template <int DTA>
+int launch_pair_b(int dtb, const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const ActSrc &src, int64_t k,
+                  hipStream_t s, const Fuse &fz) {
+    switch (dtb) {
+        case CQ_Q4K: return launch_pair<DTA, CQ_Q4K>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q5K: return launch_pair<DTA, CQ_Q5K>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q6K: return launch_pair<DTA, CQ_Q6K>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+    }
+    return CQ_ERR_DTYPE;
+}
+}  // namespace
+
+// h[ffn] = silu(W1 . xn) * (W3 . xn), xn = quantize(rms_norm(x) * norm_weight); W3 row r lies pair_off bytes behind W1 row r.
+// CQ_ERR_RANGE when a row is longer than one wave step.
+int cq_matvec_norm_swiglu_launch(int w_dtype, const void *w1, const void *w3, const float *x, const float *partials, const float *norm_weight,
+                                 float eps, float *dst, int64_t k, int64_t ffn, hipStream_t s) {
+    if (ffn == 0) return CQ_OK;
+    ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0};
+    const int64_t off = (const uint8_t *)w3 - (const uint8_t *)w1;
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_swiglu1<CQ_Q4_0>(w1, off, src, dst, k, ffn, s, fz);
+        case CQ_Q8_0: return launch_swiglu1<CQ_Q8_0>(w1, off, src, dst, k, ffn, s, fz);
+        case CQ_Q4K: return launch_swiglu1<CQ_Q4K>(w1, off, src, dst, k, ffn, s, fz);
+        case CQ_Q5K: return launch_swiglu1<CQ_Q5K>(w1, off, src, dst, k, ffn, s, fz);
+        case CQ_Q6K: return launch_swiglu1<CQ_Q6K>(w1, off, src, dst, k, ffn, s, fz);
+    }
+    return CQ_ERR_DTYPE;
+}
+
+// dst_a[na] = Wa . xn and dst_b[nb] = Wb . xn in one launch, xn = quantize(rms_norm(x) * norm_weight); both K-quants.
+int cq_matvec_norm_pair_launch(int dta, const void *wa, int64_t na, float *dsta, int dtb, const void *wb, int64_t nb, float *dstb, const float *x,
+                               const float *partials, const float *norm_weight, float eps, int64_t k, hipStream_t s) {
+    if (!cq_is_kquant(dta) || !cq_is_kquant(dtb) || dta == CQ_Q8K || dtb == CQ_Q8K) return CQ_ERR_DTYPE;
+    if (na == 0 || nb == 0) return CQ_ERR_SHAPE;
+    if (cq_act_layout(dta, k, 1).total > LDS_BUDGET) return CQ_ERR_RANGE;
+    ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0};
+    switch (dta) {
+        case CQ_Q4K: return launch_pair_b<CQ_Q4K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q5K: return launch_pair_b<CQ_Q5K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q6K: return launch_pair_b<CQ_Q6K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
     }
     return CQ_ERR_DTYPE;
 }

@@ -531,6 +531,59 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
     }
 }
 
+// Two-stage variant for long logit rows: up to 128 workgroups each leave (value, index) of their contiguous chunk,
+// one small workgroup finishes.  Ties still resolve to the lowest index: chunks are contiguous and ordered.
+constexpr int ARGMAX_PARTS = 128;
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ logits, int n, int chunk, float *__restrict__ pv,
+                                                             int *__restrict__ pi) {
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    const int lo = blockIdx.x * chunk, hi = min(n, lo + chunk);
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+        const float v = logits[i];
+        if (v > best || idx == 0x7fffffff) { best = v; idx = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(idx, o, 64);
+        if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) { best = ov; idx = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = best; bi[threadIdx.x >> 6] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++)
+            if (bi[w] != 0x7fffffff && (idx == 0x7fffffff || bv[w] > best || (bv[w] == best && bi[w] < idx))) { best = bv[w]; idx = bi[w]; }
+        pv[blockIdx.x] = best;
+        pi[blockIdx.x] = idx;
+    }
+}
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int parts,
+                                                          int32_t *__restrict__ token_out, int32_t *__restrict__ history,
+                                                          int32_t *__restrict__ counter, int32_t *__restrict__ pos_dev) {
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < parts; i += 64) {
+        const float v = pv[i];
+        const int j = pi[i];
+        if (j != 0x7fffffff && (idx == 0x7fffffff || v > best || (v == best && j < idx))) { best = v; idx = j; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(idx, o, 64);
+        if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) { best = ov; idx = oi; }
+    }
+    if (threadIdx.x == 0) {
+        token_out[0] = idx;
+        if (history && counter) history[counter[0]] = idx;
+        if (counter) counter[0] += 1;
+        if (pos_dev) pos_dev[0] += 1;
+    }
+}
+
 inline bool misaligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
 template <int HD>
@@ -711,10 +764,21 @@ int cq_nn_silu_mul(const float *gate_dev, const float *up_dev, float *out_dev, i
 }
 
 int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
-                 void *stream) {
+                 void *workspace_dev, void *stream) {
     if (n <= 0) return CQ_ERR_SHAPE;
     if (!logits_dev || !token_out_dev) return CQ_ERR_NULL;
     if (n > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (workspace_dev && misaligned(workspace_dev, 4)) return CQ_ERR_ALIGN;
+    if (workspace_dev && n >= 8192) {
+        const int chunk = (int)((n + ARGMAX_PARTS - 1) / ARGMAX_PARTS);
+        const int parts = (int)((n + chunk - 1) / chunk);
+        float *pv = (float *)workspace_dev;
+        int *pi = (int *)workspace_dev + ARGMAX_PARTS;
+        hipLaunchKernelGGL(argmax_partial_kernel, dim3(parts), dim3(256), 0, (hipStream_t)stream, logits_dev, (int)n, chunk, pv, pi);
+        hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (const float *)pv, (const int *)pi, parts,
+                           token_out_dev, history_dev, counter_dev, pos_dev);
+        return (int)hipGetLastError();
+    }
     hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits_dev, (int)n, token_out_dev, history_dev, counter_dev,
                        pos_dev);
     return (int)hipGetLastError();

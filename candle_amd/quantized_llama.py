@@ -144,6 +144,7 @@ class ModelWeights:
         self.pos_dev = torch.zeros(1, dtype=torch.int32, device=self.device)
         self.counter_dev = torch.zeros(1, dtype=torch.int32, device=self.device)
         self.history_dev = torch.zeros(cfg.ctx, dtype=torch.int32, device=self.device)
+        self.argmax_ws = torch.zeros(1024, dtype=torch.uint8, device=self.device)      # CQ_NN_ARGMAX_WORKSPACE
         return plan
 
     def _alloc_activations(self, max_rows: int):
@@ -314,12 +315,20 @@ class ModelWeights:
         for lw in self.layers:
             w = lw.w
             wq, wk, wv = w["attention_wq"], w["attention_wk"], w["attention_wv"]
+            kq = (GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
             if wq.dtype == wk.dtype and wk.ptr == wq.ptr + wq.nbytes:
-                norm_mm(wq, qd + kvd, lw.attention_norm, qk.data_ptr())
+                if wq.dtype in kq and wv.dtype in kq:
+                    # q|k and v in one launch even though their formats differ
+                    ck("cq_nn_qmatmul_norm_pair", L.cq_nn_qmatmul_norm_pair(int(wq.dtype), wq.ptr, qd + kvd, qk.data_ptr(), int(wv.dtype), wv.ptr,
+                                                                            kvd, v.data_ptr(), x.data_ptr(), part.data_ptr(),
+                                                                            lw.attention_norm.data_ptr(), cfg.rms_eps, cfg.hidden, sp))
+                else:
+                    norm_mm(wq, qd + kvd, lw.attention_norm, qk.data_ptr())
+                    norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
             else:
                 norm_mm(wq, qd, lw.attention_norm, qk.data_ptr())
                 norm_mm(wk, kvd, lw.attention_norm, qk.data_ptr() + 4 * qd)
-            norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
+                norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
             q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
             # rope, cache append, attention and the merge of the key splits in one kernel          :217-261
             wo = w["attention_wo"]
@@ -336,13 +345,18 @@ class ModelWeights:
                                                                                 x.data_ptr(), part.data_ptr(), wo.k, cfg.hidden, sp))
             else:
                 resid_mm(wo, att.data_ptr(), None)
-            w1, w3 = w["feed_forward_w1"], w["feed_forward_w3"]
-            if w1.dtype == w3.dtype and w3.ptr == w1.ptr + w1.nbytes:
-                norm_mm(w1, 2 * cfg.ffn, lw.ffn_norm, gu.data_ptr())
+            w1, w3, w2 = w["feed_forward_w1"], w["feed_forward_w3"], w["feed_forward_w2"]
+            one_step = cfg.hidden <= (4096 if w1.dtype in kq else 2048)
+            if w1.dtype == w3.dtype and one_step:
+                # h = silu(w1 xn) * (w3 xn) straight out of the paired-row matvec                    :56-63
+                ck("cq_nn_qmatmul_norm_swiglu", L.cq_nn_qmatmul_norm_swiglu(int(w1.dtype), w1.ptr, w3.ptr, x.data_ptr(), part.data_ptr(),
+                                                                            lw.ffn_norm.data_ptr(), cfg.rms_eps, self.h.data_ptr(), cfg.hidden,
+                                                                            cfg.ffn, sp))
+                resid_mm(w2, self.h.data_ptr(), None)
             else:
                 norm_mm(w1, cfg.ffn, lw.ffn_norm, gu.data_ptr())
                 norm_mm(w3, cfg.ffn, lw.ffn_norm, gu.data_ptr() + 4 * cfg.ffn)
-            resid_mm(w["feed_forward_w2"], gu.data_ptr(), gu.data_ptr() + 4 * cfg.ffn)
+                resid_mm(w2, gu.data_ptr(), gu.data_ptr() + 4 * cfg.ffn)
         norm_mm(self.output, cfg.vocab, self.norm, self.logits.data_ptr())
 
     def forward(self, x: torch.Tensor, index_pos: int) -> torch.Tensor:
@@ -364,7 +378,8 @@ class ModelWeights:
         """One greedy step driven entirely from device state: token_dev at position pos_dev -> next token_dev, pos_dev + 1."""
         self._enqueue(self.token_dev.data_ptr(), 1, 0, self.pos_dev.data_ptr(), max_kv_len, sp)
         _lib.check("cq_nn_argmax", self.L.cq_nn_argmax(self.logits.data_ptr(), self.cfg.vocab, self.token_dev.data_ptr(),
-                                                       self.history_dev.data_ptr(), self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), sp))
+                                                       self.history_dev.data_ptr(), self.counter_dev.data_ptr(), self.pos_dev.data_ptr(),
+                                                       self.argmax_ws.data_ptr(), sp))
 
     def generate_greedy(self, prompt: Sequence[int], n_new: int, use_graph: bool = True) -> dict:
         """The loop of candle-examples/examples/quantized/main.rs:616-690 with temperature <= 0 (Sampling::ArgMax):
@@ -382,7 +397,8 @@ class ModelWeights:
         self.counter_dev.zero_()
         self.pos_dev.fill_(len(prompt) - 1)       # argmax advances it to the position of the token it emits
         _lib.check("cq_nn_argmax", self.L.cq_nn_argmax(logits.data_ptr(), cfg.vocab, self.token_dev.data_ptr(), self.history_dev.data_ptr(),
-                                                       self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), stream.cuda_stream))
+                                                       self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), self.argmax_ws.data_ptr(),
+                                                       stream.cuda_stream))
         torch.cuda.synchronize(dev)
         t1 = time.perf_counter()
         prompt_seconds = t1 - t0

@@ -91,6 +91,16 @@ int cq_nn_qmatmul_norm(int w_dtype, const void *w_dev, const float *x_dev, const
                        float eps, float *dst_dev, int64_t k, int64_t n, void *stream);
 int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
                            float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream);
+/* cq_nn_qmatmul_norm for feed_forward_w1 and feed_forward_w3 at once with the activation of Mlp::forward
+ * (quantized_llama.rs:56-63) as epilogue: dst[ffn] = silu(W1 . xn) * (W3 . xn).  Both tensors [ffn, k] in the same
+ * format.  CQ_ERR_RANGE when k is longer than one wave step per row (k > 4096 for K-quants, > 2048 for Q4_0 / Q8_0). */
+int cq_nn_qmatmul_norm_swiglu(int w_dtype, const void *w1_dev, const void *w3_dev, const float *x_dev, const float *sumsq_partials_dev,
+                              const float *norm_weight_dev, float eps, float *dst_dev, int64_t k, int64_t ffn, void *stream);
+/* cq_nn_qmatmul_norm for two weight tensors of (possibly different) K-quant formats over the same row in one launch,
+ * e.g. attention_wq|attention_wk (Q4_K) and attention_wv (Q6_K) of a Q4_K_M file.  CQ_ERR_DTYPE for other formats. */
+int cq_nn_qmatmul_norm_pair(int w_dtype_a, const void *w_a_dev, int64_t n_a, float *dst_a_dev, int w_dtype_b, const void *w_b_dev, int64_t n_b,
+                            float *dst_b_dev, const float *x_dev, const float *sumsq_partials_dev, const float *norm_weight_dev, float eps,
+                            int64_t k, void *stream);
 /* cq_nn_qmatmul_residual whose input row is the attention output still in the per-split partials of
  * cq_nn_attention_decode (out_dev == NULL there): the merge of the splits is the matvec's prologue.
  * CQ_ERR_RANGE (use the merge kernel + cq_nn_qmatmul_residual instead) when k = n_head*head_dim is longer than one
@@ -100,9 +110,11 @@ int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *att
 
 /* Greedy sampling (LogitsProcessor with Sampling::ArgMax, candle-examples/examples/quantized/main.rs:603-604):
  * token_out[0] = index of the largest logit (lowest index on ties).  Optional bookkeeping for graph replay:
- * history_dev[*counter_dev] = token; *counter_dev += 1; *pos_dev += 1. */
+ * history_dev[*counter_dev] = token; *counter_dev += 1; *pos_dev += 1.
+ * workspace_dev (optional, CQ_NN_ARGMAX_WORKSPACE bytes): lets long rows be scanned by many workgroups. */
+#define CQ_NN_ARGMAX_WORKSPACE 1024
 int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
-                 void *stream);
+                 void *workspace_dev, void *stream);
 
 #ifdef __cplusplus
 }

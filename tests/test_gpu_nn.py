@@ -224,11 +224,24 @@ def test_argmax_first_of_ties_and_bookkeeping():
     hist = torch.full((8,), -1, dtype=torch.int32, device="cuda")
     cnt = torch.tensor([2], dtype=torch.int32, device="cuda")
     pos = torch.tensor([41], dtype=torch.int32, device="cuda")
-    ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), hist.data_ptr(), cnt.data_ptr(), pos.data_ptr(), None))
+    ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), hist.data_ptr(), cnt.data_ptr(), pos.data_ptr(), None, None))
     assert tok.item() == 777 and hist.cpu().tolist() == [-1, -1, 777, -1, -1, -1, -1, -1] and cnt.item() == 3 and pos.item() == 42
     logits[5] = 60.0
-    ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), None, None, None, None))
+    ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), None, None, None, None, None))
     assert tok.item() == 5 == int(np.argmax(logits))
+    # the many-workgroup variant (workspace given): same answers, same tie rule, same bookkeeping
+    ws = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    logits[5] = 0.0
+    ok(L().cq_nn_argmax(dev(logits).data_ptr(), n, tok.data_ptr(), hist.data_ptr(), cnt.data_ptr(), pos.data_ptr(), ws.data_ptr(), None))
+    assert tok.item() == 777 and hist.cpu().tolist()[3] == 777 and cnt.item() == 4 and pos.item() == 43
+    for trial, where in enumerate([0, n - 1, 1001, 64127, 64128]):
+        lg = normal(50 + trial, (n,), 1.0)
+        lg[where] = 99.0
+        ok(L().cq_nn_argmax(dev(lg).data_ptr(), n, tok.data_ptr(), None, None, None, ws.data_ptr(), None))
+        assert tok.item() == where
+    lg = np.full((n,), -np.inf, dtype=np.float32)      # all -inf: index 0, like numpy
+    ok(L().cq_nn_argmax(dev(lg).data_ptr(), n, tok.data_ptr(), None, None, None, ws.data_ptr(), None))
+    assert tok.item() == 0
 
 
 FUSE_DTYPES = [2, 8, 12, 13, 14]      # Q4_0, Q8_0, Q4_K, Q5_K, Q6_K
@@ -289,6 +302,63 @@ def test_fused_silu_mul_matvec_residual(dtype):
     # expf on the device differs from the host's by an ulp here and there; the quantizer can turn that into a
     # one-step difference of a single int8 value
     assert rel_l2(res.cpu().numpy(), want) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", FUSE_DTYPES)
+@pytest.mark.parametrize("ffn,k", [(14336, 4096), (300, 512), (33, 2048)])
+def test_fused_norm_swiglu_matvec(dtype, ffn, k):
+    import oracle
+    lib = L()
+    x = normal(60, (1, k), 1.0)
+    nw = (1.0 + 0.1 * normal(61, (k,), 1.0)).astype(np.float32)
+    w1 = oracle.from_float(dtype, normal(62, (ffn, k), 0.03).reshape(-1))
+    w3 = oracle.from_float(dtype, normal(63, (ffn, k), 0.03).reshape(-1))
+    part = np.zeros(256, dtype=np.float32)
+    part[:5] = (x.astype(np.float64) ** 2).sum() / 5.0
+    h = torch.empty((1, ffn), device="cuda")
+    both = dev(np.concatenate([w1, w3]))                       # adjacent, as the decoder stores them
+    if dtype in (2, 8) and k > 2048:                           # longer than one wave step for 32-element blocks
+        assert lib.cq_nn_qmatmul_norm_swiglu(dtype, both.data_ptr(), both.data_ptr() + w1.size, dev(x).data_ptr(), dev(part).data_ptr(),
+                                             dev(nw).data_ptr(), 1e-5, h.data_ptr(), k, ffn, None) == -6
+        return
+    ok(lib.cq_nn_qmatmul_norm_swiglu(dtype, both.data_ptr(), both.data_ptr() + w1.size, dev(x).data_ptr(), dev(part).data_ptr(),
+                                     dev(nw).data_ptr(), 1e-5, h.data_ptr(), k, ffn, None))
+    xn = lo.rms_norm(x, nw, 1e-5)
+    want = lo.silu(oracle.matmul_fast(dtype, xn, w1, ffn, 8)) * oracle.matmul_fast(dtype, xn, w3, ffn, 8)
+    assert rel_l2(h.cpu().numpy(), want) <= 1e-4
+    # w3 anywhere else in memory, in front of w1 included
+    sep3, sep1 = dev(w3), dev(w1)
+    h2 = torch.empty((1, ffn), device="cuda")
+    ok(lib.cq_nn_qmatmul_norm_swiglu(dtype, sep1.data_ptr(), sep3.data_ptr(), dev(x).data_ptr(), dev(part).data_ptr(), dev(nw).data_ptr(), 1e-5,
+                                     h2.data_ptr(), k, ffn, None))
+    assert np.array_equal(h2.cpu().numpy(), h.cpu().numpy())
+    assert lib.cq_nn_qmatmul_norm_swiglu(dtype, sep1.data_ptr(), sep3.data_ptr(), 16, 16, 16, 1e-5, 16, 8192, ffn, None) == -6
+
+
+@pytest.mark.parametrize("dta,dtb", [(12, 14), (14, 12), (13, 13), (12, 12)])
+@pytest.mark.parametrize("na,nb,k", [(5120, 1024, 4096), (96, 4000, 1024), (64, 64, 14336)])
+def test_fused_norm_pair_matvec(dta, dtb, na, nb, k):
+    import oracle
+    lib = L()
+    x = normal(70, (1, k), 1.0)
+    nw = (1.0 + 0.1 * normal(71, (k,), 1.0)).astype(np.float32)
+    wa = oracle.from_float(dta, normal(72, (na, k), 0.03).reshape(-1))
+    wb = oracle.from_float(dtb, normal(73, (nb, k), 0.03).reshape(-1))
+    part = np.zeros(256, dtype=np.float32)
+    part[0] = (x.astype(np.float64) ** 2).sum()
+    ya, yb = torch.empty((1, na), device="cuda"), torch.empty((1, nb), device="cuda")
+    ok(lib.cq_nn_qmatmul_norm_pair(dta, dev(wa).data_ptr(), na, ya.data_ptr(), dtb, dev(wb).data_ptr(), nb, yb.data_ptr(), dev(x).data_ptr(),
+                                   dev(part).data_ptr(), dev(nw).data_ptr(), 1e-5, k, None))
+    # the single-tensor entry point gives the same bits
+    za, zb = torch.empty((1, na), device="cuda"), torch.empty((1, nb), device="cuda")
+    ok(lib.cq_nn_qmatmul_norm(dta, dev(wa).data_ptr(), dev(x).data_ptr(), dev(part).data_ptr(), dev(nw).data_ptr(), 1e-5, za.data_ptr(), k, na, None))
+    ok(lib.cq_nn_qmatmul_norm(dtb, dev(wb).data_ptr(), dev(x).data_ptr(), dev(part).data_ptr(), dev(nw).data_ptr(), 1e-5, zb.data_ptr(), k, nb, None))
+    assert np.array_equal(ya.cpu().numpy(), za.cpu().numpy()) and np.array_equal(yb.cpu().numpy(), zb.cpu().numpy())
+    xn = lo.rms_norm(x, nw, 1e-5)
+    assert rel_l2(ya.cpu().numpy(), oracle.matmul_fast(dta, xn, wa, na, 8)) <= 1e-3
+    assert rel_l2(yb.cpu().numpy(), oracle.matmul_fast(dtb, xn, wb, nb, 8)) <= 1e-3
+    assert lib.cq_nn_qmatmul_norm_pair(8, dev(wa).data_ptr(), na, ya.data_ptr(), dtb, dev(wb).data_ptr(), nb, yb.data_ptr(), dev(x).data_ptr(),
+                                       dev(part).data_ptr(), dev(nw).data_ptr(), 1e-5, k, None) == -1
 
 
 def test_argument_validation():
