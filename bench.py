@@ -154,7 +154,7 @@ def decode8b(args):
     mean_pos = args.prompt + (n_new + 1) / 2.0
     kv_bytes = 2 * cfg.n_layer * cfg.n_kv_head * cfg.head_dim * 4 * mean_pos
     roof_tok_s = HBM_PEAK_GBPS * 1e9 / wbytes
-    print(json.dumps({
+    out = {
         "metric": "8B-shape Q4_K_M decode tok/s (batch 1, greedy)", "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1,
         "steps": steps, "warmup": 8, "ms_per_step": round(1e3 / tok_s, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "i8 dot products, f32 glue", "data": "synthetic",
@@ -170,7 +170,10 @@ def decode8b(args):
                      "frac": round((wbytes + kv_bytes) * tok_s / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
                      "roofline_tok_s_weights_only": round(roof_tok_s, 1), "frac_of_roofline_tok_s": round(tok_s / roof_tok_s, 4)},
         "init_seconds": round(t_init, 1),
-    }))
+    }
+    del model
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -194,7 +197,8 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every configuration of the metric is single-GPU); use --gpus 1")
     if args.workload == "decode8b":
-        return decode8b(args)
+        print(json.dumps(decode8b(args)))
+        return
     if args.steps is None:
         args.steps = 4000 if args.workload == "decode" else 50
     if args.warmup is None:
@@ -340,6 +344,15 @@ def main():
                      "avg_kernel_us": round(kern_us, 3), "algorithmic_bytes_per_launch": alg_bytes},
         "extra": extra,
     }
+
+    if not args.no_extra:
+        # the second half of the metric: the 8B-shape decoder (same protocol as --workload decode8b)
+        d8 = argparse.Namespace(layers=32, prompt=512, steps=256)
+        r = decode8b(d8)
+        out["decode_8b"] = {"tok_s": r["value"], "ms_per_token": r["ms_per_step"], "prompt_tok_s": r["prompt_tok_s"],
+                            "frac_of_roofline_tok_s": r["roofline"]["frac_of_roofline_tok_s"],
+                            "roofline_tok_s": r["roofline"]["roofline_tok_s_weights_only"],
+                            "weight_bytes_per_token": r["weight_bytes_per_token"], "workload": r["config"]["workload"]}
 
     if not args.no_cpu_baseline:
         import oracle

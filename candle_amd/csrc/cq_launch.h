@@ -48,3 +48,43 @@ struct MoeArgs {
 };
 int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k);
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s);
+
+// One (expert, activation row, output row, scale) pair of either MoE entry point.
+struct PairSource {
+    int mode;
+    const uint32_t *ids_u32;
+    const int32_t *sorted_token_ids, *expert_ids;
+    const float *topk_weights;
+    int topk, input_dim1;
+    int n_pairs, num_experts, x_rows;
+};
+
+__device__ __forceinline__ bool pair_decode(const PairSource &ps, int p, int &e, int &in_row, int &out_row, float &scale) {
+    if (ps.mode == MOE_INDEXED) {
+        uint32_t id = ps.ids_u32[p];
+        e = (int)id;
+        in_row = ps.input_dim1 == 1 ? p / ps.topk : p;
+        out_row = p;
+        scale = 1.0f;
+        return id < (uint32_t)ps.num_experts;
+    }
+    e = ps.expert_ids[p];
+    int tok = ps.sorted_token_ids[p];
+    out_row = tok;
+    if (ps.topk_weights) {
+        in_row = tok;
+        // a token id outside the table would read past topk_weights; such pairs are dropped below
+        scale = (tok >= 0 && tok < ps.n_pairs) ? ps.topk_weights[tok] : 0.0f;
+    } else {
+        in_row = tok / ps.topk;
+        scale = 1.0f;
+    }
+    return e >= 0 && e < ps.num_experts && tok >= 0 && tok < ps.n_pairs && in_row < ps.x_rows;
+}
+
+// One workgroup: histogram of experts, exclusive scan, scatter of the pair descriptors.
+
+// Pairs up to which cq_moe_launch runs every pair as its own fused matvec instead of grouping by expert.
+#define CQ_MOE_DIRECT_MAX_PAIRS 256
+// CQ_ERR_RANGE when the shape is not served by the fused kernel (the caller then takes the grouped path).
+int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s);

@@ -40,11 +40,12 @@ struct ActSrc {
 //             { acc[hd], m, l, 0, 0 } the single-token attention kernel leaves (rows of one wave step only)
 //   EPI_SWIGLU a logical row r is the pair (W[r], W[r] + pair_off bytes) = (feed_forward_w1, feed_forward_w3):
 //             dst[r] = silu(W1[r] . x) * (W3[r] . x)   (rows of one wave step only)
+//   EPI_SCALE the result is multiplied by a per-launch-block scalar (Fuse::eps) before it is stored (MoE top-k weight)
 //   EPI_RESID the result is added to a residual row in place of being stored, and the workgroup leaves
 //             its partial sum of residual^2 for the next PRO_NORM consumer
 enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2, PRO_MERGE = 3 };
 constexpr int MAXS = 16;     // attention splits a PRO_MERGE prologue can merge
-enum { EPI_NONE = 0, EPI_RESID = 1, EPI_SWIGLU = 2 };
+enum { EPI_NONE = 0, EPI_RESID = 1, EPI_SWIGLU = 2, EPI_SCALE = 3 };
 constexpr int NPART = 256;   // == CQ_NN_PARTIALS
 struct Fuse {
     const float *aux;        // PRO_NORM: norm weight [k];  PRO_SILU: up [k];  PRO_MERGE: partials [k/hd][splits][hd + 4]
@@ -302,7 +303,7 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
                         ssq += sres * sres;
                     }
                 } else if (lane == 63) {
-                    store_out(dst, dst_dtype, (int64_t)b * stride_dst + r, v);
+                    store_out(dst, dst_dtype, (int64_t)b * stride_dst + r, EPI == EPI_SCALE ? v * fz.eps : v);
                 }
             }
         };
@@ -361,7 +362,7 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
                         ssq += sres * sres;
                     }
                 } else if (lane == 63) {
-                    store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, r);
+                    store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, EPI == EPI_SCALE ? r * fz.eps : r);
                 }
                 acc[b] = 0.0f;
             }
@@ -444,12 +445,14 @@ __global__ __launch_bounds__(1024) void qmv2_kernel(const uint8_t *__restrict__ 
 // Geometry of one launch.  waves == 0: as many waves per workgroup (a power of two, at most 16) as still leave every
 // wave a row when 256 workgroups are launched; otherwise the given wave count is used.
 template <int DT, int NB>
-int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int64_t stride_dst, int dst_dtype, int extra_lds, size_t &lds_bytes) {
+int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int64_t stride_dst, int dst_dtype, int extra_lds, size_t &lds_bytes,
+              int64_t max_groups = 256) {
     if (waves == 0) {
         waves = 16;
         while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
     }
-    groups = n >= 256 * (int64_t)waves ? 256 : (n + waves - 1) / waves;
+    groups = (n + waves - 1) / waves;
+    if (groups > max_groups) groups = max_groups;
     int64_t rows_per_wg = (n + groups - 1) / groups;
     groups = (n + rows_per_wg - 1) / rows_per_wg;
     const ActLayout L = cq_act_layout(DT, k, NB);
@@ -723,6 +726,69 @@ int cq_matvec_norm_pair_launch(int dta, const void *wa, int64_t na, float *dsta,
         case CQ_Q4K: return launch_pair_b<CQ_Q4K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
         case CQ_Q5K: return launch_pair_b<CQ_Q5K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
         case CQ_Q6K: return launch_pair_b<CQ_Q6K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+    }
+    return CQ_ERR_DTYPE;
+}
+
+// ---- MoE with few pairs: block (tile, pair) is one fused matvec over the pair's expert ----
+namespace {
+template <int DT, bool SINGLE>
+__global__ __launch_bounds__(1024) void moe_pair_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out, QmvGeom g,
+                                                        PairSource ps, int64_t expert_bytes) {
+    const int p = blockIdx.y;
+    int e, in_row, out_row;
+    float scale;
+    if (!pair_decode(ps, p, e, in_row, out_row, scale)) {       // uniform over the workgroup
+        if (ps.mode == MOE_INDEXED) {                           // an out-of-range id: that output row is zero
+            const int r0 = blockIdx.x * g.rows_per_wg, r1 = min(g.n, r0 + g.rows_per_wg);
+            for (int r = r0 + (int)threadIdx.x; r < r1; r += (int)blockDim.x) out[(int64_t)p * g.n + r] = 0.0f;
+        }
+        return;
+    }
+    ActSrc src{x + (int64_t)in_row * g.k, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{nullptr, nullptr, scale, nullptr, nullptr, 0, 0, 0};
+    qmv_body<DT, 1, CQ_F32, SINGLE, PRO_NONE, EPI_SCALE, false>(w + (int64_t)e * expert_bytes, src, out + (int64_t)out_row * g.n, g, fz,
+                                                                blockIdx.x, gridDim.x);
+}
+
+template <int DT>
+int launch_moe_pairs(const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s) {
+    if (cq_act_layout(DT, k, 1).total > LDS_BUDGET) return CQ_ERR_RANGE;
+    QmvGeom g;
+    int64_t groups;
+    size_t lds_bytes;
+    // wide workgroups once the pairs together hold enough rows: the activation row is quantized once per workgroup
+    int waves = (int64_t)ps.n_pairs * n >= 256 * 16 ? 16 : 0;
+    // about a thousand workgroups in total: with many pairs each workgroup takes more rows of its expert, so that
+    // the activation prologue is paid once per many rows
+    const int64_t per_pair = (1024 + ps.n_pairs - 1) / ps.n_pairs;
+    int rc = make_geom<DT, 1>(g, groups, waves, k, n, n, CQ_F32, 0, lds_bytes, per_pair < 256 ? per_pair : 256);
+    if (rc) return rc;
+    if (ps.n_pairs > 65535) return CQ_ERR_RANGE;
+    const int64_t expert_bytes = n * (int64_t)g.row_bytes;
+    const bool single = g.units <= 64;
+    const void *kp = single ? (const void *)moe_pair_kernel<DT, true> : (const void *)moe_pair_kernel<DT, false>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    dim3 grid((unsigned)groups, (unsigned)ps.n_pairs), block(64 * waves);
+    if (single)
+        hipLaunchKernelGGL((moe_pair_kernel<DT, true>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes);
+    else
+        hipLaunchKernelGGL((moe_pair_kernel<DT, false>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes);
+    return (int)hipGetLastError();
+}
+}  // namespace
+
+int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s) {
+    if (ps.n_pairs == 0 || n == 0) return CQ_OK;
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_moe_pairs<CQ_Q4_0>(w, x, out, ps, k, n, s);
+        case CQ_Q8_0: return launch_moe_pairs<CQ_Q8_0>(w, x, out, ps, k, n, s);
+        case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w, x, out, ps, k, n, s);
+        case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w, x, out, ps, k, n, s);
+        case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w, x, out, ps, k, n, s);
     }
     return CQ_ERR_DTYPE;
 }

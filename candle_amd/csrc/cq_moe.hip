@@ -36,39 +36,6 @@ inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pa
     return w;
 }
 
-struct PairSource {
-    int mode;
-    const uint32_t *ids_u32;
-    const int32_t *sorted_token_ids, *expert_ids;
-    const float *topk_weights;
-    int topk, input_dim1;
-    int n_pairs, num_experts, x_rows;
-};
-
-__device__ __forceinline__ bool pair_decode(const PairSource &ps, int p, int &e, int &in_row, int &out_row, float &scale) {
-    if (ps.mode == MOE_INDEXED) {
-        uint32_t id = ps.ids_u32[p];
-        e = (int)id;
-        in_row = ps.input_dim1 == 1 ? p / ps.topk : p;
-        out_row = p;
-        scale = 1.0f;
-        return id < (uint32_t)ps.num_experts;
-    }
-    e = ps.expert_ids[p];
-    int tok = ps.sorted_token_ids[p];
-    out_row = tok;
-    if (ps.topk_weights) {
-        in_row = tok;
-        // a token id outside the table would read past topk_weights; such pairs are dropped below
-        scale = (tok >= 0 && tok < ps.n_pairs) ? ps.topk_weights[tok] : 0.0f;
-    } else {
-        in_row = tok / ps.topk;
-        scale = 1.0f;
-    }
-    return e >= 0 && e < ps.num_experts && tok >= 0 && tok < ps.n_pairs && in_row < ps.x_rows;
-}
-
-// One workgroup: histogram of experts, exclusive scan, scatter of the pair descriptors.
 // offsets[e] .. offsets[e+1] is expert e's segment of pair_in / pair_out / pair_scale.
 __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__restrict__ offsets, int *__restrict__ cursor,
                                                          int *__restrict__ pair_in, int *__restrict__ pair_out,
@@ -201,6 +168,16 @@ int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_
 
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
+    PairSource ps;
+    ps.mode = a.mode; ps.ids_u32 = a.ids_u32; ps.sorted_token_ids = a.sorted_token_ids; ps.expert_ids = a.expert_ids;
+    ps.topk_weights = a.topk_weights; ps.topk = (int)a.topk; ps.input_dim1 = (int)a.input_dim1;
+    ps.n_pairs = (int)a.n_pairs; ps.num_experts = (int)a.num_experts; ps.x_rows = (int)a.x_rows;
+    // Few pairs (decode): every pair is its own fused matvec (activation quantization in the kernel, no scratch,
+    // no grouping pass); an expert hit by two pairs is simply read twice, the second time from cache.
+    if (a.n_pairs <= CQ_MOE_DIRECT_MAX_PAIRS) {
+        int rc = cq_moe_pairs_launch(a.w_dtype, a.w, a.x, a.out, ps, a.k, a.n, s);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
     MoeWorkspace ws = moe_workspace(a.w_dtype, a.num_experts, a.n_pairs, a.x_rows, a.k);
     uint8_t *b = (uint8_t *)workspace;
     int rc = cq_quantize_act_launch(a.w_dtype, a.x, CQ_F32, b + ws.act_off, a.k, a.x_rows, s);
@@ -208,10 +185,6 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     int *offsets = (int *)(b + ws.offsets_off), *cursor = (int *)(b + ws.cursor_off);
     int *pin = (int *)(b + ws.pin_off), *pout = (int *)(b + ws.pout_off);
     float *pscale = (float *)(b + ws.pscale_off);
-    PairSource ps;
-    ps.mode = a.mode; ps.ids_u32 = a.ids_u32; ps.sorted_token_ids = a.sorted_token_ids; ps.expert_ids = a.expert_ids;
-    ps.topk_weights = a.topk_weights; ps.topk = (int)a.topk; ps.input_dim1 = (int)a.input_dim1;
-    ps.n_pairs = (int)a.n_pairs; ps.num_experts = (int)a.num_experts; ps.x_rows = (int)a.x_rows;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n);
     if ((rc = (int)hipGetLastError())) return rc;
     ActView av = cq_act_view(b + ws.act_off, a.w_dtype, a.k, a.x_rows);

@@ -57,7 +57,7 @@ def test_indexed_moe_forward(dtype, input_dim1_is_one):
 
 
 @pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
-@pytest.mark.parametrize("tokens", [1, 16, 40])
+@pytest.mark.parametrize("tokens", [1, 16, 40, 100])      # up to 256 pairs: one fused matvec per pair; beyond: grouped by expert
 @pytest.mark.parametrize("is_prefill", [False, True])
 def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     """The two call shapes of FusedMoeGGUF::forward (fused_moe.rs:263-294): gate/up without
@@ -84,6 +84,27 @@ def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     want2 = oracle.moe_gemm_gguf(dtype, x2, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
     err2 = rel_l2(got2.cpu().numpy(), want2)
     assert err2 <= TOL and err2 <= TIGHT, err2
+
+
+@pytest.mark.parametrize("batch", [4, 120])                 # 12 pairs (per-pair kernels) and 360 pairs (grouped path)
+def test_indexed_moe_forward_out_of_range_id_gives_zero_row(batch):
+    import candle_amd as ca
+    E, n, k, topk = 8, 48, 512, 3
+    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=55)
+    ids, _, _, _ = route(batch, E, topk, seed=56)
+    ids = ids.astype(np.int64)
+    ids[1, 2] = E + 3                                        # not an expert
+    x = normal(57, (batch, 1, k), 1.0)
+    out = qt.indexed_moe_forward(torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda())
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.all(got[1, 2] == 0.0)
+    good = ids.copy()
+    good[1, 2] = 0
+    want = oracle.indexed_moe_forward(oracle.Q4K, blocks, (E, n, k), x, good.astype(np.uint32))
+    mask = np.ones((batch, topk), dtype=bool)
+    mask[1, 2] = False
+    assert rel_l2(got[mask], want[mask]) <= TIGHT
 
 
 def test_moe_gemm_is_invariant_to_pair_order():
