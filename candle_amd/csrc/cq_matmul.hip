@@ -20,11 +20,10 @@
 //   are rounded to f16 (relative 2^-11 per operand) and multiplied at full MFMA rate; the result stays
 //   well inside the 1e-3 tolerance (measured ~2e-4) but is not integer-exact like the decode path.
 //
-// Tiling: workgroup = 4 waves (2 x 2), block tile 128 (m) x 128 (n), wave tile 64 x 64 as 2 x 2
-// v_mfma_f32_32x32x16_f16 tiles.  K advances 64 elements per LDS stage: 256 threads dequantize the
-// 128 x 64 weight tile and convert the 128 x 64 int8 activation tile to f16 in LDS (row stride padded
-// to 144 bytes); the raw bytes of the next stage are loaded into registers before the MFMAs of the
-// current one.
+// Tiling: workgroup = 4 waves (2 x 2), block tile 128 (m) x 64 (n), wave tile 64 x 32 as 2 x 1
+// v_mfma_f32_32x32x16_f16 tiles (128 x 128 / 64 x 64 for long Q4_0 / Q8_0 problems).  K advances 64 elements per
+// LDS stage: the threads dequantize the weight tile and convert the 128 x 64 int8 activation tile to f16 in LDS
+// (row stride padded to 144 bytes); raw bytes are requested two stages ahead into two register sets.
 #include "cq_device.h"
 #include "cq_launch.h"
 
@@ -34,7 +33,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BM = 128, BK = 64;
 constexpr int LDK = BK + 8;            // padded row stride in halves (144 bytes)
 
 // ---- integer bytes -> f16 pairs ------------------------------------------------------------------
@@ -273,11 +272,14 @@ __device__ __forceinline__ void lds_write32h(_Float16 *dstrow, const uint32_t v[
     p[3] = u32x4{v[12], v[13], v[14], v[15]};
 }
 
-template <int DT>
-__global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k, int n, int rows,
-                                                  int64_t stride_dst) {
+// NJ = 32-column MFMA tiles per wave: block tile 128 x (64 * NJ).  NJ = 1 halves the accumulators so that two
+// workgroups share a CU and one converts operands while the other feeds the matrix cores.
+template <int DT, int NJ>
+__global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k,
+                                                                     int n, int rows, int64_t stride_dst) {
     typedef Stage<DT> S;
     constexpr bool KQ = S::KQ;
+    constexpr int BN = 64 * NJ, WN = 32 * NJ;
     __shared__ __align__(16) _Float16 As[BM * LDK];
     __shared__ __align__(16) _Float16 Bs[BN * LDK];
     __shared__ __align__(16) _Float16 Bs2[S::TERMS == 2 ? BN * LDK : 8];   // exact remainders of a two-term format
@@ -288,47 +290,56 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = wv >> 1, wn = wv & 1;
     const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    const bool bstage = tid < 2 * BN;                            // threads that also stage a weight row (wave-uniform)
     const int nsb = k >> 8;                                     // 256-element spans
     const int64_t row_bytes = (int64_t)(k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
 
     // staging role of this thread: (row r_l of the tile, 32-element half)
     const int r_l = tid >> 1, half = tid & 1;
-    const int wrow = min(n0 + r_l, n - 1);
+    const int wrow = min(n0 + (bstage ? r_l : 0), n - 1);
     const int arow = min(m0 + r_l, rows - 1);
     const bool arow_ok = m0 + r_l < rows;
     const uint8_t *wrow_p = w + wrow * row_bytes;
     const int8_t *aq_p = av.qs + (int64_t)arow * k;
 
-    f32x16 acc[2][2], sb[2][2];
+    f32x16 acc[2][NJ], sb[2][NJ];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) { acc[i][j][e] = 0.0f; sb[i][j][e] = 0.0f; }
 
-    typename S::Raw wraw;
-    u32x4 a0, a1;
-    auto load_stage = [&](int kb, int g) {
-        S::load(wraw, wrow_p, kb, g, half);
+    // raw bytes are requested two stages ahead (two register sets, chosen by the parity of the stage): one stage of
+    // conversion + MFMA work is shorter than a trip to memory
+    typename S::Raw wraw2[2];
+    u32x4 a02[2], a12[2];
+    auto load_stage = [&](int kb, int g, typename S::Raw &wr, u32x4 &x0, u32x4 &x1) {
+        if (bstage) S::load(wr, wrow_p, kb, g, half);
         const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
-        a0 = *reinterpret_cast<const u32x4 *>(q);
-        a1 = *reinterpret_cast<const u32x4 *>(q + 16);
+        x0 = *reinterpret_cast<const u32x4 *>(q);
+        x1 = *reinterpret_cast<const u32x4 *>(q + 16);
     };
-    load_stage(0, 0);
+    load_stage(0, 0, wraw2[0], a02[0], a12[0]);
+    load_stage(0, 1, wraw2[1], a02[1], a12[1]);
 
     for (int kb = 0; kb < nsb; kb++) {
+#pragma unroll
         for (int g = 0; g < 4; g++) {
+            typename S::Raw &wraw = wraw2[g & 1];
+            u32x4 &a0 = a02[g & 1], &a1 = a12[g & 1];
             // ---- write the staged raw data of (kb, g) to LDS as f16 ----
             uint32_t hv[16];
-            if constexpr (S::TERMS == 2) {
-                uint32_t hr[16];
-                S::convert2(wraw, g, half, hv, hr);
-                lds_write32h(Bs2 + r_l * LDK + 32 * half, hr);
-            } else {
-                S::convert(wraw, g, half, hv);
+            if (bstage) {
+                if constexpr (S::TERMS == 2) {
+                    uint32_t hr[16];
+                    S::convert2(wraw, g, half, hv, hr);
+                    lds_write32h(Bs2 + r_l * LDK + 32 * half, hr);
+                } else {
+                    S::convert(wraw, g, half, hv);
+                }
+                lds_write32h(Bs + r_l * LDK + 32 * half, hv);
             }
-            lds_write32h(Bs + r_l * LDK + 32 * half, hv);
             uint32_t ascale2 = 0;
             if (!KQ) {
                 float d8 = av.d[2 * ((int64_t)arow * (k >> 5) + kb * 8 + 2 * g + half)];   // already f16-representable
@@ -341,10 +352,13 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
             }
             lds_write32h(As + r_l * LDK + 32 * half, hv);
             if (KQ && g == 0) {
-                float d, dmin;
-                int mins[8];
-                S::header(wraw, d, dmin, mins);
-                if (half == 0) { sD[r_l] = d; sDmin[r_l] = dmin; sD8[r_l] = arow_ok ? av.d[(int64_t)arow * (k >> 8) + kb] : 0.0f; }
+                float d = 0.0f, dmin = 0.0f;
+                int mins[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (bstage) S::header(wraw, d, dmin, mins);
+                if (half == 0) {
+                    if (bstage) { sD[r_l] = d; sDmin[r_l] = dmin; }
+                    sD8[r_l] = arow_ok ? av.d[(int64_t)arow * (k >> 8) + kb] : 0.0f;
+                }
                 if (S::HAS_MIN) {
                     // Bm[n][j] = min[j/2] for j in 8*half .. 8*half+7 ; Am[m][j] = bsums16[j]
                     uint32_t mv[4];
@@ -353,7 +367,7 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
                         uint32_t hm = f2h_bits((float)mins[4 * half + i]);
                         mv[i] = hm | (hm << 16);
                     }
-                    *reinterpret_cast<u32x4 *>(Bm + r_l * 24 + 8 * half) = u32x4{mv[0], mv[1], mv[2], mv[3]};
+                    if (bstage) *reinterpret_cast<u32x4 *>(Bm + r_l * 24 + 8 * half) = u32x4{mv[0], mv[1], mv[2], mv[3]};
                     u32x4 bs = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
                     const uint32_t b4[4] = {bs.x, bs.y, bs.z, bs.w};
                     uint32_t bv[4];
@@ -366,49 +380,50 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
                 }
             }
             __syncthreads();
-            // ---- raw bytes of the next stage go in flight while the matrix cores work ----
+            // ---- the register set just consumed is refilled with the stage after next ----
             {
-                int ng = g + 1, nkb = kb;
-                if (ng == 4) { ng = 0; nkb = kb + 1; }
-                if (nkb < nsb) load_stage(nkb, ng);
+                const int ng = (g + 2) & 3, nkb = g >= 2 ? kb + 1 : kb;
+                if (nkb < nsb) load_stage(nkb, ng, wraw, a0, a1);
             }
             // ---- 4 k-slices of 16: 2 x 2 MFMA tiles per wave ----
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                half8 af[2], bf[2];
+                half8 af[2], bf[NJ];
 #pragma unroll
-                for (int t = 0; t < 2; t++) {
+                for (int t = 0; t < 2; t++)
                     af[t] = *reinterpret_cast<const half8 *>(As + (wm * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
-                    bf[t] = *reinterpret_cast<const half8 *>(Bs + (wn * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
-                }
+#pragma unroll
+                for (int t = 0; t < NJ; t++)
+                    bf[t] = *reinterpret_cast<const half8 *>(Bs + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
                 for (int i = 0; i < 2; i++)
 #pragma unroll
-                    for (int j = 0; j < 2; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
+                    for (int j = 0; j < NJ; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
                 if constexpr (S::TERMS == 2) {
 #pragma unroll
-                    for (int t = 0; t < 2; t++)
-                        bf[t] = *reinterpret_cast<const half8 *>(Bs2 + (wn * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
+                    for (int t = 0; t < NJ; t++)
+                        bf[t] = *reinterpret_cast<const half8 *>(Bs2 + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
                     for (int i = 0; i < 2; i++)
 #pragma unroll
-                        for (int j = 0; j < 2; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
+                        for (int j = 0; j < NJ; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
                 }
             }
             if (KQ && g == 3) {
                 // ---- end of the super-block: mins term and the f32 scales ----
-                f32x16 mt[2][2];
+                f32x16 mt[2][NJ];
                 if (S::HAS_MIN) {
-                    half8 am[2], bm[2];
+                    half8 am[2], bm[NJ];
 #pragma unroll
-                    for (int t = 0; t < 2; t++) {
+                    for (int t = 0; t < 2; t++)
                         am[t] = *reinterpret_cast<const half8 *>(Am + (wm * 64 + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
-                        bm[t] = *reinterpret_cast<const half8 *>(Bm + (wn * 64 + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
-                    }
+#pragma unroll
+                    for (int t = 0; t < NJ; t++)
+                        bm[t] = *reinterpret_cast<const half8 *>(Bm + (wn * WN + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
 #pragma unroll
                     for (int i = 0; i < 2; i++)
 #pragma unroll
-                        for (int j = 0; j < 2; j++) {
+                        for (int j = 0; j < NJ; j++) {
                             f32x16 z;
 #pragma unroll
                             for (int e = 0; e < 16; e++) z[e] = 0.0f;
@@ -416,8 +431,8 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
                         }
                 }
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const int nl = wn * 64 + j * 32 + (lane & 31);
+                for (int j = 0; j < NJ; j++) {
+                    const int nl = wn * WN + j * 32 + (lane & 31);
                     const float d = sD[nl], dmin = sDmin[nl];
 #pragma unroll
                     for (int i = 0; i < 2; i++) {
@@ -440,8 +455,8 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int nn = n0 + wn * 64 + j * 32 + (lane & 31);
+        for (int j = 0; j < NJ; j++) {
+            const int nn = n0 + wn * WN + j * 32 + (lane & 31);
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int mm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
@@ -453,9 +468,16 @@ __global__ __launch_bounds__(256) void qmm_kernel(const uint8_t *__restrict__ w,
 
 template <int DT>
 int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
-    dim3 grid((unsigned)((rows + BM - 1) / BM), (unsigned)((n + BN - 1) / BN));
+    // 128 x 64 tiles (two or three workgroups per CU) everywhere except long Q4_0 / Q8_0 problems, whose cheaper
+    // operand conversion leaves the 128 x 128 tile (one workgroup per CU, half the activation conversions) ahead
+    const bool wide = !Stage<DT>::KQ && rows >= 1024;
+    const int bn = wide ? 128 : 64;
+    dim3 grid((unsigned)((rows + BM - 1) / BM), (unsigned)((n + bn - 1) / bn));
     if (grid.y > 65535) return CQ_ERR_RANGE;
-    hipLaunchKernelGGL((qmm_kernel<DT>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst);
+    if (wide)
+        hipLaunchKernelGGL((qmm_kernel<DT, 2>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst);
+    else
+        hipLaunchKernelGGL((qmm_kernel<DT, 1>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst);
     return (int)hipGetLastError();
 }
 
