@@ -20,6 +20,29 @@ __global__ __launch_bounds__(256) void quantize_q80_kernel(const void *__restric
     cq_quantize_q80_span<XDT>(x, span, threadIdx.x & 63, total, qs, ds);
 }
 
+// Gathering variants (f32 rows): destination row i of the scratch is row row_map[i] of x.  k is a multiple of 256.
+__global__ __launch_bounds__(256) void quantize_q8k_gather_kernel(const float *__restrict__ x, const int *__restrict__ row_map, int kb,
+                                                                  int8_t *__restrict__ qs, float *__restrict__ dout, int16_t *__restrict__ bsums,
+                                                                  int64_t n_blocks) {
+    const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= n_blocks) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = blk / kb, b = blk - row * kb;
+    float v[4];
+    cq_load4<CQ_F32>(x, ((int64_t)row_map[row] * kb + b) * 256 + lane * 4, v);
+    cq_quantize_q8k_vals(v, blk, lane, qs, dout, bsums);
+}
+__global__ __launch_bounds__(256) void quantize_q80_gather_kernel(const float *__restrict__ x, const int *__restrict__ row_map, int kb,
+                                                                  int8_t *__restrict__ qs, float *__restrict__ ds, int64_t n_spans) {
+    const int64_t span = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (span >= n_spans) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = span / kb, b = span - row * kb;
+    float v[4];
+    cq_load4<CQ_F32>(x, ((int64_t)row_map[row] * kb + b) * 256 + lane * 4, v);
+    cq_quantize_q80_vals(v, true, span * 256 + lane * 4, lane, qs, ds);
+}
+
 template <int XDT>
 int launch_quantize_act(int w_dtype, const void *x, void *scratch, int64_t k, int64_t rows, hipStream_t s) {
     ActLayout L = cq_act_layout(w_dtype, k, rows);
@@ -49,4 +72,23 @@ int cq_quantize_act_launch(int w_dtype, const void *x, int x_dtype, void *scratc
         case CQ_BF16: return launch_quantize_act<CQ_BF16>(w_dtype, x, scratch, k, rows, s);
     }
     return CQ_ERR_DTYPE;
+}
+
+// Scratch rows [0, rows) = quantized x[row_map[i]]; the layout is that of `rows_alloc` rows (rows_alloc >= rows).
+int cq_quantize_act_gather_launch(int w_dtype, const float *x, const int *row_map, void *scratch, int64_t k, int64_t rows, int64_t rows_alloc,
+                                  hipStream_t s) {
+    if (k % 256) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    ActLayout L = cq_act_layout(w_dtype, k, rows_alloc);
+    uint8_t *b = (uint8_t *)scratch;
+    const int64_t spans = rows * (k / 256);
+    const int64_t grid = (spans + 3) / 4;
+    if (grid > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (cq_is_kquant(w_dtype))
+        hipLaunchKernelGGL(quantize_q8k_gather_kernel, dim3((unsigned)grid), dim3(256), 0, s, x, row_map, (int)(k / 256), (int8_t *)(b + L.qs_off),
+                           (float *)(b + L.d_off), (int16_t *)(b + L.bs_off), spans);
+    else
+        hipLaunchKernelGGL(quantize_q80_gather_kernel, dim3((unsigned)grid), dim3(256), 0, s, x, row_map, (int)(k / 256), (int8_t *)(b + L.qs_off),
+                           (float *)(b + L.d_off), spans);
+    return (int)hipGetLastError();
 }

@@ -88,3 +88,17 @@ __device__ __forceinline__ bool pair_decode(const PairSource &ps, int p, int &e,
 #define CQ_MOE_DIRECT_MAX_PAIRS 256
 // CQ_ERR_RANGE when the shape is not served by the fused kernel (the caller then takes the grouped path).
 int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s);
+
+int cq_quantize_act_gather_launch(int w_dtype, const float *x, const int *row_map, void *scratch, int64_t k, int64_t rows, int64_t rows_alloc,
+                                  hipStream_t s);
+// Expert-grouped MoE, 8 pairs per weight pass.  Chunk c (c < *n_chunks) covers sorted pairs [first[c], first[c] + count[c]) of expert[c];
+// the activation scratch holds the quantized rows in sorted-pair order (layout of rows_alloc rows).
+#define CQ_MOE_CHUNK 8
+struct MoeChunks {
+    const int *n_chunks, *expert, *first, *count;
+    const int *pair_out;
+    const float *pair_scale;
+    int max_chunks;
+};
+int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k,
+                         int64_t n, hipStream_t s);

@@ -41,11 +41,13 @@ struct ActSrc {
 //   EPI_SWIGLU a logical row r is the pair (W[r], W[r] + pair_off bytes) = (feed_forward_w1, feed_forward_w3):
 //             dst[r] = silu(W1[r] . x) * (W3[r] . x)   (rows of one wave step only)
 //   EPI_SCALE the result is multiplied by a per-launch-block scalar (Fuse::eps) before it is stored (MoE top-k weight)
+//   EPI_MOE   activation row b of the launch block belongs to output row row_map[b] and is scaled by row_scale[b];
+//             rows b >= nvalid are padding and are not stored (8 router pairs of one expert per weight pass)
 //   EPI_RESID the result is added to a residual row in place of being stored, and the workgroup leaves
 //             its partial sum of residual^2 for the next PRO_NORM consumer
 enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2, PRO_MERGE = 3 };
 constexpr int MAXS = 16;     // attention splits a PRO_MERGE prologue can merge
-enum { EPI_NONE = 0, EPI_RESID = 1, EPI_SWIGLU = 2, EPI_SCALE = 3 };
+enum { EPI_NONE = 0, EPI_RESID = 1, EPI_SWIGLU = 2, EPI_SCALE = 3, EPI_MOE = 4 };
 constexpr int NPART = 256;   // == CQ_NN_PARTIALS
 struct Fuse {
     const float *aux;        // PRO_NORM: norm weight [k];  PRO_SILU: up [k];  PRO_MERGE: partials [k/hd][splits][hd + 4]
@@ -55,6 +57,9 @@ struct Fuse {
     float *part_out;         // EPI_RESID: [NPART]
     int splits, hd_shift;    // PRO_MERGE
     int64_t pair_off;        // EPI_SWIGLU: byte distance from a row of w1 to the same row of w3
+    const int *row_map;      // EPI_MOE
+    const float *row_scale;
+    int nvalid;
 };
 
 // Launch geometry, computed once on the host so the kernel prologue is a handful of scalar loads
@@ -123,7 +128,7 @@ template <int DT, int NB, int SRC, bool SINGLE, int PRO, int EPI, bool PRE>
 __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const ActSrc &src, void *__restrict__ dst, const QmvGeom &g, const Fuse &fz,
                                          const int block, const int nblocks) {
     typedef Fmt<DT> F;
-    static_assert((PRO == PRO_NONE && EPI == EPI_NONE) || (NB == 1 && SRC == CQ_F32), "fusions are for one f32 row");
+    static_assert((PRO == PRO_NONE && (EPI == EPI_NONE || EPI == EPI_MOE)) || (NB == 1 && SRC == CQ_F32), "fusions are for one f32 row");
     static_assert(PRO != PRO_MERGE || (SINGLE && !PRE), "the merge prologue preloads one span per wave");
     static_assert(EPI != EPI_SWIGLU || SINGLE, "the paired-row epilogue is written for rows of one wave step");
     constexpr bool FUSED = SRC != SRC_SCRATCH;
@@ -199,9 +204,18 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
     // PRE (rows of 2..4 wave steps, e.g. K = 14336): all steps of the wave's first row are issued here, so the
     // whole first row streams in behind the activation prologue instead of one step of it
     typename F::W pre[PRE ? 4 : 1];
+    // BLOCKED (rows of one wave step, more than two activation rows): weight rows are taken RB at a time and held in
+    // registers while each activation row is read from LDS once per block, not once per weight row
+    constexpr bool BLOCKED = SINGLE && NB > 2;
+    constexpr int RB = 4;
+    typename F::W wA[BLOCKED ? RB : 1], wB[BLOCKED ? RB : 1];
+    const int last_j = max(my_rows - 1, 0);
     if (PRE) {
 #pragma unroll
         for (int i = 0; i < 4; i++) F::load_w(pre[i], wp, min(lane + 64 * i, units - 1));
+    } else if (BLOCKED) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) F::load_w(wA[r], wp + (int64_t)min(r, last_j) * wave_stride, u0);
     } else {
         F::load_w(wa, wp, u0);
     }
@@ -275,6 +289,17 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
     __syncthreads();
     if (EPI != EPI_RESID && my_rows == 0) return;
     float ssq = 0.0f;            // EPI_RESID: lane 63 accumulates residual^2 of this wave's rows
+    constexpr bool MOE_TAB = EPI == EPI_MOE && !(SINGLE && NB > 2);      // the blocked path reads them per b instead
+    int64_t moe_off[MOE_TAB ? NB : 1];
+    float moe_sc[MOE_TAB ? NB : 1];
+    if (MOE_TAB) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const bool live = b < fz.nvalid;
+            moe_off[b] = live ? (int64_t)fz.row_map[b] * stride_dst : -1;
+            moe_sc[b] = live ? fz.row_scale[b] : 0.0f;
+        }
+    }
 
     ActRow ar[NB];
 #pragma unroll
@@ -302,11 +327,53 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
                         fz.resid[r] = sres;
                         ssq += sres * sres;
                     }
+                } else if (EPI == EPI_MOE) {
+                    if (lane == 63 && moe_off[MOE_TAB ? b : 0] >= 0) ((float *)dst)[moe_off[MOE_TAB ? b : 0] + r] = v * moe_sc[MOE_TAB ? b : 0];
                 } else if (lane == 63) {
                     store_out(dst, dst_dtype, (int64_t)b * stride_dst + r, EPI == EPI_SCALE ? v * fz.eps : v);
                 }
             }
         };
+        if (BLOCKED) {
+            auto load_block = [&](typename F::W (&wr)[BLOCKED ? RB : 1], int j0) {
+#pragma unroll
+                for (int r = 0; r < RB; r++) F::load_w(wr[BLOCKED ? r : 0], wp + (int64_t)min(j0 + r, last_j) * wave_stride, u0);
+            };
+            auto compute_block = [&](const typename F::W (&wr)[BLOCKED ? RB : 1], int j0) {
+                // not unrolled over the activation rows: everything that depends on b is recomputed from b, so the
+                // registers hold two blocks of weight rows and one activation unit, whatever NB is
+#pragma unroll 1
+                for (int b = 0; b < NB; b++) {
+                    const ActRow arb = act_row(lqs, ld, lbs, DT, b, k);
+                    F::load_a(areg[0], arb, u0);
+                    int64_t off = (int64_t)b * stride_dst;
+                    float sc = 1.0f;
+                    if (EPI == EPI_MOE) {
+                        const bool live = b < fz.nvalid;
+                        off = live ? (int64_t)fz.row_map[live ? b : 0] * stride_dst : -1;
+                        sc = live ? fz.row_scale[live ? b : 0] : 0.0f;
+                    }
+#pragma unroll
+                    for (int r = 0; r < RB; r++) {
+                        float v = F::dot(wr[BLOCKED ? r : 0], areg[0], u0);
+                        v = wave_sum_to_lane63(valid ? v : 0.0f);
+                        const int rr = row + ((j0 + r) << g.nw_shift);
+                        if (lane == 63 && j0 + r < my_rows && off >= 0) {
+                            if (EPI == EPI_MOE) ((float *)dst)[off + rr] = v * sc;
+                            else store_out(dst, dst_dtype, off + rr, v);
+                        }
+                    }
+                }
+            };
+            for (int j = 0; j < my_rows; j += 2 * RB) {
+                load_block(wB, j + RB);
+                compute_block(wA, j);
+                if (j + RB >= my_rows) break;
+                load_block(wA, j + 2 * RB);
+                compute_block(wB, j + RB);
+            }
+            return;
+        }
         if (EPI == EPI_SWIGLU) {
             // wa = W1[row] (already in flight), wb = W3[row]; the next W1 row is requested before W3 is reduced
             for (int j = 0; j < my_rows; j++) {
@@ -361,6 +428,8 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
                         fz.resid[row] = sres;
                         ssq += sres * sres;
                     }
+                } else if (EPI == EPI_MOE) {
+                    if (lane == 63 && moe_off[MOE_TAB ? b : 0] >= 0) ((float *)dst)[moe_off[MOE_TAB ? b : 0] + row] = r * moe_sc[MOE_TAB ? b : 0];
                 } else if (lane == 63) {
                     store_out(dst, dst_dtype, (int64_t)b * stride_dst + row, EPI == EPI_SCALE ? r * fz.eps : r);
                 }
@@ -426,8 +495,10 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
     }
 }
 
+// More than two activation rows keep blocks of weight rows in registers: workgroups of 8 waves (256 VGPRs per
+// lane) instead of 16 (128).
 template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
-__global__ __launch_bounds__(1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g, Fuse fz) {
+__global__ __launch_bounds__(NB > 2 ? 512 : 1024) void qmv_kernel(const uint8_t *__restrict__ w, ActSrc src, void *__restrict__ dst, QmvGeom g, Fuse fz) {
     qmv_body<DT, NB, SRC, SINGLE, PRO, EPI, PRE>(w, src, dst, g, fz, blockIdx.x, gridDim.x);
 }
 
@@ -448,7 +519,7 @@ template <int DT, int NB>
 int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int64_t stride_dst, int dst_dtype, int extra_lds, size_t &lds_bytes,
               int64_t max_groups = 256) {
     if (waves == 0) {
-        waves = 16;
+        waves = NB > 2 ? 8 : 16;
         while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
     }
     groups = (n + waves - 1) / waves;
@@ -472,7 +543,7 @@ int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int
 
 template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
 int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s,
-               const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0}) {
+               const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0}) {
     QmvGeom g;
     int64_t groups;
     int waves = 0;
@@ -604,7 +675,7 @@ int cq_matvec_norm_launch(int w_dtype, const void *w, const float *x, const floa
                           int64_t k, int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
     return launch_fused_dt<PRO_NORM, EPI_NONE>(w_dtype, w, src, dst, k, n, s, fz);
 }
 
@@ -613,7 +684,7 @@ int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const 
                               int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{up, nullptr, 0.0f, residual, partials_out, 0, 0, 0};
+    Fuse fz{up, nullptr, 0.0f, residual, partials_out, 0, 0, 0, nullptr, nullptr, 0};
     if (up) return launch_fused_dt<PRO_SILU, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
     return launch_fused_dt<PRO_NONE, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
 }
@@ -636,7 +707,7 @@ int cq_matvec_residual_attn_launch(int w_dtype, const void *w, const float *attn
     if (splits < 1 || splits > MAXS || head_dim < 4 || (head_dim & (head_dim - 1)) || k % head_dim) return CQ_ERR_RANGE;
     int sh = 0;
     while ((1 << sh) < head_dim) sh++;
-    Fuse fz{attn_partials, nullptr, 0.0f, residual, partials_out, (int)splits, sh, 0};
+    Fuse fz{attn_partials, nullptr, 0.0f, residual, partials_out, (int)splits, sh, 0, nullptr, nullptr, 0};
     switch (w_dtype) {
         case CQ_Q4_0: return launch_merge1<CQ_Q4_0>(w, nullptr, k, n, s, fz);
         case CQ_Q8_0: return launch_merge1<CQ_Q8_0>(w, nullptr, k, n, s, fz);
@@ -702,7 +773,7 @@ int cq_matvec_norm_swiglu_launch(int w_dtype, const void *w1, const void *w3, co
                                  float eps, float *dst, int64_t k, int64_t ffn, hipStream_t s) {
     if (ffn == 0) return CQ_OK;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
     const int64_t off = (const uint8_t *)w3 - (const uint8_t *)w1;
     switch (w_dtype) {
         case CQ_Q4_0: return launch_swiglu1<CQ_Q4_0>(w1, off, src, dst, k, ffn, s, fz);
@@ -721,7 +792,7 @@ int cq_matvec_norm_pair_launch(int dta, const void *wa, int64_t na, float *dsta,
     if (na == 0 || nb == 0) return CQ_ERR_SHAPE;
     if (cq_act_layout(dta, k, 1).total > LDS_BUDGET) return CQ_ERR_RANGE;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0};
+    Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
     switch (dta) {
         case CQ_Q4K: return launch_pair_b<CQ_Q4K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
         case CQ_Q5K: return launch_pair_b<CQ_Q5K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
@@ -746,7 +817,7 @@ __global__ __launch_bounds__(1024) void moe_pair_kernel(const uint8_t *__restric
         return;
     }
     ActSrc src{x + (int64_t)in_row * g.k, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{nullptr, nullptr, scale, nullptr, nullptr, 0, 0, 0};
+    Fuse fz{nullptr, nullptr, scale, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
     qmv_body<DT, 1, CQ_F32, SINGLE, PRO_NONE, EPI_SCALE, false>(w + (int64_t)e * expert_bytes, src, out + (int64_t)out_row * g.n, g, fz,
                                                                 blockIdx.x, gridDim.x);
 }
@@ -789,6 +860,62 @@ int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, 
         case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w, x, out, ps, k, n, s);
         case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w, x, out, ps, k, n, s);
         case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w, x, out, ps, k, n, s);
+    }
+    return CQ_ERR_DTYPE;
+}
+
+// ---- MoE grouped by expert: block (tile, chunk) runs up to 8 pairs of one expert against one pass over its rows ----
+namespace {
+template <int DT, bool SINGLE>
+__global__ __launch_bounds__(512) void moe_chunk_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ out, QmvGeom g, MoeChunks mc,
+                                                         int64_t expert_bytes) {
+    const int c = blockIdx.y;
+    if (c >= mc.n_chunks[0]) return;                            // uniform over the workgroup
+    const int first = mc.first[c];
+    ActSrc src{nullptr, cq_act_view_rows(av, DT, g.k, first)};
+    Fuse fz{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0, mc.pair_out + first, mc.pair_scale + first, mc.count[c]};
+    qmv_body<DT, CQ_MOE_CHUNK, SRC_SCRATCH, SINGLE, PRO_NONE, EPI_MOE, false>(w + (int64_t)mc.expert[c] * expert_bytes, src, out, g, fz, blockIdx.x,
+                                                                              gridDim.x);
+}
+
+template <int DT>
+int launch_moe_chunks(const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k, int64_t n,
+                      hipStream_t s) {
+    if (cq_act_layout(DT, k, CQ_MOE_CHUNK).total > LDS_BUDGET) return CQ_ERR_RANGE;
+    QmvGeom g;
+    int64_t groups;
+    size_t lds_bytes;
+    int waves = 8;
+    const int64_t per_chunk = (2048 + mc.max_chunks - 1) / mc.max_chunks;
+    int rc = make_geom<DT, CQ_MOE_CHUNK>(g, groups, waves, k, n, n, CQ_F32, 0, lds_bytes, per_chunk < 256 ? per_chunk : 256);
+    if (rc) return rc;
+    if (mc.max_chunks > 65535) return CQ_ERR_RANGE;
+    const int64_t expert_bytes = n * (int64_t)g.row_bytes;
+    const bool single = g.units <= 64;
+    const void *kp = single ? (const void *)moe_chunk_kernel<DT, true> : (const void *)moe_chunk_kernel<DT, false>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    ActView av = cq_act_view(scratch, DT, k, rows_alloc);
+    dim3 grid((unsigned)groups, (unsigned)mc.max_chunks), block(64 * waves);
+    if (single)
+        hipLaunchKernelGGL((moe_chunk_kernel<DT, true>), grid, block, lds_bytes, s, (const uint8_t *)w, av, out, g, mc, expert_bytes);
+    else
+        hipLaunchKernelGGL((moe_chunk_kernel<DT, false>), grid, block, lds_bytes, s, (const uint8_t *)w, av, out, g, mc, expert_bytes);
+    return (int)hipGetLastError();
+}
+}  // namespace
+
+int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k,
+                         int64_t n, hipStream_t s) {
+    if (mc.max_chunks == 0 || n == 0) return CQ_OK;
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_moe_chunks<CQ_Q4_0>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q8_0: return launch_moe_chunks<CQ_Q8_0>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q4K: return launch_moe_chunks<CQ_Q4K>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q5K: return launch_moe_chunks<CQ_Q5K>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q6K: return launch_moe_chunks<CQ_Q6K>(w, scratch, rows_alloc, out, mc, k, n, s);
     }
     return CQ_ERR_DTYPE;
 }

@@ -21,25 +21,31 @@
 namespace {
 
 struct MoeWorkspace {
-    int64_t act_off, offsets_off, cursor_off, pin_off, pout_off, pscale_off, total;
+    int64_t act_off, offsets_off, cursor_off, pin_off, pout_off, pscale_off, chunk_off, max_chunks, rows_alloc, total;
 };
 
 inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k) {
     MoeWorkspace w;
     w.act_off = 0;
-    w.offsets_off = cq_act_layout(w_dtype, k, x_rows).total;
+    // the chunked path quantizes the activation rows in expert-sorted pair order (plus one chunk of padding rows);
+    // the older per-expert kernel quantizes the x rows as they are: room for the larger of the two
+    w.rows_alloc = n_pairs + CQ_MOE_CHUNK;
+    w.max_chunks = n_pairs / CQ_MOE_CHUNK + (num_experts < n_pairs ? num_experts : n_pairs) + 1;
+    w.offsets_off = cq_act_layout(w_dtype, k, w.rows_alloc > x_rows ? w.rows_alloc : x_rows).total;
     w.cursor_off = w.offsets_off + cq_align256((num_experts + 1) * 4);
     w.pin_off = w.cursor_off + cq_align256(num_experts * 4);
     w.pout_off = w.pin_off + cq_align256(n_pairs * 4);
     w.pscale_off = w.pout_off + cq_align256(n_pairs * 4);
-    w.total = w.pscale_off + cq_align256(n_pairs * 4);
+    w.chunk_off = w.pscale_off + cq_align256(n_pairs * 4);
+    w.total = w.chunk_off + cq_align256((3 * w.max_chunks + 1) * 4);      // n_chunks | expert[] | first[] | count[]
     return w;
 }
 
 // offsets[e] .. offsets[e+1] is expert e's segment of pair_in / pair_out / pair_scale.
 __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__restrict__ offsets, int *__restrict__ cursor,
                                                          int *__restrict__ pair_in, int *__restrict__ pair_out,
-                                                         float *__restrict__ pair_scale, float *__restrict__ out, int n) {
+                                                         float *__restrict__ pair_scale, float *__restrict__ out, int n, int *__restrict__ chunks,
+                                                         int max_chunks) {
     __shared__ int carry;
     const int tid = threadIdx.x;
     const int E = ps.num_experts;
@@ -75,7 +81,24 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
         if (tid == 1023) carry += buf[1023];
         __syncthreads();
     }
-    if (tid == 0) offsets[E] = carry;
+    if (tid == 0) { offsets[E] = carry; chunks[0] = 0; }
+    __syncthreads();
+    // positions behind the last valid pair are never part of a chunk, but the gathering quantizer walks all n_pairs
+    // rows: give them a valid source row
+    for (int p = carry + tid; p < ps.n_pairs; p += 1024) pair_in[p] = 0;
+    // chunk table: expert e's segment in pieces of CQ_MOE_CHUNK pairs (any order: chunks are independent)
+    for (int e = tid; e < E; e += 1024) {
+        const int seg0 = offsets[e], cnt = offsets[e + 1] - seg0;     // offsets[e + 1] of the last sweep's neighbour is final here
+        const int cc = (cnt + CQ_MOE_CHUNK - 1) / CQ_MOE_CHUNK;
+        if (cc > 0) {
+            const int base = atomicAdd(&chunks[0], cc);
+            for (int i = 0; i < cc; i++) {
+                chunks[1 + base + i] = e;
+                chunks[1 + max_chunks + base + i] = seg0 + i * CQ_MOE_CHUNK;
+                chunks[1 + 2 * max_chunks + base + i] = min(CQ_MOE_CHUNK, cnt - i * CQ_MOE_CHUNK);
+            }
+        }
+    }
     __syncthreads();
     for (int p = tid; p < ps.n_pairs; p += 1024) {
         int e, in_row, out_row;
@@ -180,13 +203,23 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     }
     MoeWorkspace ws = moe_workspace(a.w_dtype, a.num_experts, a.n_pairs, a.x_rows, a.k);
     uint8_t *b = (uint8_t *)workspace;
-    int rc = cq_quantize_act_launch(a.w_dtype, a.x, CQ_F32, b + ws.act_off, a.k, a.x_rows, s);
-    if (rc) return rc;
+    int rc;
     int *offsets = (int *)(b + ws.offsets_off), *cursor = (int *)(b + ws.cursor_off);
     int *pin = (int *)(b + ws.pin_off), *pout = (int *)(b + ws.pout_off);
     float *pscale = (float *)(b + ws.pscale_off);
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n);
+    int *chunks = (int *)(b + ws.chunk_off);
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
+                       (int)ws.max_chunks);
     if ((rc = (int)hipGetLastError())) return rc;
+    if (a.k % 256 == 0) {
+        // Many pairs: activation rows quantized in expert-sorted order, then CQ_MOE_CHUNK pairs of an expert per pass
+        // over its rows (the matvec body with 8 activation rows in LDS).
+        if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;
+        MoeChunks mc{chunks, chunks + 1, chunks + 1 + ws.max_chunks, chunks + 1 + 2 * ws.max_chunks, pout, pscale, (int)ws.max_chunks};
+        rc = cq_moe_chunks_launch(a.w_dtype, a.w, b + ws.act_off, ws.rows_alloc, a.out, mc, a.k, a.n, s);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
+    if ((rc = cq_quantize_act_launch(a.w_dtype, a.x, CQ_F32, b + ws.act_off, a.k, a.x_rows, s))) return rc;
     ActView av = cq_act_view(b + ws.act_off, a.w_dtype, a.k, a.x_rows);
     switch (a.w_dtype) {
         case CQ_Q4_0: return launch_moe_matvec<CQ_Q4_0>(a, av, offsets, pin, pout, pscale, s);
