@@ -48,7 +48,8 @@ SIGNATURES = {
     "cq_nn_attention": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp]),
     "cq_nn_attention_decode_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "cq_nn_attention_decode_splits": (_i64, [_i64]),
-    "cq_nn_attention_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp]),
+    "cq_nn_attention_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64,
+                                      _vp]),
     "cq_nn_silu_mul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "cq_nn_argmax": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
 }

@@ -316,8 +316,27 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
                                                                       const float *__restrict__ v_new, float *k_cache, float *v_cache,
                                                                       const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                                       float *__restrict__ part, const int32_t *__restrict__ pos_dev, int pos0,
-                                                                      int ctx, float scale, int splits) {
+                                                                      int ctx, float scale, int splits, const u32x4 *__restrict__ pf,
+                                                                      int64_t pf_chunks, uint32_t *__restrict__ pf_sink) {
     constexpr int NW = ATTD_WAVES;
+    if ((int)blockIdx.y >= splits) {
+        // Workgroups beyond the attention splits only read: they pull the weights the following kernels will stream
+        // (attention_wo, feed_forward_w1 / w3) through the memory-side cache while this latency-bound kernel leaves
+        // the HBM idle.  Nothing is computed from the data; the store below never executes for real weights.
+        const int64_t nthreads = (int64_t)gridDim.x * ((int)gridDim.y - splits) * (64 * NW);
+        int64_t i = ((int64_t)((int)blockIdx.y - splits) * gridDim.x + blockIdx.x) * (64 * NW) + threadIdx.x;
+        uint32_t acc = 0;
+        for (; i + 3 * nthreads < pf_chunks; i += 4 * nthreads) {
+            const u32x4 a = pf[i], b = pf[i + nthreads], c = pf[i + 2 * nthreads], d = pf[i + 3 * nthreads];
+            acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+        }
+        for (; i < pf_chunks; i += nthreads) {
+            const u32x4 a = pf[i];
+            acc ^= a.x ^ a.y ^ a.z ^ a.w;
+        }
+        if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
+        return;
+    }
     constexpr int DPL = HD / 64, EPL = HD / 16, IT = ATT_SPLIT / (4 * NW), VU = ATT_SPLIT / NW;
     __shared__ float sc[G * ATT_SPLIT];
     __shared__ float red[NW * G * HD];
@@ -706,8 +725,9 @@ int64_t cq_nn_attention_decode_splits(int64_t max_kv_len) {
 int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const float *v_new_dev, float *k_cache_dev, float *v_cache_dev,
                            const float *cos_dev, const float *sin_dev, float *out_dev, const int32_t *pos_dev, int64_t pos, int64_t n_head,
                            int64_t n_kv_head, int64_t head_dim, int64_t ctx, int64_t max_kv_len, float scale, void *partials_dev,
-                           int64_t partials_bytes, void *stream) {
+                           int64_t partials_bytes, const void *prefetch_dev, int64_t prefetch_bytes, void *stream) {
     if (n_head <= 0 || n_kv_head <= 0 || n_head % n_kv_head || ctx <= 0 || pos < 0 || max_kv_len <= 0 || max_kv_len > ctx) return CQ_ERR_SHAPE;
+    if (prefetch_bytes < 0 || (prefetch_bytes > 0 && (!prefetch_dev || misaligned(prefetch_dev, 16)))) return CQ_ERR_ALIGN;
     if (head_dim != 64 && head_dim != 128) return CQ_ERR_RANGE;
     if (!q_dev || !k_new_dev || !v_new_dev || !k_cache_dev || !v_cache_dev || !cos_dev || !sin_dev || !partials_dev) return CQ_ERR_NULL;
     if (misaligned(q_dev, 16) || misaligned(k_new_dev, 16) || misaligned(v_new_dev, 16) || misaligned(k_cache_dev, 16) ||
@@ -719,11 +739,19 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     if (splits > ATTD_MAX_SPLITS || ctx > 0x7fffffffLL) return CQ_ERR_RANGE;
     const int G = (int)(n_head / n_kv_head);
     float *part = (float *)partials_dev;
-    dim3 grid((unsigned)n_kv_head, (unsigned)splits);
+    // read-only workgroups for the prefetch range: enough, with the attention ones, for one per CU
+    const int64_t pf_chunks = prefetch_bytes / 16;
+    int64_t pf_rows = 0;
+    if (pf_chunks > 0) {
+        pf_rows = (256 - n_kv_head * splits + n_kv_head - 1) / n_kv_head;
+        if (pf_rows < 1) pf_rows = 1;
+    }
+    dim3 grid((unsigned)n_kv_head, (unsigned)(splits + pf_rows));
     hipStream_t s = (hipStream_t)stream;
 #define CQ_ATTD(HH, GG)                                                                                                                   \
     hipLaunchKernelGGL((attn_decode_kernel<HH, GG>), grid, dim3(64 * ATTD_WAVES), 0, s, q_dev, k_new_dev, v_new_dev, k_cache_dev, v_cache_dev, \
-                       cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits)
+                       cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits, (const u32x4 *)prefetch_dev, pf_chunks,   \
+                       (uint32_t *)nullptr)
     if (head_dim == 128) {
         switch (G) {
             case 1: CQ_ATTD(128, 1); break;

@@ -84,6 +84,7 @@ class LayerWeights:
         self.ffn_norm: Optional[torch.Tensor] = None
         self.k_cache: Optional[torch.Tensor] = None
         self.v_cache: Optional[torch.Tensor] = None
+        self.prefetch_span = 0       # bytes from attention_wo to the end of this layer's weights
 
 
 class ModelWeights:
@@ -105,6 +106,10 @@ class ModelWeights:
         self._graph = None
         self._graph_key = None
         self.fuse_decode = True      # single-token steps use the fused matvec prologues / epilogues
+        # bytes of the weights behind attention (wo, w1, w3, w2 are contiguous) that the attention launch's idle CUs
+        # would pull through the memory-side cache ahead of the kernels that stream them.  Measured on the 8B shape:
+        # no gain at 4-24 MB and a loss beyond (the time moves into the attention launch), so it is off.
+        self.prefetch_bytes = 0
 
     # ------------------------------------------------------------------------------------------ construction
     def _alloc(self, dtypes: Dict[str, GgmlDType]):
@@ -133,6 +138,8 @@ class ModelWeights:
                 self.layers[li].w[name] = w
         f32 = dict(dtype=torch.float32, device=self.device)
         for lw in self.layers:
+            w2 = lw.w["feed_forward_w2"]
+            lw.prefetch_span = (w2.ptr + w2.nbytes - lw.w["attention_wo"].ptr) // 16 * 16
             lw.k_cache = torch.zeros((cfg.n_kv_head, cfg.ctx, cfg.head_dim), **f32)
             lw.v_cache = torch.zeros((cfg.n_kv_head, cfg.ctx, cfg.head_dim), **f32)
         cos, sin = precomput_freqs_cis(cfg.head_dim, cfg.rope_theta, cfg.ctx)
@@ -338,7 +345,9 @@ class ModelWeights:
                                                                   self.cos.data_ptr(), self.sin.data_ptr(),
                                                                   None if merge_in_wo else att.data_ptr(), pos_dev_ptr, pos,
                                                                   cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
-                                                                  self.attd_ws.data_ptr(), self.attd_ws.numel(), sp))
+                                                                  self.attd_ws.data_ptr(), self.attd_ws.numel(),
+                                                                  wo.ptr if self.prefetch_bytes else None,
+                                                                  min(self.prefetch_bytes, lw.prefetch_span), sp))
             if merge_in_wo:
                 ck("cq_nn_qmatmul_residual_attn", L.cq_nn_qmatmul_residual_attn(int(wo.dtype), wo.ptr, self.attd_ws.data_ptr(),
                                                                                 L.cq_nn_attention_decode_splits(max_kv_len), cfg.head_dim,

@@ -66,13 +66,15 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
  * every head ([n_head][splits][head_dim + 4] floats, splits = cq_nn_attention_decode_splits(max_kv_len), at most 16,
  * i.e. max_kv_len <= 2048; -1 beyond).  When out_dev != NULL a second small kernel merges them into
  * out_dev [n_head*head_dim]; with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn.
+ * prefetch_dev / prefetch_bytes (optional, 16-byte aligned): a byte range that extra read-only workgroups of this
+ * otherwise latency-bound launch pull through the memory-side cache, e.g. the weights of the kernels that follow.
  * No counterpart in the reference, which runs these as separate tensor ops (quantized_llama.rs:217-261). */
 int64_t cq_nn_attention_decode_workspace_bytes(int64_t n_head, int64_t head_dim, int64_t max_kv_len);
 int64_t cq_nn_attention_decode_splits(int64_t max_kv_len);
 int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const float *v_new_dev, float *k_cache_dev, float *v_cache_dev,
                            const float *cos_dev, const float *sin_dev, float *out_dev, const int32_t *pos_dev, int64_t pos, int64_t n_head,
                            int64_t n_kv_head, int64_t head_dim, int64_t ctx, int64_t max_kv_len, float scale, void *partials_dev,
-                           int64_t partials_bytes, void *stream);
+                           int64_t partials_bytes, const void *prefetch_dev, int64_t prefetch_bytes, void *stream);
 
 /* out = silu(gate) * up with silu(v) = v / (1 + exp(-v)): Mlp::forward, quantized_llama.rs:56-63
  * (candle_nn::ops::silu, candle-core/src/op.rs Silu::f32).  gate/up rows may be strided views of one buffer. */

@@ -164,9 +164,12 @@ def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
     want = attention_oracle(want_q, kc_ref, vc_ref, pos, H, KV, D)
     for attempt in range(2):
         kc, vc, out = dev(kc0), dev(vc0), torch.zeros((1, H * D), device="cuda")
+        # second attempt: the launch also carries read-only workgroups over a 5 MB range (ragged: not a multiple of the stride)
+        pf = torch.zeros(5 * 1024 * 1024 + 48, dtype=torch.uint8, device="cuda") if attempt else None
         ok(lib.cq_nn_attention_decode(dev(q).data_ptr(), dev(k).data_ptr(), dev(v).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(),
                                       dev(sin).data_ptr(), out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv,
-                                      float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None))
+                                      float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, pf.data_ptr() if attempt else None,
+                                      pf.numel() if attempt else 0, None))
         torch.cuda.synchronize()
         assert rel_l2(out.cpu().numpy(), want) <= TOL, attempt
         assert np.allclose(kc.cpu().numpy()[:, pos], want_k[:, 0], rtol=1e-6, atol=1e-6)
@@ -190,7 +193,7 @@ def test_attention_merge_as_matvec_prologue(dtype, pos, max_kv):
     ws = torch.zeros(wsb, dtype=torch.uint8, device="cuda")
     att = torch.empty((1, k), device="cuda")
     args = (dev(q).data_ptr(), dev(kn).data_ptr(), dev(vn).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(), dev(sin).data_ptr())
-    tail = (None, pos, H, KV, D, ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None)
+    tail = (None, pos, H, KV, D, ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None, 0, None)
     ok(lib.cq_nn_attention_decode(*args, att.data_ptr(), *tail))
     res0 = normal(46, (1, hidden), 1.0)
     r1, r2 = dev(res0), dev(res0)
