@@ -736,8 +736,14 @@ int launch_pair(const void *wa, int64_t na, float *dsta, const void *wb, int64_t
     int waves = 0;
     int rc = na >= nb ? make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, 0, lds_a) : make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, 0, lds_b);
     if (rc) return rc;
-    if ((rc = make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, 0, lds_a))) return rc;
-    if ((rc = make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, 0, lds_b))) return rc;
+    // 256 workgroups in total (one per CU: a 16-wave workgroup fills a CU's registers, so a 257th would wait for a
+    // whole workgroup to finish), shared between the tensors in proportion to their bytes
+    const double bytes_a = (double)na * BlockInfo<DTA>::bytes / BlockInfo<DTA>::elems, bytes_b = (double)nb * BlockInfo<DTB>::bytes / BlockInfo<DTB>::elems;
+    int64_t share_a = (int64_t)(256.0 * bytes_a / (bytes_a + bytes_b) + 0.5);
+    if (share_a < 1) share_a = 1;
+    if (share_a > 255) share_a = 255;
+    if ((rc = make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, 0, lds_a, share_a))) return rc;
+    if ((rc = make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, 0, lds_b, 256 - share_a))) return rc;
     const size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
     const bool single = k / 64 <= 64;                     // every K-quant unit is 64 elements
     if (lds_bytes > 48 * 1024) {
