@@ -25,6 +25,7 @@ The JSON line carries, besides the driver contract fields:
                                    the prefill matmul (other BASELINE configurations; not the headline line):
                                    TFLOP/s of QMatMul::forward and of its MFMA kernel against the 2.5 PFLOP/s
                                    dense f16 peak
+    python bench.py --workload moe    the Qwen3-30B-A3B-shaped expert matmuls of one MoE layer at 1 / 16 / 256 tokens
     python bench.py --workload decode8b [--steps 256] [--prompt 512]
                                    the 8B-shape Q4_K_M decoder: prompt and decode tok/s against the weight-streaming
                                    roofline (8 TB/s / weight bytes per token)
@@ -176,12 +177,82 @@ def decode8b(args):
     return out
 
 
+def moe(args):
+    """BASELINE configs[4]: Qwen3-30B-A3B-shaped MoE layer (128 experts, top-8, hidden 2048, expert FFN 768, Q4_K):
+    the three expert matmuls of one layer (gate, up on [tokens, hidden]; down on [tokens*8, ffn]) through
+    QTensor::indexed_moe_forward, rotated over several distinct layers, for 1 / 16 / 256 tokens."""
+    import torch
+
+    from candle_amd import _lib
+
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    E, H, F, TOPK, NL = 128, 2048, 768, 8, 6
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+
+    def experts(n, k):
+        nb = L.cq_storage_bytes(Q4K, E * n * k)
+        w = torch.empty(nb, dtype=torch.uint8, device=dev)
+        for e in range(E):
+            wf = torch.randn((n, k), generator=gen, device=dev) * 0.02
+            _lib.check("cq_quantize", L.cq_quantize(Q4K, wf.data_ptr(), w.data_ptr() + e * (nb // E), n * k, None))
+        torch.cuda.synchronize()
+        return w
+
+    gate, up, down = [experts(F, H) for _ in range(NL)], [experts(F, H) for _ in range(NL)], [experts(H, F) for _ in range(NL)]
+    router = torch.randn((E, H), generator=gen, device=dev)
+    results = []
+    for tokens in (1, 16, 256):
+        x = torch.randn((tokens, H), generator=gen, device=dev)
+        _, ids = torch.topk(torch.softmax(x @ router.t(), -1), TOPK, dim=-1)
+        ids32 = ids.to(torch.int32).contiguous()
+        distinct = int(torch.unique(ids).numel())
+        xg = x.reshape(tokens, 1, H).contiguous()
+        h = torch.randn((tokens, TOPK, F), generator=gen, device=dev)
+        o1, o2 = torch.empty((tokens, TOPK, F), device=dev), torch.empty((tokens, TOPK, F), device=dev)
+        o3 = torch.empty((tokens, TOPK, H), device=dev)
+        nws = max(L.cq_indexed_moe_workspace_bytes(Q4K, E, F, H, tokens, TOPK, 1), L.cq_indexed_moe_workspace_bytes(Q4K, E, H, F, tokens, TOPK, TOPK))
+        ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+
+        def layer(i, sp):
+            for w, src, dst, n, k, d1 in ((gate[i % NL], xg, o1, F, H, 1), (up[i % NL], xg, o2, F, H, 1), (down[i % NL], h, o3, H, F, TOPK)):
+                _lib.check("cq_indexed_moe_forward", L.cq_indexed_moe_forward(Q4K, w.data_ptr(), src.data_ptr(), ids32.data_ptr(), dst.data_ptr(),
+                                                                              E, n, k, tokens, TOPK, d1, ws.data_ptr(), nws, sp))
+
+        st = torch.cuda.Stream(device=dev)
+        with torch.cuda.stream(st):
+            layer(0, st.cuda_stream)
+            st.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=st):
+                for i in range(NL):
+                    layer(i, torch.cuda.current_stream().cuda_stream)
+            g.replay()
+            st.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 20
+            e0.record(st)
+            for _ in range(reps):
+                g.replay()
+            e1.record(st)
+            st.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * NL)
+        alg = distinct * 3 * 884736
+        results.append({"tokens": tokens, "distinct_experts": distinct, "layer_us": round(us, 1), "algorithmic_MB": round(alg / 1e6, 1),
+                        "GBps": round(alg / us / 1e3, 1), "tok_s_48_layers_expert_matmuls_only": round(tokens / (48 * us * 1e-6), 1)})
+    print(json.dumps({"metric": "Qwen3-30B-A3B-shape MoE layer, expert matmuls (Q4_K, 128 experts, top-8)", "unit": "us per layer", "n_gpus": 1,
+                      "data": "synthetic", "config": {"workload": "gate + up [tokens, 2048] -> 768 and down [tokens*8, 768] -> 2048 via indexed_moe_forward, "
+                                                                  "6 distinct layers rotated (2 GB), HIP graph"},
+                      "results": results}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", choices=["decode", "prefill", "decode8b"], default="decode")
+    ap.add_argument("--workload", choices=["decode", "prefill", "decode8b", "moe"], default="decode")
     ap.add_argument("--layers", type=int, default=32, help="--workload decode8b: number of decoder layers")
     ap.add_argument("--prompt", type=int, default=512, help="--workload decode8b: prompt tokens")
     ap.add_argument("--wdtype", choices=sorted(WDTYPES), default="q4k", help="weight format of --workload prefill")
@@ -199,6 +270,8 @@ def main():
     if args.workload == "decode8b":
         print(json.dumps(decode8b(args)))
         return
+    if args.workload == "moe":
+        return moe(args)
     if args.steps is None:
         args.steps = 4000 if args.workload == "decode" else 50
     if args.warmup is None:
