@@ -102,3 +102,8 @@ struct MoeChunks {
 };
 int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k,
                          int64_t n, hipStream_t s);
+
+// Pairs from which a K-quant MoE call goes through the MFMA kernel (tiles of up to 128 expert-sorted rows).
+#define CQ_MOE_MFMA_MIN_PAIRS 1024
+int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k, int64_t n,
+                         hipStream_t s);

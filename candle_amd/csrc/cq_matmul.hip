@@ -274,9 +274,11 @@ __device__ __forceinline__ void lds_write32h(_Float16 *dstrow, const uint32_t v[
 
 // NJ = 32-column MFMA tiles per wave: block tile 128 x (64 * NJ).  NJ = 1 halves the accumulators so that two
 // workgroups share a CU and one converts operands while the other feeds the matrix cores.
-template <int DT, int NJ>
+// MOE: blockIdx.x is a tile of the chunk table: up to 128 expert-sorted activation rows [first, first + count) of
+// expert e; the weights are that expert's [n, k] matrix and output rows are scattered through pair_out with pair_scale.
+template <int DT, int NJ, bool MOE = false>
 __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k,
-                                                                     int n, int rows, int64_t stride_dst) {
+                                                                     int n, int rows, int64_t stride_dst, MoeChunks mc, int64_t expert_bytes) {
     typedef Stage<DT> S;
     constexpr bool KQ = S::KQ;
     constexpr int BN = 64 * NJ, WN = 32 * NJ;
@@ -289,7 +291,14 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = wv >> 1, wn = wv & 1;
-    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    int m0 = blockIdx.x * BM;
+    const int n0 = blockIdx.y * BN;
+    if (MOE) {
+        if ((int)blockIdx.x >= mc.n_chunks[0]) return;           // uniform over the workgroup
+        m0 = mc.first[blockIdx.x];
+        rows = m0 + mc.count[blockIdx.x];
+        w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
+    }
     const bool bstage = tid < 2 * BN;                            // threads that also stage a weight row (wave-uniform)
     const int nsb = k >> 8;                                     // 256-element spans
     const int64_t row_bytes = (int64_t)(k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
@@ -461,7 +470,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
             for (int e = 0; e < 16; e++) {
                 const int mm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                 float v = KQ ? acc[i][j][e] : sb[i][j][e];
-                if (mm < rows && nn < n) dst[(int64_t)mm * stride_dst + nn] = v;
+                if (mm < rows && nn < n) {
+                    if (MOE) dst[(int64_t)mc.pair_out[mm] * stride_dst + nn] = v * mc.pair_scale[mm];
+                    else dst[(int64_t)mm * stride_dst + nn] = v;
+                }
             }
         }
 }
@@ -474,10 +486,13 @@ int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t 
     const int bn = wide ? 128 : 64;
     dim3 grid((unsigned)((rows + BM - 1) / BM), (unsigned)((n + bn - 1) / bn));
     if (grid.y > 65535) return CQ_ERR_RANGE;
+    const MoeChunks none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (wide)
-        hipLaunchKernelGGL((qmm_kernel<DT, 2>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst);
+        hipLaunchKernelGGL((qmm_kernel<DT, 2>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst, none,
+                           (int64_t)0);
     else
-        hipLaunchKernelGGL((qmm_kernel<DT, 1>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst);
+        hipLaunchKernelGGL((qmm_kernel<DT, 1>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst, none,
+                           (int64_t)0);
     return (int)hipGetLastError();
 }
 
@@ -503,6 +518,31 @@ int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t co
     if (grid > 0x7fffffffLL) return CQ_ERR_RANGE;
     hipLaunchKernelGGL(convert_f32_kernel, dim3((unsigned)grid), dim3(256), 0, s, src, dst, dst_dtype, count);
     return (int)hipGetLastError();
+}
+
+namespace {
+template <int DT>
+int launch_qmm_moe(const void *w, const ActView &av, float *out, const MoeChunks &mc, int64_t k, int64_t n, hipStream_t s) {
+    dim3 grid((unsigned)mc.max_chunks, (unsigned)((n + 63) / 64));
+    if (grid.y > 65535) return CQ_ERR_RANGE;
+    const int64_t expert_bytes = n * (k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
+    hipLaunchKernelGGL((qmm_kernel<DT, 1, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc, expert_bytes);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k, int64_t n,
+                         hipStream_t s) {
+    if (mc.max_chunks == 0 || n == 0) return CQ_OK;
+    if (k % 256) return CQ_ERR_SHAPE;
+    ActView av = cq_act_view(scratch, w_dtype, k, rows_alloc);
+    switch (w_dtype) {
+        case CQ_Q4K: return launch_qmm_moe<CQ_Q4K>(w, av, out, mc, k, n, s);
+        case CQ_Q5K: return launch_qmm_moe<CQ_Q5K>(w, av, out, mc, k, n, s);
+        case CQ_Q6K: return launch_qmm_moe<CQ_Q6K>(w, av, out, mc, k, n, s);
+    }
+    return CQ_ERR_DTYPE;
 }
 
 // k is a multiple of 256 for the MFMA kernel (always true for K-quants); Q4_0 / Q8_0 rows whose length

@@ -45,7 +45,7 @@ inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pa
 __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__restrict__ offsets, int *__restrict__ cursor,
                                                          int *__restrict__ pair_in, int *__restrict__ pair_out,
                                                          float *__restrict__ pair_scale, float *__restrict__ out, int n, int *__restrict__ chunks,
-                                                         int max_chunks) {
+                                                         int max_chunks, int chunk) {
     __shared__ int carry;
     const int tid = threadIdx.x;
     const int E = ps.num_experts;
@@ -86,16 +86,16 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
     // positions behind the last valid pair are never part of a chunk, but the gathering quantizer walks all n_pairs
     // rows: give them a valid source row
     for (int p = carry + tid; p < ps.n_pairs; p += 1024) pair_in[p] = 0;
-    // chunk table: expert e's segment in pieces of CQ_MOE_CHUNK pairs (any order: chunks are independent)
+    // chunk table: expert e's segment in pieces of `chunk` pairs (any order: chunks are independent)
     for (int e = tid; e < E; e += 1024) {
         const int seg0 = offsets[e], cnt = offsets[e + 1] - seg0;     // offsets[e + 1] of the last sweep's neighbour is final here
-        const int cc = (cnt + CQ_MOE_CHUNK - 1) / CQ_MOE_CHUNK;
+        const int cc = (cnt + chunk - 1) / chunk;
         if (cc > 0) {
             const int base = atomicAdd(&chunks[0], cc);
             for (int i = 0; i < cc; i++) {
                 chunks[1 + base + i] = e;
-                chunks[1 + max_chunks + base + i] = seg0 + i * CQ_MOE_CHUNK;
-                chunks[1 + 2 * max_chunks + base + i] = min(CQ_MOE_CHUNK, cnt - i * CQ_MOE_CHUNK);
+                chunks[1 + max_chunks + base + i] = seg0 + i * chunk;
+                chunks[1 + 2 * max_chunks + base + i] = min(chunk, cnt - i * chunk);
             }
         }
     }
@@ -208,9 +208,17 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     int *pin = (int *)(b + ws.pin_off), *pout = (int *)(b + ws.pout_off);
     float *pscale = (float *)(b + ws.pscale_off);
     int *chunks = (int *)(b + ws.chunk_off);
+    // Hundreds of pairs per call on K-quant experts: the expert-sorted rows go through the MFMA prefill kernel in tiles
+    // of up to 128 rows of one expert (integer-exact like the other K-quant paths).  Otherwise 8 pairs per matvec pass.
+    const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
-                       (int)ws.max_chunks);
+                       (int)ws.max_chunks, mfma ? 128 : CQ_MOE_CHUNK);
     if ((rc = (int)hipGetLastError())) return rc;
+    if (mfma) {
+        if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;
+        MoeChunks mc{chunks, chunks + 1, chunks + 1 + ws.max_chunks, chunks + 1 + 2 * ws.max_chunks, pout, pscale, (int)ws.max_chunks};
+        return cq_matmul_moe_launch(a.w_dtype, a.w, b + ws.act_off, ws.rows_alloc, a.out, mc, a.k, a.n, s);
+    }
     if (a.k % 256 == 0) {
         // Many pairs: activation rows quantized in expert-sorted order, then CQ_MOE_CHUNK pairs of an expert per pass
         // over its rows (the matvec body with 8 activation rows in LDS).

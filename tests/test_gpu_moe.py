@@ -57,7 +57,8 @@ def test_indexed_moe_forward(dtype, input_dim1_is_one):
 
 
 @pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
-@pytest.mark.parametrize("tokens", [1, 16, 40, 100])      # up to 256 pairs: one fused matvec per pair; beyond: grouped by expert
+@pytest.mark.parametrize("tokens", [1, 16, 40, 100, 300])  # <= 256 pairs: a fused matvec per pair; beyond: grouped by expert, 8 pairs per
+                                                           # pass; from 1024 pairs on K-quants: expert tiles through the MFMA kernel
 @pytest.mark.parametrize("is_prefill", [False, True])
 def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     """The two call shapes of FusedMoeGGUF::forward (fused_moe.rs:263-294): gate/up without
@@ -86,7 +87,7 @@ def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     assert err2 <= TOL and err2 <= TIGHT, err2
 
 
-@pytest.mark.parametrize("batch", [4, 120])                 # 12 pairs (per-pair kernels) and 360 pairs (grouped path)
+@pytest.mark.parametrize("batch", [4, 120, 400])            # 12 pairs (per-pair kernels), 360 (grouped matvec), 1200 (MFMA tiles)
 def test_indexed_moe_forward_out_of_range_id_gives_zero_row(batch):
     import candle_amd as ca
     E, n, k, topk = 8, 48, 512, 3
