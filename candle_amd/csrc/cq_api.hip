@@ -165,7 +165,12 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     if (workspace_bytes < cq_qmatmul_workspace_bytes(w_dtype, m, k, n)) return CQ_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     // decode: one kernel quantizes the activations into LDS and streams W (no scratch traffic)
-    if (m <= CQ_MATVEC_MAX_ROWS) return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
+    if (m <= 2) return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
+    // 3..8 rows: every workgroup re-quantizing all rows costs more than one small kernel that does it once
+    if (m <= CQ_MATVEC_MAX_ROWS) {
+        if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
+        return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, dst_dtype, k, n, m, n, s);
+    }
     if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
     if (dst_dtype == CQ_F32)
         return cq_matmul_launch(w_dtype, w_dev, workspace_dev, (float *)dst_dev, k, n, m, n, s);
