@@ -148,8 +148,13 @@ int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float
 int64_t cq_qmatmul_workspace_bytes(int w_dtype, int64_t m, int64_t k, int64_t n) {
     if (check_mm_shape(w_dtype, k, n, m)) return -1;
     int64_t bytes = cq_act_layout(w_dtype, k, m).total;
-    // the MFMA path writes f32 and converts afterwards when the caller wants f16 / bf16
-    if (m > CQ_MATVEC_MAX_ROWS) bytes += cq_align256(m * n * 4);
+    // the MFMA path writes f32 and converts afterwards when the caller wants f16 / bf16; small grids split K into
+    // partial planes that a second kernel adds up
+    if (m > CQ_MATVEC_MAX_ROWS) {
+        bytes += cq_align256(m * n * 4);
+        const int sp = cq_qmm_splits(k, n, m);
+        if (sp > 1) bytes += cq_align256((int64_t)sp * m * n * 4);
+    }
     return bytes;
 }
 
@@ -172,10 +177,11 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
         return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, dst_dtype, k, n, m, n, s);
     }
     if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
-    if (dst_dtype == CQ_F32)
-        return cq_matmul_launch(w_dtype, w_dev, workspace_dev, (float *)dst_dev, k, n, m, n, s);
     float *tmp = (float *)((uint8_t *)workspace_dev + cq_act_layout(w_dtype, k, m).total);
-    if ((rc = cq_matmul_launch(w_dtype, w_dev, workspace_dev, tmp, k, n, m, n, s))) return rc;
+    float *split_ws = cq_qmm_splits(k, n, m) > 1 ? (float *)((uint8_t *)tmp + cq_align256(m * n * 4)) : nullptr;
+    if (dst_dtype == CQ_F32)
+        return cq_matmul_launch(w_dtype, w_dev, workspace_dev, (float *)dst_dev, k, n, m, n, s, split_ws);
+    if ((rc = cq_matmul_launch(w_dtype, w_dev, workspace_dev, tmp, k, n, m, n, s, split_ws))) return rc;
     return cq_convert_f32_launch(tmp, dst_dev, dst_dtype, m * n, s);
 }
 

@@ -25,8 +25,10 @@ int cq_matvec_norm_swiglu_launch(int w_dtype, const void *w1, const void *w3, co
                                  float eps, float *dst, int64_t k, int64_t ffn, hipStream_t s);
 int cq_matvec_norm_pair_launch(int dta, const void *wa, int64_t na, float *dsta, int dtb, const void *wb, int64_t nb, float *dstb, const float *x,
                                const float *partials, const float *norm_weight, float eps, int64_t k, hipStream_t s);
+// split_ws: optional workspace of cq_qmm_splits(k, n, rows) * rows * n floats for split-K partial planes (NULL: no split)
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
-                     int64_t stride_dst, hipStream_t s);
+                     int64_t stride_dst, hipStream_t s, float *split_ws = nullptr);
+int cq_qmm_splits(int64_t k, int64_t n, int64_t rows);
 int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t count, hipStream_t s);
 
 // ---- MoE: both public entry points reduce to "pairs" (expert, activation row, output row, scale) ----

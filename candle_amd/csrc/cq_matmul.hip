@@ -278,7 +278,8 @@ __device__ __forceinline__ void lds_write32h(_Float16 *dstrow, const uint32_t v[
 // expert e; the weights are that expert's [n, k] matrix and output rows are scattered through pair_out with pair_scale.
 template <int DT, int NJ, bool MOE = false>
 __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k,
-                                                                     int n, int rows, int64_t stride_dst, MoeChunks mc, int64_t expert_bytes) {
+                                                                     int n, int rows, int64_t stride_dst, MoeChunks mc, int64_t expert_bytes,
+                                                                     int64_t split_stride) {
     typedef Stage<DT> S;
     constexpr bool KQ = S::KQ;
     constexpr int BN = 64 * NJ, WN = 32 * NJ;
@@ -300,7 +301,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
     }
     const bool bstage = tid < 2 * BN;                            // threads that also stage a weight row (wave-uniform)
-    const int nsb = k >> 8;                                     // 256-element spans
+    // split-K: blockIdx.z takes an equal share of the 256-element spans and writes its own partial plane
+    const int nsb_all = k >> 8;
+    const int kb0 = (int)(((int64_t)nsb_all * blockIdx.z) / gridDim.z), nsb = (int)(((int64_t)nsb_all * (blockIdx.z + 1)) / gridDim.z);
+    dst += (int64_t)blockIdx.z * split_stride;
     const int64_t row_bytes = (int64_t)(k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
 
     // staging role of this thread: (row r_l of the tile, 32-element half)
@@ -329,10 +333,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         x0 = *reinterpret_cast<const u32x4 *>(q);
         x1 = *reinterpret_cast<const u32x4 *>(q + 16);
     };
-    load_stage(0, 0, wraw2[0], a02[0], a12[0]);
-    load_stage(0, 1, wraw2[1], a02[1], a12[1]);
+    load_stage(kb0, 0, wraw2[0], a02[0], a12[0]);
+    load_stage(kb0, 1, wraw2[1], a02[1], a12[1]);
 
-    for (int kb = 0; kb < nsb; kb++) {
+    for (int kb = kb0; kb < nsb; kb++) {
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             typename S::Raw &wraw = wraw2[g & 1];
@@ -478,21 +482,46 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         }
 }
 
+// dst[m, n] = sum over the split planes, in split order (deterministic); n % 4 == 0 whenever split-K is chosen
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ part, float *__restrict__ dst, int splits, int64_t n,
+                                                            int64_t stride_dst, int64_t count) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= count) return;
+    f32x4 a = *reinterpret_cast<const f32x4 *>(part + i);
+    for (int sI = 1; sI < splits; sI++) {
+        const f32x4 b = *reinterpret_cast<const f32x4 *>(part + sI * count + i);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    const int64_t r = i / n, c = i - r * n;
+    float *o = dst + r * stride_dst + c;
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+
 template <int DT>
-int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s,
+               float *split_ws) {
     // 128 x 64 tiles (two or three workgroups per CU) everywhere except long Q4_0 / Q8_0 problems, whose cheaper
     // operand conversion leaves the 128 x 128 tile (one workgroup per CU, half the activation conversions) ahead
     const bool wide = !Stage<DT>::KQ && rows >= 1024;
     const int bn = wide ? 128 : 64;
-    dim3 grid((unsigned)((rows + BM - 1) / BM), (unsigned)((n + bn - 1) / bn));
+    const int splits = split_ws ? cq_qmm_splits(k, n, rows) : 1;
+    dim3 grid((unsigned)((rows + BM - 1) / BM), (unsigned)((n + bn - 1) / bn), (unsigned)splits);
     if (grid.y > 65535) return CQ_ERR_RANGE;
     const MoeChunks none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    // with split-K every split writes a contiguous [rows, n] plane of the workspace; a second kernel adds them in order
+    float *out = splits > 1 ? split_ws : dst;
+    const int64_t ld = splits > 1 ? n : stride_dst, plane = splits > 1 ? rows * n : 0;
     if (wide)
-        hipLaunchKernelGGL((qmm_kernel<DT, 2>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst, none,
-                           (int64_t)0);
+        hipLaunchKernelGGL((qmm_kernel<DT, 2>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none, (int64_t)0,
+                           plane);
     else
-        hipLaunchKernelGGL((qmm_kernel<DT, 1>), grid, dim3(256), 0, s, (const uint8_t *)w, av, dst, (int)k, (int)n, (int)rows, stride_dst, none,
-                           (int64_t)0);
+        hipLaunchKernelGGL((qmm_kernel<DT, 1>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none, (int64_t)0,
+                           plane);
+    int rc = (int)hipGetLastError();
+    if (rc || splits == 1) return rc;
+    const int64_t count = rows * n;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((count / 4 + 255) / 256)), dim3(256), 0, s, (const float *)split_ws, dst, splits, n,
+                       stride_dst, count);
     return (int)hipGetLastError();
 }
 
@@ -526,7 +555,8 @@ int launch_qmm_moe(const void *w, const ActView &av, float *out, const MoeChunks
     dim3 grid((unsigned)mc.max_chunks, (unsigned)((n + 63) / 64));
     if (grid.y > 65535) return CQ_ERR_RANGE;
     const int64_t expert_bytes = n * (k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
-    hipLaunchKernelGGL((qmm_kernel<DT, 1, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc, expert_bytes);
+    hipLaunchKernelGGL((qmm_kernel<DT, 1, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc, expert_bytes,
+                       (int64_t)0);
     return (int)hipGetLastError();
 }
 
@@ -547,16 +577,27 @@ int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_
 
 // k is a multiple of 256 for the MFMA kernel (always true for K-quants); Q4_0 / Q8_0 rows whose length
 // is only a multiple of 32, and very small problems, go through the row-chunked matvec instead.
+// Small grids (few activation rows or few weight rows) split K so that about 256 workgroups exist.  1 = no split.
+int cq_qmm_splits(int64_t k, int64_t n, int64_t rows) {
+    if (k % 256 || n % 4 || rows <= CQ_MATVEC_MAX_ROWS) return 1;
+    const int64_t base = ((rows + BM - 1) / BM) * ((n + 63) / 64), nsb = k / 256;
+    if (base >= 192 || nsb < 8) return 1;
+    int64_t sp = (256 + base - 1) / base;
+    if (sp > 8) sp = 8;
+    if (sp > nsb / 4) sp = nsb / 4;
+    return sp < 2 ? 1 : (int)sp;
+}
+
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
-                     int64_t stride_dst, hipStream_t s) {
+                     int64_t stride_dst, hipStream_t s, float *split_ws) {
     ActView av = cq_act_view(scratch, w_dtype, k, rows);
     if (k % 256 == 0 && rows > CQ_MATVEC_MAX_ROWS) {
         switch (w_dtype) {
-            case CQ_Q4_0: return launch_qmm<CQ_Q4_0>(w, av, dst, k, n, rows, stride_dst, s);
-            case CQ_Q8_0: return launch_qmm<CQ_Q8_0>(w, av, dst, k, n, rows, stride_dst, s);
-            case CQ_Q4K: return launch_qmm<CQ_Q4K>(w, av, dst, k, n, rows, stride_dst, s);
-            case CQ_Q5K: return launch_qmm<CQ_Q5K>(w, av, dst, k, n, rows, stride_dst, s);
-            case CQ_Q6K: return launch_qmm<CQ_Q6K>(w, av, dst, k, n, rows, stride_dst, s);
+            case CQ_Q4_0: return launch_qmm<CQ_Q4_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q8_0: return launch_qmm<CQ_Q8_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q4K: return launch_qmm<CQ_Q4K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q5K: return launch_qmm<CQ_Q5K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q6K: return launch_qmm<CQ_Q6K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
         }
         return CQ_ERR_DTYPE;
     }
