@@ -102,17 +102,20 @@ int cq_matvec(int w_dtype, const void *w_dev, const void *act_scratch_dev, void 
               int64_t k, int64_t n, int64_t rows, int64_t stride_dst, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
- * Prefill matmul over pre-quantized activations (any rows >= 1), MFMA tiles with the dequantized
- * weight tile staged in LDS.  Counterpart of launch_mmq_gguf_<t> (candle-core/src/quantized/
- * fast_mmq.rs:71-111, candle-kernels/src/mmq_gguf/).  Same buffers as cq_matvec; dst is f32.
+ * Prefill matmul over pre-quantized activations (any rows >= 1): more than CQ_MATVEC_MAX_ROWS rows with k a
+ * multiple of 256 run on the f16 matrix cores with the converted operand tiles staged in LDS (K-quant operands are
+ * exact integers there, Q4_0 / Q8_0 operands are rounded to f16); other shapes take 8 rows per matvec pass.
+ * Counterpart of launch_mmq_gguf_<t> (candle-core/src/quantized/fast_mmq.rs:71-111, candle-kernels/src/mmq_gguf/).
+ * Same buffers as cq_matvec; dst is f32.
  * ------------------------------------------------------------------------------------------- */
 int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float *dst_dev,
               int64_t k, int64_t n, int64_t rows, int64_t stride_dst, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * QCudaStorage::fwd (cuda.rs:846-878), the body of CustomOp1::cuda_fwd for QTensor
- * (mod.rs:1007-1017): quantize the m activation rows, then matvec (m <= CQ_MATVEC_MAX_ROWS) or
- * MFMA matmul.  x is [m, k] contiguous (f32 / f16 / bf16), dst is [m, n] contiguous in dst_dtype
+ * (mod.rs:1007-1017): quantize the m activation rows, then matvec (m <= CQ_MATVEC_MAX_ROWS; for m <= 2 the
+ * quantization happens inside the matvec kernel) or MFMA matmul (split over k with an ordered reduction when the
+ * grid would be small).  x is [m, k] contiguous (f32 / f16 / bf16), dst is [m, n] contiguous in dst_dtype
  * (CUDA keeps the input dtype: fast_mmvq.rs:161-323).  workspace_dev: 256-byte aligned,
  * at least cq_qmatmul_workspace_bytes(w_dtype, m, k, n) bytes.
  * ------------------------------------------------------------------------------------------- */
@@ -126,7 +129,8 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
  *   w [num_experts, n, k] blocks, x [batch, input_dim1, k] f32 with input_dim1 == topk or 1,
  *   ids [batch, topk] u32  ->  out [batch, topk, n] f32,
  *   out[b, t, :] = W[ids[b, t]] . x[b, input_dim1 == 1 ? 0 : t, :].
- * Pairs are grouped by expert on the device so each expert's rows are streamed once per call.
+ * Up to 256 pairs each pair is its own fused matvec; beyond, pairs are grouped by expert on the device and an expert's
+ * rows are streamed once per 8 pairs (from 1024 pairs on K-quant experts: once per 128 pairs, on the matrix cores).
  * An id >= num_experts leaves its output row zero-filled.
  * ------------------------------------------------------------------------------------------- */
 int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk, int64_t input_dim1);
