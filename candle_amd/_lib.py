@@ -41,6 +41,12 @@ SIGNATURES = {
     "cq_nn_qmatmul_residual": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "cq_nn_qmatmul_norm_swiglu": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
     "cq_nn_qmatmul_norm_pair": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _vp, _vp, _vp, _vp, _f32, _i64, _vp]),
+    "cq_nn_qmatmul_split_planes": (_i64, [_int, _i64]),
+    "cq_nn_qmatmul_split": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "cq_nn_qmatmul_norm_merge": (_int, [_int, _vp, _vp, _vp, _i64, _vp, _f32, _vp, _i64, _i64, _vp]),
+    "cq_nn_qmatmul_norm_pair_merge": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _f32, _i64, _vp]),
+    "cq_nn_qmatmul_residual_merge": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "cq_nn_qmatmul_residual_attn_merge": (_int, [_int, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "cq_nn_qmatmul_residual_attn": (_int, [_int, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp]),
     "cq_nn_rms_norm": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "cq_nn_rope_i_kv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),

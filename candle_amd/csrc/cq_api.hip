@@ -262,15 +262,23 @@ int cq_nn_qmatmul_norm(int w_dtype, const void *w_dev, const float *x_dev, const
     return cq_matvec_norm_launch(w_dtype, w_dev, x_dev, sumsq_partials_dev, norm_weight_dev, eps, dst_dev, k, n, (hipStream_t)stream);
 }
 
-int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
-                           float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream) {
+int cq_nn_qmatmul_residual_merge(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
+                                 float *sumsq_partials_out_dev, const float *planes_dev, int64_t n_planes, int64_t k, int64_t n, void *stream) {
     int rc = check_mm_shape(w_dtype, k, n, 1);
     if (rc) return rc;
+    if (n_planes < 0 || n_planes > CQ_NN_MAX_PLANES) return CQ_ERR_RANGE;
     if (n == 0) return CQ_OK;
     if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
-    if (!x_dev || !residual_dev || !sumsq_partials_out_dev) return CQ_ERR_NULL;
-    if (!aligned(x_dev, 16) || !aligned(up_dev, 16) || !aligned(residual_dev, 4) || !aligned(sumsq_partials_out_dev, 4)) return CQ_ERR_ALIGN;
-    return cq_matvec_residual_launch(w_dtype, w_dev, x_dev, up_dev, residual_dev, sumsq_partials_out_dev, k, n, (hipStream_t)stream);
+    if (!x_dev || !residual_dev || !sumsq_partials_out_dev || (n_planes > 0 && !planes_dev)) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(up_dev, 16) || !aligned(residual_dev, 4) || !aligned(sumsq_partials_out_dev, 4) || !aligned(planes_dev, 4))
+        return CQ_ERR_ALIGN;
+    return cq_matvec_residual_launch(w_dtype, w_dev, x_dev, up_dev, residual_dev, sumsq_partials_out_dev, planes_dev, n_planes, k, n,
+                                     (hipStream_t)stream);
+}
+
+int cq_nn_qmatmul_residual(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
+                           float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream) {
+    return cq_nn_qmatmul_residual_merge(w_dtype, w_dev, x_dev, up_dev, residual_dev, sumsq_partials_out_dev, nullptr, 0, k, n, stream);
 }
 
 int cq_nn_qmatmul_norm_swiglu(int w_dtype, const void *w1_dev, const void *w3_dev, const float *x_dev, const float *sumsq_partials_dev,
@@ -298,16 +306,65 @@ int cq_nn_qmatmul_norm_pair(int w_dtype_a, const void *w_a_dev, int64_t n_a, flo
                                       norm_weight_dev, eps, k, (hipStream_t)stream);
 }
 
-int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
-                                float *residual_dev, float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream) {
+int64_t cq_nn_qmatmul_split_planes(int w_dtype, int64_t k) { return cq_matvec_ksplit_planes(w_dtype, k); }
+
+int cq_nn_qmatmul_split(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *planes_dev, int64_t k, int64_t n,
+                        void *stream) {
     int rc = check_mm_shape(w_dtype, k, n, 1);
     if (rc) return rc;
+    if (cq_matvec_ksplit_planes(w_dtype, k) == 0) return CQ_ERR_RANGE;
     if (n == 0) return CQ_OK;
     if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
-    if (!attn_partials_dev || !residual_dev || !sumsq_partials_out_dev) return CQ_ERR_NULL;
-    if (!aligned(attn_partials_dev, 16) || !aligned(residual_dev, 4) || !aligned(sumsq_partials_out_dev, 4)) return CQ_ERR_ALIGN;
-    return cq_matvec_residual_attn_launch(w_dtype, w_dev, attn_partials_dev, splits, head_dim, residual_dev, sumsq_partials_out_dev, k, n,
-                                          (hipStream_t)stream);
+    if (!x_dev || !planes_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || (up_dev && !aligned(up_dev, 16)) || !aligned(planes_dev, 16)) return CQ_ERR_ALIGN;
+    return cq_matvec_ksplit_launch(w_dtype, w_dev, x_dev, up_dev, planes_dev, k, n, (hipStream_t)stream);
+}
+
+int cq_nn_qmatmul_norm_merge(int w_dtype, const void *w_dev, const float *x_dev, const float *planes_dev, int64_t n_planes,
+                             const float *norm_weight_dev, float eps, float *dst_dev, int64_t k, int64_t n, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, 1);
+    if (rc) return rc;
+    if (n_planes < 1 || n_planes > CQ_NN_MAX_PLANES) return CQ_ERR_RANGE;
+    if (n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!x_dev || !norm_weight_dev || !dst_dev || !planes_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(norm_weight_dev, 16) || !aligned(planes_dev, 16) || !aligned(dst_dev, 4)) return CQ_ERR_ALIGN;
+    return cq_matvec_norm_merge_launch(w_dtype, w_dev, x_dev, planes_dev, n_planes, norm_weight_dev, eps, dst_dev, k, n, (hipStream_t)stream);
+}
+
+int cq_nn_qmatmul_norm_pair_merge(int w_dtype_a, const void *w_a_dev, int64_t n_a, float *dst_a_dev, int w_dtype_b, const void *w_b_dev,
+                                  int64_t n_b, float *dst_b_dev, const float *x_dev, const float *planes_dev, int64_t n_planes,
+                                  const float *norm_weight_dev, float eps, int64_t k, void *stream) {
+    int rc = check_mm_shape(w_dtype_a, k, n_a, 1);
+    if (rc || (rc = check_mm_shape(w_dtype_b, k, n_b, 1))) return rc;
+    if (n_planes < 1 || n_planes > CQ_NN_MAX_PLANES) return CQ_ERR_RANGE;
+    if ((rc = check_weight_ptr(w_dtype_a, w_a_dev)) || (rc = check_weight_ptr(w_dtype_b, w_b_dev))) return rc;
+    if (!x_dev || !norm_weight_dev || !dst_a_dev || !dst_b_dev || !planes_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(norm_weight_dev, 16) || !aligned(planes_dev, 16) || !aligned(dst_a_dev, 4) || !aligned(dst_b_dev, 4))
+        return CQ_ERR_ALIGN;
+    return cq_matvec_norm_pair_merge_launch(w_dtype_a, w_a_dev, n_a, dst_a_dev, w_dtype_b, w_b_dev, n_b, dst_b_dev, x_dev, planes_dev, n_planes,
+                                            norm_weight_dev, eps, k, (hipStream_t)stream);
+}
+
+int cq_nn_qmatmul_residual_attn_merge(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
+                                      float *residual_dev, float *sumsq_partials_out_dev, const float *planes_dev, int64_t n_planes, int64_t k,
+                                      int64_t n, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, 1);
+    if (rc) return rc;
+    if (n_planes < 0 || n_planes > CQ_NN_MAX_PLANES) return CQ_ERR_RANGE;
+    if (n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!attn_partials_dev || !residual_dev || !sumsq_partials_out_dev || (n_planes > 0 && !planes_dev)) return CQ_ERR_NULL;
+    if (!aligned(attn_partials_dev, 16) || !aligned(residual_dev, 4) || !aligned(sumsq_partials_out_dev, 4) || !aligned(planes_dev, 4))
+        return CQ_ERR_ALIGN;
+    return cq_matvec_residual_attn_launch(w_dtype, w_dev, attn_partials_dev, splits, head_dim, residual_dev, sumsq_partials_out_dev, planes_dev,
+                                          n_planes, k, n, (hipStream_t)stream);
+}
+
+int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
+                                float *residual_dev, float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream) {
+    return cq_nn_qmatmul_residual_attn_merge(w_dtype, w_dev, attn_partials_dev, splits, head_dim, residual_dev, sumsq_partials_out_dev, nullptr, 0,
+                                             k, n, stream);
 }
 
 }  // extern "C"

@@ -193,6 +193,57 @@ template <> struct Fmt<CQ_Q6K> {
     }
 };
 
+// Q6_K rows of more than one wave step: 8 lanes per super-block.  Lane j of a super-block takes the 16 bytes
+// ql[16j, 16j + 16) — so one load instruction reads each super-block's ql as one 128-byte run, and a 14336-element
+// row is exactly 7 full wave steps — plus the qh bytes of the same 16 `l` positions.
+// j = 4h + 2p + c: low nibbles are elements 128h + 32p + 16c + [0, 16) (qh bits 2p, 2p + 1), high nibbles the
+// elements 64 further on (qh bits 2p + 4, 2p + 5); k_quants.rs:2265-2274.
+struct FmtQ6Narrow {
+    static constexpr int UE = 32, UPB = 8;
+    struct W { u32x4 ql, qh; u32x2 sc; uint32_t d; };
+    struct A { u32x4 lo, hi; int bs_lo, bs_hi; float d8; };
+    static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *blk = row + (u >> 3) * 210;
+        const int j = u & 7, h = j >> 2, c = j & 1;
+        w.ql = ld_u<u32x4>(blk + 16 * j);
+        w.qh = ld_u<u32x4>(blk + 128 + 32 * h + 16 * c);
+        w.sc = ld_u<u32x2>(blk + 192 + 8 * h);              // the 8 scales of this half
+        w.d = ld_u<uint16_t>(blk + 208);
+    }
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) {
+        const int sb = u >> 3, j = u & 7, h = j >> 2, idx = 8 * h + (j & 3);      // 16-element group of the low nibbles
+        const int8_t *q = ar.qs + sb * 256 + 16 * idx;
+        a.lo = *reinterpret_cast<const u32x4 *>(q);
+        a.hi = *reinterpret_cast<const u32x4 *>(q + 64);
+        a.bs_lo = ar.bsums[sb * 16 + idx];
+        a.bs_hi = ar.bsums[sb * 16 + idx + 4];
+        a.d8 = ar.d[sb];
+    }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int u) {
+        const int pc = u & 3, p = (u >> 1) & 1;
+        const int s_lo = (int)(int8_t)((w.sc.x >> (8 * pc)) & 0xff), s_hi = (int)(int8_t)((w.sc.y >> (8 * pc)) & 0xff);
+        const uint32_t ql[4] = {w.ql.x, w.ql.y, w.ql.z, w.ql.w};
+        const uint32_t qh[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
+        const uint32_t al[4] = {a.lo.x, a.lo.y, a.lo.z, a.lo.w};
+        const uint32_t ah[4] = {a.hi.x, a.hi.y, a.hi.z, a.hi.w};
+        // unsigned 6-bit values; the -32 offset is applied through the 16-element sums
+        int dl = -32 * a.bs_lo, dh = -32 * a.bs_hi;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t hs = qh[i] >> (2 * p);
+            dl = sdot4((ql[i] & 0x0f0f0f0fu) | ((hs << 4) & 0x30303030u), al[i], dl);
+            dh = sdot4(((ql[i] >> 4) & 0x0f0f0f0fu) | (hs & 0x30303030u), ah[i], dh);
+        }
+        const int S = __mul24(s_lo, dl) + __mul24(s_hi, dh);
+        return (h2f(w.d) * a.d8) * (float)S;
+    }
+};
+
+// The unit decomposition a kernel instance uses: rows of one wave step (SINGLE) and register-blocked instances
+// keep Fmt<DT>.
+template <int DT, int NB, bool SINGLE> struct UnitFmt { typedef Fmt<DT> type; };
+template <> struct UnitFmt<CQ_Q6K, 1, false> { typedef FmtQ6Narrow type; };
+
 // ---- Q4_0 / Q8_0: one 32-element block per unit, Q8_0-quantized activations ------------------
 struct A0 {
     u32x4 a0, a1;

@@ -17,14 +17,23 @@ int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtyp
 // single-row decoder fusions (see the Fuse struct in cq_matvec.hip); partial-sum buffers hold 256 floats
 int cq_matvec_norm_launch(int w_dtype, const void *w, const float *x, const float *partials, const float *norm_weight, float eps, float *dst,
                           int64_t k, int64_t n, hipStream_t s);
-int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const float *up, float *residual, float *partials_out, int64_t k,
-                              int64_t n, hipStream_t s);
+// planes / n_planes (optional, at most 4): K-slice planes of a split matvec still to be added to the residual row
+int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const float *up, float *residual, float *partials_out,
+                              const float *planes, int64_t n_planes, int64_t k, int64_t n, hipStream_t s);
 int cq_matvec_residual_attn_launch(int w_dtype, const void *w, const float *attn_partials, int64_t splits, int64_t head_dim, float *residual,
-                                   float *partials_out, int64_t k, int64_t n, hipStream_t s);
+                                   float *partials_out, const float *planes, int64_t n_planes, int64_t k, int64_t n, hipStream_t s);
 int cq_matvec_norm_swiglu_launch(int w_dtype, const void *w1, const void *w3, const float *x, const float *partials, const float *norm_weight,
                                  float eps, float *dst, int64_t k, int64_t ffn, hipStream_t s);
 int cq_matvec_norm_pair_launch(int dta, const void *wa, int64_t na, float *dsta, int dtb, const void *wb, int64_t nb, float *dstb, const float *x,
                                const float *partials, const float *norm_weight, float eps, int64_t k, hipStream_t s);
+// a long-row matvec split along K into planes, and the PRO_NORM consumers that add the planes back (see cq_matvec.hip)
+int64_t cq_matvec_ksplit_planes(int w_dtype, int64_t k);
+int cq_matvec_ksplit_launch(int w_dtype, const void *w, const float *x, const float *up, float *planes, int64_t k, int64_t n, hipStream_t s);
+int cq_matvec_norm_merge_launch(int w_dtype, const void *w, const float *x, const float *planes, int64_t n_planes, const float *norm_weight,
+                                float eps, float *dst, int64_t k, int64_t n, hipStream_t s);
+int cq_matvec_norm_pair_merge_launch(int dta, const void *wa, int64_t na, float *dsta, int dtb, const void *wb, int64_t nb, float *dstb,
+                                     const float *x, const float *planes, int64_t n_planes, const float *norm_weight, float eps, int64_t k,
+                                     hipStream_t s);
 // split_ws: optional workspace of cq_qmm_splits(k, n, rows) * rows * n floats for split-K partial planes (NULL: no split)
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s, float *split_ws = nullptr);

@@ -45,9 +45,16 @@ struct ActSrc {
 //             rows b >= nvalid are padding and are not stored (8 router pairs of one expert per weight pass)
 //   EPI_RESID the result is added to a residual row in place of being stored, and the workgroup leaves
 //             its partial sum of residual^2 for the next PRO_NORM consumer
-enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2, PRO_MERGE = 3 };
+//   PRO_NORM_SPLIT like PRO_NORM, but the row is ((x + planes[0]) + planes[1]) + ... (the K-slice partial results of a
+//             split matvec, added in this fixed order); sum(x^2) is computed here.  x itself is left as it is
+//   EPI_RESID_SPLIT like EPI_RESID, with the same planes added to the residual row first (same order), so the row
+//             leaves this kernel merged
+enum { PRO_NONE = 0, PRO_NORM = 1, PRO_SILU = 2, PRO_MERGE = 3, PRO_NORM_SPLIT = 4 };
+constexpr bool pro_is_split(int pro) { return pro == PRO_NORM_SPLIT; }
 constexpr int MAXS = 16;     // attention splits a PRO_MERGE prologue can merge
-enum { EPI_NONE = 0, EPI_RESID = 1, EPI_SWIGLU = 2, EPI_SCALE = 3, EPI_MOE = 4 };
+constexpr int MAXP = 4;      // K-slice planes a PRO_NORM_SPLIT prologue / EPI_RESID_SPLIT epilogue can add
+enum { EPI_NONE = 0, EPI_RESID = 1, EPI_SWIGLU = 2, EPI_SCALE = 3, EPI_MOE = 4, EPI_RESID_SPLIT = 5 };
+constexpr bool epi_is_resid(int epi) { return epi == EPI_RESID || epi == EPI_RESID_SPLIT; }
 constexpr int NPART = 256;   // == CQ_NN_PARTIALS
 struct Fuse {
     const float *aux;        // PRO_NORM: norm weight [k];  PRO_SILU: up [k];  PRO_MERGE: partials [k/hd][splits][hd + 4]
@@ -60,6 +67,8 @@ struct Fuse {
     const int *row_map;      // EPI_MOE
     const float *row_scale;
     int nvalid;
+    const float *planes;     // PRO_NORM_SPLIT: [n_planes][k];  EPI_RESID_SPLIT: [n_planes][n]
+    int n_planes;
 };
 
 // Launch geometry, computed once on the host so the kernel prologue is a handful of scalar loads
@@ -70,7 +79,7 @@ struct QmvGeom {
     int lds_d_off, lds_bs_off; // LDS sections (the scratch layout for NB rows)
     int nw_shift;              // log2(waves per workgroup)
     int row_bytes;             // bytes of one row of W
-    int lds_red_off;           // EPI_RESID: 16 floats behind the activation sections
+    int lds_red_off;           // EPI_RESID / PRO_NORM_SPLIT: 16 floats behind the activation sections
     int dst_dtype;
     int64_t stride_dst;
 };
@@ -127,11 +136,14 @@ __device__ __forceinline__ void merge_reduce(const MergeRegs<MS> &r, bool ok, fl
 template <int DT, int NB, int SRC, bool SINGLE, int PRO, int EPI, bool PRE>
 __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const ActSrc &src, void *__restrict__ dst, const QmvGeom &g, const Fuse &fz,
                                          const int block, const int nblocks) {
-    typedef Fmt<DT> F;
+    typedef typename UnitFmt<DT, NB, SINGLE>::type F;
     static_assert((PRO == PRO_NONE && (EPI == EPI_NONE || EPI == EPI_MOE)) || (NB == 1 && SRC == CQ_F32), "fusions are for one f32 row");
     static_assert(PRO != PRO_MERGE || (SINGLE && !PRE), "the merge prologue preloads one span per wave");
+    static_assert(!pro_is_split(PRO) || !PRE, "the plane-merging prologue holds one span per wave");
     static_assert(EPI != EPI_SWIGLU || SINGLE, "the paired-row epilogue is written for rows of one wave step");
     constexpr bool FUSED = SRC != SRC_SCRATCH;
+    constexpr bool RESID = epi_is_resid(EPI);
+    constexpr int ME = EPI == EPI_RESID_SPLIT ? MAXP : 1;          // planes added to the residual row
     constexpr int XDT = FUSED ? SRC : CQ_F32;
     extern __shared__ __align__(16) uint8_t lds[];
     int8_t *lqs = (int8_t *)lds;
@@ -170,6 +182,8 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
     float pp[NPART / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
     constexpr int MS = PRO == PRO_MERGE ? MAXS : 1;
     MergeRegs<MS> mg;
+    constexpr int MP = PRO == PRO_NORM_SPLIT ? MAXP : 1;
+    float pl[MP][4];
     if (FUSED && PRO == PRO_MERGE) {
         merge_load<MS>(fz, xbase, xbase < total, mg);
     } else if (FUSED) {
@@ -181,6 +195,13 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
         if (PRO == PRO_NORM) {
 #pragma unroll
             for (int i = 0; i < NPART / 64; i++) pp[i] = fz.part_in[lane + 64 * i];
+        }
+        if (pro_is_split(PRO)) {
+            // unconditional loads (a plane that is not there re-reads the last one and is zeroed when it is added):
+            // branches here would make the compiler wait for these loads before it issues the weight loads
+            const int xc = min(xbase, total - 4);
+#pragma unroll
+            for (int sI = 0; sI < MP; sI++) cq_load4<CQ_F32>(fz.planes, (int64_t)min(sI, fz.n_planes - 1) * k + xc, pl[sI]);
         }
     } else {
         if (tid < (total >> 4)) c_qs = ((const u32x4 *)src.av.qs)[tid];
@@ -220,6 +241,10 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
         F::load_w(wa, wp, u0);
     }
 
+    // every load above is issued before the first wait below (the scheduler would otherwise sink some of the
+    // weight loads behind the waits for the activation loads)
+    if (pro_is_split(PRO)) __builtin_amdgcn_sched_barrier(0);
+
     // 2. activations -> LDS
     if (FUSED) {
         // The first span is peeled out of the loop on purpose: its values are already in xv, and as
@@ -234,10 +259,30 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
             pm = sqrtf(sum2 / (float)k + fz.eps);
         }
         if (PRO == PRO_MERGE) merge_reduce<MS>(mg, xbase < total, xv[0]);
+        if (pro_is_split(PRO)) {
+            // the merged row (absent planes are zeros) and sum(x^2) over the whole row in a fixed order: one span
+            // per wave, so a workgroup-wide reduction is needed
+#pragma unroll
+            for (int sI = 0; sI < MP; sI++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) xv[0][e] += (sI < fz.n_planes && xbase < total) ? pl[sI][e] : 0.0f;
+            const float ss = wave_sum((xv[0][0] * xv[0][0] + xv[0][1] * xv[0][1]) + (xv[0][2] * xv[0][2] + xv[0][3] * xv[0][3]));
+            float *red = (float *)(lds + g.lds_red_off);
+            if (lane == 0) red[wv] = ss;
+            if (wv == 0 && lane >= nwaves && lane < 16) red[lane] = 0.0f;        // slots of waves that do not exist
+            __syncthreads();
+            // four broadcast reads and a fixed order of additions (no loop over the wave count: each trip would
+            // be a dependent LDS round trip)
+            const f32x4 r0 = ((const f32x4 *)red)[0], r1 = ((const f32x4 *)red)[1], r2 = ((const f32x4 *)red)[2], r3 = ((const f32x4 *)red)[3];
+            const float sum2 = ((((r0.x + r0.y) + (r0.z + r0.w)) + ((r1.x + r1.y) + (r1.z + r1.w))) +
+                                (((r2.x + r2.y) + (r2.z + r2.w)) + ((r3.x + r3.y) + (r3.z + r3.w))));
+            pm = sqrtf(sum2 / (float)k + fz.eps);
+        }
 #pragma unroll
         for (int j = 0; j < XS; j++) {
             const int span = wv_s + (j << g.nw_shift);
             if (PRO == PRO_NORM || PRO == PRO_SILU) pro_apply<PRO>(xv[j], av4[j], pm);
+            if (pro_is_split(PRO)) pro_apply<PRO_NORM>(xv[j], av4[j], pm);
             if (span < spans) {
                 if (cq_is_kquant(DT))
                     cq_quantize_q8k_vals(xv[j], span, lane, lqs, ld, lbs);
@@ -287,8 +332,26 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
         }
     }
     __syncthreads();
-    if (EPI != EPI_RESID && my_rows == 0) return;
+    if (!RESID && my_rows == 0) return;
     float ssq = 0.0f;            // EPI_RESID: lane 63 accumulates residual^2 of this wave's rows
+    // The residual value of a row (and, EPI_RESID_SPLIT, the plane values to add to it) is requested together with the
+    // row's weights and travels behind them in the same in-order load queue.  Unconditional loads: a plane that is
+    // not there re-reads the last one and counts as zero.
+    auto load_res = [&](int r, float &rv, float (&pv)[ME]) {
+        const int rc = min(r, n - 1);
+        rv = fz.resid[rc];
+        if (EPI == EPI_RESID_SPLIT) {
+#pragma unroll
+            for (int sI = 0; sI < ME; sI++) pv[sI] = fz.planes[(int64_t)min(sI, fz.n_planes - 1) * n + rc];
+        }
+    };
+    auto merge_res = [&](float rv, const float (&pv)[ME]) {
+        if (EPI == EPI_RESID_SPLIT) {
+#pragma unroll
+            for (int sI = 0; sI < ME; sI++) rv += sI < fz.n_planes ? pv[sI] : 0.0f;
+        }
+        return rv;
+    };
     constexpr bool MOE_TAB = EPI == EPI_MOE && !(SINGLE && NB > 2);      // the blocked path reads them per b instead
     int64_t moe_off[MOE_TAB ? NB : 1];
     float moe_sc[MOE_TAB ? NB : 1];
@@ -321,7 +384,7 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
                 if (!CACHE) F::load_a(areg[b], ar[b], u0);
                 float v = F::dot(cur, areg[b], u0);
                 v = wave_sum_to_lane63(valid ? v : 0.0f);
-                if (EPI == EPI_RESID) {
+                if (RESID) {
                     if (lane == 63) {
                         const float sres = res + v;                     // (x + residual), quantized_llama.rs:584,591
                         fz.resid[r] = sres;
@@ -393,18 +456,18 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
         // ping-pong between wa and wb: the next row's loads are in flight while this one is reduced;
         // the prefetch past the last row re-reads it instead of branching around the load.  The residual
         // value of a row travels behind its weights in the same in-order load queue.
-        float ra = 0.0f, rb = 0.0f;
-        if (EPI == EPI_RESID) ra = fz.resid[min(row, n - 1)];
+        float ra = 0.0f, rb = 0.0f, pa[ME], pb[ME];
+        if (RESID) load_res(row, ra, pa);
         for (int j = 0; j < my_rows; j += 2) {
             const uint8_t *p1 = j + 1 < my_rows ? wp + wave_stride : wp;
             F::load_w(wb, p1, u0);
-            if (EPI == EPI_RESID) rb = fz.resid[min(row + nwaves, n - 1)];
-            one_row(wa, row, ra);
+            if (RESID) load_res(row + nwaves, rb, pb);
+            one_row(wa, row, merge_res(ra, pa));
             if (j + 1 >= my_rows) break;
             const uint8_t *p2 = j + 2 < my_rows ? p1 + wave_stride : p1;
             F::load_w(wa, p2, u0);
-            if (EPI == EPI_RESID) ra = fz.resid[min(row + 2 * nwaves, n - 1)];
-            one_row(wb, row + nwaves, rb);
+            if (RESID) load_res(row + 2 * nwaves, ra, pa);
+            one_row(wb, row + nwaves, merge_res(rb, pb));
             row += 2 * nwaves;
             wp = p2;
         }
@@ -416,15 +479,15 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
         for (int b = 0; b < NB; b++) acc[b] = 0.0f;
         int total_steps = my_rows * steps;
         int i = 0;
-        float rcur = 0.0f;
-        if (EPI == EPI_RESID) rcur = fz.resid[min(row, n - 1)];
+        float rcur = 0.0f, pcur[ME];
+        if (RESID) load_res(row, rcur, pcur);
         auto finish_row = [&]() {
 #pragma unroll
             for (int b = 0; b < NB; b++) {
                 float r = wave_sum_to_lane63(acc[b]);
-                if (EPI == EPI_RESID) {
+                if (RESID) {
                     if (lane == 63) {
-                        const float sres = rcur + r;
+                        const float sres = merge_res(rcur, pcur) + r;
                         fz.resid[row] = sres;
                         ssq += sres * sres;
                     }
@@ -436,7 +499,7 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
                 acc[b] = 0.0f;
             }
             row += nwaves;
-            if (EPI == EPI_RESID) rcur = fz.resid[min(row, n - 1)];   // consumed a whole row of steps later
+            if (RESID) load_res(row, rcur, pcur);   // consumed a whole row of steps later
         };
         auto accumulate = [&](const typename F::W &cur, int step) {
             const int u = lane + 64 * step;
@@ -480,7 +543,7 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
             one_step(wb, wa, t + 1);
         }
     }
-    if (EPI == EPI_RESID) {
+    if (RESID) {
         // the workgroup's partial of sum(residual^2), summed in a fixed order; block 0 clears the unused slots
         float *red = (float *)(lds + g.lds_red_off);
         if (lane == 63) red[wv] = ssq;
@@ -518,6 +581,9 @@ __global__ __launch_bounds__(1024) void qmv2_kernel(const uint8_t *__restrict__ 
 template <int DT, int NB>
 int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int64_t stride_dst, int dst_dtype, int extra_lds, size_t &lds_bytes,
               int64_t max_groups = 256) {
+    // units of the instance that will run: rows longer than one wave step of Fmt<DT> may use another decomposition
+    const bool single = k / Fmt<DT>::UE <= 64;
+    const int ue = single ? Fmt<DT>::UE : UnitFmt<DT, NB, false>::type::UE;
     if (waves == 0) {
         waves = NB > 2 ? 8 : 16;
         while (waves > 1 && n < 256 * (int64_t)waves) waves >>= 1;
@@ -530,7 +596,7 @@ int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int
     lds_bytes = (size_t)L.total + extra_lds;
     g.lds_red_off = (int)L.total;
     g.k = (int)k; g.n = (int)n; g.rows_per_wg = (int)rows_per_wg;
-    g.units = (int)(k / Fmt<DT>::UE); g.steps = (g.units + 63) >> 6;
+    g.units = (int)(k / ue); g.steps = (g.units + 63) >> 6;
     g.lds_d_off = (int)L.d_off; g.lds_bs_off = (int)L.bs_off;
     g.nw_shift = 0;
     while ((1 << g.nw_shift) < waves) g.nw_shift++;
@@ -541,6 +607,15 @@ int make_geom(QmvGeom &g, int64_t &groups, int &waves, int64_t k, int64_t n, int
     return CQ_OK;
 }
 
+// PRO_NORM_SPLIT: the smallest workgroup (a power of two of waves) that gives every 256-element span its own wave
+inline int split_min_waves(int64_t k) {
+    const int64_t spans = (k + 255) / 256;
+    if (spans > 16) return 0;
+    int w = 1;
+    while (w < spans) w <<= 1;
+    return w;
+}
+
 template <int DT, int NB, int SRC, bool SINGLE, int PRO = PRO_NONE, int EPI = EPI_NONE, bool PRE = false>
 int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s,
                const Fuse &fz = Fuse{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0}) {
@@ -548,21 +623,31 @@ int launch_cfg(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64
     int64_t groups;
     int waves = 0;
     size_t lds_bytes;
-    int rc = make_geom<DT, NB>(g, groups, waves, k, n, stride_dst, dst_dtype, EPI == EPI_RESID ? 64 : 0, lds_bytes);
+    constexpr int XL = epi_is_resid(EPI) || pro_is_split(PRO) ? 64 : 0;
+    int rc = make_geom<DT, NB>(g, groups, waves, k, n, stride_dst, dst_dtype, XL, lds_bytes);
     if (rc) return rc;
+    Fuse f2 = fz;
+    if (pro_is_split(PRO)) {
+        const int need = split_min_waves(k);                        // one span per wave
+        if (need == 0) return CQ_ERR_RANGE;
+        if (waves < need) {
+            waves = need;
+            if ((rc = make_geom<DT, NB>(g, groups, waves, k, n, stride_dst, dst_dtype, XL, lds_bytes))) return rc;
+        }
+    }
     auto kern = qmv_kernel<DT, NB, SRC, SINGLE, PRO, EPI, PRE>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * waves), lds_bytes, s, (const uint8_t *)w, src, dst, g, fz);
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * waves), lds_bytes, s, (const uint8_t *)w, src, dst, g, f2);
     return (int)hipGetLastError();
 }
 
 template <int DT, int NB, int SRC>
 int launch_nb(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
     if (k / Fmt<DT>::UE <= 64) return launch_cfg<DT, NB, SRC, true>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-    if (NB == 1 && k / Fmt<DT>::UE <= 256)
+    if (NB == 1 && k / UnitFmt<DT, NB, false>::type::UE <= 256)
         return launch_cfg<DT, NB, SRC, false, PRO_NONE, EPI_NONE, NB == 1>(w, src, dst, dst_dtype, k, n, stride_dst, s);
     return launch_cfg<DT, NB, SRC, false>(w, src, dst, dst_dtype, k, n, stride_dst, s);
 }
@@ -654,8 +739,12 @@ template <int DT, int PRO, int EPI>
 int launch_fused1(const void *w, const ActSrc &src, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
     if (cq_act_layout(DT, k, 1).total + 64 > LDS_BUDGET) return CQ_ERR_RANGE;
     if (k / Fmt<DT>::UE <= 64) return launch_cfg<DT, 1, CQ_F32, true, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
-    if (k / Fmt<DT>::UE <= 256) return launch_cfg<DT, 1, CQ_F32, false, PRO, EPI, true>(w, src, dst, CQ_F32, k, n, n, s, fz);
-    return launch_cfg<DT, 1, CQ_F32, false, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
+    if constexpr (pro_is_split(PRO)) {
+        return CQ_ERR_RANGE;                                 // one span per wave: rows of one wave step only
+    } else {
+        if (k / UnitFmt<DT, 1, false>::type::UE <= 256) return launch_cfg<DT, 1, CQ_F32, false, PRO, EPI, true>(w, src, dst, CQ_F32, k, n, n, s, fz);
+        return launch_cfg<DT, 1, CQ_F32, false, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
+    }
 }
 template <int PRO, int EPI>
 int launch_fused_dt(int w_dtype, const void *w, const ActSrc &src, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
@@ -679,12 +768,17 @@ int cq_matvec_norm_launch(int w_dtype, const void *w, const float *x, const floa
     return launch_fused_dt<PRO_NORM, EPI_NONE>(w_dtype, w, src, dst, k, n, s, fz);
 }
 
-// residual[n] += W . quantize(up ? silu(x) * up : x); partials_out[256] = partial sums of residual^2
-int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const float *up, float *residual, float *partials_out, int64_t k,
-                              int64_t n, hipStream_t s) {
+// residual[n] = (residual + planes[0] + ...) + W . quantize(up ? silu(x) * up : x); partials_out[256] = partial sums of residual^2
+int cq_matvec_residual_launch(int w_dtype, const void *w, const float *x, const float *up, float *residual, float *partials_out,
+                              const float *planes, int64_t n_planes, int64_t k, int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
+    if (n_planes < 0 || n_planes > MAXP) return CQ_ERR_RANGE;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{up, nullptr, 0.0f, residual, partials_out, 0, 0, 0, nullptr, nullptr, 0};
+    Fuse fz{up, nullptr, 0.0f, residual, partials_out, 0, 0, 0, nullptr, nullptr, 0, planes, (int)n_planes};
+    if (n_planes > 0) {
+        if (up) return launch_fused_dt<PRO_SILU, EPI_RESID_SPLIT>(w_dtype, w, src, nullptr, k, n, s, fz);
+        return launch_fused_dt<PRO_NONE, EPI_RESID_SPLIT>(w_dtype, w, src, nullptr, k, n, s, fz);
+    }
     if (up) return launch_fused_dt<PRO_SILU, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
     return launch_fused_dt<PRO_NONE, EPI_RESID>(w_dtype, w, src, nullptr, k, n, s, fz);
 }
@@ -694,6 +788,7 @@ template <int DT>
 int launch_merge1(const void *w, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
     if (k / Fmt<DT>::UE > 64) return CQ_ERR_RANGE;          // one wave step per row, one span per wave
     ActSrc src{nullptr, ActView{nullptr, nullptr, nullptr}};
+    if (fz.n_planes > 0) return launch_cfg<DT, 1, CQ_F32, true, PRO_MERGE, EPI_RESID_SPLIT>(w, src, dst, CQ_F32, k, n, n, s, fz);
     return launch_cfg<DT, 1, CQ_F32, true, PRO_MERGE, EPI_RESID>(w, src, dst, CQ_F32, k, n, n, s, fz);
 }
 }  // namespace
@@ -702,12 +797,13 @@ int launch_merge1(const void *w, void *dst, int64_t k, int64_t n, hipStream_t s,
 // CQ_ERR_RANGE when the row is longer than one wave step (k > 4096 for K-quants, > 2048 for Q4_0 / Q8_0),
 // when splits > 16, or when head_dim is not a power of two.
 int cq_matvec_residual_attn_launch(int w_dtype, const void *w, const float *attn_partials, int64_t splits, int64_t head_dim, float *residual,
-                                   float *partials_out, int64_t k, int64_t n, hipStream_t s) {
+                                   float *partials_out, const float *planes, int64_t n_planes, int64_t k, int64_t n, hipStream_t s) {
     if (n == 0) return CQ_OK;
     if (splits < 1 || splits > MAXS || head_dim < 4 || (head_dim & (head_dim - 1)) || k % head_dim) return CQ_ERR_RANGE;
+    if (n_planes < 0 || n_planes > MAXP) return CQ_ERR_RANGE;
     int sh = 0;
     while ((1 << sh) < head_dim) sh++;
-    Fuse fz{attn_partials, nullptr, 0.0f, residual, partials_out, (int)splits, sh, 0, nullptr, nullptr, 0};
+    Fuse fz{attn_partials, nullptr, 0.0f, residual, partials_out, (int)splits, sh, 0, nullptr, nullptr, 0, planes, (int)n_planes};
     switch (w_dtype) {
         case CQ_Q4_0: return launch_merge1<CQ_Q4_0>(w, nullptr, k, n, s, fz);
         case CQ_Q8_0: return launch_merge1<CQ_Q8_0>(w, nullptr, k, n, s, fz);
@@ -726,48 +822,65 @@ int launch_swiglu1(const void *w1, int64_t pair_off, const ActSrc &src, float *d
     return launch_cfg<DT, 1, CQ_F32, true, PRO_NORM, EPI_SWIGLU>(w1, src, dst, CQ_F32, k, ffn, ffn, s, fz);
 }
 
-template <int DTA, int DTB>
+template <int DTA, int DTB, int PRO>
 int launch_pair(const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const ActSrc &src, int64_t k, hipStream_t s,
-                const Fuse &fz) {
+                const Fuse &fz_in) {
+    constexpr int XL = pro_is_split(PRO) ? 64 : 0;
     QmvGeom ga, gb;
     int64_t groups_a, groups_b;
     size_t lds_a, lds_b;
     // one block size for both segments: that of the larger tensor
     int waves = 0;
-    int rc = na >= nb ? make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, 0, lds_a) : make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, 0, lds_b);
+    int rc = na >= nb ? make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, XL, lds_a) : make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, XL, lds_b);
     if (rc) return rc;
+    if (pro_is_split(PRO)) {
+        const int need = split_min_waves(k);                        // one span per wave
+        if (need == 0) return CQ_ERR_RANGE;
+        if (waves < need) waves = need;
+    }
     // 256 workgroups in total (one per CU: a 16-wave workgroup fills a CU's registers, so a 257th would wait for a
     // whole workgroup to finish), shared between the tensors in proportion to their bytes
     const double bytes_a = (double)na * BlockInfo<DTA>::bytes / BlockInfo<DTA>::elems, bytes_b = (double)nb * BlockInfo<DTB>::bytes / BlockInfo<DTB>::elems;
     int64_t share_a = (int64_t)(256.0 * bytes_a / (bytes_a + bytes_b) + 0.5);
     if (share_a < 1) share_a = 1;
     if (share_a > 255) share_a = 255;
-    if ((rc = make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, 0, lds_a, share_a))) return rc;
-    if ((rc = make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, 0, lds_b, 256 - share_a))) return rc;
+    if ((rc = make_geom<DTA, 1>(ga, groups_a, waves, k, na, na, CQ_F32, XL, lds_a, share_a))) return rc;
+    if ((rc = make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, XL, lds_b, 256 - share_a))) return rc;
     const size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
     const bool single = k / 64 <= 64;                     // every K-quant unit is 64 elements
+    const Fuse &fz = fz_in;
     if (lds_bytes > 48 * 1024) {
-        const void *kp = single ? (const void *)qmv2_kernel<DTA, DTB, true, PRO_NORM> : (const void *)qmv2_kernel<DTA, DTB, false, PRO_NORM>;
+        const void *kp = single ? (const void *)qmv2_kernel<DTA, DTB, true, PRO> : (const void *)qmv2_kernel<DTA, DTB, false, PRO>;
         hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
     }
     dim3 grid((unsigned)(groups_a + groups_b)), block(64 * waves);
     if (single)
-        hipLaunchKernelGGL((qmv2_kernel<DTA, DTB, true, PRO_NORM>), grid, block, lds_bytes, s, (const uint8_t *)wa, (const uint8_t *)wb, src,
+        hipLaunchKernelGGL((qmv2_kernel<DTA, DTB, true, PRO>), grid, block, lds_bytes, s, (const uint8_t *)wa, (const uint8_t *)wb, src,
                            (void *)dsta, (void *)dstb, ga, gb, fz, (int)groups_a);
     else
-        hipLaunchKernelGGL((qmv2_kernel<DTA, DTB, false, PRO_NORM>), grid, block, lds_bytes, s, (const uint8_t *)wa, (const uint8_t *)wb, src,
+        hipLaunchKernelGGL((qmv2_kernel<DTA, DTB, false, PRO>), grid, block, lds_bytes, s, (const uint8_t *)wa, (const uint8_t *)wb, src,
                            (void *)dsta, (void *)dstb, ga, gb, fz, (int)groups_a);
     return (int)hipGetLastError();
 }
 
-template <int DTA>
+template <int DTA, int PRO>
 int launch_pair_b(int dtb, const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const ActSrc &src, int64_t k,
                   hipStream_t s, const Fuse &fz) {
     switch (dtb) {
-        case CQ_Q4K: return launch_pair<DTA, CQ_Q4K>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
-        case CQ_Q5K: return launch_pair<DTA, CQ_Q5K>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
-        case CQ_Q6K: return launch_pair<DTA, CQ_Q6K>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q4K: return launch_pair<DTA, CQ_Q4K, PRO>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q5K: return launch_pair<DTA, CQ_Q5K, PRO>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q6K: return launch_pair<DTA, CQ_Q6K, PRO>(wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+    }
+    return CQ_ERR_DTYPE;
+}
+template <int PRO>
+int launch_pair_a(int dta, int dtb, const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const ActSrc &src, int64_t k,
+                  hipStream_t s, const Fuse &fz) {
+    switch (dta) {
+        case CQ_Q4K: return launch_pair_b<CQ_Q4K, PRO>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q5K: return launch_pair_b<CQ_Q5K, PRO>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+        case CQ_Q6K: return launch_pair_b<CQ_Q6K, PRO>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
     }
     return CQ_ERR_DTYPE;
 }
@@ -799,10 +912,103 @@ int cq_matvec_norm_pair_launch(int dta, const void *wa, int64_t na, float *dsta,
     if (cq_act_layout(dta, k, 1).total > LDS_BUDGET) return CQ_ERR_RANGE;
     ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
     Fuse fz{norm_weight, partials, eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
-    switch (dta) {
-        case CQ_Q4K: return launch_pair_b<CQ_Q4K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
-        case CQ_Q5K: return launch_pair_b<CQ_Q5K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
-        case CQ_Q6K: return launch_pair_b<CQ_Q6K>(dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+    return launch_pair_a<PRO_NORM>(dta, dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+}
+
+// The same two launches for a row still split over K-slice planes: ((x + planes[0]) + planes[1]) + ... is
+// normalized, with the sum of squares computed in the kernel.
+int cq_matvec_norm_pair_merge_launch(int dta, const void *wa, int64_t na, float *dsta, int dtb, const void *wb, int64_t nb, float *dstb,
+                                     const float *x, const float *planes, int64_t n_planes, const float *norm_weight, float eps, int64_t k,
+                                     hipStream_t s) {
+    if (!cq_is_kquant(dta) || !cq_is_kquant(dtb) || dta == CQ_Q8K || dtb == CQ_Q8K) return CQ_ERR_DTYPE;
+    if (na == 0 || nb == 0) return CQ_ERR_SHAPE;
+    if (n_planes < 1 || n_planes > MAXP) return CQ_ERR_RANGE;
+    if (cq_act_layout(dta, k, 1).total + 64 > LDS_BUDGET) return CQ_ERR_RANGE;
+    ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{norm_weight, nullptr, eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0, planes, (int)n_planes};
+    return launch_pair_a<PRO_NORM_SPLIT>(dta, dtb, wa, na, dsta, wb, nb, dstb, src, k, s, fz);
+}
+
+int cq_matvec_norm_merge_launch(int w_dtype, const void *w, const float *x, const float *planes, int64_t n_planes, const float *norm_weight,
+                                float eps, float *dst, int64_t k, int64_t n, hipStream_t s) {
+    if (n == 0) return CQ_OK;
+    if (n_planes < 1 || n_planes > MAXP) return CQ_ERR_RANGE;
+    ActSrc src{x, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{norm_weight, nullptr, eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0, planes, (int)n_planes};
+    return launch_fused_dt<PRO_NORM_SPLIT, EPI_NONE>(w_dtype, w, src, dst, k, n, s, fz);
+}
+
+// ---- a matvec split along K: plane s holds W[:, slice s] . quantize(x[slice s]) for every row ----
+// Each workgroup quantizes only its slice of the activation row (the cost of quantizing a long row in every
+// workgroup is what this removes); the planes are added in a fixed order by the consumers' PRO_NORM_SPLIT prologue
+// and EPI_RESID_SPLIT epilogue.
+namespace {
+template <int DT, int PRO>
+__global__ __launch_bounds__(1024) void qmv_ksplit_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, const float *__restrict__ up,
+                                                          float *__restrict__ planes, QmvGeom g, int slice_bytes) {
+    const int ks = blockIdx.y;
+    ActSrc src{x + (int64_t)ks * g.k, ActView{nullptr, nullptr, nullptr}};
+    Fuse fz{PRO == PRO_SILU ? up + (int64_t)ks * g.k : nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
+    qmv_body<DT, 1, CQ_F32, true, PRO, EPI_NONE, false>(w + (int64_t)ks * slice_bytes, src, planes + (int64_t)ks * g.n, g, fz, blockIdx.x, gridDim.x);
+}
+
+// The fewest equal slices (2 .. MAXP, whole blocks each) that one wave step per row covers; 0: none.  Few planes keep
+// the consumers cheap: every workgroup of a consumer reads every plane.
+template <int DT>
+int64_t ksplit_planes(int64_t k) {
+    constexpr int be = BlockInfo<DT>::elems;
+    if (k <= 0 || k % be) return 0;
+    const int64_t nblk = k / be;
+    for (int64_t p = 2; p <= MAXP; p++)
+        if (nblk % p == 0 && (k / p) / Fmt<DT>::UE <= 64) return p;
+    return 0;
+}
+
+template <int DT>
+int launch_ksplit(const void *w, const float *x, const float *up, float *planes, int64_t k, int64_t n, hipStream_t s) {
+    const int64_t n_planes = ksplit_planes<DT>(k);
+    if (n_planes == 0) return CQ_ERR_RANGE;
+    const int64_t slice = k / n_planes;
+    QmvGeom g;
+    int64_t groups;
+    int waves = 0;
+    size_t lds_bytes;
+    int rc = make_geom<DT, 1>(g, groups, waves, slice, n, n, CQ_F32, 0, lds_bytes, 256 / n_planes);
+    if (rc) return rc;
+    const int slice_bytes = g.row_bytes;
+    const int64_t rb = (k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
+    if (rb > 0x3fffffff) return CQ_ERR_RANGE;
+    g.row_bytes = (int)rb;                                  // rows are still a whole row of W apart
+    dim3 grid((unsigned)groups, (unsigned)n_planes), block(64 * waves);
+    if (up)
+        hipLaunchKernelGGL((qmv_ksplit_kernel<DT, PRO_SILU>), grid, block, lds_bytes, s, (const uint8_t *)w, x, up, planes, g, slice_bytes);
+    else
+        hipLaunchKernelGGL((qmv_ksplit_kernel<DT, PRO_NONE>), grid, block, lds_bytes, s, (const uint8_t *)w, x, up, planes, g, slice_bytes);
+    return (int)hipGetLastError();
+}
+}  // namespace
+
+// number of planes cq_matvec_ksplit_launch writes for this format and row length; 0: not available
+int64_t cq_matvec_ksplit_planes(int w_dtype, int64_t k) {
+    switch (w_dtype) {
+        case CQ_Q4_0: return ksplit_planes<CQ_Q4_0>(k);
+        case CQ_Q8_0: return ksplit_planes<CQ_Q8_0>(k);
+        case CQ_Q4K: return ksplit_planes<CQ_Q4K>(k);
+        case CQ_Q5K: return ksplit_planes<CQ_Q5K>(k);
+        case CQ_Q6K: return ksplit_planes<CQ_Q6K>(k);
+    }
+    return 0;
+}
+
+// planes[s][n] = W[:, slice s] . quantize((up ? silu(x) * up : x)[slice s])
+int cq_matvec_ksplit_launch(int w_dtype, const void *w, const float *x, const float *up, float *planes, int64_t k, int64_t n, hipStream_t s) {
+    if (n == 0) return CQ_OK;
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_ksplit<CQ_Q4_0>(w, x, up, planes, k, n, s);
+        case CQ_Q8_0: return launch_ksplit<CQ_Q8_0>(w, x, up, planes, k, n, s);
+        case CQ_Q4K: return launch_ksplit<CQ_Q4K>(w, x, up, planes, k, n, s);
+        case CQ_Q5K: return launch_ksplit<CQ_Q5K>(w, x, up, planes, k, n, s);
+        case CQ_Q6K: return launch_ksplit<CQ_Q6K>(w, x, up, planes, k, n, s);
     }
     return CQ_ERR_DTYPE;
 }
@@ -843,7 +1049,7 @@ int launch_moe_pairs(const void *w, const float *x, float *out, const PairSource
     if (rc) return rc;
     if (ps.n_pairs > 65535) return CQ_ERR_RANGE;
     const int64_t expert_bytes = n * (int64_t)g.row_bytes;
-    const bool single = g.units <= 64;
+    const bool single = k / Fmt<DT>::UE <= 64;
     const void *kp = single ? (const void *)moe_pair_kernel<DT, true> : (const void *)moe_pair_kernel<DT, false>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -897,7 +1103,7 @@ int launch_moe_chunks(const void *w, const void *scratch, int64_t rows_alloc, fl
     if (rc) return rc;
     if (mc.max_chunks > 65535) return CQ_ERR_RANGE;
     const int64_t expert_bytes = n * (int64_t)g.row_bytes;
-    const bool single = g.units <= 64;
+    const bool single = k / Fmt<DT>::UE <= 64;
     const void *kp = single ? (const void *)moe_chunk_kernel<DT, true> : (const void *)moe_chunk_kernel<DT, false>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);

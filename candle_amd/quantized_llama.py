@@ -105,7 +105,8 @@ class ModelWeights:
         self._slab: Optional[torch.Tensor] = None
         self._graph = None
         self._graph_key = None
-        self.fuse_decode = True      # single-token steps use the fused matvec prologues / epilogues
+        self.fuse_decode = True            # single-token steps use the fused matvec prologues / epilogues
+        self.split_w2 = True               # ... and feed_forward_w2 as a K-split matvec where the shapes allow it
         # bytes of the weights behind attention (wo, w1, w3, w2 are contiguous) that the attention launch's idle CUs
         # would pull through the memory-side cache ahead of the kernels that stream them.  Measured on the 8B shape:
         # no gain at 4-24 MB and a loss beyond (the time moves into the attention launch), so it is off.
@@ -161,6 +162,7 @@ class ModelWeights:
         self.max_rows = max_rows
         self._graph = None                 # a captured step holds the old buffer addresses
         self.x = torch.empty((max_rows, cfg.hidden), **f32)
+        self.planes = torch.empty((4, cfg.hidden), **f32)       # decode: K-slice planes of a split feed_forward_w2 (CQ_NN_MAX_PLANES)
         self.xn = torch.empty((max_rows, cfg.hidden), **f32)
         self.qk = torch.empty((max_rows, qd + kvd), **f32)
         self.v = torch.empty((max_rows, kvd), **f32)
@@ -302,36 +304,51 @@ class ModelWeights:
     def _enqueue_decode_fused(self, ids_ptr: int, pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
         """The same single-token step with the glue folded into the matvec kernels: the residual add is the
         epilogue of attention_wo / feed_forward_w2 (which also leaves sum(x^2) as partial sums), rms_norm and
-        silu(w1 x) * w3 x are the prologues of the matvecs that consume them."""
+        silu(w1 x) * w3 x are the prologues of the matvecs that consume them.  A long feed_forward_w2 row is split
+        along K into planes; the next rms_norm prologue reads the residual row plus the planes, and the next residual
+        add (attention_wo) folds them into the row."""
         cfg, L = self.cfg, self.L
         qd, kvd = cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim
         scale = float(np.float32(1.0 / math.sqrt(cfg.head_dim)))
         ck = _lib.check
-        x, qk, v, att, gu, part = self.x, self.qk, self.v, self.att, self.gu, self.partials
-        ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), 1, cfg.hidden, cfg.vocab,
-                                                part.data_ptr(), sp))
+        qk, v, att, gu, part, planes = self.qk, self.v, self.att, self.gu, self.partials, self.planes
+        kq = (GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
+        cur = self.x.data_ptr()                                    # the residual row
+        pending = 0                                                # planes of the previous feed_forward_w2 not yet added to it
+        ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, cur, 1, cfg.hidden, cfg.vocab, part.data_ptr(), sp))
+
+        def one_step(w: _W) -> bool:
+            return w.k <= (4096 if w.dtype in kq else 2048)
 
         def norm_mm(w: _W, n: int, norm_w: torch.Tensor, dst_ptr: int):
-            ck("cq_nn_qmatmul_norm", L.cq_nn_qmatmul_norm(int(w.dtype), w.ptr, x.data_ptr(), part.data_ptr(), norm_w.data_ptr(), cfg.rms_eps,
-                                                          dst_ptr, w.k, n, sp))
+            if pending:
+                ck("cq_nn_qmatmul_norm_merge", L.cq_nn_qmatmul_norm_merge(int(w.dtype), w.ptr, cur, planes.data_ptr(), pending,
+                                                                          norm_w.data_ptr(), cfg.rms_eps, dst_ptr, w.k, n, sp))
+            else:
+                ck("cq_nn_qmatmul_norm", L.cq_nn_qmatmul_norm(int(w.dtype), w.ptr, cur, part.data_ptr(), norm_w.data_ptr(), cfg.rms_eps,
+                                                              dst_ptr, w.k, n, sp))
 
         def resid_mm(w: _W, src_ptr: int, up_ptr: Optional[int]):
-            ck("cq_nn_qmatmul_residual", L.cq_nn_qmatmul_residual(int(w.dtype), w.ptr, src_ptr, up_ptr, x.data_ptr(), part.data_ptr(), w.k,
-                                                                  cfg.hidden, sp))
+            ck("cq_nn_qmatmul_residual_merge", L.cq_nn_qmatmul_residual_merge(int(w.dtype), w.ptr, src_ptr, up_ptr, cur, part.data_ptr(),
+                                                                              planes.data_ptr() if pending else None, pending, w.k,
+                                                                              cfg.hidden, sp))
 
-        for lw in self.layers:
+        for li, lw in enumerate(self.layers):
             w = lw.w
             wq, wk, wv = w["attention_wq"], w["attention_wk"], w["attention_wv"]
-            kq = (GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
-            if wq.dtype == wk.dtype and wk.ptr == wq.ptr + wq.nbytes:
-                if wq.dtype in kq and wv.dtype in kq:
-                    # q|k and v in one launch even though their formats differ
-                    ck("cq_nn_qmatmul_norm_pair", L.cq_nn_qmatmul_norm_pair(int(wq.dtype), wq.ptr, qd + kvd, qk.data_ptr(), int(wv.dtype), wv.ptr,
-                                                                            kvd, v.data_ptr(), x.data_ptr(), part.data_ptr(),
-                                                                            lw.attention_norm.data_ptr(), cfg.rms_eps, cfg.hidden, sp))
+            if wq.dtype == wk.dtype and wk.ptr == wq.ptr + wq.nbytes and wq.dtype in kq and wv.dtype in kq:
+                # q|k and v in one launch even though their formats differ
+                if pending:
+                    ck("cq_nn_qmatmul_norm_pair_merge", L.cq_nn_qmatmul_norm_pair_merge(
+                        int(wq.dtype), wq.ptr, qd + kvd, qk.data_ptr(), int(wv.dtype), wv.ptr, kvd, v.data_ptr(), cur, planes.data_ptr(),
+                        pending, lw.attention_norm.data_ptr(), cfg.rms_eps, cfg.hidden, sp))
                 else:
-                    norm_mm(wq, qd + kvd, lw.attention_norm, qk.data_ptr())
-                    norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
+                    ck("cq_nn_qmatmul_norm_pair", L.cq_nn_qmatmul_norm_pair(int(wq.dtype), wq.ptr, qd + kvd, qk.data_ptr(), int(wv.dtype), wv.ptr,
+                                                                            kvd, v.data_ptr(), cur, part.data_ptr(),
+                                                                            lw.attention_norm.data_ptr(), cfg.rms_eps, cfg.hidden, sp))
+            elif wq.dtype == wk.dtype and wk.ptr == wq.ptr + wq.nbytes:
+                norm_mm(wq, qd + kvd, lw.attention_norm, qk.data_ptr())
+                norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
             else:
                 norm_mm(wq, qd, lw.attention_norm, qk.data_ptr())
                 norm_mm(wk, kvd, lw.attention_norm, qk.data_ptr() + 4 * qd)
@@ -339,8 +356,7 @@ class ModelWeights:
             q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
             # rope, cache append, attention and the merge of the key splits in one kernel          :217-261
             wo = w["attention_wo"]
-            merge_in_wo = qd <= (4096 if wo.dtype in (GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K) else 2048) and \
-                (cfg.head_dim & (cfg.head_dim - 1)) == 0
+            merge_in_wo = qd <= (4096 if wo.dtype in kq else 2048) and (cfg.head_dim & (cfg.head_dim - 1)) == 0
             ck("cq_nn_attention_decode", L.cq_nn_attention_decode(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
                                                                   self.cos.data_ptr(), self.sin.data_ptr(),
                                                                   None if merge_in_wo else att.data_ptr(), pos_dev_ptr, pos,
@@ -348,24 +364,35 @@ class ModelWeights:
                                                                   self.attd_ws.data_ptr(), self.attd_ws.numel(),
                                                                   wo.ptr if self.prefetch_bytes else None,
                                                                   min(self.prefetch_bytes, lw.prefetch_span), sp))
+            # attention_wo adds to the residual row, and folds the pending planes into it
             if merge_in_wo:
-                ck("cq_nn_qmatmul_residual_attn", L.cq_nn_qmatmul_residual_attn(int(wo.dtype), wo.ptr, self.attd_ws.data_ptr(),
-                                                                                L.cq_nn_attention_decode_splits(max_kv_len), cfg.head_dim,
-                                                                                x.data_ptr(), part.data_ptr(), wo.k, cfg.hidden, sp))
+                ck("cq_nn_qmatmul_residual_attn_merge", L.cq_nn_qmatmul_residual_attn_merge(
+                    int(wo.dtype), wo.ptr, self.attd_ws.data_ptr(), L.cq_nn_attention_decode_splits(max_kv_len), cfg.head_dim, cur,
+                    part.data_ptr(), planes.data_ptr() if pending else None, pending, wo.k, cfg.hidden, sp))
             else:
                 resid_mm(wo, att.data_ptr(), None)
+            pending = 0
             w1, w3, w2 = w["feed_forward_w1"], w["feed_forward_w3"], w["feed_forward_w2"]
-            one_step = cfg.hidden <= (4096 if w1.dtype in kq else 2048)
-            if w1.dtype == w3.dtype and one_step:
+            # the consumers of this layer's residual row: the next layer's q / k / v projections, or the output head
+            nxt = self.layers[li + 1].w if li + 1 < len(self.layers) else None
+            consumers = [nxt["attention_wq"], nxt["attention_wk"], nxt["attention_wv"]] if nxt else [self.output]
+            n_split = L.cq_nn_qmatmul_split_planes(int(w2.dtype), w2.k) if self.split_w2 and cfg.hidden <= 4096 and \
+                all(one_step(c) for c in consumers) else 0
+            if w1.dtype == w3.dtype and one_step(w1):
                 # h = silu(w1 xn) * (w3 xn) straight out of the paired-row matvec                    :56-63
-                ck("cq_nn_qmatmul_norm_swiglu", L.cq_nn_qmatmul_norm_swiglu(int(w1.dtype), w1.ptr, w3.ptr, x.data_ptr(), part.data_ptr(),
+                ck("cq_nn_qmatmul_norm_swiglu", L.cq_nn_qmatmul_norm_swiglu(int(w1.dtype), w1.ptr, w3.ptr, cur, part.data_ptr(),
                                                                             lw.ffn_norm.data_ptr(), cfg.rms_eps, self.h.data_ptr(), cfg.hidden,
                                                                             cfg.ffn, sp))
-                resid_mm(w2, self.h.data_ptr(), None)
+                src_ptr, up_ptr = self.h.data_ptr(), None
             else:
                 norm_mm(w1, cfg.ffn, lw.ffn_norm, gu.data_ptr())
                 norm_mm(w3, cfg.ffn, lw.ffn_norm, gu.data_ptr() + 4 * cfg.ffn)
-                resid_mm(w2, gu.data_ptr(), gu.data_ptr() + 4 * cfg.ffn)
+                src_ptr, up_ptr = gu.data_ptr(), gu.data_ptr() + 4 * cfg.ffn
+            if n_split:
+                ck("cq_nn_qmatmul_split", L.cq_nn_qmatmul_split(int(w2.dtype), w2.ptr, src_ptr, up_ptr, planes.data_ptr(), w2.k, cfg.hidden, sp))
+                pending = n_split
+            else:
+                resid_mm(w2, src_ptr, up_ptr)
         norm_mm(self.output, cfg.vocab, self.norm, self.logits.data_ptr())
 
     def forward(self, x: torch.Tensor, index_pos: int) -> torch.Tensor:

@@ -110,6 +110,35 @@ int cq_nn_qmatmul_norm_pair(int w_dtype_a, const void *w_a_dev, int64_t n_a, flo
 int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
                                 float *residual_dev, float *sumsq_partials_out_dev, int64_t k, int64_t n, void *stream);
 
+/* A long-row matvec split along K, for feed_forward_w2 of a decode step (Mlp::forward, quantized_llama.rs:56-63, and the
+ * residual add :590-591 it feeds).  Quantizing a 14336-element activation row in every workgroup costs more than
+ * streaming the weights those workgroups read, so the row is cut into cq_nn_qmatmul_split_planes(w_dtype, k) equal
+ * slices of whole blocks (the fewest, from 2 to CQ_NN_MAX_PLANES, of at most 4096 elements for K-quants and 2048 for
+ * Q4_0 / Q8_0: 4 x 3584 for k = 14336 K-quants; 0 = not available for this k), each workgroup quantizes one slice
+ * (bit-identical: Q8_K / Q8_0 blocks are independent), and
+ *   planes[s][n] = W[:, slice s] . quantize((up ? silu(x) * up : x)[slice s]).
+ * The residual row x[n] is not touched; until the planes are merged into it every reader adds them in the fixed order
+ * ((x + planes[0]) + planes[1]) + ...:
+ *   cq_nn_qmatmul_norm_merge / _norm_pair_merge   cq_nn_qmatmul_norm / _norm_pair over that sum (sum(x^2) computed
+ *                                                 in the kernel; CQ_ERR_RANGE when k is longer than one wave step per row);
+ *   cq_nn_qmatmul_residual_merge / _residual_attn_merge   cq_nn_qmatmul_residual / _residual_attn that first add the
+ *                                                 planes to the residual row, so the row leaves merged (n_planes = 0:
+ *                                                 the plain call). */
+#define CQ_NN_MAX_PLANES 4
+int64_t cq_nn_qmatmul_split_planes(int w_dtype, int64_t k);
+int cq_nn_qmatmul_split(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *planes_dev, int64_t k, int64_t n,
+                        void *stream);
+int cq_nn_qmatmul_norm_merge(int w_dtype, const void *w_dev, const float *x_dev, const float *planes_dev, int64_t n_planes,
+                             const float *norm_weight_dev, float eps, float *dst_dev, int64_t k, int64_t n, void *stream);
+int cq_nn_qmatmul_norm_pair_merge(int w_dtype_a, const void *w_a_dev, int64_t n_a, float *dst_a_dev, int w_dtype_b, const void *w_b_dev,
+                                  int64_t n_b, float *dst_b_dev, const float *x_dev, const float *planes_dev, int64_t n_planes,
+                                  const float *norm_weight_dev, float eps, int64_t k, void *stream);
+int cq_nn_qmatmul_residual_merge(int w_dtype, const void *w_dev, const float *x_dev, const float *up_dev, float *residual_dev,
+                                 float *sumsq_partials_out_dev, const float *planes_dev, int64_t n_planes, int64_t k, int64_t n, void *stream);
+int cq_nn_qmatmul_residual_attn_merge(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,
+                                      float *residual_dev, float *sumsq_partials_out_dev, const float *planes_dev, int64_t n_planes, int64_t k,
+                                      int64_t n, void *stream);
+
 /* Greedy sampling (LogitsProcessor with Sampling::ArgMax, candle-examples/examples/quantized/main.rs:603-604):
  * token_out[0] = index of the largest logit (lowest index on ties).  Optional bookkeeping for graph replay:
  * history_dev[*counter_dev] = token; *counter_dev += 1; *pos_dev += 1.

@@ -96,6 +96,39 @@ def test_generate_greedy_graph_equals_eager_equals_oracle():
     assert a == want
 
 
+DEEP_FFN = dict(n_layer=3, hidden=256, n_head=4, n_kv_head=2, head_dim=64, ffn=4096, vocab=320, rope_theta=10000.0, rms_eps=1e-5, ctx=64)
+
+
+@pytest.mark.parametrize("dtypes", [MIX, LEGACY], ids=["q4km", "legacy"])
+def test_decode_with_split_feed_forward_w2(dtypes):
+    """ffn long enough for feed_forward_w2 to run as a K-split matvec (Q6_K / Q8_0: two 2048-element slices): the
+    planes are merged by the next layer's rms_norm prologue and by the output head."""
+    # (Q8_0 activation blocks store their scale as f16: where the f32 glue differs from the CPU's by an ulp, a scale
+    # can round the other way and move a whole block by 1e-3, so the Q4_0 / Q8_0 model is compared on a seed where
+    # none does; the split-against-unsplit comparison below does not depend on that)
+    cfg, t, model = make(DEEP_FFN, dtypes, seed=44)
+    assert model.L.cq_nn_qmatmul_split_planes(int(dtypes["feed_forward_w2"]), cfg.ffn) == 2
+    ref = lo.LlamaOracle(cfg, t, threads=8)
+    prompt = [7, 141, 59, 26, 5]
+    model.forward(torch.tensor([prompt], dtype=torch.int32), 0)
+    ref.forward(prompt, 0)
+    tok = 9
+    for step in range(3):
+        got = model.forward(torch.tensor([[tok]], dtype=torch.int32), len(prompt) + step).cpu().numpy()
+        want = ref.forward([tok], len(prompt) + step)
+        assert rel_l2(got, want) <= (TOL if dtypes is MIX else 1e-5), step
+        tok = int(np.argmax(want))
+    # and the same step with the split switched off
+    model.split_w2 = False
+    unsplit = model.forward(torch.tensor([[tok]], dtype=torch.int32), len(prompt) + 3).cpu().numpy()
+    model.split_w2 = True
+    split = model.forward(torch.tensor([[tok]], dtype=torch.int32), len(prompt) + 3).cpu().numpy()
+    assert rel_l2(split, unsplit) <= 1e-5
+    a = model.generate_greedy(prompt, 8, use_graph=True)["tokens"]
+    b = model.generate_greedy(prompt, 8, use_graph=False)["tokens"]
+    assert a == b
+
+
 def test_long_context_decode_uses_split_attention():
     # positions beyond 256 keys: more than one attention split, device-side position
     cfg, t, model = make(WIDE, MIX, seed=25)

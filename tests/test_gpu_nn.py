@@ -364,6 +364,137 @@ def test_fused_norm_pair_matvec(dta, dtb, na, nb, k):
                                        dev(part).data_ptr(), dev(nw).data_ptr(), 1e-5, k, None) == -1
 
 
+def split_planes(dtype, k):
+    """The fewest equal slices of whole blocks (2..4) that are at most one wave step long: 64 units of 64 elements for
+    K-quants, of 32 elements for Q4_0 / Q8_0."""
+    blk, unit = (256, 64) if dtype in (12, 13, 14) else (32, 32)
+    if k % blk:
+        return 0
+    for p in range(2, 5):
+        if (k // blk) % p == 0 and (k // p) // unit <= 64:
+            return p
+    return 0
+
+
+@pytest.mark.parametrize("dtype,k", [(14, 14336), (12, 14336), (14, 4096), (12, 8192), (13, 16384), (2, 4096), (8, 6144)])
+@pytest.mark.parametrize("n,with_up", [(4096, False), (300, True)])
+def test_split_matvec_planes_and_merge_consumers(dtype, k, n, with_up):
+    """feed_forward_w2 split along K: the planes add up to the unsplit matvec (each K-slice quantized exactly like the
+    CPU, so a plane equals the CPU matmul over that slice), and the rms_norm consumers that add the planes back
+    equal rms_norm + matmul over the merged row."""
+    import oracle
+    lib = L()
+    S = split_planes(dtype, k)
+    assert S >= 2 and lib.cq_nn_qmatmul_split_planes(dtype, k) == S
+    x = normal(80, (1, k), 1.0)
+    up = normal(81, (1, k), 1.0)
+    w = oracle.from_float(dtype, normal(82, (n, k), 0.02).reshape(-1))
+    planes = torch.full((S, n), 5.0, device="cuda")
+    ok(lib.cq_nn_qmatmul_split(dtype, dev(w).data_ptr(), dev(x).data_ptr(), dev(up).data_ptr() if with_up else None, planes.data_ptr(), k, n, None))
+    h = (lo.silu(x) * up).astype(np.float32) if with_up else x
+    got = planes.cpu().numpy()
+    want_total = oracle.matmul_fast(dtype, h, w, n, 8)
+    acc = np.zeros((1, n), dtype=np.float32)
+    for s_ in range(S):
+        acc = acc + got[s_:s_ + 1]
+    assert rel_l2(acc, want_total) <= (1e-4 if with_up else 1e-5)
+    # one plane on its own: the matmul over that K-slice
+    sl = k // S
+    blk_bytes, blk_elems = {2: (18, 32), 8: (34, 32), 12: (144, 256), 13: (176, 256), 14: (210, 256)}[dtype]
+    rows_b = np.asarray(w).view(np.uint8).reshape(n, k // blk_elems * blk_bytes)
+    w_slice = np.ascontiguousarray(rows_b[:, sl // blk_elems * blk_bytes:2 * sl // blk_elems * blk_bytes]).reshape(-1)
+    want1 = oracle.matmul_fast(dtype, np.ascontiguousarray(h[:, sl:2 * sl]), w_slice, n, 8)
+    assert rel_l2(got[1:2], want1) <= (1e-4 if with_up else 1e-5)
+
+    # consumers: hidden row r (length n, must be whole blocks) + planes -> rms_norm -> matvec
+    if n % 256 or S > 4:
+        return
+    r0 = normal(83, (1, n), 1.0)
+    nw = (1.0 + 0.1 * normal(84, (n,), 1.0)).astype(np.float32)
+    merged_want = r0.copy()
+    for s_ in range(S):
+        merged_want = merged_want + got[s_:s_ + 1]
+    xn = lo.rms_norm(merged_want, nw, 1e-5)
+    na, nb = 1536, 512
+    wa = oracle.from_float(12, normal(85, (na, n), 0.03).reshape(-1))
+    wb = oracle.from_float(14, normal(86, (nb, n), 0.03).reshape(-1))
+    ya, yb = torch.empty((1, na), device="cuda"), torch.empty((1, nb), device="cuda")
+    rd = dev(r0)
+    ok(lib.cq_nn_qmatmul_norm_pair_merge(12, dev(wa).data_ptr(), na, ya.data_ptr(), 14, dev(wb).data_ptr(), nb, yb.data_ptr(), rd.data_ptr(),
+                                         planes.data_ptr(), S, dev(nw).data_ptr(), 1e-5, n, None))
+    assert rel_l2(ya.cpu().numpy(), oracle.matmul_fast(12, xn, wa, na, 8)) <= 1e-3
+    assert rel_l2(yb.cpu().numpy(), oracle.matmul_fast(14, xn, wb, nb, 8)) <= 1e-3
+    assert np.array_equal(rd.cpu().numpy(), r0)                               # the residual row itself is only read
+    # single-tensor consumer (the output head); a short tensor still gets one wave per span
+    for dt_c, n_c in ((14, 2000), (12, 40)):
+        wc = oracle.from_float(dt_c, normal(87, (n_c, n), 0.03).reshape(-1))
+        yc = torch.empty((1, n_c), device="cuda")
+        ok(lib.cq_nn_qmatmul_norm_merge(dt_c, dev(wc).data_ptr(), rd.data_ptr(), planes.data_ptr(), S, dev(nw).data_ptr(), 1e-5, yc.data_ptr(),
+                                        n, n_c, None))
+        assert rel_l2(yc.cpu().numpy(), oracle.matmul_fast(dt_c, xn, wc, n_c, 8)) <= 1e-3
+    # the residual add that folds the planes into the row: row = merged + W . y, and its sum of squares
+    for up_too in (False, True):
+        kk = 512
+        y = normal(88, (1, kk), 1.0)
+        u = normal(89, (1, kk), 1.0)
+        wr = oracle.from_float(12, normal(90, (n, kk), 0.05).reshape(-1))
+        res = dev(r0)
+        part = torch.empty((256,), device="cuda")
+        ok(lib.cq_nn_qmatmul_residual_merge(12, dev(wr).data_ptr(), dev(y).data_ptr(), dev(u).data_ptr() if up_too else None, res.data_ptr(),
+                                            part.data_ptr(), planes.data_ptr(), S, kk, n, None))
+        act = (lo.silu(y) * u).astype(np.float32) if up_too else y
+        want_res = merged_want + oracle.matmul_fast(12, act, wr, n, 8)
+        got_res = res.cpu().numpy()
+        assert rel_l2(got_res, want_res) <= (1e-4 if up_too else 1e-5)
+        assert np.isclose(part.cpu().numpy().astype(np.float64).sum(), float((got_res.astype(np.float64) ** 2).sum()), rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [12, 14, 2])
+def test_attention_merge_prologue_with_planes(dtype):
+    """attention_wo fed from the attention partials, folding two pending planes into the residual row."""
+    import oracle
+    lib = L()
+    D, max_kv, k, n = 128, 512, 1024, 1024
+    splits = lib.cq_nn_attention_decode_splits(max_kv)
+    rec = D + 4
+    rng = np.random.default_rng(91)
+    Hn = k // D
+    partials = np.zeros((Hn, splits, rec), dtype=np.float32)
+    partials[:, :, :D] = rng.standard_normal((Hn, splits, D)).astype(np.float32)
+    partials[:, :, D] = rng.standard_normal((Hn, splits)).astype(np.float32)           # m
+    partials[:, :, D + 1] = rng.uniform(0.5, 2.0, (Hn, splits)).astype(np.float32)     # l
+    m = partials[:, :, D].max(axis=1, keepdims=True)
+    wgt = np.exp(partials[:, :, D] - m)
+    att = ((wgt[:, :, None] * partials[:, :, :D]).sum(axis=1) / (wgt * partials[:, :, D + 1]).sum(axis=1, keepdims=True)).reshape(1, k)
+    w = oracle.from_float(dtype, normal(92, (n, k), 0.05).reshape(-1))
+    r0 = normal(93, (1, n), 1.0)
+    pl = normal(94, (2, n), 0.5)
+    res, part = dev(r0), torch.empty((256,), device="cuda")
+    ok(lib.cq_nn_qmatmul_residual_attn_merge(dtype, dev(w).data_ptr(), dev(partials).data_ptr(), splits, D, res.data_ptr(), part.data_ptr(),
+                                             dev(pl).data_ptr(), 2, k, n, None))
+    want = ((r0 + pl[0:1]) + pl[1:2]) + oracle.matmul_fast(dtype, att.astype(np.float32), w, n, 8)
+    assert rel_l2(res.cpu().numpy(), want) <= 1e-4
+    # and without planes it is the plain call
+    res2, res3 = dev(r0), dev(r0)
+    ok(lib.cq_nn_qmatmul_residual_attn_merge(dtype, dev(w).data_ptr(), dev(partials).data_ptr(), splits, D, res2.data_ptr(), part.data_ptr(),
+                                             None, 0, k, n, None))
+    ok(lib.cq_nn_qmatmul_residual_attn(dtype, dev(w).data_ptr(), dev(partials).data_ptr(), splits, D, res3.data_ptr(), part.data_ptr(), k, n, None))
+    assert np.array_equal(res2.cpu().numpy(), res3.cpu().numpy())
+
+
+def test_split_matvec_availability():
+    lib = L()
+    assert lib.cq_nn_qmatmul_split_planes(12, 14336) == 4 and lib.cq_nn_qmatmul_split_planes(14, 14336) == 4
+    assert lib.cq_nn_qmatmul_split_planes(8, 14336) == 0          # would need 7 planes: more than a consumer adds
+    assert lib.cq_nn_qmatmul_split_planes(14, 256) == 0           # a single block: nothing to split
+    assert lib.cq_nn_qmatmul_split_planes(12, 256 * 17) == 0      # 17 blocks: no equal split into 2..4 slices
+    assert lib.cq_nn_qmatmul_split_planes(12, 256 * 1024) == 0    # slices longer than a wave step even in 4 planes
+    assert lib.cq_nn_qmatmul_split_planes(15, 4096) == 0
+    assert lib.cq_nn_qmatmul_split(12, 256, 256, None, 256, 256 * 17, 64, None) == -6
+    assert lib.cq_nn_qmatmul_norm_merge(12, 256, 256, 256, 2, 256, 1e-5, 256, 8192, 64, None) == -6
+    assert lib.cq_nn_qmatmul_norm_merge(12, 256, 256, 256, 5, 256, 1e-5, 256, 4096, 64, None) == -6
+
+
 def test_argument_validation():
     lib = L()
     assert lib.cq_nn_rms_norm(16, None, 16, None, 16, 1, 6, 1e-5, None) == -2          # dim % 4
