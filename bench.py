@@ -202,6 +202,13 @@ def moe(args):
 
     gate, up, down = [experts(F, H) for _ in range(NL)], [experts(F, H) for _ in range(NL)], [experts(H, F) for _ in range(NL)]
     router = torch.randn((E, H), generator=gen, device=dev)
+    from candle_amd.fused_moe import FusedMoeGGUF
+    from candle_amd.quantized import GgmlDType, QStorage, QTensor
+
+    def qt(buf, n, k):
+        return QTensor.new(QStorage(buf, GgmlDType.Q4K), (E, n, k))
+
+    fused = [FusedMoeGGUF(router, qt(gate[i], F, H), qt(up[i], F, H), qt(down[i], H, F), True, TOPK) for i in range(NL)]
     results = []
     for tokens in (1, 16, 256):
         x = torch.randn((tokens, H), generator=gen, device=dev)
@@ -238,12 +245,34 @@ def moe(args):
             e1.record(st)
             st.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / (reps * NL)
+        # the whole layer as FusedMoeGGUF::forward runs it: router + softmax + top-k, sort by expert, three grouped
+        # matmuls (moe_gemm_gguf), silu(gate) * up, sum over top-k
+        x3 = x.reshape(1, tokens, H)
+        y = torch.empty((tokens, H), device=dev)
+        with torch.cuda.stream(st):
+            fused[0].forward(x3, tokens > 1, out=y)
+            st.synchronize()
+            g2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g2, stream=st):
+                for i in range(NL):
+                    fused[i].forward(x3, tokens > 1, out=y)
+            g2.replay()
+            st.synchronize()
+            e0.record(st)
+            for _ in range(reps):
+                g2.replay()
+            e1.record(st)
+            st.synchronize()
+        fused_us = e0.elapsed_time(e1) * 1e3 / (reps * NL)
         alg = distinct * 3 * 884736
         results.append({"tokens": tokens, "distinct_experts": distinct, "layer_us": round(us, 1), "algorithmic_MB": round(alg / 1e6, 1),
-                        "GBps": round(alg / us / 1e3, 1), "tok_s_48_layers_expert_matmuls_only": round(tokens / (48 * us * 1e-6), 1)})
+                        "GBps": round(alg / us / 1e3, 1), "tok_s_48_layers_expert_matmuls_only": round(tokens / (48 * us * 1e-6), 1),
+                        "fused_moe_layer_us": round(fused_us, 1)})
     print(json.dumps({"metric": "Qwen3-30B-A3B-shape MoE layer, expert matmuls (Q4_K, 128 experts, top-8)", "unit": "us per layer", "n_gpus": 1,
                       "data": "synthetic", "config": {"workload": "gate + up [tokens, 2048] -> 768 and down [tokens*8, 768] -> 2048 via indexed_moe_forward, "
-                                                                  "6 distinct layers rotated (2 GB), HIP graph"},
+                                                                  "6 distinct layers rotated (2 GB), HIP graph; fused_moe_layer_us: the same "
+                                                                  "layers through FusedMoeGGUF::forward (router, top-k, sort, moe_gemm_gguf x3, "
+                                                                  "silu*up, sum over top-k)"},
                       "results": results}))
 
 

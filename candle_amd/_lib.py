@@ -48,6 +48,9 @@ SIGNATURES = {
     "cq_nn_qmatmul_residual_merge": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "cq_nn_qmatmul_residual_attn_merge": (_int, [_int, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "cq_nn_qmatmul_residual_attn": (_int, [_int, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _vp]),
+    "cq_nn_moe_route": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "cq_nn_moe_sort": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
+    "cq_nn_moe_sum": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "cq_nn_rms_norm": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "cq_nn_rope_i_kv": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "cq_nn_attention_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),

@@ -1,7 +1,8 @@
 // Decoder glue around the quantized matmuls of candle's quantized llama
 // (candle-transformers/src/models/quantized_llama.rs:191-266, 568-596): embedding lookup, residual add +
 // RMS norm, interleaved rotary embedding + KV-cache append, causal GQA attention over the cache,
-// silu(gate) * up, and greedy argmax.  All f32, like the reference's CPU path.  Token ids and the
+// silu(gate) * up, and greedy argmax; and the routing glue of the fused MoE layer (candle-transformers/src/fused_moe.rs:
+// 222-301): router + softmax + top-k, the sort of the pairs by expert, the sum over top-k.  All f32, like the reference's CPU path.  Token ids and the
 // decode position can be read from device memory so that a whole decode step (including "pick the next
 // token, advance the position") can be captured in a HIP graph and replayed without host round trips.
 #include "cq_device.h"
@@ -603,6 +604,141 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float *__restric
     }
 }
 
+// ---- MoE routing around the grouped expert matmuls (FusedMoeGGUF::forward, candle-transformers/src/fused_moe.rs:222-301) ----
+constexpr int ROUTE_MAX_EXPERTS = 1024, ROUTE_MAX_TOPK = 64;
+
+// router_logits = x . router_w^T (a bias-free f32 Linear, :233): a workgroup takes 16 experts of one token, a wave 4
+// of them, with the loads of all four rows in flight together (the router matrix of 128 x 2048 is 1 MB: one workgroup
+// per token walking it row by row would be latency-bound).
+__global__ __launch_bounds__(256) void moe_logits_kernel(const float *__restrict__ x, const float *__restrict__ router_w, float *__restrict__ logits,
+                                                         int hidden, int n_experts) {
+    const int t = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int e0 = blockIdx.x * 16 + wv * 4;
+    if (e0 >= n_experts) return;
+    const float *xr = x + (int64_t)t * hidden;
+    const float *w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) w[i] = router_w + (int64_t)min(e0 + i, n_experts - 1) * hidden;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int k = lane * 4; k < hidden; k += 256) {
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(xr + k);
+        f32x4 b[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) b[i] = *reinterpret_cast<const f32x4 *>(w[i] + k);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            acc[i] = fmaf(a.x, b[i].x, acc[i]);
+            acc[i] = fmaf(a.y, b[i].y, acc[i]);
+            acc[i] = fmaf(a.z, b[i].z, acc[i]);
+            acc[i] = fmaf(a.w, b[i].w, acc[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float v = wave_sum(acc[i]);
+        if (lane == 0 && e0 + i < n_experts) logits[(int64_t)t * n_experts + e0 + i] = v;
+    }
+}
+
+// One workgroup per token: softmax over the experts (:235-236), the topk largest probabilities in descending order
+// (:238-243; equal values: lower expert first, as the stable descending arg_sort of candle-core/src/sort.rs:48-53
+// leaves them) and the optional renormalisation (:245-247).
+__global__ __launch_bounds__(256) void moe_topk_kernel(const float *__restrict__ logits, uint32_t *__restrict__ topk_ids,
+                                                       float *__restrict__ topk_weights, int n_experts, int topk, int renorm) {
+    __shared__ float prob[ROUTE_MAX_EXPERTS];
+    __shared__ float sel[ROUTE_MAX_TOPK];
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    for (int e = tid; e < n_experts; e += 256) prob[e] = logits[(int64_t)t * n_experts + e];
+    __syncthreads();
+    // softmax_last_dim (candle-nn/src/ops.rs): max, exp(x - max), sum, divide
+    float m = -INFINITY;
+    for (int e = tid; e < n_experts; e += 256) m = fmaxf(m, prob[e]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, CQ_WAVE));
+    if (lane == 0) red[wv] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float part = 0.0f;
+    for (int e = tid; e < n_experts; e += 256) {
+        const float ex = expf(prob[e] - m);
+        prob[e] = ex;
+        part += ex;
+    }
+    const float total = block_sum_256(part, red);
+    for (int e = tid; e < n_experts; e += 256) prob[e] = prob[e] / total;
+    __syncthreads();
+    if (wv != 0) return;
+    // one wave picks the topk: every round the largest remaining probability, the lowest expert among equals
+    volatile float *vp = prob;
+    for (int j = 0; j < topk; j++) {
+        float bv = -1.0f;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < n_experts; e += 64) {
+            const float v = vp[e];
+            if (v > bv) { bv = v; bi = e; }            // ascending e within a lane: the first of equals stays
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, CQ_WAVE);
+            const int oi = __shfl_xor(bi, o, CQ_WAVE);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == 0) {
+            topk_ids[(int64_t)t * topk + j] = (uint32_t)bi;       // no finite probability left (NaN logits): an id no expert has
+            sel[j] = bv;
+            if (bi < n_experts) vp[bi] = -2.0f;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (lane == 0) {
+        float sum = 0.0f;
+        for (int j = 0; j < topk; j++) sum += sel[j];
+        for (int j = 0; j < topk; j++) topk_weights[(int64_t)t * topk + j] = renorm ? sel[j] / sum : sel[j];
+    }
+}
+
+// (expert_ids, sorted_token_ids) = topk_ids.flatten().sort_last_dim(ascending) (fused_moe.rs:249-260) as a counting
+// sort in one workgroup.  candle's sort is unstable (candle-core/src/sort.rs:282-297), so the order of the pairs
+// inside an expert's segment is unspecified there too; here it depends on the order the LDS atomics are served in.
+// Ids outside [0, n_experts) are larger than every valid id and end up behind them, unchanged.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const uint32_t *__restrict__ ids, int32_t *__restrict__ expert_ids,
+                                                        int32_t *__restrict__ sorted_token_ids, int n_pairs, int n_experts) {
+    extern __shared__ int cnt[];                 // [n_experts + 1] counts, then [n_experts + 1] running offsets
+    int *off = cnt + n_experts + 1;
+    const int tid = threadIdx.x;
+    for (int e = tid; e <= n_experts; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int p = tid; p < n_pairs; p += 1024) atomicAdd(&cnt[min(ids[p], (uint32_t)n_experts)], 1);
+    __syncthreads();
+    for (int e = tid; e <= n_experts; e += 1024) {
+        int before = 0;
+        for (int j = 0; j < e; j++) before += cnt[j];
+        off[e] = before;
+    }
+    __syncthreads();
+    for (int p = tid; p < n_pairs; p += 1024) {
+        const uint32_t id = ids[p];
+        const int pos = atomicAdd(&off[min(id, (uint32_t)n_experts)], 1);
+        expert_ids[pos] = (int32_t)id;
+        sorted_token_ids[pos] = p;
+    }
+}
+
+// ys.reshape((tokens, topk, dim)).sum(-2) (fused_moe.rs:296): the topk rows of a token added in slot order
+__global__ __launch_bounds__(256) void moe_sum_kernel(const float *__restrict__ y, float *__restrict__ out, int topk, int dim) {
+    const int t = blockIdx.y;
+    const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (c >= dim) return;
+    const float *src = y + (int64_t)t * topk * dim + c;
+    f32x4 acc = *reinterpret_cast<const f32x4 *>(src);
+    for (int j = 1; j < topk; j++) {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(src + (int64_t)j * dim);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    *reinterpret_cast<f32x4 *>(out + (int64_t)t * dim + c) = acc;
+}
+
 inline bool misaligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
 template <int HD>
@@ -809,6 +945,45 @@ int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int
     }
     hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits_dev, (int)n, token_out_dev, history_dev, counter_dev,
                        pos_dev);
+    return (int)hipGetLastError();
+}
+
+int cq_nn_moe_route(const float *x_dev, const float *router_w_dev, uint32_t *topk_ids_dev, float *topk_weights_dev, float *logits_dev,
+                    int64_t tokens, int64_t hidden, int64_t num_experts, int64_t topk, int norm_topk_prob, void *stream) {
+    if (tokens < 0 || hidden <= 0 || hidden % 4 || num_experts <= 0 || topk <= 0 || topk > num_experts) return CQ_ERR_SHAPE;
+    if (num_experts > ROUTE_MAX_EXPERTS || topk > ROUTE_MAX_TOPK || tokens > 65535 || hidden > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (tokens == 0) return CQ_OK;
+    if (!x_dev || !router_w_dev || !topk_ids_dev || !topk_weights_dev || !logits_dev) return CQ_ERR_NULL;
+    if (misaligned(x_dev, 16) || misaligned(router_w_dev, 16) || misaligned(topk_ids_dev, 4) || misaligned(topk_weights_dev, 4) ||
+        misaligned(logits_dev, 4))
+        return CQ_ERR_ALIGN;
+    hipLaunchKernelGGL(moe_logits_kernel, dim3((unsigned)((num_experts + 15) / 16), (unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x_dev,
+                       router_w_dev, logits_dev, (int)hidden, (int)num_experts);
+    hipLaunchKernelGGL(moe_topk_kernel, dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (const float *)logits_dev, topk_ids_dev,
+                       topk_weights_dev, (int)num_experts, (int)topk, norm_topk_prob);
+    return (int)hipGetLastError();
+}
+
+int cq_nn_moe_sort(const uint32_t *topk_ids_dev, int32_t *expert_ids_dev, int32_t *sorted_token_ids_dev, int64_t n_pairs, int64_t num_experts,
+                   void *stream) {
+    if (n_pairs < 0 || num_experts <= 0) return CQ_ERR_SHAPE;
+    if (num_experts > 8191 || n_pairs > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (n_pairs == 0) return CQ_OK;
+    if (!topk_ids_dev || !expert_ids_dev || !sorted_token_ids_dev) return CQ_ERR_NULL;
+    if (misaligned(topk_ids_dev, 4) || misaligned(expert_ids_dev, 4) || misaligned(sorted_token_ids_dev, 4)) return CQ_ERR_ALIGN;
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 2 * (num_experts + 1) * sizeof(int), (hipStream_t)stream, topk_ids_dev, expert_ids_dev,
+                       sorted_token_ids_dev, (int)n_pairs, (int)num_experts);
+    return (int)hipGetLastError();
+}
+
+int cq_nn_moe_sum(const float *y_dev, float *out_dev, int64_t tokens, int64_t topk, int64_t dim, void *stream) {
+    if (tokens < 0 || topk <= 0 || dim <= 0 || dim % 4) return CQ_ERR_SHAPE;
+    if (tokens > 65535 || topk > 0x7fffffffLL || dim > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (tokens == 0) return CQ_OK;
+    if (!y_dev || !out_dev) return CQ_ERR_NULL;
+    if (misaligned(y_dev, 16) || misaligned(out_dev, 16)) return CQ_ERR_ALIGN;
+    hipLaunchKernelGGL(moe_sum_kernel, dim3((unsigned)((dim / 4 + 255) / 256), (unsigned)tokens), dim3(256), 0, (hipStream_t)stream, y_dev, out_dev,
+                       (int)topk, (int)dim);
     return (int)hipGetLastError();
 }
 

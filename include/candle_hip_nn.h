@@ -147,6 +147,29 @@ int cq_nn_qmatmul_residual_attn_merge(int w_dtype, const void *w_dev, const floa
 int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
                  void *workspace_dev, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Routing glue of FusedMoeGGUF::forward (candle-transformers/src/fused_moe.rs:222-301) around the three
+ * cq_moe_gemm_gguf calls (candle_hip_quant.h):
+ * cq_nn_moe_route  router_logits = x . router_w^T (bias-free f32 Linear :233), softmax over the experts (:235-236),
+ *                  topk_ids = the topk largest probabilities in descending order (:238-241; equal values: lower
+ *                  expert first, as candle's stable descending arg_sort leaves them, candle-core/src/sort.rs:48-53),
+ *                  topk_weights = those probabilities, divided by their sum when norm_topk_prob (:243-247).
+ *                  x [tokens, hidden], router_w [num_experts, hidden], topk_ids u32 / topk_weights f32 [tokens, topk];
+ *                  logits_dev [tokens, num_experts] f32 receives the router logits (two launches: the dot products
+ *                  spread over tokens x num_experts/16 workgroups, then softmax + top-k per token).
+ *                  num_experts <= 1024, topk <= 64, tokens <= 65535 per call.
+ * cq_nn_moe_sort   (expert_ids, sorted_token_ids) = topk_ids.flatten().sort_last_dim(ascending) (:249-260): n_pairs =
+ *                  tokens * topk entries each.  The order of the pairs of one expert is unspecified, as it is with
+ *                  candle's unstable sort (candle-core/src/sort.rs:282-297); nothing downstream depends on it.
+ * cq_nn_moe_sum    out[t, :] = sum over the topk rows y[t * topk + j, :] in slot order (:296).
+ * silu(gate) * up between the calls (:281) is cq_nn_silu_mul with rows = n_pairs.
+ * ------------------------------------------------------------------------------------------- */
+int cq_nn_moe_route(const float *x_dev, const float *router_w_dev, uint32_t *topk_ids_dev, float *topk_weights_dev, float *logits_dev,
+                    int64_t tokens, int64_t hidden, int64_t num_experts, int64_t topk, int norm_topk_prob, void *stream);
+int cq_nn_moe_sort(const uint32_t *topk_ids_dev, int32_t *expert_ids_dev, int32_t *sorted_token_ids_dev, int64_t n_pairs, int64_t num_experts,
+                   void *stream);
+int cq_nn_moe_sum(const float *y_dev, float *out_dev, int64_t tokens, int64_t topk, int64_t dim, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
