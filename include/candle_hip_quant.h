@@ -146,8 +146,8 @@ int cq_indexed_moe_forward(int w_dtype, const void *w_dev, const float *x_dev, c
  *   out[tok, :] = (topk_weights ? topk_weights[tok] : 1) * W[e] . x[in_row, :]
  *   x [size_m or size_m/topk, k] f32, out [size_m, n] f32, sorted_token_ids / expert_ids int32 [size_m]
  *   (both device pointers), topk_weights f32 [size_m] device pointer or NULL.
- * `is_prefill` selects the MFMA grouped kernel (the reference's WMMA prefill kernel) instead of the
- * expert-grouped matvec; both give the same values up to f32 summation order.
+ * `is_prefill` does not change the result: the number of pairs selects the kernel (as for cq_indexed_moe_forward
+ * above), and every path quantizes the activations like candle's CPU path.
  * ------------------------------------------------------------------------------------------- */
 int64_t cq_moe_gemm_workspace_bytes(int w_dtype, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int has_topk_weights);
 int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const int32_t *sorted_token_ids_dev,
