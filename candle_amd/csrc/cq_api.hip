@@ -250,6 +250,24 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
     return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
 }
 
+int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_dev, const void *w_up_dev, const int32_t *sorted_token_ids_dev,
+                            const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
+                            int64_t k, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, size_m);
+    if (rc) return rc;
+    if (num_experts <= 0 || topk <= 0 || size_m % topk != 0) return CQ_ERR_SHAPE;
+    if (num_experts > (1 << 20) || size_m > CQ_MOE_DIRECT_MAX_PAIRS) return CQ_ERR_RANGE;
+    if (size_m == 0 || n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_gate_dev)) || (rc = check_weight_ptr(w_dtype, w_up_dev))) return rc;
+    if (!x_dev || !sorted_token_ids_dev || !expert_ids_dev || !out_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(sorted_token_ids_dev, 4) || !aligned(expert_ids_dev, 4) || !aligned(out_dev, 4)) return CQ_ERR_ALIGN;
+    PairSource ps;
+    ps.mode = MOE_SORTED; ps.ids_u32 = nullptr; ps.sorted_token_ids = sorted_token_ids_dev; ps.expert_ids = expert_ids_dev;
+    ps.topk_weights = nullptr; ps.topk = (int)topk; ps.input_dim1 = 0;
+    ps.n_pairs = (int)size_m; ps.num_experts = (int)num_experts; ps.x_rows = (int)(size_m / topk);
+    return cq_moe_pairs_swiglu_launch(w_dtype, w_gate_dev, w_up_dev, x_dev, out_dev, ps, k, n, (hipStream_t)stream);
+}
+
 // ---- single-row decoder fusions, declared in include/candle_hip_nn.h ----
 int cq_nn_qmatmul_norm(int w_dtype, const void *w_dev, const float *x_dev, const float *sumsq_partials_dev, const float *norm_weight_dev,
                        float eps, float *dst_dev, int64_t k, int64_t n, void *stream) {

@@ -99,6 +99,8 @@ __device__ __forceinline__ bool pair_decode(const PairSource &ps, int p, int &e,
 #define CQ_MOE_DIRECT_MAX_PAIRS 256
 // CQ_ERR_RANGE when the shape is not served by the fused kernel (the caller then takes the grouped path).
 int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s);
+int cq_moe_pairs_swiglu_launch(int w_dtype, const void *w_gate, const void *w_up, const float *x, float *out, const PairSource &ps, int64_t k,
+                               int64_t n, hipStream_t s);
 
 int cq_quantize_act_gather_launch(int w_dtype, const float *x, const int *row_map, void *scratch, int64_t k, int64_t rows, int64_t rows_alloc,
                                   hipStream_t s);

@@ -1015,9 +1015,11 @@ int cq_matvec_ksplit_launch(int w_dtype, const void *w, const float *x, const fl
 
 // ---- MoE with few pairs: block (tile, pair) is one fused matvec over the pair's expert ----
 namespace {
-template <int DT, bool SINGLE>
+// SWIGLU: w is the gate expert tensor, the up experts lie pair_off bytes behind it, and the pair's row is
+// silu(gate . x) * (up . x) (rows of one wave step only).
+template <int DT, bool SINGLE, bool SWIGLU = false>
 __global__ __launch_bounds__(1024) void moe_pair_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out, QmvGeom g,
-                                                        PairSource ps, int64_t expert_bytes) {
+                                                        PairSource ps, int64_t expert_bytes, int64_t pair_off) {
     const int p = blockIdx.y;
     int e, in_row, out_row;
     float scale;
@@ -1029,14 +1031,16 @@ __global__ __launch_bounds__(1024) void moe_pair_kernel(const uint8_t *__restric
         return;
     }
     ActSrc src{x + (int64_t)in_row * g.k, ActView{nullptr, nullptr, nullptr}};
-    Fuse fz{nullptr, nullptr, scale, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
-    qmv_body<DT, 1, CQ_F32, SINGLE, PRO_NONE, EPI_SCALE, false>(w + (int64_t)e * expert_bytes, src, out + (int64_t)out_row * g.n, g, fz,
-                                                                blockIdx.x, gridDim.x);
+    Fuse fz{nullptr, nullptr, scale, nullptr, nullptr, 0, 0, pair_off, nullptr, nullptr, 0};
+    qmv_body<DT, 1, CQ_F32, SINGLE, PRO_NONE, SWIGLU ? EPI_SWIGLU : EPI_SCALE, false>(w + (int64_t)e * expert_bytes, src,
+                                                                                      out + (int64_t)out_row * g.n, g, fz, blockIdx.x, gridDim.x);
 }
 
 template <int DT>
-int launch_moe_pairs(const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s) {
+int launch_moe_pairs(const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s, bool swiglu = false,
+                     int64_t pair_off = 0) {
     if (cq_act_layout(DT, k, 1).total > LDS_BUDGET) return CQ_ERR_RANGE;
+    if (swiglu && k / Fmt<DT>::UE > 64) return CQ_ERR_RANGE;         // the paired-row epilogue is for rows of one wave step
     QmvGeom g;
     int64_t groups;
     size_t lds_bytes;
@@ -1044,22 +1048,26 @@ int launch_moe_pairs(const void *w, const float *x, float *out, const PairSource
     int waves = (int64_t)ps.n_pairs * n >= 256 * 16 ? 16 : 0;
     // about a thousand workgroups in total: with many pairs each workgroup takes more rows of its expert, so that
     // the activation prologue is paid once per many rows
-    const int64_t per_pair = (1024 + ps.n_pairs - 1) / ps.n_pairs;
+    const int64_t per_pair = ((swiglu ? 2048 : 1024) + ps.n_pairs - 1) / ps.n_pairs;
     int rc = make_geom<DT, 1>(g, groups, waves, k, n, n, CQ_F32, 0, lds_bytes, per_pair < 256 ? per_pair : 256);
     if (rc) return rc;
     if (ps.n_pairs > 65535) return CQ_ERR_RANGE;
     const int64_t expert_bytes = n * (int64_t)g.row_bytes;
     const bool single = k / Fmt<DT>::UE <= 64;
-    const void *kp = single ? (const void *)moe_pair_kernel<DT, true> : (const void *)moe_pair_kernel<DT, false>;
+    const void *kp = swiglu   ? (const void *)moe_pair_kernel<DT, true, true>
+                     : single ? (const void *)moe_pair_kernel<DT, true>
+                              : (const void *)moe_pair_kernel<DT, false>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
     }
     dim3 grid((unsigned)groups, (unsigned)ps.n_pairs), block(64 * waves);
-    if (single)
-        hipLaunchKernelGGL((moe_pair_kernel<DT, true>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes);
+    if (swiglu)
+        hipLaunchKernelGGL((moe_pair_kernel<DT, true, true>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes, pair_off);
+    else if (single)
+        hipLaunchKernelGGL((moe_pair_kernel<DT, true>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes, (int64_t)0);
     else
-        hipLaunchKernelGGL((moe_pair_kernel<DT, false>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes);
+        hipLaunchKernelGGL((moe_pair_kernel<DT, false>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes, (int64_t)0);
     return (int)hipGetLastError();
 }
 }  // namespace
@@ -1072,6 +1080,22 @@ int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, 
         case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w, x, out, ps, k, n, s);
         case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w, x, out, ps, k, n, s);
         case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w, x, out, ps, k, n, s);
+    }
+    return CQ_ERR_DTYPE;
+}
+
+// out[pair, :] = silu(W_gate[e] . x) * (W_up[e] . x) for at most CQ_MOE_DIRECT_MAX_PAIRS pairs; the two expert tensors have one
+// shape and format.  CQ_ERR_RANGE when a row is longer than one wave step.
+int cq_moe_pairs_swiglu_launch(int w_dtype, const void *w_gate, const void *w_up, const float *x, float *out, const PairSource &ps, int64_t k,
+                               int64_t n, hipStream_t s) {
+    if (ps.n_pairs == 0 || n == 0) return CQ_OK;
+    const int64_t off = (const uint8_t *)w_up - (const uint8_t *)w_gate;
+    switch (w_dtype) {
+        case CQ_Q4_0: return launch_moe_pairs<CQ_Q4_0>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q8_0: return launch_moe_pairs<CQ_Q8_0>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w_gate, x, out, ps, k, n, s, true, off);
     }
     return CQ_ERR_DTYPE;
 }

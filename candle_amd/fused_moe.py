@@ -95,14 +95,23 @@ class FusedMoeGGUF:
                                                       tw_ptr, out_t.data_ptr(), E, topk, pairs, n, k, 1 if is_prefill else 0,
                                                       self.ws.data_ptr(), self.ws.numel(), sp))
 
-        gemm(x2.data_ptr(), self.gate_experts, None, self.gate_out, self.inter, hidden)
-        gemm(x2.data_ptr(), self.up_experts, None, self.up_out, self.inter, hidden)
-        # up * silu(gate), in chunks of rows the elementwise launch takes
-        for r0 in range(0, pairs, 65535):
-            r = min(65535, pairs - r0)
-            off = 4 * r0 * self.inter
-            ck("cq_nn_silu_mul", L.cq_nn_silu_mul(self.gate_out.data_ptr() + off, self.up_out.data_ptr() + off, self.down_in.data_ptr() + off, r,
-                                                  self.inter, self.inter, self.inter, sp))
+        # decode-sized calls: gate, up and the activation in one launch
+        fused = -6
+        if pairs <= 256:
+            fused = L.cq_moe_gemm_gguf_swiglu(dt, x2.data_ptr(), self.gate_experts.device_ptr(), self.up_experts.device_ptr(),
+                                              self.sorted_token_ids.data_ptr(), self.expert_ids.data_ptr(), self.down_in.data_ptr(), E, topk,
+                                              pairs, self.inter, hidden, sp)
+            if fused != -6:
+                ck("cq_moe_gemm_gguf_swiglu", fused)
+        if fused == -6:                                          # CQ_ERR_RANGE: not a shape of the fused launch
+            gemm(x2.data_ptr(), self.gate_experts, None, self.gate_out, self.inter, hidden)
+            gemm(x2.data_ptr(), self.up_experts, None, self.up_out, self.inter, hidden)
+            # up * silu(gate), in chunks of rows the elementwise launch takes
+            for r0 in range(0, pairs, 65535):
+                r = min(65535, pairs - r0)
+                off = 4 * r0 * self.inter
+                ck("cq_nn_silu_mul", L.cq_nn_silu_mul(self.gate_out.data_ptr() + off, self.up_out.data_ptr() + off, self.down_in.data_ptr() + off,
+                                                      r, self.inter, self.inter, self.inter, sp))
         gemm(self.down_in.data_ptr(), self.down_experts, self.topk_weights.data_ptr(), self.down_out, hidden, self.inter)
         for t0 in range(0, tokens, 65535):
             t = min(65535, tokens - t0)

@@ -155,6 +155,15 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
                      int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int is_prefill,
                      void *workspace_dev, int64_t workspace_bytes, void *stream);
 
+/* The gate and up matmuls of FusedMoeGGUF::forward with its activation (candle-transformers/src/fused_moe.rs:263-281: two
+ * moe_gemm_gguf calls without topk_weights, then up * silu(gate)) in one launch, for decode-sized calls:
+ *   out[tok, :] = silu(W_gate[e] . x[tok / topk, :]) * (W_up[e] . x[tok / topk, :])
+ * w_gate / w_up [num_experts, n, k] of one format.  CQ_ERR_RANGE (use the two calls and cq_nn_silu_mul) when
+ * size_m > 256 or k is longer than one wave step per row (4096 for K-quants, 2048 for Q4_0 / Q8_0).  Needs no workspace. */
+int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_dev, const void *w_up_dev, const int32_t *sorted_token_ids_dev,
+                            const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
+                            int64_t k, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

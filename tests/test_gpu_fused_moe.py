@@ -80,6 +80,36 @@ def test_sum_kernel():
     assert np.array_equal(out.cpu().numpy(), acc)
 
 
+@pytest.mark.parametrize("dtype,k", [(oracle.Q4K, 2048), (oracle.Q6K, 512), (oracle.Q8_0, 1024)])
+@pytest.mark.parametrize("tokens", [1, 5, 32])
+def test_gate_up_swiglu_in_one_launch(dtype, k, tokens):
+    """cq_moe_gemm_gguf_swiglu == moe_gemm_gguf(gate), moe_gemm_gguf(up), up * silu(gate) of the oracle."""
+    from oracle.llama_oracle import silu
+    E, n, topk = 16, 384, 4
+    pairs = tokens * topk
+    gate_b = oracle.from_float(dtype, normal(70, E * n * k, 0.05))
+    up_b = oracle.from_float(dtype, normal(71, E * n * k, 0.05))
+    x = normal(72, (tokens, k), 1.0)
+    rng = np.random.default_rng(73)
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(tokens)]).astype(np.uint32)
+    expert_ids, sorted_token_ids = fm.sort_pairs(ids)
+    g = oracle.moe_gemm_gguf(dtype, x, gate_b, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+    u = oracle.moe_gemm_gguf(dtype, x, up_b, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+    want = (u * silu(g)).astype(np.float32)
+    both = torch.from_numpy(np.concatenate([up_b, gate_b])).cuda()          # up in front of gate: a negative distance
+    out = torch.full((pairs, n), 7.0, device="cuda")
+    xd = torch.from_numpy(x).cuda()
+    ed, sd = torch.from_numpy(expert_ids).cuda(), torch.from_numpy(sorted_token_ids).cuda()
+    assert L().cq_moe_gemm_gguf_swiglu(dtype, xd.data_ptr(), both.data_ptr() + up_b.size, both.data_ptr(), sd.data_ptr(), ed.data_ptr(),
+                                       out.data_ptr(), E, topk, pairs, n, k, None) == 0
+    assert rel_l2(out.cpu().numpy(), want) <= 1e-5
+    # more pairs than the fused launch takes, or rows of more than one wave step: the caller falls back
+    assert L().cq_moe_gemm_gguf_swiglu(dtype, xd.data_ptr(), both.data_ptr(), both.data_ptr(), sd.data_ptr(), ed.data_ptr(), out.data_ptr(),
+                                       E, topk, 260, n, k, None) == -6
+    assert L().cq_moe_gemm_gguf_swiglu(dtype, xd.data_ptr(), both.data_ptr(), both.data_ptr(), sd.data_ptr(), ed.data_ptr(), out.data_ptr(),
+                                       E, topk, pairs, n, 8192, None) == -6
+
+
 def build_layer(dtype, E, hidden, inter, topk, norm, seed):
     from candle_amd.fused_moe import FusedMoeGGUF
     from candle_amd.quantized import GgmlDType, QStorage, QTensor
