@@ -116,7 +116,12 @@ struct MoeChunks {
 int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k,
                          int64_t n, hipStream_t s);
 
-// Pairs from which a K-quant MoE call goes through the MFMA kernel (tiles of up to 128 expert-sorted rows).
-#define CQ_MOE_MFMA_MIN_PAIRS 1024
+// Pairs from which a K-quant MoE call goes through the MFMA kernel (tiles of expert-sorted rows): everything the
+// per-pair kernels do not take.  Measured on 128 experts of 768 x 2048: 264-1016 pairs take 211-229 us per layer on
+// 32-row tiles against 427-644 us on the 8-pairs-per-pass matvec.
+#define CQ_MOE_MFMA_MIN_PAIRS 257
+// rows of one MFMA tile of an expert: the small tile while experts average fewer than 64 rows
+#define CQ_MOE_TILE_SMALL 32
+#define CQ_MOE_TILE_LARGE 128
 int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k, int64_t n,
-                         hipStream_t s);
+                         int tile_rows, hipStream_t s);

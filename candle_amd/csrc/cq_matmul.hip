@@ -274,25 +274,29 @@ __device__ __forceinline__ void lds_write32h(_Float16 *dstrow, const uint32_t v[
 
 // NJ = 32-column MFMA tiles per wave: block tile 128 x (64 * NJ).  NJ = 1 halves the accumulators so that two
 // workgroups share a CU and one converts operands while the other feeds the matrix cores.
-// MOE: blockIdx.x is a tile of the chunk table: up to 128 expert-sorted activation rows [first, first + count) of
+// MOE: blockIdx.x is a tile of the chunk table: up to BMT expert-sorted activation rows [first, first + count) of
 // expert e; the weights are that expert's [n, k] matrix and output rows are scattered through pair_out with pair_scale.
-template <int DT, int NJ, bool MOE = false>
+// SM (experts with few rows each): the block tile is 32 (m) x 128 (n), the four waves side by side along n, so that a
+// 16-row expert fills half of its tiles instead of an eighth, and one workgroup converts twice the weight rows per stage.
+template <int DT, int NJ, bool MOE = false, bool SM = false>
 __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k,
                                                                      int n, int rows, int64_t stride_dst, MoeChunks mc, int64_t expert_bytes,
                                                                      int64_t split_stride) {
     typedef Stage<DT> S;
     constexpr bool KQ = S::KQ;
-    constexpr int BN = 64 * NJ, WN = 32 * NJ;
-    __shared__ __align__(16) _Float16 As[BM * LDK];
+    static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
+    constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;             // rows of the block tile, 32-row MFMA tiles per wave
+    constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
+    __shared__ __align__(16) _Float16 As[BMT * LDK];
     __shared__ __align__(16) _Float16 Bs[BN * LDK];
     __shared__ __align__(16) _Float16 Bs2[S::TERMS == 2 ? BN * LDK : 8];   // exact remainders of a two-term format
-    __shared__ __align__(16) _Float16 Am[BM * 24];    // bsums16 of the super-block, as f16 (row stride 24 halves)
+    __shared__ __align__(16) _Float16 Am[BMT * 24];   // bsums16 of the super-block, as f16 (row stride 24 halves)
     __shared__ __align__(16) _Float16 Bm[BN * 24];    // sub-block mins duplicated per 16-element group
-    __shared__ float sD[BN], sDmin[BN], sD8[BM];
+    __shared__ float sD[BN], sDmin[BN], sD8[BMT];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const int wm = wv >> 1, wn = wv & 1;
-    int m0 = blockIdx.x * BM;
+    const int wm = SM ? 0 : wv >> 1, wn = SM ? wv : wv & 1;
+    int m0 = blockIdx.x * BMT;
     const int n0 = blockIdx.y * BN;
     if (MOE) {
         if ((int)blockIdx.x >= mc.n_chunks[0]) return;           // uniform over the workgroup
@@ -301,6 +305,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
     }
     const bool bstage = tid < 2 * BN;                            // threads that also stage a weight row (wave-uniform)
+    const bool astage = tid < 2 * BMT;                           // threads that stage an activation row (wave-uniform)
     // split-K: blockIdx.z takes an equal share of the 256-element spans and writes its own partial plane
     const int nsb_all = k >> 8;
     const int kb0 = (int)(((int64_t)nsb_all * blockIdx.z) / gridDim.z), nsb = (int)(((int64_t)nsb_all * (blockIdx.z + 1)) / gridDim.z);
@@ -310,14 +315,14 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     // staging role of this thread: (row r_l of the tile, 32-element half)
     const int r_l = tid >> 1, half = tid & 1;
     const int wrow = min(n0 + (bstage ? r_l : 0), n - 1);
-    const int arow = min(m0 + r_l, rows - 1);
-    const bool arow_ok = m0 + r_l < rows;
+    const int arow = min(m0 + (astage ? r_l : 0), rows - 1);
+    const bool arow_ok = astage && m0 + r_l < rows;
     const uint8_t *wrow_p = w + wrow * row_bytes;
     const int8_t *aq_p = av.qs + (int64_t)arow * k;
 
-    f32x16 acc[2][NJ], sb[2][NJ];
+    f32x16 acc[MI][NJ], sb[MI][NJ];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < NJ; j++)
 #pragma unroll
@@ -329,9 +334,11 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     u32x4 a02[2], a12[2];
     auto load_stage = [&](int kb, int g, typename S::Raw &wr, u32x4 &x0, u32x4 &x1) {
         if (bstage) S::load(wr, wrow_p, kb, g, half);
-        const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
-        x0 = *reinterpret_cast<const u32x4 *>(q);
-        x1 = *reinterpret_cast<const u32x4 *>(q + 16);
+        if (astage) {
+            const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
+            x0 = *reinterpret_cast<const u32x4 *>(q);
+            x1 = *reinterpret_cast<const u32x4 *>(q + 16);
+        }
     };
     load_stage(kb0, 0, wraw2[0], a02[0], a12[0]);
     load_stage(kb0, 1, wraw2[1], a02[1], a12[1]);
@@ -353,24 +360,26 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
                 }
                 lds_write32h(Bs + r_l * LDK + 32 * half, hv);
             }
-            uint32_t ascale2 = 0;
-            if (!KQ) {
-                float d8 = av.d[2 * ((int64_t)arow * (k >> 5) + kb * 8 + 2 * g + half)];   // already f16-representable
-                ascale2 = h2_splat(d8);
-            }
-            act_convert(a0, a1, !KQ, ascale2, hv);
-            if (!arow_ok) {
+            if (astage) {
+                uint32_t ascale2 = 0;
+                if (!KQ) {
+                    float d8 = av.d[2 * ((int64_t)arow * (k >> 5) + kb * 8 + 2 * g + half)];   // already f16-representable
+                    ascale2 = h2_splat(d8);
+                }
+                act_convert(a0, a1, !KQ, ascale2, hv);
+                if (!arow_ok) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) hv[i] = 0;
+                    for (int i = 0; i < 16; i++) hv[i] = 0;
+                }
+                lds_write32h(As + r_l * LDK + 32 * half, hv);
             }
-            lds_write32h(As + r_l * LDK + 32 * half, hv);
             if (KQ && g == 0) {
                 float d = 0.0f, dmin = 0.0f;
                 int mins[8] = {0, 0, 0, 0, 0, 0, 0, 0};
                 if (bstage) S::header(wraw, d, dmin, mins);
                 if (half == 0) {
                     if (bstage) { sD[r_l] = d; sDmin[r_l] = dmin; }
-                    sD8[r_l] = arow_ok ? av.d[(int64_t)arow * (k >> 8) + kb] : 0.0f;
+                    if (astage) sD8[r_l] = arow_ok ? av.d[(int64_t)arow * (k >> 8) + kb] : 0.0f;
                 }
                 if (S::HAS_MIN) {
                     // Bm[n][j] = min[j/2] for j in 8*half .. 8*half+7 ; Am[m][j] = bsums16[j]
@@ -381,15 +390,17 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
                         mv[i] = hm | (hm << 16);
                     }
                     if (bstage) *reinterpret_cast<u32x4 *>(Bm + r_l * 24 + 8 * half) = u32x4{mv[0], mv[1], mv[2], mv[3]};
-                    u32x4 bs = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
-                    const uint32_t b4[4] = {bs.x, bs.y, bs.z, bs.w};
-                    uint32_t bv[4];
+                    if (astage) {
+                        u32x4 bs = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
+                        const uint32_t b4[4] = {bs.x, bs.y, bs.z, bs.w};
+                        uint32_t bv[4];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        uint32_t lo = f2h_bits((float)(int16_t)(b4[i] & 0xffff)), hi = f2h_bits((float)(int16_t)(b4[i] >> 16));
-                        bv[i] = arow_ok ? (lo | (hi << 16)) : 0u;
+                        for (int i = 0; i < 4; i++) {
+                            uint32_t lo = f2h_bits((float)(int16_t)(b4[i] & 0xffff)), hi = f2h_bits((float)(int16_t)(b4[i] >> 16));
+                            bv[i] = arow_ok ? (lo | (hi << 16)) : 0u;
+                        }
+                        *reinterpret_cast<u32x4 *>(Am + r_l * 24 + 8 * half) = u32x4{bv[0], bv[1], bv[2], bv[3]};
                     }
-                    *reinterpret_cast<u32x4 *>(Am + r_l * 24 + 8 * half) = u32x4{bv[0], bv[1], bv[2], bv[3]};
                 }
             }
             __syncthreads();
@@ -401,15 +412,15 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
             // ---- 4 k-slices of 16: 2 x 2 MFMA tiles per wave ----
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                half8 af[2], bf[NJ];
+                half8 af[MI], bf[NJ];
 #pragma unroll
-                for (int t = 0; t < 2; t++)
+                for (int t = 0; t < MI; t++)
                     af[t] = *reinterpret_cast<const half8 *>(As + (wm * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
                 for (int t = 0; t < NJ; t++)
                     bf[t] = *reinterpret_cast<const half8 *>(Bs + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+                for (int i = 0; i < MI; i++)
 #pragma unroll
                     for (int j = 0; j < NJ; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
                 if constexpr (S::TERMS == 2) {
@@ -417,24 +428,24 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
                     for (int t = 0; t < NJ; t++)
                         bf[t] = *reinterpret_cast<const half8 *>(Bs2 + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
-                    for (int i = 0; i < 2; i++)
+                    for (int i = 0; i < MI; i++)
 #pragma unroll
                         for (int j = 0; j < NJ; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
                 }
             }
             if (KQ && g == 3) {
                 // ---- end of the super-block: mins term and the f32 scales ----
-                f32x16 mt[2][NJ];
+                f32x16 mt[MI][NJ];
                 if (S::HAS_MIN) {
-                    half8 am[2], bm[NJ];
+                    half8 am[MI], bm[NJ];
 #pragma unroll
-                    for (int t = 0; t < 2; t++)
+                    for (int t = 0; t < MI; t++)
                         am[t] = *reinterpret_cast<const half8 *>(Am + (wm * 64 + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
 #pragma unroll
                     for (int t = 0; t < NJ; t++)
                         bm[t] = *reinterpret_cast<const half8 *>(Bm + (wn * WN + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
 #pragma unroll
-                    for (int i = 0; i < 2; i++)
+                    for (int i = 0; i < MI; i++)
 #pragma unroll
                         for (int j = 0; j < NJ; j++) {
                             f32x16 z;
@@ -448,7 +459,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
                     const int nl = wn * WN + j * 32 + (lane & 31);
                     const float d = sD[nl], dmin = sDmin[nl];
 #pragma unroll
-                    for (int i = 0; i < 2; i++) {
+                    for (int i = 0; i < MI; i++) {
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
                             const int ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
@@ -466,7 +477,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
 
     // ---- epilogue: C layout of the 32x32 tile: column = lane % 32, row = 8*(e/4) + 4*(lane/32) + e%4 ----
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
             const int nn = n0 + wn * WN + j * 32 + (lane & 31);
@@ -551,26 +562,33 @@ int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t co
 
 namespace {
 template <int DT>
-int launch_qmm_moe(const void *w, const ActView &av, float *out, const MoeChunks &mc, int64_t k, int64_t n, hipStream_t s) {
-    dim3 grid((unsigned)mc.max_chunks, (unsigned)((n + 63) / 64));
+int launch_qmm_moe(const void *w, const ActView &av, float *out, const MoeChunks &mc, int64_t k, int64_t n, int tile_rows, hipStream_t s) {
+    const int bn = tile_rows == 32 ? 128 : 64;
+    dim3 grid((unsigned)mc.max_chunks, (unsigned)((n + bn - 1) / bn));
     if (grid.y > 65535) return CQ_ERR_RANGE;
     const int64_t expert_bytes = n * (k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
-    hipLaunchKernelGGL((qmm_kernel<DT, 1, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc, expert_bytes,
-                       (int64_t)0);
+    if (tile_rows == 32)
+        hipLaunchKernelGGL((qmm_kernel<DT, 1, true, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc,
+                           expert_bytes, (int64_t)0);
+    else
+        hipLaunchKernelGGL((qmm_kernel<DT, 1, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc, expert_bytes,
+                           (int64_t)0);
     return (int)hipGetLastError();
 }
 
 }  // namespace
 
+// tile_rows: rows of one chunk of the table, CQ_MOE_TILE_SMALL (32) or CQ_MOE_TILE_LARGE (128)
 int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k, int64_t n,
-                         hipStream_t s) {
+                         int tile_rows, hipStream_t s) {
     if (mc.max_chunks == 0 || n == 0) return CQ_OK;
     if (k % 256) return CQ_ERR_SHAPE;
+    if (tile_rows != CQ_MOE_TILE_SMALL && tile_rows != CQ_MOE_TILE_LARGE) return CQ_ERR_RANGE;
     ActView av = cq_act_view(scratch, w_dtype, k, rows_alloc);
     switch (w_dtype) {
-        case CQ_Q4K: return launch_qmm_moe<CQ_Q4K>(w, av, out, mc, k, n, s);
-        case CQ_Q5K: return launch_qmm_moe<CQ_Q5K>(w, av, out, mc, k, n, s);
-        case CQ_Q6K: return launch_qmm_moe<CQ_Q6K>(w, av, out, mc, k, n, s);
+        case CQ_Q4K: return launch_qmm_moe<CQ_Q4K>(w, av, out, mc, k, n, tile_rows, s);
+        case CQ_Q5K: return launch_qmm_moe<CQ_Q5K>(w, av, out, mc, k, n, tile_rows, s);
+        case CQ_Q6K: return launch_qmm_moe<CQ_Q6K>(w, av, out, mc, k, n, tile_rows, s);
     }
     return CQ_ERR_DTYPE;
 }

@@ -211,13 +211,14 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     // Hundreds of pairs per call on K-quant experts: the expert-sorted rows go through the MFMA prefill kernel in tiles
     // of up to 128 rows of one expert (integer-exact like the other K-quant paths).  Otherwise 8 pairs per matvec pass.
     const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
+    const int tile_rows = a.n_pairs < 64 * a.num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
-                       (int)ws.max_chunks, mfma ? 128 : CQ_MOE_CHUNK);
+                       (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);
     if ((rc = (int)hipGetLastError())) return rc;
     if (mfma) {
         if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;
         MoeChunks mc{chunks, chunks + 1, chunks + 1 + ws.max_chunks, chunks + 1 + 2 * ws.max_chunks, pout, pscale, (int)ws.max_chunks};
-        return cq_matmul_moe_launch(a.w_dtype, a.w, b + ws.act_off, ws.rows_alloc, a.out, mc, a.k, a.n, s);
+        return cq_matmul_moe_launch(a.w_dtype, a.w, b + ws.act_off, ws.rows_alloc, a.out, mc, a.k, a.n, tile_rows, s);
     }
     if (a.k % 256 == 0) {
         // Many pairs: activation rows quantized in expert-sorted order, then CQ_MOE_CHUNK pairs of an expert per pass

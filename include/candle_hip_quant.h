@@ -130,7 +130,8 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
  *   ids [batch, topk] u32  ->  out [batch, topk, n] f32,
  *   out[b, t, :] = W[ids[b, t]] . x[b, input_dim1 == 1 ? 0 : t, :].
  * Up to 256 pairs each pair is its own fused matvec; beyond, pairs are grouped by expert on the device and an expert's
- * rows are streamed once per 8 pairs (from 1024 pairs on K-quant experts: once per 128 pairs, on the matrix cores).
+ * rows are streamed once per tile of 32 or 128 pairs on the matrix cores (K-quant experts; integer-exact) or once per
+ * 8 pairs by the matvec kernel (Q4_0 / Q8_0 experts).
  * An id >= num_experts leaves its output row zero-filled.
  * ------------------------------------------------------------------------------------------- */
 int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk, int64_t input_dim1);

@@ -58,7 +58,7 @@ def test_indexed_moe_forward(dtype, input_dim1_is_one):
 
 @pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("tokens", [1, 16, 40, 100, 300])  # <= 256 pairs: a fused matvec per pair; beyond: grouped by expert, 8 pairs per
-                                                           # pass; from 1024 pairs on K-quants: expert tiles through the MFMA kernel
+                                                           # pass (Q4_0 / Q8_0) or expert tiles of 32 / 128 rows through the MFMA kernel (K-quants)
 @pytest.mark.parametrize("is_prefill", [False, True])
 def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     """The two call shapes of FusedMoeGGUF::forward (fused_moe.rs:263-294): gate/up without
@@ -85,6 +85,24 @@ def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     want2 = oracle.moe_gemm_gguf(dtype, x2, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
     err2 = rel_l2(got2.cpu().numpy(), want2)
     assert err2 <= TOL and err2 <= TIGHT, err2
+
+
+@pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q5K, oracle.Q6K], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("E,n", [(64, 160), (8, 160)])      # 1200 pairs: about 19 rows per expert (32-row tiles of the MFMA
+                                                            # kernel, 128 weight rows wide) or 150 (128-row tiles); n is ragged
+def test_moe_gemm_gguf_mfma_tile_sizes(dtype, E, n):
+    import candle_amd as ca
+    k, topk, tokens = 512, 4, 300
+    blocks, qt = make_experts(dtype, E, n, k, seed=65)
+    ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=66)
+    sti, eid = torch.from_numpy(sorted_token_ids).cuda(), torch.from_numpy(expert_ids).cuda()
+    x2 = normal(67, (tokens * topk, k), 1.0)
+    twf = tw.reshape(-1)
+    got = ca.moe_gemm_gguf(torch.from_numpy(x2).cuda(), qt, torch.from_numpy(twf).cuda(), sti, eid, topk, True)
+    torch.cuda.synchronize()
+    want = oracle.moe_gemm_gguf(dtype, x2, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
+    err = rel_l2(got.cpu().numpy(), want)
+    assert err <= TIGHT, err
 
 
 @pytest.mark.parametrize("batch", [4, 120, 400])            # 12 pairs (per-pair kernels), 360 (grouped matvec), 1200 (MFMA tiles)
