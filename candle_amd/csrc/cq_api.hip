@@ -150,7 +150,7 @@ int64_t cq_qmatmul_workspace_bytes(int w_dtype, int64_t m, int64_t k, int64_t n)
     int64_t bytes = cq_act_layout(w_dtype, k, m).total;
     // the MFMA path writes f32 and converts afterwards when the caller wants f16 / bf16; small grids split K into
     // partial planes that a second kernel adds up
-    if (m > CQ_MATVEC_MAX_ROWS) {
+    if (m > CQ_MATVEC_MAX_ROWS || cq_use_mfma(w_dtype, m, k)) {
         bytes += cq_align256(m * n * 4);
         const int sp = cq_qmm_splits(k, n, m);
         if (sp > 1) bytes += cq_align256((int64_t)sp * m * n * 4);
@@ -172,7 +172,7 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     // decode: one kernel quantizes the activations into LDS and streams W (no scratch traffic)
     if (m <= 2) return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
     // 3..8 rows: every workgroup re-quantizing all rows costs more than one small kernel that does it once
-    if (m <= CQ_MATVEC_MAX_ROWS) {
+    if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) {
         if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
         return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, dst_dtype, k, n, m, n, s);
     }

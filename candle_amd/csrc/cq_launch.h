@@ -38,6 +38,7 @@ int cq_matvec_norm_pair_merge_launch(int dta, const void *wa, int64_t na, float 
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s, float *split_ws = nullptr);
 int cq_qmm_splits(int64_t k, int64_t n, int64_t rows);
+bool cq_use_mfma(int w_dtype, int64_t rows, int64_t k);
 int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t count, hipStream_t s);
 
 // ---- MoE: both public entry points reduce to "pairs" (expert, activation row, output row, scale) ----
@@ -120,7 +121,8 @@ int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_
 // per-pair kernels do not take.  Measured on 128 experts of 768 x 2048: 264-1016 pairs take 211-229 us per layer on
 // 32-row tiles against 427-644 us on the 8-pairs-per-pass matvec.
 #define CQ_MOE_MFMA_MIN_PAIRS 257
-// rows of one MFMA tile of an expert: the small tile while experts average fewer than 64 rows
+// rows of one MFMA tile of an expert: the small tile while experts average fewer than 40 rows (two small tiles cost
+// more than one large one)
 #define CQ_MOE_TILE_SMALL 32
 #define CQ_MOE_TILE_LARGE 128
 int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k, int64_t n,

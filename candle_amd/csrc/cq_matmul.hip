@@ -34,6 +34,8 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 128, BK = 64;
+constexpr int CQ_QMM_SMALL_ROWS = 32;      // up to here the 32-row block tile is used (measured, 14336 x 4096 Q4_K: 16 / 32 rows
+                                           // 37 / 38 us against 62 us on the 128-row tile; 64 rows as two tiles 73 us)
 constexpr int LDK = BK + 8;            // padded row stride in halves (144 bytes)
 
 // ---- integer bytes -> f16 pairs ------------------------------------------------------------------
@@ -305,7 +307,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
     }
     const bool bstage = tid < 2 * BN;                            // threads that also stage a weight row (wave-uniform)
-    const bool astage = tid < 2 * BMT;                           // threads that stage an activation row (wave-uniform)
+    const bool astage = SM ? tid < 2 * BMT : true;               // threads that stage an activation row (wave-uniform)
     // split-K: blockIdx.z takes an equal share of the 256-element spans and writes its own partial plane
     const int nsb_all = k >> 8;
     const int kb0 = (int)(((int64_t)nsb_all * blockIdx.z) / gridDim.z), nsb = (int)(((int64_t)nsb_all * (blockIdx.z + 1)) / gridDim.z);
@@ -514,15 +516,21 @@ int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t 
     // 128 x 64 tiles (two or three workgroups per CU) everywhere except long Q4_0 / Q8_0 problems, whose cheaper
     // operand conversion leaves the 128 x 128 tile (one workgroup per CU, half the activation conversions) ahead
     const bool wide = !Stage<DT>::KQ && rows >= 1024;
-    const int bn = wide ? 128 : 64;
+    // a few dozen activation rows (batched decode): 32 x 128 tiles, so that the matrix cores and the activation staging
+    // are not spent on 128-row tiles that are mostly padding
+    const bool small = rows <= CQ_QMM_SMALL_ROWS;
+    const int bn = wide || small ? 128 : 64, bm = small ? 32 : BM;
     const int splits = split_ws ? cq_qmm_splits(k, n, rows) : 1;
-    dim3 grid((unsigned)((rows + BM - 1) / BM), (unsigned)((n + bn - 1) / bn), (unsigned)splits);
+    dim3 grid((unsigned)((rows + bm - 1) / bm), (unsigned)((n + bn - 1) / bn), (unsigned)splits);
     if (grid.y > 65535) return CQ_ERR_RANGE;
     const MoeChunks none{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     // with split-K every split writes a contiguous [rows, n] plane of the workspace; a second kernel adds them in order
     float *out = splits > 1 ? split_ws : dst;
     const int64_t ld = splits > 1 ? n : stride_dst, plane = splits > 1 ? rows * n : 0;
-    if (wide)
+    if (small)
+        hipLaunchKernelGGL((qmm_kernel<DT, 1, false, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none,
+                           (int64_t)0, plane);
+    else if (wide)
         hipLaunchKernelGGL((qmm_kernel<DT, 2>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none, (int64_t)0,
                            plane);
     else
@@ -597,8 +605,9 @@ int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_
 // is only a multiple of 32, and very small problems, go through the row-chunked matvec instead.
 // Small grids (few activation rows or few weight rows) split K so that about 256 workgroups exist.  1 = no split.
 int cq_qmm_splits(int64_t k, int64_t n, int64_t rows) {
-    if (k % 256 || n % 4 || rows <= CQ_MATVEC_MAX_ROWS) return 1;
-    const int64_t base = ((rows + BM - 1) / BM) * ((n + 63) / 64), nsb = k / 256;
+    if (k % 256 || n % 4 || rows < 1) return 1;
+    const int64_t base = rows <= CQ_QMM_SMALL_ROWS ? ((rows + 31) / 32) * ((n + 127) / 128) : ((rows + BM - 1) / BM) * ((n + 63) / 64);
+    const int64_t nsb = k / 256;
     if (base >= 192 || nsb < 8) return 1;
     int64_t sp = (256 + base - 1) / base;
     if (sp > 8) sp = 8;
@@ -606,10 +615,17 @@ int cq_qmm_splits(int64_t k, int64_t n, int64_t rows) {
     return sp < 2 ? 1 : (int)sp;
 }
 
+// Which row counts go to the matrix cores: everything beyond the matvec kernel's 8 rows (measured, Q4_K 14336 x 4096 /
+// 4096 x 14336: 8 rows on the matvec 27 / 28 us, 9-32 rows on the 32-row MFMA tile 36-41 us).
+bool cq_use_mfma(int w_dtype, int64_t rows, int64_t k) {
+    (void)w_dtype;
+    return k % 256 == 0 && rows > CQ_MATVEC_MAX_ROWS;
+}
+
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s, float *split_ws) {
     ActView av = cq_act_view(scratch, w_dtype, k, rows);
-    if (k % 256 == 0 && rows > CQ_MATVEC_MAX_ROWS) {
+    if (cq_use_mfma(w_dtype, rows, k)) {
         switch (w_dtype) {
             case CQ_Q4_0: return launch_qmm<CQ_Q4_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q8_0: return launch_qmm<CQ_Q8_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);

@@ -211,7 +211,7 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     // Hundreds of pairs per call on K-quant experts: the expert-sorted rows go through the MFMA prefill kernel in tiles
     // of up to 128 rows of one expert (integer-exact like the other K-quant paths).  Otherwise 8 pairs per matvec pass.
     const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
-    const int tile_rows = a.n_pairs < 64 * a.num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE;
+    const int tile_rows = a.n_pairs < 40 * a.num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
                        (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);
     if ((rc = (int)hipGetLastError())) return rc;
