@@ -42,31 +42,37 @@ inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pa
 }
 
 // offsets[e] .. offsets[e+1] is expert e's segment of pair_in / pair_out / pair_scale.
+// LC: the per-expert counters live in LDS (up to GROUP_LDS_EXPERTS experts) instead of the global `cursor` array: the
+// two passes of atomics are then LDS atomics, not trips of one workgroup to the L2.
+constexpr int GROUP_LDS_EXPERTS = 4096;
+template <bool LC>
 __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__restrict__ offsets, int *__restrict__ cursor,
                                                          int *__restrict__ pair_in, int *__restrict__ pair_out,
                                                          float *__restrict__ pair_scale, float *__restrict__ out, int n, int *__restrict__ chunks,
                                                          int max_chunks, int chunk) {
-    __shared__ int carry;
+    __shared__ int carry, n_chunks;
+    __shared__ int buf[1024];
+    __shared__ int lcur[LC ? GROUP_LDS_EXPERTS : 1];
+    int *cur = LC ? lcur : cursor;
     const int tid = threadIdx.x;
     const int E = ps.num_experts;
-    for (int e = tid; e < E; e += 1024) cursor[e] = 0;
+    for (int e = tid; e < E; e += 1024) cur[e] = 0;
     __syncthreads();
     for (int p = tid; p < ps.n_pairs; p += 1024) {
         int e, in_row, out_row;
         float scale;
-        if (pair_decode(ps, p, e, in_row, out_row, scale)) atomicAdd(&cursor[e], 1);
+        if (pair_decode(ps, p, e, in_row, out_row, scale)) atomicAdd(&cur[e], 1);
     }
-    if (tid == 0) carry = 0;
+    if (tid == 0) { carry = 0; n_chunks = 0; }
     __syncthreads();
-    // exclusive scan of the counts, 1024 experts per sweep
+    // exclusive scan of the counts, 1024 experts per sweep (only as many doubling steps as the sweep is wide)
     for (int base = 0; base < E; base += 1024) {
         int e = base + tid;
-        int c = e < E ? cursor[e] : 0;
-        // inclusive scan inside the workgroup through shared memory
-        __shared__ int buf[1024];
+        int c = e < E ? cur[e] : 0;
+        const int width = min(1024, E - base);
         buf[tid] = c;
         __syncthreads();
-        for (int o = 1; o < 1024; o <<= 1) {
+        for (int o = 1; o < width; o <<= 1) {
             int v = tid >= o ? buf[tid - o] : 0;
             __syncthreads();
             buf[tid] += v;
@@ -75,36 +81,31 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
         int start = carry + buf[tid] - c;
         if (e < E) {
             offsets[e] = start;
-            cursor[e] = start;
+            cur[e] = start;
+            // chunk table: expert e's segment in pieces of `chunk` pairs (any order: chunks are independent)
+            const int cc = (c + chunk - 1) / chunk;
+            if (cc > 0) {
+                const int cb = atomicAdd(&n_chunks, cc);
+                for (int i = 0; i < cc; i++) {
+                    chunks[1 + cb + i] = e;
+                    chunks[1 + max_chunks + cb + i] = start + i * chunk;
+                    chunks[1 + 2 * max_chunks + cb + i] = min(chunk, c - i * chunk);
+                }
+            }
         }
         __syncthreads();
-        if (tid == 1023) carry += buf[1023];
+        if (tid == width - 1) carry += buf[tid];              // the inclusive sum of the sweep
         __syncthreads();
     }
-    if (tid == 0) { offsets[E] = carry; chunks[0] = 0; }
-    __syncthreads();
+    if (tid == 0) { offsets[E] = carry; chunks[0] = n_chunks; }
     // positions behind the last valid pair are never part of a chunk, but the gathering quantizer walks all n_pairs
     // rows: give them a valid source row
     for (int p = carry + tid; p < ps.n_pairs; p += 1024) pair_in[p] = 0;
-    // chunk table: expert e's segment in pieces of `chunk` pairs (any order: chunks are independent)
-    for (int e = tid; e < E; e += 1024) {
-        const int seg0 = offsets[e], cnt = offsets[e + 1] - seg0;     // offsets[e + 1] of the last sweep's neighbour is final here
-        const int cc = (cnt + chunk - 1) / chunk;
-        if (cc > 0) {
-            const int base = atomicAdd(&chunks[0], cc);
-            for (int i = 0; i < cc; i++) {
-                chunks[1 + base + i] = e;
-                chunks[1 + max_chunks + base + i] = seg0 + i * chunk;
-                chunks[1 + 2 * max_chunks + base + i] = min(chunk, cnt - i * chunk);
-            }
-        }
-    }
-    __syncthreads();
     for (int p = tid; p < ps.n_pairs; p += 1024) {
         int e, in_row, out_row;
         float scale;
         if (pair_decode(ps, p, e, in_row, out_row, scale)) {
-            int pos = atomicAdd(&cursor[e], 1);
+            int pos = atomicAdd(&cur[e], 1);
             pair_in[pos] = in_row;
             pair_out[pos] = out_row;
             pair_scale[pos] = scale;
@@ -212,8 +213,12 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     // of up to 128 rows of one expert (integer-exact like the other K-quant paths).  Otherwise 8 pairs per matvec pass.
     const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
     const int tile_rows = a.n_pairs < 40 * a.num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE;
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
-                       (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);
+    if (a.num_experts <= GROUP_LDS_EXPERTS)
+        hipLaunchKernelGGL(moe_group_kernel<true>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
+                           (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);
+    else
+        hipLaunchKernelGGL(moe_group_kernel<false>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
+                           (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);
     if ((rc = (int)hipGetLastError())) return rc;
     if (mfma) {
         if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;
