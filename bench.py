@@ -210,7 +210,7 @@ def moe(args):
 
     fused = [FusedMoeGGUF(router, qt(gate[i], F, H), qt(up[i], F, H), qt(down[i], H, F), True, TOPK) for i in range(NL)]
     results = []
-    for tokens in (1, 16, 256):
+    for tokens in [int(t) for t in args.moe_tokens.split(",")]:
         x = torch.randn((tokens, H), generator=gen, device=dev)
         _, ids = torch.topk(torch.softmax(x @ router.t(), -1), TOPK, dim=-1)
         ids32 = ids.to(torch.int32).contiguous()
@@ -284,6 +284,7 @@ def main():
     ap.add_argument("--workload", choices=["decode", "prefill", "decode8b", "moe"], default="decode")
     ap.add_argument("--layers", type=int, default=32, help="--workload decode8b: number of decoder layers")
     ap.add_argument("--prompt", type=int, default=512, help="--workload decode8b: prompt tokens")
+    ap.add_argument("--moe-tokens", default="1,16,256", help="--workload moe: token counts, comma separated")
     ap.add_argument("--wdtype", choices=sorted(WDTYPES), default="q4k", help="weight format of --workload prefill")
     ap.add_argument("--n", type=int, default=14336)
     ap.add_argument("--k", type=int, default=4096)
