@@ -111,11 +111,31 @@ __device__ __forceinline__ float oct_max(float v) {
     return v;
 }
 
-// wave64 butterfly sum; every lane ends with the total.
+// wave64 sum; every lane ends with the total (through a scalar register).  DPP row shifts and row broadcasts: six
+// VALU steps, where a butterfly of __shfl_xor is six trips through the LDS crossbar.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, CQ_WAVE);
-    return v;
+#define CQ_AD(ctrl, rmask, bc) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, rmask, 0xf, bc))
+    CQ_AD(CQ_DPP_ROW_SHR(1), 0xf, true);
+    CQ_AD(CQ_DPP_ROW_SHR(2), 0xf, true);
+    CQ_AD(CQ_DPP_ROW_SHR(4), 0xf, true);
+    CQ_AD(CQ_DPP_ROW_SHR(8), 0xf, true);      // lane 15 of each row: row sum
+    CQ_AD(CQ_DPP_ROW_BCAST15, 0xa, false);
+    CQ_AD(CQ_DPP_ROW_BCAST31, 0xc, false);    // lane 63: wave sum
+#undef CQ_AD
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// wave64 maximum of any float, in every lane
+__device__ __forceinline__ float wave_max(float v) {
+#define CQ_MX(ctrl, rmask) v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), ctrl, rmask, 0xf, false)))
+    CQ_MX(CQ_DPP_ROW_SHR(1), 0xf);
+    CQ_MX(CQ_DPP_ROW_SHR(2), 0xf);
+    CQ_MX(CQ_DPP_ROW_SHR(4), 0xf);
+    CQ_MX(CQ_DPP_ROW_SHR(8), 0xf);
+    CQ_MX(CQ_DPP_ROW_BCAST15, 0xa);
+    CQ_MX(CQ_DPP_ROW_BCAST31, 0xc);
+#undef CQ_MX
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // ---------------------------------------------------------------------------------------------

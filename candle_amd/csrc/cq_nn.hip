@@ -218,8 +218,7 @@ __global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, 
             s[i] = sc[g * ATT_SPLIT + lane + 64 * i];
             m = fmaxf(m, s[i]);
         }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        m = wave_max(m);
         float l = 0.0f;
 #pragma unroll
         for (int i = 0; i < ATT_SPLIT / 64; i++) {
@@ -434,8 +433,7 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
             s[i] = sc[g * ATT_SPLIT + lane + 64 * i];
             m = fmaxf(m, s[i]);
         }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        m = wave_max(m);
         float l = 0.0f;
 #pragma unroll
         for (int i = 0; i < ATT_SPLIT / 64; i++) {
@@ -654,8 +652,7 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float *__restrict__
     // softmax_last_dim (candle-nn/src/ops.rs): max, exp(x - max), sum, divide
     float m = -INFINITY;
     for (int e = tid; e < n_experts; e += 256) m = fmaxf(m, prob[e]);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, CQ_WAVE));
+    m = wave_max(m);
     if (lane == 0) red[wv] = m;
     __syncthreads();
     m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
