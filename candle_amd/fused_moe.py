@@ -54,6 +54,7 @@ class FusedMoeGGUF:
         self.router_logits = torch.empty((tokens, self.num_experts), **f32)
         self.expert_ids = torch.empty(pairs, dtype=torch.int32, device=dev)
         self.sorted_token_ids = torch.empty(pairs, dtype=torch.int32, device=dev)
+        self.pair_iota = torch.arange(pairs, dtype=torch.int32, device=dev)
         self.gate_out = torch.empty((pairs, self.inter), **f32)
         self.up_out = torch.empty((pairs, self.inter), **f32)
         self.down_in = torch.empty((pairs, self.inter), **f32)
@@ -88,19 +89,25 @@ class FusedMoeGGUF:
             ck("cq_nn_moe_route", L.cq_nn_moe_route(x2.data_ptr() + 4 * t0 * hidden, self.gate.data_ptr(), self.topk_ids.data_ptr() + 4 * t0 * topk,
                                                     self.topk_weights.data_ptr() + 4 * t0 * topk, self.router_logits.data_ptr() + 4 * t0 * E,
                                                     t, hidden, E, topk, 1 if self.norm_topk_prob else 0, sp))
-        ck("cq_nn_moe_sort", L.cq_nn_moe_sort(self.topk_ids.data_ptr(), self.expert_ids.data_ptr(), self.sorted_token_ids.data_ptr(), pairs, E, sp))
+        # (expert_ids, sorted_token_ids) of fused_moe.rs:249-260.  The grouped matmuls give every pair its own row whatever
+        # the order of the pairs, and up to 256 pairs each pair is its own matvec launch block, so the sort is skipped there:
+        # the pairs are taken in token order (expert_ids = topk_ids, sorted_token_ids = 0, 1, 2, ...).
+        if pairs <= 256:
+            eid_ptr, sti_ptr = self.topk_ids.data_ptr(), self.pair_iota.data_ptr()
+        else:
+            ck("cq_nn_moe_sort", L.cq_nn_moe_sort(self.topk_ids.data_ptr(), self.expert_ids.data_ptr(), self.sorted_token_ids.data_ptr(), pairs, E,
+                                                  sp))
+            eid_ptr, sti_ptr = self.expert_ids.data_ptr(), self.sorted_token_ids.data_ptr()
 
         def gemm(x_ptr, w: QTensor, tw_ptr, out_t, n, k):
-            ck("cq_moe_gemm_gguf", L.cq_moe_gemm_gguf(dt, x_ptr, w.device_ptr(), self.sorted_token_ids.data_ptr(), self.expert_ids.data_ptr(),
-                                                      tw_ptr, out_t.data_ptr(), E, topk, pairs, n, k, 1 if is_prefill else 0,
-                                                      self.ws.data_ptr(), self.ws.numel(), sp))
+            ck("cq_moe_gemm_gguf", L.cq_moe_gemm_gguf(dt, x_ptr, w.device_ptr(), sti_ptr, eid_ptr, tw_ptr, out_t.data_ptr(), E, topk, pairs, n, k,
+                                                      1 if is_prefill else 0, self.ws.data_ptr(), self.ws.numel(), sp))
 
         # decode-sized calls: gate, up and the activation in one launch
         fused = -6
         if pairs <= 256:
-            fused = L.cq_moe_gemm_gguf_swiglu(dt, x2.data_ptr(), self.gate_experts.device_ptr(), self.up_experts.device_ptr(),
-                                              self.sorted_token_ids.data_ptr(), self.expert_ids.data_ptr(), self.down_in.data_ptr(), E, topk,
-                                              pairs, self.inter, hidden, sp)
+            fused = L.cq_moe_gemm_gguf_swiglu(dt, x2.data_ptr(), self.gate_experts.device_ptr(), self.up_experts.device_ptr(), sti_ptr, eid_ptr,
+                                              self.down_in.data_ptr(), E, topk, pairs, self.inter, hidden, sp)
             if fused != -6:
                 ck("cq_moe_gemm_gguf_swiglu", fused)
         if fused == -6:                                          # CQ_ERR_RANGE: not a shape of the fused launch
