@@ -419,7 +419,16 @@ def main():
         _lib.check("cq_quantize_act", L.cq_quantize_act(Q4K, x.data_ptr(), 0, ws.data_ptr(), k, m, None))
         torch.cuda.synchronize()
         preq_us = event_us(capture(matvec_prequantized), args.steps)
-        extra = {"infinity_cache_resident_us": round(resident_us, 3),
+        # the yardstick: a kernel that only reads the same rotated tensors, same launch shape
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        read_bytes = wbytes - wbytes % 16
+
+        def plain_read(i, sp):
+            _lib.check("cq_bench_read", L.cq_bench_read(weights[i % pool].data_ptr(), read_bytes, sink.data_ptr(), sp))
+
+        read_us = event_us(capture(plain_read), args.steps)
+        extra = {"plain_read_us": round(read_us, 3), "plain_read_GBps": round(read_bytes / (read_us * 1e-6) / 1e9, 1),
+                 "infinity_cache_resident_us": round(resident_us, 3),
                  "infinity_cache_resident_GBps": round(alg_bytes / (resident_us * 1e-6) / 1e9, 1),
                  "prequantized_matvec_us": round(preq_us, 3),
                  "prequantized_matvec_GBps": round(alg_bytes / (preq_us * 1e-6) / 1e9, 1)}

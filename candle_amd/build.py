@@ -20,7 +20,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "obj")
 LIB = os.path.join(HERE, "libcandle_hip_quant.so")
 
-SOURCES = ["cq_api.hip", "cq_dequant.hip", "cq_actquant.hip", "cq_matvec.hip", "cq_matmul.hip", "cq_moe.hip", "cq_quantize.hip", "cq_nn.hip"]
+SOURCES = ["cq_api.hip", "cq_dequant.hip", "cq_actquant.hip", "cq_matvec.hip", "cq_matmul.hip", "cq_moe.hip", "cq_quantize.hip", "cq_nn.hip", "cq_bench.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

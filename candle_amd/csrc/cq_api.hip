@@ -96,6 +96,14 @@ int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem
     return cq_dequantize_launch(dtype, blocks_dev, out_dev, elem_count, out_dtype, (hipStream_t)stream);
 }
 
+int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stream) {
+    if (bytes < 0 || bytes % 16) return CQ_ERR_SHAPE;
+    if (bytes == 0) return CQ_OK;
+    if (!src_dev || !sink_dev) return CQ_ERR_NULL;
+    if (!aligned(src_dev, 16) || !aligned(sink_dev, 4)) return CQ_ERR_ALIGN;
+    return cq_bench_read_launch(src_dev, bytes, sink_dev, (hipStream_t)stream);
+}
+
 int cq_quantize(int dtype, const float *x_dev, void *blocks_dev, int64_t elem_count, void *stream) {
     if (!block_dtype(dtype)) return CQ_ERR_DTYPE;
     if (elem_count < 0 || elem_count % cq_block_size(dtype) != 0) return CQ_ERR_SHAPE;

@@ -165,6 +165,11 @@ int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_
                             const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
                             int64_t k, void *stream);
 
+/* Measurement aid, no counterpart in the reference: a kernel that only reads `bytes` (a multiple of 16) of a device
+ * buffer, with the launch shape of the decode matvec (256 workgroups of 1024 threads).  bench.py times it over the same
+ * rotated weight tensors as the matvec, as the figure for what this GPU delivers to a launch of that size. */
+int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
