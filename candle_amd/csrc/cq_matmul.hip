@@ -603,13 +603,17 @@ int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_
 
 // k is a multiple of 256 for the MFMA kernel (always true for K-quants); Q4_0 / Q8_0 rows whose length
 // is only a multiple of 32, and very small problems, go through the row-chunked matvec instead.
-// Small grids (few activation rows or few weight rows) split K so that about 256 workgroups exist.  1 = no split.
+// Small grids (few activation rows or few weight rows) split K so that about 512 workgroups exist.  1 = no split.
 int cq_qmm_splits(int64_t k, int64_t n, int64_t rows) {
     if (k % 256 || n % 4 || rows < 1) return 1;
     const int64_t base = rows <= CQ_QMM_SMALL_ROWS ? ((rows + 31) / 32) * ((n + 127) / 128) : ((rows + BM - 1) / BM) * ((n + 63) / 64);
     const int64_t nsb = k / 256;
-    if (base >= 192 || nsb < 8) return 1;
-    int64_t sp = (256 + base - 1) / base;
+    // about two workgroups per CU: one converts operands while the other feeds the matrix cores (measured against a target
+    // of one per CU: Q6_K 4096 x 14336 at 128 / 256 / 512 rows 69 / 131 / 248 -> 57 / 105 / 200 us, Q4_K 4096 x 4096 at 512
+    // rows 67 -> 54 us; three per CU is no better)
+    const int64_t target = 512;
+    if (base >= target * 3 / 4 || nsb < 8) return 1;
+    int64_t sp = (target + base - 1) / base;
     if (sp > 8) sp = 8;
     if (sp > nsb / 4) sp = nsb / 4;
     return sp < 2 ? 1 : (int)sp;
