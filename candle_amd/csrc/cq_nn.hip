@@ -169,6 +169,16 @@ __global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, 
     const int kv_len = min(pos0 + (pos_dev ? pos_dev[0] : 0) + r + 1, ctx);
     const int j0 = sp * ATT_SPLIT;
     const int cnt = min(kv_len - j0, ATT_SPLIT);      // keys in this split (may be <= 0)
+    if (cnt <= 0 && splits > 1) {
+        // a split entirely behind this row's position (the grid is sized for the last row): an empty partial, which the
+        // combine kernel skips, and nothing else — with a causal prompt that is three splits in eight
+        if (tid < G) {
+            float *pp = part + (((int64_t)r * n_head + kvh * G + tid) * splits + sp) * (HD + 2);
+            pp[0] = -INFINITY;
+            pp[1] = 0.0f;
+        }
+        return;
+    }
     const float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
     const int last = max(cnt - 1, 0);                 // loads of masked keys are redirected to a valid row
 
