@@ -24,6 +24,7 @@
 // v_mfma_f32_32x32x16_f16 tiles (128 x 128 / 64 x 64 for long Q4_0 / Q8_0 problems).  K advances 64 elements per
 // LDS stage: the threads dequantize the weight tile and convert the 128 x 64 int8 activation tile to f16 in LDS
 // (row stride padded to 144 bytes); raw bytes are requested two stages ahead into two register sets.
+#include <cstdlib>
 #include "cq_device.h"
 #include "cq_launch.h"
 
@@ -289,12 +290,15 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
     constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;             // rows of the block tile, 32-row MFMA tiles per wave
     constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
-    __shared__ __align__(16) _Float16 As[BMT * LDK];
-    __shared__ __align__(16) _Float16 Bs[BN * LDK];
-    __shared__ __align__(16) _Float16 Bs2[S::TERMS == 2 ? BN * LDK : 8];   // exact remainders of a two-term format
-    __shared__ __align__(16) _Float16 Am[BMT * 24];   // bsums16 of the super-block, as f16 (row stride 24 halves)
-    __shared__ __align__(16) _Float16 Bm[BN * 24];    // sub-block mins duplicated per 16-element group
-    __shared__ float sD[BN], sDmin[BN], sD8[BMT];
+    // every LDS array exists twice: while the matrix cores work on one stage, the threads convert the next one into
+    // the other copy (one barrier per stage); the per-super-block arrays alternate with the super-block
+    constexpr int NMIN = S::HAS_MIN ? 24 : 0;
+    __shared__ __align__(16) _Float16 As[2][BMT * LDK];
+    __shared__ __align__(16) _Float16 Bs[2][BN * LDK];
+    __shared__ __align__(16) _Float16 Bs2[2][S::TERMS == 2 ? BN * LDK : 8];   // exact remainders of a two-term format
+    __shared__ __align__(16) _Float16 Am[2][BMT * NMIN + 8];   // bsums16 of the super-block, as f16 (row stride 24 halves)
+    __shared__ __align__(16) _Float16 Bm[2][BN * NMIN + 8];    // sub-block mins duplicated per 16-element group
+    __shared__ float sD[2][BN], sDmin[2][BN], sD8[2][BMT];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = SM ? 0 : wv >> 1, wn = SM ? wv : wv & 1;
@@ -306,7 +310,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         rows = m0 + mc.count[blockIdx.x];
         w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
     }
-    const bool bstage = tid < 2 * BN;                            // threads that also stage a weight row (wave-uniform)
+    const bool bstage = 2 * BN >= 256 ? true : tid < 2 * BN;    // threads that also stage a weight row (wave-uniform)
     const bool astage = SM ? tid < 2 * BMT : true;               // threads that stage an activation row (wave-uniform)
     // split-K: blockIdx.z takes an equal share of the 256-element spans and writes its own partial plane
     const int nsb_all = k >> 8;
@@ -319,6 +323,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     const int wrow = min(n0 + (bstage ? r_l : 0), n - 1);
     const int arow = min(m0 + (astage ? r_l : 0), rows - 1);
     const bool arow_ok = astage && m0 + r_l < rows;
+    const uint32_t amask = arow_ok ? 0xffffffffu : 0u;
     const uint8_t *wrow_p = w + wrow * row_bytes;
     const int8_t *aq_p = av.qs + (int64_t)arow * k;
 
@@ -330,97 +335,112 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
 #pragma unroll
             for (int e = 0; e < 16; e++) { acc[i][j][e] = 0.0f; sb[i][j][e] = 0.0f; }
 
-    // raw bytes are requested two stages ahead (two register sets, chosen by the parity of the stage): one stage of
-    // conversion + MFMA work is shorter than a trip to memory
+    // Raw bytes are requested two stages ahead (two register sets, chosen by the parity of the stage): one stage of
+    // conversion + MFMA work is shorter than a trip to memory.  Stage (kb, g) covers k = 256 kb + 64 g + [0, 64).
+    // Positions past the end of this split's range are clamped to its last super-block: what they load and convert
+    // lands in LDS copies nobody reads.
     typename S::Raw wraw2[2];
-    u32x4 a02[2], a12[2];
-    auto load_stage = [&](int kb, int g, typename S::Raw &wr, u32x4 &x0, u32x4 &x1) {
+    u32x4 a02[2], a12[2], abs0 = u32x4{0, 0, 0, 0};
+    float ad8[2] = {0.0f, 0.0f};
+    auto load_stage = [&](int kb, int g, typename S::Raw &wr, u32x4 &x0, u32x4 &x1, float &d8) {
+        kb = min(kb, nsb - 1);
         if (bstage) S::load(wr, wrow_p, kb, g, half);
         if (astage) {
             const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
             x0 = *reinterpret_cast<const u32x4 *>(q);
             x1 = *reinterpret_cast<const u32x4 *>(q + 16);
+            if (!KQ) d8 = av.d[2 * ((int64_t)arow * (k >> 5) + kb * 8 + 2 * g + half)];   // already f16-representable
+            if (KQ && g == 0) {
+                d8 = av.d[(int64_t)arow * (k >> 8) + kb];
+                if (S::HAS_MIN) abs0 = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
+            }
         }
     };
-    load_stage(kb0, 0, wraw2[0], a02[0], a12[0]);
-    load_stage(kb0, 1, wraw2[1], a02[1], a12[1]);
+    // what one thread contributes to the LDS image of a stage
+    struct Conv {
+        uint32_t w[16], w2[S::TERMS == 2 ? 16 : 1], a[16];
+        float d, dmin, d8;
+        uint32_t mv[4], bv[4];
+    };
+    auto convert_stage = [&](int g, const typename S::Raw &wraw, const u32x4 &a0, const u32x4 &a1, float d8, Conv &c) {
+        if (bstage) {
+            if constexpr (S::TERMS == 2) S::convert2(wraw, g, half, c.w, c.w2);
+            else S::convert(wraw, g, half, c.w);
+        }
+        if (astage) {
+            act_convert(a0, a1, !KQ, KQ ? 0u : h2_splat(d8), c.a);
+#pragma unroll
+            for (int i = 0; i < 16; i++) c.a[i] &= amask;        // rows past the end contribute zeros (no branch)
+        }
+        if (KQ && g == 0) {
+            int mins[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            c.d = 0.0f; c.dmin = 0.0f;
+            if (bstage) S::header(wraw, c.d, c.dmin, mins);
+            c.d8 = arow_ok ? d8 : 0.0f;
+            if (S::HAS_MIN) {
+                // Bm[n][j] = min[j/2] for j in 8*half .. 8*half+7 ; Am[m][j] = bsums16[j]
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t hm = f2h_bits((float)mins[4 * half + i]);
+                    c.mv[i] = hm | (hm << 16);
+                }
+                const uint32_t b4[4] = {abs0.x, abs0.y, abs0.z, abs0.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t lo = f2h_bits((float)(int16_t)(b4[i] & 0xffff)), hi = f2h_bits((float)(int16_t)(b4[i] >> 16));
+                    c.bv[i] = arow_ok ? (lo | (hi << 16)) : 0u;
+                }
+            }
+        }
+    };
+    // buf: LDS copy of the stage (its parity); hb: copy of the per-super-block arrays (parity of the super-block)
+    auto store_stage = [&](int g, int buf, int hb, const Conv &c) {
+        if (bstage) {
+            if constexpr (S::TERMS == 2) lds_write32h(Bs2[buf] + r_l * LDK + 32 * half, c.w2);
+            lds_write32h(Bs[buf] + r_l * LDK + 32 * half, c.w);
+        }
+        if (astage) lds_write32h(As[buf] + r_l * LDK + 32 * half, c.a);
+        if (KQ && g == 0) {
+            // both threads of a row hold the same values: both write them (no branch)
+            if (bstage) { sD[hb][r_l] = c.d; sDmin[hb][r_l] = c.dmin; }
+            if (astage) sD8[hb][r_l] = c.d8;
+            if (S::HAS_MIN) {
+                if (bstage) *reinterpret_cast<u32x4 *>(Bm[hb] + r_l * 24 + 8 * half) = u32x4{c.mv[0], c.mv[1], c.mv[2], c.mv[3]};
+                if (astage) *reinterpret_cast<u32x4 *>(Am[hb] + r_l * 24 + 8 * half) = u32x4{c.bv[0], c.bv[1], c.bv[2], c.bv[3]};
+            }
+        }
+    };
+    load_stage(kb0, 0, wraw2[0], a02[0], a12[0], ad8[0]);
+    load_stage(kb0, 1, wraw2[1], a02[1], a12[1], ad8[1]);
+    {
+        Conv c;
+        convert_stage(0, wraw2[0], a02[0], a12[0], ad8[0], c);
+        store_stage(0, 0, kb0 & 1, c);
+        load_stage(kb0, 2, wraw2[0], a02[0], a12[0], ad8[0]);
+    }
+    __syncthreads();
 
     for (int kb = kb0; kb < nsb; kb++) {
+        const int hb = kb & 1;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            typename S::Raw &wraw = wraw2[g & 1];
-            u32x4 &a0 = a02[g & 1], &a1 = a12[g & 1];
-            // ---- write the staged raw data of (kb, g) to LDS as f16 ----
-            uint32_t hv[16];
-            if (bstage) {
-                if constexpr (S::TERMS == 2) {
-                    uint32_t hr[16];
-                    S::convert2(wraw, g, half, hv, hr);
-                    lds_write32h(Bs2 + r_l * LDK + 32 * half, hr);
-                } else {
-                    S::convert(wraw, g, half, hv);
-                }
-                lds_write32h(Bs + r_l * LDK + 32 * half, hv);
-            }
-            if (astage) {
-                uint32_t ascale2 = 0;
-                if (!KQ) {
-                    float d8 = av.d[2 * ((int64_t)arow * (k >> 5) + kb * 8 + 2 * g + half)];   // already f16-representable
-                    ascale2 = h2_splat(d8);
-                }
-                act_convert(a0, a1, !KQ, ascale2, hv);
-                if (!arow_ok) {
-#pragma unroll
-                    for (int i = 0; i < 16; i++) hv[i] = 0;
-                }
-                lds_write32h(As + r_l * LDK + 32 * half, hv);
-            }
-            if (KQ && g == 0) {
-                float d = 0.0f, dmin = 0.0f;
-                int mins[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (bstage) S::header(wraw, d, dmin, mins);
-                if (half == 0) {
-                    if (bstage) { sD[r_l] = d; sDmin[r_l] = dmin; }
-                    if (astage) sD8[r_l] = arow_ok ? av.d[(int64_t)arow * (k >> 8) + kb] : 0.0f;
-                }
-                if (S::HAS_MIN) {
-                    // Bm[n][j] = min[j/2] for j in 8*half .. 8*half+7 ; Am[m][j] = bsums16[j]
-                    uint32_t mv[4];
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        uint32_t hm = f2h_bits((float)mins[4 * half + i]);
-                        mv[i] = hm | (hm << 16);
-                    }
-                    if (bstage) *reinterpret_cast<u32x4 *>(Bm + r_l * 24 + 8 * half) = u32x4{mv[0], mv[1], mv[2], mv[3]};
-                    if (astage) {
-                        u32x4 bs = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
-                        const uint32_t b4[4] = {bs.x, bs.y, bs.z, bs.w};
-                        uint32_t bv[4];
-#pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            uint32_t lo = f2h_bits((float)(int16_t)(b4[i] & 0xffff)), hi = f2h_bits((float)(int16_t)(b4[i] >> 16));
-                            bv[i] = arow_ok ? (lo | (hi << 16)) : 0u;
-                        }
-                        *reinterpret_cast<u32x4 *>(Am + r_l * 24 + 8 * half) = u32x4{bv[0], bv[1], bv[2], bv[3]};
-                    }
-                }
-            }
-            __syncthreads();
-            // ---- the register set just consumed is refilled with the stage after next ----
-            {
-                const int ng = (g + 2) & 3, nkb = g >= 2 ? kb + 1 : kb;
-                if (nkb < nsb) load_stage(nkb, ng, wraw, a0, a1);
-            }
-            // ---- 4 k-slices of 16: 2 x 2 MFMA tiles per wave ----
+            // ---- the next stage is converted in registers while the MFMAs of this one are in flight ----
+            const int ng = (g + 1) & 3, nb = (g + 1) & 1;
+            Conv c;
+            convert_stage(ng, wraw2[nb], a02[nb], a12[nb], ad8[nb], c);
+            // its register set is refilled with the stage two further on
+            load_stage(g == 0 ? kb : kb + 1, (g + 3) & 3, wraw2[nb], a02[nb], a12[nb], ad8[nb]);
+            // ---- 4 k-slices of 16: MI x NJ MFMA tiles per wave ----
+            const _Float16 *Ab = As[g & 1], *Bb = Bs[g & 1], *Bb2 = Bs2[g & 1];
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
                 half8 af[MI], bf[NJ];
 #pragma unroll
                 for (int t = 0; t < MI; t++)
-                    af[t] = *reinterpret_cast<const half8 *>(As + (wm * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
+                    af[t] = *reinterpret_cast<const half8 *>(Ab + (wm * 64 + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
                 for (int t = 0; t < NJ; t++)
-                    bf[t] = *reinterpret_cast<const half8 *>(Bs + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
+                    bf[t] = *reinterpret_cast<const half8 *>(Bb + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
                 for (int i = 0; i < MI; i++)
 #pragma unroll
@@ -428,13 +448,14 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
                 if constexpr (S::TERMS == 2) {
 #pragma unroll
                     for (int t = 0; t < NJ; t++)
-                        bf[t] = *reinterpret_cast<const half8 *>(Bs2 + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
+                        bf[t] = *reinterpret_cast<const half8 *>(Bb2 + (wn * WN + t * 32 + (lane & 31)) * LDK + ks * 16 + 8 * (lane >> 5));
 #pragma unroll
                     for (int i = 0; i < MI; i++)
 #pragma unroll
                         for (int j = 0; j < NJ; j++) sb[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], sb[i][j], 0, 0, 0);
                 }
             }
+            store_stage(ng, nb, g == 3 ? hb ^ 1 : hb, c);
             if (KQ && g == 3) {
                 // ---- end of the super-block: mins term and the f32 scales ----
                 f32x16 mt[MI][NJ];
@@ -442,10 +463,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
                     half8 am[MI], bm[NJ];
 #pragma unroll
                     for (int t = 0; t < MI; t++)
-                        am[t] = *reinterpret_cast<const half8 *>(Am + (wm * 64 + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
+                        am[t] = *reinterpret_cast<const half8 *>(Am[hb] + (wm * 64 + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
 #pragma unroll
                     for (int t = 0; t < NJ; t++)
-                        bm[t] = *reinterpret_cast<const half8 *>(Bm + (wn * WN + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
+                        bm[t] = *reinterpret_cast<const half8 *>(Bm[hb] + (wn * WN + t * 32 + (lane & 31)) * 24 + 8 * (lane >> 5));
 #pragma unroll
                     for (int i = 0; i < MI; i++)
 #pragma unroll
@@ -459,7 +480,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
 #pragma unroll
                 for (int j = 0; j < NJ; j++) {
                     const int nl = wn * WN + j * 32 + (lane & 31);
-                    const float d = sD[nl], dmin = sDmin[nl];
+                    const float d = sD[hb][nl], dmin = sDmin[hb][nl];
 #pragma unroll
                     for (int i = 0; i < MI; i++) {
 #pragma unroll
@@ -467,7 +488,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
                             const int ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                             float t = d * sb[i][j][e];
                             if (S::HAS_MIN) t = fmaf(-dmin, mt[i][j][e], t);
-                            acc[i][j][e] = fmaf(sD8[ml], t, acc[i][j][e]);
+                            acc[i][j][e] = fmaf(sD8[hb][ml], t, acc[i][j][e]);
                             sb[i][j][e] = 0.0f;
                         }
                     }
@@ -495,6 +516,264 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         }
 }
 
+// ---- Q4_K on the int8 matrix cores ----------------------------------------------------------------------------------
+// The 6-bit sub-block scale is split as sc = 8 hi + lo (hi, lo < 8): lo * q and hi * q stay below 128, so they are int8
+// operands, and     S[m,n] = sum_k q8[m,k] * sc * q[n,k] = 8 * sum_k q8 (hi q) + sum_k q8 (lo q)
+// is two v_mfma_i32_32x32x32_i8 chains with exact int32 sums over the super-block — the integer the CPU vec_dot forms
+// (k_quants.rs:1460-1540) — followed by the same f32 step as above: acc += d8 * (d * S - dmin * M).  Against the f16
+// formulation: the activations go to LDS as the raw int8 (no conversion, half the bytes), four weights take one
+// v_pk_mul_lo_u16 per term, and a k-slice of 32 needs as many LDS bytes as a k-slice of 16 did.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+constexpr int LDB = BK + 16;           // padded row stride in bytes of an int8 LDS row (80)
+
+__device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, (u16x2)(__builtin_bit_cast(u16x2, a) * __builtin_bit_cast(u16x2, b)));
+}
+__device__ __forceinline__ void lds_write32b(int8_t *dstrow, const uint32_t v[8]) {
+    u32x4 *p = reinterpret_cast<u32x4 *>(dstrow);
+    p[0] = u32x4{v[0], v[1], v[2], v[3]};
+    p[1] = u32x4{v[4], v[5], v[6], v[7]};
+}
+
+// Same tiling and template parameters as qmm_kernel.  Only the activations pass through LDS (double-buffered, one
+// barrier per stage: the next stage is written while the matrix cores work on this one).  The weights never do: the B
+// operand of a 32 x 32 x 32 MFMA wants, in lane (n, kg), 16 consecutive k of row n — for Q4_K the nibbles of one 16-byte
+// piece of the row, low nibbles for the even sub-block of a 64-element stage and high nibbles for the odd one — so every
+// lane loads its own piece (two stages ahead), multiplies it by the two halves of its sub-block scales and feeds the
+// MFMAs from registers.  The lane also holds d, dmin and the sub-block mins of its row for the end of the super-block.
+template <int NJ, bool MOE = false, bool SM = false>
+__global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst,
+                                                                            int k, int n, int rows, int64_t stride_dst, MoeChunks mc,
+                                                                            int64_t expert_bytes, int64_t split_stride) {
+    static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
+    constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;
+    constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
+    __shared__ __align__(16) int8_t As[2][BMT * LDB];
+    __shared__ __align__(16) _Float16 Am[2][BMT * 24];         // bsums16 of the super-block, as f16 (row stride 24 halves)
+    __shared__ float sD8[2][BMT];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int wm = SM ? 0 : wv >> 1, wn = SM ? wv : wv & 1;
+    int m0 = blockIdx.x * BMT;
+    const int n0 = blockIdx.y * BN;
+    if (MOE) {
+        if ((int)blockIdx.x >= mc.n_chunks[0]) return;           // uniform over the workgroup
+        m0 = mc.first[blockIdx.x];
+        rows = m0 + mc.count[blockIdx.x];
+        w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
+    }
+    const bool astage = SM ? tid < 2 * BMT : true;               // threads that stage an activation row (wave-uniform)
+    const int nsb_all = k >> 8;
+    const int kb0 = (int)(((int64_t)nsb_all * blockIdx.z) / gridDim.z), nsb = (int)(((int64_t)nsb_all * (blockIdx.z + 1)) / gridDim.z);
+    dst += (int64_t)blockIdx.z * split_stride;
+    const int64_t row_bytes = (int64_t)(k / 256) * 144;
+
+    // activation staging role: (row r_l of the tile, 32-element half of the stage)
+    const int r_l = tid >> 1, half = tid & 1;
+    const int arow = min(m0 + (astage ? r_l : 0), rows - 1);
+    const bool arow_ok = astage && m0 + r_l < rows;
+    const uint32_t amask = arow_ok ? 0xffffffffu : 0u;
+    const int8_t *aq_p = av.qs + (int64_t)arow * k;
+    // weight role: row of each of the wave's NJ column tiles, and which 16 k of a 32-element slice
+    const int kg = lane >> 5;
+    const uint8_t *wrow_p[NJ];
+#pragma unroll
+    for (int t = 0; t < NJ; t++) wrow_p[t] = w + (int64_t)min(n0 + wn * WN + t * 32 + (lane & 31), n - 1) * row_bytes;
+
+    f32x16 acc[MI][NJ];
+    i32x16 sl[MI][NJ], sh[MI][NJ];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) { acc[i][j][e] = 0.0f; sl[i][j][e] = 0; sh[i][j][e] = 0; }
+
+    // Loads run ahead of their use (two register sets each, chosen by the parity of the stage).  Stage (kb, g) covers
+    // k = 256 kb + 64 g + [0, 64).  Positions past the end of this split's range are clamped to its last super-block:
+    // what they load is converted into an LDS copy, or registers, that nobody reads.
+    u32x4 bq[2][NJ], hdr_cur[NJ], hdr_next[NJ];
+    u32x4 a02[2], a12[2], abs0 = u32x4{0, 0, 0, 0};
+    float ad8 = 0.0f;
+    auto load_b = [&](int kb, int g, u32x4 q[NJ]) {
+        kb = min(kb, nsb - 1);
+#pragma unroll
+        for (int t = 0; t < NJ; t++) q[t] = *reinterpret_cast<const u32x4 *>(wrow_p[t] + (int64_t)kb * 144 + 16 + 32 * g + 16 * kg);
+    };
+    auto load_hdr = [&](int kb, u32x4 h[NJ]) {
+        kb = min(kb, nsb - 1);
+#pragma unroll
+        for (int t = 0; t < NJ; t++) h[t] = *reinterpret_cast<const u32x4 *>(wrow_p[t] + (int64_t)kb * 144);
+    };
+    auto load_a = [&](int kb, int g, u32x4 &x0, u32x4 &x1) {
+        kb = min(kb, nsb - 1);
+        if (astage) {
+            const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
+            x0 = *reinterpret_cast<const u32x4 *>(q);
+            x1 = *reinterpret_cast<const u32x4 *>(q + 16);
+            if (g == 0) {
+                ad8 = av.d[(int64_t)arow * (k >> 8) + kb];
+                abs0 = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
+            }
+        }
+    };
+    // what one thread contributes to the LDS image of a stage
+    struct Conv {
+        uint32_t a[8];
+        float d8;
+        uint32_t bv[4];
+    };
+    auto convert_a = [&](int g, const u32x4 &a0, const u32x4 &a1, Conv &c) {
+        const uint32_t a8[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) c.a[i] = a8[i] & amask;                  // rows past the end contribute zeros
+        if (g == 0) {
+            c.d8 = arow_ok ? ad8 : 0.0f;
+            const uint32_t b4[4] = {abs0.x, abs0.y, abs0.z, abs0.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t lo = f2h_bits((float)(int16_t)(b4[i] & 0xffff)), hi = f2h_bits((float)(int16_t)(b4[i] >> 16));
+                c.bv[i] = (lo | (hi << 16)) & amask;
+            }
+        }
+    };
+    // buf: LDS copy of the stage (its parity); hb: copy of the per-super-block arrays (parity of the super-block)
+    auto store_a = [&](int g, int buf, int hb, const Conv &c) {
+        if (astage) {
+            lds_write32b(As[buf] + r_l * LDB + 32 * half, c.a);
+            if (g == 0) {
+                sD8[hb][r_l] = c.d8;                                          // both threads of a row write the same value
+                *reinterpret_cast<u32x4 *>(Am[hb] + r_l * 24 + 8 * half) = u32x4{c.bv[0], c.bv[1], c.bv[2], c.bv[3]};
+            }
+        }
+    };
+    load_a(kb0, 0, a02[0], a12[0]);
+    load_a(kb0, 1, a02[1], a12[1]);
+    load_hdr(kb0, hdr_cur);
+    load_b(kb0, 0, bq[0]);
+    load_b(kb0, 1, bq[1]);
+#pragma unroll
+    for (int t = 0; t < NJ; t++) hdr_next[t] = hdr_cur[t];
+    {
+        Conv c;
+        convert_a(0, a02[0], a12[0], c);
+        store_a(0, 0, kb0 & 1, c);
+        load_a(kb0, 2, a02[0], a12[0]);
+    }
+    __syncthreads();
+
+    for (int kb = kb0; kb < nsb; kb++) {
+        const int hb = kb & 1;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            // ---- activations of the next stage: registers -> (after the MFMAs) the other LDS copy ----
+            const int ng = (g + 1) & 3, nb = (g + 1) & 1;
+            Conv c;
+            convert_a(ng, a02[nb], a12[nb], c);
+            load_a(g == 0 ? kb : kb + 1, (g + 3) & 3, a02[nb], a12[nb]);
+            // ---- weights of this stage: sub-blocks 2 g (low nibbles) and 2 g + 1 (high nibbles) ----
+            i32x4 bl[2][NJ], bh[2][NJ];
+#pragma unroll
+            for (int t = 0; t < NJ; t++) {
+                const u32x4 q = bq[g & 1][t], h = hdr_cur[t];
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    // 6-bit scale of sub-block j = 2 g + ks (utils.rs:50-60); j < 4 exactly when g < 2
+                    const int sft = 16 * (g & 1) + 8 * ks;
+                    const uint32_t sc = g < 2 ? (h.y >> sft) & 63u : ((h.w >> sft) & 0xFu) | (((h.y >> sft) >> 2) & 0x30u);
+                    const uint32_t lo2 = (sc & 7u) * 0x00010001u, hi2 = (sc >> 3) * 0x00010001u;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const uint32_t v = (ks ? q[i] >> 4 : q[i]) & 0x0f0f0f0fu;        // four weights, one per byte
+                        bl[ks][t][i] = (int)pk_mul_u16(v, lo2);                             // bytes stay below 128: no carries
+                        bh[ks][t][i] = (int)pk_mul_u16(v, hi2);
+                    }
+                }
+            }
+            load_b(g < 2 ? kb : kb + 1, (g + 2) & 3, bq[g & 1]);
+            if (g == 2) load_hdr(kb + 1, hdr_next);
+            // ---- 2 k-slices of 32: MI x NJ tiles, two MFMA chains each ----
+            const int8_t *Ab = As[g & 1];
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                i32x4 af[MI];
+#pragma unroll
+                for (int t = 0; t < MI; t++)
+                    af[t] = *reinterpret_cast<const i32x4 *>(Ab + (wm * 64 + t * 32 + (lane & 31)) * LDB + ks * 32 + 16 * kg);
+#pragma unroll
+                for (int i = 0; i < MI; i++)
+#pragma unroll
+                    for (int j = 0; j < NJ; j++) {
+                        if (g == 0 && ks == 0) {                    // first slice of the super-block: the sums start from zero
+                            i32x16 z;
+#pragma unroll
+                            for (int e = 0; e < 16; e++) z[e] = 0;
+                            sl[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bl[ks][j], z, 0, 0, 0);
+                            sh[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bh[ks][j], z, 0, 0, 0);
+                        } else {
+                            sl[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bl[ks][j], sl[i][j], 0, 0, 0);
+                            sh[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bh[ks][j], sh[i][j], 0, 0, 0);
+                        }
+                    }
+            }
+            store_a(ng, nb, g == 3 ? hb ^ 1 : hb, c);
+            if (g == 3) {
+                // ---- end of the super-block: mins term and the f32 scales ----
+                half8 am[MI];
+#pragma unroll
+                for (int t = 0; t < MI; t++)
+                    am[t] = *reinterpret_cast<const half8 *>(Am[hb] + (wm * 64 + t * 32 + (lane & 31)) * 24 + 8 * kg);
+#pragma unroll
+                for (int j = 0; j < NJ; j++) {
+                    const u32x4 h = hdr_cur[j];
+                    const float d = h2f(h.x), dmin = h2f(h.x >> 16);
+                    // B operand of the mins MFMA: element 2 i, 2 i + 1 of this lane = min of sub-block 4 kg + i, one per
+                    // byte first (sub-blocks 0-3: low 6 bits of h.z; 4-7: high nibbles of h.w | top bits of h.z)
+                    const uint32_t mine = kg ? ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u) : h.z & 0x3f3f3f3fu;
+                    u32x4 mv;
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        mv[i] = pk_add((0x6400u | ((mine >> (8 * i)) & 0xffu)) * 0x00010001u, 0xe400e400u);   // (1024 + min) - 1024, twice
+                    const half8 bm = __builtin_bit_cast(half8, mv);
+#pragma unroll
+                    for (int i = 0; i < MI; i++) {
+                        f32x16 z;
+#pragma unroll
+                        for (int e = 0; e < 16; e++) z[e] = 0.0f;
+                        const f32x16 mt = __builtin_amdgcn_mfma_f32_32x32x16_f16(am[i], bm, z, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 16; e++) {
+                            const int ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * kg + (e & 3);
+                            float t = d * (float)(8 * sh[i][j][e] + sl[i][j][e]);
+                            t = fmaf(-dmin, mt[e], t);
+                            acc[i][j][e] = fmaf(sD8[hb][ml], t, acc[i][j][e]);
+                        }
+                    }
+                    hdr_cur[j] = hdr_next[j];
+                }
+            }
+            __syncthreads();
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const int nn = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int mm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * kg + (e & 3);
+                if (mm < rows && nn < n) {
+                    if (MOE) dst[(int64_t)mc.pair_out[mm] * stride_dst + nn] = acc[i][j][e] * mc.pair_scale[mm];
+                    else dst[(int64_t)mm * stride_dst + nn] = acc[i][j][e];
+                }
+            }
+        }
+}
+
 // dst[m, n] = sum over the split planes, in split order (deterministic); n % 4 == 0 whenever split-K is chosen
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ part, float *__restrict__ dst, int splits, int64_t n,
                                                             int64_t stride_dst, int64_t count) {
@@ -510,12 +789,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
     o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
 }
 
+typedef void (*QmmFn)(const uint8_t *, ActView, float *, int, int, int, int64_t, MoeChunks, int64_t, int64_t);
+// the kernel of a format and tile shape: Q4_K runs on the int8 matrix cores, the other formats on the f16 ones
+template <int DT, int NJ, bool MOE, bool SM>
+QmmFn qmm_fn() {
+    if constexpr (DT == CQ_Q4K) {
+        if (!getenv("CQ_Q4K_F16")) return qmm_q4k_i8_kernel<NJ, MOE, SM>;
+    }
+    return qmm_kernel<DT, NJ, MOE, SM>;
+}
+
 template <int DT>
 int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s,
                float *split_ws) {
     // 128 x 64 tiles (two or three workgroups per CU) everywhere except long Q4_0 / Q8_0 problems, whose cheaper
     // operand conversion leaves the 128 x 128 tile (one workgroup per CU, half the activation conversions) ahead
-    const bool wide = !Stage<DT>::KQ && rows >= 1024;
+    const bool wide = getenv("CQ_WIDE") ? rows >= 64 : !Stage<DT>::KQ && rows >= 1024;
     // a few dozen activation rows (batched decode): 32 x 128 tiles, so that the matrix cores and the activation staging
     // are not spent on 128-row tiles that are mostly padding
     const bool small = rows <= CQ_QMM_SMALL_ROWS;
@@ -528,13 +817,13 @@ int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t 
     float *out = splits > 1 ? split_ws : dst;
     const int64_t ld = splits > 1 ? n : stride_dst, plane = splits > 1 ? rows * n : 0;
     if (small)
-        hipLaunchKernelGGL((qmm_kernel<DT, 1, false, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none,
+        hipLaunchKernelGGL((qmm_fn<DT, 1, false, true>()), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none,
                            (int64_t)0, plane);
     else if (wide)
-        hipLaunchKernelGGL((qmm_kernel<DT, 2>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none, (int64_t)0,
+        hipLaunchKernelGGL((qmm_fn<DT, 2, false, false>()), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none, (int64_t)0,
                            plane);
     else
-        hipLaunchKernelGGL((qmm_kernel<DT, 1>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none, (int64_t)0,
+        hipLaunchKernelGGL((qmm_fn<DT, 1, false, false>()), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, (int)rows, ld, none, (int64_t)0,
                            plane);
     int rc = (int)hipGetLastError();
     if (rc || splits == 1) return rc;
@@ -576,10 +865,10 @@ int launch_qmm_moe(const void *w, const ActView &av, float *out, const MoeChunks
     if (grid.y > 65535) return CQ_ERR_RANGE;
     const int64_t expert_bytes = n * (k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
     if (tile_rows == 32)
-        hipLaunchKernelGGL((qmm_kernel<DT, 1, true, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc,
+        hipLaunchKernelGGL((qmm_fn<DT, 1, true, true>()), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc,
                            expert_bytes, (int64_t)0);
     else
-        hipLaunchKernelGGL((qmm_kernel<DT, 1, true>), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc, expert_bytes,
+        hipLaunchKernelGGL((qmm_fn<DT, 1, true, false>()), grid, dim3(256), 0, s, (const uint8_t *)w, av, out, (int)k, (int)n, 0, n, mc, expert_bytes,
                            (int64_t)0);
     return (int)hipGetLastError();
 }

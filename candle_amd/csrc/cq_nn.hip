@@ -143,6 +143,7 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(float *__restrict__ q, con
 // With one split the normalized result is written directly; otherwise (m, l, unnormalized acc) partials
 // go to the workspace and attn_combine_kernel merges them.
 constexpr int ATT_SPLIT = 128;
+constexpr int CQ_ATTN_ROWS_MIN = 16;        // query rows from which a workgroup takes several rows (attn_rows_kernel)
 
 __device__ __forceinline__ float row16_sum(float v) {      // sum over each aligned group of 16 lanes, in every lane
 #define CQ_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
@@ -286,6 +287,158 @@ __global__ __launch_bounds__(256) void attn_kernel(const float *__restrict__ q, 
             float *pp = part + (((int64_t)r * n_head + head) * splits + sp) * (HD + 2);
             pp[2 + d] = a;
             if (d == 0) { pp[0] = ml[2 * g]; pp[1] = ml[2 * g + 1]; }
+        }
+    }
+}
+
+// The same attention for R consecutive query rows per workgroup (prompts and wide batches): the K and V rows of a split
+// are loaded once for the R * G (row, head) pairs that use them instead of once per row, which is what bounds the
+// one-row kernel on a long prompt (every workgroup pulls 2 * ATT_SPLIT * HD floats through the L2).  Per (row, head) the
+// arithmetic and its order are those of attn_kernel; each row keeps its own causal length.
+template <int HD, int G, int R>
+__global__ __launch_bounds__(256) void attn_rows_kernel(const float *__restrict__ q, int64_t q_stride, const float *__restrict__ k_cache,
+                                                        const float *__restrict__ v_cache, float *__restrict__ out, float *__restrict__ part,
+                                                        const int32_t *__restrict__ pos_dev, int pos0, int rows, int n_head, int ctx,
+                                                        float scale, int splits) {
+    constexpr int VH = G * R;                     // (row, head) pairs of the workgroup, vh = rr * G + g
+    static_assert(VH % 4 == 0 && VH <= 16, "pairs per workgroup");
+    constexpr int DPL = HD / 64, EPL = HD / 16, IT = ATT_SPLIT / 16;
+    __shared__ __attribute__((aligned(16))) float sc[ATT_SPLIT * VH];       // [key][vh]
+    __shared__ float red[4 * VH * HD];
+    __shared__ float ml[2 * VH];
+    const int kvh = blockIdx.x, r0 = blockIdx.y * R, sp = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int nr = min(R, rows - r0);                 // valid rows of this workgroup (>= 1)
+    const int base_len = pos0 + (pos_dev ? pos_dev[0] : 0) + r0 + 1;
+    const int j0 = sp * ATT_SPLIT;
+    const int cnt_max = min(min(base_len + nr - 1, ctx) - j0, ATT_SPLIT);   // keys of the last valid row
+    if (cnt_max <= 0 && splits > 1) {
+        if (tid < VH && tid / G < nr) {
+            float *pp = part + (((int64_t)(r0 + tid / G) * n_head + kvh * G + tid % G) * splits + sp) * (HD + 2);
+            pp[0] = -INFINITY;
+            pp[1] = 0.0f;
+        }
+        return;
+    }
+    const float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
+    const int last = max(cnt_max - 1, 0);
+
+    // ---- phase 1: scores of 16 keys per step, the K rows held in registers across the R rows ----
+    {
+        const int sub = lane & 15, kq = lane >> 4;
+        f32x4 kd[IT][EPL / 4];
+#pragma unroll
+        for (int it = 0; it < IT; it++) {
+            const int key = min(it * 16 + wv * 4 + kq, last);
+            const f32x4 *kr = reinterpret_cast<const f32x4 *>(kb + (int64_t)(j0 + key) * HD + EPL * sub);
+#pragma unroll
+            for (int c = 0; c < EPL / 4; c++) kd[it][c] = kr[c];
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) {
+            const int row = r0 + min(rr, nr - 1);
+            const int cnt = min(min(base_len + rr, ctx) - j0, ATT_SPLIT);
+            f32x4 qf[G][EPL / 4];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const f32x4 *qr = reinterpret_cast<const f32x4 *>(q + row * q_stride + (int64_t)(kvh * G + g) * HD + EPL * sub);
+#pragma unroll
+                for (int c = 0; c < EPL / 4; c++) qf[g][c] = qr[c];
+            }
+#pragma unroll
+            for (int it = 0; it < IT; it++) {
+                const int key = it * 16 + wv * 4 + kq;
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    float a = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < EPL / 4; c++) {
+                        a += qf[g][c].x * kd[it][c].x;
+                        a += qf[g][c].y * kd[it][c].y;
+                        a += qf[g][c].z * kd[it][c].z;
+                        a += qf[g][c].w * kd[it][c].w;
+                    }
+                    a = row16_sum(a);
+                    if (sub == 0) sc[key * VH + rr * G + g] = key < cnt ? a * scale : -INFINITY;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 2: wave w reduces pairs vh = w, w + 4, ... ----
+    for (int vh = wv; vh < VH; vh += 4) {
+        float s[ATT_SPLIT / 64], m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < ATT_SPLIT / 64; i++) {
+            s[i] = sc[(lane + 64 * i) * VH + vh];
+            m = fmaxf(m, s[i]);
+        }
+        m = wave_max(m);
+        float l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < ATT_SPLIT / 64; i++) {
+            const float p = s[i] > -INFINITY ? __expf(s[i] - m) : 0.0f;
+            sc[(lane + 64 * i) * VH + vh] = p;
+            l += p;
+        }
+        l = wave_sum(l);
+        if (lane == 0) { ml[2 * vh] = m; ml[2 * vh + 1] = l; }
+    }
+    __syncthreads();
+
+    // ---- phase 3: wave w accumulates the values of keys w, w + 4, ... for every pair ----
+    float o[VH][DPL];
+#pragma unroll
+    for (int v = 0; v < VH; v++)
+#pragma unroll
+        for (int e = 0; e < DPL; e++) o[v][e] = 0.0f;
+    for (int jb = 0; jb < cnt_max; jb += 32) {
+        float vv[8][DPL];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int j = min(jb + wv + 4 * u, last);
+            if (DPL == 2) {
+                const float2 t = *reinterpret_cast<const float2 *>(vb + (int64_t)(j0 + j) * HD + 2 * lane);
+                vv[u][0] = t.x; vv[u][DPL - 1] = t.y;
+            } else {
+#pragma unroll
+                for (int e = 0; e < DPL; e++) vv[u][e] = vb[(int64_t)(j0 + j) * HD + DPL * lane + e];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int j = jb + wv + 4 * u;                // < ATT_SPLIT; masked entries hold p = 0
+#pragma unroll
+            for (int v4 = 0; v4 < VH / 4; v4++) {
+                const f32x4 p = *reinterpret_cast<const f32x4 *>(&sc[j * VH + 4 * v4]);
+#pragma unroll
+                for (int e = 0; e < DPL; e++) {
+                    o[4 * v4 + 0][e] += p.x * vv[u][e];
+                    o[4 * v4 + 1][e] += p.y * vv[u][e];
+                    o[4 * v4 + 2][e] += p.z * vv[u][e];
+                    o[4 * v4 + 3][e] += p.w * vv[u][e];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VH; v++)
+#pragma unroll
+        for (int e = 0; e < DPL; e++) red[(wv * VH + v) * HD + DPL * lane + e] = o[v][e];
+    __syncthreads();
+    for (int i = tid; i < VH * HD; i += 256) {
+        const int vh = i / HD, d = i - vh * HD;
+        const int rr = vh / G, g = vh - rr * G;
+        if (rr >= nr) continue;
+        const float a = red[(0 * VH + vh) * HD + d] + red[(1 * VH + vh) * HD + d] + red[(2 * VH + vh) * HD + d] + red[(3 * VH + vh) * HD + d];
+        const int head = kvh * G + g;
+        if (splits == 1) {
+            out[((int64_t)(r0 + rr) * n_head + head) * HD + d] = a / ml[2 * vh + 1];
+        } else {
+            float *pp = part + (((int64_t)(r0 + rr) * n_head + head) * splits + sp) * (HD + 2);
+            pp[2 + d] = a;
+            if (d == 0) { pp[0] = ml[2 * vh]; pp[1] = ml[2 * vh + 1]; }
         }
     }
 }
@@ -764,6 +917,25 @@ int launch_attn(int G, dim3 grid, hipStream_t s, const float *q, int64_t q_strid
     return (int)hipGetLastError();
 }
 
+// rows per workgroup of attn_rows_kernel for a grouping of G query heads per kv head (G * R <= 16 pairs)
+inline int attn_rows_per_group(int G) { return G == 8 ? 2 : 4; }
+
+template <int HD>
+int launch_attn_rows(int G, dim3 grid, hipStream_t s, const float *q, int64_t q_stride, const float *kc, const float *vc, float *out,
+                     float *part, const int32_t *pos_dev, int pos0, int rows, int n_head, int ctx, float scale, int splits) {
+#define CQ_ATT(GG, RR)                                                                                                              \
+    case GG:                                                                                                                        \
+        hipLaunchKernelGGL((attn_rows_kernel<HD, GG, RR>), grid, dim3(256), 0, s, q, q_stride, kc, vc, out, part, pos_dev, pos0,    \
+                           rows, n_head, ctx, scale, splits);                                                                       \
+        break;
+    switch (G) {
+        CQ_ATT(1, 4) CQ_ATT(2, 4) CQ_ATT(4, 4) CQ_ATT(8, 2)
+        default: return CQ_ERR_RANGE;
+    }
+#undef CQ_ATT
+    return (int)hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" {
@@ -837,10 +1009,21 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
     const int G = (int)(n_head / n_kv_head);
     dim3 grid((unsigned)n_kv_head, (unsigned)rows, (unsigned)splits);
     hipStream_t s = (hipStream_t)stream;
-    int rc = head_dim == 128 ? launch_attn<128>(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev, pos_dev,
+    int rc;
+    if (rows >= CQ_ATTN_ROWS_MIN && (G == 1 || G == 2 || G == 4 || G == 8)) {
+        // prompts and wide batches: several query rows share each load of the keys and values
+        const int R = attn_rows_per_group(G);
+        grid.y = (unsigned)((rows + R - 1) / R);
+        rc = head_dim == 128 ? launch_attn_rows<128>(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev,
+                                                     pos_dev, (int)pos, (int)rows, (int)n_head, (int)ctx, scale, (int)splits)
+                             : launch_attn_rows<64>(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev,
+                                                    pos_dev, (int)pos, (int)rows, (int)n_head, (int)ctx, scale, (int)splits);
+    } else {
+        rc = head_dim == 128 ? launch_attn<128>(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev, pos_dev,
                                                 (int)pos, (int)n_head, (int)ctx, scale, (int)splits)
                              : launch_attn<64>(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev, pos_dev,
                                                (int)pos, (int)n_head, (int)ctx, scale, (int)splits);
+    }
     if (rc) return rc;
     if (splits > 1) {
         if (head_dim == 128)

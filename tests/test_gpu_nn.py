@@ -116,7 +116,8 @@ def attention_oracle(q, kc, vc, pos, H, KV, D):
 
 
 @pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (4, 4, 128), (8, 2, 128)])
-@pytest.mark.parametrize("rows,pos,ctx", [(1, 0, 32), (1, 199, 256), (1, 600, 1024), (7, 250, 512), (3, 0, 16)])
+@pytest.mark.parametrize("rows,pos,ctx", [(1, 0, 32), (1, 199, 256), (1, 600, 1024), (7, 250, 512), (3, 0, 16),
+                                          (16, 0, 64), (37, 100, 512), (130, 0, 256), (21, 250, 300)])
 def test_attention(H, KV, D, rows, pos, ctx):
     q = normal(8, (rows, H * D), 1.0)
     kc, vc = normal(9, (KV, ctx, D), 1.0), normal(10, (KV, ctx, D), 1.0)
@@ -129,6 +130,25 @@ def test_attention(H, KV, D, rows, pos, ctx):
                                ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None))
         torch.cuda.synchronize()
         assert rel_l2(out.cpu().numpy(), attention_oracle(q, kc, vc, pos, H, KV, D)) <= TOL
+
+
+@pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (4, 4, 128), (32, 8, 128)])
+def test_attention_rows_share_keys_with_position_on_device(H, KV, D):
+    """16 rows and more go several to a workgroup; the position may come from device memory (a captured graph)."""
+    rows, pos, ctx = 19, 120, 384
+    q = normal(14, (rows, H * D), 1.0)
+    kc, vc = normal(15, (KV, ctx, D), 1.0), normal(16, (KV, ctx, D), 1.0)
+    out = torch.full((rows + 1, H * D), 7.0, device="cuda")
+    pos_dev = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    lib = L()
+    wsb = lib.cq_nn_attention_workspace_bytes(rows, H, D, ctx)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+    ok(lib.cq_nn_attention(dev(q).data_ptr(), H * D, dev(kc).data_ptr(), dev(vc).data_ptr(), out.data_ptr(), pos_dev.data_ptr(), 0, rows, H, KV, D,
+                           ctx, ctx, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert rel_l2(got[:rows], attention_oracle(q, kc, vc, pos, H, KV, D)) <= TOL
+    assert np.all(got[rows] == 7.0)                       # the padding rows of the last workgroup write nothing
 
 
 def test_attention_single_key_returns_value():
