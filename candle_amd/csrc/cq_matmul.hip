@@ -526,15 +526,8 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-constexpr int LDB = BK + 16;           // padded row stride in bytes of an int8 LDS row (80)
-
 __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, (u16x2)(__builtin_bit_cast(u16x2, a) * __builtin_bit_cast(u16x2, b)));
-}
-__device__ __forceinline__ void lds_write32b(int8_t *dstrow, const uint32_t v[8]) {
-    u32x4 *p = reinterpret_cast<u32x4 *>(dstrow);
-    p[0] = u32x4{v[0], v[1], v[2], v[3]};
-    p[1] = u32x4{v[4], v[5], v[6], v[7]};
 }
 
 // Same tiling and template parameters as qmm_kernel.  Only the activations pass through LDS (double-buffered, one
@@ -550,7 +543,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
     static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
     constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;
     constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
-    __shared__ __align__(16) int8_t As[2][BMT * LDB];
+    __shared__ __align__(16) int8_t As[2][BMT * BK];
     __shared__ __align__(16) _Float16 Am[2][BMT * 24];         // bsums16 of the super-block, as f16 (row stride 24 halves)
     __shared__ float sD8[2][BMT];
 
@@ -570,12 +563,21 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
     dst += (int64_t)blockIdx.z * split_stride;
     const int64_t row_bytes = (int64_t)(k / 256) * 144;
 
-    // activation staging role: (row r_l of the tile, 32-element half of the stage)
+    // activation staging roles.  Per stage a thread copies two 16-byte pieces: piece pc of rows r_p and r_p + BMT / 2 (four
+    // neighbouring lanes read 64 contiguous bytes of a row).  Per super-block, thread (r_l, half) brings d8 and eight
+    // of the sixteen bsums of row r_l.
     const int r_l = tid >> 1, half = tid & 1;
+    const int r_p = tid >> 2, pc = tid & 3;
+    // LDS image of a stage: 64 bytes per row, the four 16-byte pieces of row r stored at piece ^ ((r >> 1) & 3).  Eight
+    // neighbouring lanes then hit eight different 16-byte bank groups both when they write (four rows x two halves)
+    // and when they read MFMA operands (eight rows, one piece).
+    const int swz_w = (r_p >> 1) & 3, swz_r = (lane >> 1) & 3;      // BMT / 2 is a multiple of 8: both rows of a thread share swz_w
     const int arow = min(m0 + (astage ? r_l : 0), rows - 1);
     const bool arow_ok = astage && m0 + r_l < rows;
     const uint32_t amask = arow_ok ? 0xffffffffu : 0u;
-    const int8_t *aq_p = av.qs + (int64_t)arow * k;
+    const int prow0 = min(m0 + r_p, rows - 1), prow1 = min(m0 + r_p + BMT / 2, rows - 1);
+    const uint32_t pmask0 = m0 + r_p < rows ? 0xffffffffu : 0u, pmask1 = m0 + r_p + BMT / 2 < rows ? 0xffffffffu : 0u;
+    const int8_t *aq_p0 = av.qs + (int64_t)prow0 * k + 16 * pc, *aq_p1 = av.qs + (int64_t)prow1 * k + 16 * pc;
     // weight role: row of each of the wave's NJ column tiles, and which 16 k of a 32-element slice
     const int kg = lane >> 5;
     const uint8_t *wrow_p[NJ];
@@ -610,9 +612,8 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
     auto load_a = [&](int kb, int g, u32x4 &x0, u32x4 &x1) {
         kb = min(kb, nsb - 1);
         if (astage) {
-            const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
-            x0 = *reinterpret_cast<const u32x4 *>(q);
-            x1 = *reinterpret_cast<const u32x4 *>(q + 16);
+            x0 = *reinterpret_cast<const u32x4 *>(aq_p0 + kb * 256 + 64 * g);
+            x1 = *reinterpret_cast<const u32x4 *>(aq_p1 + kb * 256 + 64 * g);
             if (g == 0) {
                 ad8 = av.d[(int64_t)arow * (k >> 8) + kb];
                 abs0 = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
@@ -628,7 +629,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
     auto convert_a = [&](int g, const u32x4 &a0, const u32x4 &a1, Conv &c) {
         const uint32_t a8[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) c.a[i] = a8[i] & amask;                  // rows past the end contribute zeros
+        for (int i = 0; i < 8; i++) c.a[i] = a8[i] & (i < 4 ? pmask0 : pmask1);   // rows past the end contribute zeros
         if (g == 0) {
             c.d8 = arow_ok ? ad8 : 0.0f;
             const uint32_t b4[4] = {abs0.x, abs0.y, abs0.z, abs0.w};
@@ -642,7 +643,8 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
     // buf: LDS copy of the stage (its parity); hb: copy of the per-super-block arrays (parity of the super-block)
     auto store_a = [&](int g, int buf, int hb, const Conv &c) {
         if (astage) {
-            lds_write32b(As[buf] + r_l * LDB + 32 * half, c.a);
+            *reinterpret_cast<u32x4 *>(As[buf] + r_p * BK + 16 * (pc ^ swz_w)) = u32x4{c.a[0], c.a[1], c.a[2], c.a[3]};
+            *reinterpret_cast<u32x4 *>(As[buf] + (r_p + BMT / 2) * BK + 16 * (pc ^ swz_w)) = u32x4{c.a[4], c.a[5], c.a[6], c.a[7]};
             if (g == 0) {
                 sD8[hb][r_l] = c.d8;                                          // both threads of a row write the same value
                 *reinterpret_cast<u32x4 *>(Am[hb] + r_l * 24 + 8 * half) = u32x4{c.bv[0], c.bv[1], c.bv[2], c.bv[3]};
@@ -701,7 +703,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
                 i32x4 af[MI];
 #pragma unroll
                 for (int t = 0; t < MI; t++)
-                    af[t] = *reinterpret_cast<const i32x4 *>(Ab + (wm * 64 + t * 32 + (lane & 31)) * LDB + ks * 32 + 16 * kg);
+                    af[t] = *reinterpret_cast<const i32x4 *>(Ab + (wm * 64 + t * 32 + (lane & 31)) * BK + 16 * ((2 * ks + kg) ^ swz_r));
 #pragma unroll
                 for (int i = 0; i < MI; i++)
 #pragma unroll
