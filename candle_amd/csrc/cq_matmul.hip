@@ -530,12 +530,15 @@ __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, (u16x2)(__builtin_bit_cast(u16x2, a) * __builtin_bit_cast(u16x2, b)));
 }
 
-// Same tiling and template parameters as qmm_kernel.  Only the activations pass through LDS (double-buffered, one
-// barrier per stage: the next stage is written while the matrix cores work on this one).  The weights never do: the B
-// operand of a 32 x 32 x 32 MFMA wants, in lane (n, kg), 16 consecutive k of row n — for Q4_K the nibbles of one 16-byte
-// piece of the row, low nibbles for the even sub-block of a 64-element stage and high nibbles for the odd one — so every
-// lane loads its own piece (two stages ahead), multiplies it by the two halves of its sub-block scales and feeds the
-// MFMAs from registers.  The lane also holds d, dmin and the sub-block mins of its row for the end of the super-block.
+// Same tiling and template parameters as qmm_kernel; a stage is 128 elements of k (half a super-block), held twice in
+// LDS: while the matrix cores work on one copy the threads fill the other (one barrier per stage).  What goes through
+// LDS is raw: the int8 activations, and the weight rows' packed nibbles and 16-byte headers as they lie in memory, both
+// copied with fully used cache lines (8 lanes per 128-byte activation row, 4 per 64-byte weight row) because the
+// address path of the vector cache, not the matrix cores, is what the tile loads saturate first.  Each lane then builds
+// its own MFMA B operands: lane (n, kg) of a 32 x 32 x 32 MFMA wants 16 consecutive k of row n, which for Q4_K are the
+// nibbles of one 16-byte piece — low nibbles for the even sub-block of a 64-element pair, high nibbles for the odd
+// one — times the two halves of the sub-block scale.  16-byte pieces are XOR-swizzled inside their rows so that eight
+// neighbouring lanes always touch eight different bank groups.
 template <int NJ, bool MOE = false, bool SM = false>
 __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst,
                                                                             int k, int n, int rows, int64_t stride_dst, MoeChunks mc,
@@ -543,7 +546,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
     static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
     constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;
     constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
-    __shared__ __align__(16) int8_t As[2][BMT * BK];
+    constexpr int NA = BMT / 32, NB = BN / 64;                 // 16-byte pieces a thread copies per stage: activations, weights
+    __shared__ __align__(16) int8_t As[2][BMT * 128];          // [row][8 pieces], piece p of row r at p ^ (r & 7)
+    __shared__ __align__(16) uint8_t Bq[2][BN * 64];           // [row][4 pieces], piece p of row r at p ^ ((r >> 1) & 3)
+    __shared__ __align__(16) uint8_t Bhd[2][BN * 16];          // block headers (d, dmin, scales), per super-block parity
     __shared__ __align__(16) _Float16 Am[2][BMT * 24];         // bsums16 of the super-block, as f16 (row stride 24 halves)
     __shared__ float sD8[2][BMT];
 
@@ -557,32 +563,28 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
         rows = m0 + mc.count[blockIdx.x];
         w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
     }
-    const bool astage = SM ? tid < 2 * BMT : true;               // threads that stage an activation row (wave-uniform)
     const int nsb_all = k >> 8;
     const int kb0 = (int)(((int64_t)nsb_all * blockIdx.z) / gridDim.z), nsb = (int)(((int64_t)nsb_all * (blockIdx.z + 1)) / gridDim.z);
     dst += (int64_t)blockIdx.z * split_stride;
     const int64_t row_bytes = (int64_t)(k / 256) * 144;
 
-    // activation staging roles.  Per stage a thread copies two 16-byte pieces: piece pc of rows r_p and r_p + BMT / 2 (four
-    // neighbouring lanes read 64 contiguous bytes of a row).  Per super-block, thread (r_l, half) brings d8 and eight
-    // of the sixteen bsums of row r_l.
-    const int r_l = tid >> 1, half = tid & 1;
-    const int r_p = tid >> 2, pc = tid & 3;
-    // LDS image of a stage: 64 bytes per row, the four 16-byte pieces of row r stored at piece ^ ((r >> 1) & 3).  Eight
-    // neighbouring lanes then hit eight different 16-byte bank groups both when they write (four rows x two halves)
-    // and when they read MFMA operands (eight rows, one piece).
-    const int swz_w = (r_p >> 1) & 3, swz_r = (lane >> 1) & 3;      // BMT / 2 is a multiple of 8: both rows of a thread share swz_w
-    const int arow = min(m0 + (astage ? r_l : 0), rows - 1);
-    const bool arow_ok = astage && m0 + r_l < rows;
-    const uint32_t amask = arow_ok ? 0xffffffffu : 0u;
-    const int prow0 = min(m0 + r_p, rows - 1), prow1 = min(m0 + r_p + BMT / 2, rows - 1);
-    const uint32_t pmask0 = m0 + r_p < rows ? 0xffffffffu : 0u, pmask1 = m0 + r_p + BMT / 2 < rows ? 0xffffffffu : 0u;
-    const int8_t *aq_p0 = av.qs + (int64_t)prow0 * k + 16 * pc, *aq_p1 = av.qs + (int64_t)prow1 * k + 16 * pc;
-    // weight role: row of each of the wave's NJ column tiles, and which 16 k of a 32-element slice
-    const int kg = lane >> 5;
-    const uint8_t *wrow_p[NJ];
+    // ---- copy roles.  Rows past the end of the tile are clamped to a valid row: an output row depends on its own
+    // activation row only, and the rows past the end are not stored ----
+    const int ra = tid >> 3, pa = tid & 7;                       // activations: piece pa of rows ra + 32 i
+    const int rb = tid >> 2, pb = tid & 3;                       // weights: piece pb of rows rb + 64 i
+    const int rh = tid & (BN - 1);                               // header of weight row rh
+    const int rs = (tid >> 1) & (BMT - 1), half = tid & 1;       // d8 and eight of the sixteen bsums of activation row rs
+    const int8_t *a_src[NA];
 #pragma unroll
-    for (int t = 0; t < NJ; t++) wrow_p[t] = w + (int64_t)min(n0 + wn * WN + t * 32 + (lane & 31), n - 1) * row_bytes;
+    for (int i = 0; i < NA; i++) a_src[i] = av.qs + (int64_t)min(m0 + ra + 32 * i, rows - 1) * k + 16 * pa;
+    const uint8_t *b_src[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++) b_src[i] = w + (int64_t)min(n0 + rb + 64 * i, n - 1) * row_bytes + 16 + 16 * pb;
+    const uint8_t *h_src = w + (int64_t)min(n0 + rh, n - 1) * row_bytes;
+    const int srow = min(m0 + rs, rows - 1);
+    const int a_dst = ra * 128 + 16 * (pa ^ (ra & 7)), b_dst = rb * 64 + 16 * (pb ^ ((rb >> 1) & 3));
+    // ---- MFMA operand roles ----
+    const int kg = lane >> 5, swz_a = lane & 7, swz_b = (lane >> 1) & 3;
 
     f32x16 acc[MI][NJ];
     i32x16 sl[MI][NJ], sh[MI][NJ];
@@ -593,135 +595,107 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
 #pragma unroll
             for (int e = 0; e < 16; e++) { acc[i][j][e] = 0.0f; sl[i][j][e] = 0; sh[i][j][e] = 0; }
 
-    // Loads run ahead of their use (two register sets each, chosen by the parity of the stage).  Stage (kb, g) covers
-    // k = 256 kb + 64 g + [0, 64).  Positions past the end of this split's range are clamped to its last super-block:
-    // what they load is converted into an LDS copy, or registers, that nobody reads.
-    u32x4 bq[2][NJ], hdr_cur[NJ], hdr_next[NJ];
-    u32x4 a02[2], a12[2], abs0 = u32x4{0, 0, 0, 0};
-    float ad8 = 0.0f;
-    auto load_b = [&](int kb, int g, u32x4 q[NJ]) {
+    // registers of the stage in flight.  Stage (kb, s2) covers k = 256 kb + 128 s2 + [0, 128).  Positions past the end of
+    // this split's range are clamped to its last super-block: what they bring lands in an LDS copy that nobody reads.
+    u32x4 ga[NA], gb[NB], ghdr = u32x4{0, 0, 0, 0}, gbs = u32x4{0, 0, 0, 0};
+    float gd8 = 0.0f;
+    auto load_stage = [&](int kb, int s2) {
         kb = min(kb, nsb - 1);
 #pragma unroll
-        for (int t = 0; t < NJ; t++) q[t] = *reinterpret_cast<const u32x4 *>(wrow_p[t] + (int64_t)kb * 144 + 16 + 32 * g + 16 * kg);
-    };
-    auto load_hdr = [&](int kb, u32x4 h[NJ]) {
-        kb = min(kb, nsb - 1);
+        for (int i = 0; i < NA; i++) ga[i] = *reinterpret_cast<const u32x4 *>(a_src[i] + kb * 256 + 128 * s2);
 #pragma unroll
-        for (int t = 0; t < NJ; t++) h[t] = *reinterpret_cast<const u32x4 *>(wrow_p[t] + (int64_t)kb * 144);
-    };
-    auto load_a = [&](int kb, int g, u32x4 &x0, u32x4 &x1) {
-        kb = min(kb, nsb - 1);
-        if (astage) {
-            x0 = *reinterpret_cast<const u32x4 *>(aq_p0 + kb * 256 + 64 * g);
-            x1 = *reinterpret_cast<const u32x4 *>(aq_p1 + kb * 256 + 64 * g);
-            if (g == 0) {
-                ad8 = av.d[(int64_t)arow * (k >> 8) + kb];
-                abs0 = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
-            }
+        for (int i = 0; i < NB; i++) gb[i] = *reinterpret_cast<const u32x4 *>(b_src[i] + (int64_t)kb * 144 + 64 * s2);
+        if (s2 == 0) {
+            ghdr = *reinterpret_cast<const u32x4 *>(h_src + (int64_t)kb * 144);
+            gd8 = av.d[(int64_t)srow * (k >> 8) + kb];
+            gbs = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)srow * (k >> 4) + kb * 16 + 8 * half);
         }
     };
-    // what one thread contributes to the LDS image of a stage
-    struct Conv {
-        uint32_t a[8];
-        float d8;
-        uint32_t bv[4];
-    };
-    auto convert_a = [&](int g, const u32x4 &a0, const u32x4 &a1, Conv &c) {
-        const uint32_t a8[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    // buf: LDS copy of the stage (s2); hb: copy of the per-super-block arrays (parity of the super-block)
+    auto store_stage = [&](int s2, int hb) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) c.a[i] = a8[i] & (i < 4 ? pmask0 : pmask1);   // rows past the end contribute zeros
-        if (g == 0) {
-            c.d8 = arow_ok ? ad8 : 0.0f;
-            const uint32_t b4[4] = {abs0.x, abs0.y, abs0.z, abs0.w};
+        for (int i = 0; i < NA; i++) *reinterpret_cast<u32x4 *>(As[s2] + a_dst + 32 * 128 * i) = ga[i];
+#pragma unroll
+        for (int i = 0; i < NB; i++) *reinterpret_cast<u32x4 *>(Bq[s2] + b_dst + 64 * 64 * i) = gb[i];
+        if (s2 == 0) {
+            // threads that share a row write the same values
+            *reinterpret_cast<u32x4 *>(Bhd[hb] + 16 * rh) = ghdr;
+            sD8[hb][rs] = gd8;
+            const uint32_t b4[4] = {gbs.x, gbs.y, gbs.z, gbs.w};
+            u32x4 bv;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 uint32_t lo = f2h_bits((float)(int16_t)(b4[i] & 0xffff)), hi = f2h_bits((float)(int16_t)(b4[i] >> 16));
-                c.bv[i] = (lo | (hi << 16)) & amask;
+                bv[i] = lo | (hi << 16);
             }
+            *reinterpret_cast<u32x4 *>(Am[hb] + rs * 24 + 8 * half) = bv;
         }
     };
-    // buf: LDS copy of the stage (its parity); hb: copy of the per-super-block arrays (parity of the super-block)
-    auto store_a = [&](int g, int buf, int hb, const Conv &c) {
-        if (astage) {
-            *reinterpret_cast<u32x4 *>(As[buf] + r_p * BK + 16 * (pc ^ swz_w)) = u32x4{c.a[0], c.a[1], c.a[2], c.a[3]};
-            *reinterpret_cast<u32x4 *>(As[buf] + (r_p + BMT / 2) * BK + 16 * (pc ^ swz_w)) = u32x4{c.a[4], c.a[5], c.a[6], c.a[7]};
-            if (g == 0) {
-                sD8[hb][r_l] = c.d8;                                          // both threads of a row write the same value
-                *reinterpret_cast<u32x4 *>(Am[hb] + r_l * 24 + 8 * half) = u32x4{c.bv[0], c.bv[1], c.bv[2], c.bv[3]};
-            }
-        }
-    };
-    load_a(kb0, 0, a02[0], a12[0]);
-    load_a(kb0, 1, a02[1], a12[1]);
-    load_hdr(kb0, hdr_cur);
-    load_b(kb0, 0, bq[0]);
-    load_b(kb0, 1, bq[1]);
-#pragma unroll
-    for (int t = 0; t < NJ; t++) hdr_next[t] = hdr_cur[t];
-    {
-        Conv c;
-        convert_a(0, a02[0], a12[0], c);
-        store_a(0, 0, kb0 & 1, c);
-        load_a(kb0, 2, a02[0], a12[0]);
-    }
+    load_stage(kb0, 0);
+    store_stage(0, kb0 & 1);
+    load_stage(kb0, 1);
     __syncthreads();
 
     for (int kb = kb0; kb < nsb; kb++) {
         const int hb = kb & 1;
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            // ---- activations of the next stage: registers -> (after the MFMAs) the other LDS copy ----
-            const int ng = (g + 1) & 3, nb = (g + 1) & 1;
-            Conv c;
-            convert_a(ng, a02[nb], a12[nb], c);
-            load_a(g == 0 ? kb : kb + 1, (g + 3) & 3, a02[nb], a12[nb]);
-            // ---- weights of this stage: sub-blocks 2 g (low nibbles) and 2 g + 1 (high nibbles) ----
-            i32x4 bl[2][NJ], bh[2][NJ];
+        for (int s2 = 0; s2 < 2; s2++) {
+            const int8_t *Ab = As[s2];
+            const uint8_t *Bb = Bq[s2];
+            u32x4 hdr[NJ];
 #pragma unroll
-            for (int t = 0; t < NJ; t++) {
-                const u32x4 q = bq[g & 1][t], h = hdr_cur[t];
+            for (int t = 0; t < NJ; t++) hdr[t] = *reinterpret_cast<const u32x4 *>(Bhd[hb] + 16 * (wn * WN + t * 32 + (lane & 31)));
 #pragma unroll
-                for (int ks = 0; ks < 2; ks++) {
-                    // 6-bit scale of sub-block j = 2 g + ks (utils.rs:50-60); j < 4 exactly when g < 2
-                    const int sft = 16 * (g & 1) + 8 * ks;
-                    const uint32_t sc = g < 2 ? (h.y >> sft) & 63u : ((h.w >> sft) & 0xFu) | (((h.y >> sft) >> 2) & 0x30u);
-                    const uint32_t lo2 = (sc & 7u) * 0x00010001u, hi2 = (sc >> 3) * 0x00010001u;
+            for (int gg = 0; gg < 2; gg++) {
+                const int g = 2 * s2 + gg;
+                // ---- weights of sub-blocks 2 g (low nibbles) and 2 g + 1 (high nibbles) ----
+                i32x4 bl[2][NJ], bh[2][NJ];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const uint32_t v = (ks ? q[i] >> 4 : q[i]) & 0x0f0f0f0fu;        // four weights, one per byte
-                        bl[ks][t][i] = (int)pk_mul_u16(v, lo2);                             // bytes stay below 128: no carries
-                        bh[ks][t][i] = (int)pk_mul_u16(v, hi2);
-                    }
-                }
-            }
-            load_b(g < 2 ? kb : kb + 1, (g + 2) & 3, bq[g & 1]);
-            if (g == 2) load_hdr(kb + 1, hdr_next);
-            // ---- 2 k-slices of 32: MI x NJ tiles, two MFMA chains each ----
-            const int8_t *Ab = As[g & 1];
+                for (int t = 0; t < NJ; t++) {
+                    const u32x4 q = *reinterpret_cast<const u32x4 *>(Bb + (wn * WN + t * 32 + (lane & 31)) * 64 + 16 * ((2 * gg + kg) ^ swz_b));
+                    const u32x4 h = hdr[t];
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-                i32x4 af[MI];
+                    for (int ks = 0; ks < 2; ks++) {
+                        // 6-bit scale of sub-block j = 2 g + ks (utils.rs:50-60); j < 4 exactly when g < 2
+                        const int sft = 16 * (g & 1) + 8 * ks;
+                        const uint32_t sc = g < 2 ? (h.y >> sft) & 63u : ((h.w >> sft) & 0xFu) | (((h.y >> sft) >> 2) & 0x30u);
+                        const uint32_t lo2 = (sc & 7u) * 0x00010001u, hi2 = (sc >> 3) * 0x00010001u;
 #pragma unroll
-                for (int t = 0; t < MI; t++)
-                    af[t] = *reinterpret_cast<const i32x4 *>(Ab + (wm * 64 + t * 32 + (lane & 31)) * BK + 16 * ((2 * ks + kg) ^ swz_r));
-#pragma unroll
-                for (int i = 0; i < MI; i++)
-#pragma unroll
-                    for (int j = 0; j < NJ; j++) {
-                        if (g == 0 && ks == 0) {                    // first slice of the super-block: the sums start from zero
-                            i32x16 z;
-#pragma unroll
-                            for (int e = 0; e < 16; e++) z[e] = 0;
-                            sl[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bl[ks][j], z, 0, 0, 0);
-                            sh[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bh[ks][j], z, 0, 0, 0);
-                        } else {
-                            sl[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bl[ks][j], sl[i][j], 0, 0, 0);
-                            sh[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bh[ks][j], sh[i][j], 0, 0, 0);
+                        for (int i = 0; i < 4; i++) {
+                            const uint32_t v = (ks ? q[i] >> 4 : q[i]) & 0x0f0f0f0fu;    // four weights, one per byte
+                            bl[ks][t][i] = (int)pk_mul_u16(v, lo2);                         // bytes stay below 128: no carries
+                            bh[ks][t][i] = (int)pk_mul_u16(v, hi2);
                         }
                     }
+                }
+                // ---- 2 k-slices of 32: MI x NJ tiles, two MFMA chains each ----
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    i32x4 af[MI];
+#pragma unroll
+                    for (int t = 0; t < MI; t++)
+                        af[t] = *reinterpret_cast<const i32x4 *>(Ab + (wm * 64 + t * 32 + (lane & 31)) * 128 + 16 * ((4 * gg + 2 * ks + kg) ^ swz_a));
+#pragma unroll
+                    for (int i = 0; i < MI; i++)
+#pragma unroll
+                        for (int j = 0; j < NJ; j++) {
+                            if (g == 0 && ks == 0) {                    // first slice of the super-block: the sums start from zero
+                                i32x16 z;
+#pragma unroll
+                                for (int e = 0; e < 16; e++) z[e] = 0;
+                                sl[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bl[ks][j], z, 0, 0, 0);
+                                sh[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bh[ks][j], z, 0, 0, 0);
+                            } else {
+                                sl[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bl[ks][j], sl[i][j], 0, 0, 0);
+                                sh[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bh[ks][j], sh[i][j], 0, 0, 0);
+                            }
+                        }
+                }
             }
-            store_a(ng, nb, g == 3 ? hb ^ 1 : hb, c);
-            if (g == 3) {
+            // ---- the stage in flight goes to the other LDS copy; its registers take the stage after it ----
+            store_stage(s2 ^ 1, s2 ? hb ^ 1 : hb);
+            load_stage(kb + 1, s2);
+            if (s2 == 1) {
                 // ---- end of the super-block: mins term and the f32 scales ----
                 half8 am[MI];
 #pragma unroll
@@ -729,7 +703,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
                     am[t] = *reinterpret_cast<const half8 *>(Am[hb] + (wm * 64 + t * 32 + (lane & 31)) * 24 + 8 * kg);
 #pragma unroll
                 for (int j = 0; j < NJ; j++) {
-                    const u32x4 h = hdr_cur[j];
+                    const u32x4 h = hdr[j];
                     const float d = h2f(h.x), dmin = h2f(h.x >> 16);
                     // B operand of the mins MFMA: element 2 i, 2 i + 1 of this lane = min of sub-block 4 kg + i, one per
                     // byte first (sub-blocks 0-3: low 6 bits of h.z; 4-7: high nibbles of h.w | top bits of h.z)
@@ -753,7 +727,6 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
                             acc[i][j][e] = fmaf(sD8[hb][ml], t, acc[i][j][e]);
                         }
                     }
-                    hdr_cur[j] = hdr_next[j];
                 }
             }
             __syncthreads();
