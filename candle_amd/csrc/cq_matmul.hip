@@ -5,26 +5,28 @@
 // candle-kernels/src/mmq_gguf/).  The arithmetic follows the CPU path instead of the CUDA one:
 // activations are the Q8_K / Q8_0 quantization written by cq_quantize_act.
 //
-// K-quants (Q4_K, Q5_K, Q6_K) — integer-exact formulation on the f16 matrix cores:
+// Q5_K, Q6_K — integer-exact formulation on the f16 matrix cores (qmm_kernel):
 //   per 256-element super-block kb      S[m,n] = sum_k q8[m,k] * (sc[n,sub(k)] * q[n,k])
-//   operands are small integers held exactly in f16 (|q8| <= 128, |sc*q| <= 1953 for Q4_K/Q5_K),
+//   operands are small integers held exactly in f16 (|q8| <= 128, |sc*q| <= 1953 for Q5_K),
 //   products accumulate in f32, and once per super-block
 //       acc[m,n] += d8[m,kb] * ( d[n,kb] * S[m,n] - dmin[n,kb] * M[m,n] ),
-//       M[m,n] = sum_{j<16} bsums16[m,j] * min[n,j/2]          (one extra K=16 MFMA, Q4_K/Q5_K only)
-//   — the same integers the CPU vec_dot sums (k_quants.rs:1460-1540, 1714-1801, 2035-2092).  For Q6_K
+//       M[m,n] = sum_{j<16} bsums16[m,j] * min[n,j/2]          (one extra K=16 MFMA, Q5_K only)
+//   — the same integers the CPU vec_dot sums (k_quants.rs:1714-1801, 2035-2092).  For Q6_K
 //   the product sc*(q-32) can reach 4096, beyond the exact-integer range of f16, so it is fed as two
 //   terms: its f16 rounding and the exact remainder in {-1, 0, 1} (a second MFMA per k-slice).  This
 //   matters: a 1e-4 perturbation of one matmul is amplified to ~1e-2 in a decoder's logits by the
 //   activation quantizers downstream, an exact one is not.
+// Q4_K — the same sums on the int8 matrix cores (qmm_q4k_i8_kernel, k_quants.rs:1460-1540): the 6-bit sub-block scale
+//   is split into two 3-bit halves so that scale * weight fits int8; S is exact in int32.
 // Q4_0 / Q8_0 — both operands carry a per-32 f16 scale, so the dequantized values d*(q-8) and d8*q8
 //   are rounded to f16 (relative 2^-11 per operand) and multiplied at full MFMA rate; the result stays
 //   well inside the 1e-3 tolerance (measured ~2e-4) but is not integer-exact like the decode path.
 //
-// Tiling: workgroup = 4 waves (2 x 2), block tile 128 (m) x 64 (n), wave tile 64 x 32 as 2 x 1
-// v_mfma_f32_32x32x16_f16 tiles (128 x 128 / 64 x 64 for long Q4_0 / Q8_0 problems).  K advances 64 elements per
-// LDS stage: the threads dequantize the weight tile and convert the 128 x 64 int8 activation tile to f16 in LDS
-// (row stride padded to 144 bytes); raw bytes are requested two stages ahead into two register sets.
-#include <cstdlib>
+// Tiling: workgroup = 4 waves (2 x 2), block tile 128 (m) x 64 (n), wave tile 64 x 32 as 2 x 1 MFMA tiles of 32 x 32
+// (128 x 128 / 64 x 64 for large Q4_0 / Q8_0 problems, 32 x 128 with the waves side by side for up to 32 rows).
+// qmm_kernel advances K by 64 elements per LDS stage: the threads dequantize the weight tile and convert the 128 x 64 int8
+// activation tile to f16 into one of two LDS copies (row stride padded to 144 bytes) while the MFMAs run on the other;
+// raw bytes are requested two stages ahead into two register sets.
 #include "cq_device.h"
 #include "cq_launch.h"
 
@@ -78,38 +80,6 @@ __device__ __forceinline__ void k4_sub_scale_min(uint32_t u0, uint32_t u1, uint3
 // ---- per-format staging of one (row, 32-element sub-block) of W into 16 dwords of f16 pairs -------
 // raw: what one thread loads for (row n, k-range [kb*256 + 64*g + 32*half, +32)).
 template <int DT> struct Stage;
-
-template <> struct Stage<CQ_Q4K> {
-    static constexpr bool KQ = true, HAS_MIN = true;
-    static constexpr int TERMS = 1;
-    struct Raw { u32x4 hdr, q0, q1; };
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int) {
-        const uint8_t *blk = row + (int64_t)kb * 144;
-        r.hdr = *reinterpret_cast<const u32x4 *>(blk);
-        r.q0 = *reinterpret_cast<const u32x4 *>(blk + 16 + 32 * g);
-        r.q1 = *reinterpret_cast<const u32x4 *>(blk + 32 + 32 * g);
-    }
-    static __device__ __forceinline__ void header(const Raw &r, float &d, float &dmin, int mins[8]) {
-        d = h2f(r.hdr.x);
-        dmin = h2f(r.hdr.x >> 16);
-#pragma unroll
-        for (int j = 0; j < 8; j++) { int sc; k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, j, sc, mins[j]); }
-    }
-    // 32 values sc*q as f16 pairs, element order = k order
-    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) {
-        int sc, mn;
-        k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g + half, sc, mn);
-        const uint32_t s2 = h2_splat((float)sc), c2 = h2_splat(-1024.0f * (float)sc);
-        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            uint32_t v = (half ? (q[i] >> 4) : q[i]) & 0x0f0f0f0fu, lo, hi;
-            bytes_to_h1024(v, lo, hi);
-            out[2 * i] = pk_fma(lo, s2, c2);        // (1024 + q) * sc - 1024 * sc = sc * q, one exact rounding
-            out[2 * i + 1] = pk_fma(hi, s2, c2);
-        }
-    }
-};
 
 template <> struct Stage<CQ_Q5K> {
     static constexpr bool KQ = true, HAS_MIN = true;
@@ -768,18 +738,18 @@ typedef void (*QmmFn)(const uint8_t *, ActView, float *, int, int, int, int64_t,
 // the kernel of a format and tile shape: Q4_K runs on the int8 matrix cores, the other formats on the f16 ones
 template <int DT, int NJ, bool MOE, bool SM>
 QmmFn qmm_fn() {
-    if constexpr (DT == CQ_Q4K) {
-        if (!getenv("CQ_Q4K_F16")) return qmm_q4k_i8_kernel<NJ, MOE, SM>;
-    }
-    return qmm_kernel<DT, NJ, MOE, SM>;
+    if constexpr (DT == CQ_Q4K) return qmm_q4k_i8_kernel<NJ, MOE, SM>;
+    else return qmm_kernel<DT, NJ, MOE, SM>;
 }
 
 template <int DT>
 int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s,
                float *split_ws) {
-    // 128 x 64 tiles (two or three workgroups per CU) everywhere except long Q4_0 / Q8_0 problems, whose cheaper
-    // operand conversion leaves the 128 x 128 tile (one workgroup per CU, half the activation conversions) ahead
-    const bool wide = getenv("CQ_WIDE") ? rows >= 64 : !Stage<DT>::KQ && rows >= 1024;
+    // 128 x 64 tiles (two workgroups per CU) everywhere except Q4_0 / Q8_0 problems whose grid of 128 x 128 tiles still
+    // covers the chip: their cheap operand conversion leaves that tile (one workgroup per CU, half the activation
+    // conversions) ahead (measured in TFLOP/s, Q4_0 14336 x 4096: 512 rows 471 -> 582, 2048 rows 527 -> 650; Q8_0
+    // 4096 x 4096: 2048 rows 419 -> 520, but 512 rows, a grid of 128, 340 -> 207)
+    const bool wide = !cq_is_kquant(DT) && ((rows + 127) / 128) * ((n + 127) / 128) >= 384;
     // a few dozen activation rows (batched decode): 32 x 128 tiles, so that the matrix cores and the activation staging
     // are not spent on 128-row tiles that are mostly padding
     const bool small = rows <= CQ_QMM_SMALL_ROWS;
@@ -883,11 +853,13 @@ int cq_qmm_splits(int64_t k, int64_t n, int64_t rows) {
     return sp < 2 ? 1 : (int)sp;
 }
 
-// Which row counts go to the matrix cores: everything beyond the matvec kernel's 8 rows (measured, Q4_K 14336 x 4096 /
-// 4096 x 14336: 8 rows on the matvec 27 / 28 us, 9-32 rows on the 32-row MFMA tile 36-41 us).
+// Which row counts go to the matrix cores: everything beyond the matvec kernel's 8 rows, and for Q4_K, whose int8 kernel is
+// the faster one, from 6 rows (measured, Q4_K 14336 x 4096 / 4096 x 14336 in us: matvec at 4 / 5 / 6 / 8 rows 19.4 / 21.6 /
+// 23.4 / 27.5 and 18.3 / 20.8 / 23.6 / 29.9, the 32-row MFMA tile 20.7 and 22.3 at any of them, 21.3 / 23.0 at 16 / 32 rows).
+constexpr int CQ_Q4K_MFMA_MIN_ROWS = 6;
 bool cq_use_mfma(int w_dtype, int64_t rows, int64_t k) {
-    (void)w_dtype;
-    return k % 256 == 0 && rows > CQ_MATVEC_MAX_ROWS;
+    if (k % 256) return false;
+    return rows > CQ_MATVEC_MAX_ROWS || (w_dtype == CQ_Q4K && rows >= CQ_Q4K_MFMA_MIN_ROWS);
 }
 
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
