@@ -77,40 +77,46 @@ __device__ __forceinline__ void k4_sub_scale_min(uint32_t u0, uint32_t u1, uint3
     }
 }
 
-// ---- per-format staging of one (row, 32-element sub-block) of W into 16 dwords of f16 pairs -------
-// raw: what one thread loads for (row n, k-range [kb*256 + 64*g + 32*half, +32)).
+// ---- per-format staging of NW = 32 or 16 consecutive weights of one row into NW / 2 dwords of f16 pairs -------
+// A 64-element stage (kb, g) of a row is split between 64 / NW threads; thread `part` takes elements
+// 256 kb + 64 g + NW part + [0, NW).  jh = the 32-element half of the stage these lie in, sx = which 16 of that half
+// (NW = 16 only).  Raw<NW>: what the thread loads for them.
 template <int DT> struct Stage;
 
 template <> struct Stage<CQ_Q5K> {
     static constexpr bool KQ = true, HAS_MIN = true;
     static constexpr int TERMS = 1;
-    struct Raw { u32x4 hdr, h0, h1, q0, q1; };
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int) {
+    template <int NW> struct Raw { u32x4 hdr, h[NW / 16], q[NW / 16]; };
+    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
         const uint8_t *blk = row + (int64_t)kb * 176;
+        const int sx = NW == 16 ? part & 1 : 0;
         r.hdr = *reinterpret_cast<const u32x4 *>(blk);
-        r.h0 = *reinterpret_cast<const u32x4 *>(blk + 16);
-        r.h1 = *reinterpret_cast<const u32x4 *>(blk + 32);
-        r.q0 = *reinterpret_cast<const u32x4 *>(blk + 48 + 32 * g);
-        r.q1 = *reinterpret_cast<const u32x4 *>(blk + 64 + 32 * g);
+#pragma unroll
+        for (int i = 0; i < NW / 16; i++) {
+            r.h[i] = *reinterpret_cast<const u32x4 *>(blk + 16 + 16 * (sx + i));
+            r.q[i] = *reinterpret_cast<const u32x4 *>(blk + 48 + 32 * g + 16 * (sx + i));
+        }
     }
-    static __device__ __forceinline__ void header(const Raw &r, float &d, float &dmin, int mins[8]) {
+    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &r, float &d, float &dmin) {
         d = h2f(r.hdr.x);
         dmin = h2f(r.hdr.x >> 16);
-#pragma unroll
-        for (int j = 0; j < 8; j++) { int sc; k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, j, sc, mins[j]); }
     }
-    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) {
+    // the four sub-block mins 4 hi .. 4 hi + 3, one per byte (utils.rs:50-60)
+    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &r, int hi) {
+        return hi ? ((r.hdr.w >> 4) & 0x0f0f0f0fu) | ((r.hdr.z >> 2) & 0x30303030u) : r.hdr.z & 0x3f3f3f3fu;
+    }
+    template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int g, int part, uint32_t out[NW / 2]) {
+        const int jh = NW == 16 ? part >> 1 : part;
         int sc, mn;
-        k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g + half, sc, mn);
+        k4_sub_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g + jh, sc, mn);
         const uint32_t s2 = h2_splat((float)sc), c2 = h2_splat(-1024.0f * (float)sc);
-        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-        const uint32_t h[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            uint32_t hb = (h[i] >> (2 * g + half)) & 0x01010101u;
-            uint32_t v = ((half ? (q[i] >> 4) : q[i]) & 0x0f0f0f0fu) | (hb << 4), lo, hi;
+        for (int i = 0; i < NW / 4; i++) {
+            const uint32_t hb = (r.h[i >> 2][i & 3] >> (2 * g + jh)) & 0x01010101u;
+            const uint32_t v = ((r.q[i >> 2][i & 3] >> (4 * jh)) & 0x0f0f0f0fu) | (hb << 4);
+            uint32_t lo, hi;
             bytes_to_h1024(v, lo, hi);
-            out[2 * i] = pk_fma(lo, s2, c2);
+            out[2 * i] = pk_fma(lo, s2, c2);        // (1024 + q) * sc - 1024 * sc = sc * q, one exact rounding
             out[2 * i + 1] = pk_fma(hi, s2, c2);
         }
     }
@@ -119,38 +125,40 @@ template <> struct Stage<CQ_Q5K> {
 template <> struct Stage<CQ_Q6K> {
     static constexpr bool KQ = true, HAS_MIN = false;
     static constexpr int TERMS = 2;      // sc * (q - 32) reaches 4096: f16 head + exact remainder in {-1, 0, 1}
-    // sub-block (g, half) = elements 64g + 32half + [0, 32): half h6 = g >> 1 of the block, quarter = 2*(g&1) + half
-    struct Raw { u32x4 l0, l1, h0, h1; uint32_t sc, d; };
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
+    // 32-element half (g, jh) = elements 64g + 32jh + [0, 32): half h6 = g >> 1 of the block, quarter = 2*(g&1) + jh
+    template <int NW> struct Raw { u32x4 l[NW / 16], h[NW / 16]; uint32_t sc, d; };
+    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
         const uint8_t *blk = row + (int64_t)kb * 210;
-        const int h6 = g >> 1, quarter = 2 * (g & 1) + half;
+        const int jh = NW == 16 ? part >> 1 : part, sx = NW == 16 ? part & 1 : 0;
+        const int h6 = g >> 1, quarter = 2 * (g & 1) + jh;
         const uint8_t *ql = blk + 64 * h6 + ((quarter & 1) ? 32 : 0);   // ql[l] or ql[l + 32], l = 0..31
-        r.l0 = ld_u<u32x4>(ql);
-        r.l1 = ld_u<u32x4>(ql + 16);
-        r.h0 = ld_u<u32x4>(blk + 128 + 32 * h6);
-        r.h1 = ld_u<u32x4>(blk + 128 + 32 * h6 + 16);
-        // scales of this quarter: index 8*h6 + 2*quarter + {0, 1} (l / 16)
-        r.sc = ld_u<uint16_t>(blk + 192 + 8 * h6 + 2 * quarter);
+#pragma unroll
+        for (int i = 0; i < NW / 16; i++) {
+            r.l[i] = ld_u<u32x4>(ql + 16 * (sx + i));
+            r.h[i] = ld_u<u32x4>(blk + 128 + 32 * h6 + 16 * (sx + i));
+        }
+        // scales of this quarter: index 8*h6 + 2*quarter + l / 16
+        if (NW == 16) r.sc = blk[192 + 8 * h6 + 2 * quarter + sx];
+        else r.sc = ld_u<uint16_t>(blk + 192 + 8 * h6 + 2 * quarter);
         r.d = ld_u<uint16_t>(blk + 208);
     }
-    static __device__ __forceinline__ void header(const Raw &r, float &d, float &dmin, int mins[8]) {
+    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &r, float &d, float &dmin) {
         d = h2f(r.d);
         dmin = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 8; j++) mins[j] = 0;
     }
-    static __device__ __forceinline__ void convert(const Raw &r, int g, int half, uint32_t out[16]) { convert2(r, g, half, out, out); }
+    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &, int) { return 0; }
     // out = f16(sc * (q - 32)) (rounds odd products above 2048 to even), rem = sc * (q - 32) - out exactly
-    static __device__ __forceinline__ void convert2(const Raw &r, int g, int half, uint32_t out[16], uint32_t rem[16]) {
-        const int quarter = 2 * (g & 1) + half;
-        const uint32_t sA = h2_splat((float)(int8_t)(r.sc & 0xff)), sB = h2_splat((float)(int8_t)(r.sc >> 8));
+    template <int NW>
+    static __device__ __forceinline__ void convert2(const Raw<NW> &r, int g, int part, uint32_t out[NW / 2], uint32_t rem[NW / 2]) {
+        const int jh = NW == 16 ? part >> 1 : part;
+        const int quarter = 2 * (g & 1) + jh;
+        const uint32_t sA = h2_splat((float)(int8_t)(r.sc & 0xff)), sB = h2_splat((float)(int8_t)((r.sc >> 8) & 0xff));
         const uint32_t off = h2_splat(-1056.0f);                       // -(1024 + 32)
-        const uint32_t ql[8] = {r.l0.x, r.l0.y, r.l0.z, r.l0.w, r.l1.x, r.l1.y, r.l1.z, r.l1.w};
-        const uint32_t qh[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            uint32_t lo4 = ((quarter >= 2) ? (ql[i] >> 4) : ql[i]) & 0x0f0f0f0fu;
-            uint32_t hi2 = ((qh[i] >> (2 * quarter)) & 0x03030303u) << 4;
+        for (int i = 0; i < NW / 4; i++) {
+            const uint32_t lw = r.l[i >> 2][i & 3], hw = r.h[i >> 2][i & 3];
+            uint32_t lo4 = (lw >> (quarter >= 2 ? 4 : 0)) & 0x0f0f0f0fu;
+            uint32_t hi2 = ((hw >> (2 * quarter)) & 0x03030303u) << 4;
             uint32_t lo, hi;
             bytes_to_h1024(lo4 | hi2, lo, hi);
             const uint32_t s2 = i < 4 ? sA : sB;                         // l / 16
@@ -167,29 +175,34 @@ template <> struct Stage<CQ_Q6K> {
 template <> struct Stage<CQ_Q4_0> {
     static constexpr bool KQ = false, HAS_MIN = false;
     static constexpr int TERMS = 1;
-    struct Raw { u32x4 qs; uint32_t d; };
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
-        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + half) * 18;
+    template <int NW> struct Raw { u32x4 qs; uint32_t d; };
+    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
+        const int jh = NW == 16 ? part >> 1 : part;
+        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + jh) * 18;
         r.d = ld_u<uint16_t>(blk);
         r.qs = ld_u<u32x4>(blk + 2);
     }
-    static __device__ __forceinline__ void header(const Raw &, float &d, float &dmin, int mins[8]) {
-        d = 1.0f; dmin = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 8; j++) mins[j] = 0;
-    }
-    static __device__ __forceinline__ void convert(const Raw &r, int, int, uint32_t out[16]) {
+    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &, float &d, float &dmin) { d = 1.0f; dmin = 0.0f; }
+    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &, int) { return 0; }
+    // elements 0..15 of a block are the low nibbles of its 16 bytes, elements 16..31 the high nibbles
+    template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int, int part, uint32_t out[NW / 2]) {
         const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1032.0f);   // -(1024 + 8)
         const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             uint32_t lo, hi;
-            bytes_to_h1024(q[i] & 0x0f0f0f0fu, lo, hi);               // elements 4i..4i+3
-            out[2 * i] = pk_mul(pk_add(lo, off), d2);
-            out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
-            bytes_to_h1024((q[i] >> 4) & 0x0f0f0f0fu, lo, hi);        // elements 16+4i..
-            out[8 + 2 * i] = pk_mul(pk_add(lo, off), d2);
-            out[8 + 2 * i + 1] = pk_mul(pk_add(hi, off), d2);
+            if constexpr (NW == 32) {
+                bytes_to_h1024(q[i] & 0x0f0f0f0fu, lo, hi);               // elements 4i..4i+3
+                out[2 * i] = pk_mul(pk_add(lo, off), d2);
+                out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
+                bytes_to_h1024((q[i] >> 4) & 0x0f0f0f0fu, lo, hi);        // elements 16+4i..
+                out[8 + 2 * i] = pk_mul(pk_add(lo, off), d2);
+                out[8 + 2 * i + 1] = pk_mul(pk_add(hi, off), d2);
+            } else {
+                bytes_to_h1024((q[i] >> (4 * (part & 1))) & 0x0f0f0f0fu, lo, hi);
+                out[2 * i] = pk_mul(pk_add(lo, off), d2);
+                out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
+            }
         }
     }
 };
@@ -197,25 +210,22 @@ template <> struct Stage<CQ_Q4_0> {
 template <> struct Stage<CQ_Q8_0> {
     static constexpr bool KQ = false, HAS_MIN = false;
     static constexpr int TERMS = 1;
-    struct Raw { u32x4 q0, q1; uint32_t d; };
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *row, int kb, int g, int half) {
-        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + half) * 34;
+    template <int NW> struct Raw { u32x4 q[NW / 16]; uint32_t d; };
+    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
+        const int jh = NW == 16 ? part >> 1 : part, sx = NW == 16 ? part & 1 : 0;
+        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + jh) * 34;
         r.d = ld_u<uint16_t>(blk);
-        r.q0 = ld_u<u32x4>(blk + 2);
-        r.q1 = ld_u<u32x4>(blk + 18);
-    }
-    static __device__ __forceinline__ void header(const Raw &, float &d, float &dmin, int mins[8]) {
-        d = 1.0f; dmin = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 8; j++) mins[j] = 0;
+        for (int i = 0; i < NW / 16; i++) r.q[i] = ld_u<u32x4>(blk + 2 + 16 * (sx + i));
     }
-    static __device__ __forceinline__ void convert(const Raw &r, int, int, uint32_t out[16]) {
+    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &, float &d, float &dmin) { d = 1.0f; dmin = 0.0f; }
+    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &, int) { return 0; }
+    template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int, int, uint32_t out[NW / 2]) {
         const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1152.0f);   // -(1024 + 128)
-        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
+        for (int i = 0; i < NW / 4; i++) {
             uint32_t lo, hi;
-            bytes_to_h1024(q[i] ^ 0x80808080u, lo, hi);               // int8 -> biased unsigned
+            bytes_to_h1024(r.q[i >> 2][i & 3] ^ 0x80808080u, lo, hi);               // int8 -> biased unsigned
             out[2 * i] = pk_mul(pk_add(lo, off), d2);
             out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
         }
@@ -237,12 +247,11 @@ __device__ __forceinline__ void act_convert(const u32x4 &a0, const u32x4 &a1, bo
     }
 }
 
-__device__ __forceinline__ void lds_write32h(_Float16 *dstrow, const uint32_t v[16]) {
+// NH halves (NH / 2 dwords of f16 pairs) to a 16-byte aligned LDS address
+template <int NH> __device__ __forceinline__ void lds_write_h(_Float16 *dstrow, const uint32_t *v) {
     u32x4 *p = reinterpret_cast<u32x4 *>(dstrow);
-    p[0] = u32x4{v[0], v[1], v[2], v[3]};
-    p[1] = u32x4{v[4], v[5], v[6], v[7]};
-    p[2] = u32x4{v[8], v[9], v[10], v[11]};
-    p[3] = u32x4{v[12], v[13], v[14], v[15]};
+#pragma unroll
+    for (int i = 0; i < NH / 8; i++) p[i] = u32x4{v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]};
 }
 
 // NJ = 32-column MFMA tiles per wave: block tile 128 x (64 * NJ).  NJ = 1 halves the accumulators so that two
@@ -280,7 +289,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
         rows = m0 + mc.count[blockIdx.x];
         w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
     }
-    const bool bstage = 2 * BN >= 256 ? true : tid < 2 * BN;    // threads that also stage a weight row (wave-uniform)
+    // every thread stages NW = 64 / TPR weights of one row per stage (16 when the tile has 64 weight rows, else 32), so
+    // that all waves carry the same conversion work and the loop body has no wave-dependent branch
+    constexpr int TPR = 256 / BN, NW = 64 / TPR;
+    static_assert(TPR == 2 || TPR == 4, "weight rows of the block tile");
     const bool astage = SM ? tid < 2 * BMT : true;               // threads that stage an activation row (wave-uniform)
     // split-K: blockIdx.z takes an equal share of the 256-element spans and writes its own partial plane
     const int nsb_all = k >> 8;
@@ -288,9 +300,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     dst += (int64_t)blockIdx.z * split_stride;
     const int64_t row_bytes = (int64_t)(k / BlockInfo<DT>::elems) * BlockInfo<DT>::bytes;
 
-    // staging role of this thread: (row r_l of the tile, 32-element half)
+    // staging roles of this thread: activations (row r_l of the tile, 32-element half), weights (row r_w, part of NW)
     const int r_l = tid >> 1, half = tid & 1;
-    const int wrow = min(n0 + (bstage ? r_l : 0), n - 1);
+    const int r_w = tid / TPR, part = tid % TPR;
+    const int wrow = min(n0 + r_w, n - 1);
     const int arow = min(m0 + (astage ? r_l : 0), rows - 1);
     const bool arow_ok = astage && m0 + r_l < rows;
     const uint32_t amask = arow_ok ? 0xffffffffu : 0u;
@@ -309,12 +322,13 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     // conversion + MFMA work is shorter than a trip to memory.  Stage (kb, g) covers k = 256 kb + 64 g + [0, 64).
     // Positions past the end of this split's range are clamped to its last super-block: what they load and convert
     // lands in LDS copies nobody reads.
-    typename S::Raw wraw2[2];
+    typedef typename S::template Raw<NW> WRaw;
+    WRaw wraw2[2];
     u32x4 a02[2], a12[2], abs0 = u32x4{0, 0, 0, 0};
     float ad8[2] = {0.0f, 0.0f};
-    auto load_stage = [&](int kb, int g, typename S::Raw &wr, u32x4 &x0, u32x4 &x1, float &d8) {
+    auto load_stage = [&](int kb, int g, WRaw &wr, u32x4 &x0, u32x4 &x1, float &d8) {
         kb = min(kb, nsb - 1);
-        if (bstage) S::load(wr, wrow_p, kb, g, half);
+        S::template load<NW>(wr, wrow_p, kb, g, part);
         if (astage) {
             const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
             x0 = *reinterpret_cast<const u32x4 *>(q);
@@ -328,31 +342,28 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     };
     // what one thread contributes to the LDS image of a stage
     struct Conv {
-        uint32_t w[16], w2[S::TERMS == 2 ? 16 : 1], a[16];
+        uint32_t w[NW / 2], w2[S::TERMS == 2 ? NW / 2 : 1], a[16];
         float d, dmin, d8;
-        uint32_t mv[4], bv[4];
+        uint32_t mv[8 / TPR], bv[4];
     };
-    auto convert_stage = [&](int g, const typename S::Raw &wraw, const u32x4 &a0, const u32x4 &a1, float d8, Conv &c) {
-        if (bstage) {
-            if constexpr (S::TERMS == 2) S::convert2(wraw, g, half, c.w, c.w2);
-            else S::convert(wraw, g, half, c.w);
-        }
+    auto convert_stage = [&](int g, const WRaw &wraw, const u32x4 &a0, const u32x4 &a1, float d8, Conv &c) {
+        if constexpr (S::TERMS == 2) S::template convert2<NW>(wraw, g, part, c.w, c.w2);
+        else S::template convert<NW>(wraw, g, part, c.w);
         if (astage) {
             act_convert(a0, a1, !KQ, KQ ? 0u : h2_splat(d8), c.a);
 #pragma unroll
             for (int i = 0; i < 16; i++) c.a[i] &= amask;        // rows past the end contribute zeros (no branch)
         }
         if (KQ && g == 0) {
-            int mins[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            c.d = 0.0f; c.dmin = 0.0f;
-            if (bstage) S::header(wraw, c.d, c.dmin, mins);
+            S::template header<NW>(wraw, c.d, c.dmin);
             c.d8 = arow_ok ? d8 : 0.0f;
             if (S::HAS_MIN) {
-                // Bm[n][j] = min[j/2] for j in 8*half .. 8*half+7 ; Am[m][j] = bsums16[j]
+                // Bm[n][2 j], Bm[n][2 j + 1] = min of sub-block j, this thread's share j = (8 / TPR) part + i; Am[m][j] = bsums16[j]
+                const uint32_t mine = S::template mins4<NW>(wraw, (8 / TPR) * part >= 4);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    uint32_t hm = f2h_bits((float)mins[4 * half + i]);
-                    c.mv[i] = hm | (hm << 16);
+                for (int i = 0; i < 8 / TPR; i++) {
+                    const uint32_t mb = (mine >> (8 * (((8 / TPR) * part + i) & 3))) & 0xffu;
+                    c.mv[i] = pk_add((0x6400u | mb) * 0x00010001u, 0xe400e400u);    // (1024 + min) - 1024 in both halves
                 }
                 const uint32_t b4[4] = {abs0.x, abs0.y, abs0.z, abs0.w};
 #pragma unroll
@@ -365,17 +376,18 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t
     };
     // buf: LDS copy of the stage (its parity); hb: copy of the per-super-block arrays (parity of the super-block)
     auto store_stage = [&](int g, int buf, int hb, const Conv &c) {
-        if (bstage) {
-            if constexpr (S::TERMS == 2) lds_write32h(Bs2[buf] + r_l * LDK + 32 * half, c.w2);
-            lds_write32h(Bs[buf] + r_l * LDK + 32 * half, c.w);
-        }
-        if (astage) lds_write32h(As[buf] + r_l * LDK + 32 * half, c.a);
+        if constexpr (S::TERMS == 2) lds_write_h<NW>(Bs2[buf] + r_w * LDK + NW * part, c.w2);
+        lds_write_h<NW>(Bs[buf] + r_w * LDK + NW * part, c.w);
+        if (astage) lds_write_h<32>(As[buf] + r_l * LDK + 32 * half, c.a);
         if (KQ && g == 0) {
-            // both threads of a row hold the same values: both write them (no branch)
-            if (bstage) { sD[hb][r_l] = c.d; sDmin[hb][r_l] = c.dmin; }
+            // the threads of a row hold the same values: all of them write (no branch)
+            sD[hb][r_w] = c.d; sDmin[hb][r_w] = c.dmin;
             if (astage) sD8[hb][r_l] = c.d8;
             if (S::HAS_MIN) {
-                if (bstage) *reinterpret_cast<u32x4 *>(Bm[hb] + r_l * 24 + 8 * half) = u32x4{c.mv[0], c.mv[1], c.mv[2], c.mv[3]};
+                if constexpr (TPR == 2)
+                    *reinterpret_cast<u32x4 *>(Bm[hb] + r_w * 24 + 8 * part) = u32x4{c.mv[0], c.mv[1], c.mv[2], c.mv[3]};
+                else
+                    *reinterpret_cast<uint2 *>(Bm[hb] + r_w * 24 + 4 * part) = uint2{c.mv[0], c.mv[1]};
                 if (astage) *reinterpret_cast<u32x4 *>(Am[hb] + r_l * 24 + 8 * half) = u32x4{c.bv[0], c.bv[1], c.bv[2], c.bv[3]};
             }
         }
