@@ -445,121 +445,139 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const float *__restrict_
 }
 
 // The prompt's attention on the f32 matrix cores (head_dim 128): a workgroup takes the 32 (row, head) pairs of 32 / G
-// consecutive query rows and one split of 128 keys.  Scores: wave w forms the 32 x 32 tile of its 32 keys with 64
-// v_mfma_f32_32x32x2f32 steps over the head dimension (A = q, B = k, one float4 per lane and eight dims); the tiles meet in
-// LDS (key-major, row stride 33 floats so that neither the tile's column-wise writes nor the row-wise reads collide),
-// the softmax over the split runs as in attn_kernel, and wave w forms output columns [32 w, 32 w + 32) with 64 steps over
-// the keys (A = p from LDS, B = v).  f32 throughout: the products and sums are those of attn_kernel in another order.
+// consecutive query rows and walks over the keys in splits of 128, keeping a running maximum, sum and output per pair
+// (no partial results in memory, no combine pass).  Per split: wave w forms the 32 x 32 score tile of its 32 keys with 64
+// v_mfma_f32_32x32x2f32 steps over the head dimension (A = q, B = k, one float4 per lane and eight dims); the tiles meet
+// in LDS (key-major, row stride 33 floats so that neither the tile's column-wise writes nor the row-wise reads collide),
+// the softmax over the split runs as in attn_kernel, wave w forms output columns [32 w, 32 w + 32) of the split with 64
+// steps over the keys (A = p from LDS, B = v), and the split is merged into the running state:
+//   M' = max(M, m), out = out e^{M - M'} + out_split e^{m - M'}, L likewise.   f32 throughout.
 typedef float mf32x16 __attribute__((ext_vector_type(16)));
 constexpr int ATT_SCP = 33;                       // floats per key in the score tile
 
 template <int G>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(const float *__restrict__ q, int64_t q_stride, const float *__restrict__ k_cache,
-                                                        const float *__restrict__ v_cache, float *__restrict__ out, float *__restrict__ part,
+                                                        const float *__restrict__ v_cache, float *__restrict__ out,
                                                         const int32_t *__restrict__ pos_dev, int pos0, int rows, int n_head, int ctx,
-                                                        float scale, int splits) {
+                                                        float scale) {
     constexpr int HD = 128, VH = 32, R = VH / G;     // pair vh = rr * G + g
     static_assert(ATT_SPLIT == 128, "one 32-key tile per wave");
     __shared__ float sc[ATT_SPLIT * ATT_SCP];
-    __shared__ float ml[2 * VH];
-    const int kvh = blockIdx.x, r0 = blockIdx.y * R, sp = blockIdx.z;
+    __shared__ float ml[2 * VH];                      // (m, l) of the current split
+    __shared__ float run[2 * VH];                     // running (M, L)
+    __shared__ float fac[2 * VH];                     // e^{M - M'}, e^{m - M'}
+    const int kvh = blockIdx.x, r0 = blockIdx.y * R;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int x = lane & 31, kk = lane >> 5;          // operand row / column of this lane, and which of a step's two k
     const int nr = min(R, rows - r0);                 // valid rows of this workgroup (>= 1)
     const int base_len = pos0 + (pos_dev ? pos_dev[0] : 0) + r0 + 1;
-    const int j0 = sp * ATT_SPLIT;
-    const int cnt_max = min(min(base_len + nr - 1, ctx) - j0, ATT_SPLIT);   // keys of the last valid row
-    if (cnt_max <= 0 && splits > 1) {
-        if (tid < VH && tid / G < nr) {
-            float *pp = part + (((int64_t)(r0 + tid / G) * n_head + kvh * G + tid % G) * splits + sp) * (HD + 2);
-            pp[0] = -INFINITY;
-            pp[1] = 0.0f;
-        }
-        return;
-    }
+    const int len_last = min(base_len + nr - 1, ctx);                       // keys of the last valid row (>= 1)
+    const int n_sp = (len_last + ATT_SPLIT - 1) / ATT_SPLIT;
     const float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
-    const int last = max(cnt_max - 1, 0);             // loads of masked keys are redirected to a valid row
+    if (tid < VH) { run[2 * tid] = -INFINITY; run[2 * tid + 1] = 0.0f; }
 
-    // ---- scores of keys [32 wv, 32 wv + 32): dims 8 c + 4 kk + i go to step 4 c + i ----
+    // q of pair x: dims 8 c + 4 kk + i go to MFMA step 4 c + i
+    f32x4 qd[HD / 8];
     {
-        f32x4 kd[HD / 8], qd[HD / 8];
-        const float *kr = kb + (int64_t)(j0 + min(32 * wv + x, last)) * HD + 4 * kk;
-#pragma unroll
-        for (int c = 0; c < HD / 8; c++) kd[c] = *reinterpret_cast<const f32x4 *>(kr + 8 * c);
         const float *qr = q + (int64_t)(r0 + min(x / G, nr - 1)) * q_stride + (int64_t)(kvh * G + x % G) * HD + 4 * kk;
 #pragma unroll
         for (int c = 0; c < HD / 8; c++) qd[c] = *reinterpret_cast<const f32x4 *>(qr + 8 * c);
-        mf32x16 s;
-#pragma unroll
-        for (int e = 0; e < 16; e++) s[e] = 0.0f;
-#pragma unroll
-        for (int c = 0; c < HD / 8; c++) {
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].x, kd[c].x, s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].y, kd[c].y, s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].z, kd[c].z, s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].w, kd[c].w, s, 0, 0, 0);
-        }
-        // tile layout: column (key) = x, row (pair) = 8 (e / 4) + 4 kk + e % 4
-        const int key = 32 * wv + x;
-#pragma unroll
-        for (int e = 0; e < 16; e++) {
-            const int vh = 8 * (e >> 2) + 4 * kk + (e & 3);
-            const int cnt = min(min(base_len + vh / G, ctx) - j0, ATT_SPLIT);
-            sc[key * ATT_SCP + vh] = key < cnt ? s[e] * scale : -INFINITY;
-        }
     }
-    __syncthreads();
-
-    // ---- softmax over the split: wave w reduces pairs vh = w, w + 4, ... ----
-    for (int vh = wv; vh < VH; vh += 4) {
-        float s[ATT_SPLIT / 64], m = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < ATT_SPLIT / 64; i++) {
-            s[i] = sc[(lane + 64 * i) * ATT_SCP + vh];
-            m = fmaxf(m, s[i]);
-        }
-        m = wave_max(m);
-        float l = 0.0f;
-#pragma unroll
-        for (int i = 0; i < ATT_SPLIT / 64; i++) {
-            const float p = s[i] > -INFINITY ? __expf(s[i] - m) : 0.0f;
-            sc[(lane + 64 * i) * ATT_SCP + vh] = p;
-            l += p;
-        }
-        l = wave_sum(l);
-        if (lane == 0) { ml[2 * vh] = m; ml[2 * vh + 1] = l; }
-    }
-    __syncthreads();
-
-    // ---- output columns [32 wv, 32 wv + 32): step t takes keys 2 t + kk (masked keys hold p = 0) ----
     mf32x16 o;
 #pragma unroll
     for (int e = 0; e < 16; e++) o[e] = 0.0f;
-    const int nsteps = (cnt_max + 1) >> 1;                       // uniform over the workgroup
-    for (int t0 = 0; t0 < nsteps; t0 += 16) {
-        float vv[16], pv[16];
+
+    for (int sp = 0; sp < n_sp; sp++) {
+        const int j0 = sp * ATT_SPLIT;
+        const int cnt_max = min(len_last - j0, ATT_SPLIT);                  // >= 1
+        const int last = cnt_max - 1;                 // loads of masked keys are redirected to a valid row
+        // ---- scores of keys [32 wv, 32 wv + 32) ----
+        {
+            f32x4 kd[HD / 8];
+            const float *kr = kb + (int64_t)(j0 + min(32 * wv + x, last)) * HD + 4 * kk;
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
-            const int key = 2 * (t0 + u) + kk;                     // < ATT_SPLIT + 30: clamped for the loads, p = 0 beyond cnt
-            vv[u] = vb[(int64_t)(j0 + min(key, last)) * HD + 32 * wv + x];
-            pv[u] = key < ATT_SPLIT ? sc[min(key, ATT_SPLIT - 1) * ATT_SCP + x] : 0.0f;
+            for (int c = 0; c < HD / 8; c++) kd[c] = *reinterpret_cast<const f32x4 *>(kr + 8 * c);
+            mf32x16 s;
+#pragma unroll
+            for (int e = 0; e < 16; e++) s[e] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < HD / 8; c++) {
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].x, kd[c].x, s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].y, kd[c].y, s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].z, kd[c].z, s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(qd[c].w, kd[c].w, s, 0, 0, 0);
+            }
+            // tile layout: column (key) = x, row (pair) = 8 (e / 4) + 4 kk + e % 4
+            const int key = 32 * wv + x;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int vh = 8 * (e >> 2) + 4 * kk + (e & 3);
+                const int cnt = min(base_len + vh / G, ctx) - j0;            // keys of this pair's row in the split (may be <= 0)
+                sc[key * ATT_SCP + vh] = key < cnt ? s[e] * scale : -INFINITY;
+            }
         }
+        __syncthreads();
+
+        // ---- softmax over the split: wave w reduces pairs vh = w, w + 4, ... ----
+        for (int vh = wv; vh < VH; vh += 4) {
+            float s[ATT_SPLIT / 64], m = -INFINITY;
 #pragma unroll
-        for (int u = 0; u < 16; u++) o = __builtin_amdgcn_mfma_f32_32x32x2f32(pv[u], vv[u], o, 0, 0, 0);
+            for (int i = 0; i < ATT_SPLIT / 64; i++) {
+                s[i] = sc[(lane + 64 * i) * ATT_SCP + vh];
+                m = fmaxf(m, s[i]);
+            }
+            m = wave_max(m);
+            float l = 0.0f;
+#pragma unroll
+            for (int i = 0; i < ATT_SPLIT / 64; i++) {
+                const float p = s[i] > -INFINITY ? __expf(s[i] - m) : 0.0f;
+                sc[(lane + 64 * i) * ATT_SCP + vh] = p;
+                l += p;
+            }
+            l = wave_sum(l);
+            if (lane == 0) { ml[2 * vh] = m; ml[2 * vh + 1] = l; }
+        }
+        __syncthreads();
+        if (tid < VH) {
+            const float m = ml[2 * tid], l = ml[2 * tid + 1], M = run[2 * tid], L = run[2 * tid + 1];
+            const float Mn = fmaxf(M, m);
+            const float fa = L > 0.0f ? __expf(M - Mn) : 0.0f, fb = l > 0.0f ? __expf(m - Mn) : 0.0f;
+            run[2 * tid] = Mn;
+            run[2 * tid + 1] = L * fa + l * fb;
+            fac[2 * tid] = fa;
+            fac[2 * tid + 1] = fb;
+        }
+
+        // ---- output columns [32 wv, 32 wv + 32) of the split: step t takes keys 2 t + kk (masked keys hold p = 0) ----
+        mf32x16 os;
+#pragma unroll
+        for (int e = 0; e < 16; e++) os[e] = 0.0f;
+        const int nsteps = (cnt_max + 1) >> 1;                       // uniform over the workgroup
+        for (int t0 = 0; t0 < nsteps; t0 += 16) {
+            float vv[16], pv[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                const int key = 2 * (t0 + u) + kk;                     // < ATT_SPLIT; clamped for the loads, p = 0 beyond cnt
+                vv[u] = vb[(int64_t)(j0 + min(key, last)) * HD + 32 * wv + x];
+                pv[u] = sc[key * ATT_SCP + x];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; u++) os = __builtin_amdgcn_mfma_f32_32x32x2f32(pv[u], vv[u], os, 0, 0, 0);
+        }
+        __syncthreads();                              // fac is written, and every wave is done with sc
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int vh = 8 * (e >> 2) + 4 * kk + (e & 3);
+            o[e] = o[e] * fac[2 * vh] + os[e] * fac[2 * vh + 1];
+        }
     }
+    __syncthreads();
 #pragma unroll
     for (int e = 0; e < 16; e++) {
         const int vh = 8 * (e >> 2) + 4 * kk + (e & 3);
         const int rr = vh / G, g = vh - rr * G;
         if (rr >= nr) continue;
-        const int head = kvh * G + g, d = 32 * wv + x;
-        if (splits == 1) {
-            out[((int64_t)(r0 + rr) * n_head + head) * HD + d] = o[e] / ml[2 * vh + 1];
-        } else {
-            float *pp = part + (((int64_t)(r0 + rr) * n_head + head) * splits + sp) * (HD + 2);
-            pp[2 + d] = o[e];
-            if (d == 0) { pp[0] = ml[2 * vh]; pp[1] = ml[2 * vh + 1]; }
-        }
+        out[((int64_t)(r0 + rr) * n_head + kvh * G + g) * HD + 32 * wv + x] = o[e] / run[2 * vh + 1];
     }
 }
 
@@ -1038,11 +1056,11 @@ int launch_attn(int G, dim3 grid, hipStream_t s, const float *q, int64_t q_strid
 }
 
 int launch_attn_mfma(int G, dim3 grid, hipStream_t s, const float *q, int64_t q_stride, const float *kc, const float *vc, float *out,
-                     float *part, const int32_t *pos_dev, int pos0, int rows, int n_head, int ctx, float scale, int splits) {
-#define CQ_ATT(GG)                                                                                                               \
-    case GG:                                                                                                                     \
-        hipLaunchKernelGGL((attn_mfma_kernel<GG>), grid, dim3(256), 0, s, q, q_stride, kc, vc, out, part, pos_dev, pos0, rows,   \
-                           n_head, ctx, scale, splits);                                                                         \
+                     const int32_t *pos_dev, int pos0, int rows, int n_head, int ctx, float scale) {
+#define CQ_ATT(GG)                                                                                                                \
+    case GG:                                                                                                                      \
+        hipLaunchKernelGGL((attn_mfma_kernel<GG>), grid, dim3(256), 0, s, q, q_stride, kc, vc, out, pos_dev, pos0, rows, n_head,  \
+                           ctx, scale);                                                                                           \
         break;
     switch (G) {
         CQ_ATT(1) CQ_ATT(2) CQ_ATT(4) CQ_ATT(8)
@@ -1146,11 +1164,10 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
     hipStream_t s = (hipStream_t)stream;
     int rc;
     if (rows >= CQ_ATTN_MFMA_MIN && head_dim == 128 && (G == 1 || G == 2 || G == 4 || G == 8)) {
-        // prompts: 32 (row, head) pairs per workgroup on the f32 matrix cores
+        // prompts: 32 (row, head) pairs per workgroup on the f32 matrix cores, all splits in one pass (nothing to combine)
         const int R = 32 / G;
-        grid.y = (unsigned)((rows + R - 1) / R);
-        rc = launch_attn_mfma(G, grid, s, q_dev, q_stride, k_cache_dev, v_cache_dev, out_dev, (float *)workspace_dev, pos_dev, (int)pos,
-                              (int)rows, (int)n_head, (int)ctx, scale, (int)splits);
+        return launch_attn_mfma(G, dim3((unsigned)n_kv_head, (unsigned)((rows + R - 1) / R)), s, q_dev, q_stride, k_cache_dev, v_cache_dev,
+                                out_dev, pos_dev, (int)pos, (int)rows, (int)n_head, (int)ctx, scale);
     } else if (rows >= CQ_ATTN_ROWS_MIN && (G == 1 || G == 2 || G == 4 || G == 8)) {
         // prompts and wide batches: several query rows share each load of the keys and values
         const int R = attn_rows_per_group(G);
