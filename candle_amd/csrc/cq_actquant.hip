@@ -43,6 +43,38 @@ __global__ __launch_bounds__(256) void quantize_q80_gather_kernel(const float *_
     cq_quantize_q80_vals(v, true, span * 256 + lane * 4, lane, qs, ds);
 }
 
+// silu(gate) * up computed on the fly (the expression of silu_mul_kernel) and quantized: the f32 product never exists in
+// memory.  Row r of the product is gate[r * gate_stride + i] , up[r * up_stride + i], i < 256 kb.
+__device__ __forceinline__ void load_swiglu4(const float *gate, const float *up, int64_t gi, int64_t ui, float v[4]) {
+    const f32x4 g = *reinterpret_cast<const f32x4 *>(gate + gi), u = *reinterpret_cast<const f32x4 *>(up + ui);
+    v[0] = g.x / (1.0f + expf(-g.x)) * u.x;
+    v[1] = g.y / (1.0f + expf(-g.y)) * u.y;
+    v[2] = g.z / (1.0f + expf(-g.z)) * u.z;
+    v[3] = g.w / (1.0f + expf(-g.w)) * u.w;
+}
+__global__ __launch_bounds__(256) void quantize_q8k_swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up, int64_t gate_stride,
+                                                                  int64_t up_stride, int kb, int8_t *__restrict__ qs, float *__restrict__ dout,
+                                                                  int16_t *__restrict__ bsums, int64_t n_blocks) {
+    const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= n_blocks) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = blk / kb, off = (blk - row * kb) * 256 + lane * 4;
+    float v[4];
+    load_swiglu4(gate, up, row * gate_stride + off, row * up_stride + off, v);
+    cq_quantize_q8k_vals(v, blk, lane, qs, dout, bsums);
+}
+__global__ __launch_bounds__(256) void quantize_q80_swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up, int64_t gate_stride,
+                                                                  int64_t up_stride, int kb, int8_t *__restrict__ qs, float *__restrict__ ds,
+                                                                  int64_t n_spans) {
+    const int64_t span = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (span >= n_spans) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = span / kb, off = (span - row * kb) * 256 + lane * 4;
+    float v[4];
+    load_swiglu4(gate, up, row * gate_stride + off, row * up_stride + off, v);
+    cq_quantize_q80_vals(v, true, span * 256 + lane * 4, lane, qs, ds);
+}
+
 template <int XDT>
 int launch_quantize_act(int w_dtype, const void *x, void *scratch, int64_t k, int64_t rows, hipStream_t s) {
     ActLayout L = cq_act_layout(w_dtype, k, rows);
@@ -90,5 +122,24 @@ int cq_quantize_act_gather_launch(int w_dtype, const float *x, const int *row_ma
     else
         hipLaunchKernelGGL(quantize_q80_gather_kernel, dim3((unsigned)grid), dim3(256), 0, s, x, row_map, (int)(k / 256), (int8_t *)(b + L.qs_off),
                            (float *)(b + L.d_off), spans);
+    return (int)hipGetLastError();
+}
+
+// Scratch rows [0, rows) = quantized silu(gate[r]) * up[r].  k is a multiple of 256; strides in floats, multiples of 4.
+int cq_quantize_act_swiglu_launch(int w_dtype, const float *gate, const float *up, int64_t gate_stride, int64_t up_stride, void *scratch, int64_t k,
+                                  int64_t rows, hipStream_t s) {
+    if (k % 256) return CQ_ERR_SHAPE;
+    if (rows == 0) return CQ_OK;
+    ActLayout L = cq_act_layout(w_dtype, k, rows);
+    uint8_t *b = (uint8_t *)scratch;
+    const int64_t spans = rows * (k / 256);
+    const int64_t grid = (spans + 3) / 4;
+    if (grid > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (cq_is_kquant(w_dtype))
+        hipLaunchKernelGGL(quantize_q8k_swiglu_kernel, dim3((unsigned)grid), dim3(256), 0, s, gate, up, gate_stride, up_stride, (int)(k / 256),
+                           (int8_t *)(b + L.qs_off), (float *)(b + L.d_off), (int16_t *)(b + L.bs_off), spans);
+    else
+        hipLaunchKernelGGL(quantize_q80_swiglu_kernel, dim3((unsigned)grid), dim3(256), 0, s, gate, up, gate_stride, up_stride, (int)(k / 256),
+                           (int8_t *)(b + L.qs_off), (float *)(b + L.d_off), spans);
     return (int)hipGetLastError();
 }

@@ -193,6 +193,25 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     return cq_convert_f32_launch(tmp, dst_dev, dst_dtype, m * n, s);
 }
 
+int cq_nn_qmatmul_swiglu_rows(int w_dtype, const void *w_dev, const float *gate_dev, const float *up_dev, int64_t gate_stride, int64_t up_stride,
+                              float *dst_dev, int64_t m, int64_t k, int64_t n, void *workspace_dev, int64_t workspace_bytes, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, m);
+    if (rc) return rc;
+    if (k % 256) return CQ_ERR_RANGE;
+    if (gate_stride < k || up_stride < k || gate_stride % 4 || up_stride % 4) return CQ_ERR_SHAPE;
+    if (m == 0 || n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_dev))) return rc;
+    if (!gate_dev || !up_dev || !dst_dev || !workspace_dev) return CQ_ERR_NULL;
+    if (!aligned(gate_dev, 16) || !aligned(up_dev, 16) || !aligned(workspace_dev, 256) || !aligned(dst_dev, 4)) return CQ_ERR_ALIGN;
+    if (workspace_bytes < cq_qmatmul_workspace_bytes(w_dtype, m, k, n)) return CQ_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    if ((rc = cq_quantize_act_swiglu_launch(w_dtype, gate_dev, up_dev, gate_stride, up_stride, workspace_dev, k, m, s))) return rc;
+    if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, CQ_F32, k, n, m, n, s);
+    float *tmp = (float *)((uint8_t *)workspace_dev + cq_act_layout(w_dtype, k, m).total);
+    float *split_ws = cq_qmm_splits(k, n, m) > 1 ? (float *)((uint8_t *)tmp + cq_align256(m * n * 4)) : nullptr;
+    return cq_matmul_launch(w_dtype, w_dev, workspace_dev, dst_dev, k, n, m, n, s, split_ws);
+}
+
 int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk,
                                        int64_t input_dim1) {
     if (check_mm_shape(w_dtype, k, n, batch) || num_experts <= 0 || topk <= 0) return -1;

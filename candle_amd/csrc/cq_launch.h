@@ -6,6 +6,8 @@
 int cq_dequantize_launch(int dtype, const void *blocks, void *out, int64_t elems, int out_dtype, hipStream_t s);
 int cq_quantize_launch(int dtype, const float *x, void *blocks, int64_t elems, hipStream_t s);
 int cq_quantize_act_launch(int w_dtype, const void *x, int x_dtype, void *scratch, int64_t k, int64_t rows, hipStream_t s);
+int cq_quantize_act_swiglu_launch(int w_dtype, const float *gate, const float *up, int64_t gate_stride, int64_t up_stride, void *scratch, int64_t k,
+                                  int64_t rows, hipStream_t s);
 int cq_matvec_launch(int w_dtype, const void *w, const void *scratch, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s);
 // same, over an already resolved (possibly row-offset) view of the activation scratch

@@ -293,8 +293,14 @@ class ModelWeights:
                 self._mm(w1, cfg.ffn, xn, gu.data_ptr(), rows, sp)
                 self._mm(w3, cfg.ffn, xn, gu.data_ptr() + 4 * rows * cfg.ffn, rows, sp)
                 g_ptr, u_ptr, gs = gu.data_ptr(), gu.data_ptr() + 4 * rows * cfg.ffn, cfg.ffn
-            ck("cq_nn_silu_mul", L.cq_nn_silu_mul(g_ptr, u_ptr, h.data_ptr(), rows, cfg.ffn, gs, gs, sp))
-            self._mm(w["feed_forward_w2"], cfg.hidden, h, delta.data_ptr(), rows, sp)
+            w2 = w["feed_forward_w2"]
+            if rows > 2 and cfg.ffn % 256 == 0:
+                # silu(w1 x) * w3 x goes straight into the activation quantizer of w2
+                ck("cq_nn_qmatmul_swiglu_rows", L.cq_nn_qmatmul_swiglu_rows(int(w2.dtype), w2.ptr, g_ptr, u_ptr, gs, gs, delta.data_ptr(), rows,
+                                                                            w2.k, cfg.hidden, self.ws.data_ptr(), self.ws.numel(), sp))
+            else:
+                ck("cq_nn_silu_mul", L.cq_nn_silu_mul(g_ptr, u_ptr, h.data_ptr(), rows, cfg.ffn, gs, gs, sp))
+                self._mm(w2, cfg.hidden, h, delta.data_ptr(), rows, sp)
         # last token only: x += mlp; final norm; output head                              :593-596
         last = 4 * (rows - 1) * cfg.hidden
         ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr() + last, delta.data_ptr() + last, self.norm.data_ptr(), None, xn.data_ptr(), 1,

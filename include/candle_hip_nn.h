@@ -81,6 +81,14 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
 int cq_nn_silu_mul(const float *gate_dev, const float *up_dev, float *out_dev, int64_t rows, int64_t dim, int64_t gate_stride, int64_t up_stride,
                    void *stream);
 
+/* dst [m, n] = QMatMul::forward(silu(gate) * up) for m rows: Mlp::forward's feed_forward_w2 (quantized_llama.rs:56-63) with
+ * the activation folded into the activation quantizer, so the f32 product [m, k] is never written.  Results are those of
+ * cq_nn_silu_mul followed by cq_qmatmul_forward (same arithmetic; for m <= 2 that pair quantizes inside the matvec kernel
+ * instead).  k % 256 == 0 (else CQ_ERR_RANGE: use the two calls); gate/up rows may be strided views of one buffer
+ * (strides in floats, multiples of 4); workspace as cq_qmatmul_workspace_bytes(w_dtype, m, k, n). */
+int cq_nn_qmatmul_swiglu_rows(int w_dtype, const void *w_dev, const float *gate_dev, const float *up_dev, int64_t gate_stride, int64_t up_stride,
+                              float *dst_dev, int64_t m, int64_t k, int64_t n, void *workspace_dev, int64_t workspace_bytes, void *stream);
+
 /* Single-row (decode) fusions of the glue into the quantized matvec kernel.  No counterpart in the reference,
  * which runs these as separate tensor ops; results equal the unfused sequence up to f32 summation order.
  *

@@ -239,6 +239,38 @@ def test_silu_mul_strided_views():
     assert rel_l2(out.cpu().numpy(), want) <= TOL
 
 
+@pytest.mark.parametrize("dtype", [12, 14, 13, 2, 8])
+@pytest.mark.parametrize("m,k,n", [(3, 512, 96), (8, 1024, 200), (40, 2048, 130), (130, 768, 64)])
+def test_silu_mul_folded_into_the_quantizer_of_a_matmul(dtype, m, k, n):
+    """feed_forward_w2 over several rows: equal to cq_nn_silu_mul + cq_qmatmul_forward (same arithmetic, bit for bit), and to
+    the CPU sequence within what the device's expf may move through the quantizer."""
+    import oracle
+    lib = L()
+    gu = normal(70, (m, 2 * k), 1.5)
+    w = oracle.from_float(dtype, normal(71, (n, k), 0.03).reshape(-1))
+    g, wd = dev(gu), dev(w)
+    wsb = lib.cq_qmatmul_workspace_bytes(dtype, m, k, n)
+    ws = torch.empty(max(wsb, 256), dtype=torch.uint8, device="cuda")
+    fused = torch.empty((m, n), device="cuda")
+    ok(lib.cq_nn_qmatmul_swiglu_rows(dtype, wd.data_ptr(), g.data_ptr(), g.data_ptr() + 4 * k, 2 * k, 2 * k, fused.data_ptr(), m, k, n,
+                                     ws.data_ptr(), wsb, None))
+    h = torch.empty((m, k), device="cuda")
+    two = torch.empty((m, n), device="cuda")
+    ok(lib.cq_nn_silu_mul(g.data_ptr(), g.data_ptr() + 4 * k, h.data_ptr(), m, k, 2 * k, 2 * k, None))
+    ok(lib.cq_qmatmul_forward(dtype, wd.data_ptr(), h.data_ptr(), 0, two.data_ptr(), 0, m, k, n, ws.data_ptr(), wsb, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(fused.cpu().numpy(), two.cpu().numpy())
+    hh = (lo.silu(gu[:, :k]) * gu[:, k:]).astype(np.float32)
+    assert rel_l2(fused.cpu().numpy(), oracle.matmul_fast(dtype, hh, w, n, 8)) <= (1e-3 if dtype in (2, 8) and m > 8 else 1e-4)
+
+
+def test_silu_mul_folded_argument_errors():
+    lib = L()
+    assert lib.cq_nn_qmatmul_swiglu_rows(8, 256, 256, 256, 96, 96, 256, 4, 96, 64, 256, 1 << 20, None) == -6      # k % 256
+    assert lib.cq_nn_qmatmul_swiglu_rows(12, 256, 256, 256, 256, 510, 256, 4, 512, 64, 256, 1 << 20, None) == -2  # stride < k
+    assert lib.cq_nn_qmatmul_swiglu_rows(12, 256, 256, 256, 512, 512, 256, 4, 512, 64, 256, 16, None) == -5       # workspace
+
+
 def test_argmax_first_of_ties_and_bookkeeping():
     n = 128256
     logits = normal(15, (n,), 1.0)
