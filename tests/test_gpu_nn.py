@@ -115,7 +115,7 @@ def attention_oracle(q, kc, vc, pos, H, KV, D):
     return out
 
 
-@pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (4, 4, 128), (8, 2, 128)])
+@pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (4, 4, 128), (8, 2, 128), (4, 2, 128)])
 @pytest.mark.parametrize("rows,pos,ctx", [(1, 0, 32), (1, 199, 256), (1, 600, 1024), (7, 250, 512), (3, 0, 16),
                                           (16, 0, 64), (37, 100, 512), (130, 0, 256), (21, 250, 300), (70, 100, 512), (64, 0, 64), (66, 900, 1024)])
 def test_attention(H, KV, D, rows, pos, ctx):
