@@ -277,6 +277,31 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
     return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
 }
 
+int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, const void *w_b_dev, const int32_t *sorted_token_ids_dev,
+                          const int32_t *expert_ids_dev, float *out_a_dev, float *out_b_dev, int64_t num_experts, int64_t topk, int64_t size_m,
+                          int64_t n, int64_t k, int is_prefill, void *workspace_dev, int64_t workspace_bytes, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, size_m);
+    if (rc) return rc;
+    if (num_experts <= 0 || topk <= 0 || size_m % topk != 0) return CQ_ERR_SHAPE;
+    if (num_experts > (1 << 20)) return CQ_ERR_RANGE;
+    if (size_m == 0 || n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_a_dev)) || (rc = check_weight_ptr(w_dtype, w_b_dev))) return rc;
+    if (!x_dev || !sorted_token_ids_dev || !expert_ids_dev || !out_a_dev || !out_b_dev || !workspace_dev) return CQ_ERR_NULL;
+    if (!aligned(x_dev, 16) || !aligned(sorted_token_ids_dev, 4) || !aligned(expert_ids_dev, 4) || !aligned(out_a_dev, 4) ||
+        !aligned(out_b_dev, 4) || !aligned(workspace_dev, 256))
+        return CQ_ERR_ALIGN;
+    if (workspace_bytes < cq_moe_gemm_workspace_bytes(w_dtype, num_experts, topk, size_m, n, k, 0)) return CQ_ERR_WORKSPACE;
+    MoeArgs a;
+    a.w_dtype = w_dtype; a.w = w_a_dev; a.x = x_dev; a.out = out_a_dev;
+    a.w_b = w_b_dev; a.out_b = out_b_dev;
+    a.num_experts = num_experts; a.n = n; a.k = k;
+    a.n_pairs = size_m; a.x_rows = size_m / topk;
+    a.mode = MOE_SORTED; a.ids_u32 = nullptr; a.topk = topk; a.input_dim1 = 0;
+    a.sorted_token_ids = sorted_token_ids_dev; a.expert_ids = expert_ids_dev; a.topk_weights = nullptr;
+    a.prefill = is_prefill;
+    return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
+}
+
 int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_dev, const void *w_up_dev, const int32_t *sorted_token_ids_dev,
                             const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
                             int64_t k, void *stream) {

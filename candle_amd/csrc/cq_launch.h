@@ -60,6 +60,9 @@ struct MoeArgs {
     const int32_t *sorted_token_ids, *expert_ids;
     const float *topk_weights;
     int prefill;
+    // optional second grouped matmul over the same x and pairs (gate and up of an expert MLP): out_b = x W_b^T
+    const void *w_b = nullptr;
+    float *out_b = nullptr;
 };
 int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k);
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s);

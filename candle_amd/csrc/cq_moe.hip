@@ -192,6 +192,16 @@ int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_
 
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
+    const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
+    if (a.w_b && !mfma) {
+        // only the MFMA path shares its grouping pass and quantized activations between two weight tensors
+        MoeArgs one = a;
+        one.w_b = nullptr; one.out_b = nullptr;
+        int rc = cq_moe_launch(one, workspace, s);
+        if (rc) return rc;
+        one.w = a.w_b; one.out = a.out_b;
+        return cq_moe_launch(one, workspace, s);
+    }
     PairSource ps;
     ps.mode = a.mode; ps.ids_u32 = a.ids_u32; ps.sorted_token_ids = a.sorted_token_ids; ps.expert_ids = a.expert_ids;
     ps.topk_weights = a.topk_weights; ps.topk = (int)a.topk; ps.input_dim1 = (int)a.input_dim1;
@@ -211,7 +221,6 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     int *chunks = (int *)(b + ws.chunk_off);
     // Hundreds of pairs per call on K-quant experts: the expert-sorted rows go through the MFMA prefill kernel in tiles
     // of up to 128 rows of one expert (integer-exact like the other K-quant paths).  Otherwise 8 pairs per matvec pass.
-    const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
     const int tile_rows = a.n_pairs < 40 * a.num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE;
     if (a.num_experts <= GROUP_LDS_EXPERTS)
         hipLaunchKernelGGL(moe_group_kernel<true>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
@@ -223,7 +232,9 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if (mfma) {
         if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;
         MoeChunks mc{chunks, chunks + 1, chunks + 1 + ws.max_chunks, chunks + 1 + 2 * ws.max_chunks, pout, pscale, (int)ws.max_chunks};
-        return cq_matmul_moe_launch(a.w_dtype, a.w, b + ws.act_off, ws.rows_alloc, a.out, mc, a.k, a.n, tile_rows, s);
+        rc = cq_matmul_moe_launch(a.w_dtype, a.w, b + ws.act_off, ws.rows_alloc, a.out, mc, a.k, a.n, tile_rows, s);
+        if (!rc && a.w_b) rc = cq_matmul_moe_launch(a.w_dtype, a.w_b, b + ws.act_off, ws.rows_alloc, a.out_b, mc, a.k, a.n, tile_rows, s);
+        return rc;
     }
     if (a.k % 256 == 0) {
         // Many pairs: activation rows quantized in expert-sorted order, then CQ_MOE_CHUNK pairs of an expert per pass

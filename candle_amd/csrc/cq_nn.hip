@@ -970,17 +970,16 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float *__restrict__
     // one wave picks the topk: every round the largest remaining probability, the lowest expert among equals
     volatile float *vp = prob;
     for (int j = 0; j < topk; j++) {
+        // the largest remaining value (selected entries hold -2, NaNs never compare greater), then the lowest expert holding it
         float bv = -1.0f;
+        for (int e = lane; e < n_experts; e += 64) bv = fmaxf(bv, vp[e]);
+        bv = wave_max(bv);
         int bi = 0x7fffffff;
-        for (int e = lane; e < n_experts; e += 64) {
-            const float v = vp[e];
-            if (v > bv) { bv = v; bi = e; }            // ascending e within a lane: the first of equals stays
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ov = __shfl_xor(bv, o, CQ_WAVE);
-            const int oi = __shfl_xor(bi, o, CQ_WAVE);
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        if (bv > -1.0f) {
+            for (int e0 = 0; e0 < n_experts; e0 += 64) {
+                const unsigned long long hit = __ballot(e0 + lane < n_experts && vp[min(e0 + lane, n_experts - 1)] == bv);
+                if (hit) { bi = e0 + __builtin_ctzll(hit); break; }
+            }
         }
         if (lane == 0) {
             topk_ids[(int64_t)t * topk + j] = (uint32_t)bi;       // no finite probability left (NaN logits): an id no expert has

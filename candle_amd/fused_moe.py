@@ -111,8 +111,10 @@ class FusedMoeGGUF:
             if fused != -6:
                 ck("cq_moe_gemm_gguf_swiglu", fused)
         if fused == -6:                                          # CQ_ERR_RANGE: not a shape of the fused launch
-            gemm(x2.data_ptr(), self.gate_experts, None, self.gate_out, self.inter, hidden)
-            gemm(x2.data_ptr(), self.up_experts, None, self.up_out, self.inter, hidden)
+            # gate and up share x and the pairs: one grouping pass and one activation quantization for both
+            ck("cq_moe_gemm_gguf_pair", L.cq_moe_gemm_gguf_pair(dt, x2.data_ptr(), self.gate_experts.device_ptr(), self.up_experts.device_ptr(),
+                                                                sti_ptr, eid_ptr, self.gate_out.data_ptr(), self.up_out.data_ptr(), E, topk, pairs,
+                                                                self.inter, hidden, 1 if is_prefill else 0, self.ws.data_ptr(), self.ws.numel(), sp))
             # up * silu(gate), in chunks of rows the elementwise launch takes
             for r0 in range(0, pairs, 65535):
                 r = min(65535, pairs - r0)

@@ -156,6 +156,15 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
                      int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int is_prefill,
                      void *workspace_dev, int64_t workspace_bytes, void *stream);
 
+/* Two moe_gemm_gguf calls without topk_weights over the same x and the same pairs — the gate and up matmuls of
+ * FusedMoeGGUF::forward (candle-transformers/src/fused_moe.rs:263-276) — as one call: out_a = x W_a^T, out_b = x W_b^T per
+ * pair, results identical to two cq_moe_gemm_gguf calls.  With more than 256 pairs on K-quant experts the pairs are
+ * grouped by expert and the activations quantized once for both; otherwise it is the two calls.  w_a / w_b
+ * [num_experts, n, k] of one format; workspace as cq_moe_gemm_workspace_bytes(..., has_topk_weights = 0). */
+int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, const void *w_b_dev, const int32_t *sorted_token_ids_dev,
+                          const int32_t *expert_ids_dev, float *out_a_dev, float *out_b_dev, int64_t num_experts, int64_t topk, int64_t size_m,
+                          int64_t n, int64_t k, int is_prefill, void *workspace_dev, int64_t workspace_bytes, void *stream);
+
 /* The gate and up matmuls of FusedMoeGGUF::forward with its activation (candle-transformers/src/fused_moe.rs:263-281: two
  * moe_gemm_gguf calls without topk_weights, then up * silu(gate)) in one launch, for decode-sized calls:
  *   out[tok, :] = silu(W_gate[e] . x[tok / topk, :]) * (W_up[e] . x[tok / topk, :])

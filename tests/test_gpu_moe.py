@@ -105,6 +105,35 @@ def test_moe_gemm_gguf_mfma_tile_sizes(dtype, E, n):
     assert err <= TIGHT, err
 
 
+@pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q6K, oracle.Q8_0], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("tokens", [10, 300])               # 40 pairs: two plain calls; 1200 pairs: one grouping for both (K-quants)
+def test_moe_gemm_gguf_pair_equals_two_calls(dtype, tokens):
+    """cq_moe_gemm_gguf_pair (gate and up of an expert MLP in one call) gives what two cq_moe_gemm_gguf calls give."""
+    import candle_amd as ca
+    from candle_amd import _lib
+    lib = _lib.lib()
+    E, n, k, topk = 16, 96, 512, 4
+    blocks_a, qa = make_experts(dtype, E, n, k, seed=75)
+    blocks_b, qb = make_experts(dtype, E, n, k, seed=76)
+    ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=77)
+    sti, eid = torch.from_numpy(sorted_token_ids).cuda(), torch.from_numpy(expert_ids).cuda()
+    x = torch.from_numpy(normal(78, (tokens, k), 1.0)).cuda()
+    pairs = tokens * topk
+    wsb = lib.cq_moe_gemm_workspace_bytes(int(dtype), E, topk, pairs, n, k, 0)
+    ws = torch.empty(max(wsb, 256), dtype=torch.uint8, device="cuda")
+    out_a, out_b = torch.full((pairs, n), 7.0, device="cuda"), torch.full((pairs, n), 7.0, device="cuda")
+    _lib.check("pair", lib.cq_moe_gemm_gguf_pair(int(dtype), x.data_ptr(), qa.device_ptr(), qb.device_ptr(), sti.data_ptr(), eid.data_ptr(),
+                                                 out_a.data_ptr(), out_b.data_ptr(), E, topk, pairs, n, k, 1, ws.data_ptr(), wsb, None))
+    one_a = ca.moe_gemm_gguf(x, qa, None, sti, eid, topk, True)
+    one_b = ca.moe_gemm_gguf(x, qb, None, sti, eid, topk, True)
+    torch.cuda.synchronize()
+    assert np.array_equal(out_a.cpu().numpy(), one_a.cpu().numpy()) and np.array_equal(out_b.cpu().numpy(), one_b.cpu().numpy())
+    want_b = oracle.moe_gemm_gguf(dtype, x.cpu().numpy(), blocks_b, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+    assert rel_l2(out_b.cpu().numpy(), want_b) <= TIGHT
+    assert lib.cq_moe_gemm_gguf_pair(int(dtype), x.data_ptr(), qa.device_ptr(), qb.device_ptr(), sti.data_ptr(), eid.data_ptr(),
+                                     out_a.data_ptr(), out_b.data_ptr(), E, topk, pairs, n, k, 1, ws.data_ptr(), 16, None) == -5
+
+
 @pytest.mark.parametrize("batch", [4, 120, 400])            # 12 pairs (per-pair kernels), 360 (grouped matvec), 1200 (MFMA tiles)
 def test_indexed_moe_forward_out_of_range_id_gives_zero_row(batch):
     import candle_amd as ca
