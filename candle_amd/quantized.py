@@ -65,6 +65,7 @@ _BLOCK_SIZE = {d: (1 if d in (GgmlDType.F32, GgmlDType.F16, GgmlDType.BF16) else
 _KERNEL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q8K)
 _MATMUL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
 _TORCH_TO_CQ = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 30}
+_TORCH_PLAIN = {GgmlDType.F32: torch.float32, GgmlDType.F16: torch.float16, GgmlDType.BF16: torch.bfloat16}
 
 
 def _stream_ptr() -> int:
@@ -171,6 +172,12 @@ class QStorage:
 
     def dequantize(self, elem_count: int, f16: bool = False) -> torch.Tensor:
         """QCudaStorage::dequantize / dequantize_f16 (cuda.rs:639-702)."""
+        if self._dtype in _TORCH_PLAIN:
+            # plain arrays (norm weights, unquantized embeddings of a file): a reinterpretation and a dtype cast, no blocks
+            if elem_count * self._dtype.type_size() > self._data.numel():
+                raise ValueError("dequantize: elem_count exceeds the storage")
+            t = self._data[:elem_count * self._dtype.type_size()].view(_TORCH_PLAIN[self._dtype])
+            return t.to(torch.float16 if f16 else torch.float32).clone()
         if self._dtype not in _KERNEL_DTYPES:
             raise NotImplementedError(f"dequantize is not implemented for {self._dtype.name}")
         if elem_count // self.block_size() * self._dtype.type_size() > self._data.numel():

@@ -117,12 +117,14 @@ class ModelWeights:
         cfg, L = self.cfg, self.L
         shapes = _layer_shapes(cfg)
         total, plan = 0, []
+        # a format per tensor role, which "blk.{i}.{role}" entries override for single layers (files mix formats per layer)
+        dt_of = lambda li, name: GgmlDType(dtypes.get(f"blk.{li}.{name}", dtypes[name]))
         for li in range(cfg.n_layer):
             for name in _LAYER_ORDER:
                 n, k = shapes[name]
-                nb = L.cq_storage_bytes(int(dtypes[name]), n * k)
+                nb = L.cq_storage_bytes(int(dt_of(li, name)), n * k)
                 if nb < 0:
-                    raise ValueError(f"{name}: {n}x{k} is not a whole number of {dtypes[name].name} blocks")
+                    raise ValueError(f"{name}: {n}x{k} is not a whole number of {dt_of(li, name).name} blocks")
                 plan.append((li, name, total, nb, n, k))
                 total += (nb + 255) // 256 * 256
         nb = L.cq_storage_bytes(int(dtypes["output"]), cfg.vocab * cfg.hidden)
@@ -132,7 +134,7 @@ class ModelWeights:
         base = self._slab.data_ptr()
         self.layers = [LayerWeights() for _ in range(cfg.n_layer)]
         for li, name, off, nb, n, k in plan:
-            w = _W(base + off, dtypes[name], n, k, nb)
+            w = _W(base + off, GgmlDType(dtypes[name]) if li < 0 else dt_of(li, name), n, k, nb)
             if li < 0:
                 self.output = w
             else:
@@ -214,16 +216,21 @@ class ModelWeights:
         self = cls(cfg, device)
         dtypes = {name: GgmlDType(tensors[f"blk.0.{name}"][0]) for name in _LAYER_ORDER}
         dtypes["output"] = GgmlDType(tensors["output"][0])
+        for li in range(cfg.n_layer):
+            for name in _LAYER_ORDER:
+                dtypes[f"blk.{li}.{name}"] = GgmlDType(tensors[f"blk.{li}.{name}"][0])
+        for key, dt in dtypes.items():
+            if dt not in (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K):
+                raise NotImplementedError(f"{key}: no matmul kernel for {dt.name} weights")
         plan = self._alloc(dtypes)
         for li, name, off, nb, n, k in plan:
             dt, blocks = tensors["output" if li < 0 else f"blk.{li}.{name}"]
-            if GgmlDType(dt) != dtypes[name]:
-                raise ValueError("every layer must use the same format per tensor role")
             raw = np.frombuffer(bytes(blocks), dtype=np.uint8)
             if raw.size != nb:
                 raise ValueError(f"{name}: expected {nb} bytes of blocks, got {raw.size}")
             self._slab[off:off + nb].copy_(torch.from_numpy(raw.copy()))
-        as_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device)
+        as_dev = lambda a: (a.to(device=self.device, dtype=torch.float32).contiguous() if isinstance(a, torch.Tensor)
+                            else torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(self.device))
         self.tok_embeddings = as_dev(tensors["tok_embeddings"])
         self.norm = as_dev(tensors["norm"])
         for i, lw in enumerate(self.layers):
@@ -231,6 +238,72 @@ class ModelWeights:
             lw.ffn_norm = as_dev(tensors[f"blk.{i}.ffn_norm"])
         torch.cuda.synchronize(self.device)
         return self
+
+    # architectures whose rope pairs (i, i + d/2) instead of (2i, 2i + 1) (quantized_llama.rs:396-428)
+    _NEOX_ARCHS = ("qwen", "qwen2", "qwen2moe", "qwen3", "qwen3moe", "falcon", "grok", "dbrx", "phi2", "phi3", "phimoe", "stablelm",
+                   "starcoder2", "bert", "nomic-bert", "jina-bert-v2", "olmo2", "olmoe", "codeshell", "plamo")
+
+    @classmethod
+    def from_gguf(cls, ct, reader, device="cuda:0", ctx: int = 4096) -> "ModelWeights":
+        """ModelWeights::from_gguf (quantized_llama.rs:367-540): hyper-parameters from the metadata, tensors by their
+        GGUF names, the matmul weights uploaded as the raw blocks of the file.  ``ct`` is a ``gguf_file.Content``,
+        ``reader`` the open file; ``ctx`` stands for MAX_SEQ_LEN (rows of the rope tables and of the KV cache)."""
+        from .gguf_file import GgufError
+
+        def md_get(key):
+            v = ct.metadata.get(key)
+            if v is None:
+                raise GgufError(f"cannot find {key} in metadata")
+            return v
+
+        def md_u32_or(key, default):
+            v = ct.metadata.get(key)
+            try:
+                return default if v is None else v.to_u32()
+            except GgufError:
+                return default
+
+        if md_u32_or("llama.expert_count", 0) > 1:
+            raise NotImplementedError("mixture-of-experts llama files: the expert layer is candle_amd.fused_moe.FusedMoeGGUF")
+        head_count = md_get("llama.attention.head_count").to_u32()
+        head_count_kv = md_get("llama.attention.head_count_kv").to_u32()
+        block_count = md_get("llama.block_count").to_u32()
+        embedding_length = md_get("llama.embedding_length").to_u32()
+        rope_dim = md_get("llama.rope.dimension_count").to_u32()
+        rms_norm_eps = md_get("llama.attention.layer_norm_rms_epsilon").to_f32()
+        fb = ct.metadata.get("llama.rope.freq_base")
+        try:
+            rope_freq_base = 10000.0 if fb is None else fb.to_f32()
+        except GgufError:
+            rope_freq_base = 10000.0
+        arch = ct.metadata.get("general.architecture")
+        arch = arch.v if arch is not None and isinstance(arch.v, str) else ""
+        if arch in cls._NEOX_ARCHS:
+            raise NotImplementedError(f"architecture {arch!r} uses the non-interleaved rope, which this decoder does not implement")
+        head_dim = embedding_length // head_count
+        if rope_dim != head_dim:
+            raise NotImplementedError(f"rope over {rope_dim} of {head_dim} head dimensions is not implemented")
+
+        tok_embeddings_q = ct.tensor(reader, "token_embd.weight", device)
+        tensors = {"tok_embeddings": tok_embeddings_q.dequantize(),
+                   "norm": ct.tensor(reader, "output_norm.weight", device).dequantize()}
+        out_name = "output.weight" if "output.weight" in ct.tensor_infos else "token_embd.weight"      # tied embeddings
+        info, raw = ct.tensor_bytes(reader, out_name)
+        tensors["output"] = (info.ggml_dtype, raw)
+        names = {"attention_wq": "attn_q", "attention_wk": "attn_k", "attention_wv": "attn_v", "attention_wo": "attn_output",
+                 "feed_forward_w1": "ffn_gate", "feed_forward_w2": "ffn_down", "feed_forward_w3": "ffn_up"}
+        ffn = None
+        for i in range(block_count):
+            for mine, theirs in names.items():
+                info, raw = ct.tensor_bytes(reader, f"blk.{i}.{theirs}.weight")
+                tensors[f"blk.{i}.{mine}"] = (info.ggml_dtype, raw)
+                if mine == "feed_forward_w1":
+                    ffn = info.shape[0]
+            tensors[f"blk.{i}.attention_norm"] = ct.tensor(reader, f"blk.{i}.attn_norm.weight", device).dequantize()
+            tensors[f"blk.{i}.ffn_norm"] = ct.tensor(reader, f"blk.{i}.ffn_norm.weight", device).dequantize()
+        cfg = Config(n_layer=block_count, hidden=embedding_length, n_head=head_count, n_kv_head=head_count_kv, head_dim=head_dim, ffn=ffn,
+                     vocab=tok_embeddings_q.shape()[0], rope_theta=float(rope_freq_base), rms_eps=float(rms_norm_eps), ctx=ctx)
+        return cls.from_blocks(cfg, tensors, device)
 
     def weight_bytes_per_token(self) -> int:
         """Quantized weight bytes one decode step streams (every matmul weight once)."""
