@@ -16,6 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 # GGUF type codes (candle-core/src/quantized/mod.rs:300-342)
 Q4_0, Q8_0, Q4K, Q5K, Q6K, Q8K = 2, 8, 12, 13, 14, 15
+Q4_1, Q5_0, Q5_1, Q8_1, Q2K, Q3K = 3, 6, 7, 9, 10, 11        # to_float / from_float only
 DTYPES = {"q4_0": Q4_0, "q8_0": Q8_0, "q4k": Q4K, "q5k": Q5K, "q6k": Q6K, "q8k": Q8K}
 
 _f32p = ctypes.POINTER(ctypes.c_float)

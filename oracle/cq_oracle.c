@@ -23,6 +23,10 @@
  *   closed-form and brute-force checks.  The MoE functions have no reference CPU counterpart
  *   (mod.rs:776-782 panics off-GPU); they are a composition of the pinned matmul and are pinned
  *   by brute force against per-pair matmul calls.
+ *   to_float / from_float for Q4_1, Q5_0, Q5_1, Q2_K, Q3_K are pinned by the reference's quantize -> dequantize vectors for
+ *   those formats (quantized_tests.rs:379-474, 751-844) and its error bounds; Q8_1 (no vector in the reference) by its
+ *   closed form (the Q8_0 quantizer plus s = d * sum).  These formats have no vec_dot here: the reference's matmul
+ *   kernels for them are outside the path this oracle serves.
  */
 #include <math.h>
 #include <stdint.h>
@@ -45,6 +49,12 @@ enum {
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[QK4_0 / 2]; } block_q4_0;                     /* 18 B */
 typedef struct { uint16_t d; int8_t qs[QK8_0]; } block_q8_0;                          /* 34 B */
+typedef struct { uint16_t d, m; uint8_t qs[16]; } block_q4_1;                           /* 20 B */
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } block_q5_0;               /* 22 B */
+typedef struct { uint16_t d, m; uint8_t qh[4]; uint8_t qs[16]; } block_q5_1;            /* 24 B */
+typedef struct { uint16_t d, s; int8_t qs[32]; } block_q8_1;                            /* 36 B */
+typedef struct { uint8_t scales[QK_K / 16]; uint8_t qs[QK_K / 4]; uint16_t d, dmin; } block_q2_K;   /* 84 B */
+typedef struct { uint8_t hmask[QK_K / 8]; uint8_t qs[QK_K / 4]; uint8_t scales[12]; uint16_t d; } block_q3_K; /* 110 B */
 typedef struct { uint16_t d, dmin; uint8_t scales[K_SCALE_SIZE]; uint8_t qs[QK_K / 2]; } block_q4_K; /* 144 B */
 typedef struct { uint16_t d, dmin; uint8_t scales[K_SCALE_SIZE]; uint8_t qh[QK_K / 8]; uint8_t qs[QK_K / 2]; } block_q5_K; /* 176 B */
 typedef struct { uint8_t ql[QK_K / 2]; uint8_t qh[QK_K / 4]; int8_t scales[QK_K / 16]; uint16_t d; } block_q6_K; /* 210 B */
@@ -53,6 +63,8 @@ typedef struct { float d; int8_t qs[QK_K]; int16_t bsums[QK_K / 16]; } block_q8_
 
 _Static_assert(sizeof(block_q4_0) == 18, "q4_0");
 _Static_assert(sizeof(block_q8_0) == 34, "q8_0");
+_Static_assert(sizeof(block_q4_1) == 20 && sizeof(block_q5_0) == 22 && sizeof(block_q5_1) == 24 && sizeof(block_q8_1) == 36, "32-element blocks");
+_Static_assert(sizeof(block_q2_K) == 84 && sizeof(block_q3_K) == 110, "q2_K / q3_K");
 _Static_assert(sizeof(block_q4_K) == 144, "q4_K");
 _Static_assert(sizeof(block_q5_K) == 176, "q5_K");
 _Static_assert(sizeof(block_q6_K) == 210, "q6_K");
@@ -797,12 +809,313 @@ static float q6_K_q8_K_vec_dot(int64_t n, const block_q6_K *xs, const block_q8_K
 }
 
 /* ==========================================================================================
+ * The remaining GgmlDType block formats: to_float / from_float only.
+ * ======================================================================================== */
+static inline uint32_t rd_u32le(const uint8_t *p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24); }
+static inline void wr_u32le(uint8_t *p, uint32_t v) { p[0] = (uint8_t)v; p[1] = (uint8_t)(v >> 8); p[2] = (uint8_t)(v >> 16); p[3] = (uint8_t)(v >> 24); }
+static inline float f32_min_rust(float a, float b) { return (a != a) ? b : ((b != b) ? a : (a < b ? a : b)); }   /* f32::min ignores NaN */
+static inline float f32_max_rust(float a, float b) { return (a != a) ? b : ((b != b) ? a : (a > b ? a : b)); }
+
+static void q4_1_from_float(const float *xs, block_q4_1 *ys, int64_t k) {   /* k_quants.rs:353-389 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float *x = xs + i * 32;
+        float min = INFINITY, max = -INFINITY;
+        for (int j = 0; j < 32; j++) { min = f32_min_rust(x[j], min); max = f32_max_rust(x[j], max); }
+        float d = (max - min) / 15.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        ys[i].d = cqo_f32_to_f16(d);
+        ys[i].m = cqo_f32_to_f16(min);
+        for (int j = 0; j < 16; j++) {
+            float x0 = (x[j] - min) * id, x1 = (x[16 + j] - min) * id;
+            uint8_t xi0 = sat_u8(x0 + 0.5f), xi1 = sat_u8(x1 + 0.5f);
+            if (xi0 > 15) xi0 = 15;
+            if (xi1 > 15) xi1 = 15;
+            ys[i].qs[j] = (uint8_t)(xi0 | (xi1 << 4));
+        }
+    }
+}
+static void q4_1_to_float(const block_q4_1 *xs, float *ys, int64_t k) {     /* :392-412 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        float d = cqo_f16_to_f32(xs[i].d), m = cqo_f16_to_f32(xs[i].m);
+        for (int j = 0; j < 16; j++) {
+            ys[i * 32 + j] = (float)(xs[i].qs[j] & 0x0F) * d + m;
+            ys[i * 32 + j + 16] = (float)(xs[i].qs[j] >> 4) * d + m;
+        }
+    }
+}
+
+static void q5_0_from_float(const float *xs, block_q5_0 *ys, int64_t k) {   /* :457-493 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float *x = xs + i * 32;
+        float amax = 0.0f, max = 0.0f;
+        for (int j = 0; j < 32; j++) if (amax < fabsf(x[j])) { amax = fabsf(x[j]); max = x[j]; }
+        float d = max / -16.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        ys[i].d = cqo_f32_to_f16(d);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            float x0 = x[j] * id, x1 = x[j + 16] * id;
+            int8_t a = sat_i8(x0 + 16.5f), b = sat_i8(x1 + 16.5f);
+            uint8_t xi0 = (uint8_t)(a < 31 ? a : 31), xi1 = (uint8_t)(b < 31 ? b : 31);
+            ys[i].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (((uint32_t)xi0 & 0x10) >> 4) << j;
+            qh |= (((uint32_t)xi1 & 0x10) >> 4) << (j + 16);
+        }
+        wr_u32le(ys[i].qh, qh);
+    }
+}
+static void q5_0_to_float(const block_q5_0 *xs, float *ys, int64_t k) {     /* :496-518 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        float d = cqo_f16_to_f32(xs[i].d);
+        uint32_t qh = rd_u32le(xs[i].qh);
+        for (int j = 0; j < 16; j++) {
+            uint8_t xh_0 = (uint8_t)(((qh >> j) << 4) & 0x10), xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+            int32_t x0 = (int32_t)((xs[i].qs[j] & 0x0F) | xh_0) - 16, x1 = (int32_t)((xs[i].qs[j] >> 4) | xh_1) - 16;
+            ys[i * 32 + j] = (float)x0 * d;
+            ys[i * 32 + j + 16] = (float)x1 * d;
+        }
+    }
+}
+
+static void q5_1_from_float(const float *xs, block_q5_1 *ys, int64_t k) {   /* :564-604 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float *x = xs + i * 32;
+        float min = INFINITY, max = -INFINITY;
+        for (int j = 0; j < 32; j++) { min = f32_min_rust(x[j], min); max = f32_max_rust(x[j], max); }
+        float d = (max - min) / 31.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        ys[i].d = cqo_f32_to_f16(d);
+        ys[i].m = cqo_f32_to_f16(min);
+        uint32_t qh = 0;
+        for (int j = 0; j < 16; j++) {
+            float x0 = (x[j] - min) * id, x1 = (x[16 + j] - min) * id;
+            uint8_t xi0 = sat_u8(x0 + 0.5f), xi1 = sat_u8(x1 + 0.5f);
+            ys[i].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (((uint32_t)xi0 & 0x10) >> 4) << j;
+            qh |= (((uint32_t)xi1 & 0x10) >> 4) << (j + 16);
+        }
+        wr_u32le(ys[i].qh, qh);
+    }
+}
+static void q5_1_to_float(const block_q5_1 *xs, float *ys, int64_t k) {     /* :607-631 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        float d = cqo_f16_to_f32(xs[i].d), m = cqo_f16_to_f32(xs[i].m);
+        uint32_t qh = rd_u32le(xs[i].qh);
+        for (int j = 0; j < 16; j++) {
+            uint8_t xh_0 = (uint8_t)(((qh >> j) << 4) & 0x10), xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+            uint8_t x0 = (uint8_t)((xs[i].qs[j] & 0x0F) | xh_0), x1 = (uint8_t)((xs[i].qs[j] >> 4) | xh_1);
+            ys[i * 32 + j] = (float)x0 * d + m;
+            ys[i * 32 + j + 16] = (float)x1 * d + m;
+        }
+    }
+}
+
+static void q8_1_from_float(const float *xs, block_q8_1 *ys, int64_t k) {   /* :770-799 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float *x = xs + i * 32;
+        float amax = 0.0f;
+        for (int j = 0; j < 32; j++) amax = f32_max_rust(amax, fabsf(x[j]));
+        float d = amax / 127.0f;
+        float id = d != 0.0f ? 1.0f / d : 0.0f;
+        ys[i].d = cqo_f32_to_f16(d);
+        int32_t sum = 0;
+        for (int j = 0; j < 16; j++) {
+            ys[i].qs[j] = sat_i8(roundf(x[j] * id));
+            ys[i].qs[j + 16] = sat_i8(roundf(x[j + 16] * id));
+            sum += (int32_t)ys[i].qs[j] + (int32_t)ys[i].qs[j + 16];
+        }
+        /* f16::from_f32(sum as f32) * ys.d: the product of two f16 values, computed in f32 and rounded back to f16 */
+        ys[i].s = cqo_f32_to_f16(cqo_f16_to_f32(cqo_f32_to_f16((float)sum)) * cqo_f16_to_f32(ys[i].d));
+    }
+}
+static void q8_1_to_float(const block_q8_1 *xs, float *ys, int64_t k) {     /* :801-816 */
+    for (int64_t i = 0; i < k / 32; i++) {
+        float d = cqo_f16_to_f32(xs[i].d);
+        for (int j = 0; j < 32; j++) ys[i * 32 + j] = (float)xs[i].qs[j] * d;
+    }
+}
+
+static void q2_K_from_float(const float *xs, block_q2_K *ys, int64_t k) {   /* :891-953 */
+    const float Q4SCALE = 15.0f;
+    for (int64_t b = 0; b < k / QK_K; b++) {
+        const float *x = xs + b * QK_K;
+        block_q2_K *blk = ys + b;
+        float mins[16], scales[16];
+        for (int j = 0; j < 16; j++) make_qkx1_quants(3, 5, x + 16 * j, 16, &scales[j], &mins[j]);
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < 16; j++) { max_scale = f32_max_rust(scales[j], max_scale); max_min = f32_max_rust(mins[j], max_min); }
+        if (max_scale > 0.0f) {
+            float iscale = Q4SCALE / max_scale;
+            for (int j = 0; j < 16; j++) blk->scales[j] = (uint8_t)nearest_int(iscale * scales[j]);
+            blk->d = cqo_f32_to_f16(max_scale / Q4SCALE);
+        } else {
+            for (int j = 0; j < 16; j++) blk->scales[j] = 0;
+            blk->d = cqo_f32_to_f16(0.0f);
+        }
+        if (max_min > 0.0f) {
+            float iscale = Q4SCALE / max_min;
+            for (int j = 0; j < 16; j++) blk->scales[j] |= (uint8_t)((uint8_t)nearest_int(iscale * mins[j]) << 4);
+            blk->dmin = cqo_f32_to_f16(max_min / Q4SCALE);
+        } else {
+            blk->dmin = cqo_f32_to_f16(0.0f);
+        }
+        uint8_t big_l[QK_K];
+        memset(big_l, 0, sizeof(big_l));
+        for (int j = 0; j < 16; j++) {
+            float d = cqo_f16_to_f32(blk->d) * (float)(blk->scales[j] & 0xF);
+            if (d == 0.0f) continue;
+            float dm = cqo_f16_to_f32(blk->dmin) * (float)(blk->scales[j] >> 4);
+            for (int ii = 0; ii < 16; ii++) big_l[16 * j + ii] = (uint8_t)clamp_i32(nearest_int((x[16 * j + ii] + dm) / d), 0, 3);
+        }
+        for (int j = 0; j < QK_K; j += 128)
+            for (int l = 0; l < 32; l++)
+                blk->qs[j / 4 + l] = (uint8_t)(big_l[j + l] | (big_l[j + l + 32] << 2) | (big_l[j + l + 64] << 4) | (big_l[j + l + 96] << 6));
+    }
+}
+static void q2_K_to_float(const block_q2_K *xs, float *ys, int64_t k) {     /* :1013-1049 */
+    for (int64_t b = 0; b < k / QK_K; b++) {
+        const block_q2_K *blk = xs + b;
+        float *y = ys + b * QK_K;
+        float d = cqo_f16_to_f32(blk->d), min = cqo_f16_to_f32(blk->dmin);
+        int is = 0;
+        for (int h = 0; h < 2; h++) {
+            const uint8_t *qs = blk->qs + 32 * h;
+            int yi = 128 * h;
+            for (int shift = 0; shift < 8; shift += 2) {
+                for (int half = 0; half < 2; half++) {
+                    uint8_t sc = blk->scales[is++];
+                    float dl = d * (float)(sc & 0xF), ml = min * (float)(sc >> 4);
+                    for (int l = 0; l < 16; l++) y[yi++] = dl * (float)((qs[16 * half + l] >> shift) & 3) - ml;
+                }
+            }
+        }
+    }
+}
+
+/* utils.rs:287-352 make_q3_quants(x, nmax, do_rmse = true) -> scale (the levels are not used by the caller) */
+static float make_q3_quants(const float *x, int n, int32_t nmax) {
+    int8_t l[64];
+    float max = 0.0f, amax = 0.0f;
+    for (int i = 0; i < n; i++) { float ax = fabsf(x[i]); if (ax > amax) { amax = ax; max = x[i]; } }
+    if (amax == 0.0f) return 0.0f;
+    float iscale = -(float)nmax / max;
+    float sumlx = 0.0f, suml2 = 0.0f;
+    for (int i = 0; i < n; i++) {
+        int32_t li = clamp_i32(sat_i32(roundf(iscale * x[i])), -nmax, nmax - 1);
+        l[i] = (int8_t)li;
+        float w = x[i] * x[i];
+        sumlx += w * x[i] * (float)li;
+        suml2 += w * (float)(li * li);
+    }
+    for (int t = 0; t < 5; t++) {
+        int n_changed = 0;
+        for (int i = 0; i < n; i++) {
+            float w = x[i] * x[i];
+            float slx = sumlx - w * x[i] * (float)l[i];
+            if (slx > 0.0f) {
+                float sl2 = suml2 - w * (float)((int32_t)l[i] * (int32_t)l[i]);
+                int32_t new_l = clamp_i32(sat_i32(roundf(x[i] * sl2 / slx)), -nmax, nmax - 1);
+                if (new_l != (int32_t)l[i]) {
+                    slx += w * x[i] * (float)new_l;
+                    sl2 += w * (float)(new_l * new_l);
+                    if (sl2 > 0.0f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                        l[i] = (int8_t)new_l;
+                        sumlx = slx;
+                        suml2 = sl2;
+                        n_changed++;
+                    }
+                }
+            }
+        }
+        if (n_changed == 0) break;
+    }
+    return sumlx / suml2;
+}
+
+static void q3_K_from_float(const float *xs, block_q3_K *ys, int64_t k) {   /* :1190-1269 */
+    for (int64_t b = 0; b < k / QK_K; b++) {
+        const float *x = xs + b * QK_K;
+        block_q3_K *blk = ys + b;
+        float scales[16];
+        for (int j = 0; j < 16; j++) scales[j] = make_q3_quants(x + 16 * j, 16, 4);
+        float max_scale = 0.0f;
+        for (int j = 0; j < 16; j++) if (fabsf(scales[j]) > fabsf(max_scale)) max_scale = scales[j];
+        memset(blk->scales, 0, sizeof(blk->scales));
+        if (max_scale != 0.0f) {
+            float iscale = -32.0f / max_scale;
+            for (int j = 0; j < 16; j++) {
+                int32_t l_val = clamp_i32(nearest_int(iscale * scales[j]), -32, 31) + 32;
+                if (j < 8) blk->scales[j] = (uint8_t)(l_val & 0xF);
+                else blk->scales[j - 8] |= (uint8_t)((l_val & 0xF) << 4);
+                l_val >>= 4;
+                blk->scales[j % 4 + 8] |= (uint8_t)(l_val << (2 * (j / 4)));
+            }
+            blk->d = cqo_f32_to_f16(1.0f / iscale);
+        } else {
+            blk->d = cqo_f32_to_f16(0.0f);
+        }
+        int8_t l[QK_K];
+        memset(l, 0, sizeof(l));
+        for (int j = 0; j < 16; j++) {
+            uint8_t sc = j < 8 ? (blk->scales[j] & 0xF) : (blk->scales[j - 8] >> 4);
+            int8_t scs = (int8_t)((int8_t)(sc | (((blk->scales[8 + j % 4] >> (2 * (j / 4))) & 3) << 4)) - 32);
+            float d = cqo_f16_to_f32(blk->d) * (float)scs;
+            if (d != 0.0f)
+                for (int ii = 0; ii < 16; ii++) l[16 * j + ii] = (int8_t)(clamp_i32(nearest_int(x[16 * j + ii] / d), -4, 3) + 4);
+        }
+        memset(blk->hmask, 0, sizeof(blk->hmask));
+        int m = 0;
+        uint8_t hm = 1;
+        for (int i = 0; i < QK_K; i++) {
+            if (l[i] > 3) { blk->hmask[m] |= hm; l[i] -= 4; }
+            if (++m == QK_K / 8) { m = 0; hm <<= 1; }
+        }
+        for (int j = 0; j < QK_K; j += 128)
+            for (int v = 0; v < 32; v++)
+                blk->qs[j / 4 + v] = (uint8_t)(l[j + v] | (l[j + v + 32] << 2) | (l[j + v + 64] << 4) | (l[j + v + 96] << 6));
+    }
+}
+static void q3_K_to_float(const block_q3_K *xs, float *ys, int64_t k) {     /* :1369-1421 */
+    const uint32_t KMASK1 = 0x03030303u, KMASK2 = 0x0f0f0f0fu;
+    for (int64_t b = 0; b < k / QK_K; b++) {
+        const block_q3_K *blk = xs + b;
+        float *y = ys + b * QK_K;
+        uint32_t aux[4];
+        aux[0] = rd_u32le(blk->scales); aux[1] = rd_u32le(blk->scales + 4); aux[2] = rd_u32le(blk->scales + 8);
+        uint32_t tmp = aux[2];
+        aux[2] = ((aux[0] >> 4) & KMASK2) | (((tmp >> 4) & KMASK1) << 4);
+        aux[3] = ((aux[1] >> 4) & KMASK2) | (((tmp >> 6) & KMASK1) << 4);
+        aux[0] = (aux[0] & KMASK2) | ((tmp & KMASK1) << 4);
+        aux[1] = (aux[1] & KMASK2) | (((tmp >> 2) & KMASK1) << 4);
+        int8_t scales[16];
+        for (int i = 0; i < 16; i++) scales[i] = (int8_t)((aux[i / 4] >> (8 * (i % 4))) & 0xff);
+        float d_all = cqo_f16_to_f32(blk->d);
+        uint8_t m = 1;
+        int is = 0;
+        for (int h = 0; h < 2; h++) {
+            const uint8_t *qs = blk->qs + 32 * h;
+            for (int shift = 0; shift < 8; shift += 2) {
+                for (int si = 0; si < 2; si++) {
+                    float dl = d_all * ((float)scales[is++] - 32.0f);
+                    for (int i = 0; i < 16; i++) {
+                        int8_t q = (int8_t)((qs[i + 16 * si] >> shift) & 3);
+                        int8_t v = (int8_t)(q - ((blk->hmask[i + 16 * si] & m) == 0 ? 4 : 0));
+                        y[128 * h + 16 * (shift) + 16 * si + i] = dl * (float)v;       /* shift / 2 * 32 + 16 si + i */
+                    }
+                }
+                m <<= 1;
+            }
+        }
+    }
+}
+
+/* ==========================================================================================
  * dtype dispatch (mod.rs:386-421 type_size/block_size) and the exported entry points
  * ======================================================================================== */
 int64_t cqo_block_size(int dtype) {
     switch (dtype) {
-        case CQ_Q4_0: case CQ_Q8_0: return 32;
-        case CQ_Q4K: case CQ_Q5K: case CQ_Q6K: case CQ_Q8K: return QK_K;
+        case CQ_Q4_0: case CQ_Q8_0: case CQ_Q4_1: case CQ_Q5_0: case CQ_Q5_1: case CQ_Q8_1: return 32;
+        case CQ_Q4K: case CQ_Q5K: case CQ_Q6K: case CQ_Q8K: case CQ_Q2K: case CQ_Q3K: return QK_K;
         default: return 0;
     }
 }
@@ -815,6 +1128,12 @@ int64_t cqo_type_size(int dtype) {
         case CQ_Q5K: return sizeof(block_q5_K);
         case CQ_Q6K: return sizeof(block_q6_K);
         case CQ_Q8K: return sizeof(block_q8_K);
+        case CQ_Q4_1: return sizeof(block_q4_1);
+        case CQ_Q5_0: return sizeof(block_q5_0);
+        case CQ_Q5_1: return sizeof(block_q5_1);
+        case CQ_Q8_1: return sizeof(block_q8_1);
+        case CQ_Q2K: return sizeof(block_q2_K);
+        case CQ_Q3K: return sizeof(block_q3_K);
         default: return 0;
     }
 }
@@ -839,6 +1158,12 @@ int cqo_to_float(int dtype, const void *blocks, float *ys, int64_t k) {
         case CQ_Q5K: q5_K_to_float((const block_q5_K *)blocks, ys, k); return 0;
         case CQ_Q6K: q6_K_to_float((const block_q6_K *)blocks, ys, k); return 0;
         case CQ_Q8K: q8_K_to_float((const block_q8_K *)blocks, ys, k); return 0;
+        case CQ_Q4_1: q4_1_to_float((const block_q4_1 *)blocks, ys, k); return 0;
+        case CQ_Q5_0: q5_0_to_float((const block_q5_0 *)blocks, ys, k); return 0;
+        case CQ_Q5_1: q5_1_to_float((const block_q5_1 *)blocks, ys, k); return 0;
+        case CQ_Q8_1: q8_1_to_float((const block_q8_1 *)blocks, ys, k); return 0;
+        case CQ_Q2K: q2_K_to_float((const block_q2_K *)blocks, ys, k); return 0;
+        case CQ_Q3K: q3_K_to_float((const block_q3_K *)blocks, ys, k); return 0;
     }
     return -1;
 }
@@ -854,6 +1179,12 @@ int cqo_from_float(int dtype, const float *xs, void *blocks, int64_t k) {
         case CQ_Q5K: q5_K_from_float(xs, (block_q5_K *)blocks, k); return 0;
         case CQ_Q6K: q6_K_from_float(xs, (block_q6_K *)blocks, k); return 0;
         case CQ_Q8K: q8_K_from_float(xs, (block_q8_K *)blocks, k); return 0;
+        case CQ_Q4_1: q4_1_from_float(xs, (block_q4_1 *)blocks, k); return 0;
+        case CQ_Q5_0: q5_0_from_float(xs, (block_q5_0 *)blocks, k); return 0;
+        case CQ_Q5_1: q5_1_from_float(xs, (block_q5_1 *)blocks, k); return 0;
+        case CQ_Q8_1: q8_1_from_float(xs, (block_q8_1 *)blocks, k); return 0;
+        case CQ_Q2K: q2_K_from_float(xs, (block_q2_K *)blocks, k); return 0;
+        case CQ_Q3K: q3_K_from_float(xs, (block_q3_K *)blocks, k); return 0;
     }
     return -1;
 }

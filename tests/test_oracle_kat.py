@@ -131,6 +131,75 @@ def test_kat_kquant_test_vector2(dtype, spots, tol_small, tol_big):
     assert np.all(np.abs(dst_big - big) < tol_big)
 
 
+# ---------------------------------------------------------------- KAT-4..6 : Q4_1, Q5_0, Q5_1 on 0..127
+Q4_1_WANT = [v for base in (0.0, 32.0, 64.0, 96.0) for v in
+             ([base, base] + [x for q in (2.066, 4.133, 6.199, 8.266, 10.332, 12.398, 14.465, 16.531, 18.598, 20.664, 22.73, 24.797,
+                                          26.863, 28.93, 30.996) for x in (base + q, base + q)])]      # quantized_tests.rs:392-406
+Q5_0_WANT = [-0.0, 1.938, 1.938, 3.875, 3.875, 5.813, 5.813, 7.75, 7.75, 9.688, 9.688, 11.625,
+             11.625, 13.563, 13.563, 15.5, 15.5, 17.438, 17.438, 19.375, 19.375, 21.313, 21.313,
+             23.25, 23.25, 25.188, 25.188, 27.125, 27.125, 29.063, 29.063, 31.0, 31.5, 31.5, 35.438,
+             35.438, 35.438, 35.438, 39.375, 39.375, 39.375, 39.375, 43.313, 43.313, 43.313, 43.313,
+             47.25, 47.25, 47.25, 47.25, 51.188, 51.188, 51.188, 51.188, 55.125, 55.125, 55.125,
+             55.125, 59.063, 59.063, 59.063, 59.063, 63.0, 63.0, 65.313, 65.313, 65.313, 65.313,
+             65.313, 71.25, 71.25, 71.25, 71.25, 71.25, 71.25, 77.188, 77.188, 77.188, 77.188,
+             77.188, 77.188, 83.125, 83.125, 83.125, 83.125, 83.125, 83.125, 89.063, 89.063, 89.063,
+             89.063, 89.063, 89.063, 95.0, 95.0, 95.0, 95.25, 95.25, 95.25, 95.25, 103.188, 103.188,
+             103.188, 103.188, 103.188, 103.188, 103.188, 103.188, 111.125, 111.125, 111.125,
+             111.125, 111.125, 111.125, 111.125, 111.125, 119.063, 119.063, 119.063, 119.063,
+             119.063, 119.063, 119.063, 119.063, 127.0, 127.0, 127.0, 127.0]                            # :425-438
+
+
+def test_kat_q4_1_q5_0_q5_1_roundtrip_arange128():
+    src = np.arange(128, dtype=np.float32)
+    got = round3(oracle.to_float(oracle.Q4_1, oracle.from_float(oracle.Q4_1, src)))
+    assert got.tolist() == [float(round3([v])[0]) for v in Q4_1_WANT]
+    got = round3(oracle.to_float(oracle.Q5_0, oracle.from_float(oracle.Q5_0, src)))
+    assert got.tolist() == [float(np.float32(v)) for v in Q5_0_WANT]
+    got = round3(oracle.to_float(oracle.Q5_1, oracle.from_float(oracle.Q5_1, src)))             # :458-470: exact
+    assert got.tolist() == src.tolist()
+
+
+# ---------------------------------------------------------------- KAT-7..8 : Q2K, Q3K spot values + bounds
+@pytest.mark.parametrize("dtype,spots,tol_small,tol_big", [
+    (oracle.Q2K, [-0.499, -0.366, -0.249, 0.0, 0.295, 0.492], 0.1, 6.0),       # :751-797
+    (oracle.Q3K, [-0.493, -0.37, -0.243, -0.0, 0.292, 0.492], 0.03, 3.5),      # :799-844
+])
+def test_kat_q2k_q3k_test_vector2(dtype, spots, tol_small, tol_big):
+    src = get_test_vector2(0.5, 1024)
+    dst = oracle.to_float(dtype, oracle.from_float(dtype, src))
+    assert np.all(np.abs(dst - src) < tol_small)
+    got = round3(dst)[[0, 128, 256, 512, 800, 1023]]
+    assert got.tolist() == [float(np.float32(s)) for s in spots]
+    big = get_test_vector2(128.0, 1024)
+    dst_big = oracle.to_float(dtype, oracle.from_float(dtype, big))
+    assert np.all(np.abs(dst_big - big) < tol_big)
+
+
+@pytest.mark.parametrize("dtype,ceiling", [(oracle.Q4_1, 0.002), (oracle.Q5_0, 0.002), (oracle.Q5_1, 0.002), (oracle.Q8_1, 0.002),
+                                           (oracle.Q2K, 0.0075), (oracle.Q3K, 0.004)])
+def test_bound_quantization_rmse_remaining_formats(dtype, ceiling):
+    # quantized_tests.rs:12-17,531-552 with the 2-bit / 3-bit ceilings of :14-15
+    src = ggml_like_vector(0.0)
+    dst = oracle.to_float(dtype, oracle.from_float(dtype, src))
+    err = np.sqrt(np.sum((src - dst).astype(np.float32) ** 2, dtype=np.float32)) / np.float32(src.size)
+    assert err <= ceiling
+
+
+def test_q8_1_closed_form():
+    """No vector in the reference: Q8_1 is the Q8_0 quantizer (same d, same int8 values in the same order) plus
+    s = f16(f16(sum) * d) (k_quants.rs:770-799)."""
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(32 * 40) * 3).astype(np.float32)
+    b1 = oracle.from_float(oracle.Q8_1, x).reshape(-1, 36)
+    b0 = oracle.from_float(oracle.Q8_0, x).reshape(-1, 34)
+    assert np.array_equal(b1[:, :2], b0[:, :2]) and np.array_equal(b1[:, 4:], b0[:, 2:])
+    d = b1[:, :2].copy().view(np.float16).astype(np.float32).reshape(-1)
+    sums = b1[:, 4:].copy().view(np.int8).astype(np.int32).sum(axis=1)
+    want_s = (sums.astype(np.float32).astype(np.float16).astype(np.float32) * d).astype(np.float16)
+    assert np.array_equal(b1[:, 2:4].copy().view(np.float16).reshape(-1), want_s)
+    assert np.array_equal(oracle.to_float(oracle.Q8_1, b1.reshape(-1)), oracle.to_float(oracle.Q8_0, b0.reshape(-1)))
+
+
 # ---------------------------------------------------------------- BOUND-1 : ggml quantization RMSE ceiling
 @pytest.mark.parametrize("dtype", [oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q8K])
 def test_bound_quantization_rmse(dtype):
