@@ -13,6 +13,10 @@ inline bool matmul_weight_dtype(int dt) {
 }
 
 inline bool block_dtype(int dt) { return matmul_weight_dtype(dt) || dt == CQ_Q8K; }
+// every GGUF block format can be stored and dequantized; the matmul-family and quantize entry points take fewer
+inline bool storage_dtype(int dt) {
+    return block_dtype(dt) || dt == CQ_Q4_1 || dt == CQ_Q5_0 || dt == CQ_Q5_1 || dt == CQ_Q8_1 || dt == CQ_Q2K || dt == CQ_Q3K;
+}
 
 inline bool float_dtype(int dt) { return dt == CQ_F32 || dt == CQ_F16 || dt == CQ_BF16; }
 
@@ -87,7 +91,7 @@ int64_t cq_storage_bytes(int dtype, int64_t elem_count) {
 }
 
 int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem_count, int out_dtype, void *stream) {
-    if (!block_dtype(dtype)) return CQ_ERR_DTYPE;
+    if (!storage_dtype(dtype)) return CQ_ERR_DTYPE;
     if (out_dtype != CQ_F32 && out_dtype != CQ_F16) return CQ_ERR_DTYPE;
     if (elem_count < 0 || elem_count % cq_block_size(dtype) != 0) return CQ_ERR_SHAPE;
     if (elem_count == 0) return CQ_OK;

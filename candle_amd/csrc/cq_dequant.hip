@@ -4,8 +4,10 @@
 // store), so a wave writes 1 KiB / 512 B of contiguous output; the kernel is write-bound
 // (4 B out per 0.5-1.06 B in).  The arithmetic is the CPU to_float, evaluated in the same order:
 //   Q4_0 k_quants.rs:219-239, Q8_0 :640-656, Q4_K :1667-1694, Q5_K :1962-1996, Q6_K :2247-2278,
-//   Q8_K :2360-2371 (candle-core/src/quantized/k_quants.rs).
-// All products are exactly representable in f32, so results are bit-identical to the CPU.
+//   Q8_K :2360-2371, and the formats that exist here only as storage (no matmul kernels): Q4_1 :392-412, Q5_0 :496-518,
+//   Q5_1 :607-631, Q8_1 :801-816, Q2_K :1013-1049, Q3_K :1369-1421 (candle-core/src/quantized/k_quants.rs).
+// All products are exactly representable in f32 (so a fused multiply-add rounds like the CPU's multiply then add), and
+// results are bit-identical to the CPU.
 #include "cq_device.h"
 
 namespace {
@@ -91,6 +93,70 @@ template <> __device__ __forceinline__ void dequant4<CQ_Q6K>(const uint8_t *blk,
     }
 }
 
+template <> __device__ __forceinline__ void dequant4<CQ_Q4_1>(const uint8_t *blk, int e, float out[4]) {
+    uint32_t dm = ld_u<uint32_t>(blk);
+    float d = h2f(dm), m = h2f(dm >> 16);
+    uint32_t q = ld_u<uint32_t>(blk + 4 + (e & 15));
+    if (e >= 16) q >>= 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[i] = (float)((q >> (8 * i)) & 0xF) * d + m;
+}
+
+// Q5_0 / Q5_1: bit j of the little-endian u32 qh is the fifth bit of element j (both halves of the block)
+template <> __device__ __forceinline__ void dequant4<CQ_Q5_0>(const uint8_t *blk, int e, float out[4]) {
+    float d = h2f(ld_u<uint16_t>(blk));
+    uint32_t qh = ld_u<uint32_t>(blk + 2) >> e;
+    uint32_t q = ld_u<uint32_t>(blk + 6 + (e & 15));
+    if (e >= 16) q >>= 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[i] = (float)((int)(((q >> (8 * i)) & 0xF) | (((qh >> i) & 1) << 4)) - 16) * d;
+}
+
+template <> __device__ __forceinline__ void dequant4<CQ_Q5_1>(const uint8_t *blk, int e, float out[4]) {
+    uint32_t dm = ld_u<uint32_t>(blk);
+    float d = h2f(dm), m = h2f(dm >> 16);
+    uint32_t qh = ld_u<uint32_t>(blk + 4) >> e;
+    uint32_t q = ld_u<uint32_t>(blk + 8 + (e & 15));
+    if (e >= 16) q >>= 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[i] = (float)(((q >> (8 * i)) & 0xF) | (((qh >> i) & 1) << 4)) * d + m;
+}
+
+template <> __device__ __forceinline__ void dequant4<CQ_Q8_1>(const uint8_t *blk, int e, float out[4]) {
+    float d = h2f(ld_u<uint16_t>(blk));
+    uint32_t q = ld_u<uint32_t>(blk + 4 + e);
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[i] = (float)(int8_t)((q >> (8 * i)) & 0xFF) * d;
+}
+
+// Q2_K / Q3_K: element e = 128 h + 32 j + l holds bits [2 j, 2 j + 2) of qs[32 h + l]; its scale is number 8 h + 2 j + l / 16
+template <> __device__ __forceinline__ void dequant4<CQ_Q2K>(const uint8_t *blk, int e, float out[4]) {
+    uint32_t dm = ld_u<uint32_t>(blk + 80);
+    float d = h2f(dm), dmin = h2f(dm >> 16);
+    int h = e >> 7, j = (e >> 5) & 3, l = e & 31;
+    uint32_t sc = blk[8 * h + 2 * j + (l >> 4)];
+    float dl = d * (float)(sc & 0xF), ml = dmin * (float)(sc >> 4);
+    uint32_t q = ld_u<uint32_t>(blk + 16 + 32 * h + l) >> (2 * j);
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[i] = dl * (float)((q >> (8 * i)) & 3) - ml;
+}
+
+template <> __device__ __forceinline__ void dequant4<CQ_Q3K>(const uint8_t *blk, int e, float out[4]) {
+    float d_all = h2f(ld_u<uint16_t>(blk + 108));
+    int h = e >> 7, j = (e >> 5) & 3, l = e & 31;
+    // 6-bit scale number is: low four bits in scales[is % 8] (low nibble for is < 8, high nibble otherwise), top two bits in
+    // scales[8 + is % 4] at bit 2 (is / 4); stored with an offset of 32
+    int is = 8 * h + 2 * j + (l >> 4);
+    const uint8_t *sc = blk + 96;
+    int lo = is < 8 ? (sc[is] & 0xF) : (sc[is - 8] >> 4);
+    int hi = (sc[8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+    float dl = d_all * ((float)(int8_t)(lo | (hi << 4)) - 32.0f);
+    uint32_t q = ld_u<uint32_t>(blk + 32 + 32 * h + l) >> (2 * j);
+    uint32_t hm = ld_u<uint32_t>(blk + l) >> (4 * h + j);          // hmask bit set: no -4
+#pragma unroll
+    for (int i = 0; i < 4; i++) out[i] = dl * (float)((int)((q >> (8 * i)) & 3) - (((hm >> (8 * i)) & 1) ? 0 : 4));
+}
+
 template <int DT, bool F16OUT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ blocks, void *__restrict__ out, int64_t n_quads) {
     constexpr int E = BlockInfo<DT>::elems, B = BlockInfo<DT>::bytes;
@@ -134,6 +200,12 @@ int cq_dequantize_launch(int dtype, const void *blocks, void *out, int64_t elems
         case CQ_Q5K: return launch_dequant<CQ_Q5K>(blocks, out, elems, out_dtype, s);
         case CQ_Q6K: return launch_dequant<CQ_Q6K>(blocks, out, elems, out_dtype, s);
         case CQ_Q8K: return launch_dequant<CQ_Q8K>(blocks, out, elems, out_dtype, s);
+        case CQ_Q4_1: return launch_dequant<CQ_Q4_1>(blocks, out, elems, out_dtype, s);
+        case CQ_Q5_0: return launch_dequant<CQ_Q5_0>(blocks, out, elems, out_dtype, s);
+        case CQ_Q5_1: return launch_dequant<CQ_Q5_1>(blocks, out, elems, out_dtype, s);
+        case CQ_Q8_1: return launch_dequant<CQ_Q8_1>(blocks, out, elems, out_dtype, s);
+        case CQ_Q2K: return launch_dequant<CQ_Q2K>(blocks, out, elems, out_dtype, s);
+        case CQ_Q3K: return launch_dequant<CQ_Q3K>(blocks, out, elems, out_dtype, s);
     }
     return CQ_ERR_DTYPE;
 }

@@ -24,6 +24,12 @@ template <> struct BlockInfo<CQ_Q4K> { static constexpr int elems = 256, bytes =
 template <> struct BlockInfo<CQ_Q5K> { static constexpr int elems = 256, bytes = 176; };
 template <> struct BlockInfo<CQ_Q6K> { static constexpr int elems = 256, bytes = 210; };
 template <> struct BlockInfo<CQ_Q8K> { static constexpr int elems = 256, bytes = 292; };
+template <> struct BlockInfo<CQ_Q4_1> { static constexpr int elems = 32, bytes = 20; };
+template <> struct BlockInfo<CQ_Q5_0> { static constexpr int elems = 32, bytes = 22; };
+template <> struct BlockInfo<CQ_Q5_1> { static constexpr int elems = 32, bytes = 24; };
+template <> struct BlockInfo<CQ_Q8_1> { static constexpr int elems = 32, bytes = 36; };
+template <> struct BlockInfo<CQ_Q2K> { static constexpr int elems = 256, bytes = 84; };
+template <> struct BlockInfo<CQ_Q3K> { static constexpr int elems = 256, bytes = 110; };
 
 __host__ __device__ inline bool cq_is_kquant(int dt) { return dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q8K; }
 __host__ __device__ inline bool cq_is_q0(int dt) { return dt == CQ_Q4_0 || dt == CQ_Q8_0; }

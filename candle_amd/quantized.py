@@ -63,6 +63,8 @@ _BLOCK_SIZE = {d: (1 if d in (GgmlDType.F32, GgmlDType.F16, GgmlDType.BF16) else
 
 # block formats the HIP kernels implement
 _KERNEL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q8K)
+# ... and the ones that can be stored and dequantized only
+_DEQUANT_DTYPES = _KERNEL_DTYPES + (GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q8_1, GgmlDType.Q2K, GgmlDType.Q3K)
 _MATMUL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
 _TORCH_TO_CQ = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 30}
 _TORCH_PLAIN = {GgmlDType.F32: torch.float32, GgmlDType.F16: torch.float16, GgmlDType.BF16: torch.bfloat16}
@@ -178,7 +180,7 @@ class QStorage:
                 raise ValueError("dequantize: elem_count exceeds the storage")
             t = self._data[:elem_count * self._dtype.type_size()].view(_TORCH_PLAIN[self._dtype])
             return t.to(torch.float16 if f16 else torch.float32).clone()
-        if self._dtype not in _KERNEL_DTYPES:
+        if self._dtype not in _DEQUANT_DTYPES:
             raise NotImplementedError(f"dequantize is not implemented for {self._dtype.name}")
         if elem_count // self.block_size() * self._dtype.type_size() > self._data.numel():
             raise ValueError("dequantize: elem_count exceeds the storage")

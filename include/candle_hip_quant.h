@@ -62,7 +62,8 @@ int64_t cq_storage_bytes(int dtype, int64_t elem_count);
  * QTensor::dequantize / dequantize_f16 (mod.rs:689-710; CUDA: cuda.rs:105-223,
  * candle-kernels/src/quantized.cu:780-1156).  Bit-exact with GgmlType::to_float on the CPU; the
  * f16 result equals the f32 result rounded to nearest even.
- *   dtype: Q4_0, Q8_0, Q4K, Q5K, Q6K, Q8K.   out_dtype: CQ_F32 or CQ_F16.
+ *   dtype: every block format of GgmlDType — Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K (the matmul-family
+ *   entry points and cq_quantize take Q4_0, Q8_0, Q4K, Q5K, Q6K (+ Q8K for cq_quantize) only).   out_dtype: CQ_F32 or CQ_F16.
  *   blocks_dev: 2-byte aligned.  out_dev: 16-byte aligned.
  * ------------------------------------------------------------------------------------------- */
 int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem_count, int out_dtype, void *stream);

@@ -15,7 +15,10 @@ from tests.util import bits_equal_or_both_nan, normal
 pytestmark = pytest.mark.gpu
 
 DTYPES = [oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q8K]
-NAMES = {oracle.Q4_0: "q4_0", oracle.Q8_0: "q8_0", oracle.Q4K: "q4k", oracle.Q5K: "q5k", oracle.Q6K: "q6k", oracle.Q8K: "q8k"}
+# formats that exist on the GPU as storage only (dequantize, no matmul / quantize kernels)
+STORAGE_DTYPES = [oracle.Q4_1, oracle.Q5_0, oracle.Q5_1, oracle.Q8_1, oracle.Q2K, oracle.Q3K]
+NAMES = {oracle.Q4_0: "q4_0", oracle.Q8_0: "q8_0", oracle.Q4K: "q4k", oracle.Q5K: "q5k", oracle.Q6K: "q6k", oracle.Q8K: "q8k",
+         oracle.Q4_1: "q4_1", oracle.Q5_0: "q5_0", oracle.Q5_1: "q5_1", oracle.Q8_1: "q8_1", oracle.Q2K: "q2k", oracle.Q3K: "q3k"}
 
 
 def _candle():
@@ -39,7 +42,7 @@ def gpu_quantize(dtype, x: np.ndarray) -> np.ndarray:
 
 
 # ------------------------------------------------------------------------------- dequantize
-@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("dtype", DTYPES + STORAGE_DTYPES, ids=lambda d: NAMES[d])
 def test_dequantize_random_bytes_bit_exact(dtype):
     # every byte pattern is a valid block, including NaN / Inf / subnormal f16 scales
     rng = np.random.Generator(np.random.PCG64(100 + dtype))
@@ -51,7 +54,7 @@ def test_dequantize_random_bytes_bit_exact(dtype):
     assert bits_equal_or_both_nan(got, want)
 
 
-@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("dtype", DTYPES + STORAGE_DTYPES, ids=lambda d: NAMES[d])
 def test_dequantize_quantized_gaussian_bit_exact_and_f16(dtype):
     x = normal(7, 256 * 1024, 0.02)
     blocks = oracle.from_float(dtype, x)
@@ -69,7 +72,8 @@ def test_dequantize_empty_and_errors():
     L = _lib.lib()
     assert L.cq_dequantize(int(ca.GgmlDType.Q4K), None, None, 0, 0, None) == 0          # empty is ok
     assert L.cq_dequantize(int(ca.GgmlDType.Q4K), None, None, 100, 0, None) == -2        # not a block multiple
-    assert L.cq_dequantize(int(ca.GgmlDType.Q2K), None, None, 256, 0, None) == -1        # unsupported format
+    assert L.cq_dequantize(int(ca.GgmlDType.F16), None, None, 256, 0, None) == -1        # not a block format
+    assert L.cq_quantize(int(ca.GgmlDType.Q2K), None, None, 256, None) == -1             # storage-only format: no quantizer
     assert L.cq_dequantize(int(ca.GgmlDType.Q4K), None, None, 256, 0, None) == -4        # NULL
 
 
