@@ -24,6 +24,7 @@ SIGNATURES = {
     "cq_type_size": (_i64, [_int]),
     "cq_storage_bytes": (_i64, [_int, _i64]),
     "cq_dequantize": (_int, [_int, _vp, _vp, _i64, _int, _vp]),
+    "cq_embedding": (_int, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "cq_quantize": (_int, [_int, _vp, _vp, _i64, _vp]),
     "cq_act_scratch_bytes": (_i64, [_int, _i64, _i64]),
     "cq_quantize_act": (_int, [_int, _vp, _int, _vp, _i64, _i64, _vp]),

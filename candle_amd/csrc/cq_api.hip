@@ -100,6 +100,17 @@ int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem
     return cq_dequantize_launch(dtype, blocks_dev, out_dev, elem_count, out_dtype, (hipStream_t)stream);
 }
 
+int cq_embedding(int dtype, const void *blocks_dev, const uint32_t *ids_dev, float *out_dev, int64_t n_ids, int64_t rows, int64_t hidden,
+                 void *stream) {
+    if (!storage_dtype(dtype)) return CQ_ERR_DTYPE;
+    if (n_ids < 0 || rows <= 0 || hidden <= 0 || hidden % cq_block_size(dtype) != 0) return CQ_ERR_SHAPE;
+    if (rows > 0x7fffffffLL || hidden > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (n_ids == 0) return CQ_OK;
+    if (!blocks_dev || !ids_dev || !out_dev) return CQ_ERR_NULL;
+    if (!aligned(blocks_dev, 2) || !aligned(ids_dev, 4) || !aligned(out_dev, 16)) return CQ_ERR_ALIGN;
+    return cq_embedding_launch(dtype, blocks_dev, ids_dev, out_dev, n_ids, rows, hidden, (hipStream_t)stream);
+}
+
 int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stream) {
     if (bytes < 0 || bytes % 16) return CQ_ERR_SHAPE;
     if (bytes == 0) return CQ_OK;

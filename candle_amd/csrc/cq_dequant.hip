@@ -178,6 +178,36 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
     }
 }
 
+// QTensor::embedding: output row r is row ids[r] of the [rows, hidden] block matrix, dequantized (mod.rs:449-473).  An id
+// outside [0, rows) gives a row of zeros (the CPU path reports an error instead; the host wrapper checks the ids).
+template <int DT>
+__global__ __launch_bounds__(256) void embedding_rows_kernel(const uint8_t *__restrict__ blocks, const uint32_t *__restrict__ ids,
+                                                             float *__restrict__ out, int64_t n_quads, int quads_per_row, int rows) {
+    constexpr int E = BlockInfo<DT>::elems, B = BlockInfo<DT>::bytes;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n_quads) return;
+    const int64_t r = t / quads_per_row;
+    const int64_t col = (t - r * quads_per_row) * 4;
+    const uint32_t id = ids[r];
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (id < (uint32_t)rows) {
+        const int64_t elem = (int64_t)id * quads_per_row * 4 + col;
+        const int64_t ib = elem / E;
+        dequant4<DT>(blocks + ib * B, (int)(elem - ib * E), v);
+    }
+    reinterpret_cast<f32x4 *>(out)[t] = f32x4{v[0], v[1], v[2], v[3]};
+}
+
+template <int DT> int launch_embedding(const void *blocks, const uint32_t *ids, float *out, int64_t n_ids, int64_t rows, int64_t hidden, hipStream_t s) {
+    const int64_t quads = n_ids * (hidden / 4);
+    if (quads == 0) return CQ_OK;
+    const int64_t grid = (quads + 255) / 256;
+    if (grid > 0x7fffffffLL) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL((embedding_rows_kernel<DT>), dim3((unsigned)grid), dim3(256), 0, s, (const uint8_t *)blocks, ids, out, quads, (int)(hidden / 4),
+                       (int)rows);
+    return (int)hipGetLastError();
+}
+
 template <int DT> int launch_dequant(const void *blocks, void *out, int64_t elems, int out_dtype, hipStream_t s) {
     int64_t quads = elems / 4;
     if (quads == 0) return CQ_OK;
@@ -206,6 +236,16 @@ int cq_dequantize_launch(int dtype, const void *blocks, void *out, int64_t elems
         case CQ_Q8_1: return launch_dequant<CQ_Q8_1>(blocks, out, elems, out_dtype, s);
         case CQ_Q2K: return launch_dequant<CQ_Q2K>(blocks, out, elems, out_dtype, s);
         case CQ_Q3K: return launch_dequant<CQ_Q3K>(blocks, out, elems, out_dtype, s);
+    }
+    return CQ_ERR_DTYPE;
+}
+
+int cq_embedding_launch(int dtype, const void *blocks, const uint32_t *ids, float *out, int64_t n_ids, int64_t rows, int64_t hidden, hipStream_t s) {
+    switch (dtype) {
+#define CQ_EMB(DT) case DT: return launch_embedding<DT>(blocks, ids, out, n_ids, rows, hidden, s);
+        CQ_EMB(CQ_Q4_0) CQ_EMB(CQ_Q4_1) CQ_EMB(CQ_Q5_0) CQ_EMB(CQ_Q5_1) CQ_EMB(CQ_Q8_0) CQ_EMB(CQ_Q8_1)
+        CQ_EMB(CQ_Q2K) CQ_EMB(CQ_Q3K) CQ_EMB(CQ_Q4K) CQ_EMB(CQ_Q5K) CQ_EMB(CQ_Q6K) CQ_EMB(CQ_Q8K)
+#undef CQ_EMB
     }
     return CQ_ERR_DTYPE;
 }

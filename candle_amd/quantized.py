@@ -254,6 +254,32 @@ class QTensor:
         t = self.storage.dequantize(self.elem_count(), f16=True).reshape(self._shape)
         return t if device is None else t.to(device)
 
+    def embedding(self, ids: torch.Tensor) -> torch.Tensor:
+        """mod.rs:712-748: rows ``ids`` of a [rows, hidden] tensor, dequantized -> ids.shape + (hidden,) in f32."""
+        if len(self._shape) != 2:
+            raise ValueError(f"embedding expects a rank-2 tensor, got shape {self._shape}")
+        rows, hidden = self._shape
+        dt = self.dtype()
+        if hidden % dt.block_size():
+            raise ValueError(f"quantized embedding hidden size {hidden} is not divisible by block size {dt.block_size()}")
+        dev = self.device()
+        flat = ids.to(dev).reshape(-1).to(torch.int64)
+        if flat.numel() and (int(flat.max()) >= rows or int(flat.min()) < 0):
+            bad = int(flat[(flat >= rows) | (flat < 0)][0])
+            raise ValueError(f"embedding id {bad} is out of range for {rows} rows")
+        out_shape = tuple(ids.shape) + (hidden,)
+        if dt in _TORCH_PLAIN:                                   # plain arrays: an index_select on the typed view
+            w = self.storage._data[:rows * hidden * dt.type_size()].view(_TORCH_PLAIN[dt]).reshape(rows, hidden)
+            return w.index_select(0, flat).to(torch.float32).reshape(out_shape)
+        if dt not in _DEQUANT_DTYPES:
+            raise NotImplementedError(f"embedding is not implemented for {dt.name}")
+        ids32 = flat.to(torch.int32).contiguous()                # u32 values
+        out = torch.empty((flat.numel(), hidden), dtype=torch.float32, device=dev)
+        L = _lib.lib()
+        _lib.check("cq_embedding", L.cq_embedding(int(dt), self.storage.device_ptr(), ids32.data_ptr(), out.data_ptr(), flat.numel(), rows, hidden,
+                                                  _stream_ptr()))
+        return out.reshape(out_shape)
+
     def storage_size_in_bytes(self) -> int:
         return self.storage.size_in_bytes()
 

@@ -69,6 +69,16 @@ int64_t cq_storage_bytes(int dtype, int64_t elem_count);
 int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem_count, int out_dtype, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * QTensor::embedding (mod.rs:712-748, CPU kernel :449-473): out [n_ids, hidden] f32, row r = row ids[r] of the
+ * [rows, hidden] block matrix, dequantized (bit-exact with dequantize + index_select).  Every block format of
+ * cq_dequantize; hidden a multiple of the block size.  An id >= rows gives a row of zeros where the CPU path returns
+ * an error (a launch cannot); callers that need the error check the ids first.
+ *   blocks_dev: 2-byte aligned.  ids_dev: u32.  out_dev: 16-byte aligned.
+ * ------------------------------------------------------------------------------------------- */
+int cq_embedding(int dtype, const void *blocks_dev, const uint32_t *ids_dev, float *out_dev, int64_t n_ids, int64_t rows, int64_t hidden,
+                 void *stream);
+
+/* ---------------------------------------------------------------------------------------------
  * QTensor::quantize on a device tensor (mod.rs:543-562).  The CUDA backend copies to the host,
  * runs GgmlType::from_float and copies back (cuda.rs:704-725); here the same arithmetic runs on the
  * GPU, one thread per block, and produces the same bytes as the CPU from_float.

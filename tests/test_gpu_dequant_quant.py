@@ -198,3 +198,55 @@ def test_act_quant_f16_bf16_inputs_widen_first():
         for r in range(2):
             blk = oracle.from_float(oracle.Q8K, widened[r]).reshape(k // 256, 292)
             assert np.array_equal(qs[r], blk[:, 4:260].copy().view(np.int8).reshape(-1))
+
+
+# ------------------------------------------------------------------------------- QTensor::embedding
+def embedding_weight():
+    # quantized_tests.rs:265-273
+    i = np.arange(8 * 256, dtype=np.float32)
+    return (np.sin(i * np.float32(0.003)) * np.float32(0.5) + np.cos(i * np.float32(0.007)) * np.float32(0.25)).astype(np.float32).reshape(8, 256)
+
+
+@pytest.mark.parametrize("dtype", DTYPES + STORAGE_DTYPES, ids=lambda d: NAMES[d])
+def test_quantized_embedding_equals_dequantize_then_index_select(dtype):
+    """quantized_tests.rs:287-322 (tolerance 1e-6 there; the rows are bit-identical here), then a larger table with
+    repeated and boundary ids."""
+    ca = _candle()
+    w = embedding_weight()
+    blocks = oracle.from_float(dtype, w.reshape(-1))
+    q = ca.QTensor.new(ca.QStorage.from_data(blocks, "cuda", ca.GgmlDType(dtype)), (8, 256))
+    ids = torch.tensor([[3, 1], [3, 7]], dtype=torch.int32)
+    got = q.embedding(ids)
+    want = oracle.to_float(dtype, blocks, w.size).reshape(8, 256)[[3, 1, 3, 7]].reshape(2, 2, 256)
+    assert got.shape == (2, 2, 256) and np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert torch.equal(got, q.dequantize().index_select(0, ids.reshape(-1).cuda().long()).reshape(2, 2, 256))
+    rows, hidden = 1000, 768
+    big = normal(9, rows * hidden, 0.05)
+    bb = oracle.from_float(dtype, big)
+    qb = ca.QTensor.new(ca.QStorage.from_data(bb, "cuda", ca.GgmlDType(dtype)), (rows, hidden))
+    idb = np.array([0, 999, 5, 5, 512, 0, 998], dtype=np.int64)
+    gotb = qb.embedding(torch.from_numpy(idb)).cpu().numpy()
+    wantb = oracle.to_float(dtype, bb, big.size).reshape(rows, hidden)[idb]
+    assert np.array_equal(gotb.view(np.uint32), wantb.view(np.uint32))
+    with pytest.raises(ValueError):
+        qb.embedding(torch.tensor([1000]))
+
+
+def test_embedding_of_plain_arrays_and_launch_rules():
+    ca = _candle()
+    from candle_amd import _lib
+    w = embedding_weight()
+    for dt, arr in ((ca.GgmlDType.F32, w), (ca.GgmlDType.F16, w.astype(np.float16))):
+        q = ca.QTensor.new(ca.QStorage.from_data(arr.tobytes(), "cuda", dt), (8, 256))
+        got = q.embedding(torch.tensor([7, 0])).cpu().numpy()
+        assert np.array_equal(got, arr[[7, 0]].astype(np.float32))
+    L = _lib.lib()
+    blocks = torch.zeros(8 * 144, dtype=torch.uint8, device="cuda")
+    ids = torch.tensor([2, 9], dtype=torch.int32, device="cuda")
+    out = torch.full((2, 256), 5.0, device="cuda")
+    # the launch itself cannot fail on an id: such a row is zeros
+    assert L.cq_embedding(12, blocks.data_ptr(), ids.data_ptr(), out.data_ptr(), 2, 8, 256, None) == 0
+    torch.cuda.synchronize()
+    assert torch.all(out[1] == 0.0)
+    assert L.cq_embedding(12, blocks.data_ptr(), ids.data_ptr(), out.data_ptr(), 2, 8, 100, None) == -2
+    assert L.cq_embedding(1, blocks.data_ptr(), ids.data_ptr(), out.data_ptr(), 2, 8, 256, None) == -1
