@@ -258,10 +258,11 @@ template <int NH> __device__ __forceinline__ void lds_write_h(_Float16 *dstrow, 
 // workgroups share a CU and one converts operands while the other feeds the matrix cores.
 // MOE: blockIdx.x is a tile of the chunk table: up to BMT expert-sorted activation rows [first, first + count) of
 // expert e; the weights are that expert's [n, k] matrix and output rows are scattered through pair_out with pair_scale.
-// SM (experts with few rows each): the block tile is 32 (m) x 128 (n), the four waves side by side along n, so that a
+// SM (experts with few rows each): the block tile is 32 (m) x 128 (n) (one workgroup per CU for a two-term format, whose
+// two weight tiles fill the LDS), the four waves side by side along n, so that a
 // 16-row expert fills half of its tiles instead of an eighth, and one workgroup converts twice the weight rows per stage.
 template <int DT, int NJ, bool MOE = false, bool SM = false>
-__global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k,
+__global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 : 1) void qmm_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst, int k,
                                                                      int n, int rows, int64_t stride_dst, MoeChunks mc, int64_t expert_bytes,
                                                                      int64_t split_stride) {
     typedef Stage<DT> S;
