@@ -25,8 +25,10 @@
  *   by brute force against per-pair matmul calls.
  *   to_float / from_float for Q4_1, Q5_0, Q5_1, Q2_K, Q3_K are pinned by the reference's quantize -> dequantize vectors for
  *   those formats (quantized_tests.rs:379-474, 751-844) and its error bounds; Q8_1 (no vector in the reference) by its
- *   closed form (the Q8_0 quantizer plus s = d * sum).  These formats have no vec_dot here: the reference's matmul
- *   kernels for them are outside the path this oracle serves.
+ *   closed form (the Q8_0 quantizer plus s = d * sum).  vec_dot / matmul for Q4_1, Q5_0, Q5_1, Q2_K, Q3_K are pinned by
+ *   the reference's dot-product error ceilings (quantized_tests.rs:1101-1191), its seeded matmul values for Q2_K and
+ *   Q3_K (:1331-1381), and the identity vec_dot(w, a) == sum(to_float(w) * to_float(a)) evaluated in f64 with the
+ *   pinned to_float functions (random blocks, every bit of qs / qh / hmask / scales exercised).
  */
 #include <math.h>
 #include <stdint.h>
@@ -1110,6 +1112,140 @@ static void q3_K_to_float(const block_q3_K *xs, float *ys, int64_t k) {     /* :
 }
 
 /* ==========================================================================================
+ * vec_dot of the remaining formats against their VecDotType (Q8_1, Q8_0, Q8_1, Q8_K, Q8_K)
+ * ======================================================================================== */
+static float q4_1_q8_1_vec_dot(int64_t n, const block_q4_1 *xs, const block_q8_1 *ys) { /* k_quants.rs:323-351 */
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < n / 32; i++) {
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) {
+            int32_t v0 = xs[i].qs[j] & 0x0F, v1 = xs[i].qs[j] >> 4;
+            sumi += v0 * (int32_t)ys[i].qs[j] + v1 * (int32_t)ys[i].qs[j + 16];
+        }
+        float t = (float)sumi * cqo_f16_to_f32(xs[i].d) * cqo_f16_to_f32(ys[i].d);
+        float u = cqo_f16_to_f32(xs[i].m) * cqo_f16_to_f32(ys[i].s);
+        sumf += t + u;
+    }
+    return sumf;
+}
+
+static float q5_0_q8_0_vec_dot(int64_t n, const block_q5_0 *xs, const block_q8_0 *ys) { /* :434-455 */
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < n / 32; i++) {
+        uint32_t qh = rd_u32le(xs[i].qh);
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) {
+            int32_t xh_0 = (int32_t)(uint8_t)(((qh & (1u << j)) >> j) << 4);
+            int32_t xh_1 = (int32_t)(uint8_t)((qh & (1u << (j + 16))) >> (j + 12));
+            int32_t x0 = ((xs[i].qs[j] & 0x0F) | xh_0) - 16;
+            int32_t x1 = ((xs[i].qs[j] >> 4) | xh_1) - 16;
+            sumi += x0 * (int32_t)ys[i].qs[j] + x1 * (int32_t)ys[i].qs[j + 16];
+        }
+        sumf += (float)sumi * cqo_f16_to_f32(xs[i].d) * cqo_f16_to_f32(ys[i].d);
+    }
+    return sumf;
+}
+
+static float q5_1_q8_1_vec_dot(int64_t n, const block_q5_1 *xs, const block_q8_1 *ys) { /* :530-562 */
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < n / 32; i++) {
+        uint32_t qh = rd_u32le(xs[i].qh);
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) {
+            int32_t xh_0 = (int32_t)(((qh >> j) << 4) & 0x10);
+            int32_t xh_1 = (int32_t)((qh >> (j + 12)) & 0x10);
+            int32_t x0 = (xs[i].qs[j] & 0xF) | xh_0;
+            int32_t x1 = (xs[i].qs[j] >> 4) | xh_1;
+            sumi += x0 * (int32_t)ys[i].qs[j] + x1 * (int32_t)ys[i].qs[j + 16];
+        }
+        float t = (float)sumi * cqo_f16_to_f32(xs[i].d) * cqo_f16_to_f32(ys[i].d);
+        float u = cqo_f16_to_f32(xs[i].m) * cqo_f16_to_f32(ys[i].s);
+        sumf += t + u;
+    }
+    return sumf;
+}
+
+static float q2_K_q8_K_vec_dot(int64_t n, const block_q2_K *xs, const block_q8_K *ys) { /* :838-886 */
+    float sumf = 0.0f;
+    for (int64_t i = 0; i < n / QK_K; i++) {
+        const block_q2_K *x = xs + i;
+        const block_q8_K *y = ys + i;
+        const uint8_t *q2 = x->qs;
+        const int8_t *q8 = y->qs;
+        int32_t summs = 0;
+        for (int j = 0; j < 16; j++) summs += (int32_t)y->bsums[j] * (int32_t)(x->scales[j] >> 4);
+        float dall = y->d * cqo_f16_to_f32(x->d);
+        float dmin = y->d * cqo_f16_to_f32(x->dmin);
+        int32_t isum = 0;
+        int is = 0;
+        for (int h = 0; h < QK_K / 128; h++) {
+            for (int shift = 0; shift < 8; shift += 2) {
+                for (int half = 0; half < 2; half++) {
+                    int32_t d = x->scales[is++] & 0xF;
+                    int32_t isuml = 0;
+                    for (int l = 16 * half; l < 16 * half + 16; l++) isuml += (int32_t)q8[l] * (int32_t)((q2[l] >> shift) & 3);
+                    isum += d * isuml;
+                }
+                q8 += 32;
+            }
+            q2 += 32;
+        }
+        sumf += dall * (float)isum - dmin * (float)summs;
+    }
+    return sumf;
+}
+
+static float q3_K_q8_K_vec_dot(int64_t n, const block_q3_K *xs, const block_q8_K *ys) { /* :1068-1187 */
+    const uint32_t KMASK1 = 0x03030303u, KMASK2 = 0x0f0f0f0fu;
+    int8_t aux8[QK_K];
+    int16_t aux16[8];
+    float sums[8] = {0};
+    int32_t aux32[8];
+    for (int64_t i = 0; i < n / QK_K; i++) {
+        const block_q3_K *x = xs + i;
+        const block_q8_K *y = ys + i;
+        const uint8_t *q3 = x->qs;
+        const int8_t *q8 = y->qs;
+        memset(aux32, 0, sizeof(aux32));
+        int8_t *a = aux8;
+        uint8_t m = 1;
+        for (int h = 0; h < QK_K / 128; h++) {
+            for (int shift = 0; shift < 8; shift += 2) {
+                for (int l = 0; l < 32; l++) {
+                    int8_t v = (int8_t)((q3[l] >> shift) & 3);
+                    a[l] = (int8_t)(v - ((x->hmask[l] & m) != 0 ? 0 : 4));
+                }
+                a += 32;
+                m <<= 1;
+            }
+            q3 += 32;
+        }
+        a = aux8;
+        uint32_t auxs[4];
+        auxs[0] = rd_u32le(x->scales); auxs[1] = rd_u32le(x->scales + 4); auxs[2] = rd_u32le(x->scales + 8);
+        uint32_t tmp = auxs[2];
+        auxs[2] = ((auxs[0] >> 4) & KMASK2) | (((tmp >> 4) & KMASK1) << 4);
+        auxs[3] = ((auxs[1] >> 4) & KMASK2) | (((tmp >> 6) & KMASK1) << 4);
+        auxs[0] = (auxs[0] & KMASK2) | ((tmp & KMASK1) << 4);
+        auxs[1] = (auxs[1] & KMASK2) | (((tmp >> 2) & KMASK1) << 4);
+        for (int j = 0; j < 16; j++) {
+            int32_t scale = (int32_t)(int8_t)((auxs[j / 4] >> (8 * (j % 4))) & 0xff) - 32;
+            for (int r = 0; r < 2; r++) {
+                for (int l = 0; l < 8; l++) aux16[l] = (int16_t)((int16_t)q8[l] * (int16_t)a[l]);
+                for (int l = 0; l < 8; l++) aux32[l] += scale * (int32_t)aux16[l];
+                q8 += 8;
+                a += 8;
+            }
+        }
+        float d = cqo_f16_to_f32(x->d) * y->d;
+        for (int l = 0; l < 8; l++) sums[l] += d * (float)aux32[l];
+    }
+    float s = 0.0f;
+    for (int l = 0; l < 8; l++) s += sums[l];
+    return s;
+}
+
+/* ==========================================================================================
  * dtype dispatch (mod.rs:386-421 type_size/block_size) and the exported entry points
  * ======================================================================================== */
 int64_t cqo_block_size(int dtype) {
@@ -1141,8 +1277,9 @@ int64_t cqo_type_size(int dtype) {
 /* the activation ("VecDotType") block type for a weight type: k_quants.rs:216,637,1427,1701,2002,2284 */
 int cqo_vec_dot_type(int dtype) {
     switch (dtype) {
-        case CQ_Q4_0: case CQ_Q8_0: return CQ_Q8_0;
-        case CQ_Q4K: case CQ_Q5K: case CQ_Q6K: case CQ_Q8K: return CQ_Q8K;
+        case CQ_Q4_0: case CQ_Q8_0: case CQ_Q5_0: return CQ_Q8_0;
+        case CQ_Q4_1: case CQ_Q5_1: return CQ_Q8_1;                               /* :317,524 */
+        case CQ_Q2K: case CQ_Q3K: case CQ_Q4K: case CQ_Q5K: case CQ_Q6K: case CQ_Q8K: return CQ_Q8K;   /* :822,1055 */
         default: return -1;
     }
 }
@@ -1200,6 +1337,11 @@ int cqo_vec_dot(int dtype, int64_t n, const void *xs, const void *ys, float *out
         case CQ_Q5K: *out = q5_K_q8_K_vec_dot(n, (const block_q5_K *)xs, (const block_q8_K *)ys); return 0;
         case CQ_Q6K: *out = q6_K_q8_K_vec_dot(n, (const block_q6_K *)xs, (const block_q8_K *)ys); return 0;
         case CQ_Q8K: *out = q8_K_q8_K_vec_dot(n, (const block_q8_K *)xs, (const block_q8_K *)ys); return 0;
+        case CQ_Q4_1: *out = q4_1_q8_1_vec_dot(n, (const block_q4_1 *)xs, (const block_q8_1 *)ys); return 0;
+        case CQ_Q5_0: *out = q5_0_q8_0_vec_dot(n, (const block_q5_0 *)xs, (const block_q8_0 *)ys); return 0;
+        case CQ_Q5_1: *out = q5_1_q8_1_vec_dot(n, (const block_q5_1 *)xs, (const block_q8_1 *)ys); return 0;
+        case CQ_Q2K: *out = q2_K_q8_K_vec_dot(n, (const block_q2_K *)xs, (const block_q8_K *)ys); return 0;
+        case CQ_Q3K: *out = q3_K_q8_K_vec_dot(n, (const block_q3_K *)xs, (const block_q8_K *)ys); return 0;
     }
     return -1;
 }

@@ -212,7 +212,8 @@ def test_bound_quantization_rmse(dtype):
 
 # ---------------------------------------------------------------- BOUND-2 : dot-product error vs ggml ceilings
 GGML_DOT_ERR = {oracle.Q4_0: 0.001143, oracle.Q8_0: 0.000092, oracle.Q4K: 0.002425, oracle.Q5K: 0.000740,
-                oracle.Q6K: 0.000952, oracle.Q8K: 0.00065}   # quantized_tests.rs:1101-1122
+                oracle.Q6K: 0.000952, oracle.Q8K: 0.00065,   # quantized_tests.rs:1101-1122
+                oracle.Q2K: 0.004086, oracle.Q3K: 0.017, oracle.Q4_1: 0.008, oracle.Q5_0: 0.001353, oracle.Q5_1: 0.00149}
 
 
 @pytest.mark.parametrize("dtype", list(GGML_DOT_ERR))
@@ -251,6 +252,8 @@ SEEDED_MATMUL = [
     (oracle.Q5K, [1.161, 1.498, -0.175, 1.739]),   # :1409-1434
     (oracle.Q6K, [1.293, 1.497, -0.159, 1.737]),   # :1436-1459
     (oracle.Q8K, [1.241, 1.52, -0.2, 1.7]),        # :1461-1483
+    (oracle.Q2K, [0.887, 0.428, 0.219, 1.669]),    # :1331-1354
+    (oracle.Q3K, [1.001, 1.425, -0.311, 1.493]),   # :1357-1380
 ]
 
 
@@ -265,7 +268,8 @@ def test_kat_seeded_matmul(dtype, want):
 
 
 # ---------------------------------------------------------------- test_matmul (1,3,4,256) mean relative error
-@pytest.mark.parametrize("dtype", [oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q8K])
+@pytest.mark.parametrize("dtype", [oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q8K,
+                                   oracle.Q4_1, oracle.Q5_0, oracle.Q5_1, oracle.Q2K, oracle.Q3K])
 def test_matmul_relative_error_ramp(dtype):
     # quantized_tests.rs:19-54 with (b,m,n,k) = (1,3,4,256): mean |mm - res| / |mm| <= 0.02
     m, n, k = 3, 4, 256
@@ -279,7 +283,8 @@ def test_matmul_relative_error_ramp(dtype):
 
 
 # ---------------------------------------------------------------- INV-1 : batching invariance
-@pytest.mark.parametrize("dtype", [oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K])
+@pytest.mark.parametrize("dtype", [oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K,
+                                   oracle.Q4_1, oracle.Q5_0, oracle.Q5_1, oracle.Q2K, oracle.Q3K])
 def test_batching_invariance(dtype):
     # quantized_tests.rs:224-259: the same rows give bit-identical outputs at any batch size on the CPU
     lhs, rhs = stdrng.get_random_tensors(2, 256, 6)
@@ -288,3 +293,49 @@ def test_batching_invariance(dtype):
     mm6 = oracle.matmul(dtype, np.concatenate([lhs, lhs, lhs]), w, 6)
     for i in range(3):
         assert np.array_equal(mm6[2 * i:2 * i + 2].view(np.uint32), mm.view(np.uint32))
+
+
+# ---------------------------------------------------------------- vec_dot of Q4_1, Q5_0, Q5_1, Q2_K, Q3_K
+# byte offsets of the f16 fields (d, m / dmin) inside a block, k_quants.rs:86-147
+F16_FIELDS = {oracle.Q4_1: (0, 2), oracle.Q5_0: (0,), oracle.Q5_1: (0, 2), oracle.Q2K: (80, 82), oracle.Q3K: (108,),
+              oracle.Q4_0: (0,), oracle.Q8_0: (0,), oracle.Q4K: (0, 2), oracle.Q5K: (0, 2), oracle.Q6K: (208,)}
+
+
+def random_weight_blocks(dtype, nblocks, rng):
+    """Random block bytes (every bit of qs / qh / hmask / scales in play) with finite f16 scale fields."""
+    ts = oracle.type_size(dtype)
+    b = rng.integers(0, 256, size=(nblocks, ts), dtype=np.uint8)
+    for off in F16_FIELDS[dtype]:
+        h = rng.uniform(-2.0, 2.0, size=nblocks).astype(np.float16).view(np.uint16)
+        b[:, off] = (h & 0xff).astype(np.uint8)
+        b[:, off + 1] = (h >> 8).astype(np.uint8)
+    return b.reshape(-1)
+
+
+def exact_activations(n, rng):
+    """Activations every CPU quantizer represents exactly: x = 2^e * q with integer |q| <= 60 and one 127 per 32-element
+    block (so d = amax / 127 = 2^e, q is recovered unchanged, |sum q| <= 2048 and the Q8_1 field s = d * sum is exact)."""
+    q = rng.integers(-60, 61, size=n).astype(np.float32)
+    q[np.arange(0, n, 32) + rng.integers(0, 32, size=n // 32)] = 127.0
+    return (q * np.float32(2.0 ** -5)).astype(np.float32)
+
+
+@pytest.mark.parametrize("dtype", list(F16_FIELDS))
+def test_vec_dot_is_the_dot_product_of_the_dequantized_operands(dtype):
+    # With exactly representable activations vec_dot(w, q(a)) is, in real arithmetic, sum(to_float(w) * to_float(q(a))):
+    # the pinned to_float functions fix every index, shift, mask, offset and scale of the integer part; what is left is
+    # f32 rounding of the block sums.  A wrong nibble / high-bit / sub-block pairing changes the value by O(1).
+    rng = np.random.default_rng(1234 + dtype)
+    n = 1024
+    vdt = oracle.vec_dot_type(dtype)
+    for _ in range(8):
+        w = random_weight_blocks(dtype, n // oracle.block_size(dtype), rng)
+        a = exact_activations(n, rng)
+        aq = oracle.from_float(vdt, a)
+        assert np.array_equal(oracle.to_float(vdt, aq), a)
+        wf = oracle.to_float(dtype, w).astype(np.float64)
+        want = float(np.sum(wf * a.astype(np.float64)))
+        scale = float(np.sum(np.abs(wf * a.astype(np.float64))))
+        got = oracle.vec_dot(dtype, n, w, aq)
+        assert abs(got - want) <= 2e-6 * scale
+        assert abs(float(oracle.matmul(dtype, a.reshape(1, n), w, 1)[0, 0]) - got) <= 1e-6 * scale
