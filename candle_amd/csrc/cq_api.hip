@@ -8,15 +8,17 @@ namespace {
 
 inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
+// weight formats of the matmul-family entry points: the five with matrix-core kernels and five more that take the
+// matvec kernels at any row count (cq_has_mfma)
 inline bool matmul_weight_dtype(int dt) {
-    return dt == CQ_Q4_0 || dt == CQ_Q8_0 || dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K;
+    return cq_has_mfma(dt) || dt == CQ_Q4_1 || dt == CQ_Q5_0 || dt == CQ_Q5_1 || dt == CQ_Q2K || dt == CQ_Q3K;
 }
 
+// formats cq_quantize produces
+inline bool quantize_dtype(int dt) { return cq_has_mfma(dt) || dt == CQ_Q8K; }
 inline bool block_dtype(int dt) { return matmul_weight_dtype(dt) || dt == CQ_Q8K; }
 // every GGUF block format can be stored and dequantized; the matmul-family and quantize entry points take fewer
-inline bool storage_dtype(int dt) {
-    return block_dtype(dt) || dt == CQ_Q4_1 || dt == CQ_Q5_0 || dt == CQ_Q5_1 || dt == CQ_Q8_1 || dt == CQ_Q2K || dt == CQ_Q3K;
-}
+inline bool storage_dtype(int dt) { return block_dtype(dt) || dt == CQ_Q8_1; }
 
 inline bool float_dtype(int dt) { return dt == CQ_F32 || dt == CQ_F16 || dt == CQ_BF16; }
 
@@ -120,7 +122,7 @@ int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stre
 }
 
 int cq_quantize(int dtype, const float *x_dev, void *blocks_dev, int64_t elem_count, void *stream) {
-    if (!block_dtype(dtype)) return CQ_ERR_DTYPE;
+    if (!quantize_dtype(dtype)) return CQ_ERR_DTYPE;
     if (elem_count < 0 || elem_count % cq_block_size(dtype) != 0) return CQ_ERR_SHAPE;
     if (elem_count == 0) return CQ_OK;
     if (!x_dev || !blocks_dev) return CQ_ERR_NULL;
@@ -193,7 +195,9 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     if (workspace_bytes < cq_qmatmul_workspace_bytes(w_dtype, m, k, n)) return CQ_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     // decode: one kernel quantizes the activations into LDS and streams W (no scratch traffic)
-    if (m <= 2) return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
+    // (the formats without a matrix-core kernel have the fused instance for f32 activations only)
+    if (m <= 2 && (cq_has_mfma(w_dtype) || x_dtype == CQ_F32))
+        return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
     // 3..8 rows: every workgroup re-quantizing all rows costs more than one small kernel that does it once
     if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) {
         if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;

@@ -4,13 +4,15 @@
 //   Q4_K / Q5_K: one 64-element group g of a super-block (32 bytes of qs = two 16-byte loads, the
 //                matching qh bytes for Q5_K) + the 16-byte block header; 4 lanes per super-block
 //   Q6_K       : 16 `l` positions of one 128-element half (3 x 16 bytes); 4 lanes per super-block
-//   Q4_0 / Q8_0: one 32-element block
+//   Q4_0 / Q8_0: one 32-element block (also Q4_1, Q5_0, Q5_1)
+//   Q2_K / Q3_K: the 16 bytes qs[32h + 16c, +16) of a super-block = 16 positions of the four 32-element quarters of
+//                half h, the element set of a Q6_K unit; 4 lanes per super-block
 // so a wave64 step covers 16 super-blocks (4096 elements) of a K-quant row or 64 blocks (2048
 // elements) of a Q4_0 / Q8_0 row.  For each format Fmt<DT> gives the raw weight registers (W), the
 // activation registers (A) and the dot product of one unit: exact integer arithmetic inside the
 // unit, one f32 scaling at the end, following the CPU vec_dot of
 // candle-core/src/quantized/k_quants.rs (Q4_0 :294-311, Q8_0 :720-738, Q4_K :1460-1540,
-// Q5_K :1714-1801, Q6_K :2035-2092).
+// Q5_K :1714-1801, Q6_K :2035-2092, Q4_1 :323-351, Q5_0 :434-455, Q5_1 :530-562, Q2_K :838-886, Q3_K :1068-1187).
 #pragma once
 #include "cq_device.h"
 
@@ -239,6 +241,79 @@ struct FmtQ6Narrow {
     }
 };
 
+// ---- Q2_K / Q3_K: unit (h, c) = qs bytes [32h + 16c, +16), i.e. elements 128h + 32i + 16c + [0,16) for the four
+// quarters i (bit pairs 2i, 2i + 1 of each byte) with scale index 8h + 2i + c — the element set and activation
+// registers of a Q6_K unit (k_quants.rs:1013-1049, 1369-1421).
+template <> struct Fmt<CQ_Q2K> {
+    static constexpr int UE = 64, UPB = 4;
+    struct W { u32x4 qs; u32x2 sc; uint32_t dd; };
+    typedef Fmt<CQ_Q6K>::A A;
+    static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *blk = row + (u >> 2) * 84;
+        w.qs = ld_u<u32x4>(blk + 16 + 16 * (u & 3));
+        w.sc = ld_u<u32x2>(blk + 8 * ((u >> 1) & 1));       // the 8 scale / min bytes of this half
+        w.dd = ld_u<uint32_t>(blk + 80);                     // d | dmin << 16
+    }
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { Fmt<CQ_Q6K>::load_a(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int u) {
+        const int c = u & 1;
+        const uint32_t s0 = w.sc.x >> (8 * c), s1 = w.sc.y >> (8 * c);
+        const uint32_t scb[4] = {s0 & 0xff, (s0 >> 16) & 0xff, s1 & 0xff, (s1 >> 16) & 0xff};
+        const uint32_t q[4] = {w.qs.x, w.qs.y, w.qs.z, w.qs.w};
+        int isum = 0, summs = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t A4[4] = {a.a[i].x, a.a[i].y, a.a[i].z, a.a[i].w};
+            int t = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) t = sdot4((q[j] >> (2 * i)) & 0x03030303u, A4[j], t);
+            isum += __mul24((int)(scb[i] & 0xf), t);
+            summs += __mul24((int)(scb[i] >> 4), a.bs[i]);
+        }
+        const float d = h2f(w.dd), dmin = h2f(w.dd >> 16);
+        return a.d8 * (d * (float)isum - dmin * (float)summs);
+    }
+};
+
+template <> struct Fmt<CQ_Q3K> {
+    static constexpr int UE = 64, UPB = 4;
+    struct W { u32x4 qs, hm; uint32_t s0, s1, s2, d; };
+    typedef Fmt<CQ_Q6K>::A A;
+    static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *blk = row + (u >> 2) * 110;
+        w.hm = ld_u<u32x4>(blk + 16 * (u & 1));              // hmask[16c, +16)
+        w.qs = ld_u<u32x4>(blk + 32 + 16 * (u & 3));
+        w.s0 = ld_u<uint32_t>(blk + 96);
+        w.s1 = ld_u<uint32_t>(blk + 100);
+        w.s2 = ld_u<uint32_t>(blk + 104);
+        w.d = ld_u<uint16_t>(blk + 108);
+    }
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { Fmt<CQ_Q6K>::load_a(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int u) {
+        const int h = (u >> 1) & 1, c = u & 1;
+        // the eight 6-bit scales of half h as two dwords of bytes (k_quants.rs:1148-1156): low nibbles from
+        // scales[0..8) (half 0) or their high nibbles (half 1), bits 4-5 from the bit pairs of scales[8..12)
+        const uint32_t t2 = w.s2 >> (4 * h);
+        const uint32_t e0 = ((w.s0 >> (4 * h)) & 0x0f0f0f0fu) | ((t2 & 0x03030303u) << 4);
+        const uint32_t e1 = ((w.s1 >> (4 * h)) & 0x0f0f0f0fu) | (((t2 >> 2) & 0x03030303u) << 4);
+        const uint32_t x0 = e0 >> (8 * c), x1 = e1 >> (8 * c);
+        const int sc[4] = {(int)(x0 & 0xff) - 32, (int)((x0 >> 16) & 0xff) - 32, (int)(x1 & 0xff) - 32, (int)((x1 >> 16) & 0xff) - 32};
+        const uint32_t q[4] = {w.qs.x, w.qs.y, w.qs.z, w.qs.w};
+        const uint32_t hm[4] = {w.hm.x >> (4 * h), w.hm.y >> (4 * h), w.hm.z >> (4 * h), w.hm.w >> (4 * h)};
+        int S = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t A4[4] = {a.a[i].x, a.a[i].y, a.a[i].z, a.a[i].w};
+            // value = (2 bits | hmask bit << 2) - 4: the -4 goes through the 16-element sum
+            int t = -4 * a.bs[i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) t = sdot4(((q[j] >> (2 * i)) & 0x03030303u) | (((hm[j] >> i) & 0x01010101u) << 2), A4[j], t);
+            S += __mul24(sc[i], t);
+        }
+        return (h2f(w.d) * a.d8) * (float)S;
+    }
+};
+
 // The unit decomposition a kernel instance uses: rows of one wave step (SINGLE) and register-blocked instances
 // keep Fmt<DT>.
 template <int DT, int NB, bool SINGLE> struct UnitFmt { typedef Fmt<DT> type; };
@@ -299,6 +374,83 @@ template <> struct Fmt<CQ_Q8_0> {
         s = sdot4(w.q1.x, a.a1.x, s); s = sdot4(w.q1.y, a.a1.y, s);
         s = sdot4(w.q1.z, a.a1.z, s); s = sdot4(w.q1.w, a.a1.w, s);
         return (float)s * h2f(w.d) * a.d8;
+    }
+};
+
+// ---- Q4_1 / Q5_0 / Q5_1: one 32-element block per unit, Q8_0 activation registers.  The CPU path quantizes the
+// activations of Q4_1 / Q5_1 to Q8_1, whose qs and d are those of Q8_0 and whose s = f16(f16(sum) * d)
+// (k_quants.rs:770-799) follows from the {d, sum} pair the Q8_0 scratch holds.
+__device__ __forceinline__ float q8_1_s(const A0 &a) { return h2f(f2h_bits(h2f(f2h_bits((float)a.s8)) * a.d8)); }
+
+// four bits -> bit 4 of four bytes
+__device__ __forceinline__ uint32_t spread4_to_bit4(uint32_t b) { return (((b & 0xfu) * 0x00204081u) & 0x01010101u) << 4; }
+
+template <> struct Fmt<CQ_Q4_1> {
+    static constexpr int UE = 32, UPB = 1;
+    struct W { u32x4 qs; uint32_t dm; };
+    typedef A0 A;
+    static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *blk = row + u * 20;
+        w.dm = ld_u<uint32_t>(blk);                          // d | m << 16
+        w.qs = ld_u<u32x4>(blk + 4);
+    }
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
+        const uint32_t M4 = 0x0f0f0f0fu;
+        int s = 0;
+        s = sdot4(w.qs.x & M4, a.a0.x, s); s = sdot4(w.qs.y & M4, a.a0.y, s);
+        s = sdot4(w.qs.z & M4, a.a0.z, s); s = sdot4(w.qs.w & M4, a.a0.w, s);
+        s = sdot4((w.qs.x >> 4) & M4, a.a1.x, s); s = sdot4((w.qs.y >> 4) & M4, a.a1.y, s);
+        s = sdot4((w.qs.z >> 4) & M4, a.a1.z, s); s = sdot4((w.qs.w >> 4) & M4, a.a1.w, s);
+        return (float)s * h2f(w.dm) * a.d8 + h2f(w.dm >> 16) * q8_1_s(a);
+    }
+};
+
+// unsigned 5-bit values of a Q5_0 / Q5_1 block: qh bit j belongs to element j (low nibbles), bit j + 16 to element j + 16
+__device__ __forceinline__ int dot_q5(const u32x4 &qs, uint32_t qh, const A0 &a, int s) {
+    const uint32_t M4 = 0x0f0f0f0fu;
+    const uint32_t q[4] = {qs.x, qs.y, qs.z, qs.w};
+    const uint32_t lo[4] = {a.a0.x, a.a0.y, a.a0.z, a.a0.w};
+    const uint32_t hi[4] = {a.a1.x, a.a1.y, a.a1.z, a.a1.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        s = sdot4((q[i] & M4) | spread4_to_bit4(qh >> (4 * i)), lo[i], s);
+        s = sdot4(((q[i] >> 4) & M4) | spread4_to_bit4(qh >> (16 + 4 * i)), hi[i], s);
+    }
+    return s;
+}
+
+template <> struct Fmt<CQ_Q5_0> {
+    static constexpr int UE = 32, UPB = 1;
+    struct W { u32x4 qs; uint32_t qh, d; };
+    typedef A0 A;
+    static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *blk = row + u * 22;
+        w.d = ld_u<uint16_t>(blk);
+        w.qh = ld_u<uint32_t>(blk + 2);
+        w.qs = ld_u<u32x4>(blk + 6);
+    }
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
+        const int s = dot_q5(w.qs, w.qh, a, -16 * a.s8);    // sum((q - 16) * y) = sum(q * y) - 16 * sum(y)
+        return (float)s * h2f(w.d) * a.d8;
+    }
+};
+
+template <> struct Fmt<CQ_Q5_1> {
+    static constexpr int UE = 32, UPB = 1;
+    struct W { u32x4 qs; uint32_t dm, qh; };
+    typedef A0 A;
+    static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
+        const uint8_t *blk = row + u * 24;
+        w.dm = ld_u<uint32_t>(blk);                          // d | m << 16
+        w.qh = ld_u<uint32_t>(blk + 4);
+        w.qs = ld_u<u32x4>(blk + 8);
+    }
+    static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
+    static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
+        const int s = dot_q5(w.qs, w.qh, a, 0);
+        return (float)s * h2f(w.dm) * a.d8 + h2f(w.dm >> 16) * q8_1_s(a);
     }
 };
 

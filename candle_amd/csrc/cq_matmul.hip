@@ -871,7 +871,7 @@ int cq_qmm_splits(int64_t k, int64_t n, int64_t rows) {
 // 23.4 / 27.5 and 18.3 / 20.8 / 23.6 / 29.9, the 32-row MFMA tile 20.7 and 22.3 at any of them, 21.3 / 23.0 at 16 / 32 rows).
 constexpr int CQ_Q4K_MFMA_MIN_ROWS = 6;
 bool cq_use_mfma(int w_dtype, int64_t rows, int64_t k) {
-    if (k % 256) return false;
+    if (k % 256 || !cq_has_mfma(w_dtype)) return false;
     return rows > CQ_MATVEC_MAX_ROWS || (w_dtype == CQ_Q4K && rows >= CQ_Q4K_MFMA_MIN_ROWS);
 }
 

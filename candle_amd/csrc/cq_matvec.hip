@@ -655,6 +655,15 @@ int launch_nb(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_
 template <int DT, int SRC>
 int launch_rows(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst,
                 hipStream_t s) {
+    // The formats without a matrix-core kernel have the fused instances QMatMul::forward uses (f32 activations, one or
+    // two rows); everything else of theirs goes through the pre-quantized scratch.
+    if constexpr (!cq_has_mfma(DT) && SRC != SRC_SCRATCH) {
+        if constexpr (SRC == CQ_F32) {
+            if (rows == 1) return launch_nb<DT, 1, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            if (rows == 2) return launch_nb<DT, 2, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        }
+        return CQ_ERR_RANGE;
+    } else
     switch (rows) {
         case 1: return launch_nb<DT, 1, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
         case 2: return launch_nb<DT, 2, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
@@ -677,6 +686,11 @@ int launch_dt(int w_dtype, const void *w, const ActSrc &src, void *dst, int dst_
         case CQ_Q4K: return launch_rows<CQ_Q4K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
         case CQ_Q5K: return launch_rows<CQ_Q5K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
         case CQ_Q6K: return launch_rows<CQ_Q6K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q4_1: return launch_rows<CQ_Q4_1, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q5_0: return launch_rows<CQ_Q5_0, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q5_1: return launch_rows<CQ_Q5_1, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q2K: return launch_rows<CQ_Q2K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case CQ_Q3K: return launch_rows<CQ_Q3K, SRC>(w, src, dst, dst_dtype, k, n, rows, stride_dst, s);
     }
     return CQ_ERR_DTYPE;
 }
@@ -1080,6 +1094,11 @@ int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, 
         case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w, x, out, ps, k, n, s);
         case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w, x, out, ps, k, n, s);
         case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w, x, out, ps, k, n, s);
+        case CQ_Q4_1: return launch_moe_pairs<CQ_Q4_1>(w, x, out, ps, k, n, s);
+        case CQ_Q5_0: return launch_moe_pairs<CQ_Q5_0>(w, x, out, ps, k, n, s);
+        case CQ_Q5_1: return launch_moe_pairs<CQ_Q5_1>(w, x, out, ps, k, n, s);
+        case CQ_Q2K: return launch_moe_pairs<CQ_Q2K>(w, x, out, ps, k, n, s);
+        case CQ_Q3K: return launch_moe_pairs<CQ_Q3K>(w, x, out, ps, k, n, s);
     }
     return CQ_ERR_DTYPE;
 }
@@ -1096,6 +1115,11 @@ int cq_moe_pairs_swiglu_launch(int w_dtype, const void *w_gate, const void *w_up
         case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w_gate, x, out, ps, k, n, s, true, off);
         case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w_gate, x, out, ps, k, n, s, true, off);
         case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q4_1: return launch_moe_pairs<CQ_Q4_1>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q5_0: return launch_moe_pairs<CQ_Q5_0>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q5_1: return launch_moe_pairs<CQ_Q5_1>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q2K: return launch_moe_pairs<CQ_Q2K>(w_gate, x, out, ps, k, n, s, true, off);
+        case CQ_Q3K: return launch_moe_pairs<CQ_Q3K>(w_gate, x, out, ps, k, n, s, true, off);
     }
     return CQ_ERR_DTYPE;
 }
@@ -1152,6 +1176,11 @@ int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_
         case CQ_Q4K: return launch_moe_chunks<CQ_Q4K>(w, scratch, rows_alloc, out, mc, k, n, s);
         case CQ_Q5K: return launch_moe_chunks<CQ_Q5K>(w, scratch, rows_alloc, out, mc, k, n, s);
         case CQ_Q6K: return launch_moe_chunks<CQ_Q6K>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q4_1: return launch_moe_chunks<CQ_Q4_1>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q5_0: return launch_moe_chunks<CQ_Q5_0>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q5_1: return launch_moe_chunks<CQ_Q5_1>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q2K: return launch_moe_chunks<CQ_Q2K>(w, scratch, rows_alloc, out, mc, k, n, s);
+        case CQ_Q3K: return launch_moe_chunks<CQ_Q3K>(w, scratch, rows_alloc, out, mc, k, n, s);
     }
     return CQ_ERR_DTYPE;
 }

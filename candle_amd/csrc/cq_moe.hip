@@ -192,7 +192,7 @@ int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_
 
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
-    const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
+    const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && cq_has_mfma(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
     if (a.w_b && !mfma) {
         // only the MFMA path shares its grouping pass and quantized activations between two weight tensors
         MoeArgs one = a;
@@ -252,6 +252,11 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
         case CQ_Q4K: return launch_moe_matvec<CQ_Q4K>(a, av, offsets, pin, pout, pscale, s);
         case CQ_Q5K: return launch_moe_matvec<CQ_Q5K>(a, av, offsets, pin, pout, pscale, s);
         case CQ_Q6K: return launch_moe_matvec<CQ_Q6K>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q4_1: return launch_moe_matvec<CQ_Q4_1>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q5_0: return launch_moe_matvec<CQ_Q5_0>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q5_1: return launch_moe_matvec<CQ_Q5_1>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q2K: return launch_moe_matvec<CQ_Q2K>(a, av, offsets, pin, pout, pscale, s);
+        case CQ_Q3K: return launch_moe_matvec<CQ_Q3K>(a, av, offsets, pin, pout, pscale, s);
     }
     return CQ_ERR_DTYPE;
 }

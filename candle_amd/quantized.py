@@ -65,7 +65,11 @@ _BLOCK_SIZE = {d: (1 if d in (GgmlDType.F32, GgmlDType.F16, GgmlDType.BF16) else
 _KERNEL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q8K)
 # ... and the ones that can be stored and dequantized only
 _DEQUANT_DTYPES = _KERNEL_DTYPES + (GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q8_1, GgmlDType.Q2K, GgmlDType.Q3K)
-_MATMUL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
+# QMatMul weights: the first five also have matrix-core (prefill) kernels, the others take the matvec kernels at any row count
+_MATMUL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K,
+                  GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q2K, GgmlDType.Q3K)
+# expert formats of the two MoE entry points: the reference's (cuda.rs:543-548 + moe.rs:210-215) plus Q4_0
+_MOE_DTYPES = (GgmlDType.Q8_0, GgmlDType.Q2K, GgmlDType.Q3K, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q4_0)
 _TORCH_TO_CQ = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 30}
 _TORCH_PLAIN = {GgmlDType.F32: torch.float32, GgmlDType.F16: torch.float16, GgmlDType.BF16: torch.bfloat16}
 
@@ -319,7 +323,7 @@ class QTensor:
         """mod.rs:758-784 -> cuda.rs:587-622.  self [E, n, k]; x [batch, topk or 1, k] f32; ids [batch, topk] u32."""
         if not (x.is_cuda and ids.is_cuda):
             raise RuntimeError("Non-cuda indexed_moe_forward is not implemented!")
-        if self.dtype() not in (GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q4_0):
+        if self.dtype() not in _MOE_DTYPES:
             raise ValueError(f"The given quantized dtype {self.dtype().name} is not supported for indexed_moe_forward!")
         if len(self._shape) != 3 or x.dim() != 3 or ids.dim() != 2:
             raise ValueError("indexed_moe_forward expects weights [E,n,k], x [batch, topk or 1, k], ids [batch, topk]")
@@ -414,8 +418,8 @@ def moe_gemm_gguf(input: torch.Tensor, weights: QTensor, topk_weights: Optional[
         size_m *= topk
     E, size_n, size_k1 = weights.shape()
     assert size_k == size_k1, f"input {size_k} and weight {size_k1} last dim mismatch!"
-    if weights.dtype() not in (GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q4_0):
-        raise ValueError("moe_gemm_gguf `ISQ` only accept q4_0, q4k, q5k, q6k or q8_0 weights!")
+    if weights.dtype() not in _MOE_DTYPES:
+        raise ValueError("moe_gemm_gguf `ISQ` only accept q2k, q3k, q4k, q5k, q6k or q8_0 weights!")
     assert size_k % 8 == 0, "size_k must divisible by 8"
     for name, t in (("sorted_token_ids", sorted_token_ids), ("experts_ids", experts_ids)):
         if not t.is_cuda:

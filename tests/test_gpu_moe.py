@@ -14,8 +14,8 @@ pytestmark = pytest.mark.gpu
 
 TOL = 1e-3
 TIGHT = 2e-6
-WDTYPES = [oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q4_0]
-NAMES = {oracle.Q4_0: "q4_0", oracle.Q8_0: "q8_0", oracle.Q4K: "q4k", oracle.Q5K: "q5k", oracle.Q6K: "q6k"}
+WDTYPES = [oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q4_0, oracle.Q2K, oracle.Q3K]
+NAMES = {oracle.Q4_0: "q4_0", oracle.Q8_0: "q8_0", oracle.Q4K: "q4k", oracle.Q5K: "q5k", oracle.Q6K: "q6k", oracle.Q2K: "q2k", oracle.Q3K: "q3k"}
 
 
 def make_experts(dtype, E, n, k, seed):

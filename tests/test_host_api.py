@@ -62,7 +62,7 @@ def test_check_shape_errors():
 
 def test_argument_validation_codes_without_gpu():
     L = _lib.lib()
-    Q4K, Q2K, Q8K = 12, 10, 15
+    Q4K, Q8_1, Q8K = 12, 9, 15
     OK, DTYPE, SHAPE, ALIGN, NULL, WS, RANGE = 0, -1, -2, -3, -4, -5, -6
     # scratch sizes: K-quants: qs + d + bsums sections, each rounded up to 256 bytes
     assert L.cq_act_scratch_bytes(Q4K, 4096, 1) == 4096 + 256 + 512
@@ -73,7 +73,7 @@ def test_argument_validation_codes_without_gpu():
     assert L.cq_quantize_act(Q4K, 16, 0, 256, 4000, 1, None) == SHAPE
     assert L.cq_quantize_act(Q4K, 8, 0, 256, 4096, 1, None) == ALIGN           # x must be 16-byte aligned
     assert L.cq_quantize_act(Q4K, 16, 12, 256, 4096, 1, None) == DTYPE         # activations must be f32/f16/bf16
-    assert L.cq_matvec(Q2K, 16, 256, 16, 0, 256, 4, 1, 4, None) == DTYPE
+    assert L.cq_matvec(Q8_1, 16, 256, 16, 0, 256, 4, 1, 4, None) == DTYPE      # Q8_1 is an activation format
     assert L.cq_matvec(Q8K, 16, 256, 16, 0, 256, 4, 1, 4, None) == DTYPE       # Q8K is not a matmul weight type
     assert L.cq_matvec(Q4K, 16, 256, 16, 0, 256, 4, 9, 4, None) == RANGE       # more than CQ_MATVEC_MAX_ROWS
     assert L.cq_matvec(Q4K, 16, 256, 16, 0, 256, 4, 1, 3, None) == SHAPE       # stride_dst < n
