@@ -14,8 +14,6 @@ inline bool matmul_weight_dtype(int dt) {
     return cq_has_mfma(dt) || dt == CQ_Q4_1 || dt == CQ_Q5_0 || dt == CQ_Q5_1 || dt == CQ_Q2K || dt == CQ_Q3K;
 }
 
-// formats cq_quantize produces
-inline bool quantize_dtype(int dt) { return cq_has_mfma(dt) || dt == CQ_Q8K; }
 inline bool block_dtype(int dt) { return matmul_weight_dtype(dt) || dt == CQ_Q8K; }
 // every GGUF block format can be stored and dequantized; the matmul-family and quantize entry points take fewer
 inline bool storage_dtype(int dt) { return block_dtype(dt) || dt == CQ_Q8_1; }
@@ -122,7 +120,7 @@ int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stre
 }
 
 int cq_quantize(int dtype, const float *x_dev, void *blocks_dev, int64_t elem_count, void *stream) {
-    if (!quantize_dtype(dtype)) return CQ_ERR_DTYPE;
+    if (!storage_dtype(dtype)) return CQ_ERR_DTYPE;
     if (elem_count < 0 || elem_count % cq_block_size(dtype) != 0) return CQ_ERR_SHAPE;
     if (elem_count == 0) return CQ_OK;
     if (!x_dev || !blocks_dev) return CQ_ERR_NULL;

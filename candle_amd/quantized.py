@@ -61,9 +61,8 @@ _BLOCK_SIZE = {d: (1 if d in (GgmlDType.F32, GgmlDType.F16, GgmlDType.BF16) else
                    32 if d in (GgmlDType.Q4_0, GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q8_0, GgmlDType.Q8_1)
                    else 256) for d in GgmlDType}
 
-# block formats the HIP kernels implement
+# every block format can be stored, quantized, dequantized and used as an embedding table
 _KERNEL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q8K)
-# ... and the ones that can be stored and dequantized only
 _DEQUANT_DTYPES = _KERNEL_DTYPES + (GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q8_1, GgmlDType.Q2K, GgmlDType.Q3K)
 # QMatMul weights: the first five also have matrix-core (prefill) kernels, the others take the matvec kernels at any row count
 _MATMUL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K,
@@ -162,7 +161,7 @@ class QStorage:
     def quantize(self, src: torch.Tensor) -> None:
         """QCudaStorage::quantize (cuda.rs:704-725); runs GgmlType::from_float on the GPU."""
         _require_cuda(src, "src")
-        if self._dtype not in _KERNEL_DTYPES:
+        if self._dtype not in _DEQUANT_DTYPES:
             raise NotImplementedError(f"quantize is not implemented for {self._dtype.name}")
         src = src.to(torch.float32).contiguous().reshape(-1)
         if src.numel() // self.block_size() * self._dtype.type_size() != self._data.numel():

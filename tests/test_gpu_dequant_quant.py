@@ -15,7 +15,7 @@ from tests.util import bits_equal_or_both_nan, normal
 pytestmark = pytest.mark.gpu
 
 DTYPES = [oracle.Q4_0, oracle.Q8_0, oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q8K]
-# formats that exist on the GPU as storage only (dequantize, no matmul / quantize kernels)
+# the remaining block formats of GgmlDType
 STORAGE_DTYPES = [oracle.Q4_1, oracle.Q5_0, oracle.Q5_1, oracle.Q8_1, oracle.Q2K, oracle.Q3K]
 NAMES = {oracle.Q4_0: "q4_0", oracle.Q8_0: "q8_0", oracle.Q4K: "q4k", oracle.Q5K: "q5k", oracle.Q6K: "q6k", oracle.Q8K: "q8k",
          oracle.Q4_1: "q4_1", oracle.Q5_0: "q5_0", oracle.Q5_1: "q5_1", oracle.Q8_1: "q8_1", oracle.Q2K: "q2k", oracle.Q3K: "q3k"}
@@ -73,7 +73,7 @@ def test_dequantize_empty_and_errors():
     assert L.cq_dequantize(int(ca.GgmlDType.Q4K), None, None, 0, 0, None) == 0          # empty is ok
     assert L.cq_dequantize(int(ca.GgmlDType.Q4K), None, None, 100, 0, None) == -2        # not a block multiple
     assert L.cq_dequantize(int(ca.GgmlDType.F16), None, None, 256, 0, None) == -1        # not a block format
-    assert L.cq_quantize(int(ca.GgmlDType.Q2K), None, None, 256, None) == -1             # storage-only format: no quantizer
+    assert L.cq_quantize(int(ca.GgmlDType.F16), None, None, 256, None) == -1             # not a block format
     assert L.cq_dequantize(int(ca.GgmlDType.Q4K), None, None, 256, 0, None) == -4        # NULL
 
 
@@ -102,7 +102,7 @@ def _quant_inputs():
     yield "edge", z
 
 
-@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("dtype", DTYPES + STORAGE_DTYPES, ids=lambda d: NAMES[d])
 def test_quantize_bytes_match_cpu_from_float(dtype):
     for name, x in _quant_inputs():
         want = oracle.from_float(dtype, x)
