@@ -769,6 +769,17 @@ int launch_fused_dt(int w_dtype, const void *w, const ActSrc &src, void *dst, in
         case CQ_Q5K: return launch_fused1<CQ_Q5K, PRO, EPI>(w, src, dst, k, n, s, fz);
         case CQ_Q6K: return launch_fused1<CQ_Q6K, PRO, EPI>(w, src, dst, k, n, s, fz);
     }
+    // The formats without a matrix-core kernel have the three fusions a decoder step cannot do without: the rms_norm
+    // prologue, and the residual epilogue with and without the silu * up prologue.
+    if constexpr ((PRO == PRO_NORM && EPI == EPI_NONE) || ((PRO == PRO_NONE || PRO == PRO_SILU) && EPI == EPI_RESID)) {
+        switch (w_dtype) {
+            case CQ_Q4_1: return launch_fused1<CQ_Q4_1, PRO, EPI>(w, src, dst, k, n, s, fz);
+            case CQ_Q5_0: return launch_fused1<CQ_Q5_0, PRO, EPI>(w, src, dst, k, n, s, fz);
+            case CQ_Q5_1: return launch_fused1<CQ_Q5_1, PRO, EPI>(w, src, dst, k, n, s, fz);
+            case CQ_Q2K: return launch_fused1<CQ_Q2K, PRO, EPI>(w, src, dst, k, n, s, fz);
+            case CQ_Q3K: return launch_fused1<CQ_Q3K, PRO, EPI>(w, src, dst, k, n, s, fz);
+        }
+    }
     return CQ_ERR_DTYPE;
 }
 }  // namespace

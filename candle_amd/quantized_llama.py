@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .quantized import GgmlDType, QStorage, QTensor
+from .quantized import GgmlDType, QStorage, QTensor, _MATMUL_DTYPES
 
 
 @dataclasses.dataclass
@@ -220,7 +220,7 @@ class ModelWeights:
             for name in _LAYER_ORDER:
                 dtypes[f"blk.{li}.{name}"] = GgmlDType(tensors[f"blk.{li}.{name}"][0])
         for key, dt in dtypes.items():
-            if dt not in (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K):
+            if dt not in _MATMUL_DTYPES:
                 raise NotImplementedError(f"{key}: no matmul kernel for {dt.name} weights")
         plan = self._alloc(dtypes)
         for li, name, off, nb, n, k in plan:
@@ -392,12 +392,16 @@ class ModelWeights:
         ck = _lib.check
         qk, v, att, gu, part, planes = self.qk, self.v, self.att, self.gu, self.partials, self.planes
         kq = (GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K)
+        # formats with every decode fusion; the others (Q4_1, Q5_0, Q5_1, Q2K, Q3K) have the rms_norm prologue and the residual
+        # epilogue only: no paired launches, no attention merge inside attention_wo, no K-split planes anywhere in the model
+        full = kq + (GgmlDType.Q4_0, GgmlDType.Q8_0)
+        all_full = all(w.dtype in full for lw in self.layers for w in lw.w.values()) and self.output.dtype in full
         cur = self.x.data_ptr()                                    # the residual row
         pending = 0                                                # planes of the previous feed_forward_w2 not yet added to it
         ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, cur, 1, cfg.hidden, cfg.vocab, part.data_ptr(), sp))
 
         def one_step(w: _W) -> bool:
-            return w.k <= (4096 if w.dtype in kq else 2048)
+            return w.k <= (4096 if w.dtype in kq + (GgmlDType.Q2K, GgmlDType.Q3K) else 2048)
 
         def norm_mm(w: _W, n: int, norm_w: torch.Tensor, dst_ptr: int):
             if pending:
@@ -435,7 +439,7 @@ class ModelWeights:
             q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
             # rope, cache append, attention and the merge of the key splits in one kernel          :217-261
             wo = w["attention_wo"]
-            merge_in_wo = qd <= (4096 if wo.dtype in kq else 2048) and (cfg.head_dim & (cfg.head_dim - 1)) == 0
+            merge_in_wo = wo.dtype in full and qd <= (4096 if wo.dtype in kq else 2048) and (cfg.head_dim & (cfg.head_dim - 1)) == 0
             ck("cq_nn_attention_decode", L.cq_nn_attention_decode(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
                                                                   self.cos.data_ptr(), self.sin.data_ptr(),
                                                                   None if merge_in_wo else att.data_ptr(), pos_dev_ptr, pos,
@@ -455,9 +459,9 @@ class ModelWeights:
             # the consumers of this layer's residual row: the next layer's q / k / v projections, or the output head
             nxt = self.layers[li + 1].w if li + 1 < len(self.layers) else None
             consumers = [nxt["attention_wq"], nxt["attention_wk"], nxt["attention_wv"]] if nxt else [self.output]
-            n_split = L.cq_nn_qmatmul_split_planes(int(w2.dtype), w2.k) if self.split_w2 and cfg.hidden <= 4096 and \
+            n_split = L.cq_nn_qmatmul_split_planes(int(w2.dtype), w2.k) if self.split_w2 and all_full and cfg.hidden <= 4096 and \
                 all(one_step(c) for c in consumers) else 0
-            if w1.dtype == w3.dtype and one_step(w1):
+            if w1.dtype == w3.dtype and w1.dtype in full and one_step(w1):
                 # h = silu(w1 xn) * (w3 xn) straight out of the paired-row matvec                    :56-63
                 ck("cq_nn_qmatmul_norm_swiglu", L.cq_nn_qmatmul_norm_swiglu(int(w1.dtype), w1.ptr, w3.ptr, cur, part.data_ptr(),
                                                                             lw.ffn_norm.data_ptr(), cfg.rms_eps, self.h.data_ptr(), cfg.hidden,

@@ -18,8 +18,11 @@
  *     rely on the 512-element tail padding the CUDA backend adds
  *     (candle-core/src/quantized/cuda.rs:624-637,989-1008);
  *   - activation quantization follows candle's CPU path bit for bit (Q8_K blocks for K-quants,
- *     Q8_0 blocks for Q4_0/Q8_0: k_quants.rs:2320-2358, 658-687), so results match
- *     QMatMul::forward on the CPU up to f32 summation order.
+ *     Q8_0 blocks for Q4_0/Q5_0/Q8_0, Q8_1 blocks for Q4_1/Q5_1: k_quants.rs:2320-2358, 658-687, 770-799), so
+ *     results match QMatMul::forward on the CPU up to f32 summation order;
+ *   - weight formats of the matmul-family entry points (cq_quantize_act, cq_matvec, cq_matmul, cq_qmatmul_forward,
+ *     the MoE entry points): Q4_0, Q8_0, Q4K, Q5K, Q6K, which also have matrix-core kernels, and Q4_1, Q5_0, Q5_1,
+ *     Q2K, Q3K, which take the matvec kernels at any row count (eight activation rows per pass over the weights).
  */
 #ifndef CANDLE_HIP_QUANT_H
 #define CANDLE_HIP_QUANT_H
@@ -62,8 +65,8 @@ int64_t cq_storage_bytes(int dtype, int64_t elem_count);
  * QTensor::dequantize / dequantize_f16 (mod.rs:689-710; CUDA: cuda.rs:105-223,
  * candle-kernels/src/quantized.cu:780-1156).  Bit-exact with GgmlType::to_float on the CPU; the
  * f16 result equals the f32 result rounded to nearest even.
- *   dtype: every block format of GgmlDType — Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K (the matmul-family
- *   entry points and cq_quantize take Q4_0, Q8_0, Q4K, Q5K, Q6K (+ Q8K for cq_quantize) only).   out_dtype: CQ_F32 or CQ_F16.
+ *   dtype: every block format of GgmlDType — Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K.
+ *   out_dtype: CQ_F32 or CQ_F16.
  *   blocks_dev: 2-byte aligned.  out_dev: 16-byte aligned.
  * ------------------------------------------------------------------------------------------- */
 int cq_dequantize(int dtype, const void *blocks_dev, void *out_dev, int64_t elem_count, int out_dtype, void *stream);
@@ -82,19 +85,21 @@ int cq_embedding(int dtype, const void *blocks_dev, const uint32_t *ids_dev, flo
  * QTensor::quantize on a device tensor (mod.rs:543-562).  The CUDA backend copies to the host,
  * runs GgmlType::from_float and copies back (cuda.rs:704-725); here the same arithmetic runs on the
  * GPU, one thread per block, and produces the same bytes as the CPU from_float.
- *   dtype: Q4_0, Q8_0, Q4K, Q5K, Q6K, Q8K.   x_dev: f32, 4-byte aligned.  blocks_dev: 2-byte aligned.
+ *   dtype: every block format of cq_dequantize.   x_dev: f32, 4-byte aligned.  blocks_dev: 2-byte aligned.
  * ------------------------------------------------------------------------------------------- */
 int cq_quantize(int dtype, const float *x_dev, void *blocks_dev, int64_t elem_count, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Activation quantization, the first half of k_quants::matmul (k_quants.rs:2419-2428): each of
  * `rows` activation rows of length k is quantized to the weight type's VecDotType — Q8_K for
- * Q4K/Q5K/Q6K/Q8K, Q8_0 for Q4_0/Q8_0 — with the same results as the CPU from_float.  Replaces the
+ * Q2K/Q3K/Q4K/Q5K/Q6K/Q8K, Q8_0 for Q4_0/Q5_0/Q8_0 and for Q4_1/Q5_1 (whose Q8_1 blocks have the qs and d of Q8_0;
+ * their field s = f16(f16(sum) * d) is formed from the {d, sum} pair where it is used) — with the same results as
+ * the CPU from_float.  Replaces the
  * q8_1 quantize launch of the CUDA backend (cuda.rs:48-103, fast_mmvq.rs:296-303).
  *
  * Scratch layout (device-private, 256-byte aligned sections, in this order):
  *   K-quants : int8 qs[rows][k] | float d[rows][k/256] | int16 bsums[rows][k/16]
- *   Q4_0/Q8_0: int8 qs[rows][k] | struct { float d (f16-rounded); int32 sum; } ds[rows][k/32]
+ *   32-element formats: int8 qs[rows][k] | struct { float d (f16-rounded); int32 sum; } ds[rows][k/32]
  *   x_dtype: CQ_F32, CQ_F16 or CQ_BF16.  x_dev: 16-byte aligned, rows contiguous.  scratch_dev: 256-byte aligned.
  * ------------------------------------------------------------------------------------------- */
 int64_t cq_act_scratch_bytes(int w_dtype, int64_t k, int64_t rows);
@@ -114,7 +119,7 @@ int cq_matvec(int w_dtype, const void *w_dev, const void *act_scratch_dev, void 
 
 /* ---------------------------------------------------------------------------------------------
  * Prefill matmul over pre-quantized activations (any rows >= 1): more than CQ_MATVEC_MAX_ROWS rows with k a
- * multiple of 256 run on the f16 matrix cores with the converted operand tiles staged in LDS (K-quant operands are
+ * multiple of 256 (Q4_0, Q8_0, Q4K, Q5K, Q6K) run on the matrix cores with the converted operand tiles staged in LDS (K-quant operands are
  * exact integers there, Q4_0 / Q8_0 operands are rounded to f16); other shapes take 8 rows per matvec pass.
  * Counterpart of launch_mmq_gguf_<t> (candle-core/src/quantized/fast_mmq.rs:71-111, candle-kernels/src/mmq_gguf/).
  * Same buffers as cq_matvec; dst is f32.
@@ -142,7 +147,7 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
  *   out[b, t, :] = W[ids[b, t]] . x[b, input_dim1 == 1 ? 0 : t, :].
  * Up to 256 pairs each pair is its own fused matvec; beyond, pairs are grouped by expert on the device and an expert's
  * rows are streamed once per tile of 32 or 128 pairs on the matrix cores (K-quant experts; integer-exact) or once per
- * 8 pairs by the matvec kernel (Q4_0 / Q8_0 experts).
+ * 8 pairs by the matvec kernel (the other formats).  The reference takes Q2K-Q6K and Q8_0 experts (cuda.rs:543-548).
  * An id >= num_experts leaves its output row zero-filled.
  * ------------------------------------------------------------------------------------------- */
 int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk, int64_t input_dim1);

@@ -23,6 +23,15 @@ LEGACY = {"attention_wq": oracle.Q8_0, "attention_wk": oracle.Q4_0, "attention_w
           "feed_forward_w1": oracle.Q4_0, "feed_forward_w3": oracle.Q4_0, "feed_forward_w2": oracle.Q8_0, "output": oracle.Q8_0}
 
 
+# formats without a matrix-core kernel (rms_norm prologue and residual epilogue only), alone and mixed with the others
+OLD_32 = {"attention_wq": oracle.Q5_0, "attention_wk": oracle.Q5_0, "attention_wv": oracle.Q5_1, "attention_wo": oracle.Q4_1,
+          "feed_forward_w1": oracle.Q4_1, "feed_forward_w3": oracle.Q4_1, "feed_forward_w2": oracle.Q5_1, "output": oracle.Q5_0}
+Q3_K_M = {"attention_wq": oracle.Q3K, "attention_wk": oracle.Q3K, "attention_wv": oracle.Q5K, "attention_wo": oracle.Q4K,
+          "feed_forward_w1": oracle.Q3K, "feed_forward_w3": oracle.Q3K, "feed_forward_w2": oracle.Q5K, "output": oracle.Q6K}
+Q2_K_MIX = {"attention_wq": oracle.Q2K, "attention_wk": oracle.Q2K, "attention_wv": oracle.Q3K, "attention_wo": oracle.Q3K,
+            "feed_forward_w1": oracle.Q2K, "feed_forward_w3": oracle.Q3K, "feed_forward_w2": oracle.Q3K, "output": oracle.Q2K}
+
+
 def make(cfg_kw, dtypes, seed):
     from candle_amd.quantized_llama import Config, ModelWeights
     cfg = Config(**cfg_kw)
@@ -68,6 +77,30 @@ def test_q4_0_q8_0_model_decode_path():
     assert rel_l2(got, want) <= 1e-5
     loose = model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy()
     assert rel_l2(loose, want) <= 5e-2
+
+
+@pytest.mark.parametrize("dtypes", [OLD_32, Q3_K_M, Q2_K_MIX], ids=["q4_1-q5_0-q5_1", "q3_k_m", "q2k-q3k"])
+def test_models_in_the_remaining_formats(dtypes):
+    """Every matmul of these formats is integer-exact at any row count (eight rows per pass), so prefill and decode
+    both meet the tight bound; greedy decoding from a graph equals the eager steps."""
+    cfg, t, model = make(SMALL, dtypes, seed=41)
+    ref = lo.LlamaOracle(cfg, t)
+    rng = np.random.default_rng(42)
+    prompt = rng.integers(0, cfg.vocab, size=12).tolist()
+    got = model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy()
+    want = ref.forward(prompt, 0)
+    assert rel_l2(got, want) <= 1e-4
+    tok = int(np.argmax(want))
+    assert int(np.argmax(got)) == tok
+    for step in range(3):
+        got = model.forward(torch.tensor([[tok]], dtype=torch.int32), 12 + step).cpu().numpy()
+        want = ref.forward([tok], 12 + step)
+        assert rel_l2(got, want) <= 1e-4, step
+        tok = int(np.argmax(want))
+        assert int(np.argmax(got)) == tok, step
+    a = model.generate_greedy(prompt, 6, use_graph=False)["tokens"]
+    b = model.generate_greedy(prompt, 6, use_graph=True)["tokens"]
+    assert a == b and len(a) == 6
 
 
 def test_generate_greedy_graph_equals_eager_equals_oracle():
