@@ -8,11 +8,9 @@ namespace {
 
 inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// weight formats of the matmul-family entry points: the five with matrix-core kernels and five more that take the
-// matvec kernels at any row count (cq_has_mfma)
-inline bool matmul_weight_dtype(int dt) {
-    return cq_has_mfma(dt) || dt == CQ_Q4_1 || dt == CQ_Q5_0 || dt == CQ_Q5_1 || dt == CQ_Q2K || dt == CQ_Q3K;
-}
+// weight formats of the matmul-family entry points: those with matrix-core kernels (cq_has_mfma) and three more that take
+// the matvec kernels at any row count
+inline bool matmul_weight_dtype(int dt) { return cq_has_mfma(dt) || dt == CQ_Q4_1 || dt == CQ_Q5_0 || dt == CQ_Q5_1; }
 
 inline bool block_dtype(int dt) { return matmul_weight_dtype(dt) || dt == CQ_Q8K; }
 // every GGUF block format can be stored and dequantized; the matmul-family and quantize entry points take fewer
@@ -193,8 +191,8 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     if (workspace_bytes < cq_qmatmul_workspace_bytes(w_dtype, m, k, n)) return CQ_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     // decode: one kernel quantizes the activations into LDS and streams W (no scratch traffic)
-    // (the formats without a matrix-core kernel have the fused instance for f32 activations only)
-    if (m <= 2 && (cq_has_mfma(w_dtype) || x_dtype == CQ_F32))
+    // (Q4_1, Q5_0, Q5_1, Q2K, Q3K have the fused instance for f32 activations only)
+    if (m <= 2 && (cq_full_matvec(w_dtype) || x_dtype == CQ_F32))
         return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
     // 3..8 rows: every workgroup re-quantizing all rows costs more than one small kernel that does it once
     if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) {

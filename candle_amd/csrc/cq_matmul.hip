@@ -5,12 +5,12 @@
 // candle-kernels/src/mmq_gguf/).  The arithmetic follows the CPU path instead of the CUDA one:
 // activations are the Q8_K / Q8_0 quantization written by cq_quantize_act.
 //
-// Q5_K, Q6_K — integer-exact formulation on the f16 matrix cores (qmm_kernel):
+// Q5_K, Q6_K, Q2_K, Q3_K — integer-exact formulation on the f16 matrix cores (qmm_kernel):
 //   per 256-element super-block kb      S[m,n] = sum_k q8[m,k] * (sc[n,sub(k)] * q[n,k])
 //   operands are small integers held exactly in f16 (|q8| <= 128, |sc*q| <= 1953 for Q5_K),
 //   products accumulate in f32, and once per super-block
 //       acc[m,n] += d8[m,kb] * ( d[n,kb] * S[m,n] - dmin[n,kb] * M[m,n] ),
-//       M[m,n] = sum_{j<16} bsums16[m,j] * min[n,j/2]          (one extra K=16 MFMA, Q5_K only)
+//       M[m,n] = sum_{j<16} bsums16[m,j] * min[n, group j]     (one extra K=16 MFMA; Q5_K: min of sub-block j / 2, Q2_K: of group j)
 //   — the same integers the CPU vec_dot sums (k_quants.rs:1714-1801, 2035-2092).  For Q6_K
 //   the product sc*(q-32) can reach 4096, beyond the exact-integer range of f16, so it is fed as two
 //   terms: its f16 rounding and the exact remainder in {-1, 0, 1} (a second MFMA per k-slice).  This
@@ -101,9 +101,10 @@ template <> struct Stage<CQ_Q5K> {
         d = h2f(r.hdr.x);
         dmin = h2f(r.hdr.x >> 16);
     }
-    // the four sub-block mins 4 hi .. 4 hi + 3, one per byte (utils.rs:50-60)
-    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &r, int hi) {
-        return hi ? ((r.hdr.w >> 4) & 0x0f0f0f0fu) | ((r.hdr.z >> 2) & 0x30303030u) : r.hdr.z & 0x3f3f3f3fu;
+    // the mins of the 16-element groups 2 jp and 2 jp + 1 in bits 0-7 and 16-23: both the min of sub-block jp (utils.rs:50-60)
+    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &r, int jp) {
+        const uint32_t m4 = jp >= 4 ? ((r.hdr.w >> 4) & 0x0f0f0f0fu) | ((r.hdr.z >> 2) & 0x30303030u) : r.hdr.z & 0x3f3f3f3fu;
+        return ((m4 >> (8 * (jp & 3))) & 0xffu) * 0x00010001u;
     }
     template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int g, int part, uint32_t out[NW / 2]) {
         const int jh = NW == 16 ? part >> 1 : part;
@@ -146,7 +147,7 @@ template <> struct Stage<CQ_Q6K> {
         d = h2f(r.d);
         dmin = 0.0f;
     }
-    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &, int) { return 0; }
+    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &, int) { return 0; }
     // out = f16(sc * (q - 32)) (rounds odd products above 2048 to even), rem = sc * (q - 32) - out exactly
     template <int NW>
     static __device__ __forceinline__ void convert2(const Raw<NW> &r, int g, int part, uint32_t out[NW / 2], uint32_t rem[NW / 2]) {
@@ -172,6 +173,90 @@ template <> struct Stage<CQ_Q6K> {
     }
 };
 
+// Q2_K / Q3_K: element 128 h + 32 s + 16 c + i of a super-block is bit pair s of qs[32 h + 16 c + i] (Q3_K: plus bit 4 h + s of
+// hmask[16 c + i]), its 16-element group is 8 h + 2 s + c (k_quants.rs:1013-1049, 1369-1421).  Stage (kb, g), 32-element half jh:
+// h = g >> 1, s = 2 (g & 1) + jh.  Both products are small exact integers in f16: sc * q <= 45, (sc - 32) * (q - 4) within +-128.
+template <> struct Stage<CQ_Q2K> {
+    static constexpr bool KQ = true, HAS_MIN = true;
+    static constexpr int TERMS = 1;
+    template <int NW> struct Raw { u32x4 sc, q[NW / 16]; uint32_t dd; };
+    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
+        const uint8_t *blk = row + (int64_t)kb * 84;
+        const int sx = NW == 16 ? part & 1 : 0;
+        r.sc = ld_u<u32x4>(blk);
+#pragma unroll
+        for (int i = 0; i < NW / 16; i++) r.q[i] = ld_u<u32x4>(blk + 16 + 32 * (g >> 1) + 16 * (sx + i));
+        r.dd = ld_u<uint32_t>(blk + 80);
+    }
+    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &r, float &d, float &dmin) {
+        d = h2f(r.dd);
+        dmin = h2f(r.dd >> 16);
+    }
+    // mins (high nibbles of the scale bytes) of the 16-element groups 2 jp and 2 jp + 1, in bits 0-7 and 16-23
+    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &r, int jp) {
+        const uint32_t two = (r.sc[jp >> 1] >> (16 * (jp & 1))) & 0xffffu;      // scale bytes 2 jp, 2 jp + 1
+        return ((two >> 4) & 0xfu) | ((two >> 12) << 16);
+    }
+    template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int g, int part, uint32_t out[NW / 2]) {
+        const int jh = NW == 16 ? part >> 1 : part, sx = NW == 16 ? part & 1 : 0;
+        const int s = 2 * (g & 1) + jh, grp = 8 * (g >> 1) + 2 * s + sx;      // first 16-element group of this thread's weights
+#pragma unroll
+        for (int i = 0; i < NW / 4; i++) {
+            const int gi = grp + (i >> 2);
+            const float sc = (float)((r.sc[gi >> 2] >> (8 * (gi & 3))) & 0xfu);
+            const uint32_t s2 = h2_splat(sc), c2 = h2_splat(-1024.0f * sc);
+            uint32_t lo, hi;
+            bytes_to_h1024((r.q[i >> 2][i & 3] >> (2 * s)) & 0x03030303u, lo, hi);
+            out[2 * i] = pk_fma(lo, s2, c2);        // (1024 + q) * sc - 1024 * sc = sc * q, one exact rounding
+            out[2 * i + 1] = pk_fma(hi, s2, c2);
+        }
+    }
+};
+
+template <> struct Stage<CQ_Q3K> {
+    static constexpr bool KQ = true, HAS_MIN = false;
+    static constexpr int TERMS = 1;
+    template <int NW> struct Raw { u32x4 q[NW / 16], hm[NW / 16]; uint32_t s0, s1, s2, d; };
+    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
+        const uint8_t *blk = row + (int64_t)kb * 110;
+        const int sx = NW == 16 ? part & 1 : 0;
+#pragma unroll
+        for (int i = 0; i < NW / 16; i++) {
+            r.hm[i] = ld_u<u32x4>(blk + 16 * (sx + i));
+            r.q[i] = ld_u<u32x4>(blk + 32 + 32 * (g >> 1) + 16 * (sx + i));
+        }
+        r.s0 = ld_u<uint32_t>(blk + 96);
+        r.s1 = ld_u<uint32_t>(blk + 100);
+        r.s2 = ld_u<uint32_t>(blk + 104);
+        r.d = ld_u<uint16_t>(blk + 108);
+    }
+    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &r, float &d, float &dmin) {
+        d = h2f(r.d);
+        dmin = 0.0f;
+    }
+    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &, int) { return 0; }
+    template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int g, int part, uint32_t out[NW / 2]) {
+        const int jh = NW == 16 ? part >> 1 : part, sx = NW == 16 ? part & 1 : 0;
+        const int h = g >> 1, s = 2 * (g & 1) + jh;
+        // the eight 6-bit scales of half h, one per byte of (e0, e1) (k_quants.rs:1148-1156)
+        const uint32_t t2 = r.s2 >> (4 * h);
+        const uint32_t e0 = ((r.s0 >> (4 * h)) & 0x0f0f0f0fu) | ((t2 & 0x03030303u) << 4);
+        const uint32_t e1 = ((r.s1 >> (4 * h)) & 0x0f0f0f0fu) | (((t2 >> 2) & 0x03030303u) << 4);
+        const uint32_t off = h2_splat(-1028.0f);                               // -(1024 + 4)
+#pragma unroll
+        for (int i = 0; i < NW / 4; i++) {
+            const int gi = 2 * s + sx + (i >> 2);                               // 16-element group within the half, 0..7
+            const int sc = (int)(((gi < 4 ? e0 : e1) >> (8 * (gi & 3))) & 0xffu) - 32;
+            const uint32_t s2 = h2_splat((float)sc);
+            const uint32_t v = ((r.q[i >> 2][i & 3] >> (2 * s)) & 0x03030303u) | (((r.hm[i >> 2][i & 3] >> (4 * h + s)) & 0x01010101u) << 2);
+            uint32_t lo, hi;
+            bytes_to_h1024(v, lo, hi);
+            out[2 * i] = pk_mul(pk_add(lo, off), s2);                           // (q - 4) * (sc - 32), exact
+            out[2 * i + 1] = pk_mul(pk_add(hi, off), s2);
+        }
+    }
+};
+
 template <> struct Stage<CQ_Q4_0> {
     static constexpr bool KQ = false, HAS_MIN = false;
     static constexpr int TERMS = 1;
@@ -183,7 +268,7 @@ template <> struct Stage<CQ_Q4_0> {
         r.qs = ld_u<u32x4>(blk + 2);
     }
     template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &, float &d, float &dmin) { d = 1.0f; dmin = 0.0f; }
-    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &, int) { return 0; }
+    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &, int) { return 0; }
     // elements 0..15 of a block are the low nibbles of its 16 bytes, elements 16..31 the high nibbles
     template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int, int part, uint32_t out[NW / 2]) {
         const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1032.0f);   // -(1024 + 8)
@@ -219,7 +304,7 @@ template <> struct Stage<CQ_Q8_0> {
         for (int i = 0; i < NW / 16; i++) r.q[i] = ld_u<u32x4>(blk + 2 + 16 * (sx + i));
     }
     template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &, float &d, float &dmin) { d = 1.0f; dmin = 0.0f; }
-    template <int NW> static __device__ __forceinline__ uint32_t mins4(const Raw<NW> &, int) { return 0; }
+    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &, int) { return 0; }
     template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int, int, uint32_t out[NW / 2]) {
         const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1152.0f);   // -(1024 + 128)
 #pragma unroll
@@ -359,13 +444,10 @@ __global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 
             S::template header<NW>(wraw, c.d, c.dmin);
             c.d8 = arow_ok ? d8 : 0.0f;
             if (S::HAS_MIN) {
-                // Bm[n][2 j], Bm[n][2 j + 1] = min of sub-block j, this thread's share j = (8 / TPR) part + i; Am[m][j] = bsums16[j]
-                const uint32_t mine = S::template mins4<NW>(wraw, (8 / TPR) * part >= 4);
+                // Bm[n][j] = min of the 16-element group j, this thread's share j = 2 ((8 / TPR) part + i) + {0, 1}; Am[m][j] = bsums16[j]
 #pragma unroll
-                for (int i = 0; i < 8 / TPR; i++) {
-                    const uint32_t mb = (mine >> (8 * (((8 / TPR) * part + i) & 3))) & 0xffu;
-                    c.mv[i] = pk_add((0x6400u | mb) * 0x00010001u, 0xe400e400u);    // (1024 + min) - 1024 in both halves
-                }
+                for (int i = 0; i < 8 / TPR; i++)
+                    c.mv[i] = pk_add(0x64006400u | S::template min_pair<NW>(wraw, (8 / TPR) * part + i), 0xe400e400u);   // (1024 + min) - 1024
                 const uint32_t b4[4] = {abs0.x, abs0.y, abs0.z, abs0.w};
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -844,6 +926,8 @@ int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_
         case CQ_Q4K: return launch_qmm_moe<CQ_Q4K>(w, av, out, mc, k, n, tile_rows, s);
         case CQ_Q5K: return launch_qmm_moe<CQ_Q5K>(w, av, out, mc, k, n, tile_rows, s);
         case CQ_Q6K: return launch_qmm_moe<CQ_Q6K>(w, av, out, mc, k, n, tile_rows, s);
+        case CQ_Q2K: return launch_qmm_moe<CQ_Q2K>(w, av, out, mc, k, n, tile_rows, s);
+        case CQ_Q3K: return launch_qmm_moe<CQ_Q3K>(w, av, out, mc, k, n, tile_rows, s);
     }
     return CQ_ERR_DTYPE;
 }
@@ -885,6 +969,8 @@ int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst
             case CQ_Q4K: return launch_qmm<CQ_Q4K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q5K: return launch_qmm<CQ_Q5K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q6K: return launch_qmm<CQ_Q6K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q2K: return launch_qmm<CQ_Q2K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q3K: return launch_qmm<CQ_Q3K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
         }
         return CQ_ERR_DTYPE;
     }

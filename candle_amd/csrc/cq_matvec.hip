@@ -655,9 +655,9 @@ int launch_nb(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_
 template <int DT, int SRC>
 int launch_rows(const void *w, const ActSrc &src, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst,
                 hipStream_t s) {
-    // The formats without a matrix-core kernel have the fused instances QMatMul::forward uses (f32 activations, one or
-    // two rows); everything else of theirs goes through the pre-quantized scratch.
-    if constexpr (!cq_has_mfma(DT) && SRC != SRC_SCRATCH) {
+    // Q4_1, Q5_0, Q5_1, Q2_K, Q3_K have the fused instances QMatMul::forward uses (f32 activations, one or two rows);
+    // everything else of theirs goes through the pre-quantized scratch.
+    if constexpr (!cq_full_matvec(DT) && SRC != SRC_SCRATCH) {
         if constexpr (SRC == CQ_F32) {
             if (rows == 1) return launch_nb<DT, 1, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
             if (rows == 2) return launch_nb<DT, 2, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
@@ -769,7 +769,7 @@ int launch_fused_dt(int w_dtype, const void *w, const ActSrc &src, void *dst, in
         case CQ_Q5K: return launch_fused1<CQ_Q5K, PRO, EPI>(w, src, dst, k, n, s, fz);
         case CQ_Q6K: return launch_fused1<CQ_Q6K, PRO, EPI>(w, src, dst, k, n, s, fz);
     }
-    // The formats without a matrix-core kernel have the three fusions a decoder step cannot do without: the rms_norm
+    // Q4_1, Q5_0, Q5_1, Q2_K, Q3_K have the three fusions a decoder step cannot do without: the rms_norm
     // prologue, and the residual epilogue with and without the silu * up prologue.
     if constexpr ((PRO == PRO_NORM && EPI == EPI_NONE) || ((PRO == PRO_NONE || PRO == PRO_SILU) && EPI == EPI_RESID)) {
         switch (w_dtype) {

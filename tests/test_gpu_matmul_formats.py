@@ -1,7 +1,8 @@
-"""GPU parity of QMatMul::forward for the block formats without a matrix-core kernel (Q4_1, Q5_0, Q5_1, Q2_K, Q3_K)
-against the CPU oracle: candle's CPU path quantizes their activations to Q8_1 / Q8_0 / Q8_1 / Q8_K / Q8_K
-(k_quants.rs:317,418,524,822,1055).  The GPU quantizes to the same int8 values, so the bar is the same as for the
-other formats: relative L2 <= 1e-3 by contract, <= 2e-6 observed (f32 summation order only).
+"""GPU parity of QMatMul::forward for Q4_1, Q5_0, Q5_1, Q2_K, Q3_K weights against the CPU oracle: candle's CPU path
+quantizes their activations to Q8_1 / Q8_0 / Q8_1 / Q8_K / Q8_K (k_quants.rs:317,418,524,822,1055).  The GPU quantizes to
+the same int8 values and every kernel sums the same integers (matvec kernels; for Q2_K / Q3_K beyond 8 rows the f16 matrix
+cores with exact small-integer operands), so the bar is the same as for the other K-quants: relative L2 <= 1e-3 by
+contract, <= 2e-6 observed (f32 summation order only).
 """
 import numpy as np
 import pytest
@@ -75,9 +76,9 @@ def test_k_not_multiple_of_256(dtype):
 
 
 @pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
-@pytest.mark.parametrize("m", [9, 16, 33])
+@pytest.mark.parametrize("m", [9, 16, 33, 128])
 def test_more_than_eight_rows(dtype, m):
-    # no matrix-core kernel for these formats: eight activation rows per pass over the weights
+    # Q2_K / Q3_K: matrix cores; Q4_1 / Q5_0 / Q5_1: eight activation rows per pass over the weights
     n, k = 96, 1024
     blocks, qmm = make_weight(dtype, n, k, seed=61 + dtype)
     x = normal(62 + m, (m, k), 1.0)
@@ -123,3 +124,26 @@ def test_bit_patterns_random_blocks():
         got = forward(ca.QMatMul.from_qtensor(qt), x)
         want = oracle.matmul(dtype, x, blocks, n)
         assert rel_l2(got, want) <= TIGHT, NAMES[dtype]
+
+
+@pytest.mark.parametrize("dtype", [oracle.Q2K, oracle.Q3K], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 256), (130, 200, 512), (257, 129, 2048), (64, 384, 4096), (20, 260, 1024), (512, 96, 8192)])
+def test_prefill_tiles_ragged(dtype, m, n, k):
+    # 128 x 64 and 32 x 128 tiles with ragged edges, one super-block rows, split-K shapes (few tiles, long k)
+    blocks, qmm = make_weight(dtype, n, k, seed=71)
+    x = normal(72, (m, k), 1.0)
+    err = rel_l2(forward(qmm, x), oracle.matmul(dtype, x, blocks, n))
+    assert err <= TIGHT, err
+
+
+@pytest.mark.parametrize("dtype", [oracle.Q2K, oracle.Q3K], ids=lambda d: NAMES[d])
+def test_prefill_random_blocks(dtype):
+    # every bit of qs / hmask / scales in play on the matrix-core path (scales up to 63, mins up to 15)
+    import candle_amd as ca
+    from tests.test_oracle_kat import random_weight_blocks
+    rng = np.random.default_rng(8)
+    n, k, m = 130, 1024, 70
+    blocks = random_weight_blocks(dtype, n * k // 256, rng)
+    qt = ca.QTensor.new(ca.QStorage.from_data(blocks, "cuda", ca.GgmlDType(dtype)), (n, k))
+    x = normal(91, (m, k), 1.0)
+    assert rel_l2(forward(ca.QMatMul.from_qtensor(qt), x), oracle.matmul(dtype, x, blocks, n)) <= TIGHT

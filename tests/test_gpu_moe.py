@@ -87,7 +87,7 @@ def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     assert err2 <= TOL and err2 <= TIGHT, err2
 
 
-@pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q5K, oracle.Q6K], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q2K, oracle.Q3K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("E,n", [(64, 160), (8, 160)])      # 1200 pairs: about 19 rows per expert (32-row tiles of the MFMA
                                                             # kernel, 128 weight rows wide) or 150 (128-row tiles); n is ragged
 def test_moe_gemm_gguf_mfma_tile_sizes(dtype, E, n):
