@@ -21,8 +21,8 @@
  *     Q8_0 blocks for Q4_0/Q5_0/Q8_0, Q8_1 blocks for Q4_1/Q5_1: k_quants.rs:2320-2358, 658-687, 770-799), so
  *     results match QMatMul::forward on the CPU up to f32 summation order;
  *   - weight formats of the matmul-family entry points (cq_quantize_act, cq_matvec, cq_matmul, cq_qmatmul_forward,
- *     the MoE entry points): Q4_0, Q8_0, Q4K, Q5K, Q6K, which also have matrix-core kernels, and Q4_1, Q5_0, Q5_1,
- *     Q2K, Q3K, which take the matvec kernels at any row count (eight activation rows per pass over the weights).
+ *     the MoE entry points): Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K, which also have matrix-core kernels, and Q4_1, Q5_0,
+ *     Q5_1, which take the matvec kernels at any row count (eight activation rows per pass over the weights).
  */
 #ifndef CANDLE_HIP_QUANT_H
 #define CANDLE_HIP_QUANT_H
@@ -119,7 +119,7 @@ int cq_matvec(int w_dtype, const void *w_dev, const void *act_scratch_dev, void 
 
 /* ---------------------------------------------------------------------------------------------
  * Prefill matmul over pre-quantized activations (any rows >= 1): more than CQ_MATVEC_MAX_ROWS rows with k a
- * multiple of 256 (Q4_0, Q8_0, Q4K, Q5K, Q6K) run on the matrix cores with the converted operand tiles staged in LDS (K-quant operands are
+ * multiple of 256 (Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K) run on the matrix cores with the converted operand tiles staged in LDS (K-quant operands are
  * exact integers there, Q4_0 / Q8_0 operands are rounded to f16); other shapes take 8 rows per matvec pass.
  * Counterpart of launch_mmq_gguf_<t> (candle-core/src/quantized/fast_mmq.rs:71-111, candle-kernels/src/mmq_gguf/).
  * Same buffers as cq_matvec; dst is f32.
