@@ -45,7 +45,10 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_I8_PEAK_TOPS = 5000.0
 Q4K = 12
-WDTYPES = {"q4_0": (2, 18, 32), "q8_0": (8, 34, 32), "q4k": (12, 144, 256), "q5k": (13, 176, 256), "q6k": (14, 210, 256)}
+WDTYPES = {"q4_0": (2, 18, 32), "q8_0": (8, 34, 32), "q4k": (12, 144, 256), "q5k": (13, 176, 256), "q6k": (14, 210, 256),
+           "q4_1": (3, 20, 32), "q5_0": (6, 22, 32), "q5_1": (7, 24, 32), "q2k": (10, 84, 256), "q3k": (11, 110, 256)}
+FMT_NAMES = {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4k": "Q4_K", "q5k": "Q5_K", "q6k": "Q6_K", "q4_1": "Q4_1", "q5_0": "Q5_0", "q5_1": "Q5_1",
+             "q2k": "Q2_K", "q3k": "Q3_K"}
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "q4k_decode_matvec_1x4096x14336_pmc.txt")
 
 
@@ -290,7 +293,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="--workload decode8b: number of decoder layers")
     ap.add_argument("--prompt", type=int, default=512, help="--workload decode8b: prompt tokens")
     ap.add_argument("--moe-tokens", default="1,16,256", help="--workload moe: token counts, comma separated")
-    ap.add_argument("--wdtype", choices=sorted(WDTYPES), default="q4k", help="weight format of --workload prefill")
+    ap.add_argument("--wdtype", choices=sorted(WDTYPES), default="q4k",
+                    help="weight format of --workload prefill / decode (the metric is quoted on q4k; other formats skip the 8B decoder and the CPU baseline)")
     ap.add_argument("--n", type=int, default=14336)
     ap.add_argument("--k", type=int, default=4096)
     ap.add_argument("--batch", type=int, default=1)
@@ -324,8 +328,13 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     n, k, m = args.n, args.k, args.batch
-    wbytes = L.cq_storage_bytes(Q4K, n * k)
-    alg_bytes = algorithmic_bytes(n, k, m, 144, 256)
+    WDT, w_ts, w_bs = WDTYPES[args.wdtype]
+    fmt = FMT_NAMES[args.wdtype]
+    headline = args.wdtype == "q4k"
+    if not headline:
+        args.no_cpu_baseline = True
+    wbytes = L.cq_storage_bytes(WDT, n * k)
+    alg_bytes = algorithmic_bytes(n, k, m, w_ts, w_bs)
 
     # ---- synthetic inputs, resident in HBM --------------------------------------------------
     pool = max(2, (args.pool_mb * 1000 * 1000 + wbytes - 1) // wbytes)
@@ -337,12 +346,12 @@ def main():
     for i in range(pool):
         wf = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
         wq = torch.empty(wbytes, dtype=torch.uint8, device=dev)
-        _lib.check("cq_quantize", L.cq_quantize(Q4K, wf.data_ptr(), wq.data_ptr(), n * k, None))
+        _lib.check("cq_quantize", L.cq_quantize(WDT, wf.data_ptr(), wq.data_ptr(), n * k, None))
         weights.append(wq)
         del wf
     x = torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32)
     dst = torch.empty((m, n), dtype=torch.float32, device=dev)
-    ws_bytes = L.cq_qmatmul_workspace_bytes(Q4K, m, k, n)
+    ws_bytes = L.cq_qmatmul_workspace_bytes(WDT, m, k, n)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     torch.cuda.synchronize()
 
@@ -350,11 +359,11 @@ def main():
 
     def step(i, sp):
         """QMatMul::forward: activation quantization + matvec in one kernel."""
-        _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(Q4K, weights[i % pool].data_ptr(), x.data_ptr(), 0, dst.data_ptr(), 0,
+        _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(WDT, weights[i % pool].data_ptr(), x.data_ptr(), 0, dst.data_ptr(), 0,
                                                               m, k, n, ws.data_ptr(), ws_bytes, sp))
 
     def matvec_prequantized(i, sp):
-        _lib.check("cq_matvec", L.cq_matvec(Q4K, weights[i % pool].data_ptr(), ws.data_ptr(), dst.data_ptr(), 0, k, n, m, n, sp))
+        _lib.check("cq_matvec", L.cq_matvec(WDT, weights[i % pool].data_ptr(), ws.data_ptr(), dst.data_ptr(), 0, k, n, m, n, sp))
 
     if args.pmc_mode:
         # plain launches (one dispatch row per kernel in the counter CSV) + a copy of known size
@@ -421,7 +430,7 @@ def main():
     extra = None
     if not args.no_extra:
         resident_us = event_us(capture(step, same_weight=True), args.steps)
-        _lib.check("cq_quantize_act", L.cq_quantize_act(Q4K, x.data_ptr(), 0, ws.data_ptr(), k, m, None))
+        _lib.check("cq_quantize_act", L.cq_quantize_act(WDT, x.data_ptr(), 0, ws.data_ptr(), k, m, None))
         torch.cuda.synchronize()
         preq_us = event_us(capture(matvec_prequantized), args.steps)
         # the yardstick: a kernel that only reads the same rotated tensors, same launch shape
@@ -439,7 +448,7 @@ def main():
                  "prequantized_matvec_GBps": round(alg_bytes / (preq_us * 1e-6) / 1e9, 1)}
 
     out = {
-        "metric": "Q4_K matvec GB/s @4096x14336 (decode, batch %d)" % m,
+        "metric": "%s matvec GB/s @%dx%d (decode, batch %d)" % (fmt, k, n, m),
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -451,18 +460,19 @@ def main():
         "vs_baseline": None,
         "dtype": "i8",
         "data": "synthetic",
-        "config": {"workload": "Q4_K decode matvec 1x%d->%d, weight [%d x %d] Q4_K, batch %d, %d distinct weight tensors rotated (%.2f GB)"
-                               % (k, n, n, k, m, pool, pool * wbytes / 1e9),
-                   "step": "QMatMul::forward = Q8_K activation quantization + matvec in one kernel, launches captured in a HIP graph",
+        "config": {"workload": "%s decode matvec 1x%d->%d, weight [%d x %d] %s, batch %d, %d distinct weight tensors rotated (%.2f GB)"
+                               % (fmt, k, n, n, k, fmt, m, pool, pool * wbytes / 1e9),
+                   "step": "QMatMul::forward = %s activation quantization + matvec in one kernel, launches captured in a HIP graph"
+                           % ("Q8_K" if w_bs == 256 else "Q8_0"),
                    "n": n, "k": k, "batch": m},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
-        "roofline": {"bound": "hbm", "kernel": "qmv_kernel<Q4_K, NB=1, fused f32 activations>", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": committed_traffic(),
+        "roofline": {"bound": "hbm", "kernel": "qmv_kernel<%s, NB=%d, fused f32 activations>" % (fmt, m), "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": committed_traffic() if headline else None,
                      "avg_kernel_us": round(kern_us, 3), "algorithmic_bytes_per_launch": alg_bytes},
         "extra": extra,
     }
 
-    if not args.no_extra:
+    if not args.no_extra and headline:
         # the second half of the metric: the 8B-shape decoder (same protocol as --workload decode8b)
         d8 = argparse.Namespace(layers=32, prompt=512, steps=256)
         r = decode8b(d8)
