@@ -31,7 +31,9 @@ inline int check_mm_shape(int w_dtype, int64_t k, int64_t n, int64_t rows) {
 
 inline int check_weight_ptr(int w_dtype, const void *w) {
     if (!w) return CQ_ERR_NULL;
-    if (!aligned(w, (w_dtype == CQ_Q4K || w_dtype == CQ_Q5K) ? 16 : 2)) return CQ_ERR_ALIGN;
+    // Q4_0 / Q5_0 / Q8_0 blocks are fetched as the aligned dwords around them (cq_fmt.h)
+    const bool dwords = w_dtype == CQ_Q4_0 || w_dtype == CQ_Q5_0 || w_dtype == CQ_Q8_0;
+    if (!aligned(w, (w_dtype == CQ_Q4K || w_dtype == CQ_Q5K) ? 16 : dwords ? 4 : 2)) return CQ_ERR_ALIGN;
     return CQ_OK;
 }
 

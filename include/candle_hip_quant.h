@@ -16,7 +16,9 @@
  *   - weights are GGUF blocks exactly as stored on disk, rows contiguous, `n` rows of `k/blk` blocks
  *     (candle-core/src/quantized/k_quants.rs:77-190); kernels read only [ptr, ptr + size) and never
  *     rely on the 512-element tail padding the CUDA backend adds
- *     (candle-core/src/quantized/cuda.rs:624-637,989-1008);
+ *     (candle-core/src/quantized/cuda.rs:624-637,989-1008); the matvec kernels fetch Q4_0 / Q5_0 / Q8_0 blocks
+ *     (18 / 22 / 34 bytes) as whole aligned dwords, so a tensor of these formats whose size is 2 (mod 4) is read up
+ *     to the end of its last dword;
  *   - activation quantization follows candle's CPU path bit for bit (Q8_K blocks for K-quants,
  *     Q8_0 blocks for Q4_0/Q5_0/Q8_0, Q8_1 blocks for Q4_1/Q5_1: k_quants.rs:2320-2358, 658-687, 770-799), so
  *     results match QMatMul::forward on the CPU up to f32 summation order;
@@ -109,7 +111,7 @@ int cq_quantize_act(int w_dtype, const void *x_dev, int x_dtype, void *scratch_d
  * Decode matvec over pre-quantized activations:  dst[r, j] = sum_k W[j, k] * x^[r, k]
  * for r < rows <= CQ_MATVEC_MAX_ROWS.  Counterpart of launch_mmvq_gguf_<t>_<dst>_plain
  * (candle-kernels/src/ffi.rs:58-631, mmvq_gguf.cu:915-1008).
- *   w_dev: n rows of k/blk blocks; 16-byte aligned for Q4K/Q5K, 2-byte aligned otherwise.
+ *   w_dev: n rows of k/blk blocks; 16-byte aligned for Q4K/Q5K, 4-byte aligned for Q4_0/Q5_0/Q8_0, 2-byte aligned otherwise.
  *   act_scratch_dev: written by cq_quantize_act with the same (w_dtype, k, rows).
  *   dst_dev: f32 / f16 / bf16 (dst_dtype), row stride `stride_dst` elements (>= n).
  * ------------------------------------------------------------------------------------------- */
