@@ -21,6 +21,10 @@ inline bool float_dtype(int dt) { return dt == CQ_F32 || dt == CQ_F16 || dt == C
 inline int64_t float_size(int dt) { return dt == CQ_F32 ? 4 : 2; }
 
 // shared checks of the (w_dtype, k, n, rows) tuple of the matmul-family entry points
+// expert formats of the MoE entry points: the reference's (Q2K ... Q6K, Q8_0: candle-core/src/quantized/cuda.rs:543-548,
+// candle-nn/src/moe.rs:210-215) plus Q4_0
+inline bool moe_weight_dtype(int dt) { return cq_has_mfma(dt); }
+
 inline int check_mm_shape(int w_dtype, int64_t k, int64_t n, int64_t rows) {
     if (!matmul_weight_dtype(w_dtype)) return CQ_ERR_DTYPE;
     if (k <= 0 || n < 0 || rows < 0) return CQ_ERR_SHAPE;
@@ -231,7 +235,7 @@ int cq_nn_qmatmul_swiglu_rows(int w_dtype, const void *w_dev, const float *gate_
 
 int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk,
                                        int64_t input_dim1) {
-    if (check_mm_shape(w_dtype, k, n, batch) || num_experts <= 0 || topk <= 0) return -1;
+    if (!moe_weight_dtype(w_dtype) || check_mm_shape(w_dtype, k, n, batch) || num_experts <= 0 || topk <= 0) return -1;
     if (input_dim1 != 1 && input_dim1 != topk) return -1;
     return cq_moe_workspace_bytes_impl(w_dtype, num_experts, batch * topk, batch * input_dim1, k);
 }
@@ -239,7 +243,7 @@ int64_t cq_indexed_moe_workspace_bytes(int w_dtype, int64_t num_experts, int64_t
 int cq_indexed_moe_forward(int w_dtype, const void *w_dev, const float *x_dev, const uint32_t *ids_dev, float *out_dev,
                            int64_t num_experts, int64_t n, int64_t k, int64_t batch, int64_t topk, int64_t input_dim1,
                            void *workspace_dev, int64_t workspace_bytes, void *stream) {
-    int rc = check_mm_shape(w_dtype, k, n, batch);
+    int rc = moe_weight_dtype(w_dtype) ? check_mm_shape(w_dtype, k, n, batch) : (int)CQ_ERR_DTYPE;
     if (rc) return rc;
     if (num_experts <= 0 || topk <= 0) return CQ_ERR_SHAPE;
     if (input_dim1 != 1 && input_dim1 != topk) return CQ_ERR_SHAPE;
@@ -261,7 +265,7 @@ int cq_indexed_moe_forward(int w_dtype, const void *w_dev, const float *x_dev, c
 
 int64_t cq_moe_gemm_workspace_bytes(int w_dtype, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k,
                                     int has_topk_weights) {
-    if (check_mm_shape(w_dtype, k, n, size_m) || num_experts <= 0 || topk <= 0) return -1;
+    if (!moe_weight_dtype(w_dtype) || check_mm_shape(w_dtype, k, n, size_m) || num_experts <= 0 || topk <= 0) return -1;
     if (!has_topk_weights && size_m % topk != 0) return -1;
     int64_t x_rows = has_topk_weights ? size_m : size_m / topk;
     return cq_moe_workspace_bytes_impl(w_dtype, num_experts, size_m, x_rows, k);
@@ -271,7 +275,7 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
                      const int32_t *expert_ids_dev, const float *topk_weights_dev, float *out_dev,
                      int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int is_prefill,
                      void *workspace_dev, int64_t workspace_bytes, void *stream) {
-    int rc = check_mm_shape(w_dtype, k, n, size_m);
+    int rc = moe_weight_dtype(w_dtype) ? check_mm_shape(w_dtype, k, n, size_m) : (int)CQ_ERR_DTYPE;
     if (rc) return rc;
     if (num_experts <= 0 || topk <= 0) return CQ_ERR_SHAPE;
     if (!topk_weights_dev && size_m % topk != 0) return CQ_ERR_SHAPE;
@@ -297,7 +301,7 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
 int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, const void *w_b_dev, const int32_t *sorted_token_ids_dev,
                           const int32_t *expert_ids_dev, float *out_a_dev, float *out_b_dev, int64_t num_experts, int64_t topk, int64_t size_m,
                           int64_t n, int64_t k, int is_prefill, void *workspace_dev, int64_t workspace_bytes, void *stream) {
-    int rc = check_mm_shape(w_dtype, k, n, size_m);
+    int rc = moe_weight_dtype(w_dtype) ? check_mm_shape(w_dtype, k, n, size_m) : (int)CQ_ERR_DTYPE;
     if (rc) return rc;
     if (num_experts <= 0 || topk <= 0 || size_m % topk != 0) return CQ_ERR_SHAPE;
     if (num_experts > (1 << 20)) return CQ_ERR_RANGE;
@@ -322,7 +326,7 @@ int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, 
 int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_dev, const void *w_up_dev, const int32_t *sorted_token_ids_dev,
                             const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
                             int64_t k, void *stream) {
-    int rc = check_mm_shape(w_dtype, k, n, size_m);
+    int rc = moe_weight_dtype(w_dtype) ? check_mm_shape(w_dtype, k, n, size_m) : (int)CQ_ERR_DTYPE;
     if (rc) return rc;
     if (num_experts <= 0 || topk <= 0 || size_m % topk != 0) return CQ_ERR_SHAPE;
     if (num_experts > (1 << 20) || size_m > CQ_MOE_DIRECT_MAX_PAIRS) return CQ_ERR_RANGE;

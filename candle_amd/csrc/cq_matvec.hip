@@ -663,18 +663,19 @@ int launch_rows(const void *w, const ActSrc &src, void *dst, int dst_dtype, int6
             if (rows == 2) return launch_nb<DT, 2, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
         }
         return CQ_ERR_RANGE;
-    } else
-    switch (rows) {
-        case 1: return launch_nb<DT, 1, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-        case 2: return launch_nb<DT, 2, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-        case 3: return launch_nb<DT, 3, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-        case 4: return launch_nb<DT, 4, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-        case 5: return launch_nb<DT, 5, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-        case 6: return launch_nb<DT, 6, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-        case 7: return launch_nb<DT, 7, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
-        case 8: return launch_nb<DT, 8, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+    } else {
+        switch (rows) {
+            case 1: return launch_nb<DT, 1, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            case 2: return launch_nb<DT, 2, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            case 3: return launch_nb<DT, 3, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            case 4: return launch_nb<DT, 4, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            case 5: return launch_nb<DT, 5, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            case 6: return launch_nb<DT, 6, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            case 7: return launch_nb<DT, 7, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+            case 8: return launch_nb<DT, 8, SRC>(w, src, dst, dst_dtype, k, n, stride_dst, s);
+        }
+        return CQ_ERR_RANGE;
     }
-    return CQ_ERR_RANGE;
 }
 
 template <int SRC>
@@ -1105,9 +1106,6 @@ int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, 
         case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w, x, out, ps, k, n, s);
         case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w, x, out, ps, k, n, s);
         case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w, x, out, ps, k, n, s);
-        case CQ_Q4_1: return launch_moe_pairs<CQ_Q4_1>(w, x, out, ps, k, n, s);
-        case CQ_Q5_0: return launch_moe_pairs<CQ_Q5_0>(w, x, out, ps, k, n, s);
-        case CQ_Q5_1: return launch_moe_pairs<CQ_Q5_1>(w, x, out, ps, k, n, s);
         case CQ_Q2K: return launch_moe_pairs<CQ_Q2K>(w, x, out, ps, k, n, s);
         case CQ_Q3K: return launch_moe_pairs<CQ_Q3K>(w, x, out, ps, k, n, s);
     }
@@ -1126,9 +1124,6 @@ int cq_moe_pairs_swiglu_launch(int w_dtype, const void *w_gate, const void *w_up
         case CQ_Q4K: return launch_moe_pairs<CQ_Q4K>(w_gate, x, out, ps, k, n, s, true, off);
         case CQ_Q5K: return launch_moe_pairs<CQ_Q5K>(w_gate, x, out, ps, k, n, s, true, off);
         case CQ_Q6K: return launch_moe_pairs<CQ_Q6K>(w_gate, x, out, ps, k, n, s, true, off);
-        case CQ_Q4_1: return launch_moe_pairs<CQ_Q4_1>(w_gate, x, out, ps, k, n, s, true, off);
-        case CQ_Q5_0: return launch_moe_pairs<CQ_Q5_0>(w_gate, x, out, ps, k, n, s, true, off);
-        case CQ_Q5_1: return launch_moe_pairs<CQ_Q5_1>(w_gate, x, out, ps, k, n, s, true, off);
         case CQ_Q2K: return launch_moe_pairs<CQ_Q2K>(w_gate, x, out, ps, k, n, s, true, off);
         case CQ_Q3K: return launch_moe_pairs<CQ_Q3K>(w_gate, x, out, ps, k, n, s, true, off);
     }
@@ -1187,9 +1182,6 @@ int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_
         case CQ_Q4K: return launch_moe_chunks<CQ_Q4K>(w, scratch, rows_alloc, out, mc, k, n, s);
         case CQ_Q5K: return launch_moe_chunks<CQ_Q5K>(w, scratch, rows_alloc, out, mc, k, n, s);
         case CQ_Q6K: return launch_moe_chunks<CQ_Q6K>(w, scratch, rows_alloc, out, mc, k, n, s);
-        case CQ_Q4_1: return launch_moe_chunks<CQ_Q4_1>(w, scratch, rows_alloc, out, mc, k, n, s);
-        case CQ_Q5_0: return launch_moe_chunks<CQ_Q5_0>(w, scratch, rows_alloc, out, mc, k, n, s);
-        case CQ_Q5_1: return launch_moe_chunks<CQ_Q5_1>(w, scratch, rows_alloc, out, mc, k, n, s);
         case CQ_Q2K: return launch_moe_chunks<CQ_Q2K>(w, scratch, rows_alloc, out, mc, k, n, s);
         case CQ_Q3K: return launch_moe_chunks<CQ_Q3K>(w, scratch, rows_alloc, out, mc, k, n, s);
     }

@@ -252,9 +252,6 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
         case CQ_Q4K: return launch_moe_matvec<CQ_Q4K>(a, av, offsets, pin, pout, pscale, s);
         case CQ_Q5K: return launch_moe_matvec<CQ_Q5K>(a, av, offsets, pin, pout, pscale, s);
         case CQ_Q6K: return launch_moe_matvec<CQ_Q6K>(a, av, offsets, pin, pout, pscale, s);
-        case CQ_Q4_1: return launch_moe_matvec<CQ_Q4_1>(a, av, offsets, pin, pout, pscale, s);
-        case CQ_Q5_0: return launch_moe_matvec<CQ_Q5_0>(a, av, offsets, pin, pout, pscale, s);
-        case CQ_Q5_1: return launch_moe_matvec<CQ_Q5_1>(a, av, offsets, pin, pout, pscale, s);
         case CQ_Q2K: return launch_moe_matvec<CQ_Q2K>(a, av, offsets, pin, pout, pscale, s);
         case CQ_Q3K: return launch_moe_matvec<CQ_Q3K>(a, av, offsets, pin, pout, pscale, s);
     }

@@ -83,6 +83,8 @@ def test_argument_validation_codes_without_gpu():
     assert L.cq_qmatmul_workspace_bytes(Q4K, 1, 4096, 14336) == 4096 + 256 + 512
     assert L.cq_qmatmul_forward(Q4K, 16, 16, 0, 16, 0, 1, 4096, 8, 256, 10, None) == WS
     assert L.cq_indexed_moe_workspace_bytes(Q4K, 8, 16, 256, 2, 4, 3) == -1    # input_dim1 must be topk or 1
+    assert L.cq_indexed_moe_workspace_bytes(6, 8, 16, 256, 2, 4, 4) == -1      # Q5_0 is a matmul weight format, not an expert format
+    assert L.cq_moe_gemm_gguf(6, 16, 16, 4, 4, None, 4, 8, 4, 8, 16, 256, 0, 256, 1 << 20, None) == DTYPE
     assert L.cq_moe_gemm_workspace_bytes(Q4K, 8, 4, 6, 16, 256, 0) == -1       # size_m not a multiple of topk
     assert L.cq_moe_gemm_gguf(Q4K, 16, 16, 4, 4, None, 4, 8, 4, 8, 16, 256, 0, 256, 0, None) == WS
     assert _lib.status_string(SHAPE).startswith("invalid shape")
