@@ -1062,11 +1062,145 @@ __global__ __launch_bounds__(1024) void moe_pair_kernel(const uint8_t *__restric
                                                                                       out + (int64_t)out_row * g.n, g, fz, blockIdx.x, gridDim.x);
 }
 
+// Short expert rows (at most 32 units per row: k <= 2048 for K-quants, e.g. the 768- and 2048-element rows of a
+// Qwen3-30B-A3B expert): one wave step takes 64 / SEG weight rows, SEG = 32 or 16 lanes each, instead of leaving half or
+// more of the lanes idle.  Lane l works on unit l % SEG of row (l / SEG) of the step; the sums stay inside their
+// 16-lane DPP rows (SEG = 16) or are folded pairwise with one row broadcast (SEG = 32) and lane SEG - 1 of each segment
+// stores.  Otherwise the body of moe_pair_kernel for rows of one wave step: activation row quantized into LDS by the
+// workgroup, weights of the next step in flight while this one is reduced.
+template <int SEG> __device__ __forceinline__ float seg_sum_to_last(float v) {
+#define CQ_DPP(ctrl, rmask, bc) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, rmask, 0xf, bc))
+    v += CQ_DPP(0x111, 0xf, true);     // row_shr:1
+    v += CQ_DPP(0x112, 0xf, true);     // row_shr:2
+    v += CQ_DPP(0x114, 0xf, true);     // row_shr:4
+    v += CQ_DPP(0x118, 0xf, true);     // row_shr:8   -> lane 15 of each 16-lane row holds the row sum
+    if (SEG == 32) v += CQ_DPP(0x142, 0xa, false);    // row_bcast:15 into rows 1 and 3 -> lanes 31 and 63 hold the segment sums
+#undef CQ_DPP
+    return v;
+}
+
+template <int DT, int SEG, bool SWIGLU>
+__global__ __launch_bounds__(1024) void moe_pair_short_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ out,
+                                                              QmvGeom g, PairSource ps, int64_t expert_bytes, int64_t pair_off) {
+    typedef Fmt<DT> F;
+    constexpr int RPS = 64 / SEG;                      // weight rows per wave step
+    const int p = blockIdx.y;
+    int e, in_row, out_row;
+    float scale;
+    const int wg_row0 = blockIdx.x * g.rows_per_wg, wg_row1 = min(g.n, wg_row0 + g.rows_per_wg);
+    if (!pair_decode(ps, p, e, in_row, out_row, scale)) {       // uniform over the workgroup
+        if (ps.mode == MOE_INDEXED)                             // an out-of-range id: that output row is zero
+            for (int r = wg_row0 + (int)threadIdx.x; r < wg_row1; r += (int)blockDim.x) out[(int64_t)p * g.n + r] = 0.0f;
+        return;
+    }
+    extern __shared__ __align__(16) uint8_t lds[];
+    int8_t *lqs = (int8_t *)lds;
+    float *ld = (float *)(lds + g.lds_d_off);
+    int16_t *lbs = (int16_t *)(lds + g.lds_bs_off);
+    const int k = g.k, n = g.n;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = 1 << g.nw_shift;
+    const int sl = lane & (SEG - 1), sub = lane / SEG;
+    const bool valid = sl < g.units;
+    const int u0 = min(sl, g.units - 1);
+    const float *xr = x + (int64_t)in_row * k;
+    float *orow = out + (int64_t)out_row * n;
+    w += (int64_t)e * expert_bytes;
+
+    // the activation load goes out first (vector loads complete in order), then the first weights
+    const int total = k, spans = (k + 255) >> 8;
+    const int xbase = wv * 256 + lane * 4;
+    float xv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (xbase < total) cq_load4<CQ_F32>(xr, xbase, xv);
+    const int step_rows = RPS << g.nw_shift;           // rows the workgroup covers per step
+    int row = wg_row0 + wv * RPS + sub;                // this lane's row of the wave's current step
+    const int base0 = wg_row0 + wv * RPS;
+    const int my_steps = base0 < wg_row1 ? (wg_row1 - base0 + step_rows - 1) / step_rows : 0;
+    const int64_t row_bytes = g.row_bytes;
+    typename F::W wa, wb;
+    F::load_w(wa, w + (int64_t)min(row, n - 1) * row_bytes, u0);
+
+    if (wv < spans) {
+        if (cq_is_kquant(DT)) cq_quantize_q8k_vals(xv, wv, lane, lqs, ld, lbs);
+        else cq_quantize_q80_vals(xv, xbase < total, xbase, lane, lqs, ld);
+    }
+    for (int span = wv + nwaves; span < spans; span += nwaves) {
+        if (cq_is_kquant(DT)) cq_quantize_q8k_span<CQ_F32>(xr, span, lane, lqs, ld, lbs);
+        else cq_quantize_q80_span<CQ_F32>(xr, span, lane, total, lqs, ld);
+    }
+    __syncthreads();
+    if (my_steps == 0) return;
+    typename F::A areg;
+    F::load_a(areg, act_row(lqs, ld, lbs, DT, 0, k), u0);
+
+    if (SWIGLU) {
+        // wa = gate row (in flight), wb = up row; the next gate row is requested before the up row is reduced
+        for (int j = 0; j < my_steps; j++) {
+            const uint8_t *rp = w + (int64_t)min(row, n - 1) * row_bytes;
+            F::load_w(wb, rp + pair_off, u0);
+            float gate = seg_sum_to_last<SEG>(valid ? F::dot(wa, areg, u0) : 0.0f);
+            const int nrow = j + 1 < my_steps ? row + step_rows : row;
+            F::load_w(wa, w + (int64_t)min(nrow, n - 1) * row_bytes, u0);
+            float up = seg_sum_to_last<SEG>(valid ? F::dot(wb, areg, u0) : 0.0f);
+            if (sl == SEG - 1 && row < wg_row1) orow[row] = gate / (1.0f + expf(-gate)) * up;
+            row = nrow;
+        }
+        return;
+    }
+    for (int j = 0; j < my_steps; j += 2) {
+        const int r1 = j + 1 < my_steps ? row + step_rows : row;
+        F::load_w(wb, w + (int64_t)min(r1, n - 1) * row_bytes, u0);
+        float v = seg_sum_to_last<SEG>(valid ? F::dot(wa, areg, u0) : 0.0f);
+        if (sl == SEG - 1 && row < wg_row1) orow[row] = v * scale;
+        if (j + 1 >= my_steps) break;
+        const int r2 = j + 2 < my_steps ? r1 + step_rows : r1;
+        F::load_w(wa, w + (int64_t)min(r2, n - 1) * row_bytes, u0);
+        v = seg_sum_to_last<SEG>(valid ? F::dot(wb, areg, u0) : 0.0f);
+        if (sl == SEG - 1 && r1 < wg_row1) orow[r1] = v * scale;
+        row = r2;
+    }
+}
+
+template <int DT, int SEG>
+int launch_moe_pairs_short(const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s, bool swiglu,
+                           int64_t pair_off) {
+    constexpr int RPS = 64 / SEG;
+    QmvGeom g;
+    int64_t groups;
+    size_t lds_bytes;
+    // the geometry of launch_moe_pairs in units of wave steps (RPS rows each)
+    const int64_t n_steps = (n + RPS - 1) / RPS;
+    int waves = 16;
+    if ((int64_t)ps.n_pairs * n_steps < 256 * 16) {
+        while (waves > 1 && n_steps < 256 * (int64_t)waves) waves >>= 1;
+        // ... but at least one wave per 256-element span of the activation row (up to 8): a lone wave quantizing a
+        // 2048-element row span by span takes longer than the rows it then streams
+        const int64_t spans = (k + 255) / 256;
+        while (waves < 8 && waves < spans) waves <<= 1;
+    }
+    const int64_t per_pair = ((swiglu ? 2048 : 1024) + ps.n_pairs - 1) / ps.n_pairs;
+    int rc = make_geom<DT, 1>(g, groups, waves, k, n_steps, n, CQ_F32, 0, lds_bytes, per_pair < 256 ? per_pair : 256);
+    if (rc) return rc;
+    g.n = (int)n;
+    g.rows_per_wg *= RPS;
+    if (ps.n_pairs > 65535) return CQ_ERR_RANGE;
+    const int64_t expert_bytes = n * (int64_t)g.row_bytes;
+    dim3 grid((unsigned)groups, (unsigned)ps.n_pairs), block(64 * waves);
+    if (swiglu)
+        hipLaunchKernelGGL((moe_pair_short_kernel<DT, SEG, true>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes, pair_off);
+    else
+        hipLaunchKernelGGL((moe_pair_short_kernel<DT, SEG, false>), grid, block, lds_bytes, s, (const uint8_t *)w, x, out, g, ps, expert_bytes, (int64_t)0);
+    return (int)hipGetLastError();
+}
+
 template <int DT>
 int launch_moe_pairs(const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s, bool swiglu = false,
                      int64_t pair_off = 0) {
     if (cq_act_layout(DT, k, 1).total > LDS_BUDGET) return CQ_ERR_RANGE;
     if (swiglu && k / Fmt<DT>::UE > 64) return CQ_ERR_RANGE;         // the paired-row epilogue is for rows of one wave step
+    // short rows: several weight rows per wave step
+    if (k / Fmt<DT>::UE <= 16) return launch_moe_pairs_short<DT, 16>(w, x, out, ps, k, n, s, swiglu, pair_off);
+    if (k / Fmt<DT>::UE <= 32) return launch_moe_pairs_short<DT, 32>(w, x, out, ps, k, n, s, swiglu, pair_off);
     QmvGeom g;
     int64_t groups;
     size_t lds_bytes;
