@@ -995,6 +995,49 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float *__restrict__
     }
 }
 
+// The same routing for up to 256 experts with the row in the registers of one wave (expert e = lane + 64 i): no LDS
+// round trips between the topk rounds and no barrier.  Sums are formed in the order of moe_topk_kernel (64 experts per
+// wave sum, the four sums added in order; the selected probabilities added in slot order), so the two kernels return
+// the same bits.
+__global__ __launch_bounds__(64) void moe_topk_wave_kernel(const float *__restrict__ logits, uint32_t *__restrict__ topk_ids,
+                                                           float *__restrict__ topk_weights, int n_experts, int topk, int renorm) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    float p[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) p[i] = lane + 64 * i < n_experts ? logits[(int64_t)t * n_experts + lane + 64 * i] : -INFINITY;
+    const float m = wave_max(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])));
+    float s4[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const bool live = lane + 64 * i < n_experts;
+        p[i] = live ? expf(p[i] - m) : 0.0f;
+        s4[i] = wave_sum(p[i]);
+    }
+    const float total = s4[0] + s4[1] + s4[2] + s4[3];
+#pragma unroll
+    for (int i = 0; i < 4; i++) p[i] = lane + 64 * i < n_experts ? p[i] / total : -2.0f;     // -2: not selectable
+    float mysel = 0.0f;                                   // lane j keeps the probability of slot j
+    for (int j = 0; j < topk; j++) {
+        const float bv = wave_max(fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), -1.0f));
+        int bi = 0x7fffffff;
+        if (bv > -1.0f) {                                 // uniform
+            int cand = 0x7fffffff;
+#pragma unroll
+            for (int i = 3; i >= 0; i--)
+                if (p[i] == bv) cand = lane + 64 * i;     // the lowest expert among equals
+            bi = wave_min_int(cand);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (lane + 64 * i == bi) p[i] = -2.0f;
+        if (lane == 0) topk_ids[(int64_t)t * topk + j] = (uint32_t)bi;   // no finite probability left (NaN logits): an id no expert has
+        if (lane == j) mysel = bv;
+    }
+    float sum = 0.0f;
+    for (int j = 0; j < topk; j++) sum += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mysel), j));
+    if (lane < topk) topk_weights[(int64_t)t * topk + lane] = renorm ? mysel / sum : mysel;
+}
+
 // (expert_ids, sorted_token_ids) = topk_ids.flatten().sort_last_dim(ascending) (fused_moe.rs:249-260) as a counting
 // sort in one workgroup.  candle's sort is unstable (candle-core/src/sort.rs:282-297), so the order of the pairs
 // inside an expert's segment is unspecified there too; here it depends on the order the LDS atomics are served in.
@@ -1306,8 +1349,12 @@ int cq_nn_moe_route(const float *x_dev, const float *router_w_dev, uint32_t *top
         return CQ_ERR_ALIGN;
     hipLaunchKernelGGL(moe_logits_kernel, dim3((unsigned)((num_experts + 15) / 16), (unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x_dev,
                        router_w_dev, logits_dev, (int)hidden, (int)num_experts);
-    hipLaunchKernelGGL(moe_topk_kernel, dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (const float *)logits_dev, topk_ids_dev,
-                       topk_weights_dev, (int)num_experts, (int)topk, norm_topk_prob);
+    if (num_experts <= 256)
+        hipLaunchKernelGGL(moe_topk_wave_kernel, dim3((unsigned)tokens), dim3(64), 0, (hipStream_t)stream, (const float *)logits_dev, topk_ids_dev,
+                           topk_weights_dev, (int)num_experts, (int)topk, norm_topk_prob);
+    else
+        hipLaunchKernelGGL(moe_topk_kernel, dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (const float *)logits_dev, topk_ids_dev,
+                           topk_weights_dev, (int)num_experts, (int)topk, norm_topk_prob);
     return (int)hipGetLastError();
 }
 

@@ -21,7 +21,8 @@ def L():
     return _lib.lib()
 
 
-@pytest.mark.parametrize("tokens,E,hidden,topk,norm", [(1, 128, 2048, 8, True), (7, 16, 256, 4, False), (300, 64, 512, 6, True), (3, 5, 64, 5, True)])
+@pytest.mark.parametrize("tokens,E,hidden,topk,norm", [(1, 128, 2048, 8, True), (7, 16, 256, 4, False), (300, 64, 512, 6, True), (3, 5, 64, 5, True),
+                                                            (9, 256, 128, 8, True), (5, 300, 128, 8, True), (2, 1000, 64, 60, False)])   # > 256 experts: the LDS kernel
 def test_route_kernel(tokens, E, hidden, topk, norm):
     x, router = normal(1, (tokens, hidden), 1.0), normal(2, (E, hidden), 0.1)
     xd, rd = torch.from_numpy(x).cuda(), torch.from_numpy(router).cuda()
