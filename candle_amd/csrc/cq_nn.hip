@@ -906,34 +906,48 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float *__restric
 // ---- MoE routing around the grouped expert matmuls (FusedMoeGGUF::forward, candle-transformers/src/fused_moe.rs:222-301) ----
 constexpr int ROUTE_MAX_EXPERTS = 1024, ROUTE_MAX_TOPK = 64;
 
-// router_logits = x . router_w^T (a bias-free f32 Linear, :233): a workgroup takes 16 experts of one token, a wave 4
-// of them, with the loads of all four rows in flight together (the router matrix of 128 x 2048 is 1 MB: one workgroup
-// per token walking it row by row would be latency-bound).
+// router_logits = x . router_w^T (a bias-free f32 Linear, :233): a wave takes R experts of one token and walks the rows C
+// column chunks of 256 at a time, every load of a trip issued before the first use (the router matrix of 128 x 2048 is
+// 1 MB: walked chunk by chunk with a wait per chunk it took eight dependent memory trips, 5.2 us for one token).
+// <1, 8>: few tokens, one row per wave, a 2048-element row is one trip; <4, 2>: many tokens, the token's row is loaded once
+// per four experts.  Per lane the products are added in the same order in both, so the logits do not depend on the variant.
+template <int R, int C>
 __global__ __launch_bounds__(256) void moe_logits_kernel(const float *__restrict__ x, const float *__restrict__ router_w, float *__restrict__ logits,
                                                          int hidden, int n_experts) {
     const int t = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const int e0 = blockIdx.x * 16 + wv * 4;
+    const int e0 = (blockIdx.x * 4 + wv) * R;
     if (e0 >= n_experts) return;
     const float *xr = x + (int64_t)t * hidden;
-    const float *w[4];
+    const float *w[R];
 #pragma unroll
-    for (int i = 0; i < 4; i++) w[i] = router_w + (int64_t)min(e0 + i, n_experts - 1) * hidden;
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int k = lane * 4; k < hidden; k += 256) {
-        const f32x4 a = *reinterpret_cast<const f32x4 *>(xr + k);
-        f32x4 b[4];
+    for (int i = 0; i < R; i++) w[i] = router_w + (int64_t)min(e0 + i, n_experts - 1) * hidden;
+    float acc[R];
 #pragma unroll
-        for (int i = 0; i < 4; i++) b[i] = *reinterpret_cast<const f32x4 *>(w[i] + k);
+    for (int i = 0; i < R; i++) acc[i] = 0.0f;
+    for (int k0 = lane * 4; k0 < hidden; k0 += 256 * C) {
+        f32x4 a[C], b[R][C];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            acc[i] = fmaf(a.x, b[i].x, acc[i]);
-            acc[i] = fmaf(a.y, b[i].y, acc[i]);
-            acc[i] = fmaf(a.z, b[i].z, acc[i]);
-            acc[i] = fmaf(a.w, b[i].w, acc[i]);
+        for (int c = 0; c < C; c++) {
+            const int kc = min(k0 + 256 * c, hidden - 4);          // past the end: re-read the last vector, not used below
+            a[c] = *reinterpret_cast<const f32x4 *>(xr + kc);
+#pragma unroll
+            for (int i = 0; i < R; i++) b[i][c] = *reinterpret_cast<const f32x4 *>(w[i] + kc);
+        }
+#pragma unroll
+        for (int c = 0; c < C; c++) {
+            if (k0 + 256 * c < hidden) {
+#pragma unroll
+                for (int i = 0; i < R; i++) {
+                    acc[i] = fmaf(a[c].x, b[i][c].x, acc[i]);
+                    acc[i] = fmaf(a[c].y, b[i][c].y, acc[i]);
+                    acc[i] = fmaf(a[c].z, b[i][c].z, acc[i]);
+                    acc[i] = fmaf(a[c].w, b[i][c].w, acc[i]);
+                }
+            }
         }
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < R; i++) {
         const float v = wave_sum(acc[i]);
         if (lane == 0 && e0 + i < n_experts) logits[(int64_t)t * n_experts + e0 + i] = v;
     }
@@ -1347,8 +1361,12 @@ int cq_nn_moe_route(const float *x_dev, const float *router_w_dev, uint32_t *top
     if (misaligned(x_dev, 16) || misaligned(router_w_dev, 16) || misaligned(topk_ids_dev, 4) || misaligned(topk_weights_dev, 4) ||
         misaligned(logits_dev, 4))
         return CQ_ERR_ALIGN;
-    hipLaunchKernelGGL(moe_logits_kernel, dim3((unsigned)((num_experts + 15) / 16), (unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x_dev,
-                       router_w_dev, logits_dev, (int)hidden, (int)num_experts);
+    if (tokens * num_experts <= 4096)
+        hipLaunchKernelGGL((moe_logits_kernel<1, 8>), dim3((unsigned)((num_experts + 3) / 4), (unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x_dev,
+                           router_w_dev, logits_dev, (int)hidden, (int)num_experts);
+    else
+        hipLaunchKernelGGL((moe_logits_kernel<4, 2>), dim3((unsigned)((num_experts + 15) / 16), (unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x_dev,
+                           router_w_dev, logits_dev, (int)hidden, (int)num_experts);
     if (num_experts <= 256)
         hipLaunchKernelGGL(moe_topk_wave_kernel, dim3((unsigned)tokens), dim3(64), 0, (hipStream_t)stream, (const float *)logits_dev, topk_ids_dev,
                            topk_weights_dev, (int)num_experts, (int)topk, norm_topk_prob);
