@@ -212,3 +212,19 @@ def test_moe_qwen3_shape_single_token():
         want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, None, topk)
         err = rel_l2(got.cpu().numpy(), want)
         assert err <= TOL and err <= TIGHT, err
+
+
+@pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q6K, oracle.Q8_0, oracle.Q3K], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("n,k", [(5, 256), (1, 768), (77, 1024), (130, 2048), (9, 4096)])
+def test_short_expert_rows_ragged(dtype, n, k):
+    """Rows of at most 32 units take several weight rows per wave step (2 or 4); n is not a multiple of either, a single
+    row, and a row length (4096) that stays on the one-row-per-step kernel for K-quants."""
+    E, batch, topk = 3, 3, 2
+    blocks, qt = make_experts(dtype, E, n, k, seed=95)
+    ids = np.array([[0, 2], [1, 1], [2, 0]], dtype=np.uint32)
+    x = normal(96, (batch, topk, k), 1.0)
+    out = qt.indexed_moe_forward(torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda())
+    torch.cuda.synchronize()
+    want = oracle.indexed_moe_forward(dtype, blocks, (E, n, k), x, ids)
+    err = rel_l2(out.cpu().numpy(), want)
+    assert err <= TIGHT, err
