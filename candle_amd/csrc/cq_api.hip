@@ -323,13 +323,18 @@ int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, 
     return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
 }
 
+int cq_moe_direct_pairs(int w_dtype, int64_t num_experts, int64_t size_m, int64_t k) {
+    if (!moe_weight_dtype(w_dtype) || num_experts <= 0 || size_m < 0 || k <= 0) return 0;
+    return cq_moe_direct(w_dtype, num_experts, size_m, k) ? 1 : 0;
+}
+
 int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_dev, const void *w_up_dev, const int32_t *sorted_token_ids_dev,
                             const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
                             int64_t k, void *stream) {
     int rc = moe_weight_dtype(w_dtype) ? check_mm_shape(w_dtype, k, n, size_m) : (int)CQ_ERR_DTYPE;
     if (rc) return rc;
     if (num_experts <= 0 || topk <= 0 || size_m % topk != 0) return CQ_ERR_SHAPE;
-    if (num_experts > (1 << 20) || size_m > CQ_MOE_DIRECT_MAX_PAIRS) return CQ_ERR_RANGE;
+    if (num_experts > (1 << 20) || !cq_moe_direct(w_dtype, num_experts, size_m, k)) return CQ_ERR_RANGE;
     if (size_m == 0 || n == 0) return CQ_OK;
     if ((rc = check_weight_ptr(w_dtype, w_gate_dev)) || (rc = check_weight_ptr(w_dtype, w_up_dev))) return rc;
     if (!x_dev || !sorted_token_ids_dev || !expert_ids_dev || !out_dev) return CQ_ERR_NULL;

@@ -103,8 +103,16 @@ __device__ __forceinline__ bool pair_decode(const PairSource &ps, int p, int &e,
 
 // One workgroup: histogram of experts, exclusive scan, scatter of the pair descriptors.
 
-// Pairs up to which cq_moe_launch runs every pair as its own fused matvec instead of grouping by expert.
+// Pairs up to which cq_moe_launch runs every pair as its own fused matvec instead of grouping by expert: 256 for every
+// shape; up to 512 when the rows are short enough for the several-rows-per-wave-step kernel (at most 32 units) and an expert
+// is hit by three pairs at most on average.  Measured on 128 experts of 768 x 2048 / 2048 x 768, top-8: 256 pairs 99 us per
+// layer of three matmuls, about 3 us per further 8 pairs; the grouped MFMA path 154-163 us for 264-512 pairs.
 #define CQ_MOE_DIRECT_MAX_PAIRS 256
+inline bool cq_moe_direct(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t k) {
+    if (n_pairs <= CQ_MOE_DIRECT_MAX_PAIRS) return true;
+    const int64_t unit = cq_is_kquant(w_dtype) ? 64 : 32;
+    return k / unit <= 32 && n_pairs <= 512 && n_pairs <= 3 * num_experts;
+}
 // CQ_ERR_RANGE when the shape is not served by the fused kernel (the caller then takes the grouped path).
 int cq_moe_pairs_launch(int w_dtype, const void *w, const float *x, float *out, const PairSource &ps, int64_t k, int64_t n, hipStream_t s);
 int cq_moe_pairs_swiglu_launch(int w_dtype, const void *w_gate, const void *w_up, const float *x, float *out, const PairSource &ps, int64_t k,

@@ -208,7 +208,7 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     ps.n_pairs = (int)a.n_pairs; ps.num_experts = (int)a.num_experts; ps.x_rows = (int)a.x_rows;
     // Few pairs (decode): every pair is its own fused matvec (activation quantization in the kernel, no scratch,
     // no grouping pass); an expert hit by two pairs is simply read twice, the second time from cache.
-    if (a.n_pairs <= CQ_MOE_DIRECT_MAX_PAIRS) {
+    if (cq_moe_direct(a.w_dtype, a.num_experts, a.n_pairs, a.k)) {
         int rc = cq_moe_pairs_launch(a.w_dtype, a.w, a.x, a.out, ps, a.k, a.n, s);
         if (rc != CQ_ERR_RANGE) return rc;
     }

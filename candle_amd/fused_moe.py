@@ -90,9 +90,11 @@ class FusedMoeGGUF:
                                                     self.topk_weights.data_ptr() + 4 * t0 * topk, self.router_logits.data_ptr() + 4 * t0 * E,
                                                     t, hidden, E, topk, 1 if self.norm_topk_prob else 0, sp))
         # (expert_ids, sorted_token_ids) of fused_moe.rs:249-260.  The grouped matmuls give every pair its own row whatever
-        # the order of the pairs, and up to 256 pairs each pair is its own matvec launch block, so the sort is skipped there:
-        # the pairs are taken in token order (expert_ids = topk_ids, sorted_token_ids = 0, 1, 2, ...).
-        if pairs <= 256:
+        # the order of the pairs, and decode-sized calls (cq_moe_direct_pairs: up to 256 pairs, 512 for short expert rows) run
+        # each pair as its own matvec launch block, so the sort is skipped there: the pairs are taken in token order
+        # (expert_ids = topk_ids, sorted_token_ids = 0, 1, 2, ...).
+        direct = bool(L.cq_moe_direct_pairs(dt, E, pairs, max(hidden, self.inter)))
+        if direct:
             eid_ptr, sti_ptr = self.topk_ids.data_ptr(), self.pair_iota.data_ptr()
         else:
             ck("cq_nn_moe_sort", L.cq_nn_moe_sort(self.topk_ids.data_ptr(), self.expert_ids.data_ptr(), self.sorted_token_ids.data_ptr(), pairs, E,
@@ -105,7 +107,7 @@ class FusedMoeGGUF:
 
         # decode-sized calls: gate, up and the activation in one launch
         fused = -6
-        if pairs <= 256:
+        if direct:
             fused = L.cq_moe_gemm_gguf_swiglu(dt, x2.data_ptr(), self.gate_experts.device_ptr(), self.up_experts.device_ptr(), sti_ptr, eid_ptr,
                                               self.down_in.data_ptr(), E, topk, pairs, self.inter, hidden, sp)
             if fused != -6:

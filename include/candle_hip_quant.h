@@ -147,7 +147,7 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
  *   w [num_experts, n, k] blocks, x [batch, input_dim1, k] f32 with input_dim1 == topk or 1,
  *   ids [batch, topk] u32  ->  out [batch, topk, n] f32,
  *   out[b, t, :] = W[ids[b, t]] . x[b, input_dim1 == 1 ? 0 : t, :].
- * Up to 256 pairs each pair is its own fused matvec; beyond, pairs are grouped by expert on the device and an expert's
+ * Up to 256 pairs (512 for short rows, see cq_moe_direct_pairs) each pair is its own fused matvec; beyond, pairs are grouped by expert on the device and an expert's
  * rows are streamed once per tile of 32 or 128 pairs on the matrix cores (K-quant experts; integer-exact) or once per
  * 8 pairs by the matvec kernel (the other formats).  The reference takes Q2K-Q6K and Q8_0 experts (cuda.rs:543-548).
  * An id >= num_experts leaves its output row zero-filled.
@@ -187,10 +187,17 @@ int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, 
  * moe_gemm_gguf calls without topk_weights, then up * silu(gate)) in one launch, for decode-sized calls:
  *   out[tok, :] = silu(W_gate[e] . x[tok / topk, :]) * (W_up[e] . x[tok / topk, :])
  * w_gate / w_up [num_experts, n, k] of one format.  CQ_ERR_RANGE (use the two calls and cq_nn_silu_mul) when
- * size_m > 256 or k is longer than one wave step per row (4096 for K-quants, 2048 for Q4_0 / Q8_0).  Needs no workspace. */
+ * cq_moe_direct_pairs() is 0 for the call or k is longer than one wave step per row (4096 for K-quants, 2048 for Q4_0 / Q8_0).
+ * Needs no workspace. */
 int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_dev, const void *w_up_dev, const int32_t *sorted_token_ids_dev,
                             const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
                             int64_t k, void *stream);
+
+/* 1 when a MoE call of size_m pairs runs every pair as its own fused matvec (no grouping by expert, so the order of the
+ * pairs does not matter and a caller may skip its sort): up to 256 pairs always, up to 512 for rows of at most 32 units
+ * (k <= 2048 for K-quants, 1024 otherwise) while size_m <= 3 * num_experts.  No counterpart in the reference, which always
+ * sorts (fused_moe.rs:249-260). */
+int cq_moe_direct_pairs(int w_dtype, int64_t num_experts, int64_t size_m, int64_t k);
 
 /* Measurement aid, no counterpart in the reference: a kernel that only reads `bytes` (a multiple of 16) of a device
  * buffer, with the launch shape of the decode matvec (256 workgroups of 1024 threads).  bench.py times it over the same

@@ -228,3 +228,26 @@ def test_short_expert_rows_ragged(dtype, n, k):
     want = oracle.indexed_moe_forward(dtype, blocks, (E, n, k), x, ids)
     err = rel_l2(out.cpu().numpy(), want)
     assert err <= TIGHT, err
+
+
+@pytest.mark.parametrize("tokens", [40, 48, 49, 64])
+def test_more_than_256_pairs_on_short_rows(tokens):
+    """128 experts, top-8, 768- and 2048-element rows: up to 384 pairs (3 per expert) every pair is still its own matvec
+    block, beyond that the grouped matrix-core path takes over; both give the oracle's values."""
+    import candle_amd as ca
+    E, topk = 128, 8
+    for n, k in ((96, 2048), (160, 768)):
+        blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=97)
+        ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=98 + tokens)
+        x2 = normal(99, (tokens * topk, k), 1.0)
+        twf = tw.reshape(-1)
+        got = ca.moe_gemm_gguf(torch.from_numpy(x2).cuda(), qt, torch.from_numpy(twf).cuda(), torch.from_numpy(sorted_token_ids).cuda(),
+                               torch.from_numpy(expert_ids).cuda(), topk, False)
+        torch.cuda.synchronize()
+        want = oracle.moe_gemm_gguf(oracle.Q4K, x2, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
+        assert rel_l2(got.cpu().numpy(), want) <= TIGHT
+    from candle_amd import _lib
+    L = _lib.lib()
+    assert L.cq_moe_direct_pairs(oracle.Q4K, E, tokens * topk, 2048) == (1 if tokens * topk <= 384 else 0)
+    assert L.cq_moe_direct_pairs(oracle.Q4K, E, tokens * topk, 4096) == 0
+    assert L.cq_moe_direct_pairs(oracle.Q4K, 8, 256, 4096) == 1
