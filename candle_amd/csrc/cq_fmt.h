@@ -495,6 +495,24 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
     return v;
 }
 
+// Four wave sums at once: lane 60 + r ends with the sum of v[r] over the wave (r = 0..3).  Two transposing steps inside
+// the quads leave lane class (lane & 3) = r holding row r's quad sums (one select pair and one DPP add per step instead of
+// one DPP add per row), two row shifts collect the 16-lane rows, two cross-lane reads the four rows of the wave:
+// 15 instructions for four rows where wave_sum_to_lane63 takes 6 (plus their wait states) per row.
+__device__ __forceinline__ float wave_sum4_to_lanes60(float v0, float v1, float v2, float v3, int lane) {
+#define CQ_DPP(x, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xf, 0xf, true))
+    const bool odd = lane & 1, up = lane & 2;
+    const float a = (odd ? v1 : v0) + CQ_DPP((odd ? v0 : v1), CQ_DPP_QUAD_XOR1);     // even lanes: row 0 pairs, odd lanes: row 1 pairs
+    const float b = (odd ? v3 : v2) + CQ_DPP((odd ? v2 : v3), CQ_DPP_QUAD_XOR1);     // rows 2 / 3
+    float c = (up ? b : a) + CQ_DPP((up ? a : b), CQ_DPP_QUAD_XOR2);                 // lane & 3 = r: quad sum of row r
+    c += CQ_DPP(c, CQ_DPP_ROW_SHR(4));
+    c += CQ_DPP(c, CQ_DPP_ROW_SHR(8));                                               // lanes 12..15 of each 16-lane row: its sums
+#undef CQ_DPP
+    c += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, c)));
+    c += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, c)));
+    return c;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Output conversion (the CUDA backend keeps the activation dtype; the CPU f16 path rounds the f32
 // dot product to f16, k_quants.rs:2680-2682).

@@ -416,15 +416,20 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
                         off = live ? (int64_t)fz.row_map[live ? b : 0] * stride_dst : -1;
                         sc = live ? fz.row_scale[live ? b : 0] : 0.0f;
                     }
+                    // the four rows of the block are reduced together: lane 60 + r ends with row r
+                    static_assert(RB == 4, "wave_sum4_to_lanes60 reduces four rows");
+                    float v4[RB];
 #pragma unroll
                     for (int r = 0; r < RB; r++) {
-                        float v = F::dot(wr[BLOCKED ? r : 0], areg[0], u0);
-                        v = wave_sum_to_lane63(valid ? v : 0.0f);
+                        const float v = F::dot(wr[BLOCKED ? r : 0], areg[0], u0);
+                        v4[r] = valid ? v : 0.0f;
+                    }
+                    const float v = wave_sum4_to_lanes60(v4[0], v4[1], v4[2], v4[3], lane);
+                    const int r = lane - 60;
+                    if (r >= 0 && j0 + r < my_rows && off >= 0) {
                         const int rr = row + ((j0 + r) << g.nw_shift);
-                        if (lane == 63 && j0 + r < my_rows && off >= 0) {
-                            if (EPI == EPI_MOE) ((float *)dst)[off + rr] = v * sc;
-                            else store_out(dst, dst_dtype, off + rr, v);
-                        }
+                        if (EPI == EPI_MOE) ((float *)dst)[off + rr] = v * sc;
+                        else store_out(dst, dst_dtype, off + rr, v);
                     }
                 }
             };
