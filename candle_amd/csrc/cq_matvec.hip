@@ -458,6 +458,41 @@ __device__ __forceinline__ void qmv_body(const uint8_t *__restrict__ w, const Ac
             }
             return;
         }
+        if constexpr (DT == CQ_Q6K && NB == 1 && (EPI == EPI_NONE || EPI == EPI_SCALE)) {
+            // Q6_K plain rows: the same ping-pong, but the wave sums of four consecutive rows are formed together
+            // (wave_sum4_to_lanes60) and lanes 60..63 store them at once.  Measured per format on 14336 x 4096: Q6_K
+            // 12.86 -> 12.08 us, Q4_K 8.51 -> 8.59, Q3_K 9.27 -> 9.39: it pays for the longest dot only.
+            for (int j = 0; j < my_rows; j += 4) {
+                float v0 = 0.0f, v1 = 0.0f, v2 = 0.0f, v3 = 0.0f;
+                const uint8_t *p1 = j + 1 < my_rows ? wp + wave_stride : wp;
+                F::load_w(wb, p1, u0);
+                v0 = F::dot(wa, areg[0], u0);
+                wp = p1;
+                if (j + 1 < my_rows) {
+                    const uint8_t *p2 = j + 2 < my_rows ? p1 + wave_stride : p1;
+                    F::load_w(wa, p2, u0);
+                    v1 = F::dot(wb, areg[0], u0);
+                    wp = p2;
+                    if (j + 2 < my_rows) {
+                        const uint8_t *p3 = j + 3 < my_rows ? p2 + wave_stride : p2;
+                        F::load_w(wb, p3, u0);
+                        v2 = F::dot(wa, areg[0], u0);
+                        wp = p3;
+                        if (j + 3 < my_rows) {
+                            const uint8_t *p4 = j + 4 < my_rows ? p3 + wave_stride : p3;
+                            F::load_w(wa, p4, u0);
+                            v3 = F::dot(wb, areg[0], u0);
+                            wp = p4;
+                        }
+                    }
+                }
+                const float c = wave_sum4_to_lanes60(valid ? v0 : 0.0f, valid ? v1 : 0.0f, valid ? v2 : 0.0f, valid ? v3 : 0.0f, lane);
+                const int r = lane - 60;
+                if (r >= 0 && j + r < my_rows) store_out(dst, dst_dtype, row + r * nwaves, EPI == EPI_SCALE ? c * fz.eps : c);
+                row += 4 * nwaves;
+            }
+            return;
+        }
         // ping-pong between wa and wb: the next row's loads are in flight while this one is reduced;
         // the prefetch past the last row re-reads it instead of branching around the load.  The residual
         // value of a row travels behind its weights in the same in-order load queue.
