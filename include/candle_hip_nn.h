@@ -164,7 +164,8 @@ int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int
  *                  topk_weights = those probabilities, divided by their sum when norm_topk_prob (:243-247).
  *                  x [tokens, hidden], router_w [num_experts, hidden], topk_ids u32 / topk_weights f32 [tokens, topk];
  *                  logits_dev [tokens, num_experts] f32 receives the router logits (two launches: the dot products
- *                  spread over tokens x num_experts/16 workgroups, then softmax + top-k per token).
+ *                  spread over tokens x num_experts/16 workgroups — num_experts/4 for few tokens — then softmax + top-k
+ *                  per token, in the registers of one wave when num_experts <= 256).
  *                  num_experts <= 1024, topk <= 64, tokens <= 65535 per call.
  * cq_nn_moe_sort   (expert_ids, sorted_token_ids) = topk_ids.flatten().sort_last_dim(ascending) (:249-260): n_pairs =
  *                  tokens * topk entries each.  The order of the pairs of one expert is unspecified, as it is with
