@@ -32,6 +32,8 @@ SIGNATURES = {
     "cq_matmul": (_int, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "cq_qmatmul_workspace_bytes": (_i64, [_int, _i64, _i64, _i64]),
     "cq_qmatmul_forward": (_int, [_int, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "cq_static_workspace_bytes": (_i64, []),
+    "cq_qmatmul_forward_static": (_int, [_int, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
     "cq_indexed_moe_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _i64]),
     "cq_indexed_moe_forward": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_moe_gemm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _int]),

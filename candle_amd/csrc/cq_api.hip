@@ -4,7 +4,37 @@
 #include "cq_launch.h"
 #include "../../include/candle_hip_nn.h"
 
+#include <mutex>
+
+// Workspace of cq_qmatmul_forward_static: device memory that belongs to the library's code object, so the entry point
+// needs no allocation.  Each GPU the library runs on holds its own copy until the process ends.  In host code the
+// name of the array is not a device address: every use goes through the per-device address that hipGetSymbolAddress
+// returns (static_workspace below).
+static __device__ __align__(256) uint8_t scratch[CQ_STATIC_WORKSPACE_BYTES];
+
 namespace {
+
+constexpr int STATIC_WS_MAX_DEVICES = 64;
+std::mutex static_ws_mutex;
+void *static_ws_ptr[STATIC_WS_MAX_DEVICES];   // per device, filled on the first call made with that device current
+
+// device address of `scratch` on the current device; 0 = ok, else the hipError_t / CQ_ERR_RANGE
+int static_workspace(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= STATIC_WS_MAX_DEVICES) return CQ_ERR_RANGE;
+    std::lock_guard<std::mutex> g(static_ws_mutex);
+    if (!static_ws_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        static_ws_ptr[dev] = p;
+    }
+    *out = static_ws_ptr[dev];
+    return CQ_OK;
+}
 
 inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
@@ -212,6 +242,22 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
         return cq_matmul_launch(w_dtype, w_dev, workspace_dev, (float *)dst_dev, k, n, m, n, s, split_ws);
     if ((rc = cq_matmul_launch(w_dtype, w_dev, workspace_dev, tmp, k, n, m, n, s, split_ws))) return rc;
     return cq_convert_f32_launch(tmp, dst_dev, dst_dtype, m * n, s);
+}
+
+int64_t cq_static_workspace_bytes(void) { return CQ_STATIC_WORKSPACE_BYTES; }
+
+int cq_qmatmul_forward_static(int w_dtype, const void *w_dev, const void *x_dev, int x_dtype, void *dst_dev, int dst_dtype,
+                              int64_t m, int64_t k, int64_t n, void *stream) {
+    int rc = check_mm_shape(w_dtype, k, n, m);
+    if (rc) return rc;
+    // nothing is enqueued for a call that does not fit: the caller falls back to cq_qmatmul_forward with its own workspace
+    if (cq_qmatmul_workspace_bytes(w_dtype, m, k, n) > CQ_STATIC_WORKSPACE_BYTES) return CQ_ERR_RANGE;
+    void *ws = nullptr;
+    if ((rc = static_workspace(&ws))) return rc;
+    // every byte of the workspace that a kernel of this call reads has been written by an earlier kernel of the same
+    // call (quantized activations, then K-split planes, then the f32 result awaiting conversion), so what the previous
+    // call left there needs no clearing
+    return cq_qmatmul_forward(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, m, k, n, ws, CQ_STATIC_WORKSPACE_BYTES, stream);
 }
 
 int cq_nn_qmatmul_swiglu_rows(int w_dtype, const void *w_dev, const float *gate_dev, const float *up_dev, int64_t gate_stride, int64_t up_stride,

@@ -142,6 +142,21 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
                        int64_t m, int64_t k, int64_t n, void *workspace_dev, int64_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * cq_qmatmul_forward without a workspace argument and without any allocation.  No counterpart in the reference (its
+ * scratch is a grow-only buffer that the host allocates, fast_mmvq.rs:44-81): this entry point is for callers that
+ * cannot allocate device memory — code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The workspace is a fixed array of CQ_STATIC_WORKSPACE_BYTES inside the library's device code (one copy per GPU, held
+ * until the process ends; its address is looked up on the first call made with a device current).  Results are those
+ * of cq_qmatmul_forward bit for bit (same kernels).  A call whose cq_qmatmul_workspace_bytes() exceeds the array
+ * returns CQ_ERR_RANGE and enqueues nothing.  All calls on one GPU share the array: calls that may overlap on one GPU
+ * (different streams, different threads) race; serialize them or use cq_qmatmul_forward with separate workspaces.
+ * ------------------------------------------------------------------------------------------- */
+#define CQ_STATIC_WORKSPACE_BYTES (32ll << 20)
+int64_t cq_static_workspace_bytes(void);
+int cq_qmatmul_forward_static(int w_dtype, const void *w_dev, const void *x_dev, int x_dtype, void *dst_dev, int dst_dtype,
+                              int64_t m, int64_t k, int64_t n, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
  * QTensor::indexed_moe_forward (mod.rs:758-784 -> cuda.rs:505-622 ->
  * candle-kernels/src/quantized.cu:4670-4845):
  *   w [num_experts, n, k] blocks, x [batch, input_dim1, k] f32 with input_dim1 == topk or 1,
