@@ -21,6 +21,7 @@
 #include "cq_device.h"
 #include "cq_fmt.h"
 #include "cq_launch.h"
+#include "cq_stream.h"
 
 namespace {
 
@@ -616,6 +617,403 @@ __global__ __launch_bounds__(1024) void qmv2_kernel(const uint8_t *__restrict__ 
         qmv_body<DTB, 1, CQ_F32, SINGLE, PRO, EPI_NONE, false>(wb, src, dstb, gb, fz, blockIdx.x - blocks_a, gridDim.x - blocks_a);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Streaming kernel (cq_stream.h): one lane per super-block, weights copied HBM -> LDS.  Q4_K / Q5_K, one f32 row,
+// the same prologues and epilogues as qmv_body.  Workgroups of QS_NW waves; step s of the weight stream goes to wave
+// (s / grid) % QS_NW of workgroup s % grid, so at any moment the whole chip reads one compact window of the tensor.
+// ---------------------------------------------------------------------------------------------
+constexpr int QS_NW = 8;
+
+template <int DT, int NW, int XS, int MAXB, int PRO, int EPI>
+__device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const float *__restrict__ x, void *__restrict__ dst, const StreamGeom &g,
+                                         const Fuse &fz, const int block, const int nblocks) {
+    typedef StreamFmt<DT> SF;
+    typedef StreamAct<MAXB> SA;
+    constexpr bool RESID = epi_is_resid(EPI);
+    constexpr bool PAIR = EPI == EPI_SWIGLU;               // two weight rows per output row: two slots per wave
+    constexpr int ME = EPI == EPI_RESID_SPLIT ? MAXP : 1;
+    constexpr int SLOT = SF::NLD * 1024;
+    static_assert(PRO != PRO_MERGE || XS <= 2, "the merge prologue holds its partials in registers");
+    // two LDS variables on purpose: the compiler then knows that the LDS copies in flight (into `slots`) never touch
+    // `act` and does not wait for them before the activation accesses
+    extern __shared__ __align__(16) uint8_t slots[];
+    __shared__ __align__(16) uint8_t act[SA::BYTES];
+    __shared__ __align__(16) float red[32];                // [0, 16): sum(x^2) of the prologue, [16, 32): residual^2 of the epilogue
+    static_assert(NW == 8 || NW == 16, "the fixed-order sums below read 8 or 16 slots");
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int k = g.k, n = g.n, bpr = g.bpr;
+
+    // 0. activation loads first (vector loads complete in order: what is asked for after the weights waits for them)
+    f32x4 xt[XS], at[XS];
+    float pp[NPART / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int MS = PRO == PRO_MERGE ? MAXS : 1;
+    MergeRegs<MS> mg[PRO == PRO_MERGE ? XS : 1];
+    constexpr int MP = PRO == PRO_NORM_SPLIT ? MAXP : 1;
+    f32x4 pl[PRO == PRO_NORM_SPLIT ? XS : 1][MP];
+#pragma unroll
+    for (int j = 0; j < XS; j++) {
+        const int sc = min(wv + j * NW, bpr - 1);          // a wave without a span re-reads the last one (and dumps its result)
+        const int base = sc * 256 + lane * 4;
+        if (PRO == PRO_MERGE) {
+            merge_load<MS>(fz, base, true, mg[PRO == PRO_MERGE ? j : 0]);
+        } else {
+            xt[j] = *(const f32x4 *)(x + base);
+            if (PRO != PRO_NONE) at[j] = *(const f32x4 *)(fz.aux + base);
+            if (PRO == PRO_NORM_SPLIT) {
+#pragma unroll
+                for (int sI = 0; sI < MP; sI++) pl[PRO == PRO_NORM_SPLIT ? j : 0][sI] = *(const f32x4 *)(fz.planes + (int64_t)min(sI, fz.n_planes - 1) * k + base);
+            }
+        }
+    }
+    if (PRO == PRO_NORM) {
+#pragma unroll
+        for (int i = 0; i < NPART / 64; i++) pp[i] = fz.part_in[lane + 64 * i];
+    }
+    asm volatile("" ::: "memory");
+
+    // 1. the wave's first step on its way into LDS.  The loads are unconditional: a step that does not exist gets a
+    //    descriptor of zero bytes (its loads read nothing), so that the waits below stay counted waits.
+    uint8_t *slot = slots + wv * (PAIR ? 2 * SLOT : SLOT);
+    int step = wv * nblocks + block;
+    const int sstride = NW * nblocks;
+    const int my = step < g.total_steps ? (g.total_steps - step + sstride - 1) / sstride : 0;
+    auto issue = [&](int st, const uint8_t *wbase, uint8_t *to) {
+        const bool live = st < g.total_steps;
+        const int64_t off = (int64_t)(live ? st : 0) * g.step_bytes;
+        const int64_t left = g.w_bytes - off;
+        const int bytes = live ? (int)(left < g.step_bytes ? left : g.step_bytes) : 0;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(wbase + off), 0, bytes, 0x00020000);
+#pragma unroll
+        for (int j = 0; j < SF::NLD; j++) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(to + j * 1024), 16, lane * 16, j * 1024, 0, 0);
+    };
+    issue(step, w, slot);
+    if (PAIR) issue(step, w + fz.pair_off, slot + SLOT);
+    asm volatile("" ::: "memory");
+
+    // 2. activations -> LDS
+    float pm = 1.0f;
+    if (PRO == PRO_NORM) {
+        const float sum2 = wave_sum((pp[0] + pp[1]) + (pp[2] + pp[3]));      // fixed order: the same bits in every wave and replay
+        pm = sqrtf(sum2 / (float)k + fz.eps);
+    }
+    float xv[XS][4];
+#pragma unroll
+    for (int j = 0; j < XS; j++) {
+        if (PRO == PRO_MERGE) {
+            merge_reduce<MS>(mg[PRO == PRO_MERGE ? j : 0], true, xv[j]);
+        } else {
+            xv[j][0] = xt[j].x; xv[j][1] = xt[j].y; xv[j][2] = xt[j].z; xv[j][3] = xt[j].w;
+        }
+    }
+    if (PRO == PRO_NORM_SPLIT) {
+        // the merged row (absent planes count as zeros) and sum(x^2) over the whole row, in a fixed order
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < XS; j++) {
+            const bool own = wv + j * NW < bpr;
+#pragma unroll
+            for (int sI = 0; sI < MP; sI++) {
+                const f32x4 t = pl[PRO == PRO_NORM_SPLIT ? j : 0][sI];
+                const bool on = sI < fz.n_planes;
+                xv[j][0] += on ? t.x : 0.0f; xv[j][1] += on ? t.y : 0.0f; xv[j][2] += on ? t.z : 0.0f; xv[j][3] += on ? t.w : 0.0f;
+            }
+            const float s4 = (xv[j][0] * xv[j][0] + xv[j][1] * xv[j][1]) + (xv[j][2] * xv[j][2] + xv[j][3] * xv[j][3]);
+            ss += own ? wave_sum(s4) : 0.0f;
+        }
+        if (lane == 0) red[wv] = ss;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        const f32x4 r0 = ((const f32x4 *)red)[0], r1 = ((const f32x4 *)red)[1];
+        float sum2 = ((r0.x + r0.y) + (r0.z + r0.w)) + ((r1.x + r1.y) + (r1.z + r1.w));
+        if (NW == 16) {
+            const f32x4 r2 = ((const f32x4 *)red)[2], r3 = ((const f32x4 *)red)[3];
+            sum2 += ((r2.x + r2.y) + (r2.z + r2.w)) + ((r3.x + r3.y) + (r3.z + r3.w));
+        }
+        pm = sqrtf(sum2 / (float)k + fz.eps);
+    }
+#pragma unroll
+    for (int j = 0; j < XS; j++) {
+        const float a4[4] = {at[j].x, at[j].y, at[j].z, at[j].w};
+        if (PRO == PRO_NORM || PRO == PRO_SILU) pro_apply<PRO>(xv[j], a4, pm);
+        if (PRO == PRO_NORM_SPLIT) pro_apply<PRO_NORM>(xv[j], a4, pm);
+        const int span = wv + j * NW;
+        qs_quantize_span(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
+    }
+    // a barrier without the fence of __syncthreads(): the fence would wait for the LDS copies in flight
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // 3. the lane's place: row `rin` of the step, super-block `sb` of the row; its activations stay in registers
+    const int lp = 1 << g.lp_shift;
+    const int rin = lane >> g.lp_shift, sb = lane & (lp - 1);
+    const bool valid_sb = sb < bpr;
+    const int sbc = valid_sb ? sb : bpr - 1;
+    u32x4 areg[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) areg[i] = *(const u32x4 *)(act + sbc * QS_ACT_STRIDE + 16 * i);
+    const u32x4 aux0 = *(const u32x4 *)(act + SA::AUX_OFF + sbc * QS_AUX_STRIDE), aux1 = *(const u32x4 *)(act + SA::AUX_OFF + sbc * QS_AUX_STRIDE + 16);
+    const float d8 = __uint_as_float(aux0.x);
+    const int boff = (rin * bpr + sbc) * SF::BB;
+    const bool last = sb == lp - 1;                     // this lane ends up with the row's sum
+    float ssq = 0.0f;
+
+    for (int it = 0; it < my; it++, step += sstride) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's copies have landed
+        const int row = step * g.step_rows + rin;
+        const bool store = last && row < n;
+        // the residual value (and the planes to add to it) travels in front of the next step's copies
+        float rv = 0.0f, pv[ME];
+        if (RESID) {
+            const int rc = min(row, n - 1);
+            rv = fz.resid[rc];
+            if (EPI == EPI_RESID_SPLIT) {
+#pragma unroll
+                for (int sI = 0; sI < ME; sI++) pv[sI] = fz.planes[(int64_t)min(sI, fz.n_planes - 1) * n + rc];
+            }
+        }
+        typename SF::Blk b0, b1;
+        SF::read(b0, slot + boff);
+        if (PAIR) SF::read(b1, slot + SLOT + boff);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // every lane has its block in registers: the slot is free
+        issue(step + sstride, w, slot);
+        if (PAIR) issue(step + sstride, w + fz.pair_off, slot + SLOT);
+        asm volatile("" ::: "memory");
+        float r = SF::dot(b0, areg, d8, aux1);
+        r = qs_group_sum(valid_sb ? r : 0.0f, g.lp_shift);
+        if (PAIR) {
+            float u = SF::dot(b1, areg, d8, aux1);
+            u = qs_group_sum(valid_sb ? u : 0.0f, g.lp_shift);
+            if (store) store_out(dst, g.dst_dtype, row, r / (1.0f + expf(-r)) * u);      // Mlp::forward, quantized_llama.rs:56-63
+        } else if (RESID) {
+            if (store) {
+                if (EPI == EPI_RESID_SPLIT) {
+#pragma unroll
+                    for (int sI = 0; sI < ME; sI++) rv += sI < fz.n_planes ? pv[sI] : 0.0f;
+                }
+                const float sres = rv + r;                     // (x + residual), quantized_llama.rs:584,591
+                fz.resid[row] = sres;
+                ssq += sres * sres;
+            }
+        } else if (store) {
+            store_out(dst, g.dst_dtype, row, EPI == EPI_SCALE ? r * fz.eps : r);
+        }
+    }
+    if (RESID) {
+        // the workgroup's partial of sum(residual^2), added in a fixed order; block 0 clears the unused slots
+        ssq = wave_sum(ssq);
+        if (lane == 0) red[16 + wv] = ssq;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (tid == 0) {
+            const f32x4 r0 = ((const f32x4 *)red)[4], r1 = ((const f32x4 *)red)[5];
+            float t = ((r0.x + r0.y) + (r0.z + r0.w)) + ((r1.x + r1.y) + (r1.z + r1.w));
+            if (NW == 16) {
+                const f32x4 r2 = ((const f32x4 *)red)[6], r3 = ((const f32x4 *)red)[7];
+                t += ((r2.x + r2.y) + (r2.z + r2.w)) + ((r3.x + r3.y) + (r3.z + r3.w));
+            }
+            fz.part_out[block] = t;
+        }
+        if (block == 0)
+            for (int i = nblocks + tid; i < NPART; i += NW * 64) fz.part_out[i] = 0.0f;
+    }
+}
+
+// Kernel arguments of the streaming kernel, packed: every pointer and scalar a (PRO, EPI) pair does not use is left
+// out and the launch geometry is derived from (n, super-blocks per row) in the kernel.  What a kernel reads of its
+// argument block should lie in the first 64 bytes: a read from the next 64 (explicit arguments, or the hidden ones
+// behind them that gridDim / blockDim come from) is a second trip to memory before anything else can start
+// (measured on the 33 MB matvec: 7.67 us per launch with 56 bytes of arguments, 7.96 us with 60).
+__host__ __device__ constexpr int qs_groups(int total_steps) { return total_steps < 256 ? total_steps : 256; }
+constexpr int qs_pro_ptrs(int pro) { return pro == PRO_NORM || pro == PRO_NORM_SPLIT ? 3 : pro == PRO_SILU ? 2 : 1; }
+constexpr int qs_epi_ptrs(int epi) { return epi == EPI_RESID ? 2 : epi == EPI_RESID_SPLIT ? 3 : 1; }
+constexpr bool qs_has_f(int pro, int epi) { return pro == PRO_NORM || pro == PRO_NORM_SPLIT || epi == EPI_SCALE; }
+template <int PRO, int EPI> struct QsArgs {
+    static constexpr int NP = 1 + qs_pro_ptrs(PRO) + qs_epi_ptrs(EPI);
+    static constexpr int NI = 2 + (qs_has_f(PRO, EPI) ? 1 : 0) + (EPI == EPI_SWIGLU ? 1 : 0);
+    const void *p[NP];     // w | PRO_NONE: x; NORM: x, norm weight, partial sums; SILU: x, up; MERGE: partials; NORM_SPLIT: x, norm weight, planes
+                           //   | EPI_NONE / SCALE / SWIGLU: dst; RESID: residual, partial sums out; RESID_SPLIT: residual, partial sums out, planes
+    int i[NI];             // n | bpr + (dst_dtype << 8) + (n_planes << 16) + (splits << 20) + (hd_shift << 26) | eps or scale | pair distance / 16
+};
+
+template <int DT, int PRO, int EPI>
+QsArgs<PRO, EPI> qs_pack(const void *w, const float *x, void *dst, const StreamGeom &g, const Fuse &fz) {
+    QsArgs<PRO, EPI> a;
+    int np = 0;
+    a.p[np++] = w;
+    if (PRO != PRO_MERGE) a.p[np++] = x;
+    if (PRO != PRO_NONE) a.p[np++] = fz.aux;
+    if (PRO == PRO_NORM) a.p[np++] = fz.part_in;
+    if (PRO == PRO_NORM_SPLIT) a.p[np++] = fz.planes;
+    if (epi_is_resid(EPI)) {
+        a.p[np++] = fz.resid;
+        a.p[np++] = fz.part_out;
+        if (EPI == EPI_RESID_SPLIT) a.p[np++] = fz.planes;
+    } else {
+        a.p[np++] = dst;
+    }
+    int ni = 0;
+    a.i[ni++] = g.n;
+    a.i[ni++] = g.bpr | (g.dst_dtype << 8) | (fz.n_planes << 16) | (fz.splits << 20) | (fz.hd_shift << 26);
+    if (qs_has_f(PRO, EPI)) a.i[ni++] = __builtin_bit_cast(int, fz.eps);
+    if (EPI == EPI_SWIGLU) a.i[ni++] = (int)(fz.pair_off / 16);
+    return a;
+}
+
+template <int DT, int PRO, int EPI>
+__device__ __forceinline__ void qs_unpack(const QsArgs<PRO, EPI> &a, const uint8_t *&w, const float *&x, void *&dst, StreamGeom &g, Fuse &fz) {
+    int np = 0;
+    w = (const uint8_t *)a.p[np++];
+    x = PRO != PRO_MERGE ? (const float *)a.p[np++] : nullptr;
+    fz.aux = PRO != PRO_NONE ? (const float *)a.p[np++] : nullptr;
+    fz.part_in = PRO == PRO_NORM ? (const float *)a.p[np++] : nullptr;
+    fz.planes = PRO == PRO_NORM_SPLIT ? (const float *)a.p[np++] : nullptr;
+    dst = nullptr; fz.resid = nullptr; fz.part_out = nullptr;
+    if (epi_is_resid(EPI)) {
+        fz.resid = (float *)a.p[np++];
+        fz.part_out = (float *)a.p[np++];
+        if (EPI == EPI_RESID_SPLIT) fz.planes = (const float *)a.p[np++];
+    } else {
+        dst = (void *)a.p[np++];
+    }
+    int ni = 0;
+    const int n = a.i[ni++];
+    const uint32_t meta = (uint32_t)a.i[ni++];
+    fz.eps = qs_has_f(PRO, EPI) ? __builtin_bit_cast(float, a.i[ni++]) : 0.0f;
+    fz.pair_off = EPI == EPI_SWIGLU ? (int64_t)a.i[ni++] * 16 : 0;
+    fz.n_planes = (meta >> 16) & 15; fz.splits = (meta >> 20) & 63; fz.hd_shift = meta >> 26;
+    fz.row_map = nullptr; fz.row_scale = nullptr; fz.nvalid = 0;
+    const int bpr = meta & 255;
+    g.k = bpr * 256; g.n = n; g.bpr = bpr;
+    g.lp_shift = bpr > 1 ? 32 - __builtin_clz(bpr - 1) : 0;
+    g.step_rows = 64 >> g.lp_shift;
+    g.step_bytes = g.step_rows * bpr * StreamFmt<DT>::BB;
+    g.total_steps = (n + g.step_rows - 1) >> (6 - g.lp_shift);
+    g.dst_dtype = (meta >> 8) & 255; g.stride_dst = n;
+    g.w_bytes = (int64_t)n * (bpr * StreamFmt<DT>::BB);
+}
+
+template <int DT, int XS, int MAXB, int PRO, int EPI>
+__global__ __launch_bounds__(QS_NW * 64) void qms_kernel(QsArgs<PRO, EPI> a) {
+    const uint8_t *w; const float *x; void *dst; StreamGeom g; Fuse fz;
+    qs_unpack<DT, PRO, EPI>(a, w, x, dst, g, fz);
+    // the grid size is derived, not read: gridDim comes from the hidden arguments behind the explicit ones, and every
+    // argument byte a kernel reads beyond the first 64 costs a second trip at its start
+    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
+}
+
+// Two weight tensors over the same activation row in one launch, tensor A on the streaming body; tensor B on the
+// streaming body as well (SB) or on qmv_body.  Workgroups [0, blocks_a) take tensor A.  NW waves per workgroup: 8, or
+// 16 where qmv_body needs one wave per activation span (its plane-merging prologue).
+// Arguments of the two-tensor launch, 60 bytes: tensor B and its output are given as distances from tensor A's.
+struct Qs2Args {
+    const uint8_t *wa; const float *x, *aux, *extra; float *dsta;      // extra: partial sums (PRO_NORM) or planes (PRO_NORM_SPLIT)
+    int na, nb;
+    uint32_t meta;            // bpr | blocks_a << 8 | blocks_b << 16 | n_planes << 24
+    float eps;
+    int wb_off16;             // (wb - wa) / 16
+    int dstb_off;             // dstb - dsta, in floats
+};
+template <int DTA, int DTB, int NW, int XS, int MAXB, bool SINGLE, int PRO, bool SB>
+__global__ __launch_bounds__(NW * 64) void qms2_kernel(Qs2Args a) {
+    const int blocks_a = (a.meta >> 8) & 255, blocks_b = (a.meta >> 16) & 255, bpr = a.meta & 255;
+    Fuse fz{a.aux, PRO == PRO_NORM ? a.extra : nullptr, a.eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0, PRO == PRO_NORM_SPLIT ? a.extra : nullptr,
+            (int)(a.meta >> 24)};
+    const bool first = (int)blockIdx.x < blocks_a;
+    if (first || SB) {
+        const int n = first ? a.na : a.nb;
+        StreamGeom g;
+        g.k = bpr * 256; g.n = n; g.bpr = bpr;
+        g.lp_shift = bpr > 1 ? 32 - __builtin_clz(bpr - 1) : 0;
+        g.step_rows = 64 >> g.lp_shift;
+        g.dst_dtype = CQ_F32; g.stride_dst = n;
+        g.total_steps = (n + g.step_rows - 1) >> (6 - g.lp_shift);
+        if (first) {
+            g.step_bytes = g.step_rows * bpr * StreamFmt<DTA>::BB;
+            g.w_bytes = (int64_t)n * (bpr * StreamFmt<DTA>::BB);
+            qms_body<DTA, NW, XS, MAXB, PRO, EPI_NONE>(a.wa, a.x, a.dsta, g, fz, blockIdx.x, blocks_a);
+        } else if constexpr (SB) {
+            g.step_bytes = g.step_rows * bpr * StreamFmt<DTB>::BB;
+            g.w_bytes = (int64_t)n * (bpr * StreamFmt<DTB>::BB);
+            qms_body<DTB, NW, XS, MAXB, PRO, EPI_NONE>(a.wa + (int64_t)a.wb_off16 * 16, a.x, a.dsta + a.dstb_off, g, fz, blockIdx.x - blocks_a, blocks_b);
+        }
+    } else if constexpr (!SB) {
+        // tensor B on qmv_body: its geometry as make_geom() lays it out for NW waves and blocks_b workgroups
+        QmvGeom gb;
+        const int k = bpr * 256, n = a.nb;
+        const int rows_per_wg = (n + blocks_b - 1) / blocks_b;
+        const ActLayout L = cq_act_layout(DTB, k, 1);
+        gb.k = k; gb.n = n; gb.rows_per_wg = rows_per_wg;
+        gb.units = k / UnitFmt<DTB, 1, SINGLE>::type::UE; gb.steps = (gb.units + 63) >> 6;
+        gb.lds_d_off = (int)L.d_off; gb.lds_bs_off = (int)L.bs_off;
+        gb.nw_shift = NW == 16 ? 4 : 3;
+        gb.row_bytes = (k / BlockInfo<DTB>::elems) * BlockInfo<DTB>::bytes;
+        gb.lds_red_off = (int)L.total;
+        gb.dst_dtype = CQ_F32; gb.stride_dst = n;
+        ActSrc src{a.x, ActView{nullptr, nullptr, nullptr}};
+        qmv_body<DTB, 1, CQ_F32, SINGLE, PRO, EPI_NONE, false>(a.wa + (int64_t)a.wb_off16 * 16, src, a.dsta + a.dstb_off, gb, fz, blockIdx.x - blocks_a, blocks_b);
+    }
+}
+
+// Does the streaming kernel take this (format, k, n)?  Rows of a power of two of super-blocks (up to 64) fill every
+// lane; other row lengths put one row on a wave step and need at least three quarters of the lanes busy.
+template <int DT>
+bool stream_geom(StreamGeom &g, int64_t k, int64_t n, int dst_dtype) {
+    if (DT != CQ_Q4K && DT != CQ_Q5K) return false;
+    if (k % 256 || k <= 0 || n < 64) return false;
+    const int64_t bpr = k / 256;
+    if (bpr > 64) return false;
+    int sh = 0;
+    while ((1 << sh) < bpr) sh++;
+    if ((1 << sh) != bpr && 4 * bpr < 3 * (1 << sh)) return false;
+    const int64_t bb = BlockInfo<DT>::bytes;
+    g.k = (int)k; g.n = (int)n; g.bpr = (int)bpr; g.lp_shift = sh;
+    g.step_rows = 64 >> sh;
+    g.step_bytes = (int)(g.step_rows * bpr * bb);
+    g.total_steps = (int)((n + g.step_rows - 1) / g.step_rows);
+    g.dst_dtype = dst_dtype; g.stride_dst = n;
+    g.w_bytes = n * bpr * bb;
+    return n <= 0x7fffffff / 64;
+}
+
+template <int DT, int XS, int MAXB, int PRO, int EPI>
+int launch_stream_xs(const void *w, const float *x, void *dst, const StreamGeom &g, hipStream_t s, const Fuse &fz) {
+    constexpr bool PAIR = EPI == EPI_SWIGLU;
+    const size_t lds_bytes = (size_t)QS_NW * StreamFmt<DT>::NLD * 1024 * (PAIR ? 2 : 1);
+    if (lds_bytes + StreamAct<MAXB>::BYTES + 64 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
+    auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    const int groups = qs_groups(g.total_steps);
+    if (fz.pair_off % 16 || fz.n_planes > 15 || fz.splits > 63 || g.dst_dtype > 255) return CQ_ERR_RANGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * QS_NW), lds_bytes, s, qs_pack<DT, PRO, EPI>(w, x, dst, g, fz));
+    return (int)hipGetLastError();
+}
+
+// CQ_ERR_RANGE: not a shape (or fusion) of the streaming kernel; the caller takes qmv_kernel
+template <int DT, int PRO, int EPI>
+int launch_stream(const void *w, const float *x, void *dst, int dst_dtype, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
+    if constexpr (DT != CQ_Q4K && DT != CQ_Q5K) {
+        return CQ_ERR_RANGE;
+    } else {
+        StreamGeom g;
+        if (!stream_geom<DT>(g, k, n, dst_dtype)) return CQ_ERR_RANGE;
+        if (epi_is_resid(EPI) && n > (int64_t)256 * 64 * 1024) return CQ_ERR_RANGE;
+        const int bpr = g.bpr;
+        if constexpr (PRO == PRO_MERGE || EPI == EPI_SWIGLU) {
+            // rows of up to 4096 elements (as in qmv_kernel): the merge holds two spans of partials per wave, the paired rows two slots
+            if (bpr > 16) return CQ_ERR_RANGE;
+            if (bpr <= 8) return launch_stream_xs<DT, 1, 16, PRO, EPI>(w, x, dst, g, s, fz);
+            return launch_stream_xs<DT, 2, 16, PRO, EPI>(w, x, dst, g, s, fz);
+        } else {
+            if (bpr <= 8) return launch_stream_xs<DT, 1, 16, PRO, EPI>(w, x, dst, g, s, fz);
+            if (bpr <= 16) return launch_stream_xs<DT, 2, 16, PRO, EPI>(w, x, dst, g, s, fz);
+            if (bpr <= 32) return launch_stream_xs<DT, 4, 64, PRO, EPI>(w, x, dst, g, s, fz);
+            if (bpr <= 56) return launch_stream_xs<DT, 7, 64, PRO, EPI>(w, x, dst, g, s, fz);
+            return launch_stream_xs<DT, 8, 64, PRO, EPI>(w, x, dst, g, s, fz);
+        }
+    }
+}
+
 // Geometry of one launch.  waves == 0: as many waves per workgroup (a power of two, at most 16) as still leave every
 // wave a row when 256 workgroups are launched; otherwise the given wave count is used.
 template <int DT, int NB>
@@ -774,6 +1172,14 @@ int cq_matvec_launch(int w_dtype, const void *w, const void *scratch, void *dst,
 int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *dst, int dst_dtype, int64_t k, int64_t n,
                            int64_t rows, int64_t stride_dst, hipStream_t s) {
     if (n == 0 || rows == 0) return CQ_OK;
+    if (rows == 1 && x_dtype == CQ_F32) {
+        // one f32 row over Q4_K / Q5_K weights: the streaming kernel where it takes the shape
+        const Fuse none{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
+        int rc = CQ_ERR_RANGE;
+        if (w_dtype == CQ_Q4K) rc = launch_stream<CQ_Q4K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
+        if (w_dtype == CQ_Q5K) rc = launch_stream<CQ_Q5K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
     const int64_t xsz = x_dtype == CQ_F32 ? 4 : 2, esz = dst_dtype == CQ_F32 ? 4 : 2;
     return for_row_groups(w_dtype, k, rows, [&](int64_t r0, int64_t nb) {
         ActSrc src;
@@ -793,6 +1199,11 @@ namespace {
 template <int DT, int PRO, int EPI>
 int launch_fused1(const void *w, const ActSrc &src, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
     if (cq_act_layout(DT, k, 1).total + 64 > LDS_BUDGET) return CQ_ERR_RANGE;
+    // the plane-merging prologue keeps its range (rows of one wave step of qmv_kernel) whichever kernel runs
+    if (!pro_is_split(PRO) || k / Fmt<DT>::UE <= 64) {
+        const int rc = launch_stream<DT, PRO, EPI>(w, (const float *)src.x, dst, CQ_F32, k, n, s, fz);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
     if (k / Fmt<DT>::UE <= 64) return launch_cfg<DT, 1, CQ_F32, true, PRO, EPI>(w, src, dst, CQ_F32, k, n, n, s, fz);
     if constexpr (pro_is_split(PRO)) {
         return CQ_ERR_RANGE;                                 // one span per wave: rows of one wave step only
@@ -854,6 +1265,11 @@ template <int DT>
 int launch_merge1(const void *w, void *dst, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
     if (k / Fmt<DT>::UE > 64) return CQ_ERR_RANGE;          // one wave step per row, one span per wave
     ActSrc src{nullptr, ActView{nullptr, nullptr, nullptr}};
+    {
+        const int rc = fz.n_planes > 0 ? launch_stream<DT, PRO_MERGE, EPI_RESID_SPLIT>(w, nullptr, dst, CQ_F32, k, n, s, fz)
+                                       : launch_stream<DT, PRO_MERGE, EPI_RESID>(w, nullptr, dst, CQ_F32, k, n, s, fz);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
     if (fz.n_planes > 0) return launch_cfg<DT, 1, CQ_F32, true, PRO_MERGE, EPI_RESID_SPLIT>(w, src, dst, CQ_F32, k, n, n, s, fz);
     return launch_cfg<DT, 1, CQ_F32, true, PRO_MERGE, EPI_RESID>(w, src, dst, CQ_F32, k, n, n, s, fz);
 }
@@ -885,13 +1301,111 @@ template <int DT>
 int launch_swiglu1(const void *w1, int64_t pair_off, const ActSrc &src, float *dst, int64_t k, int64_t ffn, hipStream_t s, Fuse fz) {
     if (k / Fmt<DT>::UE > 64) return CQ_ERR_RANGE;
     fz.pair_off = pair_off;
+    {
+        const int rc = launch_stream<DT, PRO_NORM, EPI_SWIGLU>(w1, (const float *)src.x, dst, CQ_F32, k, ffn, s, fz);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
     return launch_cfg<DT, 1, CQ_F32, true, PRO_NORM, EPI_SWIGLU>(w1, src, dst, CQ_F32, k, ffn, ffn, s, fz);
+}
+
+// The two-tensor launch with tensor A (and tensor B, when its format and shape allow) on the streaming body.
+// CQ_ERR_RANGE: tensor A is not a shape of the streaming kernel.
+template <int DTA, int DTB, int NW, int XS, int MAXB, int PRO>
+int launch_pair_stream_xs(const void *wa, float *dsta, const void *wb, int64_t nb, float *dstb, const float *x, int64_t k, hipStream_t s,
+                          const Fuse &fz, const StreamGeom &ga, bool sb, const StreamGeom &gsb) {
+    constexpr int XL = pro_is_split(PRO) ? 64 : 0;
+    // 256 workgroups in total, shared between the tensors in proportion to their bytes
+    const double bytes_a = (double)ga.n * BlockInfo<DTA>::bytes / BlockInfo<DTA>::elems, bytes_b = (double)nb * BlockInfo<DTB>::bytes / BlockInfo<DTB>::elems;
+    int64_t share_a = (int64_t)(256.0 * bytes_a / (bytes_a + bytes_b) + 0.5);
+    if (share_a < 1) share_a = 1;
+    if (share_a > 255) share_a = 255;
+    const int64_t groups_a = ga.total_steps < share_a ? ga.total_steps : share_a;
+    QmvGeom gb{};
+    int64_t groups_b;
+    size_t lds_b = 0;
+    if (sb) {
+        groups_b = gsb.total_steps < 256 - share_a ? gsb.total_steps : 256 - share_a;
+    } else {
+        int waves = NW;
+        const int rc = make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, XL, lds_b, 256 - share_a);
+        if (rc) return rc;
+    }
+    const size_t lds_a = (size_t)NW * StreamFmt<DTA>::NLD * 1024;
+    const size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
+    if (lds_bytes + StreamAct<MAXB>::BYTES + 256 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
+    const bool single = k / 64 <= 64;
+    // tensor B and its output travel as 32-bit distances from tensor A's; a launch they do not fit takes qmv2_kernel
+    const int64_t wdist = (const uint8_t *)wb - (const uint8_t *)wa, ddist = dstb - dsta;
+    if (wdist % 16 || wdist / 16 > 0x7fffffffLL || wdist / 16 < -0x7fffffffLL || ddist > 0x7fffffffLL || ddist < -0x7fffffffLL) return CQ_ERR_RANGE;
+    if (groups_a > 255 || groups_b > 255 || groups_b < 1 || fz.n_planes > 15) return CQ_ERR_RANGE;
+    if (!sb) {
+        // qmv_body's geometry is rebuilt in the kernel from (nb, blocks_b): it must be what make_geom() returned
+        const int64_t rpw = (nb + groups_b - 1) / groups_b;
+        if (gb.rows_per_wg != rpw || (nb + rpw - 1) / rpw != groups_b) return CQ_ERR_RANGE;
+    }
+    Qs2Args a;
+    a.wa = (const uint8_t *)wa; a.x = x; a.aux = fz.aux; a.extra = PRO == PRO_NORM ? fz.part_in : fz.planes; a.dsta = dsta;
+    a.na = ga.n; a.nb = (int)nb;
+    a.meta = (uint32_t)ga.bpr | ((uint32_t)groups_a << 8) | ((uint32_t)groups_b << 16) | ((uint32_t)fz.n_planes << 24);
+    a.eps = fz.eps; a.wb_off16 = (int)(wdist / 16); a.dstb_off = (int)ddist;
+    dim3 grid((unsigned)(groups_a + groups_b)), block(64 * NW);
+    auto go = [&](auto kern) {
+        if (lds_bytes > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return (int)e;
+        }
+        hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, a);
+        return (int)hipGetLastError();
+    };
+    if constexpr (DTB == DTA) {
+        if (sb) return go(qms2_kernel<DTA, DTB, NW, XS, MAXB, true, PRO, true>);
+    }
+    if (single) return go(qms2_kernel<DTA, DTB, NW, XS, MAXB, true, PRO, false>);
+    return go(qms2_kernel<DTA, DTB, NW, XS, MAXB, false, PRO, false>);
+}
+
+template <int DTA, int DTB, int PRO>
+int launch_pair_stream(const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const float *x, int64_t k, hipStream_t s,
+                       const Fuse &fz) {
+    StreamGeom ga;
+    if (!stream_geom<DTA>(ga, k, na, CQ_F32)) return CQ_ERR_RANGE;
+    const int bpr = ga.bpr;
+    if (bpr > 16) return CQ_ERR_RANGE;            // longer rows: the two-tensor launch of qmv_kernel
+    StreamGeom gsb = ga;
+    bool sb = false;
+    if constexpr (DTB == DTA) sb = stream_geom<DTB>(gsb, k, nb, CQ_F32);
+    if (pro_is_split(PRO) && !sb) {
+        // qmv_body merges the planes with one activation span per wave: sixteen waves (and one span per wave here too)
+        if (StreamFmt<DTA>::NLD * 16 * 1024 + StreamAct<16>::BYTES + 256 > LDS_BUDGET) return CQ_ERR_RANGE;
+        return launch_pair_stream_xs<DTA, DTB, 16, 1, 16, PRO>(wa, dsta, wb, nb, dstb, x, k, s, fz, ga, sb, gsb);
+    }
+    if (bpr <= 8) return launch_pair_stream_xs<DTA, DTB, QS_NW, 1, 16, PRO>(wa, dsta, wb, nb, dstb, x, k, s, fz, ga, sb, gsb);
+    return launch_pair_stream_xs<DTA, DTB, QS_NW, 2, 16, PRO>(wa, dsta, wb, nb, dstb, x, k, s, fz, ga, sb, gsb);
 }
 
 template <int DTA, int DTB, int PRO>
 int launch_pair(const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const ActSrc &src, int64_t k, hipStream_t s,
                 const Fuse &fz_in) {
     constexpr int XL = pro_is_split(PRO) ? 64 : 0;
+    if constexpr (DTA == CQ_Q4K || DTA == CQ_Q5K || DTB == CQ_Q4K || DTB == CQ_Q5K) {
+        // rows the streaming kernel takes but its two-tensor launch does not (more than 4096 elements): two launches,
+        // each on the kernel a single call would get
+        StreamGeom gt;
+        const bool sa = stream_geom<DTA>(gt, k, na, CQ_F32), sbb = stream_geom<DTB>(gt, k, nb, CQ_F32);
+        if ((sa || sbb) && k / 256 > 16) {
+            const int rc = launch_fused1<DTA, PRO, EPI_NONE>(wa, src, dsta, k, na, s, fz_in);
+            return rc ? rc : launch_fused1<DTB, PRO, EPI_NONE>(wb, src, dstb, k, nb, s, fz_in);
+        }
+    }
+    if constexpr (DTA != CQ_Q4K && DTA != CQ_Q5K && (DTB == CQ_Q4K || DTB == CQ_Q5K)) {
+        // only tensor B has a streaming body: the same launch with the tensors exchanged
+        StreamGeom gt;
+        if (stream_geom<DTB>(gt, k, nb, CQ_F32) && gt.bpr <= 16) return launch_pair<DTB, DTA, PRO>(wb, nb, dstb, wa, na, dsta, src, k, s, fz_in);
+    }
+    if constexpr (DTA == CQ_Q4K || DTA == CQ_Q5K) {
+        const int rc = launch_pair_stream<DTA, DTB, PRO>(wa, na, dsta, wb, nb, dstb, (const float *)src.x, k, s, fz_in);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
     QmvGeom ga, gb;
     int64_t groups_a, groups_b;
     size_t lds_a, lds_b;

@@ -1,0 +1,210 @@
+// Streaming decode matvec for Q4_K / Q5_K weights and one f32 activation row:  dst[row] = sum_k W[row, k] * x^[k].
+//
+// The weights of a tensor are one contiguous stream of super-blocks (rows follow each other without gaps).  A wave
+// step is a run of that stream — 64 super-blocks when a row has a power of two of them, else one row — copied
+// HBM -> LDS as it lies in memory by buffer loads that write LDS directly (16 bytes per lane, whole cache lines
+// per instruction, no registers in between).  Each lane then reads ITS OWN super-block out of LDS and does the
+// whole block: the 6-bit scales and mins are decoded four at a time, the eight sub-block dots are plain
+// v_dot4_i32_i8 chains, and only the lanes of one row are added up (DPP, log2(lanes per row) steps).  Per weight
+// row this is about half the vector instructions of the four-lanes-per-super-block kernel (qmv_kernel), where every
+// lane decodes its own pair of scales and every row pays a six-step wave reduction.
+//
+// Why LDS copies and not register loads: vector loads are issued in order and block the wave's instruction stream
+// while the memory pipeline is full, so loads requested ahead of time delay the arithmetic queued behind them.
+// A copy into LDS needs no destination registers and no instruction after it until the data is used; the wave
+// asks for its next step as soon as it has moved the current block from LDS to registers, before the arithmetic.
+//
+// Same arithmetic contract as qmv_kernel: activations quantized to Q8_K exactly like BlockQ8K::from_float
+// (candle-core/src/quantized/k_quants.rs:2320-2358), integer dots exact, one f32 scaling per super-block
+// (vec_dot Q4_K x Q8_K k_quants.rs:1460-1540, Q5_K :1714-1801); only the f32 summation order differs.
+#pragma once
+#include "cq_actquant.h"
+#include "cq_device.h"
+
+namespace {
+
+typedef __attribute__((address_space(3))) void cq_lds_void;
+
+// Quantized activations in LDS: per 256-element span 272 bytes of int8 (256 + 16: the sixteen lanes of a row read
+// sixteen different spans at once, a stride of 256 bytes would put them all on the same banks) and a 32-byte record
+//   f32 d | 12 bytes unused | u8 bl[8] | i8 bh[8]      with  sum of sub-block j = 128 * bh[j] + bl[j],  0 <= bl[j] < 128
+// (the sums of the eight 32-element sub-blocks split into two int8 halves, so that sum_j min_j * sum_j is two dot4).
+constexpr int QS_ACT_STRIDE = 272;
+constexpr int QS_AUX_STRIDE = 32;
+template <int MAXB> struct StreamAct {
+    static constexpr int AUX_OFF = (MAXB + 1) * QS_ACT_STRIDE;                     // one more span: the dump for waves without a span
+    static constexpr int BYTES = AUX_OFF + (MAXB + 1) * QS_AUX_STRIDE;
+};
+
+__device__ __forceinline__ uint32_t qs_wave_umax(uint32_t v) {
+    // unsigned max through DPP (fused into v_max_u32_dpp); non-negative floats order like their bit patterns
+#define CQ_S(ctrl, rm, bc) v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, ctrl, rm, 0xf, bc))
+    CQ_S(0x111, 0xf, true); CQ_S(0x112, 0xf, true); CQ_S(0x114, 0xf, true); CQ_S(0x118, 0xf, true);
+    CQ_S(0x142, 0xa, false); CQ_S(0x143, 0xc, false);
+#undef CQ_S
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// One wave quantizes one 256-element span (lane l holds elements 4l .. 4l+3) into the LDS layout above.
+// BlockQ8K::from_float takes the FIRST element of largest magnitude for the scale; here any element of that
+// magnitude is taken: with another sign d and every q flip together and every product d * q is the same value, so
+// no result of the matvec depends on it.  NaN / Inf inputs follow the CPU arithmetic (round, saturating cast, NaN -> 0).
+__device__ __forceinline__ void qs_quantize_span(const float v[4], int span, int lane, uint8_t *act, int aux_off) {
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    amax = amax == amax ? amax : 0.0f;                // four NaNs: the CPU's `amax < |x|` never takes a NaN either
+    const uint32_t wmax = qs_wave_umax(__float_as_uint(amax));
+    const float cand = fabsf(v[0]) == amax ? v[0] : fabsf(v[1]) == amax ? v[1] : fabsf(v[2]) == amax ? v[2] : v[3];
+    const uint64_t who = __builtin_amdgcn_ballot_w64(__float_as_uint(amax) == wmax);    // never empty: compared as bit patterns
+    const int src = __builtin_ctzll(who);
+    const float maxv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cand), src));
+    uint32_t packed = 0;
+    float d = 0.0f;
+    if (wmax != 0) {
+        const float iscale = -127.0f / maxv;
+#pragma unroll
+        for (int i = 0; i < 4; i++) packed |= (uint32_t)(cq_round_sat_i8(iscale * v[i]) & 0xff) << (8 * i);
+        d = 1.0f / iscale;
+    }
+    *(uint32_t *)(act + span * QS_ACT_STRIDE + lane * 4) = packed;
+    int s = sdot4(packed, 0x01010101u, 0);
+    s = oct_sum(s);                                   // sum of the 32-element sub-block, in all eight lanes
+    uint8_t *aux = act + aux_off + span * QS_AUX_STRIDE;
+    if ((lane & 7) == 0) {
+        aux[16 + (lane >> 3)] = (uint8_t)(s & 127);
+        aux[24 + (lane >> 3)] = (uint8_t)(s >> 7);    // arithmetic shift: 128 * bh + bl == s for negative sums too
+    }
+    if (lane == 0) *(float *)aux = d;
+}
+
+// ---- per-format work of one lane on one super-block held in LDS --------------------------------------------
+template <int DT> struct StreamFmt;
+
+// sum over 32 bytes (8 dwords) of low / high nibbles against two 32-element activation sub-blocks
+__device__ __forceinline__ void qs_dot_pair_q4(const u32x4 q0, const u32x4 q1, const u32x4 a0, const u32x4 a1, const u32x4 a2, const u32x4 a3,
+                                               int &dl, int &dh) {
+    const uint32_t M4 = 0x0f0f0f0fu;
+    dl = 0; dh = 0;
+    dl = sdot4(q0.x & M4, a0.x, dl); dl = sdot4(q0.y & M4, a0.y, dl); dl = sdot4(q0.z & M4, a0.z, dl); dl = sdot4(q0.w & M4, a0.w, dl);
+    dl = sdot4(q1.x & M4, a1.x, dl); dl = sdot4(q1.y & M4, a1.y, dl); dl = sdot4(q1.z & M4, a1.z, dl); dl = sdot4(q1.w & M4, a1.w, dl);
+    // high nibbles without a shift: (q ^ 0x80) & 0xf0 is the int8 value 16 * (hi - 8) (one v_bitop3_b32), so the chain
+    // sums 16 * (hi - 8) * a; the caller adds 8 * sum(a) back through the sub-block sums
+#define CQ_HI(v) (((v) ^ 0x80808080u) & 0xf0f0f0f0u)
+    dh = sdot4(CQ_HI(q0.x), a2.x, dh); dh = sdot4(CQ_HI(q0.y), a2.y, dh); dh = sdot4(CQ_HI(q0.z), a2.z, dh); dh = sdot4(CQ_HI(q0.w), a2.w, dh);
+    dh = sdot4(CQ_HI(q1.x), a3.x, dh); dh = sdot4(CQ_HI(q1.y), a3.y, dh); dh = sdot4(CQ_HI(q1.z), a3.z, dh); dh = sdot4(CQ_HI(q1.w), a3.w, dh);
+#undef CQ_HI
+    dh >>= 4;                                          // exact: every term is a multiple of 16
+}
+
+// scales / mins of the eight sub-blocks, four to a dword (get_scale_min_k4, candle-core/src/quantized/utils.rs:50-60)
+struct QsScales { uint32_t scA, scB, mA, mB; };
+__device__ __forceinline__ QsScales qs_scales_k4(uint32_t u0, uint32_t u1, uint32_t u2) {
+    QsScales s;
+    s.scA = u0 & 0x3f3f3f3fu;
+    s.mA = u1 & 0x3f3f3f3fu;
+    s.scB = (u2 & 0x0f0f0f0fu) | ((u0 >> 2) & 0x30303030u);
+    s.mB = ((u2 >> 4) & 0x0f0f0f0fu) | ((u1 >> 2) & 0x30303030u);
+    return s;
+}
+
+// sum_j c_j * (128 * bh_j + bl_j) for the eight byte coefficients (cA: j = 0..3, cB: j = 4..7); aux = {blA, blB, bhA, bhB}
+__device__ __forceinline__ int qs_dot_sums(uint32_t cA, uint32_t cB, const u32x4 aux) {
+    return (sdot4(cB, aux.w, sdot4(cA, aux.z, 0)) << 7) + sdot4(cB, aux.y, sdot4(cA, aux.x, 0));
+}
+
+template <> struct StreamFmt<CQ_Q4K> {
+    static constexpr int BB = 144;             // bytes of a super-block
+    static constexpr int NLD = 9;              // 16-byte-per-lane loads that cover 64 super-blocks
+    struct Blk { u32x4 hdr; u32x4 q[8]; };
+    static __device__ __forceinline__ void read(Blk &b, const uint8_t *p) {
+        b.hdr = *(const u32x4 *)p;
+#pragma unroll
+        for (int i = 0; i < 8; i++) b.q[i] = *(const u32x4 *)(p + 16 + 16 * i);
+    }
+    // a[16]: the lane's 256 int8 activations; aux0.x = d8, aux1 = sub-block sums
+    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float d8, const u32x4 aux1) {
+        int D[8];
+#pragma unroll
+        for (int g = 0; g < 4; g++) qs_dot_pair_q4(b.q[2 * g], b.q[2 * g + 1], a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3], D[2 * g], D[2 * g + 1]);
+        const QsScales s = qs_scales_k4(b.hdr.y, b.hdr.z, b.hdr.w);
+        int S = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            S += __mul24((int)((s.scA >> (8 * j)) & 0xff), D[j]);
+            S += __mul24((int)((s.scB >> (8 * j)) & 0xff), D[4 + j]);
+        }
+        // the odd sub-blocks came out as sum (hi - 8) * a: add 8 * sc_j * sum_j(a)
+        S += qs_dot_sums(s.scA & 0xff00ff00u, s.scB & 0xff00ff00u, aux1) << 3;
+        const int M = qs_dot_sums(s.mA, s.mB, aux1);
+        return d8 * (h2f(b.hdr.x) * (float)S - h2f(b.hdr.x >> 16) * (float)M);
+    }
+};
+
+template <> struct StreamFmt<CQ_Q5K> {
+    static constexpr int BB = 176;
+    static constexpr int NLD = 11;
+    struct Blk { u32x4 hdr; u32x4 h[2]; u32x4 q[8]; };
+    static __device__ __forceinline__ void read(Blk &b, const uint8_t *p) {
+        b.hdr = *(const u32x4 *)p;
+        b.h[0] = *(const u32x4 *)(p + 16);
+        b.h[1] = *(const u32x4 *)(p + 32);
+#pragma unroll
+        for (int i = 0; i < 8; i++) b.q[i] = *(const u32x4 *)(p + 48 + 16 * i);
+    }
+    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float d8, const u32x4 aux1) {
+        const uint32_t M4 = 0x0f0f0f0fu;
+        const uint32_t h[8] = {b.h[0].x, b.h[0].y, b.h[0].z, b.h[0].w, b.h[1].x, b.h[1].y, b.h[1].z, b.h[1].w};
+        int D[8];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            // bytes 32g .. 32g+31 of qs: low nibbles + bit 2g of qh -> sub-block 2g, high nibbles + bit 2g+1 -> sub-block 2g+1
+            const uint32_t q[8] = {b.q[2 * g].x, b.q[2 * g].y, b.q[2 * g].z, b.q[2 * g].w, b.q[2 * g + 1].x, b.q[2 * g + 1].y, b.q[2 * g + 1].z, b.q[2 * g + 1].w};
+            const uint32_t al[8] = {a[4 * g].x, a[4 * g].y, a[4 * g].z, a[4 * g].w, a[4 * g + 1].x, a[4 * g + 1].y, a[4 * g + 1].z, a[4 * g + 1].w};
+            const uint32_t ah[8] = {a[4 * g + 2].x, a[4 * g + 2].y, a[4 * g + 2].z, a[4 * g + 2].w, a[4 * g + 3].x, a[4 * g + 3].y, a[4 * g + 3].z, a[4 * g + 3].w};
+            int dl = 0, dh = 0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint32_t hb = h[i] >> (2 * g);
+                dl = sdot4((q[i] & M4) | ((hb & 0x01010101u) << 4), al[i], dl);
+                dh = sdot4(((q[i] >> 4) & M4) | ((hb << 3) & 0x10101010u), ah[i], dh);
+            }
+            D[2 * g] = dl; D[2 * g + 1] = dh;
+        }
+        const QsScales s = qs_scales_k4(b.hdr.y, b.hdr.z, b.hdr.w);
+        int S = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            S += __mul24((int)((s.scA >> (8 * j)) & 0xff), D[j]);
+            S += __mul24((int)((s.scB >> (8 * j)) & 0xff), D[4 + j]);
+        }
+        const int M = qs_dot_sums(s.mA, s.mB, aux1);
+        return d8 * (h2f(b.hdr.x) * (float)S - h2f(b.hdr.x >> 16) * (float)M);
+    }
+};
+
+// Geometry of one launch, computed on the host.
+struct StreamGeom {
+    int k, n;
+    int bpr;              // super-blocks per row
+    int lp_shift;         // log2(lanes per row): lanes per row = bpr rounded up to a power of two
+    int step_rows;        // rows per wave step = 64 >> lp_shift
+    int step_bytes;       // step_rows * bpr * BB
+    int total_steps;      // ceil(n / step_rows)
+    int dst_dtype;
+    int64_t stride_dst;   // unused by one-row launches, kept for symmetry with QmvGeom
+    int64_t w_bytes;      // n * bpr * BB
+};
+
+// sum over aligned groups of 1 << lp_shift lanes; the last lane of each group ends with the group's sum
+__device__ __forceinline__ float qs_group_sum(float v, int lp_shift) {
+#define CQ_A(ctrl, rm, bc) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, rm, 0xf, bc))
+    if (lp_shift >= 1) CQ_A(0x111, 0xf, true);
+    if (lp_shift >= 2) CQ_A(0x112, 0xf, true);
+    if (lp_shift >= 3) CQ_A(0x114, 0xf, true);
+    if (lp_shift >= 4) CQ_A(0x118, 0xf, true);
+    if (lp_shift >= 5) CQ_A(0x142, 0xa, false);
+    if (lp_shift >= 6) CQ_A(0x143, 0xc, false);
+#undef CQ_A
+    return v;
+}
+
+}  // namespace
