@@ -624,13 +624,18 @@ __global__ __launch_bounds__(1024) void qmv2_kernel(const uint8_t *__restrict__ 
 // ---------------------------------------------------------------------------------------------
 constexpr int QS_NW = 8;
 
-template <int DT, int NW, int XS, int MAXB, int PRO, int EPI>
+template <int DT, int NW, int XS, int MAXB, int PRO, int EPI, int MSP = MAXS>
 __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const float *__restrict__ x, void *__restrict__ dst, const StreamGeom &g,
                                          const Fuse &fz, const int block, const int nblocks) {
     typedef StreamFmt<DT> SF;
     typedef StreamAct<MAXB> SA;
     constexpr bool RESID = epi_is_resid(EPI);
-    constexpr bool PAIR = EPI == EPI_SWIGLU;               // two weight rows per output row: two slots per wave
+    constexpr bool PAIR = EPI == EPI_SWIGLU;               // two weight rows per output row: a step is two sub-steps, gate rows then up rows
+    constexpr int SUBS = PAIR ? 2 : 1;
+    // 16-byte-per-lane copies of the first step requested before the activation prologue; the rest follows it.
+    // Requests beyond what the memory pipeline takes at once block the wave's instruction stream, and the prologue
+    // queued behind them would wait for the weights instead of running under their latency.
+    constexpr int PRE = NW == 16 ? 2 : 4;
     constexpr int ME = EPI == EPI_RESID_SPLIT ? MAXP : 1;
     constexpr int SLOT = SF::NLD * 1024;
     static_assert(PRO != PRO_MERGE || XS <= 2, "the merge prologue holds its partials in registers");
@@ -647,7 +652,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     // 0. activation loads first (vector loads complete in order: what is asked for after the weights waits for them)
     f32x4 xt[XS], at[XS];
     float pp[NPART / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
-    constexpr int MS = PRO == PRO_MERGE ? MAXS : 1;
+    constexpr int MS = PRO == PRO_MERGE ? MSP : 1;         // splits the merge prologue holds (the launch picks the smallest that fits)
     MergeRegs<MS> mg[PRO == PRO_MERGE ? XS : 1];
     constexpr int MP = PRO == PRO_NORM_SPLIT ? MAXP : 1;
     f32x4 pl[PRO == PRO_NORM_SPLIT ? XS : 1][MP];
@@ -674,21 +679,24 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
 
     // 1. the wave's first step on its way into LDS.  The loads are unconditional: a step that does not exist gets a
     //    descriptor of zero bytes (its loads read nothing), so that the waits below stay counted waits.
-    uint8_t *slot = slots + wv * (PAIR ? 2 * SLOT : SLOT);
-    int step = wv * nblocks + block;
+    uint8_t *slot = slots + wv * SLOT;
+    const int step0 = wv * nblocks + block;
     const int sstride = NW * nblocks;
-    const int my = step < g.total_steps ? (g.total_steps - step + sstride - 1) / sstride : 0;
-    auto issue = [&](int st, const uint8_t *wbase, uint8_t *to) {
-        const bool live = st < g.total_steps;
+    const int my = step0 < g.total_steps ? (g.total_steps - step0 + sstride - 1) / sstride : 0;
+    // sub-step t of this wave: step step0 + (t / SUBS) * sstride, of the gate tensor (even t) or the up tensor (odd t)
+    auto issue = [&](int t, int j0, int j1) {
+        const int st = step0 + (PAIR ? t >> 1 : t) * sstride;
+        const uint8_t *wbase = PAIR && (t & 1) ? w + fz.pair_off : w;
+        const bool live = t < SUBS * my;
         const int64_t off = (int64_t)(live ? st : 0) * g.step_bytes;
         const int64_t left = g.w_bytes - off;
         const int bytes = live ? (int)(left < g.step_bytes ? left : g.step_bytes) : 0;
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(wbase + off), 0, bytes, 0x00020000);
 #pragma unroll
-        for (int j = 0; j < SF::NLD; j++) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(to + j * 1024), 16, lane * 16, j * 1024, 0, 0);
+        for (int j = 0; j < SF::NLD; j++)
+            if (j >= j0 && j < j1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(slot + j * 1024), 16, lane * 16, j * 1024, 0, 0);
     };
-    issue(step, w, slot);
-    if (PAIR) issue(step, w + fz.pair_off, slot + SLOT);
+    issue(0, 0, PRE);
     asm volatile("" ::: "memory");
 
     // 2. activations -> LDS
@@ -739,6 +747,8 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         const int span = wv + j * NW;
         qs_quantize_span(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
     }
+    asm volatile("" ::: "memory");
+    issue(0, PRE, SF::NLD);
     // a barrier without the fence of __syncthreads(): the fence would wait for the LDS copies in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
@@ -756,8 +766,10 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     const bool last = sb == lp - 1;                     // this lane ends up with the row's sum
     float ssq = 0.0f;
 
-    for (int it = 0; it < my; it++, step += sstride) {
+    float gate = 0.0f;
+    for (int t = 0; t < SUBS * my; t++) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's copies have landed
+        const int step = step0 + (PAIR ? t >> 1 : t) * sstride;
         const int row = step * g.step_rows + rin;
         const bool store = last && row < n;
         // the residual value (and the planes to add to it) travels in front of the next step's copies
@@ -770,19 +782,19 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
                 for (int sI = 0; sI < ME; sI++) pv[sI] = fz.planes[(int64_t)min(sI, fz.n_planes - 1) * n + rc];
             }
         }
-        typename SF::Blk b0, b1;
+        typename SF::Blk b0;
         SF::read(b0, slot + boff);
-        if (PAIR) SF::read(b1, slot + SLOT + boff);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // every lane has its block in registers: the slot is free
-        issue(step + sstride, w, slot);
-        if (PAIR) issue(step + sstride, w + fz.pair_off, slot + SLOT);
+        issue(t + 1, 0, SF::NLD);
         asm volatile("" ::: "memory");
         float r = SF::dot(b0, areg, d8, aux1);
         r = qs_group_sum(valid_sb ? r : 0.0f, g.lp_shift);
         if (PAIR) {
-            float u = SF::dot(b1, areg, d8, aux1);
-            u = qs_group_sum(valid_sb ? u : 0.0f, g.lp_shift);
-            if (store) store_out(dst, g.dst_dtype, row, r / (1.0f + expf(-r)) * u);      // Mlp::forward, quantized_llama.rs:56-63
+            if (t & 1) {
+                if (store) store_out(dst, g.dst_dtype, row, gate / (1.0f + expf(-gate)) * r);      // Mlp::forward, quantized_llama.rs:56-63
+            } else {
+                gate = r;
+            }
         } else if (RESID) {
             if (store) {
                 if (EPI == EPI_RESID_SPLIT) {
@@ -890,13 +902,13 @@ __device__ __forceinline__ void qs_unpack(const QsArgs<PRO, EPI> &a, const uint8
     g.w_bytes = (int64_t)n * (bpr * StreamFmt<DT>::BB);
 }
 
-template <int DT, int XS, int MAXB, int PRO, int EPI>
+template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP>
 __global__ __launch_bounds__(QS_NW * 64) void qms_kernel(QsArgs<PRO, EPI> a) {
     const uint8_t *w; const float *x; void *dst; StreamGeom g; Fuse fz;
     qs_unpack<DT, PRO, EPI>(a, w, x, dst, g, fz);
     // the grid size is derived, not read: gridDim comes from the hidden arguments behind the explicit ones, and every
     // argument byte a kernel reads beyond the first 64 costs a second trip at its start
-    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
+    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
 }
 
 // Two weight tensors over the same activation row in one launch, tensor A on the streaming body; tensor B on the
@@ -973,12 +985,11 @@ bool stream_geom(StreamGeom &g, int64_t k, int64_t n, int dst_dtype) {
     return n <= 0x7fffffff / 64;
 }
 
-template <int DT, int XS, int MAXB, int PRO, int EPI>
+template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP = 1>
 int launch_stream_xs(const void *w, const float *x, void *dst, const StreamGeom &g, hipStream_t s, const Fuse &fz) {
-    constexpr bool PAIR = EPI == EPI_SWIGLU;
-    const size_t lds_bytes = (size_t)QS_NW * StreamFmt<DT>::NLD * 1024 * (PAIR ? 2 : 1);
-    if (lds_bytes + StreamAct<MAXB>::BYTES + 64 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
-    auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI>;
+    const size_t lds_bytes = (size_t)QS_NW * StreamFmt<DT>::NLD * 1024;
+    if (lds_bytes + StreamAct<MAXB>::BYTES + 256 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
+    auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI, MSP>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
@@ -987,6 +998,14 @@ int launch_stream_xs(const void *w, const float *x, void *dst, const StreamGeom 
     if (fz.pair_off % 16 || fz.n_planes > 15 || fz.splits > 63 || g.dst_dtype > 255) return CQ_ERR_RANGE;
     hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * QS_NW), lds_bytes, s, qs_pack<DT, PRO, EPI>(w, x, dst, g, fz));
     return (int)hipGetLastError();
+}
+
+// the merge prologue in the smallest capacity that holds the launch's splits
+template <int DT, int XS, int EPI>
+int launch_stream_merge(const void *w, void *dst, const StreamGeom &g, hipStream_t s, const Fuse &fz) {
+    if (fz.splits <= 4) return launch_stream_xs<DT, XS, 16, PRO_MERGE, EPI, 4>(w, nullptr, dst, g, s, fz);
+    if (fz.splits <= 8) return launch_stream_xs<DT, XS, 16, PRO_MERGE, EPI, 8>(w, nullptr, dst, g, s, fz);
+    return launch_stream_xs<DT, XS, 16, PRO_MERGE, EPI, MAXS>(w, nullptr, dst, g, s, fz);
 }
 
 // CQ_ERR_RANGE: not a shape (or fusion) of the streaming kernel; the caller takes qmv_kernel
@@ -999,9 +1018,13 @@ int launch_stream(const void *w, const float *x, void *dst, int dst_dtype, int64
         if (!stream_geom<DT>(g, k, n, dst_dtype)) return CQ_ERR_RANGE;
         if (epi_is_resid(EPI) && n > (int64_t)256 * 64 * 1024) return CQ_ERR_RANGE;
         const int bpr = g.bpr;
-        if constexpr (PRO == PRO_MERGE || EPI == EPI_SWIGLU) {
-            // rows of up to 4096 elements (as in qmv_kernel): the merge holds two spans of partials per wave, the paired rows two slots
+        if constexpr (PRO == PRO_MERGE) {
+            // rows of up to 4096 elements (as in qmv_kernel): the merge holds two spans of partials per wave
             if (bpr > 16) return CQ_ERR_RANGE;
+            if (bpr <= 8) return launch_stream_merge<DT, 1, EPI>(w, dst, g, s, fz);
+            return launch_stream_merge<DT, 2, EPI>(w, dst, g, s, fz);
+        } else if constexpr (EPI == EPI_SWIGLU) {
+            if (bpr > 16) return CQ_ERR_RANGE;                 // the range of the paired-row launch of qmv_kernel
             if (bpr <= 8) return launch_stream_xs<DT, 1, 16, PRO, EPI>(w, x, dst, g, s, fz);
             return launch_stream_xs<DT, 2, 16, PRO, EPI>(w, x, dst, g, s, fz);
         } else {
