@@ -608,18 +608,24 @@ __global__ __launch_bounds__(HD) void attn_combine_kernel(const float *__restric
 //   * a workgroup is 16 waves over one split of 128 keys, so a wave scores 8 keys and accumulates 8 values, and
 //     every K and V row is requested before anything is consumed (one memory round trip);
 //   * the result is left as per-split partials { acc[HD], m, l, 0, 0 } (stride HD + 4 floats, 16-byte aligned
-//     rows); attn_merge_kernel, or the prologue of the attention_wo matvec, merges them.
-constexpr int ATTD_WAVES = 16;
+//     rows); the last workgroup of each kv head, or the prologue of the attention_wo matvec, merges them.
 constexpr int ATTD_MAX_SPLITS = 16;
+constexpr int ATTD_COUNTER_BYTES = 256;       // arrival counters of the in-kernel merge, one int per kv head, behind the partials
+// Keys per split: 64 (workgroups of 8 waves) while that gives at most ATTD_MAX_SPLITS splits, else 128 (16 waves).  The
+// vector memory pipeline of a CU takes one instruction of a wave per 16 cycles whatever it loads, and a split asks for
+// about 28 of them per wave: with 128-key splits of 16 waves the 48 workgroups of a 768-key step spent 3 us getting
+// their loads accepted; twice the workgroups of half the size halve that.
+__host__ __device__ inline int64_t attd_split_keys(int64_t max_kv_len) { return (max_kv_len + 63) / 64 <= ATTD_MAX_SPLITS ? 64 : 128; }
+__host__ __device__ inline int64_t attd_splits(int64_t max_kv_len) { const int64_t sk = attd_split_keys(max_kv_len); return (max_kv_len + sk - 1) / sk; }
 
-template <int HD, int G>
-__global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
+template <int HD, int G, int NW, int SPLIT>
+__global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
                                                                       const float *__restrict__ v_new, float *k_cache, float *v_cache,
                                                                       const float *__restrict__ cos_t, const float *__restrict__ sin_t,
                                                                       float *__restrict__ part, const int32_t *__restrict__ pos_dev, int pos0,
                                                                       int ctx, float scale, int splits, const u32x4 *__restrict__ pf,
-                                                                      int64_t pf_chunks, uint32_t *__restrict__ pf_sink) {
-    constexpr int NW = ATTD_WAVES;
+                                                                      int64_t pf_chunks, uint32_t *__restrict__ pf_sink, float *__restrict__ out,
+                                                                      int *__restrict__ counters) {
     if ((int)blockIdx.y >= splits) {
         // Workgroups beyond the attention splits only read: they pull the weights the following kernels will stream
         // (attention_wo, feed_forward_w1 / w3) through the memory-side cache while this latency-bound kernel leaves
@@ -638,16 +644,16 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
         if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
         return;
     }
-    constexpr int DPL = HD / 64, EPL = HD / 16, IT = ATT_SPLIT / (4 * NW), VU = ATT_SPLIT / NW;
-    __shared__ float sc[G * ATT_SPLIT];
+    constexpr int DPL = HD / 64, EPL = HD / 16, IT = SPLIT / (4 * NW), VU = SPLIT / NW;
+    __shared__ float sc[G * SPLIT];
     __shared__ float red[NW * G * HD];
     __shared__ float ml[2 * G];
     const int kvh = blockIdx.x, sp = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int p = min(pos0 + (pos_dev ? pos_dev[0] : 0), ctx - 1);
     const int kv_len = p + 1;
-    const int j0 = sp * ATT_SPLIT;
-    const int cnt = min(kv_len - j0, ATT_SPLIT);
+    const int j0 = sp * SPLIT;
+    const int cnt = min(kv_len - j0, SPLIT);
     const int last = max(cnt - 1, 0);
     float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
     const int sub = lane & 15, kq = lane >> 4;
@@ -683,10 +689,17 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
     }
     // cos / sin of position p for this lane's EPL/2 pairs
     float cs[EPL / 2], sn[EPL / 2];
+    if constexpr (EPL / 2 == 4) {
+        const f32x4 c4 = *reinterpret_cast<const f32x4 *>(cos_t + (int64_t)p * (HD / 2) + 4 * sub);
+        const f32x4 s4 = *reinterpret_cast<const f32x4 *>(sin_t + (int64_t)p * (HD / 2) + 4 * sub);
+        cs[0] = c4.x; cs[1] = c4.y; cs[2] = c4.z; cs[3] = c4.w;
+        sn[0] = s4.x; sn[1] = s4.y; sn[2] = s4.z; sn[3] = s4.w;
+    } else {
 #pragma unroll
-    for (int c = 0; c < EPL / 2; c++) {
-        cs[c] = cos_t[(int64_t)p * (HD / 2) + (EPL / 2) * sub + c];
-        sn[c] = sin_t[(int64_t)p * (HD / 2) + (EPL / 2) * sub + c];
+        for (int c = 0; c < EPL / 2; c++) {
+            cs[c] = cos_t[(int64_t)p * (HD / 2) + (EPL / 2) * sub + c];
+            sn[c] = sin_t[(int64_t)p * (HD / 2) + (EPL / 2) * sub + c];
+        }
     }
     auto rope4 = [&](f32x4 &v, int c) {       // two interleaved pairs (rotary_emb.rs:52-70)
         const float a = v.x * cs[2 * c] - v.y * sn[2 * c], b = v.x * sn[2 * c] + v.y * cs[2 * c];
@@ -720,7 +733,7 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
                 a += qf[g][c].w * kd[it][c].w;
             }
             a = row16_sum(a);
-            if (sub == 0) sc[g * ATT_SPLIT + key] = key < cnt ? a * scale : -INFINITY;
+            if (sub == 0) sc[g * SPLIT + key] = key < cnt ? a * scale : -INFINITY;
         }
     }
     __syncthreads();
@@ -728,18 +741,18 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
     // ---- phase 2: wave g handles query head g ----
     if (wv < G) {
         const int g = wv;
-        float s[ATT_SPLIT / 64], m = -INFINITY;
+        float s[SPLIT / 64], m = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < ATT_SPLIT / 64; i++) {
-            s[i] = sc[g * ATT_SPLIT + lane + 64 * i];
+        for (int i = 0; i < SPLIT / 64; i++) {
+            s[i] = sc[g * SPLIT + lane + 64 * i];
             m = fmaxf(m, s[i]);
         }
         m = wave_max(m);
         float l = 0.0f;
 #pragma unroll
-        for (int i = 0; i < ATT_SPLIT / 64; i++) {
+        for (int i = 0; i < SPLIT / 64; i++) {
             const float pr = (cnt > 0 && s[i] > -INFINITY) ? __expf(s[i] - m) : 0.0f;
-            sc[g * ATT_SPLIT + lane + 64 * i] = pr;
+            sc[g * SPLIT + lane + 64 * i] = pr;
             l += pr;
         }
         l = wave_sum(l);
@@ -755,7 +768,7 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
         for (int e = 0; e < DPL; e++) o[g][e] = 0.0f;
 #pragma unroll
     for (int u = 0; u < VU; u++) {
-        const int j = wv + NW * u;                    // < ATT_SPLIT; entries at or beyond cnt hold p = 0
+        const int j = wv + NW * u;                    // < SPLIT; entries at or beyond cnt hold p = 0
         if (j0 + j == p) {
 #pragma unroll
             for (int e = 0; e < DPL; e++) vb[(int64_t)p * HD + DPL * lane + e] = vv[u][e];
@@ -763,7 +776,7 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
         if (j < cnt) {                                // wave-uniform
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                const float pr = sc[g * ATT_SPLIT + j];
+                const float pr = sc[g * SPLIT + j];
 #pragma unroll
                 for (int e = 0; e < DPL; e++) o[g][e] += pr * vv[u][e];
             }
@@ -780,27 +793,52 @@ __global__ __launch_bounds__(64 * ATTD_WAVES) void attn_decode_kernel(const floa
 #pragma unroll
         for (int w2 = 0; w2 < NW; w2++) a += red[(w2 * G + g) * HD + d];
         float *pp = part + ((int64_t)(kvh * G + g) * splits + sp) * (HD + 4);
-        pp[d] = a;
-        if (d < 4) pp[HD + d] = d == 0 ? ml[2 * g] : d == 1 ? ml[2 * g + 1] : 0.0f;
+        // device-scope stores (written through to where every CU of the GPU reads them): the in-kernel merge below reads
+        // partials of workgroups on other XCDs, whose L2 caches are not coherent with this one's
+        __hip_atomic_store(pp + d, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (d < 4) __hip_atomic_store(pp + HD + d, d == 0 ? ml[2 * g] : d == 1 ? ml[2 * g + 1] : 0.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-}
-
-// merge the { acc[HD], m, l } partials of one head: out = sum_s e^{m_s - M} acc_s / sum_s e^{m_s - M} l_s
-template <int HD>
-__global__ __launch_bounds__(HD) void attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int splits) {
-    const float *pp = part + (int64_t)blockIdx.x * splits * (HD + 4);
-    float M = -INFINITY;
-    for (int s = 0; s < splits; s++) M = fmaxf(M, pp[s * (HD + 4) + HD + 1] > 0.0f ? pp[s * (HD + 4) + HD] : -INFINITY);
-    float num = 0.0f, den = 0.0f;
-    for (int s = 0; s < splits; s++) {
-        const float l = pp[s * (HD + 4) + HD + 1];
-        if (l > 0.0f) {
-            const float w = __expf(pp[s * (HD + 4) + HD] - M);
-            num += w * pp[s * (HD + 4) + threadIdx.x];
-            den += w * l;
+    if (out == nullptr) return;
+    // The merge of the splits, once: the workgroup of this kv head that finishes last does it (no second launch, and no
+    // consumer has to pull every partial through its own CU).  Arrival is counted after a device-wide release of the
+    // partials; the last workgroup acquires, merges (split by split, in order, like the prologue of the attention_wo matvec), and leaves the counter zero.
+    // No fence: a device-scope release would write back every dirty line of this XCD's L2 (measured: 24 us per launch).
+    // The partials went out as device-scope stores; once they are acknowledged (vmcnt = 0) the arrival may be counted,
+    // and the last workgroup reads them with device-scope loads.
+    __shared__ int s_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) s_last = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == splits - 1;
+    __syncthreads();
+    if (!s_last) return;
+    auto ld = [](const float *q) { return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    for (int i = tid; i < G * HD; i += 64 * NW) {
+        const int g = i / HD, d = i - g * HD;
+        const float *pp = part + (int64_t)(kvh * G + g) * splits * (HD + 4);
+        // every load first (these bypass the caches: one after the other they would be a trip to memory each); a split
+        // that does not exist re-reads the last one and is left out of the sums
+        float mv[ATTD_MAX_SPLITS], lv[ATTD_MAX_SPLITS], av[ATTD_MAX_SPLITS];
+#pragma unroll
+        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++) {
+            const float *rec = pp + min(sI, splits - 1) * (HD + 4);
+            mv[sI] = ld(rec + HD); lv[sI] = ld(rec + HD + 1); av[sI] = ld(rec + d);
         }
+        float M = -INFINITY;
+#pragma unroll
+        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++)
+            if (sI < splits) M = fmaxf(M, lv[sI] > 0.0f ? mv[sI] : -INFINITY);
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++) {
+            if (sI < splits && lv[sI] > 0.0f) {
+                const float wgt = __expf(mv[sI] - M);
+                num += wgt * av[sI];
+                den += wgt * lv[sI];
+            }
+        }
+        out[(int64_t)(kvh * G + g) * HD + d] = num / den;
     }
-    out[(int64_t)blockIdx.x * HD + threadIdx.x] = num / den;
+    if (tid == 0) __hip_atomic_store(&counters[kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- out = silu(gate) * up, silu(v) = v / (1 + exp(-v))  (candle-core/src/op.rs Silu; quantized_llama.rs:56-63) ----
@@ -1253,12 +1291,12 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
 
 int64_t cq_nn_attention_decode_workspace_bytes(int64_t n_head, int64_t head_dim, int64_t max_kv_len) {
     if (n_head <= 0 || head_dim <= 0 || max_kv_len <= 0) return -1;
-    return n_head * attn_splits(max_kv_len) * (head_dim + 4) * 4;
+    return n_head * attd_splits(max_kv_len) * (head_dim + 4) * 4 + ATTD_COUNTER_BYTES;
 }
 
 int64_t cq_nn_attention_decode_splits(int64_t max_kv_len) {
     if (max_kv_len <= 0) return -1;
-    const int64_t s = attn_splits(max_kv_len);
+    const int64_t s = attd_splits(max_kv_len);
     return s <= ATTD_MAX_SPLITS ? s : -1;
 }
 
@@ -1275,8 +1313,10 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
         return CQ_ERR_ALIGN;
     if (!pos_dev && pos + 1 > max_kv_len) return CQ_ERR_RANGE;
     if (partials_bytes < cq_nn_attention_decode_workspace_bytes(n_head, head_dim, max_kv_len)) return CQ_ERR_WORKSPACE;
-    const int64_t splits = attn_splits(max_kv_len);
-    if (splits > ATTD_MAX_SPLITS || ctx > 0x7fffffffLL) return CQ_ERR_RANGE;
+    const int64_t splits = attd_splits(max_kv_len);
+    if (splits > ATTD_MAX_SPLITS || ctx > 0x7fffffffLL || n_kv_head > ATTD_COUNTER_BYTES / 4) return CQ_ERR_RANGE;
+    const bool fine = attd_split_keys(max_kv_len) == 64;
+    int *counters = (int *)((uint8_t *)partials_dev + n_head * splits * (head_dim + 4) * 4);
     const int G = (int)(n_head / n_kv_head);
     float *part = (float *)partials_dev;
     // read-only workgroups for the prefetch range: enough, with the attention ones, for one per CU
@@ -1289,9 +1329,14 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     dim3 grid((unsigned)n_kv_head, (unsigned)(splits + pf_rows));
     hipStream_t s = (hipStream_t)stream;
 #define CQ_ATTD(HH, GG)                                                                                                                   \
-    hipLaunchKernelGGL((attn_decode_kernel<HH, GG>), grid, dim3(64 * ATTD_WAVES), 0, s, q_dev, k_new_dev, v_new_dev, k_cache_dev, v_cache_dev, \
-                       cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits, (const u32x4 *)prefetch_dev, pf_chunks,   \
-                       (uint32_t *)nullptr)
+    if (fine)                                                                                                                             \
+        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 8, 64>), grid, dim3(64 * 8), 0, s, q_dev, k_new_dev, v_new_dev, k_cache_dev, v_cache_dev, \
+                           cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits, (const u32x4 *)prefetch_dev, pf_chunks, \
+                           (uint32_t *)nullptr, out_dev, counters);                                                                       \
+    else                                                                                                                                  \
+        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 16, 128>), grid, dim3(64 * 16), 0, s, q_dev, k_new_dev, v_new_dev, k_cache_dev,      \
+                           v_cache_dev, cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits, (const u32x4 *)prefetch_dev, \
+                           pf_chunks, (uint32_t *)nullptr, out_dev, counters)
     if (head_dim == 128) {
         switch (G) {
             case 1: CQ_ATTD(128, 1); break;
@@ -1310,12 +1355,6 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
         }
     }
 #undef CQ_ATTD
-    int rc = (int)hipGetLastError();
-    if (rc || !out_dev) return rc;
-    if (head_dim == 128)
-        hipLaunchKernelGGL((attn_merge_kernel<128>), dim3((unsigned)n_head), dim3(128), 0, s, (const float *)part, out_dev, (int)splits);
-    else
-        hipLaunchKernelGGL((attn_merge_kernel<64>), dim3((unsigned)n_head), dim3(64), 0, s, (const float *)part, out_dev, (int)splits);
     return (int)hipGetLastError();
 }
 

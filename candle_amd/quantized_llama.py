@@ -107,6 +107,7 @@ class ModelWeights:
         self._graph_key = None
         self.fuse_decode = True            # single-token steps use the fused matvec prologues / epilogues
         self.split_w2 = True               # ... and feed_forward_w2 as a K-split matvec where the shapes allow it
+        self.merge_in_wo = False           # merge the attention key splits in the prologue of attention_wo (else: in the attention kernel)
         # bytes of the weights behind attention (wo, w1, w3, w2 are contiguous) that the attention launch's idle CUs
         # would pull through the memory-side cache ahead of the kernels that stream them.  Measured on the 8B shape:
         # no gain at 4-24 MB and a loss beyond (the time moves into the attention launch), so it is off.
@@ -439,7 +440,10 @@ class ModelWeights:
             q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
             # rope, cache append, attention and the merge of the key splits in one kernel          :217-261
             wo = w["attention_wo"]
-            merge_in_wo = wo.dtype in full and qd <= (4096 if wo.dtype in kq else 2048) and (cfg.head_dim & (cfg.head_dim - 1)) == 0
+            # the attention kernel merges its key splits itself (the last workgroup of a kv head does it once); merging in
+            # the prologue of attention_wo instead makes every workgroup of that matvec read every partial
+            merge_in_wo = self.merge_in_wo and wo.dtype in full and qd <= (4096 if wo.dtype in kq else 2048) and \
+                (cfg.head_dim & (cfg.head_dim - 1)) == 0
             ck("cq_nn_attention_decode", L.cq_nn_attention_decode(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
                                                                   self.cos.data_ptr(), self.sin.data_ptr(),
                                                                   None if merge_in_wo else att.data_ptr(), pos_dev_ptr, pos,

@@ -63,9 +63,12 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
  * rope_i on q and on the new k, append of the new k and v to the cache at p, attention of the rotated q over keys
  * [0, p].  q [n_head*head_dim], k_new / v_new [n_kv_head*head_dim] are the raw projection outputs (16-byte aligned;
  * q is not modified).  The result is left in partials_dev as per-split records { acc[head_dim], m, l, 0, 0 } for
- * every head ([n_head][splits][head_dim + 4] floats, splits = cq_nn_attention_decode_splits(max_kv_len), at most 16,
- * i.e. max_kv_len <= 2048; -1 beyond).  When out_dev != NULL a second small kernel merges them into
- * out_dev [n_head*head_dim]; with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn.
+ * every head ([n_head][splits][head_dim + 4] floats, splits = cq_nn_attention_decode_splits(max_kv_len): splits of 64
+ * keys while 16 of them cover max_kv_len, else of 128 keys; at most 16, i.e. max_kv_len <= 2048; -1 beyond).  When out_dev != NULL the
+ * workgroup of each kv head that finishes last merges that head group's splits into out_dev [n_head*head_dim] (same
+ * launch, same arithmetic as a separate merge); with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn.
+ * The last 256 bytes of partials_dev are the arrival counters of that merge: they must be zero before the first call
+ * with a buffer, and every call leaves them zero.
  * prefetch_dev / prefetch_bytes (optional, 16-byte aligned): a byte range that extra read-only workgroups of this
  * otherwise latency-bound launch pull through the memory-side cache, e.g. the weights of the kernels that follow.
  * No counterpart in the reference, which runs these as separate tensor ops (quantized_llama.rs:217-261). */

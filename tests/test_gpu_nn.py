@@ -173,8 +173,11 @@ def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
     kc0, vc0 = normal(33, (KV, ctx, D), 1.0), normal(34, (KV, ctx, D), 1.0)
     kc0[:, pos:], vc0[:, pos:] = np.nan, np.nan          # nothing at or beyond the new position may be read
     wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
-    assert lib.cq_nn_attention_decode_splits(max_kv) == (max_kv + 127) // 128 and lib.cq_nn_attention_decode_splits(2049) == -1
+    # 64-key splits while at most 16 of them cover max_kv, else 128-key splits; more than 16 splits: not available
+    want_splits = (max_kv + 63) // 64 if (max_kv + 63) // 64 <= 16 else (max_kv + 127) // 128
+    assert lib.cq_nn_attention_decode_splits(max_kv) == want_splits and lib.cq_nn_attention_decode_splits(2049) == -1
     ws = torch.full((wsb,), 0xff, dtype=torch.uint8, device="cuda")
+    ws[-256:] = 0                                        # the arrival counters of the in-kernel merge start at zero
     posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
     c, s = cos[pos:pos + 1], sin[pos:pos + 1]
     want_q = lo.rope_i(q.reshape(1, H, D).transpose(1, 0, 2)[None], c, s)[0].transpose(1, 0, 2).reshape(1, H * D)
