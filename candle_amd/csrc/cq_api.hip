@@ -65,9 +65,7 @@ inline int check_mm_shape(int w_dtype, int64_t k, int64_t n, int64_t rows) {
 
 inline int check_weight_ptr(int w_dtype, const void *w) {
     if (!w) return CQ_ERR_NULL;
-    // Q4_0 / Q5_0 / Q8_0 blocks are fetched as the aligned dwords around them (cq_fmt.h)
-    const bool dwords = w_dtype == CQ_Q4_0 || w_dtype == CQ_Q5_0 || w_dtype == CQ_Q8_0;
-    if (!aligned(w, (w_dtype == CQ_Q4K || w_dtype == CQ_Q5K) ? 16 : dwords ? 4 : 2)) return CQ_ERR_ALIGN;
+    if (!aligned(w, (w_dtype == CQ_Q4K || w_dtype == CQ_Q5K) ? 16 : 2)) return CQ_ERR_ALIGN;
     return CQ_OK;
 }
 
@@ -143,14 +141,6 @@ int cq_embedding(int dtype, const void *blocks_dev, const uint32_t *ids_dev, flo
     if (!blocks_dev || !ids_dev || !out_dev) return CQ_ERR_NULL;
     if (!aligned(blocks_dev, 2) || !aligned(ids_dev, 4) || !aligned(out_dev, 16)) return CQ_ERR_ALIGN;
     return cq_embedding_launch(dtype, blocks_dev, ids_dev, out_dev, n_ids, rows, hidden, (hipStream_t)stream);
-}
-
-int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stream) {
-    if (bytes < 0 || bytes % 16) return CQ_ERR_SHAPE;
-    if (bytes == 0) return CQ_OK;
-    if (!src_dev || !sink_dev) return CQ_ERR_NULL;
-    if (!aligned(src_dev, 16) || !aligned(sink_dev, 4)) return CQ_ERR_ALIGN;
-    return cq_bench_read_launch(src_dev, bytes, sink_dev, (hipStream_t)stream);
 }
 
 int cq_quantize(int dtype, const float *x_dev, void *blocks_dev, int64_t elem_count, void *stream) {

@@ -338,67 +338,73 @@ __device__ __forceinline__ void load_act_q0(A0 &a, const ActRow &ar, int u) {
 // ---- blocks of 2 (mod 4) bytes: Q4_0 (18), Q5_0 (22), Q8_0 (34) --------------------------------
 // Every other block of such a row starts on an odd halfword, and a 16-byte load from an address that is not a multiple
 // of 4 costs the vector memory path about a quarter of its rate (measured: Q4_1 / Q5_1, the same blocks plus 2 bytes,
-// stream at 3.8 / 4.2 TB/s where Q4_0 / Q5_0 reached 3.0 / 3.1).  So a block is fetched as the aligned dwords around
-// it, starting at `a` = its address rounded down to a multiple of 4, and the halfword offset is undone in registers
-// with one byte permute per dword.  Reads stay inside [a, a + size + 2): at most the 2 bytes in front of a block that
-// starts on an odd halfword, or the 2 bytes behind one that does not — the neighbouring blocks, or for the last block of
-// a tensor the rest of its last dword.
+// stream at 3.8 / 4.2 TB/s where Q4_0 / Q5_0 reached 3.0 / 3.1).  A block of 4 j + 2 bytes is one halfword plus j whole
+// dwords, so it is fetched as exactly that: at a block address that is a multiple of 4 the dwords come first and the
+// halfword is the block's last two bytes; on an odd halfword the halfword is the block's first two bytes and the dwords
+// start 2 bytes in.  Every load is naturally aligned and none touches a byte outside [block, block + size).  The
+// halfword offset is undone in registers with one byte permute per dword.
 template <typename T> __device__ __forceinline__ T ld_a4(const void *p) {
     struct __attribute__((packed, aligned(4))) W { T v; };
     return reinterpret_cast<const W *>(p)->v;
 }
-__device__ __forceinline__ const uint8_t *align4_down(const uint8_t *p, uint32_t &sel) {
-    const uintptr_t v = (uintptr_t)p;
-    // v_perm_b32(hi, lo, sel): bytes 2..5 of the pair when the block starts at `a`, bytes 4..7 when it starts at a + 2
-    sel = (v & 2) ? 0x07060504u : 0x05040302u;
-    return (const uint8_t *)(v & ~(uintptr_t)3);
+// Splits a block of (2 + dw_bytes) bytes at `p`: returns the address of its dword run, `hw` = the address of its lone
+// halfword.  `sel` is the v_perm_b32 selector that rebuilds payload dword i (the payload starts 2 bytes into the
+// block) from the dword pair (y[i + 1], y[i]) of the sequence y = {dword run, halfword}: bytes 2..5 of the pair when
+// the run starts at the block, bytes 0..3 when it starts with the payload.
+__device__ __forceinline__ const uint8_t *split_hw(const uint8_t *p, int dw_bytes, const uint8_t *&hw, uint32_t &sel) {
+    const bool odd = ((uintptr_t)p & 2) != 0;
+    sel = odd ? 0x03020100u : 0x05040302u;
+    hw = p + (odd ? 0 : dw_bytes);
+    return p + (odd ? 2 : 0);
 }
-// dword i of the block's payload: the payload starts 2 bytes into the pair (lo, hi) or at hi
+__device__ __forceinline__ uint32_t ld_hw(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
 __device__ __forceinline__ uint32_t take_hw(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
-// the f16 scale at the start of the block: low half of the first dword, or its high half
-__device__ __forceinline__ uint32_t head_hw(uint32_t x0, uint32_t sel) { return x0 >> ((sel & 4u) << 2); }
+// the f16 scale at the start of the block: the low half of the first dword of the run, or the lone halfword
+__device__ __forceinline__ uint32_t head_hw(uint32_t y0, uint32_t hw, uint32_t sel) { return (sel & 2u) ? y0 : hw; }
 
 template <> struct Fmt<CQ_Q4_0> {
     static constexpr int UE = 32, UPB = 1;
-    struct W { u32x4 x; uint32_t x0, sel; };
+    struct W { u32x4 x; uint32_t hw, sel; };
     typedef A0 A;
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *a = align4_down(row + u * 18, w.sel);
-        w.x0 = *reinterpret_cast<const uint32_t *>(a);
-        w.x = ld_a4<u32x4>(a + 4);
+        const uint8_t *hw;
+        const uint8_t *a = split_hw(row + u * 18, 16, hw, w.sel);
+        w.x = ld_a4<u32x4>(a);
+        w.hw = ld_hw(hw);
     }
     static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
     static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
         const uint32_t M4 = 0x0f0f0f0fu;
-        const uint32_t q0 = take_hw(w.x.x, w.x0, w.sel), q1 = take_hw(w.x.y, w.x.x, w.sel), q2 = take_hw(w.x.z, w.x.y, w.sel),
-                       q3 = take_hw(w.x.w, w.x.z, w.sel);
+        const uint32_t q0 = take_hw(w.x.y, w.x.x, w.sel), q1 = take_hw(w.x.z, w.x.y, w.sel), q2 = take_hw(w.x.w, w.x.z, w.sel),
+                       q3 = take_hw(w.hw, w.x.w, w.sel);
         int s = -8 * a.s8;    // sum((q - 8) * y) = sum(q * y) - 8 * sum(y)
         s = sdot4(q0 & M4, a.a0.x, s); s = sdot4(q1 & M4, a.a0.y, s);
         s = sdot4(q2 & M4, a.a0.z, s); s = sdot4(q3 & M4, a.a0.w, s);
         s = sdot4((q0 >> 4) & M4, a.a1.x, s); s = sdot4((q1 >> 4) & M4, a.a1.y, s);
         s = sdot4((q2 >> 4) & M4, a.a1.z, s); s = sdot4((q3 >> 4) & M4, a.a1.w, s);
-        return (float)s * h2f(head_hw(w.x0, w.sel)) * a.d8;
+        return (float)s * h2f(head_hw(w.x.x, w.hw, w.sel)) * a.d8;
     }
 };
 
 template <> struct Fmt<CQ_Q8_0> {
     static constexpr int UE = 32, UPB = 1;
-    struct W { u32x4 x, y; uint32_t x0, sel; };
+    struct W { u32x4 x, y; uint32_t hw, sel; };
     typedef A0 A;
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *a = align4_down(row + u * 34, w.sel);
-        w.x0 = *reinterpret_cast<const uint32_t *>(a);
-        w.x = ld_a4<u32x4>(a + 4);
-        w.y = ld_a4<u32x4>(a + 20);
+        const uint8_t *hw;
+        const uint8_t *a = split_hw(row + u * 34, 32, hw, w.sel);
+        w.x = ld_a4<u32x4>(a);
+        w.y = ld_a4<u32x4>(a + 16);
+        w.hw = ld_hw(hw);
     }
     static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
     static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
         int s = 0;
-        s = sdot4(take_hw(w.x.x, w.x0, w.sel), a.a0.x, s); s = sdot4(take_hw(w.x.y, w.x.x, w.sel), a.a0.y, s);
-        s = sdot4(take_hw(w.x.z, w.x.y, w.sel), a.a0.z, s); s = sdot4(take_hw(w.x.w, w.x.z, w.sel), a.a0.w, s);
-        s = sdot4(take_hw(w.y.x, w.x.w, w.sel), a.a1.x, s); s = sdot4(take_hw(w.y.y, w.y.x, w.sel), a.a1.y, s);
-        s = sdot4(take_hw(w.y.z, w.y.y, w.sel), a.a1.z, s); s = sdot4(take_hw(w.y.w, w.y.z, w.sel), a.a1.w, s);
-        return (float)s * h2f(head_hw(w.x0, w.sel)) * a.d8;
+        s = sdot4(take_hw(w.x.y, w.x.x, w.sel), a.a0.x, s); s = sdot4(take_hw(w.x.z, w.x.y, w.sel), a.a0.y, s);
+        s = sdot4(take_hw(w.x.w, w.x.z, w.sel), a.a0.z, s); s = sdot4(take_hw(w.y.x, w.x.w, w.sel), a.a0.w, s);
+        s = sdot4(take_hw(w.y.y, w.y.x, w.sel), a.a1.x, s); s = sdot4(take_hw(w.y.z, w.y.y, w.sel), a.a1.y, s);
+        s = sdot4(take_hw(w.y.w, w.y.z, w.sel), a.a1.z, s); s = sdot4(take_hw(w.hw, w.y.w, w.sel), a.a1.w, s);
+        return (float)s * h2f(head_hw(w.x.x, w.hw, w.sel)) * a.d8;
     }
 };
 
@@ -447,19 +453,21 @@ __device__ __forceinline__ int dot_q5(const u32x4 &qs, uint32_t qh, const A0 &a,
 
 template <> struct Fmt<CQ_Q5_0> {
     static constexpr int UE = 32, UPB = 1;
-    struct W { u32x4 x; u32x2 h; uint32_t sel; };
+    struct W { u32x4 x; uint32_t z, hw, sel; };
     typedef A0 A;
     static __device__ __forceinline__ void load_w(W &w, const uint8_t *row, int u) {
-        const uint8_t *a = align4_down(row + u * 22, w.sel);      // 22-byte blocks: fetched as aligned dwords, see Fmt<CQ_Q4_0>
-        w.h = ld_a4<u32x2>(a);
-        w.x = ld_a4<u32x4>(a + 8);
+        const uint8_t *hw;
+        const uint8_t *a = split_hw(row + u * 22, 20, hw, w.sel);     // 22-byte blocks: a halfword and five dwords, see Fmt<CQ_Q4_0>
+        w.x = ld_a4<u32x4>(a);
+        w.z = *reinterpret_cast<const uint32_t *>(a + 16);
+        w.hw = ld_hw(hw);
     }
     static __device__ __forceinline__ void load_a(A &a, const ActRow &ar, int u) { load_act_q0(a, ar, u); }
     static __device__ __forceinline__ float dot(const W &w, const A &a, int) {
-        const uint32_t qh = take_hw(w.h.y, w.h.x, w.sel);
-        const u32x4 qs = {take_hw(w.x.x, w.h.y, w.sel), take_hw(w.x.y, w.x.x, w.sel), take_hw(w.x.z, w.x.y, w.sel), take_hw(w.x.w, w.x.z, w.sel)};
+        const uint32_t qh = take_hw(w.x.y, w.x.x, w.sel);
+        const u32x4 qs = {take_hw(w.x.z, w.x.y, w.sel), take_hw(w.x.w, w.x.z, w.sel), take_hw(w.z, w.x.w, w.sel), take_hw(w.hw, w.z, w.sel)};
         const int s = dot_q5(qs, qh, a, -16 * a.s8);    // sum((q - 16) * y) = sum(q * y) - 16 * sum(y)
-        return (float)s * h2f(head_hw(w.h.x, w.sel)) * a.d8;
+        return (float)s * h2f(head_hw(w.x.x, w.hw, w.sel)) * a.d8;
     }
 };
 

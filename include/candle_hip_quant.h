@@ -16,9 +16,7 @@
  *   - weights are GGUF blocks exactly as stored on disk, rows contiguous, `n` rows of `k/blk` blocks
  *     (candle-core/src/quantized/k_quants.rs:77-190); kernels read only [ptr, ptr + size) and never
  *     rely on the 512-element tail padding the CUDA backend adds
- *     (candle-core/src/quantized/cuda.rs:624-637,989-1008); the matvec kernels fetch Q4_0 / Q5_0 / Q8_0 blocks
- *     (18 / 22 / 34 bytes) as whole aligned dwords, so a tensor of these formats whose size is 2 (mod 4) is read up
- *     to the end of its last dword;
+ *     (candle-core/src/quantized/cuda.rs:624-637,989-1008);
  *   - activation quantization follows candle's CPU path bit for bit (Q8_K blocks for K-quants,
  *     Q8_0 blocks for Q4_0/Q5_0/Q8_0, Q8_1 blocks for Q4_1/Q5_1: k_quants.rs:2320-2358, 658-687, 770-799), so
  *     results match QMatMul::forward on the CPU up to f32 summation order;
@@ -111,7 +109,7 @@ int cq_quantize_act(int w_dtype, const void *x_dev, int x_dtype, void *scratch_d
  * Decode matvec over pre-quantized activations:  dst[r, j] = sum_k W[j, k] * x^[r, k]
  * for r < rows <= CQ_MATVEC_MAX_ROWS.  Counterpart of launch_mmvq_gguf_<t>_<dst>_plain
  * (candle-kernels/src/ffi.rs:58-631, mmvq_gguf.cu:915-1008).
- *   w_dev: n rows of k/blk blocks; 16-byte aligned for Q4K/Q5K, 4-byte aligned for Q4_0/Q5_0/Q8_0, 2-byte aligned otherwise.
+ *   w_dev: n rows of k/blk blocks; 16-byte aligned for Q4K/Q5K, 2-byte aligned otherwise.
  *   act_scratch_dev: written by cq_quantize_act with the same (w_dtype, k, rows).
  *   dst_dev: f32 / f16 / bf16 (dst_dtype), row stride `stride_dst` elements (>= n).
  * ------------------------------------------------------------------------------------------- */
@@ -213,11 +211,6 @@ int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_
  * (k <= 2048 for K-quants, 1024 otherwise) while size_m <= 3 * num_experts.  No counterpart in the reference, which always
  * sorts (fused_moe.rs:249-260). */
 int cq_moe_direct_pairs(int w_dtype, int64_t num_experts, int64_t size_m, int64_t k);
-
-/* Measurement aid, no counterpart in the reference: a kernel that only reads `bytes` (a multiple of 16) of a device
- * buffer, with the launch shape of the decode matvec (256 workgroups of 1024 threads).  bench.py times it over the same
- * rotated weight tensors as the matvec, as the figure for what this GPU delivers to a launch of that size. */
-int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stream);
 
 #ifdef __cplusplus
 }
