@@ -18,9 +18,9 @@
 //   activation quantizers downstream, an exact one is not.
 // Q4_K — the same sums on the int8 matrix cores (qmm_q4k_i8_kernel, k_quants.rs:1460-1540): the 6-bit sub-block scale
 //   is split into two 3-bit halves so that scale * weight fits int8; S is exact in int32.
-// Q4_0 / Q8_0 — both operands carry a per-32 f16 scale, so the dequantized values d*(q-8) and d8*q8
-//   are rounded to f16 (relative 2^-11 per operand) and multiplied at full MFMA rate; the result stays
-//   well inside the 1e-3 tolerance (measured ~2e-4) but is not integer-exact like the decode path.
+// Q4_0 / Q8_0 — the per-32 sums of the CPU vec_dot (k_quants.rs:294-311, 720-738) on the int8 matrix cores
+//   (qmm_q0_i8_kernel): one v_mfma_i32_32x32x32_i8 per 32-element block gives the exact int32 sum of q8 * (q - 8)
+//   resp. q8 * q, and the vector units add  (float(S) * d[n, block]) * d8[m, block]  block by block, in the CPU's order.
 //
 // Tiling: workgroup = 4 waves (2 x 2), block tile 128 (m) x 64 (n), wave tile 64 x 32 as 2 x 1 MFMA tiles of 32 x 32
 // (128 x 128 / 64 x 64 for large Q4_0 / Q8_0 problems, 32 x 128 with the waves side by side for up to 32 rows).
@@ -84,7 +84,7 @@ __device__ __forceinline__ void k4_sub_scale_min(uint32_t u0, uint32_t u1, uint3
 template <int DT> struct Stage;
 
 template <> struct Stage<CQ_Q5K> {
-    static constexpr bool KQ = true, HAS_MIN = true;
+    static constexpr bool HAS_MIN = true;
     static constexpr int TERMS = 1;
     template <int NW> struct Raw { u32x4 hdr, h[NW / 16], q[NW / 16]; };
     template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
@@ -124,7 +124,7 @@ template <> struct Stage<CQ_Q5K> {
 };
 
 template <> struct Stage<CQ_Q6K> {
-    static constexpr bool KQ = true, HAS_MIN = false;
+    static constexpr bool HAS_MIN = false;
     static constexpr int TERMS = 2;      // sc * (q - 32) reaches 4096: f16 head + exact remainder in {-1, 0, 1}
     // 32-element half (g, jh) = elements 64g + 32jh + [0, 32): half h6 = g >> 1 of the block, quarter = 2*(g&1) + jh
     template <int NW> struct Raw { u32x4 l[NW / 16], h[NW / 16]; uint32_t sc, d; };
@@ -177,7 +177,7 @@ template <> struct Stage<CQ_Q6K> {
 // hmask[16 c + i]), its 16-element group is 8 h + 2 s + c (k_quants.rs:1013-1049, 1369-1421).  Stage (kb, g), 32-element half jh:
 // h = g >> 1, s = 2 (g & 1) + jh.  Both products are small exact integers in f16: sc * q <= 45, (sc - 32) * (q - 4) within +-128.
 template <> struct Stage<CQ_Q2K> {
-    static constexpr bool KQ = true, HAS_MIN = true;
+    static constexpr bool HAS_MIN = true;
     static constexpr int TERMS = 1;
     template <int NW> struct Raw { u32x4 sc, q[NW / 16]; uint32_t dd; };
     template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
@@ -214,7 +214,7 @@ template <> struct Stage<CQ_Q2K> {
 };
 
 template <> struct Stage<CQ_Q3K> {
-    static constexpr bool KQ = true, HAS_MIN = false;
+    static constexpr bool HAS_MIN = false;
     static constexpr int TERMS = 1;
     template <int NW> struct Raw { u32x4 q[NW / 16], hm[NW / 16]; uint32_t s0, s1, s2, d; };
     template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
@@ -257,78 +257,16 @@ template <> struct Stage<CQ_Q3K> {
     }
 };
 
-template <> struct Stage<CQ_Q4_0> {
-    static constexpr bool KQ = false, HAS_MIN = false;
-    static constexpr int TERMS = 1;
-    template <int NW> struct Raw { u32x4 qs; uint32_t d; };
-    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
-        const int jh = NW == 16 ? part >> 1 : part;
-        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + jh) * 18;
-        r.d = ld_u<uint16_t>(blk);
-        r.qs = ld_u<u32x4>(blk + 2);
-    }
-    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &, float &d, float &dmin) { d = 1.0f; dmin = 0.0f; }
-    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &, int) { return 0; }
-    // elements 0..15 of a block are the low nibbles of its 16 bytes, elements 16..31 the high nibbles
-    template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int, int part, uint32_t out[NW / 2]) {
-        const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1032.0f);   // -(1024 + 8)
-        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            uint32_t lo, hi;
-            if constexpr (NW == 32) {
-                bytes_to_h1024(q[i] & 0x0f0f0f0fu, lo, hi);               // elements 4i..4i+3
-                out[2 * i] = pk_mul(pk_add(lo, off), d2);
-                out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
-                bytes_to_h1024((q[i] >> 4) & 0x0f0f0f0fu, lo, hi);        // elements 16+4i..
-                out[8 + 2 * i] = pk_mul(pk_add(lo, off), d2);
-                out[8 + 2 * i + 1] = pk_mul(pk_add(hi, off), d2);
-            } else {
-                bytes_to_h1024((q[i] >> (4 * (part & 1))) & 0x0f0f0f0fu, lo, hi);
-                out[2 * i] = pk_mul(pk_add(lo, off), d2);
-                out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
-            }
-        }
-    }
-};
-
-template <> struct Stage<CQ_Q8_0> {
-    static constexpr bool KQ = false, HAS_MIN = false;
-    static constexpr int TERMS = 1;
-    template <int NW> struct Raw { u32x4 q[NW / 16]; uint32_t d; };
-    template <int NW> static __device__ __forceinline__ void load(Raw<NW> &r, const uint8_t *row, int kb, int g, int part) {
-        const int jh = NW == 16 ? part >> 1 : part, sx = NW == 16 ? part & 1 : 0;
-        const uint8_t *blk = row + (int64_t)(kb * 8 + 2 * g + jh) * 34;
-        r.d = ld_u<uint16_t>(blk);
-#pragma unroll
-        for (int i = 0; i < NW / 16; i++) r.q[i] = ld_u<u32x4>(blk + 2 + 16 * (sx + i));
-    }
-    template <int NW> static __device__ __forceinline__ void header(const Raw<NW> &, float &d, float &dmin) { d = 1.0f; dmin = 0.0f; }
-    template <int NW> static __device__ __forceinline__ uint32_t min_pair(const Raw<NW> &, int) { return 0; }
-    template <int NW> static __device__ __forceinline__ void convert(const Raw<NW> &r, int, int, uint32_t out[NW / 2]) {
-        const uint32_t d2 = (r.d & 0xffffu) | (r.d << 16), off = h2_splat(-1152.0f);   // -(1024 + 128)
-#pragma unroll
-        for (int i = 0; i < NW / 4; i++) {
-            uint32_t lo, hi;
-            bytes_to_h1024(r.q[i >> 2][i & 3] ^ 0x80808080u, lo, hi);               // int8 -> biased unsigned
-            out[2 * i] = pk_mul(pk_add(lo, off), d2);
-            out[2 * i + 1] = pk_mul(pk_add(hi, off), d2);
-        }
-    }
-};
-
-// 32 int8 activations -> 16 dwords of f16 pairs (exact); scale2 == 0 means "leave as integers"
-__device__ __forceinline__ void act_convert(const u32x4 &a0, const u32x4 &a1, bool scaled, uint32_t scale2, uint32_t out[16]) {
+// 32 int8 activations -> 16 dwords of f16 pairs holding the same integers
+__device__ __forceinline__ void act_convert(const u32x4 &a0, const u32x4 &a1, uint32_t out[16]) {
     const uint32_t off = 0xe480e480u;    // two f16 -1152.0
     const uint32_t q[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         uint32_t lo, hi;
         bytes_to_h1024(q[i] ^ 0x80808080u, lo, hi);
-        lo = pk_add(lo, off);
-        hi = pk_add(hi, off);
-        out[2 * i] = scaled ? pk_mul(lo, scale2) : lo;
-        out[2 * i + 1] = scaled ? pk_mul(hi, scale2) : hi;
+        out[2 * i] = pk_add(lo, off);
+        out[2 * i + 1] = pk_add(hi, off);
     }
 }
 
@@ -351,7 +289,6 @@ __global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 
                                                                      int n, int rows, int64_t stride_dst, MoeChunks mc, int64_t expert_bytes,
                                                                      int64_t split_stride) {
     typedef Stage<DT> S;
-    constexpr bool KQ = S::KQ;
     static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
     constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;             // rows of the block tile, 32-row MFMA tiles per wave
     constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
@@ -419,8 +356,7 @@ __global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 
             const int8_t *q = aq_p + kb * 256 + 64 * g + 32 * half;
             x0 = *reinterpret_cast<const u32x4 *>(q);
             x1 = *reinterpret_cast<const u32x4 *>(q + 16);
-            if (!KQ) d8 = av.d[2 * ((int64_t)arow * (k >> 5) + kb * 8 + 2 * g + half)];   // already f16-representable
-            if (KQ && g == 0) {
+            if (g == 0) {
                 d8 = av.d[(int64_t)arow * (k >> 8) + kb];
                 if (S::HAS_MIN) abs0 = *reinterpret_cast<const u32x4 *>(av.bsums + (int64_t)arow * (k >> 4) + kb * 16 + 8 * half);
             }
@@ -436,11 +372,11 @@ __global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 
         if constexpr (S::TERMS == 2) S::template convert2<NW>(wraw, g, part, c.w, c.w2);
         else S::template convert<NW>(wraw, g, part, c.w);
         if (astage) {
-            act_convert(a0, a1, !KQ, KQ ? 0u : h2_splat(d8), c.a);
+            act_convert(a0, a1, c.a);
 #pragma unroll
             for (int i = 0; i < 16; i++) c.a[i] &= amask;        // rows past the end contribute zeros (no branch)
         }
-        if (KQ && g == 0) {
+        if (g == 0) {
             S::template header<NW>(wraw, c.d, c.dmin);
             c.d8 = arow_ok ? d8 : 0.0f;
             if (S::HAS_MIN) {
@@ -462,7 +398,7 @@ __global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 
         if constexpr (S::TERMS == 2) lds_write_h<NW>(Bs2[buf] + r_w * LDK + NW * part, c.w2);
         lds_write_h<NW>(Bs[buf] + r_w * LDK + NW * part, c.w);
         if (astage) lds_write_h<32>(As[buf] + r_l * LDK + 32 * half, c.a);
-        if (KQ && g == 0) {
+        if (g == 0) {
             // the threads of a row hold the same values: all of them write (no branch)
             sD[hb][r_w] = c.d; sDmin[hb][r_w] = c.dmin;
             if (astage) sD8[hb][r_l] = c.d8;
@@ -521,7 +457,7 @@ __global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 
                 }
             }
             store_stage(ng, nb, g == 3 ? hb ^ 1 : hb, c);
-            if (KQ && g == 3) {
+            if (g == 3) {
                 // ---- end of the super-block: mins term and the f32 scales ----
                 f32x16 mt[MI][NJ];
                 if (S::HAS_MIN) {
@@ -572,7 +508,7 @@ __global__ __launch_bounds__(256, NJ == 1 && !(SM && Stage<DT>::TERMS == 2) ? 2 
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int mm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                float v = KQ ? acc[i][j][e] : sb[i][j][e];
+                const float v = acc[i][j][e];
                 if (mm < rows && nn < n) {
                     if (MOE) dst[(int64_t)mc.pair_out[mm] * stride_dst + nn] = v * mc.pair_scale[mm];
                     else dst[(int64_t)mm * stride_dst + nn] = v;
@@ -814,6 +750,152 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
         }
 }
 
+// ---- Q4_0 / Q8_0 on the int8 matrix cores ----------------------------------------------------------------------------
+// Same tiling and template parameters as above.  Both operands carry an f16 scale per 32 elements, so a 32 x 32 x 32 int8
+// MFMA is exactly one block: its int32 result S is the sum the CPU vec_dot forms for that block (k_quants.rs:294-311,
+// 720-738), and each lane folds its 16 results into the f32 accumulators as (float(S) * d[n]) * d8[m], block after block
+// in k order like the CPU loop.  That scaling is three vector instructions per result and bounds the kernel; the matrix
+// cores idle most of the time.  A stage is 128 elements of k (four blocks).  The int8 activations go through LDS as
+// in the Q4_K kernel (two copies, one barrier per stage) together with the stage's four d8 per row; the weights do
+// not: lane (n, kg) of the B operand wants 16 consecutive k of row n, which are the 16 quant bytes of the block (Q4_0: low
+// nibbles for kg = 0, high nibbles for kg = 1) or one half of its 32 (Q8_0), so every lane fetches its own 16 bytes and
+// the block's scale straight from memory, one stage ahead, into registers.
+//   Q4_0: nibble q -> int8 (q - 8) on four bytes at once: (x + 0x78787878) ^ 0x80808080 (no carries: x < 16 per byte).
+template <int DT, int NJ, bool SM = false>
+__global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst,
+                                                                           int k, int n, int rows, int64_t stride_dst, MoeChunks,
+                                                                           int64_t, int64_t split_stride) {
+    static_assert(DT == CQ_Q4_0 || DT == CQ_Q8_0, "formats of one f16 scale per 32 weights");
+    static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
+    constexpr int BB = BlockInfo<DT>::bytes;
+    constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;
+    constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
+    constexpr int NA = BMT / 32;                                // 16-byte activation pieces a thread copies per stage
+    __shared__ __align__(16) int8_t As[2][BMT * 128];           // [row][8 pieces], piece p of row r at p ^ (r & 7)
+    __shared__ __align__(16) float sD8[2][4][BMT];              // d8 of the stage's four blocks
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int wm = SM ? 0 : wv >> 1, wn = SM ? wv : wv & 1;
+    const int m0 = blockIdx.x * BMT, n0 = blockIdx.y * BN;
+    // split-K over spans of 256 elements, like the other kernels; a stage is half a span
+    const int nsb_all = k >> 8;
+    const int st0 = 2 * (int)(((int64_t)nsb_all * blockIdx.z) / gridDim.z), st1 = 2 * (int)(((int64_t)nsb_all * (blockIdx.z + 1)) / gridDim.z);
+    dst += (int64_t)blockIdx.z * split_stride;
+    const int64_t row_bytes = (int64_t)(k >> 5) * BB;
+    const int kg = lane >> 5, swz_a = lane & 7;
+
+    // ---- copy roles.  Rows past the end of the tile are clamped to a valid row: an output row depends on its own
+    // activation row only, and the rows past the end are not stored ----
+    const int ra = tid >> 3, pa = tid & 7;                       // activations: piece pa of rows ra + 32 i
+    const int rs = (tid >> 1) & (BMT - 1), half = tid & 1;       // d8 of blocks 2 half, 2 half + 1 of activation row rs
+    const int8_t *a_src[NA];
+#pragma unroll
+    for (int i = 0; i < NA; i++) a_src[i] = av.qs + (int64_t)min(m0 + ra + 32 * i, rows - 1) * k + 16 * pa;
+    const float *d_src = av.d + 2 * ((int64_t)min(m0 + rs, rows - 1) * (k >> 5) + 2 * half);
+    const int a_dst = ra * 128 + 16 * (pa ^ (ra & 7));
+    // ---- weights: this lane's row of each MFMA tile, 16 bytes of quants per block ----
+    const uint8_t *b_src[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++) b_src[j] = w + (int64_t)min(n0 + wn * WN + j * 32 + (lane & 31), n - 1) * row_bytes;
+    const int q_off = DT == CQ_Q8_0 ? 2 + 16 * kg : 2;
+
+    f32x16 acc[MI][NJ];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+    // registers of a stage: activations in flight to LDS, weights of this lane.  Positions past the end of the split's
+    // range are clamped to its last stage: what they bring is not used.
+    u32x4 ga[NA], gds = u32x4{0, 0, 0, 0};
+    struct BRegs { u32x4 q[NJ][4]; uint32_t d[NJ][4]; };
+    BRegs bcur, bnxt;
+    auto load_a = [&](int st) {
+        st = min(st, st1 - 1);
+#pragma unroll
+        for (int i = 0; i < NA; i++) ga[i] = *reinterpret_cast<const u32x4 *>(a_src[i] + st * 128);
+        gds = *reinterpret_cast<const u32x4 *>(d_src + 8 * st);         // {d, sum} pairs of two blocks
+    };
+    auto load_b = [&](int st, BRegs &r) {
+        st = min(st, st1 - 1);
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const uint8_t *blk = b_src[j] + (int64_t)(4 * st + b) * BB;
+                r.q[j][b] = ld_u<u32x4>(blk + q_off);
+                r.d[j][b] = ld_u<uint16_t>(blk);
+            }
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NA; i++) *reinterpret_cast<u32x4 *>(As[buf] + a_dst + 32 * 128 * i) = ga[i];
+        // threads that share a row write the same values
+        sD8[buf][2 * half][rs] = __uint_as_float(gds.x);
+        sD8[buf][2 * half + 1][rs] = __uint_as_float(gds.z);
+    };
+    load_a(st0);
+    load_b(st0, bcur);
+    store_a(st0 & 1);
+    __syncthreads();
+
+    for (int st = st0; st < st1; st++) {
+        const int buf = st & 1;
+        load_a(st + 1);
+        load_b(st + 1, bnxt);
+        const int8_t *Ab = As[buf];
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            i32x4 bop[NJ];
+            float dw[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const u32x4 q = bcur.q[j][b];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    if constexpr (DT == CQ_Q4_0) bop[j][i] = (int)((((q[i] >> (4 * kg)) & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u);
+                    else bop[j][i] = (int)q[i];
+                }
+                dw[j] = h2f(bcur.d[j][b]);
+            }
+#pragma unroll
+            for (int i = 0; i < MI; i++) {
+                const int rl = wm * 64 + i * 32;
+                const i32x4 af = *reinterpret_cast<const i32x4 *>(Ab + (rl + (lane & 31)) * 128 + 16 * ((2 * b + kg) ^ swz_a));
+                f32x4 d8[4];
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) d8[q4] = *reinterpret_cast<const f32x4 *>(&sD8[buf][b][rl + 8 * q4 + 4 * kg]);
+#pragma unroll
+                for (int j = 0; j < NJ; j++) {
+                    i32x16 z;
+#pragma unroll
+                    for (int e = 0; e < 16; e++) z[e] = 0;
+                    const i32x16 sI = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bop[j], z, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf((float)sI[e] * dw[j], d8[e >> 2][e & 3], acc[i][j][e]);
+                }
+            }
+        }
+        store_a(buf ^ 1);
+        bcur = bnxt;
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const int nn = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int mm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * kg + (e & 3);
+                if (mm < rows && nn < n) dst[(int64_t)mm * stride_dst + nn] = acc[i][j][e];
+            }
+        }
+}
+
 // dst[m, n] = sum over the split planes, in split order (deterministic); n % 4 == 0 whenever split-K is chosen
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ part, float *__restrict__ dst, int splits, int64_t n,
                                                             int64_t stride_dst, int64_t count) {
@@ -830,11 +912,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 }
 
 typedef void (*QmmFn)(const uint8_t *, ActView, float *, int, int, int, int64_t, MoeChunks, int64_t, int64_t);
-// the kernel of a format and tile shape: Q4_K runs on the int8 matrix cores, the other formats on the f16 ones
+// the kernel of a format and tile shape: Q4_K, Q4_0 and Q8_0 run on the int8 matrix cores, the other formats on the f16 ones
 template <int DT, int NJ, bool MOE, bool SM>
 QmmFn qmm_fn() {
     if constexpr (DT == CQ_Q4K) return qmm_q4k_i8_kernel<NJ, MOE, SM>;
-    else return qmm_kernel<DT, NJ, MOE, SM>;
+    else if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0) {
+        static_assert(!MOE, "expert-grouped Q4_0 / Q8_0 rows take the matvec kernels");
+        return qmm_q0_i8_kernel<DT, NJ, SM>;
+    } else return qmm_kernel<DT, NJ, MOE, SM>;
 }
 
 template <int DT>

@@ -97,7 +97,7 @@ class LlamaOracle:
         tokens = np.asarray(tokens).reshape(-1)
         seq = tokens.shape[0]
         H, KV, D = cfg.n_head, cfg.n_kv_head, cfg.head_dim
-        x = self.t["tok_embeddings"].astype(f32)[tokens]                        # [seq, hidden]
+        x = np.asarray(self.t["tok_embeddings"])[np.asarray(tokens, dtype=np.int64)].astype(f32)                        # [seq, hidden]
         cos, sin = self.cos[index_pos:index_pos + seq], self.sin[index_pos:index_pos + seq]
         scale = f32(1.0 / math.sqrt(D))
         for li in range(cfg.n_layer):

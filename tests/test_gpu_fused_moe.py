@@ -166,6 +166,42 @@ def test_fused_moe_layer_qwen3_shape_decode_and_graph_replay():
     assert rel_l2(yh.float().cpu().numpy(), want_h) <= 2e-3          # + the f16 rounding of the output
 
 
+_QWEN3 = {}
+
+
+def _qwen3_layer():
+    """One Qwen3-30B-A3B-shape layer (128 experts, top-8, 2048 -> 768 -> 2048, Q4_K), shared by the token counts below.  The
+    expert weights are drawn and quantized on the GPU (bit-exact quantizer, tests/test_gpu_dequant_quant.py); the oracle
+    reads the same block bytes."""
+    if not _QWEN3:
+        from candle_amd.fused_moe import FusedMoeGGUF
+        from candle_amd.quantized import GgmlDType, QTensor
+        E, hidden, inter, topk = 128, 2048, 768, 8
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(60)
+        router = normal(61, (E, hidden), 0.1)
+        shapes = [(E, inter, hidden), (E, inter, hidden), (E, hidden, inter)]
+        qts = [QTensor.quantize(torch.randn(sh, generator=gen, device="cuda") * 0.05, GgmlDType.Q4K) for sh in shapes]
+        blocks = [np.frombuffer(q.data(), dtype=np.uint8) for q in qts]
+        layer = FusedMoeGGUF(torch.from_numpy(router).cuda(), qts[0], qts[1], qts[2], True, topk)
+        _QWEN3["v"] = (layer, fm.FusedMoeOracle(oracle.Q4K, router, blocks[0], blocks[1], blocks[2], E, hidden, inter, topk, True))
+    return _QWEN3["v"]
+
+
+@pytest.mark.parametrize("tokens,is_prefill", [(16, False), (16, True), (256, True), (256, False)])
+def test_fused_moe_layer_qwen3_shape_token_batches(tokens, is_prefill):
+    """16 and 256 tokens through the Qwen3-30B-A3B-shape layer: 128 and 2048 (token, expert) pairs, i.e. the per-pair
+    kernels and the expert-grouped matrix-core tiles, against the CPU restatement of FusedMoeGGUF::forward."""
+    layer, ref = _qwen3_layer()
+    x = normal(70 + tokens, (1, tokens, 2048), 1.0)
+    got = layer.forward(torch.from_numpy(x).cuda(), is_prefill).cpu().numpy()
+    want = ref.forward(x)
+    assert got.shape == want.shape == (1, tokens, 2048)
+    assert rel_l2(got, want) <= 1e-3
+    worst = max(rel_l2(got[0, r], want[0, r]) for r in range(tokens))
+    assert worst <= 1e-3, worst
+
+
 def test_fused_moe_argument_errors():
     from candle_amd.fused_moe import FusedMoeGGUF
     layer, _ = build_layer(oracle.Q4K, 4, 256, 512, 2, True, seed=60)

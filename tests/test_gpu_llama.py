@@ -63,10 +63,90 @@ def test_prefill_then_decode_logits_and_greedy_tokens(cfg_kw, dtypes):
         assert tok_g == tok_w, step
 
 
-def test_q4_0_q8_0_model_decode_path():
-    """Q4_0 / Q8_0 weights: the decode path (up to 8 rows per call) is integer-exact like the CPU.  The prefill
-    matmul rounds these formats' operands to f16 (2e-4 per call, inside the per-call bar); downstream
-    activation quantizers amplify such a perturbation, so a whole-model prefill is only checked loosely."""
+LLAMA3_8B_2L = dict(n_layer=2, hidden=4096, n_head=32, n_kv_head=8, head_dim=128, ffn=14336, vocab=128256, rope_theta=500000.0, rms_eps=1e-5, ctx=64)
+
+
+def test_8b_shape_two_layers_prefill_16_then_decode_4():
+    """Two layers of the Llama-3-8B shape with its full vocabulary (hidden 4096, 32 q / 8 kv heads of 128, FFN 14336,
+    vocab 128256; attn_v / ffn_down Q6_K, the rest and the head Q4_K): 16 prompt tokens in one forward, then 4 greedy
+    single-token steps, logits against the CPU restatement at every step.  The f32 weights are drawn and quantized on the
+    GPU (the quantizer is bit-exact against the CPU one, tests/test_gpu_dequant_quant.py) and the oracle reads the same
+    block bytes.
+
+    What "equal to the CPU" can mean at this width: rows of 4096 .. 14336 activations are re-quantized to int8 before every
+    matmul, and a difference in the last bit of an f32 sum moves some element across a rounding boundary with
+    probability near one at these row lengths; the next quantizers amplify that, and the logits of two correct
+    evaluations settle about 1e-2 apart.  The CPU path shows this against itself: its scalar and AVX2 vec_dot sum the
+    same integers in a different f32 order.  So the test holds every matmul of the model, at the model's shapes and row
+    count, to the 1e-3 bar on identical inputs (2e-6 in fact), and the whole-model logits to twice the distance between
+    the CPU's two evaluations."""
+    import candle_amd as ca
+    from candle_amd.quantized_llama import Config, ModelWeights
+    cfg = Config(**LLAMA3_8B_2L)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(51)
+    qd, kvd = cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim
+    shapes = {"attention_wq": (qd, cfg.hidden), "attention_wk": (kvd, cfg.hidden), "attention_wv": (kvd, cfg.hidden),
+              "attention_wo": (cfg.hidden, qd), "feed_forward_w1": (cfg.ffn, cfg.hidden), "feed_forward_w3": (cfg.ffn, cfg.hidden),
+              "feed_forward_w2": (cfg.hidden, cfg.ffn)}
+
+    def blocks_of(n, k, dt):
+        w = torch.randn((n, k), generator=gen, device="cuda") * 0.02
+        return (int(dt), ca.QTensor.quantize(w, ca.GgmlDType(int(dt))).data())
+
+    def norm_w():
+        return (1.0 + 0.1 * torch.randn(cfg.hidden, generator=gen, device="cuda")).cpu().numpy()
+
+    t = {}
+    for li in range(cfg.n_layer):
+        for name, (n, k) in shapes.items():
+            t[f"blk.{li}.{name}"] = blocks_of(n, k, MIX[name])
+        t[f"blk.{li}.attention_norm"] = norm_w()
+        t[f"blk.{li}.ffn_norm"] = norm_w()
+    t["output"] = blocks_of(cfg.vocab, cfg.hidden, MIX["output"])
+    t["tok_embeddings"] = torch.randn((cfg.vocab, cfg.hidden), generator=gen, device="cuda").cpu().numpy()
+    t["norm"] = norm_w()
+
+    # every matmul of the model on identical inputs: 16 rows (prefill) and 1 row (decode); the head at 1 row
+    rng = np.random.default_rng(53)
+    for name, (n, k) in list(shapes.items()) + [("output", (cfg.vocab, cfg.hidden))]:
+        dt, b = t[name if name == "output" else f"blk.1.{name}"]
+        qmm = ca.QMatMul.from_qtensor(ca.QTensor.new(ca.QStorage.from_data(b, "cuda", ca.GgmlDType(dt)), (n, k)))
+        raw = np.frombuffer(b, dtype=np.uint8)
+        for m in ((1,) if name == "output" else (1, 16)):
+            x = rng.standard_normal((m, k)).astype(np.float32)
+            y = qmm.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+            err = rel_l2(y, oracle.matmul_fast(dt, x, raw, n, 16))
+            assert err <= TOL and err <= 2e-6, (name, m, err)
+        del qmm
+
+    model = ModelWeights.from_blocks(cfg, t)
+    ref, ref_scalar = lo.LlamaOracle(cfg, t, threads=16), lo.LlamaOracle(cfg, t)
+    prompt = np.random.default_rng(52).integers(0, cfg.vocab, size=16).tolist()
+
+    def check(got, toks, pos):
+        want, want_s = ref.forward(toks, pos), ref_scalar.forward(toks, pos)
+        assert got.shape == want.shape == (1, cfg.vocab)
+        spread = rel_l2(want, want_s)
+        bound = max(TOL, 2.0 * spread)
+        assert min(rel_l2(got, want), rel_l2(got, want_s)) <= bound, (pos, rel_l2(got, want), rel_l2(got, want_s), spread)
+        # the greedy token of the GPU is one the CPU ranks within that distance of its own best
+        assert want[0, int(np.argmax(got))] >= want.max() - 4.0 * bound * float(np.abs(want).max()), pos
+        return int(np.argmax(want))
+
+    tok = check(model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy(), prompt, 0)
+    for step in range(4):
+        tok = check(model.forward(torch.tensor([[tok]], dtype=torch.int32), 16 + step).cpu().numpy(), [tok], 16 + step)
+    # the same four steps replayed from a HIP graph give the same tokens as eager single-token forwards
+    a = model.generate_greedy(prompt, 4, use_graph=False)["tokens"]
+    b = model.generate_greedy(prompt, 4, use_graph=True)["tokens"]
+    assert a == b and len(a) == 4
+
+
+def test_q4_0_q8_0_model_prefill_and_decode_paths():
+    """Q4_0 / Q8_0 weights: the matvec kernels (up to 8 rows per call) and the int8 matrix-core kernel (more rows) both sum
+    the integers of the CPU path, so the prompt meets the bar whether it goes through the model in one forward or in
+    two chunks of up to 8 tokens."""
     cfg, t, model = make(SMALL, LEGACY, seed=31)
     ref = lo.LlamaOracle(cfg, t)
     rng = np.random.default_rng(32)
@@ -75,8 +155,9 @@ def test_q4_0_q8_0_model_decode_path():
     model.forward(torch.tensor([prompt[:8]], dtype=torch.int32), 0)
     got = model.forward(torch.tensor([prompt[8:]], dtype=torch.int32), 8).cpu().numpy()
     assert rel_l2(got, want) <= 1e-5
-    loose = model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy()
-    assert rel_l2(loose, want) <= 5e-2
+    whole = model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy()
+    assert rel_l2(whole, want) <= TOL
+    assert int(np.argmax(whole)) == int(np.argmax(want))
 
 
 @pytest.mark.parametrize("dtypes", [OLD_32, Q3_K_M, Q2_K_MIX], ids=["q4_1-q5_0-q5_1", "q3_k_m", "q2k-q3k"])
@@ -188,3 +269,40 @@ def test_forward_argument_errors():
         model.forward(torch.zeros((1, 3), dtype=torch.int32), cfg.ctx - 1)
     with pytest.raises(ValueError):
         model.generate_greedy([1] * 60, 10)
+
+
+def test_random_init_with_a_per_layer_format_override():
+    """A "blk.{i}.{role}" entry gives one layer's tensor another format (and another byte size) than its role: the slab slot,
+    the recorded format and the bytes written must all follow the override.  The model's logits are checked against the CPU
+    restatement run on the blocks read back from the slab."""
+    from candle_amd.quantized import GgmlDType
+    from candle_amd.quantized_llama import Config, ModelWeights, Q4_K_M
+    cfg = Config(**SMALL)
+    dtypes = dict(Q4_K_M)
+    dtypes["blk.1.feed_forward_w2"] = GgmlDType.Q8_0       # larger than the role's Q6_K slot
+    dtypes["blk.0.attention_wq"] = GgmlDType.Q5K
+    dtypes["blk.1.attention_wo"] = GgmlDType.Q4_0          # smaller than the role's Q4_K slot
+    model = ModelWeights.random_init(cfg, seed=3, dtypes=dtypes, weight_scale=0.05)
+    base = model._slab.data_ptr()
+    t = {"tok_embeddings": model.tok_embeddings.cpu().numpy(), "norm": model.norm.cpu().numpy()}
+    for li, lw in enumerate(model.layers):
+        for name, w in lw.w.items():
+            want_dt = GgmlDType(dtypes.get(f"blk.{li}.{name}", dtypes[name]))
+            assert w.dtype == want_dt, (li, name)
+            assert w.nbytes == w.n * w.k // want_dt.block_size() * want_dt.type_size(), (li, name)
+            raw = model._slab[w.ptr - base: w.ptr - base + w.nbytes].cpu().numpy()
+            vals = oracle.to_float(int(want_dt), raw, w.n * w.k)
+            assert np.isfinite(vals).all() and 0.04 <= float(vals.std()) <= 0.06, (li, name, float(vals.std()))
+            t[f"blk.{li}.{name}"] = (int(want_dt), raw.tobytes())
+        t[f"blk.{li}.attention_norm"] = lw.attention_norm.cpu().numpy()
+        t[f"blk.{li}.ffn_norm"] = lw.ffn_norm.cpu().numpy()
+    w = model.output
+    t["output"] = (int(w.dtype), model._slab[w.ptr - base: w.ptr - base + w.nbytes].cpu().numpy().tobytes())
+    ref = lo.LlamaOracle(cfg, t)
+    prompt = [3, 17, 250, 99, 1]
+    got = model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy()
+    want = ref.forward(prompt, 0)
+    assert rel_l2(got, want) <= TOL
+    tok = int(np.argmax(want))
+    got = model.forward(torch.tensor([[tok]], dtype=torch.int32), 5).cpu().numpy()
+    assert rel_l2(got, ref.forward([tok], 5)) <= TOL

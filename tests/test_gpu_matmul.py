@@ -121,9 +121,10 @@ def test_matmul_vs_oracle(dtype, m):
 
 
 def prefill_bound(dtype):
-    """More than 8 rows run on the f16 matrix cores.  K-quant operands are exact integers there (Q6_K as an
-    f16 head plus an exact remainder term); Q4_0 / Q8_0 operands are the dequantized values rounded to f16."""
-    return {oracle.Q4K: TIGHT, oracle.Q5K: TIGHT, oracle.Q6K: TIGHT}.get(dtype, 5e-4)
+    """More than 8 rows run on the matrix cores, every format with the integer sums of the CPU path: K-quant operands
+    are exact integers (f16 cores; Q6_K as an f16 head plus an exact remainder term; Q4_K on the int8 cores), Q4_0 / Q8_0
+    blocks are one int8 MFMA each, scaled in f32 per block like the CPU loop."""
+    return TIGHT
 
 
 @pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
@@ -217,3 +218,49 @@ def test_full_size_equals_dot_of_dequantized(dtype, n, k, batch):
     sub = np.concatenate([blocks[r * rb:(r + 1) * rb] for r in rows])
     want_rows = oracle.matmul(dtype, x, sub, len(rows))
     assert rel_l2(got[:, rows], want_rows) <= (TIGHT if batch <= 8 else prefill_bound(dtype))
+
+
+_FULL = {}
+
+
+def _full_size_weight(dtype, n, k):
+    """One quantized [n, k] weight per (format, shape), shared by the row counts below: (QTensor, dequantized f64 weight on the GPU)."""
+    import candle_amd as ca
+    key = (dtype, n, k)
+    if key not in _FULL:
+        _FULL.clear()                       # one weight at a time: 14336 x 4096 doubles are 470 MB
+        w = torch.from_numpy(normal(81, (n, k), 0.02)).cuda()
+        qt = ca.QTensor.quantize(w, ca.GgmlDType(dtype))
+        _FULL[key] = (qt, qt.dequantize().double())
+    return _FULL[key]
+
+
+@pytest.mark.parametrize("dtype,n,k", [(oracle.Q6K, 4096, 14336), (oracle.Q5K, 14336, 4096), (oracle.Q4_0, 4096, 14336), (oracle.Q4_0, 14336, 4096),
+                                       (oracle.Q4K, 14336, 4096), (oracle.Q4K, 4096, 14336), (oracle.Q8_0, 14336, 4096)],
+                         ids=lambda v: NAMES.get(v, str(v)))
+@pytest.mark.parametrize("m", [128, 512, 2048])
+def test_full_size_prefill_rows(dtype, n, k, m):
+    """The prefill shapes at 128, 512 and 2048 activation rows: every output against the f64 dot of the dequantized
+    operands, three weight rows x all activation rows against the scalar oracle, and the last activation row (the ragged
+    end of the last row tile) against the oracle on 64 evenly spaced weight rows."""
+    import candle_amd as ca
+    qt, wd = _full_size_weight(dtype, n, k)
+    qmm = ca.QMatMul.from_qtensor(qt)
+    x = normal(182 + m, (m, k), 1.0)
+    got = forward(qmm, x)
+    adt = oracle.vec_dot_type(dtype)
+    xq = oracle.to_float(adt, oracle.from_float(adt, x.reshape(-1)), m * k).reshape(m, k)
+    want = (torch.from_numpy(xq).cuda().double() @ wd.t()).cpu().numpy()
+    bound = max(5e-6, prefill_bound(dtype))
+    err = rel_l2(got, want)
+    assert err <= TOL and err <= bound, err
+    worst = max(rel_l2(got[r], want[r]) for r in range(0, m, 37))
+    assert worst <= 4 * bound, worst
+    blocks = np.frombuffer(qt.data(), dtype=np.uint8)
+    rb = (k // oracle.block_size(dtype)) * oracle.type_size(dtype)
+    rows = [0, n // 2 + 1, n - 1]
+    sub = np.concatenate([blocks[r * rb:(r + 1) * rb] for r in rows])
+    assert rel_l2(got[:, rows], oracle.matmul(dtype, x, sub, len(rows))) <= prefill_bound(dtype)
+    rows = list(range(0, n, n // 64))
+    sub = np.concatenate([blocks[r * rb:(r + 1) * rb] for r in rows])
+    assert rel_l2(got[-1:, rows], oracle.matmul(dtype, x[-1:], sub, len(rows))) <= prefill_bound(dtype)

@@ -214,6 +214,43 @@ def test_moe_qwen3_shape_single_token():
         assert err <= TOL and err <= TIGHT, err
 
 
+_QWEN3_EXPERTS = {}
+
+
+@pytest.mark.parametrize("n,k", [(768, 2048), (2048, 768)])
+@pytest.mark.parametrize("tokens", [16, 256])
+@pytest.mark.parametrize("is_prefill", [False, True])
+def test_moe_qwen3_shape_token_batches(n, k, tokens, is_prefill):
+    """128 experts, top-8, Q4_K, 16 and 256 tokens: the gate/up call shape (one activation row per token, no weights) and
+    the down call shape (one row per pair, scaled by the routing weights) against the oracle, every pair row on its own."""
+    import candle_amd as ca
+    E, topk = 128, 8
+    if (n, k) not in _QWEN3_EXPERTS:
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(145)
+        qt = ca.QTensor.quantize(torch.randn((E, n, k), generator=gen, device="cuda") * 0.02, ca.GgmlDType.Q4K)
+        _QWEN3_EXPERTS[(n, k)] = (qt, np.frombuffer(qt.data(), dtype=np.uint8))
+    qt, blocks = _QWEN3_EXPERTS[(n, k)]
+    ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=146 + tokens)
+    sti, eid = torch.from_numpy(sorted_token_ids).cuda(), torch.from_numpy(expert_ids).cuda()
+    x = normal(147, (tokens, k), 1.0)
+    got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, None, sti, eid, topk, is_prefill)
+    torch.cuda.synchronize()
+    want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+    got = got.cpu().numpy()
+    assert got.shape == want.shape == (tokens * topk, n)
+    assert rel_l2(got, want) <= TIGHT
+    assert max(rel_l2(got[r], want[r]) for r in range(tokens * topk)) <= 4 * TIGHT
+    xp = normal(148, (tokens * topk, k), 1.0)
+    twf = tw.reshape(-1)
+    got = ca.moe_gemm_gguf(torch.from_numpy(xp).cuda(), qt, torch.from_numpy(twf).cuda(), sti, eid, topk, is_prefill)
+    torch.cuda.synchronize()
+    want = oracle.moe_gemm_gguf(oracle.Q4K, xp, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
+    got = got.cpu().numpy()
+    assert rel_l2(got, want) <= TIGHT
+    assert max(rel_l2(got[r], want[r]) for r in range(tokens * topk)) <= 4 * TIGHT
+
+
 @pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q6K, oracle.Q8_0, oracle.Q3K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("n,k", [(5, 256), (1, 768), (77, 1024), (130, 2048), (9, 4096)])
 def test_short_expert_rows_ragged(dtype, n, k):
