@@ -83,20 +83,71 @@ def _require_cuda(t: torch.Tensor, what: str) -> None:
 
 
 # ---------------------------------------------------------------------------------------------
-# Per-device grow-only workspace, like the Mutex-guarded scratch of fast_mmvq.rs:44-81.
+# Scratch memory of the library calls: one grow-only buffer per (device, stream), handed out under a lock that is held
+# until the call that uses it has been enqueued, like the Mutex-guarded scratch of fast_mmvq.rs:44-81 (the guard lives
+# as long as the launch).  Calls on one stream run in enqueue order, so they may share a buffer; calls on different
+# streams may overlap on the GPU and get different buffers.  A buffer that is outgrown is kept alive for the life of
+# the process (a HIP graph captured earlier may still replay into it), and growing while the stream is being captured
+# is refused: the caller runs the call once eagerly first, which sizes the buffer.
 # ---------------------------------------------------------------------------------------------
+class _Workspace:
+    def __init__(self):
+        self.lock = threading.Lock()
+        self.buf = None
+        self.retired = []
+
+    def reserve(self, nbytes: int, alloc, capturing) -> torch.Tensor:
+        """The buffer of at least ``nbytes`` bytes; the caller holds ``self.lock``."""
+        if self.buf is None or self.buf.numel() < nbytes:
+            if capturing():
+                raise RuntimeError("the workspace of this stream must grow while the stream is being captured into a graph; "
+                                   "run the call once outside the capture first")
+            if self.buf is not None:
+                self.retired.append(self.buf)
+            self.buf = alloc(max(nbytes, 1 << 20, 2 * self.buf.numel() if self.buf is not None else 0))
+        return self.buf
+
+
 _ws_lock = threading.Lock()
-_workspaces: dict[int, torch.Tensor] = {}
+_workspaces: dict = {}
 
 
-def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    idx = device.index if device.index is not None else torch.cuda.current_device()
-    with _ws_lock:
-        buf = _workspaces.get(idx)
-        if buf is None or buf.numel() < nbytes:
-            buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=torch.device("cuda", idx))
-            _workspaces[idx] = buf
+class _workspace:
+    """``with _workspace(device, nbytes) as ws:`` — the stream's scratch buffer, locked until the block (the enqueue) ends."""
+
+    def __init__(self, device: torch.device, nbytes: int):
+        self.device = device
+        self.nbytes = int(nbytes)
+        self.slot = None
+
+    def _key(self):
+        idx = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        return (idx, torch.cuda.current_stream(idx).cuda_stream)
+
+    def _alloc(self, n: int) -> torch.Tensor:
+        return torch.empty(n, dtype=torch.uint8, device=self.device)
+
+    def _capturing(self) -> bool:
+        return torch.cuda.is_current_stream_capturing()
+
+    def __enter__(self) -> torch.Tensor:
+        key = self._key()
+        with _ws_lock:
+            slot = _workspaces.get(key)
+            if slot is None:
+                slot = _workspaces[key] = _Workspace()
+        slot.lock.acquire()
+        try:
+            buf = slot.reserve(self.nbytes, self._alloc, self._capturing)
+        except BaseException:
+            slot.lock.release()
+            raise
+        self.slot = slot
         return buf
+
+    def __exit__(self, *exc) -> None:
+        self.slot.lock.release()
+        self.slot = None
 
 
 def check_shape(shape: Sequence[int], block_size: int) -> None:
@@ -312,10 +363,10 @@ class QTensor:
         dst = torch.empty((*xs.shape[:-1], n), dtype=xs.dtype, device=xs.device)
         L = _lib.lib()
         need = L.cq_qmatmul_workspace_bytes(int(self.dtype()), m, k, n)
-        ws = _workspace(xs.device, need)
         cq = _TORCH_TO_CQ[xs.dtype]
-        _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(int(self.dtype()), self.device_ptr(), xs.data_ptr(), cq,
-                                                              dst.data_ptr(), cq, m, k, n, ws.data_ptr(), ws.numel(), _stream_ptr()))
+        with _workspace(xs.device, need) as ws:
+            _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(int(self.dtype()), self.device_ptr(), xs.data_ptr(), cq,
+                                                                  dst.data_ptr(), cq, m, k, n, ws.data_ptr(), ws.numel(), _stream_ptr()))
         return dst
 
     def indexed_moe_forward(self, x: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
@@ -341,10 +392,10 @@ class QTensor:
         need = L.cq_indexed_moe_workspace_bytes(int(self.dtype()), E, n, k, batch, topk, input_dim1)
         if need < 0:
             raise ValueError("indexed_moe_forward: unsupported shape (input dim 1 must be topk or 1)")
-        ws = _workspace(x.device, need)
-        _lib.check("cq_indexed_moe_forward", L.cq_indexed_moe_forward(int(self.dtype()), self.device_ptr(), x.data_ptr(), ids32.data_ptr(),
-                                                                      out.data_ptr(), E, n, k, batch, topk, input_dim1,
-                                                                      ws.data_ptr(), ws.numel(), _stream_ptr()))
+        with _workspace(x.device, need) as ws:
+            _lib.check("cq_indexed_moe_forward", L.cq_indexed_moe_forward(int(self.dtype()), self.device_ptr(), x.data_ptr(), ids32.data_ptr(),
+                                                                          out.data_ptr(), E, n, k, batch, topk, input_dim1,
+                                                                          ws.data_ptr(), ws.numel(), _stream_ptr()))
         return out
 
     def __repr__(self) -> str:
@@ -434,9 +485,9 @@ def moe_gemm_gguf(input: torch.Tensor, weights: QTensor, topk_weights: Optional[
     need = L.cq_moe_gemm_workspace_bytes(int(weights.dtype()), E, topk, size_m, size_n, size_k, 0 if tw is None else 1)
     if need < 0:
         raise ValueError("moe_gemm_gguf: unsupported shape")
-    ws = _workspace(input.device, need)
-    _lib.check("cq_moe_gemm_gguf", L.cq_moe_gemm_gguf(int(weights.dtype()), input.data_ptr(), weights.device_ptr(), sti.data_ptr(),
-                                                      eid.data_ptr(), tw.data_ptr() if tw is not None else None, out.data_ptr(),
-                                                      E, topk, size_m, size_n, size_k, 1 if is_prefill else 0,
-                                                      ws.data_ptr(), ws.numel(), _stream_ptr()))
+    with _workspace(input.device, need) as ws:
+        _lib.check("cq_moe_gemm_gguf", L.cq_moe_gemm_gguf(int(weights.dtype()), input.data_ptr(), weights.device_ptr(), sti.data_ptr(),
+                                                          eid.data_ptr(), tw.data_ptr() if tw is not None else None, out.data_ptr(),
+                                                          E, topk, size_m, size_n, size_k, 1 if is_prefill else 0,
+                                                          ws.data_ptr(), ws.numel(), _stream_ptr()))
     return out

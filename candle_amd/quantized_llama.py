@@ -126,16 +126,16 @@ class ModelWeights:
                 nb = L.cq_storage_bytes(int(dt_of(li, name)), n * k)
                 if nb < 0:
                     raise ValueError(f"{name}: {n}x{k} is not a whole number of {dt_of(li, name).name} blocks")
-                plan.append((li, name, total, nb, n, k))
+                plan.append((li, name, total, nb, n, k, dt_of(li, name)))
                 total += (nb + 255) // 256 * 256
         nb = L.cq_storage_bytes(int(dtypes["output"]), cfg.vocab * cfg.hidden)
-        plan.append((-1, "output", total, nb, cfg.vocab, cfg.hidden))
+        plan.append((-1, "output", total, nb, cfg.vocab, cfg.hidden, GgmlDType(dtypes["output"])))
         total += (nb + 255) // 256 * 256
         self._slab = torch.empty(total, dtype=torch.uint8, device=self.device)
         base = self._slab.data_ptr()
         self.layers = [LayerWeights() for _ in range(cfg.n_layer)]
-        for li, name, off, nb, n, k in plan:
-            w = _W(base + off, GgmlDType(dtypes[name]) if li < 0 else dt_of(li, name), n, k, nb)
+        for li, name, off, nb, n, k, dt in plan:
+            w = _W(base + off, dt, n, k, nb)
             if li < 0:
                 self.output = w
             else:
@@ -190,16 +190,17 @@ class ModelWeights:
     @classmethod
     def random_init(cls, cfg: Config, seed: int = 0, device="cuda:0", dtypes: Optional[Dict[str, GgmlDType]] = None,
                     weight_scale: float = 0.02) -> "ModelWeights":
-        """Random-init weights ~N(0, weight_scale) quantized on the device (norm weights = 1, f32 embedding table)."""
+        """Random-init weights ~N(0, weight_scale) quantized on the device (norm weights = 1, f32 embedding table).
+        ``dtypes`` maps a tensor role to its format; a ``"blk.{i}.{role}"`` entry overrides the role's format for layer i."""
         self = cls(cfg, device)
         dtypes = dict(Q4_K_M if dtypes is None else dtypes)
         plan = self._alloc(dtypes)
         gen = torch.Generator(device=self.device)
         gen.manual_seed(seed)
         base = self._slab.data_ptr()
-        for li, name, off, nb, n, k in plan:
+        for li, name, off, nb, n, k, dt in plan:
             wf = torch.randn((n, k), generator=gen, device=self.device, dtype=torch.float32) * weight_scale
-            _lib.check("cq_quantize", self.L.cq_quantize(int(dtypes[name]), wf.data_ptr(), base + off, n * k, None))
+            _lib.check("cq_quantize", self.L.cq_quantize(int(dt), wf.data_ptr(), base + off, n * k, None))
             torch.cuda.synchronize(self.device)
             del wf
         self.tok_embeddings = torch.randn((cfg.vocab, cfg.hidden), generator=gen, device=self.device, dtype=torch.float32) * weight_scale
@@ -224,7 +225,7 @@ class ModelWeights:
             if dt not in _MATMUL_DTYPES:
                 raise NotImplementedError(f"{key}: no matmul kernel for {dt.name} weights")
         plan = self._alloc(dtypes)
-        for li, name, off, nb, n, k in plan:
+        for li, name, off, nb, n, k, _ in plan:
             dt, blocks = tensors["output" if li < 0 else f"blk.{li}.{name}"]
             raw = np.frombuffer(bytes(blocks), dtype=np.uint8)
             if raw.size != nb:

@@ -96,3 +96,78 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(ImportError, match="no fallback"):
         _lib.lib()
+
+
+# ---------------------------------------------------------------------------- the workspace guard (no GPU: allocation and stream stubbed)
+class _CpuWorkspace:
+    """candle_amd.quantized._workspace with the three GPU-facing hooks replaced: CPU allocations, a settable stream key and capture flag."""
+
+    def __new__(cls, stream, nbytes, capturing=False):
+        import torch
+        from candle_amd import quantized as q
+
+        class G(q._workspace):
+            def _key(self):
+                return (0, stream)
+
+            def _alloc(self, n):
+                return torch.empty(n, dtype=torch.uint8)
+
+            def _capturing(self):
+                return capturing
+
+        return G(torch.device("cpu"), nbytes)
+
+
+def test_workspace_guard_holds_the_lock_until_the_block_ends():
+    import threading
+    import time
+    events = []
+    inside = threading.Event()
+    release = threading.Event()
+
+    def first():
+        with _CpuWorkspace(stream=101, nbytes=1000) as ws:
+            events.append(("first in", ws.data_ptr()))
+            inside.set()
+            release.wait(5)
+            time.sleep(0.05)
+            events.append(("first out", ws.data_ptr()))
+
+    def second(stream, tag):
+        inside.wait(5)
+        with _CpuWorkspace(stream=stream, nbytes=5 << 20) as ws:      # larger: would replace the first thread's buffer
+            events.append((tag, ws.data_ptr()))
+
+    t1 = threading.Thread(target=first)
+    t2 = threading.Thread(target=second, args=(101, "same stream"))
+    t3 = threading.Thread(target=second, args=(202, "other stream"))
+    t1.start(); t2.start(); t3.start()
+    t3.join(5)                     # another stream's buffer is independent: not blocked by the first thread
+    assert not t3.is_alive() and [e[0] for e in events] == ["first in", "other stream"]
+    time.sleep(0.1)
+    assert t2.is_alive()           # the same stream's second call waits for the first call's enqueue to end
+    release.set()
+    t1.join(5); t2.join(5)
+    assert [e[0] for e in events] == ["first in", "other stream", "first out", "same stream"]
+    ptrs = dict(events)
+    assert ptrs["same stream"] != ptrs["first in"] and ptrs["other stream"] != ptrs["first in"]
+
+
+def test_workspace_guard_keeps_outgrown_buffers_and_refuses_to_grow_under_capture():
+    from candle_amd import quantized as q
+    with _CpuWorkspace(stream=303, nbytes=10) as a:
+        pa, na = a.data_ptr(), a.numel()
+    assert na >= 1 << 20
+    with _CpuWorkspace(stream=303, nbytes=100) as b:
+        assert b.data_ptr() == pa                     # no growth: the same buffer
+    with _CpuWorkspace(stream=303, nbytes=na + 1) as c:
+        assert c.numel() >= 2 * na                    # geometric growth bounds what the retired buffers add up to
+    slot = q._workspaces[(0, 303)]
+    assert [t.data_ptr() for t in slot.retired] == [pa]      # still alive: a captured graph may replay into it
+    with pytest.raises(RuntimeError, match="captured"):
+        with _CpuWorkspace(stream=303, nbytes=c.numel() + 1, capturing=True):
+            pass
+    assert not slot.lock.locked()                     # a refused call leaves the stream's lock free
+    with _CpuWorkspace(stream=303, nbytes=1000, capturing=True) as d:
+        assert d.data_ptr() == c.data_ptr()           # a call that fits may be captured
