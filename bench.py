@@ -11,16 +11,27 @@ the matvec, which this library runs as ONE kernel.  Inputs are resident in HBM w
 starts.  Steps rotate through a pool of distinct weight tensors larger than the 256 MB Infinity
 Cache, so every step streams its 33 MB of weights from HBM.
 
+At least 200 launches are timed after at least 20 warm-up launches, whatever --steps / --warmup say.
+
 The JSON line carries, besides the driver contract fields:
   roofline      achieved algorithmic GB/s of the dominant (only) kernel of the step, from HIP events
-                around back-to-back launches on the launch stream, against the 8 TB/s HBM peak;
+                around back-to-back launches on the launch stream, against the 8 TB/s HBM peak, with
+                the median / p10 / p90 over per-replay event pairs (one replay = one rotation of the pool);
                 `traffic` = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE runs
-                (read from the committed summary under profiles/ when present)
+                (read from the committed summary under profiles/, with the commit it was measured at)
   cpu_baseline  the C restatement of candle's CPU path (AVX2 dot products + column-split threads,
-                oracle/cq_oracle_fast.c) timed on this box's host cores on a bounded sample
+                oracle/cq_oracle_fast.c) timed on this box's host cores on bounded samples, for the headline
+                configuration and for three more (Q8_0 4096x4096 batch 1, the headline shape at batch 16,
+                Q6_K 4096x14336 at 128 rows), with the CPU model and the thread count
+  cfg1, cfg2_sweep, prefill, moe, decode_8b
+                compact records of the other configurations: the Q8_0 4096 x 4096 matvec, the Q4_K batch sweep
+                on both FFN shapes, the prefill matmuls at 128 / 512 / 2048 rows, the 48-layer MoE stack at
+                1 / 16 / 256 tokens and the 8B-shape decoder
 
     python bench.py --pmc-mode     a handful of un-graphed launches of the step kernel plus one plain
                                    256 MiB device copy, for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`
+    python bench.py --workload prefill --pmc-mode --wdtype q4k --n 14336 --k 4096 --batch 2048
+                                   the same for the prefill matmul: a few plain launches of QMatMul::forward
     python bench.py --workload prefill --wdtype q6k --n 4096 --k 14336 --batch 512
                                    the prefill matmul (other BASELINE configurations; not the headline line):
                                    TFLOP/s of QMatMul::forward and of its MFMA kernel against the 2.5 PFLOP/s
@@ -44,11 +55,15 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_I8_PEAK_TOPS = 5000.0
+MIN_TIMED_LAUNCHES = 200
+MIN_WARMUP_LAUNCHES = 20
 Q4K = 12
 WDTYPES = {"q4_0": (2, 18, 32), "q8_0": (8, 34, 32), "q4k": (12, 144, 256), "q5k": (13, 176, 256), "q6k": (14, 210, 256),
            "q4_1": (3, 20, 32), "q5_0": (6, 22, 32), "q5_1": (7, 24, 32), "q2k": (10, 84, 256), "q3k": (11, 110, 256)}
 FMT_NAMES = {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4k": "Q4_K", "q5k": "Q5_K", "q6k": "Q6_K", "q4_1": "Q4_1", "q5_0": "Q5_0", "q5_1": "Q5_1",
              "q2k": "Q2_K", "q3k": "Q3_K"}
+# formats whose prefill kernel runs on the int8 matrix cores (the others use the f16 ones)
+I8_PREFILL = ("q4k", "q4_0", "q8_0")
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "q4k_decode_matvec_1x4096x14336_pmc.txt")
 
 
@@ -58,31 +73,124 @@ def algorithmic_bytes(n, k, m, type_size, block):
 
 
 def committed_traffic():
-    """HBM bytes per launch measured with rocprofv3 --pmc (see the summary file for the commands)."""
+    """(HBM bytes per launch, commit) measured with rocprofv3 --pmc; the summary file holds the commands."""
     try:
-        m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", open(TRAFFIC_SUMMARY).read())
-        return int(m.group(1)) if m else None
+        text = open(TRAFFIC_SUMMARY).read()
     except OSError:
-        return None
+        return None, None
+    m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", text)
+    c = re.search(r"measured_at_commit\s*=\s*([0-9a-f]+)", text)
+    return (int(m.group(1)) if m else None), (c.group(1) if c else None)
 
 
-def prefill(args):
-    """QMatMul::forward with more than 8 activation rows: Q8_K / Q8_0 activation quantization kernel + MFMA matmul kernel."""
-    import torch
+def percentiles(samples):
+    xs = sorted(samples)
+    pick = lambda q: xs[min(len(xs) - 1, int(round(q * (len(xs) - 1))))]
+    return {"median": pick(0.5), "p10": pick(0.1), "p90": pick(0.9), "n": len(xs)}
 
+
+def quantized_weight(L, torch, dt, n, k, gen, dev, scale=0.02):
+    """[n, k] f32 ~N(0, scale) quantized on the device, in row chunks so that the f32 source stays below 1 GB."""
     from candle_amd import _lib
+    wbytes = L.cq_storage_bytes(dt, n * k)
+    wq = torch.empty(wbytes, dtype=torch.uint8, device=dev)
+    rows = max(1, min(n, (1 << 28) // k))
+    row_bytes = wbytes // n
+    for r0 in range(0, n, rows):
+        r = min(rows, n - r0)
+        wf = torch.randn((r, k), generator=gen, device=dev, dtype=torch.float32) * scale
+        _lib.check("cq_quantize", L.cq_quantize(dt, wf.data_ptr(), wq.data_ptr() + r0 * row_bytes, r * k, None))
+        torch.cuda.synchronize()
+        del wf
+    return wq
 
-    L = _lib.lib()
+
+class Rotation:
+    """One activation batch against a pool of distinct [n, k] weights, larger than the 256 MB Infinity Cache, captured as one
+    HIP graph per rotation of the pool; timing with HIP events on the launch stream."""
+
+    def __init__(self, L, torch, fmt, n, k, m, pool_mb, seed=1234):
+        from candle_amd import _lib
+        self.L, self.torch, self._lib = L, torch, _lib
+        self.dt, self.ts, self.bs = WDTYPES[fmt]
+        self.n, self.k, self.m = n, k, m
+        dev = torch.device("cuda:0")
+        self.wbytes = L.cq_storage_bytes(self.dt, n * k)
+        self.alg_bytes = algorithmic_bytes(n, k, m, self.ts, self.bs)
+        self.pool = max(2, (pool_mb * 1000 * 1000 + self.wbytes - 1) // self.wbytes)
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(seed)
+        self.weights = [quantized_weight(L, torch, self.dt, n, k, gen, dev) for _ in range(self.pool)]
+        self.x = torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32)
+        self.dst = torch.empty((m, n), dtype=torch.float32, device=dev)
+        self.ws_bytes = L.cq_qmatmul_workspace_bytes(self.dt, m, k, n)
+        self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
+        self.stream = torch.cuda.Stream(device=dev)
+        torch.cuda.synchronize()
+
+    def step(self, i, sp):
+        """QMatMul::forward: for up to 8 rows, activation quantization + matvec in one kernel."""
+        self._lib.check("cq_qmatmul_forward", self.L.cq_qmatmul_forward(self.dt, self.weights[i % self.pool].data_ptr(), self.x.data_ptr(), 0,
+                                                                       self.dst.data_ptr(), 0, self.m, self.k, self.n, self.ws.data_ptr(), self.ws_bytes, sp))
+
+    def capture(self, fn, same_weight=False):
+        torch = self.torch
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(self.stream):
+            fn(0, self.stream.cuda_stream)          # warm the code path before capture
+            self.stream.synchronize()
+            with torch.cuda.graph(g, stream=self.stream):
+                sp = torch.cuda.current_stream().cuda_stream
+                for i in range(self.pool):
+                    fn(0 if same_weight else i, sp)
+        return g
+
+    def run(self, graph, launches):
+        reps = max(1, (launches + self.pool - 1) // self.pool)
+        with self.torch.cuda.stream(self.stream):
+            for _ in range(reps):
+                graph.replay()
+        return reps * self.pool
+
+    def event_us(self, graph, launches, warmup):
+        """Mean microseconds per launch over back-to-back replays (one event pair around all of them)."""
+        torch = self.torch
+        self.run(graph, warmup)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(self.stream):
+            e0.record(self.stream)
+            done = self.run(graph, launches)
+            e1.record(self.stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / done
+
+    def replay_stats(self, graph, launches, warmup):
+        """Microseconds per launch of every replay on its own (an event between replays): median / p10 / p90."""
+        torch = self.torch
+        self.run(graph, warmup)
+        torch.cuda.synchronize()
+        reps = max(8, (launches + self.pool - 1) // self.pool)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        with torch.cuda.stream(self.stream):
+            ev[0].record(self.stream)
+            for r in range(reps):
+                graph.replay()
+                ev[r + 1].record(self.stream)
+        torch.cuda.synchronize()
+        st = percentiles([ev[r].elapsed_time(ev[r + 1]) * 1e3 / self.pool for r in range(reps)])
+        return {"median_us": round(st["median"], 3), "p10_us": round(st["p10"], 3), "p90_us": round(st["p90"], 3), "replays": st["n"],
+                "launches_per_replay": self.pool}
+
+
+def prefill_record(L, torch, fmt, n, k, m, steps=20, warmup=5, pmc=False):
+    """QMatMul::forward with more than 8 activation rows: Q8_K / Q8_0 activation quantization kernel + MFMA matmul kernel."""
+    from candle_amd import _lib
     dev = torch.device("cuda:0")
-    dt, ts, bs = WDTYPES[args.wdtype]
-    n, k, m = args.n, args.k, args.batch
+    dt, ts, bs = WDTYPES[fmt]
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
-    wbytes = L.cq_storage_bytes(dt, n * k)
-    wf = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
-    wq = torch.empty(wbytes, dtype=torch.uint8, device=dev)
-    _lib.check("cq_quantize", L.cq_quantize(dt, wf.data_ptr(), wq.data_ptr(), n * k, None))
-    del wf
+    wq = quantized_weight(L, torch, dt, n, k, gen, dev)
     x = torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32)
     dst = torch.empty((m, n), dtype=torch.float32, device=dev)
     ws_bytes = L.cq_qmatmul_workspace_bytes(dt, m, k, n)
@@ -97,21 +205,27 @@ def prefill(args):
     def matmul_only():
         _lib.check("cq_matmul", L.cq_matmul(dt, wq.data_ptr(), ws.data_ptr(), dst.data_ptr(), k, n, m, n, sp))
 
-    def event_us(fn, steps):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    if pmc:
         with torch.cuda.stream(stream):
-            for _ in range(args.warmup):
-                fn()
-            e0.record(stream)
-            for _ in range(steps):
-                fn()
-            e1.record(stream)
+            for _ in range(4):
+                forward()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / steps
+        return {"pmc_mode": True, "workload": "%s prefill [%d x %d] x [%d x %d]^T" % (fmt, m, k, n, k), "launches": 4}
 
-    steps = args.steps
+    def event_us(fn, count):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(count + 1)]
+        with torch.cuda.stream(stream):
+            for _ in range(warmup):
+                fn()
+            ev[0].record(stream)
+            for i in range(count):
+                fn()
+                ev[i + 1].record(stream)
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[count]) * 1e3 / count, percentiles([ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(count)])
+
     with torch.cuda.stream(stream):
-        for _ in range(args.warmup):
+        for _ in range(warmup):
             forward()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -121,20 +235,36 @@ def prefill(args):
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / steps
     flops = 2.0 * m * n * k
-    kern_us = event_us(matmul_only, steps)
-    # Q4_K runs on the int8 matrix cores (two int8 MACs per algorithmic MAC: the scale is split in two), the other formats
-    # on the f16 ones; the roofline is priced in algorithmic flop against the peak of the unit used
-    i8 = args.wdtype == "q4k"
+    kern_us, kst = event_us(matmul_only, steps)
+    # the roofline is priced in algorithmic flop against the dense peak of the matrix-core type the kernel uses
+    i8 = fmt in I8_PREFILL
     peak = MFMA_I8_PEAK_TOPS if i8 else MFMA_F16_PEAK_TFLOPS
     achieved = flops / (kern_us * 1e-6) / 1e12
+    return {"fmt": fmt, "n": n, "k": k, "m": m, "steps": steps, "warmup": warmup, "forward_ms": round(ms, 5),
+            "forward_TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1), "kernel": "qmm_q4k_i8_kernel" if fmt == "q4k" else ("qmm_q0_i8_kernel<%s>" if i8 else "qmm_kernel<%s>") % fmt,
+            "kernel_us": round(kern_us, 2), "kernel_median_us": round(kst["median"], 2), "kernel_p10_us": round(kst["p10"], 2),
+            "kernel_p90_us": round(kst["p90"], 2), "kernel_TFLOPs": round(achieved, 1), "mfma": "i8" if i8 else "f16", "peak": peak,
+            "frac": round(achieved / peak, 4)}
+
+
+def prefill(args):
+    import torch
+
+    from candle_amd import _lib
+    r = prefill_record(_lib.lib(), torch, args.wdtype, args.n, args.k, args.batch, max(args.steps, 20), max(args.warmup, 5), pmc=args.pmc_mode)
+    if args.pmc_mode:
+        print(json.dumps(r))
+        return
     print(json.dumps({
-        "metric": "%s prefill matmul TFLOP/s @%dx%d, M=%d" % (args.wdtype, n, k, m), "value": round(flops / (ms * 1e-3) / 1e12, 1),
-        "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "i8 operands, i32 accumulate" if i8 else "f16 operands, f32 accumulate", "data": "synthetic",
-        "config": {"workload": "%s prefill matmul [%d x %d] x [%d x %d]^T" % (args.wdtype, m, k, n, k),
-                   "step": "QMatMul::forward = activation quantization kernel + MFMA matmul kernel", "n": n, "k": k, "batch": m},
-        "roofline": {"bound": "mfma", "kernel": "qmm_q4k_i8_kernel" if i8 else "qmm_kernel<%s>" % args.wdtype, "achieved": round(achieved, 1),
-                     "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": None, "avg_kernel_us": round(kern_us, 2)},
+        "metric": "%s prefill matmul TFLOP/s @%dx%d, M=%d" % (args.wdtype, args.n, args.k, args.batch), "value": r["forward_TFLOPs"],
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": r["steps"], "warmup": r["warmup"], "ms_per_step": r["forward_ms"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "i8 operands, i32 accumulate" if r["mfma"] == "i8" else "f16 operands, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "%s prefill matmul [%d x %d] x [%d x %d]^T" % (args.wdtype, args.batch, args.k, args.n, args.k),
+                   "step": "QMatMul::forward = activation quantization kernel + MFMA matmul kernel", "n": args.n, "k": args.k, "batch": args.batch},
+        "roofline": {"bound": "mfma", "kernel": r["kernel"], "achieved": r["kernel_TFLOPs"], "peak": r["peak"], "unit": "TFLOP/s", "frac": r["frac"],
+                     "traffic": None, "avg_kernel_us": r["kernel_us"], "median_us": r["kernel_median_us"], "p10_us": r["kernel_p10_us"],
+                     "p90_us": r["kernel_p90_us"]},
     }))
 
 
@@ -186,37 +316,31 @@ def decode8b(args):
 
 
 def moe(args):
-    """BASELINE configs[4]: Qwen3-30B-A3B-shaped MoE layer (128 experts, top-8, hidden 2048, expert FFN 768, Q4_K):
-    the three expert matmuls of one layer (gate, up on [tokens, hidden]; down on [tokens*8, ffn]) through
-    QTensor::indexed_moe_forward, rotated over several distinct layers, for 1 / 16 / 256 tokens."""
+    """BASELINE configs[4]: Qwen3-30B-A3B-shaped MoE layer stack (48 layers, 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K,
+    16 GB of expert weights, every layer with weights of its own): the three expert matmuls of each layer (gate, up on
+    [tokens, hidden]; down on [tokens*8, ffn]) through QTensor::indexed_moe_forward, and the whole layers through
+    FusedMoeGGUF::forward, for 1 / 16 / 256 tokens, each as one HIP graph over all layers."""
     import torch
 
     from candle_amd import _lib
+    from candle_amd.fused_moe import FusedMoeGGUF
+    from candle_amd.quantized import GgmlDType, QStorage, QTensor
 
     L = _lib.lib()
     dev = torch.device("cuda:0")
-    E, H, F, TOPK, NL = 128, 2048, 768, 8, 6
+    E, H, F, TOPK, NL = 128, 2048, 768, 8, args.moe_layers
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
-
-    def experts(n, k):
-        nb = L.cq_storage_bytes(Q4K, E * n * k)
-        w = torch.empty(nb, dtype=torch.uint8, device=dev)
-        for e in range(E):
-            wf = torch.randn((n, k), generator=gen, device=dev) * 0.02
-            _lib.check("cq_quantize", L.cq_quantize(Q4K, wf.data_ptr(), w.data_ptr() + e * (nb // E), n * k, None))
-        torch.cuda.synchronize()
-        return w
-
-    gate, up, down = [experts(F, H) for _ in range(NL)], [experts(F, H) for _ in range(NL)], [experts(H, F) for _ in range(NL)]
+    gate = [quantized_weight(L, torch, Q4K, E * F, H, gen, dev) for _ in range(NL)]
+    up = [quantized_weight(L, torch, Q4K, E * F, H, gen, dev) for _ in range(NL)]
+    down = [quantized_weight(L, torch, Q4K, E * H, F, gen, dev) for _ in range(NL)]
     router = torch.randn((E, H), generator=gen, device=dev)
-    from candle_amd.fused_moe import FusedMoeGGUF
-    from candle_amd.quantized import GgmlDType, QStorage, QTensor
 
     def qt(buf, n, k):
         return QTensor.new(QStorage(buf, GgmlDType.Q4K), (E, n, k))
 
     fused = [FusedMoeGGUF(router, qt(gate[i], F, H), qt(up[i], F, H), qt(down[i], H, F), True, TOPK) for i in range(NL)]
+    reps, warm = max(1, (MIN_TIMED_LAUNCHES + NL - 1) // NL), max(1, (MIN_WARMUP_LAUNCHES + NL - 1) // NL)
     results = []
     for tokens in [int(t) for t in args.moe_tokens.split(",")]:
         x = torch.randn((tokens, H), generator=gen, device=dev)
@@ -231,57 +355,101 @@ def moe(args):
         ws = torch.empty(nws, dtype=torch.uint8, device=dev)
 
         def layer(i, sp):
-            for w, src, dst, n, k, d1 in ((gate[i % NL], xg, o1, F, H, 1), (up[i % NL], xg, o2, F, H, 1), (down[i % NL], h, o3, H, F, TOPK)):
+            for w, src, dst, n, k, d1 in ((gate[i], xg, o1, F, H, 1), (up[i], xg, o2, F, H, 1), (down[i], h, o3, H, F, TOPK)):
                 _lib.check("cq_indexed_moe_forward", L.cq_indexed_moe_forward(Q4K, w.data_ptr(), src.data_ptr(), ids32.data_ptr(), dst.data_ptr(),
                                                                               E, n, k, tokens, TOPK, d1, ws.data_ptr(), nws, sp))
 
         st = torch.cuda.Stream(device=dev)
-        with torch.cuda.stream(st):
-            layer(0, st.cuda_stream)
-            st.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=st):
-                for i in range(NL):
-                    layer(i, torch.cuda.current_stream().cuda_stream)
-            g.replay()
-            st.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            reps = 20
-            e0.record(st)
-            for _ in range(reps):
-                g.replay()
-            e1.record(st)
-            st.synchronize()
-        us = e0.elapsed_time(e1) * 1e3 / (reps * NL)
-        # the whole layer as FusedMoeGGUF::forward runs it: router + softmax + top-k, sort by expert, three grouped
-        # matmuls (moe_gemm_gguf), silu(gate) * up, sum over top-k
         x3 = x.reshape(1, tokens, H)
         y = torch.empty((tokens, H), device=dev)
-        with torch.cuda.stream(st):
-            fused[0].forward(x3, tokens > 1, out=y)
-            st.synchronize()
-            g2 = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g2, stream=st):
-                for i in range(NL):
-                    fused[i].forward(x3, tokens > 1, out=y)
-            g2.replay()
-            st.synchronize()
-            e0.record(st)
-            for _ in range(reps):
-                g2.replay()
-            e1.record(st)
-            st.synchronize()
-        fused_us = e0.elapsed_time(e1) * 1e3 / (reps * NL)
+
+        def timed(run_layer):
+            """per-layer microseconds of a graph over all NL layers: mean, and median / p10 / p90 over the replays"""
+            with torch.cuda.stream(st):
+                run_layer(0)
+                st.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=st):
+                    for i in range(NL):
+                        run_layer(i)
+                for _ in range(warm):
+                    g.replay()
+                st.synchronize()
+                ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+                ev[0].record(st)
+                for r in range(reps):
+                    g.replay()
+                    ev[r + 1].record(st)
+                st.synchronize()
+            pst = percentiles([ev[r].elapsed_time(ev[r + 1]) * 1e3 / NL for r in range(reps)])
+            return ev[0].elapsed_time(ev[reps]) * 1e3 / (reps * NL), pst
+
+        us, ust = timed(lambda i: layer(i, torch.cuda.current_stream().cuda_stream))
+        # the whole layer as FusedMoeGGUF::forward runs it: router + softmax + top-k, sort by expert, three grouped
+        # matmuls (moe_gemm_gguf), silu(gate) * up, sum over top-k
+        fused_us, fst = timed(lambda i: fused[i].forward(x3, tokens > 1, out=y))
         alg = distinct * 3 * 884736
-        results.append({"tokens": tokens, "distinct_experts": distinct, "layer_us": round(us, 1), "algorithmic_MB": round(alg / 1e6, 1),
-                        "GBps": round(alg / us / 1e3, 1), "tok_s_48_layers_expert_matmuls_only": round(tokens / (48 * us * 1e-6), 1),
-                        "fused_moe_layer_us": round(fused_us, 1)})
-    print(json.dumps({"metric": "Qwen3-30B-A3B-shape MoE layer, expert matmuls (Q4_K, 128 experts, top-8)", "unit": "us per layer", "n_gpus": 1,
-                      "data": "synthetic", "config": {"workload": "gate + up [tokens, 2048] -> 768 and down [tokens*8, 768] -> 2048 via indexed_moe_forward, "
-                                                                  "6 distinct layers rotated (2 GB), HIP graph; fused_moe_layer_us: the same "
-                                                                  "layers through FusedMoeGGUF::forward (router, top-k, sort, moe_gemm_gguf x3, "
-                                                                  "silu*up, sum over top-k)"},
-                      "results": results}))
+        results.append({"tokens": tokens, "distinct_experts": distinct, "layer_us": round(us, 1), "layer_median_us": round(ust["median"], 1),
+                        "layer_p10_us": round(ust["p10"], 1), "layer_p90_us": round(ust["p90"], 1), "algorithmic_MB": round(alg / 1e6, 1),
+                        "GBps": round(alg / us / 1e3, 1), "frac_of_hbm_peak": round(alg / us / 1e3 / HBM_PEAK_GBPS, 4),
+                        "fused_moe_layer_us": round(fused_us, 1), "fused_moe_layer_median_us": round(fst["median"], 1),
+                        "tok_s_%d_layers_fused" % NL: round(tokens / (NL * fused_us * 1e-6), 1), "timed_layer_launches": reps * NL})
+    out = {"metric": "Qwen3-30B-A3B-shape MoE layer, expert matmuls (Q4_K, 128 experts, top-8)", "unit": "us per layer", "n_gpus": 1,
+           "data": "synthetic", "config": {"workload": "gate + up [tokens, 2048] -> 768 and down [tokens*8, 768] -> 2048 via indexed_moe_forward, "
+                                                       "%d layers with distinct weights (%.1f GB) in one HIP graph; fused_moe_layer_us: the same "
+                                                       "layers through FusedMoeGGUF::forward (router, top-k, sort, moe_gemm_gguf x3, "
+                                                       "silu*up, sum over top-k)" % (NL, NL * 3 * E * F * H * 0.5625 / 1e9), "layers": NL},
+           "results": results}
+    del gate, up, down, fused
+    torch.cuda.empty_cache()
+    return out
+
+
+def cpu_info():
+    """(model name, physical cores this process may run on, threads used): threads = physical cores, at most the 16 the box allots."""
+    model, phys = "unknown", set()
+    try:
+        allowed = os.sched_getaffinity(0)
+        cur = {}
+        for line in open("/proc/cpuinfo"):
+            if ":" in line:
+                key, val = [t.strip() for t in line.split(":", 1)]
+                cur[key] = val
+            elif cur:
+                if int(cur.get("processor", -1)) in allowed:
+                    phys.add((cur.get("physical id", "0"), cur.get("core id", cur.get("processor"))))
+                model = cur.get("model name", model)
+                cur = {}
+        if cur and int(cur.get("processor", -1)) in allowed:
+            phys.add((cur.get("physical id", "0"), cur.get("core id", cur.get("processor"))))
+    except (OSError, ValueError):
+        pass
+    n_phys = max(1, len(phys))
+    return model, n_phys, max(1, min(n_phys, 16))
+
+
+def cpu_matmul_baseline(torch, fmt, n, k, m, threads, seconds, copies, seed=77):
+    """The C restatement of candle's CPU QMatMul::forward (Q8_K / Q8_0 activation quantization + AVX2 vec_dot + column split over
+    threads) on host copies of GPU-quantized weights, rotated so that the weights come from DRAM; time-bounded."""
+    import oracle
+    from candle_amd import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    dt, ts, bs = WDTYPES[fmt]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    hw = [quantized_weight(L, torch, dt, n, k, gen, dev).cpu().numpy() for _ in range(copies)]
+    hx = torch.randn((m, k), generator=gen, device=dev).cpu().numpy()
+    oracle.matmul_fast(dt, hx, hw[0], n, threads)
+    t0 = time.perf_counter()
+    it = 0
+    while time.perf_counter() - t0 < seconds or it < 2:
+        oracle.matmul_fast(dt, hx, hw[it % copies], n, threads)
+        it += 1
+    dt_s = (time.perf_counter() - t0) / it
+    alg = algorithmic_bytes(n, k, m, ts, bs)
+    return {"workload": "%s [%d x %d] x %d rows" % (FMT_NAMES[fmt], n, k, m), "ms_per_call": round(dt_s * 1e3, 4), "GBps": round(alg / dt_s / 1e9, 2),
+            "GFLOPs": round(2.0 * m * n * k / dt_s / 1e9, 1), "calls": it, "seconds": round(dt_s * it, 1), "weight_copies": copies}
 
 
 def main():
@@ -293,16 +461,17 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="--workload decode8b: number of decoder layers")
     ap.add_argument("--prompt", type=int, default=512, help="--workload decode8b: prompt tokens")
     ap.add_argument("--moe-tokens", default="1,16,256", help="--workload moe: token counts, comma separated")
+    ap.add_argument("--moe-layers", type=int, default=48, help="--workload moe: layers, each with its own expert weights (340 MB per layer)")
     ap.add_argument("--wdtype", choices=sorted(WDTYPES), default="q4k",
-                    help="weight format of --workload prefill / decode (the metric is quoted on q4k; other formats skip the 8B decoder and the CPU baseline)")
+                    help="weight format of --workload prefill / decode (the metric is quoted on q4k; other formats skip the other configurations)")
     ap.add_argument("--n", type=int, default=14336)
     ap.add_argument("--k", type=int, default=4096)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--pool-mb", type=int, default=1280, help="distinct weight bytes rotated through (MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--cpu-seconds", type=float, default=8.0, help="CPU time of the headline baseline; the three others take 3 s each")
     ap.add_argument("--pmc-mode", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the labelled context numbers (cache-resident, pre-quantized)")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline step: skip the context numbers and the other configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every configuration of the metric is single-GPU); use --gpus 1")
@@ -310,13 +479,17 @@ def main():
         print(json.dumps(decode8b(args)))
         return
     if args.workload == "moe":
-        return moe(args)
+        print(json.dumps(moe(args)))
+        return
     if args.steps is None:
         args.steps = 4000 if args.workload == "decode" else 50
     if args.warmup is None:
         args.warmup = 400 if args.workload == "decode" else 5
     if args.workload == "prefill":
         return prefill(args)
+    # the protocol's floor, whatever the flags say
+    args.steps = max(args.steps, MIN_TIMED_LAUNCHES)
+    args.warmup = max(args.warmup, MIN_WARMUP_LAUNCHES)
 
     import torch
 
@@ -328,125 +501,75 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     n, k, m = args.n, args.k, args.batch
-    WDT, w_ts, w_bs = WDTYPES[args.wdtype]
     fmt = FMT_NAMES[args.wdtype]
-    headline = args.wdtype == "q4k"
+    headline = args.wdtype == "q4k" and (n, k, m) == (14336, 4096, 1)
     if not headline:
         args.no_cpu_baseline = True
-    wbytes = L.cq_storage_bytes(WDT, n * k)
-    alg_bytes = algorithmic_bytes(n, k, m, w_ts, w_bs)
 
     # ---- synthetic inputs, resident in HBM --------------------------------------------------
-    pool = max(2, (args.pool_mb * 1000 * 1000 + wbytes - 1) // wbytes)
-    if args.pmc_mode:
-        pool = 8
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(1234)
-    weights = []
-    for i in range(pool):
-        wf = torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32) * 0.02
-        wq = torch.empty(wbytes, dtype=torch.uint8, device=dev)
-        _lib.check("cq_quantize", L.cq_quantize(WDT, wf.data_ptr(), wq.data_ptr(), n * k, None))
-        weights.append(wq)
-        del wf
-    x = torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32)
-    dst = torch.empty((m, n), dtype=torch.float32, device=dev)
-    ws_bytes = L.cq_qmatmul_workspace_bytes(WDT, m, k, n)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    torch.cuda.synchronize()
-
-    stream = torch.cuda.Stream(device=dev)
-
-    def step(i, sp):
-        """QMatMul::forward: activation quantization + matvec in one kernel."""
-        _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(WDT, weights[i % pool].data_ptr(), x.data_ptr(), 0, dst.data_ptr(), 0,
-                                                              m, k, n, ws.data_ptr(), ws_bytes, sp))
-
-    def matvec_prequantized(i, sp):
-        _lib.check("cq_matvec", L.cq_matvec(WDT, weights[i % pool].data_ptr(), ws.data_ptr(), dst.data_ptr(), 0, k, n, m, n, sp))
+    rot = Rotation(L, torch, args.wdtype, n, k, m, 270 if args.pmc_mode else args.pool_mb)
+    pool, alg_bytes, wbytes, stream = rot.pool, rot.alg_bytes, rot.wbytes, rot.stream
 
     if args.pmc_mode:
         # plain launches (one dispatch row per kernel in the counter CSV) + a copy of known size
         with torch.cuda.stream(stream):
             for i in range(2 * pool):
-                step(i, stream.cuda_stream)
+                rot.step(i, stream.cuda_stream)
             a = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
             b = torch.empty_like(a)
             stream.synchronize()
             for _ in range(4):
                 b.copy_(a)
         torch.cuda.synchronize()
-        print(json.dumps({"pmc_mode": True, "copy_bytes": 256 << 20, "step_algorithmic_bytes": alg_bytes}))
+        print(json.dumps({"pmc_mode": True, "copy_bytes": 256 << 20, "step_algorithmic_bytes": alg_bytes, "step_launches": 2 * pool}))
         return
 
-    # The step is a few microseconds of GPU work: capture one rotation over the pool in a HIP graph
+    # The step is a few microseconds of GPU work: one rotation over the pool is captured in a HIP graph
     # so that host launch latency is not what gets measured.
-    def capture(fn, same_weight=False):
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(stream):
-            fn(0, stream.cuda_stream)          # warm the code path before capture
-            stream.synchronize()
-            with torch.cuda.graph(g, stream=stream):
-                sp = torch.cuda.current_stream().cuda_stream
-                for i in range(pool):
-                    fn(0 if same_weight else i, sp)
-        return g
-
-    def run(graph, steps):
-        reps = max(1, (steps + pool - 1) // pool)
-        with torch.cuda.stream(stream):
-            for _ in range(reps):
-                graph.replay()
-        return reps * pool
-
-    def event_us(graph, steps):
-        run(graph, args.warmup)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        with torch.cuda.stream(stream):
-            e0.record(stream)
-            done = run(graph, steps)
-            e1.record(stream)
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / done
-
-    g_step = capture(step)
+    g_step = rot.capture(rot.step)
 
     # ---- timed region: K steps (rounded up to whole rotations of the pool), wall clock ------------
-    run(g_step, args.warmup)
+    rot.run(g_step, args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    done = run(g_step, args.steps)
+    done = rot.run(g_step, args.steps)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / done
     value = alg_bytes / (ms_per_step * 1e-3) / 1e9
 
     # ---- dominant kernel (the step IS one kernel): HIP events around the same back-to-back launches ----
-    kern_us = event_us(g_step, args.steps)
+    kern_us = rot.event_us(g_step, args.steps, args.warmup)
+    stats = rot.replay_stats(g_step, args.steps, args.warmup)
     achieved = alg_bytes / (kern_us * 1e-6) / 1e9
     # context numbers, labelled: the same kernel with the weights resident in the Infinity Cache (one
     # tensor reused), and the matvec over activations quantized beforehand by cq_quantize_act
     extra = None
     if not args.no_extra:
-        resident_us = event_us(capture(step, same_weight=True), args.steps)
-        _lib.check("cq_quantize_act", L.cq_quantize_act(WDT, x.data_ptr(), 0, ws.data_ptr(), k, m, None))
+        def matvec_prequantized(i, sp):
+            _lib.check("cq_matvec", L.cq_matvec(rot.dt, rot.weights[i % pool].data_ptr(), rot.ws.data_ptr(), rot.dst.data_ptr(), 0, k, n, m, n, sp))
+
+        resident_us = rot.event_us(rot.capture(rot.step, same_weight=True), args.steps, args.warmup)
+        _lib.check("cq_quantize_act", L.cq_quantize_act(rot.dt, rot.x.data_ptr(), 0, rot.ws.data_ptr(), k, m, None))
         torch.cuda.synchronize()
-        preq_us = event_us(capture(matvec_prequantized), args.steps)
-        # the yardstick: a kernel that only reads the same rotated tensors, same launch shape
-        sink = torch.zeros(4, dtype=torch.int32, device=dev)
-        read_bytes = wbytes - wbytes % 16
-
-        def plain_read(i, sp):
-            _lib.check("cq_bench_read", L.cq_bench_read(weights[i % pool].data_ptr(), read_bytes, sink.data_ptr(), sp))
-
-        read_us = event_us(capture(plain_read), args.steps)
-        extra = {"plain_read_us": round(read_us, 3), "plain_read_GBps": round(read_bytes / (read_us * 1e-6) / 1e9, 1),
-                 "infinity_cache_resident_us": round(resident_us, 3),
+        preq_us = rot.event_us(rot.capture(matvec_prequantized), args.steps, args.warmup)
+        extra = {"infinity_cache_resident_us": round(resident_us, 3),
                  "infinity_cache_resident_GBps": round(alg_bytes / (resident_us * 1e-6) / 1e9, 1),
                  "prequantized_matvec_us": round(preq_us, 3),
                  "prequantized_matvec_GBps": round(alg_bytes / (preq_us * 1e-6) / 1e9, 1)}
+        # the yardstick: a kernel that only reads the same rotated tensors, same launch shape
+        bench_lib = _lib.bench_lib()
+        if bench_lib is not None:
+            sink = torch.zeros(4, dtype=torch.int32, device=dev)
+            read_bytes = wbytes - wbytes % 16
 
+            def plain_read(i, sp):
+                _lib.check("cq_bench_read", bench_lib.cq_bench_read(rot.weights[i % pool].data_ptr(), read_bytes, sink.data_ptr(), sp))
+
+            read_us = rot.event_us(rot.capture(plain_read), args.steps, args.warmup)
+            extra.update({"plain_read_us": round(read_us, 3), "plain_read_GBps": round(read_bytes / (read_us * 1e-6) / 1e9, 1)})
+
+    traffic, traffic_commit = committed_traffic() if headline else (None, None)
     out = {
         "metric": "%s matvec GB/s @%dx%d (decode, batch %d)" % (fmt, k, n, m),
         "value": round(value, 1),
@@ -463,43 +586,81 @@ def main():
         "config": {"workload": "%s decode matvec 1x%d->%d, weight [%d x %d] %s, batch %d, %d distinct weight tensors rotated (%.2f GB)"
                                % (fmt, k, n, n, k, fmt, m, pool, pool * wbytes / 1e9),
                    "step": "QMatMul::forward = %s activation quantization + matvec in one kernel, launches captured in a HIP graph"
-                           % ("Q8_K" if w_bs == 256 else "Q8_0"),
+                           % ("Q8_K" if rot.bs == 256 else "Q8_0"),
                    "n": n, "k": k, "batch": m},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
-        "roofline": {"bound": "hbm", "kernel": "qmv_kernel<%s, NB=%d, fused f32 activations>" % (fmt, m), "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": committed_traffic() if headline else None,
-                     "avg_kernel_us": round(kern_us, 3), "algorithmic_bytes_per_launch": alg_bytes},
+        "roofline": {"bound": "hbm", "kernel": "%s<%s, %d row%s, fused f32 activations>" % (
+                         "qms_kernel" if args.wdtype in ("q4k", "q5k") and m == 1 else "qmv_kernel", fmt, m, "" if m == 1 else "s"),
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": traffic, "traffic_commit": traffic_commit, "avg_kernel_us": round(kern_us, 3), "median_us": stats["median_us"],
+                     "p10_us": stats["p10_us"], "p90_us": stats["p90_us"], "timed_launches": stats["replays"] * pool,
+                     "replays": stats["replays"], "algorithmic_bytes_per_launch": alg_bytes},
         "extra": extra,
     }
+    del rot, g_step
+    torch.cuda.empty_cache()
 
     if not args.no_extra and headline:
-        # the second half of the metric: the 8B-shape decoder (same protocol as --workload decode8b)
-        d8 = argparse.Namespace(layers=32, prompt=512, steps=256)
-        r = decode8b(d8)
-        out["decode_8b"] = {"tok_s": r["value"], "ms_per_token": r["ms_per_step"], "prompt_tok_s": r["prompt_tok_s"],
-                            "frac_of_roofline_tok_s": r["roofline"]["frac_of_roofline_tok_s"],
-                            "roofline_tok_s": r["roofline"]["roofline_tok_s_weights_only"],
-                            "weight_bytes_per_token": r["weight_bytes_per_token"], "workload": r["config"]["workload"]}
+        out.update(other_configurations(L, torch, args))
 
     if not args.no_cpu_baseline:
-        import oracle
-        cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "16")), 16)
-        host_pool = min(pool, 8)
-        hw = [weights[i].cpu().numpy() for i in range(host_pool)]
-        hx = x.cpu().numpy()
-        oracle.matmul_fast(Q4K, hx, hw[0], n, cores)
-        t0 = time.perf_counter()
-        it = 0
-        while time.perf_counter() - t0 < args.cpu_seconds:
-            oracle.matmul_fast(Q4K, hx, hw[it % host_pool], n, cores)
-            it += 1
-        dt = (time.perf_counter() - t0) / it
-        out["cpu_baseline"] = {"value": round(alg_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+        model, n_phys, threads = cpu_info()
+        head = cpu_matmul_baseline(torch, "q4k", n, k, 1, threads, args.cpu_seconds, copies=8)
+        out["cpu_baseline"] = {"value": head["GBps"], "unit": "GB/s", "cores": threads, "kind": "port",
                                "sample": "%d calls of the same 1x%d->%d Q4_K matvec over %d rotated host weight copies (%.1f s); "
                                          "C restatement of candle's CPU path: Q8_K activation quantize + AVX2 vec_dot + column split over threads"
-                                         % (it, k, n, host_pool, args.cpu_seconds),
-                               "ms_per_call": round(dt * 1e3, 4)}
+                                         % (head["calls"], k, n, head["weight_copies"], head["seconds"]),
+                               "ms_per_call": head["ms_per_call"], "cpu_model": model, "physical_cores_available": n_phys,
+                               "threads_rule": "physical cores, at most the 16 this box allots to one GPU",
+                               "others": {"cfg1_q8_0_4096x4096_b1": cpu_matmul_baseline(torch, "q8_0", 4096, 4096, 1, threads, 3.0, copies=16),
+                                          "cfg2_q4k_14336x4096_b16": cpu_matmul_baseline(torch, "q4k", 14336, 4096, 16, threads, 3.0, copies=8),
+                                          "cfg3_q6k_4096x14336_m128": cpu_matmul_baseline(torch, "q6k", 4096, 14336, 128, threads, 3.0, copies=4)}}
     print(json.dumps(out))
+
+
+def other_configurations(L, torch, args):
+    """Compact records of the configurations the metric is not quoted on."""
+    out = {}
+    # cfg1: the single Q8_0 matvec, 4096 x 4096, batch 1
+    rot = Rotation(L, torch, "q8_0", 4096, 4096, 1, 600)
+    g = rot.capture(rot.step)
+    us = rot.event_us(g, 2000, 200)
+    st = rot.replay_stats(g, 2000, 200)
+    out["cfg1"] = {"workload": "Q8_0 matvec 1x4096->4096, %d weights rotated" % rot.pool, "us": round(us, 3), "median_us": st["median_us"],
+                   "p10_us": st["p10_us"], "p90_us": st["p90_us"], "GBps": round(rot.alg_bytes / us / 1e3, 1),
+                   "frac_of_hbm_peak": round(rot.alg_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del rot, g
+    torch.cuda.empty_cache()
+    # cfg2: the Q4_K batch sweep on both FFN shapes (batch 16 takes the matrix-core kernel: two kernels per step)
+    sweep = []
+    for (n, k) in ((14336, 4096), (4096, 14336)):
+        for b in (1, 2, 4, 8, 16):
+            rot = Rotation(L, torch, "q4k", n, k, b, 600)
+            g = rot.capture(rot.step)
+            us = rot.event_us(g, 1000, 100)
+            st = rot.replay_stats(g, 1000, 100)
+            sweep.append({"n": n, "k": k, "batch": b, "us": round(us, 3), "median_us": st["median_us"], "p10_us": st["p10_us"], "p90_us": st["p90_us"],
+                          "GBps": round(rot.alg_bytes / us / 1e3, 1), "frac_of_hbm_peak": round(rot.alg_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
+            del rot, g
+            torch.cuda.empty_cache()
+    out["cfg2_sweep"] = sweep
+    # cfg3: prefill at 128 / 512 / 2048 rows
+    pf = []
+    for fmt, n, k in (("q6k", 4096, 14336), ("q5k", 14336, 4096), ("q4_0", 4096, 14336), ("q4_0", 14336, 4096), ("q4k", 14336, 4096)):
+        for m in (128, 512, 2048):
+            pf.append(prefill_record(L, torch, fmt, n, k, m, steps=20, warmup=5))
+            torch.cuda.empty_cache()
+    out["prefill"] = pf
+    # cfg4: the 8B-shape decoder (same protocol as --workload decode8b)
+    r = decode8b(argparse.Namespace(layers=32, prompt=512, steps=256))
+    out["decode_8b"] = {"tok_s": r["value"], "ms_per_token": r["ms_per_step"], "prompt_tok_s": r["prompt_tok_s"],
+                        "frac_of_roofline_tok_s": r["roofline"]["frac_of_roofline_tok_s"],
+                        "roofline_tok_s": r["roofline"]["roofline_tok_s_weights_only"],
+                        "weight_bytes_per_token": r["weight_bytes_per_token"], "workload": r["config"]["workload"]}
+    # cfg5: the 48-layer MoE stack
+    mo = moe(argparse.Namespace(moe_layers=48, moe_tokens="1,16,256"))
+    out["moe"] = {"workload": mo["config"]["workload"], "results": mo["results"]}
+    return out
 
 
 if __name__ == "__main__":

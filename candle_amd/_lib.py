@@ -37,7 +37,6 @@ SIGNATURES = {
     "cq_indexed_moe_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _i64]),
     "cq_indexed_moe_forward": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_moe_gemm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _int]),
-    "cq_bench_read": (_int, [_vp, _i64, _vp, _vp]),
     "cq_moe_gemm_gguf_swiglu": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     "cq_moe_direct_pairs": (_int, [_int, _i64, _i64, _i64]),
     "cq_moe_gemm_gguf_pair": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
@@ -98,6 +97,22 @@ def lib() -> ctypes.CDLL:
             fn.argtypes = args
         _lib = L
     return _lib
+
+
+BENCH_LIB_PATH = os.path.join(_HERE, "libcq_bench.so")
+_bench = None
+
+
+def bench_lib():
+    """libcq_bench.so, the benchmark's plain-read yardstick kernel (candle_amd/csrc/cq_bench.hip): a measurement aid that is
+    not part of the C ABI.  None when it has not been built."""
+    global _bench
+    if _bench is None and os.path.exists(BENCH_LIB_PATH):
+        B = ctypes.CDLL(BENCH_LIB_PATH)
+        B.cq_bench_read.restype = _int
+        B.cq_bench_read.argtypes = [_vp, _i64, _vp, _vp]
+        _bench = B
+    return _bench
 
 
 def status_string(status: int) -> str:

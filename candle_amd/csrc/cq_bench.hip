@@ -1,7 +1,7 @@
-// Measurement aid: a plain streaming read of a device buffer, the yardstick the decode matvec is held against
-// (what this GPU delivers to a kernel that only reads, at the same launch size and from the same memory).
+// Measurement aid, built into a library of its own (libcq_bench.so) that only the benchmark loads: a plain streaming read of
+// a device buffer, the yardstick the decode matvec is held against (what this GPU delivers to a kernel that only reads,
+// at the same launch size and from the same memory).  Not part of the quantized-matmul C ABI.
 #include "cq_device.h"
-#include "cq_launch.h"
 
 namespace {
 
@@ -26,7 +26,13 @@ __global__ __launch_bounds__(1024) void read_kernel(const u32x4 *__restrict__ p,
 
 }  // namespace
 
-int cq_bench_read_launch(const void *src, int64_t bytes, void *sink, hipStream_t s) {
-    hipLaunchKernelGGL(read_kernel, dim3(256), dim3(1024), 0, s, (const u32x4 *)src, bytes / 16, (uint32_t *)sink);
+// Reads `bytes` (a multiple of 16) of `src_dev` (16-byte aligned) on `stream`; `sink_dev` holds at least 4 bytes.
+// Returns 0, -2 for a bad size, -4 for a null pointer, -3 for a misaligned one, or the hipError_t of the launch.
+extern "C" int cq_bench_read(const void *src_dev, int64_t bytes, void *sink_dev, void *stream) {
+    if (bytes < 0 || bytes % 16) return -2;
+    if (bytes == 0) return 0;
+    if (!src_dev || !sink_dev) return -4;
+    if (((uintptr_t)src_dev & 15) || ((uintptr_t)sink_dev & 3)) return -3;
+    hipLaunchKernelGGL(read_kernel, dim3(256), dim3(1024), 0, (hipStream_t)stream, (const u32x4 *)src_dev, bytes / 16, (uint32_t *)sink_dev);
     return (int)hipGetLastError();
 }

@@ -42,7 +42,6 @@ int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst
 int cq_qmm_splits(int64_t k, int64_t n, int64_t rows);
 bool cq_use_mfma(int w_dtype, int64_t rows, int64_t k);
 int cq_embedding_launch(int dtype, const void *blocks, const uint32_t *ids, float *out, int64_t n_ids, int64_t rows, int64_t hidden, hipStream_t s);
-int cq_bench_read_launch(const void *src, int64_t bytes, void *sink, hipStream_t s);
 int cq_convert_f32_launch(const float *src, void *dst, int dst_dtype, int64_t count, hipStream_t s);
 
 // ---- MoE: both public entry points reduce to "pairs" (expert, activation row, output row, scale) ----
