@@ -755,11 +755,13 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
 // MFMA is exactly one block: its int32 result S is the sum the CPU vec_dot forms for that block (k_quants.rs:294-311,
 // 720-738), and each lane folds its 16 results into the f32 accumulators as (float(S) * d[n]) * d8[m], block after block
 // in k order like the CPU loop.  That scaling is three vector instructions per result and bounds the kernel; the matrix
-// cores idle most of the time.  A stage is 128 elements of k (four blocks).  The int8 activations go through LDS as
-// in the Q4_K kernel (two copies, one barrier per stage) together with the stage's four d8 per row; the weights do
-// not: lane (n, kg) of the B operand wants 16 consecutive k of row n, which are the 16 quant bytes of the block (Q4_0: low
-// nibbles for kg = 0, high nibbles for kg = 1) or one half of its 32 (Q8_0), so every lane fetches its own 16 bytes and
-// the block's scale straight from memory, one stage ahead, into registers.
+// cores idle most of the time.  A stage is 128 elements of k (four blocks), held twice in LDS (one barrier per stage):
+// the int8 activations as in the Q4_K kernel, the four d8 per activation row, and the weight rows' four blocks as they
+// lie in memory (72 / 136 contiguous bytes per row), copied in 8-byte pieces by neighbouring lanes so that a load
+// instruction touches a handful of cache lines, not one per lane.  Lane (n, kg) of the B operand wants 16 consecutive k of
+// row n: the 16 quant bytes of the block (Q4_0: low nibbles for kg = 0, high nibbles for kg = 1) or one half of its 32
+// (Q8_0), read from LDS at the block's own 2-byte alignment.  Needs 8-byte aligned weights (row lengths are multiples of
+// 256 elements, so every row and stage then starts on 8 bytes).
 //   Q4_0: nibble q -> int8 (q - 8) on four bytes at once: (x + 0x78787878) ^ 0x80808080 (no carries: x < 16 per byte).
 template <int DT, int NJ, bool SM = false>
 __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst,
@@ -771,7 +773,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
     constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;
     constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
     constexpr int NA = BMT / 32;                                // 16-byte activation pieces a thread copies per stage
+    constexpr int RS = 4 * BB, PPR = RS / 8;                    // bytes and 8-byte pieces of a weight row per stage
+    constexpr int NBP = (BN * PPR + 255) / 256;                 // weight pieces a thread copies per stage (the last round is partial)
     __shared__ __align__(16) int8_t As[2][BMT * 128];           // [row][8 pieces], piece p of row r at p ^ (r & 7)
+    __shared__ __align__(16) uint8_t Bq[2][BN * RS];            // [row][four blocks]
     __shared__ __align__(16) float sD8[2][4][BMT];              // d8 of the stage's four blocks
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -793,10 +798,16 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
     for (int i = 0; i < NA; i++) a_src[i] = av.qs + (int64_t)min(m0 + ra + 32 * i, rows - 1) * k + 16 * pa;
     const float *d_src = av.d + 2 * ((int64_t)min(m0 + rs, rows - 1) * (k >> 5) + 2 * half);
     const int a_dst = ra * 128 + 16 * (pa ^ (ra & 7));
-    // ---- weights: this lane's row of each MFMA tile, 16 bytes of quants per block ----
-    const uint8_t *b_src[NJ];
+    // weights: piece (tid + 256 i) of the tile's BN x PPR pieces, row-major; pieces past the end repeat the last one
+    const uint8_t *b_src[NBP];
+    int b_dst[NBP];
 #pragma unroll
-    for (int j = 0; j < NJ; j++) b_src[j] = w + (int64_t)min(n0 + wn * WN + j * 32 + (lane & 31), n - 1) * row_bytes;
+    for (int i = 0; i < NBP; i++) {
+        const int p = min(tid + 256 * i, BN * PPR - 1), r = p / PPR, c = p - r * PPR;
+        b_src[i] = w + (int64_t)min(n0 + r, n - 1) * row_bytes + 8 * c;
+        b_dst[i] = r * RS + 8 * c;
+    }
+    // MFMA operand roles: this lane's weight row of tile j, and where its 16 quant bytes sit inside a block
     const int q_off = DT == CQ_Q8_0 ? 2 + 16 * kg : 2;
 
     f32x16 acc[MI][NJ];
@@ -807,58 +818,50 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    // registers of a stage: activations in flight to LDS, weights of this lane.  Positions past the end of the split's
-    // range are clamped to its last stage: what they bring is not used.
+    // registers of the stage in flight.  Positions past the end of the split's range are clamped to its last stage: what
+    // they bring lands in an LDS copy that nobody reads.
     u32x4 ga[NA], gds = u32x4{0, 0, 0, 0};
-    struct BRegs { u32x4 q[NJ][4]; uint32_t d[NJ][4]; };
-    BRegs bcur, bnxt;
-    auto load_a = [&](int st) {
+    u32x2 gb[NBP];
+    auto load_stage = [&](int st) {
         st = min(st, st1 - 1);
 #pragma unroll
         for (int i = 0; i < NA; i++) ga[i] = *reinterpret_cast<const u32x4 *>(a_src[i] + st * 128);
         gds = *reinterpret_cast<const u32x4 *>(d_src + 8 * st);         // {d, sum} pairs of two blocks
-    };
-    auto load_b = [&](int st, BRegs &r) {
-        st = min(st, st1 - 1);
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const uint8_t *blk = b_src[j] + (int64_t)(4 * st + b) * BB;
-                r.q[j][b] = ld_u<u32x4>(blk + q_off);
-                r.d[j][b] = ld_u<uint16_t>(blk);
-            }
+        for (int i = 0; i < NBP; i++) gb[i] = *reinterpret_cast<const u32x2 *>(b_src[i] + (int64_t)st * RS);
     };
-    auto store_a = [&](int buf) {
+    auto store_stage = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < NA; i++) *reinterpret_cast<u32x4 *>(As[buf] + a_dst + 32 * 128 * i) = ga[i];
+#pragma unroll
+        for (int i = 0; i < NBP; i++) *reinterpret_cast<u32x2 *>(Bq[buf] + b_dst[i]) = gb[i];     // repeated pieces rewrite the same bytes
         // threads that share a row write the same values
         sD8[buf][2 * half][rs] = __uint_as_float(gds.x);
         sD8[buf][2 * half + 1][rs] = __uint_as_float(gds.z);
     };
-    load_a(st0);
-    load_b(st0, bcur);
-    store_a(st0 & 1);
+    load_stage(st0);
+    store_stage(st0 & 1);
     __syncthreads();
 
     for (int st = st0; st < st1; st++) {
         const int buf = st & 1;
-        load_a(st + 1);
-        load_b(st + 1, bnxt);
+        load_stage(st + 1);
         const int8_t *Ab = As[buf];
+        const uint8_t *Bb = Bq[buf];
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             i32x4 bop[NJ];
             float dw[NJ];
 #pragma unroll
             for (int j = 0; j < NJ; j++) {
-                const u32x4 q = bcur.q[j][b];
+                const uint8_t *blk = Bb + (wn * WN + j * 32 + (lane & 31)) * RS + b * BB;
+                const u32x4 q = ld_u<u32x4>(blk + q_off);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     if constexpr (DT == CQ_Q4_0) bop[j][i] = (int)((((q[i] >> (4 * kg)) & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u);
                     else bop[j][i] = (int)q[i];
                 }
-                dw[j] = h2f(bcur.d[j][b]);
+                dw[j] = h2f(ld_u<uint16_t>(blk));
             }
 #pragma unroll
             for (int i = 0; i < MI; i++) {
@@ -878,8 +881,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
                 }
             }
         }
-        store_a(buf ^ 1);
-        bcur = bnxt;
+        store_stage(buf ^ 1);
         __syncthreads();
     }
 
@@ -926,9 +928,9 @@ template <int DT>
 int launch_qmm(const void *w, const ActView &av, float *dst, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s,
                float *split_ws) {
     // 128 x 64 tiles (two workgroups per CU) everywhere except Q4_0 / Q8_0 problems whose grid of 128 x 128 tiles still
-    // covers the chip: their cheap operand conversion leaves that tile (one workgroup per CU, half the activation
-    // conversions) ahead (measured in TFLOP/s, Q4_0 14336 x 4096: 512 rows 471 -> 582, 2048 rows 527 -> 650; Q8_0
-    // 4096 x 4096: 2048 rows 419 -> 520, but 512 rows, a grid of 128, 340 -> 207)
+    // covers the chip (one workgroup per CU, half the weight-operand builds per activation row).  For the int8 kernel the
+    // two tile shapes are within 10 % of each other (measured in TFLOP/s at 2048 rows, 128 x 128 against 128 x 64 tiles:
+    // Q4_0 14336 x 4096 440 / 500, Q4_0 4096 x 14336 461 / 439, Q8_0 14336 x 4096 460 / 447; 512 rows 360 / 351).
     const bool wide = !cq_is_kquant(DT) && ((rows + 127) / 128) * ((n + 127) / 128) >= 384;
     // a few dozen activation rows (batched decode): 32 x 128 tiles, so that the matrix cores and the activation staging
     // are not spent on 128-row tiles that are mostly padding
@@ -1047,7 +1049,9 @@ bool cq_use_mfma(int w_dtype, int64_t rows, int64_t k) {
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s, float *split_ws) {
     ActView av = cq_act_view(scratch, w_dtype, k, rows);
-    if (cq_use_mfma(w_dtype, rows, k)) {
+    // the Q4_0 / Q8_0 matrix-core kernel copies weight rows in 8-byte pieces; weights at another alignment take the loop below
+    const bool q0_unaligned = (w_dtype == CQ_Q4_0 || w_dtype == CQ_Q8_0) && ((uintptr_t)w & 7) != 0;
+    if (cq_use_mfma(w_dtype, rows, k) && !q0_unaligned) {
         switch (w_dtype) {
             case CQ_Q4_0: return launch_qmm<CQ_Q4_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q8_0: return launch_qmm<CQ_Q8_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);

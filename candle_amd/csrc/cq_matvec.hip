@@ -1426,8 +1426,16 @@ int launch_pair(const void *wa, int64_t na, float *dsta, const void *wb, int64_t
         if (stream_geom<DTB>(gt, k, nb, CQ_F32) && gt.bpr <= 16) return launch_pair<DTB, DTA, PRO>(wb, nb, dstb, wa, na, dsta, src, k, s, fz_in);
     }
     if constexpr (DTA == CQ_Q4K || DTA == CQ_Q5K) {
-        const int rc = launch_pair_stream<DTA, DTB, PRO>(wa, na, dsta, wb, nb, dstb, (const float *)src.x, k, s, fz_in);
+        int rc = launch_pair_stream<DTA, DTB, PRO>(wa, na, dsta, wb, nb, dstb, (const float *)src.x, k, s, fz_in);
         if (rc != CQ_ERR_RANGE) return rc;
+        // the two-tensor launch does not take this call (the tensors or their outputs lie further apart than its 32-bit
+        // distances, or a geometry it has no kernel for): when a single call would stream, two launches, each on the
+        // kernel a single call gets, so that the results do not depend on where the buffers happen to lie
+        StreamGeom gt;
+        if (stream_geom<DTA>(gt, k, na, CQ_F32) || stream_geom<DTB>(gt, k, nb, CQ_F32)) {
+            rc = launch_fused1<DTA, PRO, EPI_NONE>(wa, src, dsta, k, na, s, fz_in);
+            return rc ? rc : launch_fused1<DTB, PRO, EPI_NONE>(wb, src, dstb, k, nb, s, fz_in);
+        }
     }
     QmvGeom ga, gb;
     int64_t groups_a, groups_b;
