@@ -171,3 +171,17 @@ def test_workspace_guard_keeps_outgrown_buffers_and_refuses_to_grow_under_captur
     assert not slot.lock.locked()                     # a refused call leaves the stream's lock free
     with _CpuWorkspace(stream=303, nbytes=1000, capturing=True) as d:
         assert d.data_ptr() == c.data_ptr()           # a call that fits may be captured
+
+
+def test_rust_ffi_declarations_match_the_headers():
+    """rust/candle-hip-quant/src/ffi.rs is generated from the two headers; the generator's check mode fails when it is stale.
+    Every ffi:: call of the crate's lib.rs names a declared entry point."""
+    import subprocess
+    import sys
+    crate = os.path.join(ROOT, "rust", "candle-hip-quant")
+    r = subprocess.run([sys.executable, os.path.join(crate, "gen_ffi.py"), "--check"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    declared = set(re.findall(r"pub fn (cq_\w+)", open(os.path.join(crate, "src", "ffi.rs")).read()))
+    assert declared == set(_lib.SIGNATURES)
+    used = set(re.findall(r"ffi::(cq_\w+)", open(os.path.join(crate, "src", "lib.rs")).read()))
+    assert used and used <= declared
