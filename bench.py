@@ -63,7 +63,7 @@ WDTYPES = {"q4_0": (2, 18, 32), "q8_0": (8, 34, 32), "q4k": (12, 144, 256), "q5k
 FMT_NAMES = {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4k": "Q4_K", "q5k": "Q5_K", "q6k": "Q6_K", "q4_1": "Q4_1", "q5_0": "Q5_0", "q5_1": "Q5_1",
              "q2k": "Q2_K", "q3k": "Q3_K"}
 # formats whose prefill kernel runs on the int8 matrix cores (the others use the f16 ones)
-I8_PREFILL = ("q4k", "q4_0", "q8_0")
+I8_PREFILL = ("q4k", "q4_0", "q8_0", "q4_1", "q5_0", "q5_1")
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "q4k_decode_matvec_1x4096x14336_pmc.txt")
 
 

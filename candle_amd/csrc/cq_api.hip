@@ -38,9 +38,8 @@ int static_workspace(void **out) {
 
 inline bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// weight formats of the matmul-family entry points: those with matrix-core kernels (cq_has_mfma) and three more that take
-// the matvec kernels at any row count
-inline bool matmul_weight_dtype(int dt) { return cq_has_mfma(dt) || dt == CQ_Q4_1 || dt == CQ_Q5_0 || dt == CQ_Q5_1; }
+// weight formats of the matmul-family entry points: every one has matvec and matrix-core kernels
+inline bool matmul_weight_dtype(int dt) { return cq_has_mfma(dt); }
 
 inline bool block_dtype(int dt) { return matmul_weight_dtype(dt) || dt == CQ_Q8K; }
 // every GGUF block format can be stored and dequantized; the matmul-family and quantize entry points take fewer
@@ -53,7 +52,9 @@ inline int64_t float_size(int dt) { return dt == CQ_F32 ? 4 : 2; }
 // shared checks of the (w_dtype, k, n, rows) tuple of the matmul-family entry points
 // expert formats of the MoE entry points: the reference's (Q2K ... Q6K, Q8_0: candle-core/src/quantized/cuda.rs:543-548,
 // candle-nn/src/moe.rs:210-215) plus Q4_0
-inline bool moe_weight_dtype(int dt) { return cq_has_mfma(dt); }
+inline bool moe_weight_dtype(int dt) {
+    return dt == CQ_Q8_0 || dt == CQ_Q2K || dt == CQ_Q3K || dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q4_0;
+}
 
 inline int check_mm_shape(int w_dtype, int64_t k, int64_t n, int64_t rows) {
     if (!matmul_weight_dtype(w_dtype)) return CQ_ERR_DTYPE;

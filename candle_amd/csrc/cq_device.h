@@ -35,9 +35,10 @@ template <> struct BlockInfo<CQ_Q3K> { static constexpr int elems = 256, bytes =
 __host__ __device__ inline bool cq_is_kquant(int dt) {
     return dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q8K || dt == CQ_Q2K || dt == CQ_Q3K;
 }
-// formats with a matrix-core kernel (cq_matmul.hip); the others take the matvec kernels at any row count
+// formats with a matrix-core kernel (cq_matmul.hip): every QMatMul weight format
 __host__ __device__ constexpr bool cq_has_mfma(int dt) {
-    return dt == CQ_Q4_0 || dt == CQ_Q8_0 || dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q2K || dt == CQ_Q3K;
+    return dt == CQ_Q4_0 || dt == CQ_Q8_0 || dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q2K || dt == CQ_Q3K || dt == CQ_Q4_1 ||
+           dt == CQ_Q5_0 || dt == CQ_Q5_1;
 }
 // formats with every fused instance of the decode matvec (f16 / bf16 activations, decoder prologues and epilogues)
 __host__ __device__ constexpr bool cq_full_matvec(int dt) { return dt == CQ_Q4_0 || dt == CQ_Q8_0 || dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K; }

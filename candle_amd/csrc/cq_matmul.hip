@@ -18,9 +18,10 @@
 //   activation quantizers downstream, an exact one is not.
 // Q4_K — the same sums on the int8 matrix cores (qmm_q4k_i8_kernel, k_quants.rs:1460-1540): the 6-bit sub-block scale
 //   is split into two 3-bit halves so that scale * weight fits int8; S is exact in int32.
-// Q4_0 / Q8_0 — the per-32 sums of the CPU vec_dot (k_quants.rs:294-311, 720-738) on the int8 matrix cores
-//   (qmm_q0_i8_kernel): one v_mfma_i32_32x32x32_i8 per 32-element block gives the exact int32 sum of q8 * (q - 8)
-//   resp. q8 * q, and the vector units add  (float(S) * d[n, block]) * d8[m, block]  block by block, in the CPU's order.
+// Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 — the per-32 sums of the CPU vec_dot (k_quants.rs:294-311, 720-738, 323-351,
+//   434-455, 530-562) on the int8 matrix cores (qmm_q0_i8_kernel): one v_mfma_i32_32x32x32_i8 per 32-element block gives
+//   the exact int32 sum of q8 * q (q - 8, q - 16 for Q4_0, Q5_0), and the vector units add
+//   (float(S) * d[n, block]) * d8[m, block]  (+ m[n, block] * s[m, block] for Q4_1 / Q5_1)  block by block, in the CPU's order.
 //
 // Tiling: workgroup = 4 waves (2 x 2), block tile 128 (m) x 64 (n), wave tile 64 x 32 as 2 x 1 MFMA tiles of 32 x 32
 // (128 x 128 / 64 x 64 for large Q4_0 / Q8_0 problems, 32 x 128 with the waves side by side for up to 32 rows).
@@ -28,6 +29,7 @@
 // activation tile to f16 into one of two LDS copies (row stride padded to 144 bytes) while the MFMAs run on the other;
 // raw bytes are requested two stages ahead into two register sets.
 #include "cq_device.h"
+#include "cq_fmt.h"
 #include "cq_launch.h"
 
 namespace {
@@ -750,26 +752,36 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q4k_i8_kernel(const 
         }
 }
 
-// ---- Q4_0 / Q8_0 on the int8 matrix cores ----------------------------------------------------------------------------
+// ---- Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 on the int8 matrix cores --------------------------------------------------------
 // Same tiling and template parameters as above.  Both operands carry an f16 scale per 32 elements, so a 32 x 32 x 32 int8
 // MFMA is exactly one block: its int32 result S is the sum the CPU vec_dot forms for that block (k_quants.rs:294-311,
-// 720-738), and each lane folds its 16 results into the f32 accumulators as (float(S) * d[n]) * d8[m], block after block
-// in k order like the CPU loop.  That scaling is three vector instructions per result and bounds the kernel; the matrix
-// cores idle most of the time.  A stage is 128 elements of k (four blocks), held twice in LDS (one barrier per stage):
-// the int8 activations as in the Q4_K kernel, the four d8 per activation row, and the weight rows' four blocks as they
-// lie in memory (72 / 136 contiguous bytes per row), copied in 8-byte pieces by neighbouring lanes so that a load
-// instruction touches a handful of cache lines, not one per lane.  Lane (n, kg) of the B operand wants 16 consecutive k of
-// row n: the 16 quant bytes of the block (Q4_0: low nibbles for kg = 0, high nibbles for kg = 1) or one half of its 32
-// (Q8_0), read from LDS at the block's own 2-byte alignment.  Needs 8-byte aligned weights (row lengths are multiples of
-// 256 elements, so every row and stage then starts on 8 bytes).
-//   Q4_0: nibble q -> int8 (q - 8) on four bytes at once: (x + 0x78787878) ^ 0x80808080 (no carries: x < 16 per byte).
+// 720-738, 323-351, 434-455, 530-562), and each lane folds its 16 results into the f32 accumulators as
+// (float(S) * d[n]) * d8[m], plus m[n] * s[m] for the formats with a block minimum (s = the Q8_1 block sum, k_quants.rs:770-799),
+// block after block in k order like the CPU loop.  That scaling is three or four vector instructions per result and
+// bounds the kernel; the matrix cores idle most of the time.  A stage is 128 elements of k (four blocks), held twice in
+// LDS (one barrier per stage): the int8 activations as in the Q4_K kernel, the four d8 (and s) per activation row, and
+// the weight rows' four blocks as they lie in memory (72 .. 136 contiguous bytes per row), copied in 8-byte pieces by
+// neighbouring lanes so that a load instruction touches a handful of cache lines, not one per lane.  Lane (n, kg) of the
+// B operand wants 16 consecutive k of row n: the 16 quant bytes of the block (4- and 5-bit formats: low nibbles for
+// kg = 0, high nibbles for kg = 1, plus 16 bits of qh) or one half of its 32 (Q8_0), read from LDS at the block's own
+// 2-byte alignment.  Needs 8-byte aligned weights (row lengths are multiples of 256 elements, so every row and stage
+// then starts on 8 bytes).
+//   nibble q -> int8 (q - 8) on four bytes at once: (x + 0x78787878) ^ 0x80808080 (no carries: x < 16 per byte);
+//   5-bit q -> (q - 16): (x + 0x70707070) ^ 0x80808080.
+template <int DT> struct Q0Info;
+template <> struct Q0Info<CQ_Q4_0> { static constexpr int QS = 2, QH = -1, MIN = -1; static constexpr uint32_t BIAS = 0x78787878u; };
+template <> struct Q0Info<CQ_Q8_0> { static constexpr int QS = 2, QH = -1, MIN = -1; static constexpr uint32_t BIAS = 0; };
+template <> struct Q0Info<CQ_Q4_1> { static constexpr int QS = 4, QH = -1, MIN = 2; static constexpr uint32_t BIAS = 0; };
+template <> struct Q0Info<CQ_Q5_0> { static constexpr int QS = 6, QH = 2, MIN = -1; static constexpr uint32_t BIAS = 0x70707070u; };
+template <> struct Q0Info<CQ_Q5_1> { static constexpr int QS = 8, QH = 4, MIN = 2; static constexpr uint32_t BIAS = 0; };
 template <int DT, int NJ, bool SM = false>
 __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst,
                                                                            int k, int n, int rows, int64_t stride_dst, MoeChunks,
                                                                            int64_t, int64_t split_stride) {
-    static_assert(DT == CQ_Q4_0 || DT == CQ_Q8_0, "formats of one f16 scale per 32 weights");
+    typedef Q0Info<DT> QI;                                      // byte offsets of qs / qh / the block minimum (-1: none)
     static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
     constexpr int BB = BlockInfo<DT>::bytes;
+    constexpr bool HAS_MIN = QI::MIN >= 0;
     constexpr int BMT = SM ? 32 : BM, MI = SM ? 1 : 2;
     constexpr int BN = SM ? 128 : 64 * NJ, WN = 32 * NJ;
     constexpr int NA = BMT / 32;                                // 16-byte activation pieces a thread copies per stage
@@ -778,6 +790,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
     __shared__ __align__(16) int8_t As[2][BMT * 128];           // [row][8 pieces], piece p of row r at p ^ (r & 7)
     __shared__ __align__(16) uint8_t Bq[2][BN * RS];            // [row][four blocks]
     __shared__ __align__(16) float sD8[2][4][BMT];              // d8 of the stage's four blocks
+    __shared__ __align__(16) float sS8[2][HAS_MIN ? 4 : 1][HAS_MIN ? BMT : 4];   // their Q8_1 sums s = f16(f16(sum) * d8)
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = SM ? 0 : wv >> 1, wn = SM ? wv : wv & 1;
@@ -808,7 +821,7 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
         b_dst[i] = r * RS + 8 * c;
     }
     // MFMA operand roles: this lane's weight row of tile j, and where its 16 quant bytes sit inside a block
-    const int q_off = DT == CQ_Q8_0 ? 2 + 16 * kg : 2;
+    const int q_off = DT == CQ_Q8_0 ? QI::QS + 16 * kg : QI::QS;
 
     f32x16 acc[MI][NJ];
 #pragma unroll
@@ -838,6 +851,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
         // threads that share a row write the same values
         sD8[buf][2 * half][rs] = __uint_as_float(gds.x);
         sD8[buf][2 * half + 1][rs] = __uint_as_float(gds.z);
+        if constexpr (HAS_MIN) {
+            sS8[buf][2 * half][rs] = h2f(f2h_bits(h2f(f2h_bits((float)(int)gds.y)) * __uint_as_float(gds.x)));
+            sS8[buf][2 * half + 1][rs] = h2f(f2h_bits(h2f(f2h_bits((float)(int)gds.w)) * __uint_as_float(gds.z)));
+        }
     };
     load_stage(st0);
     store_stage(st0 & 1);
@@ -851,25 +868,34 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             i32x4 bop[NJ];
-            float dw[NJ];
+            float dw[NJ], mw[NJ];
 #pragma unroll
             for (int j = 0; j < NJ; j++) {
                 const uint8_t *blk = Bb + (wn * WN + j * 32 + (lane & 31)) * RS + b * BB;
                 const u32x4 q = ld_u<u32x4>(blk + q_off);
+                uint32_t qh = 0;
+                if constexpr (QI::QH >= 0) qh = ld_u<uint32_t>(blk + QI::QH) >> (16 * kg);     // bit i: fifth bit of this lane's element i
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    if constexpr (DT == CQ_Q4_0) bop[j][i] = (int)((((q[i] >> (4 * kg)) & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u);
-                    else bop[j][i] = (int)q[i];
+                    uint32_t v = q[i];
+                    if constexpr (DT != CQ_Q8_0) v = (v >> (4 * kg)) & 0x0f0f0f0fu;
+                    if constexpr (QI::QH >= 0) v |= spread4_to_bit4(qh >> (4 * i));
+                    if constexpr (QI::BIAS != 0) v = (v + QI::BIAS) ^ 0x80808080u;
+                    bop[j][i] = (int)v;
                 }
                 dw[j] = h2f(ld_u<uint16_t>(blk));
+                mw[j] = HAS_MIN ? h2f(ld_u<uint16_t>(blk + (HAS_MIN ? QI::MIN : 0))) : 0.0f;
             }
 #pragma unroll
             for (int i = 0; i < MI; i++) {
                 const int rl = wm * 64 + i * 32;
                 const i32x4 af = *reinterpret_cast<const i32x4 *>(Ab + (rl + (lane & 31)) * 128 + 16 * ((2 * b + kg) ^ swz_a));
-                f32x4 d8[4];
+                f32x4 d8[4], s8[4];
 #pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) d8[q4] = *reinterpret_cast<const f32x4 *>(&sD8[buf][b][rl + 8 * q4 + 4 * kg]);
+                for (int q4 = 0; q4 < 4; q4++) {
+                    d8[q4] = *reinterpret_cast<const f32x4 *>(&sD8[buf][b][rl + 8 * q4 + 4 * kg]);
+                    if constexpr (HAS_MIN) s8[q4] = *reinterpret_cast<const f32x4 *>(&sS8[buf][b][rl + 8 * q4 + 4 * kg]);
+                }
 #pragma unroll
                 for (int j = 0; j < NJ; j++) {
                     i32x16 z;
@@ -877,7 +903,11 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
                     for (int e = 0; e < 16; e++) z[e] = 0;
                     const i32x16 sI = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bop[j], z, 0, 0, 0);
 #pragma unroll
-                    for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf((float)sI[e] * dw[j], d8[e >> 2][e & 3], acc[i][j][e]);
+                    for (int e = 0; e < 16; e++) {
+                        float t = fmaf((float)sI[e] * dw[j], d8[e >> 2][e & 3], acc[i][j][e]);
+                        if constexpr (HAS_MIN) t = fmaf(mw[j], s8[e >> 2][e & 3], t);
+                        acc[i][j][e] = t;
+                    }
                 }
             }
         }
@@ -914,12 +944,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 }
 
 typedef void (*QmmFn)(const uint8_t *, ActView, float *, int, int, int, int64_t, MoeChunks, int64_t, int64_t);
-// the kernel of a format and tile shape: Q4_K, Q4_0 and Q8_0 run on the int8 matrix cores, the other formats on the f16 ones
+// the kernel of a format and tile shape: Q4_K and the 32-element formats run on the int8 matrix cores, the others on the f16 ones
 template <int DT, int NJ, bool MOE, bool SM>
 QmmFn qmm_fn() {
     if constexpr (DT == CQ_Q4K) return qmm_q4k_i8_kernel<NJ, MOE, SM>;
-    else if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0) {
-        static_assert(!MOE, "expert-grouped Q4_0 / Q8_0 rows take the matvec kernels");
+    else if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0 || DT == CQ_Q4_1 || DT == CQ_Q5_0 || DT == CQ_Q5_1) {
+        static_assert(!MOE, "expert-grouped rows of the 32-element formats take the matvec kernels");
         return qmm_q0_i8_kernel<DT, NJ, SM>;
     } else return qmm_kernel<DT, NJ, MOE, SM>;
 }
@@ -1049,12 +1079,16 @@ bool cq_use_mfma(int w_dtype, int64_t rows, int64_t k) {
 int cq_matmul_launch(int w_dtype, const void *w, const void *scratch, float *dst, int64_t k, int64_t n, int64_t rows,
                      int64_t stride_dst, hipStream_t s, float *split_ws) {
     ActView av = cq_act_view(scratch, w_dtype, k, rows);
-    // the Q4_0 / Q8_0 matrix-core kernel copies weight rows in 8-byte pieces; weights at another alignment take the loop below
-    const bool q0_unaligned = (w_dtype == CQ_Q4_0 || w_dtype == CQ_Q8_0) && ((uintptr_t)w & 7) != 0;
+    // the matrix-core kernel of the 32-element formats copies weight rows in 8-byte pieces; weights at another alignment
+    // take the loop below
+    const bool q0_unaligned = !cq_is_kquant(w_dtype) && ((uintptr_t)w & 7) != 0;
     if (cq_use_mfma(w_dtype, rows, k) && !q0_unaligned) {
         switch (w_dtype) {
             case CQ_Q4_0: return launch_qmm<CQ_Q4_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q8_0: return launch_qmm<CQ_Q8_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q4_1: return launch_qmm<CQ_Q4_1>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q5_0: return launch_qmm<CQ_Q5_0>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
+            case CQ_Q5_1: return launch_qmm<CQ_Q5_1>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q4K: return launch_qmm<CQ_Q4K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q5K: return launch_qmm<CQ_Q5K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);
             case CQ_Q6K: return launch_qmm<CQ_Q6K>(w, av, dst, k, n, rows, stride_dst, s, split_ws);

@@ -64,7 +64,7 @@ _BLOCK_SIZE = {d: (1 if d in (GgmlDType.F32, GgmlDType.F16, GgmlDType.BF16) else
 # every block format can be stored, quantized, dequantized and used as an embedding table
 _KERNEL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K, GgmlDType.Q8K)
 _DEQUANT_DTYPES = _KERNEL_DTYPES + (GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q8_1, GgmlDType.Q2K, GgmlDType.Q3K)
-# QMatMul weights: the first five also have matrix-core (prefill) kernels, the others take the matvec kernels at any row count
+# QMatMul weights: each has a matvec kernel (up to 8 activation rows) and a matrix-core (prefill) kernel
 _MATMUL_DTYPES = (GgmlDType.Q4_0, GgmlDType.Q8_0, GgmlDType.Q4K, GgmlDType.Q5K, GgmlDType.Q6K,
                   GgmlDType.Q4_1, GgmlDType.Q5_0, GgmlDType.Q5_1, GgmlDType.Q2K, GgmlDType.Q3K)
 # expert formats of the two MoE entry points: the reference's (cuda.rs:543-548 + moe.rs:210-215) plus Q4_0

@@ -20,9 +20,9 @@
  *   - activation quantization follows candle's CPU path bit for bit (Q8_K blocks for K-quants,
  *     Q8_0 blocks for Q4_0/Q5_0/Q8_0, Q8_1 blocks for Q4_1/Q5_1: k_quants.rs:2320-2358, 658-687, 770-799), so
  *     results match QMatMul::forward on the CPU up to f32 summation order;
- *   - weight formats of the matmul-family entry points (cq_quantize_act, cq_matvec, cq_matmul, cq_qmatmul_forward;
- *     the MoE entry points take the first seven): Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K, which also have matrix-core kernels, and Q4_1, Q5_0,
- *     Q5_1, which take the matvec kernels at any row count (eight activation rows per pass over the weights).
+ *   - weight formats of the matmul-family entry points (cq_quantize_act, cq_matvec, cq_matmul, cq_qmatmul_forward): Q4_0, Q4_1,
+ *     Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K, each with a matvec kernel (up to eight activation rows) and a matrix-core
+ *     kernel; the MoE entry points take Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K.
  */
 #ifndef CANDLE_HIP_QUANT_H
 #define CANDLE_HIP_QUANT_H

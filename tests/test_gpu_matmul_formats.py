@@ -1,8 +1,8 @@
 """GPU parity of QMatMul::forward for Q4_1, Q5_0, Q5_1, Q2_K, Q3_K weights against the CPU oracle: candle's CPU path
 quantizes their activations to Q8_1 / Q8_0 / Q8_1 / Q8_K / Q8_K (k_quants.rs:317,418,524,822,1055).  The GPU quantizes to
-the same int8 values and every kernel sums the same integers (matvec kernels; for Q2_K / Q3_K beyond 8 rows the f16 matrix
-cores with exact small-integer operands), so the bar is the same as for the other K-quants: relative L2 <= 1e-3 by
-contract, <= 2e-6 observed (f32 summation order only).
+the same int8 values and every kernel sums the same integers (matvec kernels; beyond 8 rows the f16 matrix cores with
+exact small-integer operands for Q2_K / Q3_K and one int8 MFMA per block for Q4_1 / Q5_0 / Q5_1), so the bar is the same
+as for the other K-quants: relative L2 <= 1e-3 by contract, <= 2e-6 observed (f32 summation order only).
 """
 import numpy as np
 import pytest
@@ -78,7 +78,7 @@ def test_k_not_multiple_of_256(dtype):
 @pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("m", [9, 16, 33, 128])
 def test_more_than_eight_rows(dtype, m):
-    # Q2_K / Q3_K: matrix cores; Q4_1 / Q5_0 / Q5_1: eight activation rows per pass over the weights
+    # Q2_K / Q3_K: f16 matrix cores; Q4_1 / Q5_0 / Q5_1: int8 matrix cores when k is a multiple of 256
     n, k = 96, 1024
     blocks, qmm = make_weight(dtype, n, k, seed=61 + dtype)
     x = normal(62 + m, (m, k), 1.0)
@@ -147,3 +147,33 @@ def test_prefill_random_blocks(dtype):
     qt = ca.QTensor.new(ca.QStorage.from_data(blocks, "cuda", ca.GgmlDType(dtype)), (n, k))
     x = normal(91, (m, k), 1.0)
     assert rel_l2(forward(ca.QMatMul.from_qtensor(qt), x), oracle.matmul(dtype, x, blocks, n)) <= TIGHT
+
+
+@pytest.mark.parametrize("dtype", [oracle.Q4_1, oracle.Q5_0, oracle.Q5_1], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 256), (130, 200, 512), (257, 129, 2048), (64, 384, 4096), (20, 260, 1024), (512, 96, 8192)])
+def test_int8_matrix_core_tiles_ragged(dtype, m, n, k):
+    """Tile edges of the int8 matrix-core kernel: rows and columns that do not fill the block tile, the 32-row tile (20 rows),
+    one and many stages, split-K; every row on its own as well."""
+    blocks, qmm = make_weight(dtype, n, k, seed=261 + dtype)
+    x = normal(262 + m, (m, k), 1.0)
+    got = forward(qmm, x)
+    want = oracle.matmul(dtype, x, blocks, n)
+    assert rel_l2(got, want) <= TIGHT
+    assert max(rel_l2(got[r], want[r]) for r in range(m)) <= 4 * TIGHT
+
+
+@pytest.mark.parametrize("dtype,n,k", [(oracle.Q4_1, 14336, 4096), (oracle.Q5_0, 4096, 14336), (oracle.Q5_1, 14336, 4096)], ids=lambda v: NAMES.get(v, str(v)))
+@pytest.mark.parametrize("m", [128, 512])
+def test_int8_matrix_core_full_size(dtype, n, k, m):
+    """The FFN shapes at prefill row counts: three weight rows x all activation rows and the last activation row x 64 weight
+    rows against the scalar oracle."""
+    import candle_amd as ca
+    w = torch.from_numpy(normal(281, (n, k), 0.02)).cuda()
+    qt = ca.QTensor.quantize(w, ca.GgmlDType(dtype))
+    x = normal(282 + m, (m, k), 1.0)
+    got = forward(ca.QMatMul.from_qtensor(qt), x)
+    blocks = np.frombuffer(qt.data(), dtype=np.uint8)
+    rb = (k // 32) * oracle.type_size(dtype)
+    for rows, xs in (([0, n // 2 + 1, n - 1], slice(0, m)), (list(range(0, n, n // 64)), slice(m - 1, m))):
+        sub = np.concatenate([blocks[r * rb:(r + 1) * rb] for r in rows])
+        assert rel_l2(got[xs][:, rows], oracle.matmul(dtype, x[xs], sub, len(rows))) <= TIGHT
