@@ -623,6 +623,7 @@ __global__ __launch_bounds__(1024) void qmv2_kernel(const uint8_t *__restrict__ 
 // (s / grid) % QS_NW of workgroup s % grid, so at any moment the whole chip reads one compact window of the tensor.
 // ---------------------------------------------------------------------------------------------
 constexpr int QS_NW = 8;
+constexpr bool qs_streams(int dt) { return dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K; }     // formats with a StreamFmt
 
 template <int DT, int NW, int XS, int MAXB, int PRO, int EPI, int MSP = MAXS>
 __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const float *__restrict__ x, void *__restrict__ dst, const StreamGeom &g,
@@ -635,6 +636,8 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     // 16-byte-per-lane copies of the first step requested before the activation prologue; the rest follows it.
     // Requests beyond what the memory pipeline takes at once block the wave's instruction stream, and the prologue
     // queued behind them would wait for the weights instead of running under their latency.
+    // (measured on the Q6_K 4096 x 14336 matvec, 14 copies per step and seven spans per wave: 4 copies first 14.8 us,
+    // all 14 first 16.2 us, the rest spread behind the spans 15.2 us)
     constexpr int PRE = NW == 16 ? 2 : 4;
     constexpr int ME = EPI == EPI_RESID_SPLIT ? MAXP : 1;
     constexpr int SLOT = SF::NLD * 1024;
@@ -745,7 +748,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         if (PRO == PRO_NORM || PRO == PRO_SILU) pro_apply<PRO>(xv[j], a4, pm);
         if (PRO == PRO_NORM_SPLIT) pro_apply<PRO_NORM>(xv[j], a4, pm);
         const int span = wv + j * NW;
-        qs_quantize_span(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
+        qs_quantize_span<DT == CQ_Q6K>(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
     }
     asm volatile("" ::: "memory");
     issue(0, PRE, SF::NLD);
@@ -760,7 +763,14 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     u32x4 areg[16];
 #pragma unroll
     for (int i = 0; i < 16; i++) areg[i] = *(const u32x4 *)(act + sbc * QS_ACT_STRIDE + 16 * i);
-    const u32x4 aux0 = *(const u32x4 *)(act + SA::AUX_OFF + sbc * QS_AUX_STRIDE), aux1 = *(const u32x4 *)(act + SA::AUX_OFF + sbc * QS_AUX_STRIDE + 16);
+    const uint8_t *auxp = act + SA::AUX_OFF + sbc * QS_AUX_STRIDE;
+    const u32x4 aux0 = *(const u32x4 *)auxp;
+    QsAux aux1;
+    aux1.s32 = *(const u32x4 *)(auxp + 16);
+    if constexpr (DT == CQ_Q6K) {
+        aux1.bl16 = *(const u32x4 *)(auxp + 32);
+        aux1.bh16 = *(const u32x4 *)(auxp + 48);
+    }
     const float d8 = __uint_as_float(aux0.x);
     const int boff = (rin * bpr + sbc) * SF::BB;
     const bool last = sb == lp - 1;                     // this lane ends up with the row's sum
@@ -968,7 +978,7 @@ __global__ __launch_bounds__(NW * 64) void qms2_kernel(Qs2Args a) {
 // lane; other row lengths put one row on a wave step and need at least three quarters of the lanes busy.
 template <int DT>
 bool stream_geom(StreamGeom &g, int64_t k, int64_t n, int dst_dtype) {
-    if (DT != CQ_Q4K && DT != CQ_Q5K) return false;
+    if (!qs_streams(DT)) return false;
     if (k % 256 || k <= 0 || n < 64) return false;
     const int64_t bpr = k / 256;
     if (bpr > 64) return false;
@@ -976,6 +986,8 @@ bool stream_geom(StreamGeom &g, int64_t k, int64_t n, int dst_dtype) {
     while ((1 << sh) < bpr) sh++;
     if ((1 << sh) != bpr && 4 * bpr < 3 * (1 << sh)) return false;
     const int64_t bb = BlockInfo<DT>::bytes;
+    // every wave step must start on 16 bytes of the stream (Q6_K blocks are 210 bytes: steps of a multiple of 8 blocks)
+    if (((64 >> sh) * bpr * bb) % 16) return false;
     g.k = (int)k; g.n = (int)n; g.bpr = (int)bpr; g.lp_shift = sh;
     g.step_rows = 64 >> sh;
     g.step_bytes = (int)(g.step_rows * bpr * bb);
@@ -1011,7 +1023,7 @@ int launch_stream_merge(const void *w, void *dst, const StreamGeom &g, hipStream
 // CQ_ERR_RANGE: not a shape (or fusion) of the streaming kernel; the caller takes qmv_kernel
 template <int DT, int PRO, int EPI>
 int launch_stream(const void *w, const float *x, void *dst, int dst_dtype, int64_t k, int64_t n, hipStream_t s, const Fuse &fz) {
-    if constexpr (DT != CQ_Q4K && DT != CQ_Q5K) {
+    if constexpr (!qs_streams(DT)) {
         return CQ_ERR_RANGE;
     } else {
         StreamGeom g;
@@ -1196,11 +1208,12 @@ int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtyp
                            int64_t rows, int64_t stride_dst, hipStream_t s) {
     if (n == 0 || rows == 0) return CQ_OK;
     if (rows == 1 && x_dtype == CQ_F32) {
-        // one f32 row over Q4_K / Q5_K weights: the streaming kernel where it takes the shape
+        // one f32 row over Q4_K / Q5_K / Q6_K weights: the streaming kernel where it takes the shape
         const Fuse none{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
         int rc = CQ_ERR_RANGE;
         if (w_dtype == CQ_Q4K) rc = launch_stream<CQ_Q4K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
         if (w_dtype == CQ_Q5K) rc = launch_stream<CQ_Q5K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
+        if (w_dtype == CQ_Q6K) rc = launch_stream<CQ_Q6K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
         if (rc != CQ_ERR_RANGE) return rc;
     }
     const int64_t xsz = x_dtype == CQ_F32 ? 4 : 2, esz = dst_dtype == CQ_F32 ? 4 : 2;
@@ -1353,7 +1366,10 @@ int launch_pair_stream_xs(const void *wa, float *dsta, const void *wb, int64_t n
         const int rc = make_geom<DTB, 1>(gb, groups_b, waves, k, nb, nb, CQ_F32, XL, lds_b, 256 - share_a);
         if (rc) return rc;
     }
-    const size_t lds_a = (size_t)NW * StreamFmt<DTA>::NLD * 1024;
+    size_t lds_a = (size_t)NW * StreamFmt<DTA>::NLD * 1024;
+    if constexpr (qs_streams(DTB)) {
+        if (sb && (size_t)NW * StreamFmt<DTB>::NLD * 1024 > lds_a) lds_a = (size_t)NW * StreamFmt<DTB>::NLD * 1024;
+    }
     const size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
     if (lds_bytes + StreamAct<MAXB>::BYTES + 256 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
     const bool single = k / 64 <= 64;
@@ -1380,7 +1396,7 @@ int launch_pair_stream_xs(const void *wa, float *dsta, const void *wb, int64_t n
         hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, a);
         return (int)hipGetLastError();
     };
-    if constexpr (DTB == DTA) {
+    if constexpr (qs_streams(DTB)) {
         if (sb) return go(qms2_kernel<DTA, DTB, NW, XS, MAXB, true, PRO, true>);
     }
     if (single) return go(qms2_kernel<DTA, DTB, NW, XS, MAXB, true, PRO, false>);
@@ -1396,7 +1412,7 @@ int launch_pair_stream(const void *wa, int64_t na, float *dsta, const void *wb, 
     if (bpr > 16) return CQ_ERR_RANGE;            // longer rows: the two-tensor launch of qmv_kernel
     StreamGeom gsb = ga;
     bool sb = false;
-    if constexpr (DTB == DTA) sb = stream_geom<DTB>(gsb, k, nb, CQ_F32);
+    if constexpr (qs_streams(DTB)) sb = stream_geom<DTB>(gsb, k, nb, CQ_F32);
     if (pro_is_split(PRO) && !sb) {
         // qmv_body merges the planes with one activation span per wave: sixteen waves (and one span per wave here too)
         if (StreamFmt<DTA>::NLD * 16 * 1024 + StreamAct<16>::BYTES + 256 > LDS_BUDGET) return CQ_ERR_RANGE;
@@ -1410,7 +1426,7 @@ template <int DTA, int DTB, int PRO>
 int launch_pair(const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const ActSrc &src, int64_t k, hipStream_t s,
                 const Fuse &fz_in) {
     constexpr int XL = pro_is_split(PRO) ? 64 : 0;
-    if constexpr (DTA == CQ_Q4K || DTA == CQ_Q5K || DTB == CQ_Q4K || DTB == CQ_Q5K) {
+    if constexpr (qs_streams(DTA) || qs_streams(DTB)) {
         // rows the streaming kernel takes but its two-tensor launch does not (more than 4096 elements): two launches,
         // each on the kernel a single call would get
         StreamGeom gt;
@@ -1420,12 +1436,12 @@ int launch_pair(const void *wa, int64_t na, float *dsta, const void *wb, int64_t
             return rc ? rc : launch_fused1<DTB, PRO, EPI_NONE>(wb, src, dstb, k, nb, s, fz_in);
         }
     }
-    if constexpr (DTA != CQ_Q4K && DTA != CQ_Q5K && (DTB == CQ_Q4K || DTB == CQ_Q5K)) {
+    if constexpr (!qs_streams(DTA) && qs_streams(DTB)) {
         // only tensor B has a streaming body: the same launch with the tensors exchanged
         StreamGeom gt;
         if (stream_geom<DTB>(gt, k, nb, CQ_F32) && gt.bpr <= 16) return launch_pair<DTB, DTA, PRO>(wb, nb, dstb, wa, na, dsta, src, k, s, fz_in);
     }
-    if constexpr (DTA == CQ_Q4K || DTA == CQ_Q5K) {
+    if constexpr (qs_streams(DTA)) {
         int rc = launch_pair_stream<DTA, DTB, PRO>(wa, na, dsta, wb, nb, dstb, (const float *)src.x, k, s, fz_in);
         if (rc != CQ_ERR_RANGE) return rc;
         // the two-tensor launch does not take this call (the tensors or their outputs lie further apart than its 32-bit

@@ -1,4 +1,4 @@
-// Streaming decode matvec for Q4_K / Q5_K weights and one f32 activation row:  dst[row] = sum_k W[row, k] * x^[k].
+// Streaming decode matvec for Q4_K / Q5_K / Q6_K weights and one f32 activation row:  dst[row] = sum_k W[row, k] * x^[k].
 //
 // The weights of a tensor are one contiguous stream of super-blocks (rows follow each other without gaps).  A wave
 // step is a run of that stream — 64 super-blocks when a row has a power of two of them, else one row — copied
@@ -16,7 +16,7 @@
 //
 // Same arithmetic contract as qmv_kernel: activations quantized to Q8_K exactly like BlockQ8K::from_float
 // (candle-core/src/quantized/k_quants.rs:2320-2358), integer dots exact, one f32 scaling per super-block
-// (vec_dot Q4_K x Q8_K k_quants.rs:1460-1540, Q5_K :1714-1801); only the f32 summation order differs.
+// (vec_dot Q4_K x Q8_K k_quants.rs:1460-1540, Q5_K :1714-1801, Q6_K :2035-2092); only the f32 summation order differs.
 #pragma once
 #include "cq_actquant.h"
 #include "cq_device.h"
@@ -26,15 +26,19 @@ namespace {
 typedef __attribute__((address_space(3))) void cq_lds_void;
 
 // Quantized activations in LDS: per 256-element span 272 bytes of int8 (256 + 16: the sixteen lanes of a row read
-// sixteen different spans at once, a stride of 256 bytes would put them all on the same banks) and a 32-byte record
-//   f32 d | 12 bytes unused | u8 bl[8] | i8 bh[8]      with  sum of sub-block j = 128 * bh[j] + bl[j],  0 <= bl[j] < 128
-// (the sums of the eight 32-element sub-blocks split into two int8 halves, so that sum_j min_j * sum_j is two dot4).
+// sixteen different spans at once, a stride of 256 bytes would put them all on the same banks) and a 64-byte record
+//   f32 d | 12 bytes unused | u8 bl[8] | i8 bh[8] | u8 bl16[16] | i8 bh16[16]
+// with  sum of 32-element sub-block j = 128 * bh[j] + bl[j]  and  sum of 16-element group g = 128 * bh16[g] + bl16[g],
+// 0 <= bl < 128 (the sums split into two int8 halves, so that sum_j coefficient_j * sum_j is a few dot4).  The 16-element
+// sums are written for Q6_K only, whose scales cover 16 elements.
 constexpr int QS_ACT_STRIDE = 272;
-constexpr int QS_AUX_STRIDE = 32;
+constexpr int QS_AUX_STRIDE = 64;
 template <int MAXB> struct StreamAct {
     static constexpr int AUX_OFF = (MAXB + 1) * QS_ACT_STRIDE;                     // one more span: the dump for waves without a span
     static constexpr int BYTES = AUX_OFF + (MAXB + 1) * QS_AUX_STRIDE;
 };
+// what a lane keeps of its span's record besides d
+struct QsAux { u32x4 s32, bl16, bh16; };
 
 __device__ __forceinline__ uint32_t qs_wave_umax(uint32_t v) {
     // unsigned max through DPP (fused into v_max_u32_dpp); non-negative floats order like their bit patterns
@@ -49,6 +53,7 @@ __device__ __forceinline__ uint32_t qs_wave_umax(uint32_t v) {
 // BlockQ8K::from_float takes the FIRST element of largest magnitude for the scale; here any element of that
 // magnitude is taken: with another sign d and every q flip together and every product d * q is the same value, so
 // no result of the matvec depends on it.  NaN / Inf inputs follow the CPU arithmetic (round, saturating cast, NaN -> 0).
+template <bool SUM16 = false>
 __device__ __forceinline__ void qs_quantize_span(const float v[4], int span, int lane, uint8_t *act, int aux_off) {
     float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
     amax = amax == amax ? amax : 0.0f;                // four NaNs: the CPU's `amax < |x|` never takes a NaN either
@@ -67,8 +72,15 @@ __device__ __forceinline__ void qs_quantize_span(const float v[4], int span, int
     }
     *(uint32_t *)(act + span * QS_ACT_STRIDE + lane * 4) = packed;
     int s = sdot4(packed, 0x01010101u, 0);
-    s = oct_sum(s);                                   // sum of the 32-element sub-block, in all eight lanes
     uint8_t *aux = act + aux_off + span * QS_AUX_STRIDE;
+    if (SUM16) {
+        const int s16 = quad_sum(s);                  // sum of the 16-element group, in all four lanes
+        if ((lane & 3) == 0) {
+            aux[32 + (lane >> 2)] = (uint8_t)(s16 & 127);
+            aux[48 + (lane >> 2)] = (uint8_t)(s16 >> 7);
+        }
+    }
+    s = oct_sum(s);                                   // sum of the 32-element sub-block, in all eight lanes
     if ((lane & 7) == 0) {
         aux[16 + (lane >> 3)] = (uint8_t)(s & 127);
         aux[24 + (lane >> 3)] = (uint8_t)(s >> 7);    // arithmetic shift: 128 * bh + bl == s for negative sums too
@@ -120,8 +132,9 @@ template <> struct StreamFmt<CQ_Q4K> {
 #pragma unroll
         for (int i = 0; i < 8; i++) b.q[i] = *(const u32x4 *)(p + 16 + 16 * i);
     }
-    // a[16]: the lane's 256 int8 activations; aux0.x = d8, aux1 = sub-block sums
-    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float d8, const u32x4 aux1) {
+    // a[16]: the lane's 256 int8 activations; d8 and aux: the span's record
+    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float d8, const QsAux &aux) {
+        const u32x4 aux1 = aux.s32;
         int D[8];
 #pragma unroll
         for (int g = 0; g < 4; g++) qs_dot_pair_q4(b.q[2 * g], b.q[2 * g + 1], a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3], D[2 * g], D[2 * g + 1]);
@@ -150,7 +163,8 @@ template <> struct StreamFmt<CQ_Q5K> {
 #pragma unroll
         for (int i = 0; i < 8; i++) b.q[i] = *(const u32x4 *)(p + 48 + 16 * i);
     }
-    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float d8, const u32x4 aux1) {
+    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float d8, const QsAux &aux) {
+        const u32x4 aux1 = aux.s32;
         const uint32_t M4 = 0x0f0f0f0fu;
         const uint32_t h[8] = {b.h[0].x, b.h[0].y, b.h[0].z, b.h[0].w, b.h[1].x, b.h[1].y, b.h[1].z, b.h[1].w};
         int D[8];
@@ -178,6 +192,63 @@ template <> struct StreamFmt<CQ_Q5K> {
         }
         const int M = qs_dot_sums(s.mA, s.mB, aux1);
         return d8 * (h2f(b.hdr.x) * (float)S - h2f(b.hdr.x >> 16) * (float)M);
+    }
+};
+
+// Q6_K (210 bytes: ql[128] | qh[64] | int8 scales[16] | f16 d): super-blocks lie at 2-byte alignment in the stream, so a
+// lane's block is read from LDS with unaligned 16-byte reads.  Element layout (k_quants.rs:2265-2274): for half h and
+// l in [0, 32), byte ql[64h + l] holds elements 128h + l (low nibble) and 128h + 64 + l (high), byte ql[64h + 32 + l]
+// elements 128h + 32 + l and 128h + 96 + l; qh[32h + l] carries bits 4-5 of those four in its four bit pairs; scale
+// 8h + l / 16 + 2t belongs to the t-th of them.  Values are taken as unsigned 6-bit numbers; their offset of 32 goes
+// through the 16-element activation sums:  sum_g sc_g * (dot_g - 32 * sum16_g).
+template <> struct StreamFmt<CQ_Q6K> {
+    static constexpr int BB = 210;
+    static constexpr int NLD = 14;             // 64 x 210 = 13440 bytes
+    struct Blk { u32x4 ql[8]; u32x4 qh[4]; u32x4 sc; uint32_t d; };
+    static __device__ __forceinline__ void read(Blk &b, const uint8_t *p) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) b.ql[i] = ld_u<u32x4>(p + 16 * i);
+#pragma unroll
+        for (int i = 0; i < 4; i++) b.qh[i] = ld_u<u32x4>(p + 128 + 16 * i);
+        b.sc = ld_u<u32x4>(p + 192);
+        b.d = ld_u<uint16_t>(p + 208);
+    }
+    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float d8, const QsAux &aux) {
+        const uint32_t M4 = 0x0f0f0f0fu, M2 = 0x30303030u;
+        const uint32_t scw[4] = {b.sc.x, b.sc.y, b.sc.z, b.sc.w};
+        int S = 0;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+#pragma unroll
+            for (int is = 0; is < 2; is++) {
+                int g0 = 0, g1 = 0, g2 = 0, g3 = 0;                 // groups 8h + is + {0, 2, 4, 6}
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int j = 4 * is + jj;                      // dword of the 32 `l` positions
+                    const uint32_t qa = b.ql[4 * h + (j >> 2)][j & 3], qb = b.ql[4 * h + 2 + (j >> 2)][j & 3];
+                    const uint32_t hh = b.qh[2 * h + (j >> 2)][j & 3];
+                    g0 = sdot4((qa & M4) | ((hh << 4) & M2), a[8 * h + is][jj], g0);
+                    g1 = sdot4((qb & M4) | ((hh << 2) & M2), a[8 * h + 2 + is][jj], g1);
+                    g2 = sdot4(((qa >> 4) & M4) | (hh & M2), a[8 * h + 4 + is][jj], g2);
+                    g3 = sdot4(((qb >> 4) & M4) | ((hh >> 2) & M2), a[8 * h + 6 + is][jj], g3);
+                }
+                // scale bytes 8h + is + 2t: byte (is + 2t) % 4 of dword 2h + (is + 2t) / 4
+                const uint32_t w0 = scw[2 * h], w1 = scw[2 * h + 1];
+                S += __mul24((int)(int8_t)(w0 >> (8 * is)), g0);
+                S += __mul24((int)(int8_t)(w0 >> (8 * (is + 2))), g1);
+                S += __mul24((int)(int8_t)(w1 >> (8 * is)), g2);
+                S += __mul24((int)(int8_t)(w1 >> (8 * (is + 2))), g3);
+            }
+        }
+        // sum_g sc_g * sum16_g with sum16 = 128 * bh16 + bl16 (scales are signed bytes, the halves small enough for int8)
+        int C = 0, Ch = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            C = sdot4(scw[i], aux.bl16[i], C);
+            Ch = sdot4(scw[i], aux.bh16[i], Ch);
+        }
+        S -= ((Ch << 7) + C) << 5;
+        return (h2f(b.d) * d8) * (float)S;
     }
 };
 

@@ -106,7 +106,8 @@ class ModelWeights:
         self._graph = None
         self._graph_key = None
         self.fuse_decode = True            # single-token steps use the fused matvec prologues / epilogues
-        self.split_w2 = True               # ... and feed_forward_w2 as a K-split matvec where the shapes allow it
+        self.split_w2 = False              # ... and feed_forward_w2 as a K-split matvec (planes merged by its consumers) where the shapes allow it;
+                                           # off: with every format of a Q4_K_M file on the streaming kernel the unsplit step is as fast (8B shape: 608 vs 603 tok/s)
         self.merge_in_wo = False           # merge the attention key splits in the prologue of attention_wo (else: in the attention kernel)
         # bytes of the weights behind attention (wo, w1, w3, w2 are contiguous) that the attention launch's idle CUs
         # would pull through the memory-side cache ahead of the kernels that stream them.  Measured on the 8B shape:
