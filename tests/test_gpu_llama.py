@@ -221,6 +221,7 @@ def test_decode_with_split_feed_forward_w2(dtypes):
     # can round the other way and move a whole block by 1e-3, so the Q4_0 / Q8_0 model is compared on a seed where
     # none does; the split-against-unsplit comparison below does not depend on that)
     cfg, t, model = make(DEEP_FFN, dtypes, seed=44)
+    model.split_w2 = True                 # off by default
     assert model.L.cq_nn_qmatmul_split_planes(int(dtypes["feed_forward_w2"]), cfg.ffn) == 2
     ref = lo.LlamaOracle(cfg, t, threads=8)
     prompt = [7, 141, 59, 26, 5]
