@@ -812,16 +812,23 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const float *__res
     __syncthreads();
     if (!s_last) return;
     auto ld = [](const float *q) { return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    static_assert(HD % 64 == 0 && ATTD_MAX_SPLITS <= 16, "a wave stays inside one query head; lanes 0..31 fetch the (m, l) pairs");
     for (int i = tid; i < G * HD; i += 64 * NW) {
-        const int g = i / HD, d = i - g * HD;
+        const int g = i / HD, d = i - g * HD;                 // g is the same in all lanes of a wave
         const float *pp = part + (int64_t)(kvh * G + g) * splits * (HD + 4);
-        // every load first (these bypass the caches: one after the other they would be a trip to memory each); a split
-        // that does not exist re-reads the last one and is left out of the sums
-        float mv[ATTD_MAX_SPLITS], lv[ATTD_MAX_SPLITS], av[ATTD_MAX_SPLITS];
+        // Every load first (these bypass the caches: one after the other they would be a trip to memory each), and as few
+        // load instructions as possible, they are what the last workgroup's time goes into: one instruction fetches
+        // the (m, l) of all splits of the head (lane s: m of split s, lane 16 + s: l), one per existing split the
+        // accumulators.  A split that does not exist re-reads the last one and is left out of the sums.
+        const float mlv = ld(pp + min(lane & 15, splits - 1) * (HD + 4) + HD + ((lane >> 4) & 1));
+        float av[ATTD_MAX_SPLITS];
+#pragma unroll
+        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++) av[sI] = sI < splits ? ld(pp + sI * (HD + 4) + d) : 0.0f;
+        float mv[ATTD_MAX_SPLITS], lv[ATTD_MAX_SPLITS];
 #pragma unroll
         for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++) {
-            const float *rec = pp + min(sI, splits - 1) * (HD + 4);
-            mv[sI] = ld(rec + HD); lv[sI] = ld(rec + HD + 1); av[sI] = ld(rec + d);
+            mv[sI] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mlv), sI));
+            lv[sI] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mlv), 16 + sI));
         }
         float M = -INFINITY;
 #pragma unroll
