@@ -921,6 +921,104 @@ __global__ __launch_bounds__(QS_NW * 64) void qms_kernel(QsArgs<PRO, EPI> a) {
     qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
 }
 
+// ---- two activation rows on the streaming kernel -------------------------------------------------------------
+// QMatMul::forward for two f32 rows (no prologue, no epilogue): the same stream of weight steps as qms_body; a lane keeps
+// the 256 activations of its super-block for both rows and takes two dots from every block it reads.  The weights are
+// read once, as for one row; what doubles is the activation prologue and the dot products.
+struct QsRowsArgs {
+    const uint8_t *w; const float *x; void *dst;
+    int n;
+    uint32_t meta;            // bpr | dst_dtype << 8
+    int stride_dst;           // elements between the two output rows
+};
+template <int DT, int XS, int MAXB>
+__global__ __launch_bounds__(QS_NW * 64) void qms_rows2_kernel(QsRowsArgs a) {
+    typedef StreamFmt<DT> SF;
+    typedef StreamAct<MAXB> SA;
+    constexpr int NB = 2, NW = QS_NW, PRE = 4, SLOT = SF::NLD * 1024;
+    extern __shared__ __align__(16) uint8_t slots[];
+    __shared__ __align__(16) uint8_t act[NB][SA::BYTES];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = a.n, bpr = a.meta & 255, dst_dtype = (a.meta >> 8) & 255, k = bpr * 256;
+    const int lp_shift = bpr > 1 ? 32 - __builtin_clz(bpr - 1) : 0;
+    const int step_rows = 64 >> lp_shift, step_bytes = step_rows * bpr * SF::BB;
+    const int total_steps = (n + step_rows - 1) >> (6 - lp_shift);
+    const int64_t w_bytes = (int64_t)n * (bpr * SF::BB);
+    const int block = blockIdx.x, nblocks = qs_groups(total_steps);
+
+    // activation loads first, then the first copies of the wave's first step, then the quantization, then the rest
+    f32x4 xt[NB][XS];
+#pragma unroll
+    for (int r = 0; r < NB; r++)
+#pragma unroll
+        for (int j = 0; j < XS; j++) xt[r][j] = *(const f32x4 *)(a.x + (int64_t)r * k + min(wv + j * NW, bpr - 1) * 256 + lane * 4);
+    asm volatile("" ::: "memory");
+    uint8_t *slot = slots + wv * SLOT;
+    const int step0 = wv * nblocks + block, sstride = NW * nblocks;
+    const int my = step0 < total_steps ? (total_steps - step0 + sstride - 1) / sstride : 0;
+    auto issue = [&](int t, int j0, int j1) {
+        const bool live = t < my;
+        const int64_t off = (int64_t)(live ? step0 + t * sstride : 0) * step_bytes;
+        const int64_t left = w_bytes - off;
+        const int bytes = live ? (int)(left < step_bytes ? left : step_bytes) : 0;     // an absent step: a descriptor of zero bytes
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(a.w + off), 0, bytes, 0x00020000);
+#pragma unroll
+        for (int j = 0; j < SF::NLD; j++)
+            if (j >= j0 && j < j1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(slot + j * 1024), 16, lane * 16, j * 1024, 0, 0);
+    };
+    issue(0, 0, PRE);
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int r = 0; r < NB; r++)
+#pragma unroll
+        for (int j = 0; j < XS; j++) {
+            const float xv[4] = {xt[r][j].x, xt[r][j].y, xt[r][j].z, xt[r][j].w};
+            const int span = wv + j * NW;
+            qs_quantize_span<DT == CQ_Q6K>(xv, span < bpr ? span : MAXB, lane, act[r], SA::AUX_OFF);
+        }
+    asm volatile("" ::: "memory");
+    issue(0, PRE, SF::NLD);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");       // no fence: it would wait for the copies in flight
+
+    const int lp = 1 << lp_shift;
+    const int rin = lane >> lp_shift, sb = lane & (lp - 1);
+    const bool valid_sb = sb < bpr;
+    const int sbc = valid_sb ? sb : bpr - 1;
+    u32x4 areg[NB][16];
+    QsAux aux[NB];
+    float d8[NB];
+#pragma unroll
+    for (int r = 0; r < NB; r++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) areg[r][i] = *(const u32x4 *)(act[r] + sbc * QS_ACT_STRIDE + 16 * i);
+        const uint8_t *auxp = act[r] + SA::AUX_OFF + sbc * QS_AUX_STRIDE;
+        d8[r] = __uint_as_float((*(const u32x4 *)auxp).x);
+        aux[r].s32 = *(const u32x4 *)(auxp + 16);
+        if constexpr (DT == CQ_Q6K) {
+            aux[r].bl16 = *(const u32x4 *)(auxp + 32);
+            aux[r].bh16 = *(const u32x4 *)(auxp + 48);
+        }
+    }
+    const int boff = (rin * bpr + sbc) * SF::BB;
+    const bool last = sb == lp - 1;
+    for (int t = 0; t < my; t++) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const int row = (step0 + t * sstride) * step_rows + rin;
+        typename SF::Blk b0;
+        SF::read(b0, slot + boff);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        issue(t + 1, 0, SF::NLD);
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            float v = SF::dot(b0, areg[r], d8[r], aux[r]);
+            v = qs_group_sum(valid_sb ? v : 0.0f, lp_shift);
+            if (last && row < n) store_out(a.dst, dst_dtype, (int64_t)r * a.stride_dst + row, v);
+        }
+    }
+}
+
 // Two weight tensors over the same activation row in one launch, tensor A on the streaming body; tensor B on the
 // streaming body as well (SB) or on qmv_body.  Workgroups [0, blocks_a) take tensor A.  NW waves per workgroup: 8, or
 // 16 where qmv_body needs one wave per activation span (its plane-merging prologue).
@@ -1047,6 +1145,33 @@ int launch_stream(const void *w, const float *x, void *dst, int dst_dtype, int64
             return launch_stream_xs<DT, 8, 64, PRO, EPI>(w, x, dst, g, s, fz);
         }
     }
+}
+
+template <int DT, int XS, int MAXB>
+int launch_stream_rows2_xs(const void *w, const float *x, void *dst, const StreamGeom &g, int64_t stride_dst, hipStream_t s) {
+    const size_t lds_bytes = (size_t)QS_NW * StreamFmt<DT>::NLD * 1024;
+    if (lds_bytes + 2 * StreamAct<MAXB>::BYTES + 256 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
+    auto kern = qms_rows2_kernel<DT, XS, MAXB>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (stride_dst > 0x7fffffffLL || g.dst_dtype > 255) return CQ_ERR_RANGE;
+    QsRowsArgs a{(const uint8_t *)w, x, dst, g.n, (uint32_t)g.bpr | ((uint32_t)g.dst_dtype << 8), (int)stride_dst};
+    hipLaunchKernelGGL(kern, dim3((unsigned)qs_groups(g.total_steps)), dim3(64 * QS_NW), lds_bytes, s, a);
+    return (int)hipGetLastError();
+}
+
+// two f32 rows; CQ_ERR_RANGE: not a shape of the streaming kernel
+template <int DT>
+int launch_stream_rows2(const void *w, const float *x, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
+    StreamGeom g;
+    if (!stream_geom<DT>(g, k, n, dst_dtype)) return CQ_ERR_RANGE;
+    if (g.bpr <= 8) return launch_stream_rows2_xs<DT, 1, 16>(w, x, dst, g, stride_dst, s);
+    if (g.bpr <= 16) return launch_stream_rows2_xs<DT, 2, 16>(w, x, dst, g, stride_dst, s);
+    if (g.bpr <= 32) return launch_stream_rows2_xs<DT, 4, 64>(w, x, dst, g, stride_dst, s);
+    if (g.bpr <= 56) return launch_stream_rows2_xs<DT, 7, 64>(w, x, dst, g, stride_dst, s);
+    return launch_stream_rows2_xs<DT, 8, 64>(w, x, dst, g, stride_dst, s);
 }
 
 // Geometry of one launch.  waves == 0: as many waves per workgroup (a power of two, at most 16) as still leave every
@@ -1214,6 +1339,14 @@ int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtyp
         if (w_dtype == CQ_Q4K) rc = launch_stream<CQ_Q4K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
         if (w_dtype == CQ_Q5K) rc = launch_stream<CQ_Q5K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
         if (w_dtype == CQ_Q6K) rc = launch_stream<CQ_Q6K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
+        if (rc != CQ_ERR_RANGE) return rc;
+    }
+    if (rows == 2 && x_dtype == CQ_F32) {
+        // two f32 rows: both on one pass of the streaming kernel
+        int rc = CQ_ERR_RANGE;
+        if (w_dtype == CQ_Q4K) rc = launch_stream_rows2<CQ_Q4K>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
+        if (w_dtype == CQ_Q5K) rc = launch_stream_rows2<CQ_Q5K>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
+        if (w_dtype == CQ_Q6K) rc = launch_stream_rows2<CQ_Q6K>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
         if (rc != CQ_ERR_RANGE) return rc;
     }
     const int64_t xsz = x_dtype == CQ_F32 ? 4 : 2, esz = dst_dtype == CQ_F32 ? 4 : 2;
