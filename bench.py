@@ -21,8 +21,8 @@ The JSON line carries, besides the driver contract fields:
                 (read from the committed summary under profiles/, with the commit it was measured at)
   cpu_baseline  the C restatement of candle's CPU path (AVX2 dot products + column-split threads,
                 oracle/cq_oracle_fast.c) timed on this box's host cores on bounded samples, for the headline
-                configuration and for three more (Q8_0 4096x4096 batch 1, the headline shape at batch 16,
-                Q6_K 4096x14336 at 128 rows), with the CPU model and the thread count
+                configuration and for four more (Q8_0 4096x4096 batch 1, the headline shape at batch 16,
+                Q6_K 4096x14336 at 128 rows, the matvecs of an 8B-shape decode step), with the CPU model and the thread count
   cfg1, cfg2_sweep, prefill, moe, decode_8b
                 compact records of the other configurations: the Q8_0 4096 x 4096 matvec, the Q4_K batch sweep
                 on both FFN shapes, the prefill matmuls at 128 / 512 / 2048 rows, the 48-layer MoE stack at
@@ -452,6 +452,23 @@ def cpu_matmul_baseline(torch, fmt, n, k, m, threads, seconds, copies, seed=77):
             "GFLOPs": round(2.0 * m * n * k / dt_s / 1e9, 1), "calls": it, "seconds": round(dt_s * it, 1), "weight_copies": copies}
 
 
+def cpu_decode_baseline(torch, threads, seconds_each=1.0):
+    """cfg4 on the CPU restatement: the eight matvecs of one decode step of the 8B-shape Q4_K_M model (seven per layer and the
+    output head), each timed on its own at one activation row; a token is 32 layers plus the head (the f32 glue — norms,
+    rope, attention, silu — is left out, so this flatters the CPU)."""
+    shapes = [("attention_wq", "q4k", 4096, 4096), ("attention_wk", "q4k", 1024, 4096), ("attention_wv", "q6k", 1024, 4096),
+              ("attention_wo", "q4k", 4096, 4096), ("feed_forward_w1", "q4k", 14336, 4096), ("feed_forward_w3", "q4k", 14336, 4096),
+              ("feed_forward_w2", "q6k", 4096, 14336), ("output", "q4k", 128256, 4096)]
+    per = {}
+    for name, fmt, n, k in shapes:
+        r = cpu_matmul_baseline(torch, fmt, n, k, 1, threads, seconds_each, copies=2 if n > 100000 else 6)
+        per[name] = r["ms_per_call"]
+    layer_ms = sum(v for kname, v in per.items() if kname != "output")
+    token_ms = 32 * layer_ms + per["output"]
+    return {"workload": "8B-shape Q4_K_M decode, matvecs only: 32 x (wq, wk, wv, wo, w1, w3, w2) + output head, one row",
+            "ms_per_matvec": per, "layer_ms": round(layer_ms, 3), "token_ms": round(token_ms, 2), "tok_s": round(1e3 / token_ms, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -614,7 +631,8 @@ def main():
                                "threads_rule": "physical cores, at most the 16 this box allots to one GPU",
                                "others": {"cfg1_q8_0_4096x4096_b1": cpu_matmul_baseline(torch, "q8_0", 4096, 4096, 1, threads, 3.0, copies=16),
                                           "cfg2_q4k_14336x4096_b16": cpu_matmul_baseline(torch, "q4k", 14336, 4096, 16, threads, 3.0, copies=8),
-                                          "cfg3_q6k_4096x14336_m128": cpu_matmul_baseline(torch, "q6k", 4096, 14336, 128, threads, 3.0, copies=4)}}
+                                          "cfg3_q6k_4096x14336_m128": cpu_matmul_baseline(torch, "q6k", 4096, 14336, 128, threads, 3.0, copies=4),
+                                          "cfg4_decode_8b": cpu_decode_baseline(torch, threads)}}
     print(json.dumps(out))
 
 
