@@ -623,7 +623,13 @@ __global__ __launch_bounds__(1024) void qmv2_kernel(const uint8_t *__restrict__ 
 // (s / grid) % QS_NW of workgroup s % grid, so at any moment the whole chip reads one compact window of the tensor.
 // ---------------------------------------------------------------------------------------------
 constexpr int QS_NW = 8;
-constexpr bool qs_streams(int dt) { return dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K; }     // formats with a StreamFmt
+constexpr bool qs_streams(int dt) { return dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q4_0 || dt == CQ_Q8_0; }     // formats with a StreamFmt
+constexpr bool qs_wide_aux(int dt) { return dt == CQ_Q6K || dt == CQ_Q4_0 || dt == CQ_Q8_0; }      // ... whose lanes keep the whole 64-byte span record
+// the activation quantization a weight format asks for: Q8_K spans (with the 16-element sums for Q6_K) or Q8_0 blocks
+template <int DT> __device__ __forceinline__ void qs_quantize(const float v[4], int span, int lane, uint8_t *act, int aux_off) {
+    if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0) qs_quantize_span_q80(v, span, lane, act, aux_off);
+    else qs_quantize_span<DT == CQ_Q6K>(v, span, lane, act, aux_off);
+}
 
 template <int DT, int NW, int XS, int MAXB, int PRO, int EPI, int MSP = MAXS>
 __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const float *__restrict__ x, void *__restrict__ dst, const StreamGeom &g,
@@ -748,7 +754,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         if (PRO == PRO_NORM || PRO == PRO_SILU) pro_apply<PRO>(xv[j], a4, pm);
         if (PRO == PRO_NORM_SPLIT) pro_apply<PRO_NORM>(xv[j], a4, pm);
         const int span = wv + j * NW;
-        qs_quantize_span<DT == CQ_Q6K>(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
+        qs_quantize<DT>(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
     }
     asm volatile("" ::: "memory");
     issue(0, PRE, SF::NLD);
@@ -767,7 +773,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     const u32x4 aux0 = *(const u32x4 *)auxp;
     QsAux aux1;
     aux1.s32 = *(const u32x4 *)(auxp + 16);
-    if constexpr (DT == CQ_Q6K) {
+    if constexpr (qs_wide_aux(DT)) {
         aux1.bl16 = *(const u32x4 *)(auxp + 32);
         aux1.bh16 = *(const u32x4 *)(auxp + 48);
     }
@@ -975,7 +981,7 @@ __global__ __launch_bounds__(QS_NW * 64) void qms_rows2_kernel(QsRowsArgs a) {
         for (int j = 0; j < XS; j++) {
             const float xv[4] = {xt[r][j].x, xt[r][j].y, xt[r][j].z, xt[r][j].w};
             const int span = wv + j * NW;
-            qs_quantize_span<DT == CQ_Q6K>(xv, span < bpr ? span : MAXB, lane, act[r], SA::AUX_OFF);
+            qs_quantize<DT>(xv, span < bpr ? span : MAXB, lane, act[r], SA::AUX_OFF);
         }
     asm volatile("" ::: "memory");
     issue(0, PRE, SF::NLD);
@@ -995,7 +1001,7 @@ __global__ __launch_bounds__(QS_NW * 64) void qms_rows2_kernel(QsRowsArgs a) {
         const uint8_t *auxp = act[r] + SA::AUX_OFF + sbc * QS_AUX_STRIDE;
         d8[r] = __uint_as_float((*(const u32x4 *)auxp).x);
         aux[r].s32 = *(const u32x4 *)(auxp + 16);
-        if constexpr (DT == CQ_Q6K) {
+        if constexpr (qs_wide_aux(DT)) {
             aux[r].bl16 = *(const u32x4 *)(auxp + 32);
             aux[r].bh16 = *(const u32x4 *)(auxp + 48);
         }
@@ -1083,7 +1089,7 @@ bool stream_geom(StreamGeom &g, int64_t k, int64_t n, int dst_dtype) {
     int sh = 0;
     while ((1 << sh) < bpr) sh++;
     if ((1 << sh) != bpr && 4 * bpr < 3 * (1 << sh)) return false;
-    const int64_t bb = BlockInfo<DT>::bytes;
+    const int64_t bb = BlockInfo<DT>::bytes * (256 / BlockInfo<DT>::elems);       // bytes of 256 elements: a super-block, or eight blocks
     // every wave step must start on 16 bytes of the stream (Q6_K blocks are 210 bytes: steps of a multiple of 8 blocks)
     if (((64 >> sh) * bpr * bb) % 16) return false;
     g.k = (int)k; g.n = (int)n; g.bpr = (int)bpr; g.lp_shift = sh;
@@ -1126,6 +1132,7 @@ int launch_stream(const void *w, const float *x, void *dst, int dst_dtype, int64
     } else {
         StreamGeom g;
         if (!stream_geom<DT>(g, k, n, dst_dtype)) return CQ_ERR_RANGE;
+        if ((uintptr_t)w & 15) return CQ_ERR_RANGE;              // the copies into LDS move aligned 16-byte pieces
         if (epi_is_resid(EPI) && n > (int64_t)256 * 64 * 1024) return CQ_ERR_RANGE;
         const int bpr = g.bpr;
         if constexpr (PRO == PRO_MERGE) {
@@ -1166,7 +1173,7 @@ int launch_stream_rows2_xs(const void *w, const float *x, void *dst, const Strea
 template <int DT>
 int launch_stream_rows2(const void *w, const float *x, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t stride_dst, hipStream_t s) {
     StreamGeom g;
-    if (!stream_geom<DT>(g, k, n, dst_dtype)) return CQ_ERR_RANGE;
+    if (!stream_geom<DT>(g, k, n, dst_dtype) || ((uintptr_t)w & 15)) return CQ_ERR_RANGE;
     if (g.bpr <= 8) return launch_stream_rows2_xs<DT, 1, 16>(w, x, dst, g, stride_dst, s);
     if (g.bpr <= 16) return launch_stream_rows2_xs<DT, 2, 16>(w, x, dst, g, stride_dst, s);
     if (g.bpr <= 32) return launch_stream_rows2_xs<DT, 4, 64>(w, x, dst, g, stride_dst, s);
@@ -1333,12 +1340,14 @@ int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtyp
                            int64_t rows, int64_t stride_dst, hipStream_t s) {
     if (n == 0 || rows == 0) return CQ_OK;
     if (rows == 1 && x_dtype == CQ_F32) {
-        // one f32 row over Q4_K / Q5_K / Q6_K weights: the streaming kernel where it takes the shape
+        // one f32 row over Q4_K / Q5_K / Q6_K / Q4_0 / Q8_0 weights: the streaming kernel where it takes the shape
         const Fuse none{nullptr, nullptr, 0.0f, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0};
         int rc = CQ_ERR_RANGE;
         if (w_dtype == CQ_Q4K) rc = launch_stream<CQ_Q4K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
         if (w_dtype == CQ_Q5K) rc = launch_stream<CQ_Q5K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
         if (w_dtype == CQ_Q6K) rc = launch_stream<CQ_Q6K, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
+        if (w_dtype == CQ_Q4_0) rc = launch_stream<CQ_Q4_0, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
+        if (w_dtype == CQ_Q8_0) rc = launch_stream<CQ_Q8_0, PRO_NONE, EPI_NONE>(w, (const float *)x, dst, dst_dtype, k, n, s, none);
         if (rc != CQ_ERR_RANGE) return rc;
     }
     if (rows == 2 && x_dtype == CQ_F32) {
@@ -1347,6 +1356,8 @@ int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtyp
         if (w_dtype == CQ_Q4K) rc = launch_stream_rows2<CQ_Q4K>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
         if (w_dtype == CQ_Q5K) rc = launch_stream_rows2<CQ_Q5K>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
         if (w_dtype == CQ_Q6K) rc = launch_stream_rows2<CQ_Q6K>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
+        if (w_dtype == CQ_Q4_0) rc = launch_stream_rows2<CQ_Q4_0>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
+        if (w_dtype == CQ_Q8_0) rc = launch_stream_rows2<CQ_Q8_0>(w, (const float *)x, dst, dst_dtype, k, n, stride_dst, s);
         if (rc != CQ_ERR_RANGE) return rc;
     }
     const int64_t xsz = x_dtype == CQ_F32 ? 4 : 2, esz = dst_dtype == CQ_F32 ? 4 : 2;
@@ -1540,7 +1551,7 @@ template <int DTA, int DTB, int PRO>
 int launch_pair_stream(const void *wa, int64_t na, float *dsta, const void *wb, int64_t nb, float *dstb, const float *x, int64_t k, hipStream_t s,
                        const Fuse &fz) {
     StreamGeom ga;
-    if (!stream_geom<DTA>(ga, k, na, CQ_F32)) return CQ_ERR_RANGE;
+    if (!stream_geom<DTA>(ga, k, na, CQ_F32) || ((uintptr_t)wa & 15)) return CQ_ERR_RANGE;
     const int bpr = ga.bpr;
     if (bpr > 16) return CQ_ERR_RANGE;            // longer rows: the two-tensor launch of qmv_kernel
     StreamGeom gsb = ga;

@@ -1,4 +1,5 @@
-// Streaming decode matvec for Q4_K / Q5_K / Q6_K weights and one f32 activation row:  dst[row] = sum_k W[row, k] * x^[k].
+// Streaming decode matvec for Q4_K / Q5_K / Q6_K / Q4_0 / Q8_0 weights and one f32 activation row:
+// dst[row] = sum_k W[row, k] * x^[k].  For Q4_0 / Q8_0 a "super-block" below is eight consecutive 32-element blocks.
 //
 // The weights of a tensor are one contiguous stream of super-blocks (rows follow each other without gaps).  A wave
 // step is a run of that stream — 64 super-blocks when a row has a power of two of them, else one row — copied
@@ -16,7 +17,9 @@
 //
 // Same arithmetic contract as qmv_kernel: activations quantized to Q8_K exactly like BlockQ8K::from_float
 // (candle-core/src/quantized/k_quants.rs:2320-2358), integer dots exact, one f32 scaling per super-block
-// (vec_dot Q4_K x Q8_K k_quants.rs:1460-1540, Q5_K :1714-1801, Q6_K :2035-2092); only the f32 summation order differs.
+// (vec_dot Q4_K x Q8_K k_quants.rs:1460-1540, Q5_K :1714-1801, Q6_K :2035-2092); Q4_0 / Q8_0 rows take Q8_0 activation
+// blocks like BlockQ8_0::from_float (k_quants.rs:658-687) and the per-block sums of their vec_dot (:294-311, 720-738),
+// in block order; only the f32 summation order of the K-quant rows differs.
 #pragma once
 #include "cq_actquant.h"
 #include "cq_device.h"
@@ -30,7 +33,8 @@ typedef __attribute__((address_space(3))) void cq_lds_void;
 //   f32 d | 12 bytes unused | u8 bl[8] | i8 bh[8] | u8 bl16[16] | i8 bh16[16]
 // with  sum of 32-element sub-block j = 128 * bh[j] + bl[j]  and  sum of 16-element group g = 128 * bh16[g] + bl16[g],
 // 0 <= bl < 128 (the sums split into two int8 halves, so that sum_j coefficient_j * sum_j is a few dot4).  The 16-element
-// sums are written for Q6_K only, whose scales cover 16 elements.
+// sums are written for Q6_K only, whose scales cover 16 elements.  Q8_0 activations (for Q4_0 / Q8_0 weights) have a scale
+// per 32 elements: their record keeps the eight f32 scales in the last 32 bytes and the 32-element sums where they are.
 constexpr int QS_ACT_STRIDE = 272;
 constexpr int QS_AUX_STRIDE = 64;
 template <int MAXB> struct StreamAct {
@@ -86,6 +90,25 @@ __device__ __forceinline__ void qs_quantize_span(const float v[4], int span, int
         aux[24 + (lane >> 3)] = (uint8_t)(s >> 7);    // arithmetic shift: 128 * bh + bl == s for negative sums too
     }
     if (lane == 0) *(float *)aux = d;
+}
+
+// The same span as eight Q8_0 blocks (cq_quantize_q80_vals, cq_actquant.h: BlockQ8_0::from_float with the f16-rounded scale).
+__device__ __forceinline__ void qs_quantize_span_q80(const float v[4], int span, int lane, uint8_t *act, int aux_off) {
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    amax = oct_max(amax);                             // a 32-element block = eight neighbouring lanes
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) packed |= (uint32_t)(cq_round_sat_i8(v[i] * id) & 0xff) << (8 * i);
+    *(uint32_t *)(act + span * QS_ACT_STRIDE + lane * 4) = packed;
+    int s = oct_sum(sdot4(packed, 0x01010101u, 0));
+    uint8_t *aux = act + aux_off + span * QS_AUX_STRIDE;
+    if ((lane & 7) == 0) {
+        aux[16 + (lane >> 3)] = (uint8_t)(s & 127);
+        aux[24 + (lane >> 3)] = (uint8_t)(s >> 7);
+        ((float *)(aux + 32))[lane >> 3] = h2f(f2h_bits(d));      // the CPU stores d as f16 and multiplies by its f32 value
+    }
 }
 
 // ---- per-format work of one lane on one super-block held in LDS --------------------------------------------
@@ -249,6 +272,78 @@ template <> struct StreamFmt<CQ_Q6K> {
         }
         S -= ((Ch << 7) + C) << 5;
         return (h2f(b.d) * d8) * (float)S;
+    }
+};
+
+// ---- Q4_0 / Q8_0: eight blocks of 18 / 34 bytes per lane -------------------------------------------------------------
+// The lane's 144 / 272 bytes start on 16 bytes; inside them block b starts at byte 18 b / 34 b, so the quants of the even
+// blocks sit 2 bytes off the dword grid and are put back with one v_alignbyte_b32 per dword.  `aux.bl16 | aux.bh16` hold the
+// eight f32 activation scales, `aux.s32` the eight block sums as (bl, bh).
+__device__ __forceinline__ float qs_q0_scale(const QsAux &aux, int b) {
+    return __uint_as_float(b < 4 ? aux.bl16[b] : aux.bh16[b - 4]);
+}
+// dword i of the payload that starts `off` bytes into the dword array r (off even, known at compile time)
+template <int N> __device__ __forceinline__ uint32_t qs_dword_at(const uint32_t (&r)[N], int off) {
+    const int w = off >> 2;
+    return (off & 2) ? __builtin_amdgcn_alignbyte(r[w + 1 < N ? w + 1 : w], r[w], 2) : r[w];
+}
+template <int N> __device__ __forceinline__ uint32_t qs_half_at(const uint32_t (&r)[N], int off) {
+    return (off & 2) ? r[off >> 2] >> 16 : r[off >> 2] & 0xffffu;
+}
+
+template <> struct StreamFmt<CQ_Q8_0> {
+    static constexpr int BB = 272;             // eight blocks
+    static constexpr int NLD = 17;
+    struct Blk { uint32_t r[68]; };
+    static __device__ __forceinline__ void read(Blk &b, const uint8_t *p) {
+#pragma unroll
+        for (int i = 0; i < 17; i++) {
+            const u32x4 t = *(const u32x4 *)(p + 16 * i);
+            b.r[4 * i] = t.x; b.r[4 * i + 1] = t.y; b.r[4 * i + 2] = t.z; b.r[4 * i + 3] = t.w;
+        }
+    }
+    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float, const QsAux &aux) {
+        float sumf = 0.0f;
+#pragma unroll
+        for (int blk = 0; blk < 8; blk++) {
+            int s = 0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) s = sdot4(qs_dword_at(b.r, 34 * blk + 2 + 4 * i), a[2 * blk + (i >> 2)][i & 3], s);
+            sumf += (float)s * h2f(qs_half_at(b.r, 34 * blk)) * qs_q0_scale(aux, blk);
+        }
+        return sumf;
+    }
+};
+
+template <> struct StreamFmt<CQ_Q4_0> {
+    static constexpr int BB = 144;
+    static constexpr int NLD = 9;
+    struct Blk { uint32_t r[36]; };
+    static __device__ __forceinline__ void read(Blk &b, const uint8_t *p) {
+#pragma unroll
+        for (int i = 0; i < 9; i++) {
+            const u32x4 t = *(const u32x4 *)(p + 16 * i);
+            b.r[4 * i] = t.x; b.r[4 * i + 1] = t.y; b.r[4 * i + 2] = t.z; b.r[4 * i + 3] = t.w;
+        }
+    }
+    static __device__ __forceinline__ float dot(const Blk &b, const u32x4 (&a)[16], float, const QsAux &aux) {
+        const uint32_t M4 = 0x0f0f0f0fu;
+        float sumf = 0.0f;
+#pragma unroll
+        for (int blk = 0; blk < 8; blk++) {
+            // sum((q - 8) * y) = sum(q * y) - 8 * sum(y); the block sum is 128 * bh + bl
+            const uint32_t bl = (aux.s32[blk >> 2] >> (8 * (blk & 3))) & 0xffu;
+            const int bh = (int)(int8_t)(aux.s32[2 + (blk >> 2)] >> (8 * (blk & 3)));
+            int s = -8 * (128 * bh + (int)bl);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t q = qs_dword_at(b.r, 18 * blk + 2 + 4 * i);
+                s = sdot4(q & M4, a[2 * blk][i], s);
+                s = sdot4((q >> 4) & M4, a[2 * blk + 1][i], s);
+            }
+            sumf += (float)s * h2f(qs_half_at(b.r, 18 * blk)) * qs_q0_scale(aux, blk);
+        }
+        return sumf;
     }
 };
 
