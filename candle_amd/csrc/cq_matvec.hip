@@ -631,10 +631,15 @@ template <int DT> __device__ __forceinline__ void qs_quantize(const float v[4], 
     else qs_quantize_span<DT == CQ_Q6K>(v, span, lane, act, aux_off);
 }
 
-template <int DT, int NW, int XS, int MAXB, int PRO, int EPI, int MSP = MAXS>
+// PROD: the workgroup has one more wave, a producer, that requests the first step of all NW working waves at once and does
+// nothing else.  A wave that has asked for more than the memory pipeline takes is stopped at its next copy, so a working
+// wave can only ask for a few copies before its activation prologue; with rows of several spans per wave that prologue is
+// long, and the weights would wait for it.  The producer can be stopped: nobody queues behind it.
+template <int DT, int NW, int XS, int MAXB, int PRO, int EPI, int MSP = MAXS, bool PROD = false>
 __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const float *__restrict__ x, void *__restrict__ dst, const StreamGeom &g,
                                          const Fuse &fz, const int block, const int nblocks) {
     typedef StreamFmt<DT> SF;
+    static_assert(!PROD || (PRO != PRO_MERGE && EPI != EPI_SWIGLU), "the producer wave serves the long-row launches only");
     typedef StreamAct<MAXB> SA;
     constexpr bool RESID = epi_is_resid(EPI);
     constexpr bool PAIR = EPI == EPI_SWIGLU;               // two weight rows per output row: a step is two sub-steps, gate rows then up rows
@@ -657,6 +662,33 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int k = g.k, n = g.n, bpr = g.bpr;
+    const int sstride = NW * nblocks;
+    // sub-step t of wave wq: step wq * nblocks + block + (t / SUBS) * sstride, of the gate tensor (even t) or the up tensor
+    // (odd t); copies [j0, j1) of it.  The loads are unconditional: a step that does not exist gets a descriptor of zero
+    // bytes (its loads read nothing), so that the waits below stay counted waits.
+    auto issue_for = [&](int wq, int t, int j0, int j1) {
+        const int s0 = wq * nblocks + block;
+        const int st = s0 + (PAIR ? t >> 1 : t) * sstride;
+        const uint8_t *wbase = PAIR && (t & 1) ? w + fz.pair_off : w;
+        const bool live = st < g.total_steps;
+        const int64_t off = (int64_t)(live ? st : 0) * g.step_bytes;
+        const int64_t left = g.w_bytes - off;
+        const int bytes = live ? (int)(left < g.step_bytes ? left : g.step_bytes) : 0;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(wbase + off), 0, bytes, 0x00020000);
+#pragma unroll
+        for (int j = 0; j < SF::NLD; j++)
+            if (j >= j0 && j < j1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(slots + wq * SLOT + j * 1024), 16, lane * 16, j * 1024, 0, 0);
+    };
+    if (PROD && wv == NW) {
+        // the producer wave: every working wave's first step, then the workgroup's barriers (one with PRO_NORM_SPLIT, the
+        // one that opens the steps, one with the residual epilogues), the second of them once the copies have landed
+#pragma unroll 1
+        for (int wq = 0; wq < NW; wq++) issue_for(wq, 0, 0, SF::NLD);
+        if (PRO == PRO_NORM_SPLIT) asm volatile("s_barrier" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        if (RESID) asm volatile("s_barrier" ::: "memory");
+        return;
+    }
 
     // 0. activation loads first (vector loads complete in order: what is asked for after the weights waits for them)
     f32x4 xt[XS], at[XS];
@@ -686,26 +718,12 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     }
     asm volatile("" ::: "memory");
 
-    // 1. the wave's first step on its way into LDS.  The loads are unconditional: a step that does not exist gets a
-    //    descriptor of zero bytes (its loads read nothing), so that the waits below stay counted waits.
+    // 1. the wave's first step on its way into LDS (with a producer wave that is the producer's part)
     uint8_t *slot = slots + wv * SLOT;
     const int step0 = wv * nblocks + block;
-    const int sstride = NW * nblocks;
     const int my = step0 < g.total_steps ? (g.total_steps - step0 + sstride - 1) / sstride : 0;
-    // sub-step t of this wave: step step0 + (t / SUBS) * sstride, of the gate tensor (even t) or the up tensor (odd t)
-    auto issue = [&](int t, int j0, int j1) {
-        const int st = step0 + (PAIR ? t >> 1 : t) * sstride;
-        const uint8_t *wbase = PAIR && (t & 1) ? w + fz.pair_off : w;
-        const bool live = t < SUBS * my;
-        const int64_t off = (int64_t)(live ? st : 0) * g.step_bytes;
-        const int64_t left = g.w_bytes - off;
-        const int bytes = live ? (int)(left < g.step_bytes ? left : g.step_bytes) : 0;
-        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(wbase + off), 0, bytes, 0x00020000);
-#pragma unroll
-        for (int j = 0; j < SF::NLD; j++)
-            if (j >= j0 && j < j1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(slot + j * 1024), 16, lane * 16, j * 1024, 0, 0);
-    };
-    issue(0, 0, PRE);
+    auto issue = [&](int t, int j0, int j1) { issue_for(wv, t, j0, j1); };
+    if (!PROD) issue(0, 0, PRE);
     asm volatile("" ::: "memory");
 
     // 2. activations -> LDS
@@ -757,7 +775,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         qs_quantize<DT>(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
     }
     asm volatile("" ::: "memory");
-    issue(0, PRE, SF::NLD);
+    if (!PROD) issue(0, PRE, SF::NLD);
     // a barrier without the fence of __syncthreads(): the fence would wait for the LDS copies in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
@@ -918,13 +936,13 @@ __device__ __forceinline__ void qs_unpack(const QsArgs<PRO, EPI> &a, const uint8
     g.w_bytes = (int64_t)n * (bpr * StreamFmt<DT>::BB);
 }
 
-template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP>
-__global__ __launch_bounds__(QS_NW * 64) void qms_kernel(QsArgs<PRO, EPI> a) {
+template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP, bool PROD>
+__global__ __launch_bounds__((QS_NW + (PROD ? 1 : 0)) * 64) void qms_kernel(QsArgs<PRO, EPI> a) {
     const uint8_t *w; const float *x; void *dst; StreamGeom g; Fuse fz;
     qs_unpack<DT, PRO, EPI>(a, w, x, dst, g, fz);
     // the grid size is derived, not read: gridDim comes from the hidden arguments behind the explicit ones, and every
     // argument byte a kernel reads beyond the first 64 costs a second trip at its start
-    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
+    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP, PROD>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
 }
 
 // ---- two activation rows on the streaming kernel -------------------------------------------------------------
@@ -1105,14 +1123,16 @@ template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP = 1>
 int launch_stream_xs(const void *w, const float *x, void *dst, const StreamGeom &g, hipStream_t s, const Fuse &fz) {
     const size_t lds_bytes = (size_t)QS_NW * StreamFmt<DT>::NLD * 1024;
     if (lds_bytes + StreamAct<MAXB>::BYTES + 256 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
-    auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI, MSP>;
+    // rows of more than two spans per wave get the producer wave
+    constexpr bool PROD = XS > 2;
+    auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI, MSP, PROD>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
     }
     const int groups = qs_groups(g.total_steps);
     if (fz.pair_off % 16 || fz.n_planes > 15 || fz.splits > 63 || g.dst_dtype > 255) return CQ_ERR_RANGE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * QS_NW), lds_bytes, s, qs_pack<DT, PRO, EPI>(w, x, dst, g, fz));
+    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * (QS_NW + (PROD ? 1 : 0))), lds_bytes, s, qs_pack<DT, PRO, EPI>(w, x, dst, g, fz));
     return (int)hipGetLastError();
 }
 
