@@ -626,9 +626,17 @@ constexpr int QS_NW = 8;
 constexpr bool qs_streams(int dt) { return dt == CQ_Q4K || dt == CQ_Q5K || dt == CQ_Q6K || dt == CQ_Q4_0 || dt == CQ_Q8_0; }     // formats with a StreamFmt
 constexpr bool qs_wide_aux(int dt) { return dt == CQ_Q6K || dt == CQ_Q4_0 || dt == CQ_Q8_0; }      // ... whose lanes keep the whole 64-byte span record
 // the activation quantization a weight format asks for: Q8_K spans (with the 16-element sums for Q6_K) or Q8_0 blocks
-template <int DT> __device__ __forceinline__ void qs_quantize(const float v[4], int span, int lane, uint8_t *act, int aux_off) {
-    if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0) qs_quantize_span_q80(v, span, lane, act, aux_off);
-    else qs_quantize_span<DT == CQ_Q6K>(v, span, lane, act, aux_off);
+template <int DT, int NS>
+__device__ __forceinline__ void qs_quantize(const float (&v)[NS][4], int span0, int stride, int limit, int dump, int lane, uint8_t *act, int aux_off) {
+    if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0) {
+#pragma unroll
+        for (int j = 0; j < NS; j++) {
+            const int span = span0 + j * stride;
+            qs_quantize_span_q80(v[j], span < limit ? span : dump, lane, act, aux_off);
+        }
+    } else {
+        qs_quantize_spans<DT == CQ_Q6K, NS>(v, span0, stride, limit, dump, lane, act, aux_off);
+    }
 }
 
 // PROD: the workgroup has one more wave, a producer, that requests the first step of all NW working waves at once and does
@@ -771,9 +779,8 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         const float a4[4] = {at[j].x, at[j].y, at[j].z, at[j].w};
         if (PRO == PRO_NORM || PRO == PRO_SILU) pro_apply<PRO>(xv[j], a4, pm);
         if (PRO == PRO_NORM_SPLIT) pro_apply<PRO_NORM>(xv[j], a4, pm);
-        const int span = wv + j * NW;
-        qs_quantize<DT>(xv[j], span < bpr ? span : MAXB, lane, act, SA::AUX_OFF);
     }
+    qs_quantize<DT, XS>(xv, wv, NW, bpr, MAXB, lane, act, SA::AUX_OFF);
     asm volatile("" ::: "memory");
     if (!PROD) issue(0, PRE, SF::NLD);
     // a barrier without the fence of __syncthreads(): the fence would wait for the LDS copies in flight
@@ -994,13 +1001,12 @@ __global__ __launch_bounds__(QS_NW * 64) void qms_rows2_kernel(QsRowsArgs a) {
     issue(0, 0, PRE);
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int r = 0; r < NB; r++)
+    for (int r = 0; r < NB; r++) {
+        float xv[XS][4];
 #pragma unroll
-        for (int j = 0; j < XS; j++) {
-            const float xv[4] = {xt[r][j].x, xt[r][j].y, xt[r][j].z, xt[r][j].w};
-            const int span = wv + j * NW;
-            qs_quantize<DT>(xv, span < bpr ? span : MAXB, lane, act[r], SA::AUX_OFF);
-        }
+        for (int j = 0; j < XS; j++) { xv[j][0] = xt[r][j].x; xv[j][1] = xt[r][j].y; xv[j][2] = xt[r][j].z; xv[j][3] = xt[r][j].w; }
+        qs_quantize<DT, XS>(xv, wv, NW, bpr, MAXB, lane, act[r], SA::AUX_OFF);
+    }
     asm volatile("" ::: "memory");
     issue(0, PRE, SF::NLD);
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");       // no fence: it would wait for the copies in flight

@@ -53,27 +53,55 @@ __device__ __forceinline__ uint32_t qs_wave_umax(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
-// One wave quantizes one 256-element span (lane l holds elements 4l .. 4l+3) into the LDS layout above.
-// BlockQ8K::from_float takes the FIRST element of largest magnitude for the scale; here any element of that
-// magnitude is taken: with another sign d and every q flip together and every product d * q is the same value, so
-// no result of the matvec depends on it.  NaN / Inf inputs follow the CPU arithmetic (round, saturating cast, NaN -> 0).
-template <bool SUM16 = false>
-__device__ __forceinline__ void qs_quantize_span(const float v[4], int span, int lane, uint8_t *act, int aux_off) {
+// f32::round (half away from zero) followed by Rust's `as i8` (saturating, NaN -> 0) in five instructions.  Adding the largest
+// float below one half, with the sign of x, carries exactly the values whose fraction is at least one half to the next
+// integer: the sum is rounded to nearest, a fraction of one half ends within a quarter of an ulp of that integer and a
+// smaller fraction at least an ulp of x below it (checked against trunc / compare / add on every float of magnitude
+// 2^-8 .. 2^25).  v_cvt_i32_f32 truncates, saturates and turns NaN into 0.
+__device__ __forceinline__ int qs_round_i8(float x) {
+    const float t = x + __builtin_copysignf(0.49999997f, x);
+    int q;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(t));
+    return min(max(q, -128), 127);
+}
+// four values in [-128, 127] -> four bytes
+__device__ __forceinline__ uint32_t qs_pack4(const int (&q)[4]) {
+    return __builtin_amdgcn_perm((uint32_t)q[1], (uint32_t)q[0], 0x0c0c0400u) | __builtin_amdgcn_perm((uint32_t)q[3], (uint32_t)q[2], 0x04000c0cu);
+}
+
+// One wave quantizes 256-element spans (lane l holds elements 4l .. 4l+3 of each) into the LDS layout above, in three
+// parts so that a wave with several spans pays for one division sequence: the largest magnitude of each span; the
+// scales of all spans, span j in lane j; the values.
+// BlockQ8K::from_float takes the FIRST element of largest magnitude, with its sign, for the scale; here the scale always
+// comes from the magnitude: with the other sign d and every q flip together and every product d * q is the same value,
+// so no result of the matvec depends on it.  NaN / Inf inputs follow the CPU arithmetic (round, saturating cast, NaN -> 0).
+__device__ __forceinline__ uint32_t qs_span_umax(const float v[4]) {
     float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
     amax = amax == amax ? amax : 0.0f;                // four NaNs: the CPU's `amax < |x|` never takes a NaN either
-    const uint32_t wmax = qs_wave_umax(__float_as_uint(amax));
-    const float cand = fabsf(v[0]) == amax ? v[0] : fabsf(v[1]) == amax ? v[1] : fabsf(v[2]) == amax ? v[2] : v[3];
-    const uint64_t who = __builtin_amdgcn_ballot_w64(__float_as_uint(amax) == wmax);    // never empty: compared as bit patterns
-    const int src = __builtin_ctzll(who);
-    const float maxv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cand), src));
-    uint32_t packed = 0;
-    float d = 0.0f;
-    if (wmax != 0) {
-        const float iscale = -127.0f / maxv;
+    return qs_wave_umax(__float_as_uint(amax));
+}
+// iscale = -127 / max and d = 1 / iscale (both 0 for an all-zero span) of NS spans whose maxima are wave-uniform
+template <int NS>
+__device__ __forceinline__ void qs_span_scales(const uint32_t (&wmax)[NS], int lane, float (&iscale)[NS], float (&d)[NS]) {
+    uint32_t m = wmax[NS - 1];
 #pragma unroll
-        for (int i = 0; i < 4; i++) packed |= (uint32_t)(cq_round_sat_i8(iscale * v[i]) & 0xff) << (8 * i);
-        d = 1.0f / iscale;
+    for (int j = 0; j < NS - 1; j++) asm("v_writelane_b32 %0, %1, %2" : "+v"(m) : "s"(wmax[j]), "i"(j));
+    float is = -127.0f / __uint_as_float(m);
+    float dd = 1.0f / is;
+    is = m != 0 ? is : 0.0f;
+    dd = m != 0 ? dd : 0.0f;
+#pragma unroll
+    for (int j = 0; j < NS; j++) {
+        iscale[j] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, is), j));
+        d[j] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dd), j));
     }
+}
+template <bool SUM16>
+__device__ __forceinline__ void qs_span_store(const float v[4], float iscale, float d, int span, int lane, uint8_t *act, int aux_off) {
+    int q[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) q[i] = qs_round_i8(iscale * v[i]);
+    const uint32_t packed = qs_pack4(q);
     *(uint32_t *)(act + span * QS_ACT_STRIDE + lane * 4) = packed;
     int s = sdot4(packed, 0x01010101u, 0);
     uint8_t *aux = act + aux_off + span * QS_AUX_STRIDE;
@@ -91,6 +119,21 @@ __device__ __forceinline__ void qs_quantize_span(const float v[4], int span, int
     }
     if (lane == 0) *(float *)aux = d;
 }
+// NS spans of one wave: values v[j] go to LDS span span0 + j * stride, or to span `dump` when that is not below `limit`
+template <bool SUM16, int NS>
+__device__ __forceinline__ void qs_quantize_spans(const float (&v)[NS][4], int span0, int stride, int limit, int dump, int lane, uint8_t *act,
+                                                  int aux_off) {
+    uint32_t wmax[NS];
+    float iscale[NS], d[NS];
+#pragma unroll
+    for (int j = 0; j < NS; j++) wmax[j] = qs_span_umax(v[j]);
+    qs_span_scales<NS>(wmax, lane, iscale, d);
+#pragma unroll
+    for (int j = 0; j < NS; j++) {
+        const int span = span0 + j * stride;
+        qs_span_store<SUM16>(v[j], iscale[j], d[j], span < limit ? span : dump, lane, act, aux_off);
+    }
+}
 
 // The same span as eight Q8_0 blocks (cq_quantize_q80_vals, cq_actquant.h: BlockQ8_0::from_float with the f16-rounded scale).
 __device__ __forceinline__ void qs_quantize_span_q80(const float v[4], int span, int lane, uint8_t *act, int aux_off) {
@@ -98,9 +141,10 @@ __device__ __forceinline__ void qs_quantize_span_q80(const float v[4], int span,
     amax = oct_max(amax);                             // a 32-element block = eight neighbouring lanes
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
-    uint32_t packed = 0;
+    int q[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) packed |= (uint32_t)(cq_round_sat_i8(v[i] * id) & 0xff) << (8 * i);
+    for (int i = 0; i < 4; i++) q[i] = qs_round_i8(v[i] * id);
+    const uint32_t packed = qs_pack4(q);
     *(uint32_t *)(act + span * QS_ACT_STRIDE + lane * 4) = packed;
     int s = oct_sum(sdot4(packed, 0x01010101u, 0));
     uint8_t *aux = act + aux_off + span * QS_AUX_STRIDE;
