@@ -639,6 +639,18 @@ __device__ __forceinline__ void qs_quantize(const float (&v)[NS][4], int span0, 
     }
 }
 
+// The producer wave tells working wave WQ, WQ + 1, ... that their first steps have landed: vector loads complete in order, so
+// wave WQ's copies are done once no more than the copies of the waves after it are outstanding (a wave never has more than
+// 63 outstanding: a larger bound is already met).
+template <int NLD, int NW, int WQ> struct QsLanded {
+    static __device__ __forceinline__ void tell(volatile uint32_t *flags, int lane) {
+        constexpr int after = NLD * (NW - 1 - WQ) > 63 ? 63 : NLD * (NW - 1 - WQ);
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(after) : "memory");
+        if (lane == 0) flags[WQ] = 1u;
+        if constexpr (WQ + 1 < NW) QsLanded<NLD, NW, WQ + 1>::tell(flags, lane);
+    }
+};
+
 // PROD: the workgroup has one more wave, a producer, that requests the first step of all NW working waves at once and does
 // nothing else.  A wave that has asked for more than the memory pipeline takes is stopped at its next copy, so a working
 // wave can only ask for a few copies before its activation prologue; with rows of several spans per wave that prologue is
@@ -667,6 +679,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     __shared__ __align__(16) uint8_t act[SA::BYTES];
     __shared__ __align__(16) float red[32];                // [0, 16): sum(x^2) of the prologue, [16, 32): residual^2 of the epilogue
     static_assert(NW == 8 || NW == 16, "the fixed-order sums below read 8 or 16 slots");
+    static_assert(!PROD || NW == 8, "the producer's flags live in the sum slots that only sixteen waves use");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int k = g.k, n = g.n, bpr = g.bpr;
@@ -687,14 +700,20 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         for (int j = 0; j < SF::NLD; j++)
             if (j >= j0 && j < j1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(slots + wq * SLOT + j * 1024), 16, lane * 16, j * 1024, 0, 0);
     };
+    // red[8, 16) (unused with eight working waves): one flag per working wave, set by the producer when the wave's first
+    // step has landed.  The producer clears them before the barrier that opens the steps and sets them after it.
+    volatile uint32_t *landed = (volatile uint32_t *)&red[8];
     if (PROD && wv == NW) {
-        // the producer wave: every working wave's first step, then the workgroup's barriers (one with PRO_NORM_SPLIT, the
-        // one that opens the steps, one with the residual epilogues), the second of them once the copies have landed
+        // the producer wave: every working wave's first step, the workgroup's barriers (one with PRO_NORM_SPLIT, the one
+        // that opens the steps, one with the residual epilogues), and between them a word to each wave as its step lands,
+        // so that the first waves ask for their second step while the first steps of the last ones are still arriving
+        if (lane < NW) landed[lane] = 0u;
 #pragma unroll 1
         for (int wq = 0; wq < NW; wq++) issue_for(wq, 0, 0, SF::NLD);
         if (PRO == PRO_NORM_SPLIT) asm volatile("s_barrier" ::: "memory");
-        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        if (RESID) asm volatile("s_barrier" ::: "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        QsLanded<SF::NLD, NW, 0>::tell(landed, lane);
+        if (RESID) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         return;
     }
 
@@ -808,6 +827,11 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     float ssq = 0.0f;
 
     float gate = 0.0f;
+    if (PROD) {
+        // the wave's first step is the producer's: wait for its word (every wave of the workgroup is resident, and the
+        // producer waits for nothing but its own copies)
+        while (landed[wv] == 0u) __builtin_amdgcn_s_sleep(1);
+    }
     for (int t = 0; t < SUBS * my; t++) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's copies have landed
         const int step = step0 + (PAIR ? t >> 1 : t) * sstride;
