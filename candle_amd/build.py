@@ -6,7 +6,9 @@
 hipcc cross-compiles for gfx950 without a GPU present.  Flags:
   -ffp-contract=off   the quantizers and the dequantizer must round exactly like the scalar CPU code
                       (kernels that want an FMA call fmaf explicitly);
-  -packed-fp32-ops    disabled: hipcc must not form packed-f32 instructions from scalar float code.
+  -packed-fp32-ops    disabled: hipcc must not form packed-f32 instructions from scalar float code;
+  -amdgpu-kernarg-preload-count=14   the first fourteen dwords of scalar kernel arguments are placed in SGPRs at wave
+                      launch (kernels keep an entry that loads them for firmware without the feature).
 """
 from __future__ import annotations
 
@@ -30,6 +32,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
 ]
 

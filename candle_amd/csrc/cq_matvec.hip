@@ -976,6 +976,33 @@ __global__ __launch_bounds__((QS_NW + (PROD ? 1 : 0)) * 64) void qms_kernel(QsAr
     qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP, PROD>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
 }
 
+// The same kernel with its argument block handed over as fourteen 32-bit scalars (every block of at most 56 bytes): scalar
+// arguments can be placed in SGPRs when the wave is launched (the build asks for that), and the kernel then starts without
+// the trip to memory for its arguments.
+#define CQ_DW14_PARAMS uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t a4, uint32_t a5, uint32_t a6, uint32_t a7, uint32_t a8, \
+                       uint32_t a9, uint32_t a10, uint32_t a11, uint32_t a12, uint32_t a13
+#define CQ_DW14_LIST a0, a1, a2, a3, a4, a5, a6, a7, a8, a9, a10, a11, a12, a13
+struct Dwords14 { uint32_t d[14]; };
+template <typename A> Dwords14 to_dwords14(const A &a) {
+    static_assert(sizeof(A) <= 56, "fourteen dwords");
+    Dwords14 r{};
+    __builtin_memcpy(r.d, &a, sizeof(A));
+    return r;
+}
+template <typename A> __device__ __forceinline__ A from_dwords14(CQ_DW14_PARAMS) {
+    const uint32_t d[14] = {CQ_DW14_LIST};
+    A a;
+    __builtin_memcpy(&a, d, sizeof(A));
+    return a;
+}
+template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP, bool PROD>
+__global__ __launch_bounds__((QS_NW + (PROD ? 1 : 0)) * 64) void qms_kernel_dw(CQ_DW14_PARAMS) {
+    const QsArgs<PRO, EPI> a = from_dwords14<QsArgs<PRO, EPI>>(CQ_DW14_LIST);
+    const uint8_t *w; const float *x; void *dst; StreamGeom g; Fuse fz;
+    qs_unpack<DT, PRO, EPI>(a, w, x, dst, g, fz);
+    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP, PROD>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
+}
+
 // ---- two activation rows on the streaming kernel -------------------------------------------------------------
 // QMatMul::forward for two f32 rows (no prologue, no epilogue): the same stream of weight steps as qms_body; a lane keeps
 // the 256 activations of its super-block for both rows and takes two dots from every block it reads.  The weights are
@@ -1085,8 +1112,12 @@ struct Qs2Args {
     int wb_off16;             // (wb - wa) / 16
     int dstb_off;             // dstb - dsta, in floats
 };
+// The arguments are scalars, ordered by first use, so that the fourteen dwords placed in SGPRs at wave launch are the ones
+// the first loads need; the output pointer, needed last, is read from the argument block.
 template <int DTA, int DTB, int NW, int XS, int MAXB, bool SINGLE, int PRO, bool SB>
-__global__ __launch_bounds__(NW * 64) void qms2_kernel(Qs2Args a) {
+__global__ __launch_bounds__(NW * 64) void qms2_kernel(const uint8_t *a_wa, const float *a_x, const float *a_aux, const float *a_extra, int a_na, int a_nb,
+                                                       uint32_t a_meta, int a_wb_off16, float a_eps, int a_dstb_off, float *a_dsta) {
+    const Qs2Args a{a_wa, a_x, a_aux, a_extra, a_dsta, a_na, a_nb, a_meta, a_eps, a_wb_off16, a_dstb_off};
     const int blocks_a = (a.meta >> 8) & 255, blocks_b = (a.meta >> 16) & 255, bpr = a.meta & 255;
     Fuse fz{a.aux, PRO == PRO_NORM ? a.extra : nullptr, a.eps, nullptr, nullptr, 0, 0, 0, nullptr, nullptr, 0, PRO == PRO_NORM_SPLIT ? a.extra : nullptr,
             (int)(a.meta >> 24)};
@@ -1155,14 +1186,27 @@ int launch_stream_xs(const void *w, const float *x, void *dst, const StreamGeom 
     if (lds_bytes + StreamAct<MAXB>::BYTES + 256 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
     // rows of more than two spans per wave get the producer wave
     constexpr bool PROD = XS > 2;
-    auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI, MSP, PROD>;
-    if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return (int)e;
-    }
     const int groups = qs_groups(g.total_steps);
     if (fz.pair_off % 16 || fz.n_planes > 15 || fz.splits > 63 || g.dst_dtype > 255) return CQ_ERR_RANGE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(64 * (QS_NW + (PROD ? 1 : 0))), lds_bytes, s, qs_pack<DT, PRO, EPI>(w, x, dst, g, fz));
+    const dim3 grid((unsigned)groups), block(64 * (QS_NW + (PROD ? 1 : 0)));
+    const QsArgs<PRO, EPI> a = qs_pack<DT, PRO, EPI>(w, x, dst, g, fz);
+    if constexpr (sizeof(QsArgs<PRO, EPI>) <= 56) {
+        auto kern = qms_kernel_dw<DT, XS, MAXB, PRO, EPI, MSP, PROD>;
+        if (lds_bytes > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return (int)e;
+        }
+        const Dwords14 r = to_dwords14(a);
+        hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, r.d[0], r.d[1], r.d[2], r.d[3], r.d[4], r.d[5], r.d[6], r.d[7], r.d[8], r.d[9], r.d[10], r.d[11],
+                           r.d[12], r.d[13]);
+    } else {
+        auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI, MSP, PROD>;
+        if (lds_bytes > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return (int)e;
+        }
+        hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, a);
+    }
     return (int)hipGetLastError();
 }
 
@@ -1587,7 +1631,7 @@ int launch_pair_stream_xs(const void *wa, float *dsta, const void *wb, int64_t n
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
             if (e != hipSuccess) return (int)e;
         }
-        hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, a);
+        hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, a.wa, a.x, a.aux, a.extra, a.na, a.nb, a.meta, a.wb_off16, a.eps, a.dstb_off, a.dsta);
         return (int)hipGetLastError();
     };
     if constexpr (qs_streams(DTB)) {

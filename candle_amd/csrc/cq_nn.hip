@@ -619,13 +619,14 @@ __host__ __device__ inline int64_t attd_split_keys(int64_t max_kv_len) { return 
 __host__ __device__ inline int64_t attd_splits(int64_t max_kv_len) { const int64_t sk = attd_split_keys(max_kv_len); return (max_kv_len + sk - 1) / sk; }
 
 template <int HD, int G, int NW, int SPLIT>
-__global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const float *__restrict__ q, const float *__restrict__ k_new,
-                                                                      const float *__restrict__ v_new, float *k_cache, float *v_cache,
-                                                                      const float *__restrict__ cos_t, const float *__restrict__ sin_t,
-                                                                      float *__restrict__ part, const int32_t *__restrict__ pos_dev, int pos0,
-                                                                      int ctx, float scale, int splits, const u32x4 *__restrict__ pf,
+__global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__restrict__ pos_dev, const float *__restrict__ q, float *k_cache,
+                                                                      float *v_cache, const float *__restrict__ cos_t,
+                                                                      const float *__restrict__ sin_t, int pos0, int splits,
+                                                                      const float *__restrict__ k_new, const float *__restrict__ v_new,
+                                                                      float *__restrict__ part, int ctx, float scale, const u32x4 *__restrict__ pf,
                                                                       int64_t pf_chunks, uint32_t *__restrict__ pf_sink, float *__restrict__ out,
                                                                       int *__restrict__ counters) {
+    // (parameter order: the fourteen dwords that sit in SGPRs when the wave starts are what the first loads need)
     if ((int)blockIdx.y >= splits) {
         // Workgroups beyond the attention splits only read: they pull the weights the following kernels will stream
         // (attention_wo, feed_forward_w1 / w3) through the memory-side cache while this latency-bound kernel leaves
@@ -1337,12 +1338,12 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     hipStream_t s = (hipStream_t)stream;
 #define CQ_ATTD(HH, GG)                                                                                                                   \
     if (fine)                                                                                                                             \
-        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 8, 64>), grid, dim3(64 * 8), 0, s, q_dev, k_new_dev, v_new_dev, k_cache_dev, v_cache_dev, \
-                           cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits, (const u32x4 *)prefetch_dev, pf_chunks, \
+        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 8, 64>), grid, dim3(64 * 8), 0, s, pos_dev, q_dev, k_cache_dev, v_cache_dev, cos_dev, sin_dev, \
+                           (int)pos, (int)splits, k_new_dev, v_new_dev, part, (int)ctx, scale, (const u32x4 *)prefetch_dev, pf_chunks,       \
                            (uint32_t *)nullptr, out_dev, counters);                                                                       \
     else                                                                                                                                  \
-        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 16, 128>), grid, dim3(64 * 16), 0, s, q_dev, k_new_dev, v_new_dev, k_cache_dev,      \
-                           v_cache_dev, cos_dev, sin_dev, part, pos_dev, (int)pos, (int)ctx, scale, (int)splits, (const u32x4 *)prefetch_dev, \
+        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 16, 128>), grid, dim3(64 * 16), 0, s, pos_dev, q_dev, k_cache_dev, v_cache_dev, cos_dev,    \
+                           sin_dev, (int)pos, (int)splits, k_new_dev, v_new_dev, part, (int)ctx, scale, (const u32x4 *)prefetch_dev,          \
                            pf_chunks, (uint32_t *)nullptr, out_dev, counters)
     if (head_dim == 128) {
         switch (G) {
