@@ -68,6 +68,7 @@ SIGNATURES = {
     "cq_nn_silu_mul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "cq_nn_qmatmul_swiglu_rows": (_int, [_int, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_nn_argmax": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "cq_nn_argmax_embed": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
 }
 
 _lib = None

@@ -1014,7 +1014,8 @@ struct QsRowsArgs {
     int stride_dst;           // elements between the two output rows
 };
 template <int DT, int XS, int MAXB>
-__global__ __launch_bounds__(QS_NW * 64) void qms_rows2_kernel(QsRowsArgs a) {
+__global__ __launch_bounds__(QS_NW * 64) void qms_rows2_kernel(const uint8_t *a_w, const float *a_x, void *a_dst, int a_n, uint32_t a_meta, int a_stride_dst) {
+    const QsRowsArgs a{a_w, a_x, a_dst, a_n, a_meta, a_stride_dst};       // scalar arguments: in SGPRs when the wave starts
     typedef StreamFmt<DT> SF;
     typedef StreamAct<MAXB> SA;
     constexpr int NB = 2, NW = QS_NW, PRE = 4, SLOT = SF::NLD * 1024;
@@ -1259,7 +1260,7 @@ int launch_stream_rows2_xs(const void *w, const float *x, void *dst, const Strea
     }
     if (stride_dst > 0x7fffffffLL || g.dst_dtype > 255) return CQ_ERR_RANGE;
     QsRowsArgs a{(const uint8_t *)w, x, dst, g.n, (uint32_t)g.bpr | ((uint32_t)g.dst_dtype << 8), (int)stride_dst};
-    hipLaunchKernelGGL(kern, dim3((unsigned)qs_groups(g.total_steps)), dim3(64 * QS_NW), lds_bytes, s, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)qs_groups(g.total_steps)), dim3(64 * QS_NW), lds_bytes, s, a.w, a.x, a.dst, a.n, a.meta, a.stride_dst);
     return (int)hipGetLastError();
 }
 

@@ -949,6 +949,57 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float *__restric
     }
 }
 
+// The same last stage followed by the embedding lookup of the chosen token (embedding_kernel for one row, with its partial
+// sums of squares): the next decode step finds its input row in place and starts with its first matvec.
+__global__ __launch_bounds__(256) void argmax_final_embed_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int parts,
+                                                                 int32_t *__restrict__ token_out, int32_t *__restrict__ history,
+                                                                 int32_t *__restrict__ counter, int32_t *__restrict__ pos_dev,
+                                                                 const float *__restrict__ table, float *__restrict__ out, int dim, int64_t vocab,
+                                                                 float *__restrict__ partials) {
+    __shared__ float red[4];
+    __shared__ int s_tok;
+    if (threadIdx.x < 64) {
+        float best = -INFINITY;
+        int idx = 0x7fffffff;
+        for (int i = threadIdx.x; i < parts; i += 64) {
+            const float v = pv[i];
+            const int j = pi[i];
+            if (j != 0x7fffffff && (idx == 0x7fffffff || v > best || (v == best && j < idx))) { best = v; idx = j; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, 64);
+            const int oi = __shfl_xor(idx, o, 64);
+            if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) { best = ov; idx = oi; }
+        }
+        if (threadIdx.x == 0) {
+            s_tok = idx;
+            token_out[0] = idx;
+            if (history && counter) history[counter[0]] = idx;
+            if (counter) counter[0] += 1;
+            if (pos_dev) pos_dev[0] += 1;
+        }
+    }
+    __syncthreads();
+    const int64_t id = s_tok;
+    const bool ok = id >= 0 && id < vocab;
+    const float4 *src = reinterpret_cast<const float4 *>(table + (ok ? id : 0) * dim);
+    float4 *dst = reinterpret_cast<float4 *>(out);
+    float acc = 0.0f;
+    for (int i = threadIdx.x; i < dim / 4; i += 256) {
+        const float4 v = ok ? src[i] : float4{0.f, 0.f, 0.f, 0.f};
+        dst[i] = v;
+        acc += v.x * v.x;
+        acc += v.y * v.y;
+        acc += v.z * v.z;
+        acc += v.w * v.w;
+    }
+    if (partials) {                       // uniform branch
+        const float t = block_sum_256(acc, red);
+        partials[threadIdx.x] = threadIdx.x == 0 ? t : 0.0f;      // 256 threads == CQ_NN_PARTIALS slots
+    }
+}
+
 // ---- MoE routing around the grouped expert matmuls (FusedMoeGGUF::forward, candle-transformers/src/fused_moe.rs:222-301) ----
 constexpr int ROUTE_MAX_EXPERTS = 1024, ROUTE_MAX_TOPK = 64;
 
@@ -1396,6 +1447,23 @@ int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int
     }
     hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits_dev, (int)n, token_out_dev, history_dev, counter_dev,
                        pos_dev);
+    return (int)hipGetLastError();
+}
+
+int cq_nn_argmax_embed(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
+                       void *workspace_dev, const float *table_dev, float *out_dev, int64_t dim, int64_t vocab, float *sumsq_partials_dev,
+                       void *stream) {
+    if (n <= 0 || dim <= 0 || dim % 4 || vocab <= 0) return CQ_ERR_SHAPE;
+    if (!logits_dev || !token_out_dev || !workspace_dev || !table_dev || !out_dev) return CQ_ERR_NULL;
+    if (n > 0x7fffffffLL || dim > 0x7fffffffLL) return CQ_ERR_RANGE;
+    if (misaligned(workspace_dev, 4) || misaligned(table_dev, 16) || misaligned(out_dev, 16)) return CQ_ERR_ALIGN;
+    const int chunk = (int)((n + ARGMAX_PARTS - 1) / ARGMAX_PARTS);
+    const int parts = (int)((n + chunk - 1) / chunk);
+    float *pv = (float *)workspace_dev;
+    int *pi = (int *)workspace_dev + ARGMAX_PARTS;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(parts), dim3(256), 0, (hipStream_t)stream, logits_dev, (int)n, chunk, pv, pi);
+    hipLaunchKernelGGL(argmax_final_embed_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float *)pv, (const int *)pi, parts, token_out_dev,
+                       history_dev, counter_dev, pos_dev, table_dev, out_dev, (int)dim, vocab, sumsq_partials_dev);
     return (int)hipGetLastError();
 }
 

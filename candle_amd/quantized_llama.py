@@ -323,8 +323,10 @@ class ModelWeights:
         _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(int(w.dtype), w.ptr, src.data_ptr(), 0, dst_ptr, 0, rows, w.k, n,
                                                               self.ws.data_ptr(), self.ws.numel(), sp))
 
-    def _enqueue(self, ids_ptr: int, rows: int, pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
-        """All kernels of ModelWeights::forward (quantized_llama.rs:568-596) for `rows` new tokens; logits of the last."""
+    def _enqueue(self, ids_ptr: Optional[int], rows: int, pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
+        """All kernels of ModelWeights::forward (quantized_llama.rs:568-596) for `rows` new tokens; logits of the last.
+        ids_ptr None (fused single-token step only): the token's embedding row and its partial sums of squares are already in
+        self.x / self.partials (cq_nn_argmax_embed of the previous step put them there)."""
         cfg, L = self.cfg, self.L
         qd, kvd = cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim
         scale = float(np.float32(1.0 / math.sqrt(cfg.head_dim)))
@@ -332,6 +334,8 @@ class ModelWeights:
         x, xn, qk, v, att, delta, gu, h = self.x, self.xn, self.qk, self.v, self.att, self.delta, self.gu, self.h
         if rows == 1 and self.fuse_decode and self.L.cq_nn_attention_decode_splits(max_kv_len) > 0:
             return self._enqueue_decode_fused(ids_ptr, pos, pos_dev_ptr, max_kv_len, sp)
+        if ids_ptr is None:
+            raise ValueError("a step without token ids needs the fused single-token path")
         ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), rows, cfg.hidden, cfg.vocab, None, sp))
         for li, lw in enumerate(self.layers):
             w = lw.w
@@ -383,7 +387,7 @@ class ModelWeights:
                                              cfg.hidden, cfg.rms_eps, sp))
         self._mm(self.output, cfg.vocab, xn, self.logits.data_ptr(), 1, sp)
 
-    def _enqueue_decode_fused(self, ids_ptr: int, pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
+    def _enqueue_decode_fused(self, ids_ptr: Optional[int], pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
         """The same single-token step with the glue folded into the matvec kernels: the residual add is the
         epilogue of attention_wo / feed_forward_w2 (which also leaves sum(x^2) as partial sums), rms_norm and
         silu(w1 x) * w3 x are the prologues of the matvecs that consume them.  A long feed_forward_w2 row is split
@@ -401,7 +405,8 @@ class ModelWeights:
         all_full = all(w.dtype in full for lw in self.layers for w in lw.w.values()) and self.output.dtype in full
         cur = self.x.data_ptr()                                    # the residual row
         pending = 0                                                # planes of the previous feed_forward_w2 not yet added to it
-        ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, cur, 1, cfg.hidden, cfg.vocab, part.data_ptr(), sp))
+        if ids_ptr is not None:
+            ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, cur, 1, cfg.hidden, cfg.vocab, part.data_ptr(), sp))
 
         def one_step(w: _W) -> bool:
             return w.k <= (4096 if w.dtype in kq + (GgmlDType.Q2K, GgmlDType.Q3K) else 2048)
@@ -499,12 +504,29 @@ class ModelWeights:
         return self.logits.clone()
 
     # ------------------------------------------------------------------------------------------ greedy decode
+    def _chain_embedding(self, max_kv_len: int) -> bool:
+        """Whether the greedy steps hand the next token's embedding row over in place (the fused single-token path)."""
+        return bool(self.fuse_decode and self.L.cq_nn_attention_decode_splits(max_kv_len) > 0)
+
+    def _argmax_dev(self, logits_ptr: int, embed: bool, sp) -> None:
+        """Sampling::ArgMax into token_dev / history_dev, the position advanced; with `embed` the chosen token's embedding row
+        and its partial sums of squares go to self.x / self.partials in the same launch."""
+        L, cfg = self.L, self.cfg
+        if embed:
+            _lib.check("cq_nn_argmax_embed", L.cq_nn_argmax_embed(logits_ptr, cfg.vocab, self.token_dev.data_ptr(), self.history_dev.data_ptr(),
+                                                                 self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), self.argmax_ws.data_ptr(),
+                                                                 self.tok_embeddings.data_ptr(), self.x.data_ptr(), cfg.hidden, cfg.vocab,
+                                                                 self.partials.data_ptr(), sp))
+        else:
+            _lib.check("cq_nn_argmax", L.cq_nn_argmax(logits_ptr, cfg.vocab, self.token_dev.data_ptr(), self.history_dev.data_ptr(),
+                                                     self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), self.argmax_ws.data_ptr(), sp))
+
     def _decode_step_dev(self, max_kv_len: int, sp) -> None:
-        """One greedy step driven entirely from device state: token_dev at position pos_dev -> next token_dev, pos_dev + 1."""
-        self._enqueue(self.token_dev.data_ptr(), 1, 0, self.pos_dev.data_ptr(), max_kv_len, sp)
-        _lib.check("cq_nn_argmax", self.L.cq_nn_argmax(self.logits.data_ptr(), self.cfg.vocab, self.token_dev.data_ptr(),
-                                                       self.history_dev.data_ptr(), self.counter_dev.data_ptr(), self.pos_dev.data_ptr(),
-                                                       self.argmax_ws.data_ptr(), sp))
+        """One greedy step driven entirely from device state: token_dev at position pos_dev -> next token_dev, pos_dev + 1.
+        On the fused path the step starts from the embedding row the previous arg-max left in self.x and leaves the next one."""
+        chain = self._chain_embedding(max_kv_len)
+        self._enqueue(None if chain else self.token_dev.data_ptr(), 1, 0, self.pos_dev.data_ptr(), max_kv_len, sp)
+        self._argmax_dev(self.logits.data_ptr(), chain, sp)
 
     def generate_greedy(self, prompt: Sequence[int], n_new: int, use_graph: bool = True) -> dict:
         """The loop of candle-examples/examples/quantized/main.rs:616-690 with temperature <= 0 (Sampling::ArgMax):
@@ -521,21 +543,19 @@ class ModelWeights:
         stream = torch.cuda.current_stream(dev)
         self.counter_dev.zero_()
         self.pos_dev.fill_(len(prompt) - 1)       # argmax advances it to the position of the token it emits
-        _lib.check("cq_nn_argmax", self.L.cq_nn_argmax(logits.data_ptr(), cfg.vocab, self.token_dev.data_ptr(), self.history_dev.data_ptr(),
-                                                       self.counter_dev.data_ptr(), self.pos_dev.data_ptr(), self.argmax_ws.data_ptr(),
-                                                       stream.cuda_stream))
+        steps = n_new - 1
+        max_kv = len(prompt) + n_new
+        self._argmax_dev(logits.data_ptr(), steps > 0 and self._chain_embedding(max_kv), stream.cuda_stream)
         torch.cuda.synchronize(dev)
         t1 = time.perf_counter()
         prompt_seconds = t1 - t0
-        steps = n_new - 1
-        max_kv = len(prompt) + n_new
         if steps > 0:
             if use_graph:
                 key = max_kv
                 if self._graph is None or self._graph_key != key:
                     side = torch.cuda.Stream(device=dev)
                     # capture must not disturb the live decode state: save and restore it around the warm-up run
-                    saved = (self.token_dev.clone(), self.pos_dev.clone(), self.counter_dev.clone())
+                    saved = (self.token_dev.clone(), self.pos_dev.clone(), self.counter_dev.clone(), self.x[:1].clone(), self.partials.clone())
                     with torch.cuda.stream(side):
                         self._decode_step_dev(max_kv, side.cuda_stream)
                         side.synchronize()
@@ -544,6 +564,7 @@ class ModelWeights:
                             self._decode_step_dev(max_kv, torch.cuda.current_stream(dev).cuda_stream)
                     torch.cuda.synchronize(dev)
                     self.token_dev.copy_(saved[0]); self.pos_dev.copy_(saved[1]); self.counter_dev.copy_(saved[2])
+                    self.x[:1].copy_(saved[3]); self.partials.copy_(saved[4])
                     torch.cuda.synchronize(dev)
                     self._graph, self._graph_key = g, key
                 t1 = time.perf_counter()

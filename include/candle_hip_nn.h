@@ -157,6 +157,12 @@ int cq_nn_qmatmul_residual_attn_merge(int w_dtype, const void *w_dev, const floa
 #define CQ_NN_ARGMAX_WORKSPACE 1024
 int cq_nn_argmax(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
                  void *workspace_dev, void *stream);
+/* cq_nn_argmax (workspace_dev required) followed, in its last kernel, by the embedding lookup of the chosen token
+ * (cq_nn_embedding for one row: out_dev[0 .. dim) = table_dev[token, :], sumsq_partials_dev as there), so that a greedy
+ * decode loop (main.rs:616-690) finds the next step's input row in place and the step starts with its first matmul. */
+int cq_nn_argmax_embed(const float *logits_dev, int64_t n, int32_t *token_out_dev, int32_t *history_dev, int32_t *counter_dev, int32_t *pos_dev,
+                       void *workspace_dev, const float *table_dev, float *out_dev, int64_t dim, int64_t vocab, float *sumsq_partials_dev,
+                       void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Routing glue of FusedMoeGGUF::forward (candle-transformers/src/fused_moe.rs:222-301) around the three

@@ -302,6 +302,45 @@ def test_argmax_first_of_ties_and_bookkeeping():
     assert tok.item() == 0
 
 
+@pytest.mark.parametrize("n,dim", [(128256, 4096), (9000, 64)])
+def test_argmax_embed_equals_argmax_then_embedding(n, dim):
+    """The arg-max that also looks up the chosen token's embedding row: token, bookkeeping, row and partial sums of squares
+    equal cq_nn_argmax followed by cq_nn_embedding, bit for bit; an out-of-range vocabulary gives a zero row."""
+    table = normal(31, (n, dim), 1.0) if dim == 64 else None
+    tab = dev(table) if table is not None else torch.randn((n, dim), device="cuda", generator=torch.Generator(device="cuda").manual_seed(5))
+    ws = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    for trial, where in enumerate([0, n - 1, 4242]):
+        lg = normal(70 + trial, (n,), 1.0)
+        lg[where] = 77.0
+        if where == 4242:
+            lg[8000] = 77.0                                  # a tie: the lower index wins
+        lgd = dev(lg)
+        tok = [torch.zeros(1, dtype=torch.int32, device="cuda") for _ in range(2)]
+        hist = [torch.full((4,), -1, dtype=torch.int32, device="cuda") for _ in range(2)]
+        cnt = [torch.tensor([1], dtype=torch.int32, device="cuda") for _ in range(2)]
+        pos = [torch.tensor([9], dtype=torch.int32, device="cuda") for _ in range(2)]
+        row = [torch.full((dim,), 3.0, device="cuda") for _ in range(2)]
+        part = [torch.full((256,), 5.0, device="cuda") for _ in range(2)]
+        ok(L().cq_nn_argmax(lgd.data_ptr(), n, tok[0].data_ptr(), hist[0].data_ptr(), cnt[0].data_ptr(), pos[0].data_ptr(), ws.data_ptr(), None))
+        ok(L().cq_nn_embedding(tab.data_ptr(), tok[0].data_ptr(), row[0].data_ptr(), 1, dim, n, part[0].data_ptr(), None))
+        ok(L().cq_nn_argmax_embed(lgd.data_ptr(), n, tok[1].data_ptr(), hist[1].data_ptr(), cnt[1].data_ptr(), pos[1].data_ptr(), ws.data_ptr(),
+                                  tab.data_ptr(), row[1].data_ptr(), dim, n, part[1].data_ptr(), None))
+        torch.cuda.synchronize()
+        assert tok[0].item() == tok[1].item() == where
+        for a, b in ((hist[0], hist[1]), (cnt[0], cnt[1]), (pos[0], pos[1])):
+            assert torch.equal(a, b)
+        assert torch.equal(row[0].view(torch.int32), row[1].view(torch.int32)) and torch.equal(row[1], tab[where])
+        assert torch.equal(part[0].view(torch.int32), part[1].view(torch.int32))
+    # a table smaller than the logits row: tokens beyond it give a zero row, as cq_nn_embedding does
+    lg = normal(99, (n,), 1.0)
+    lg[n - 1] = 88.0
+    t1 = torch.zeros(1, dtype=torch.int32, device="cuda")
+    r1 = torch.full((dim,), 3.0, device="cuda")
+    ok(L().cq_nn_argmax_embed(dev(lg).data_ptr(), n, t1.data_ptr(), None, None, None, ws.data_ptr(), tab.data_ptr(), r1.data_ptr(), dim, n - 1, None, None))
+    assert t1.item() == n - 1 and bool((r1 == 0).all())
+    assert L().cq_nn_argmax_embed(dev(lg).data_ptr(), n, t1.data_ptr(), None, None, None, None, tab.data_ptr(), r1.data_ptr(), dim, n, None, None) == -4      # CQ_ERR_NULL: the workspace is required
+
+
 FUSE_DTYPES = [2, 8, 12, 13, 14]      # Q4_0, Q8_0, Q4_K, Q5_K, Q6_K
 
 
