@@ -583,8 +583,15 @@ def main():
             def plain_read(i, sp):
                 _lib.check("cq_bench_read", bench_lib.cq_bench_read(rot.weights[i % pool].data_ptr(), read_bytes, sink.data_ptr(), sp))
 
+            def plain_read_best(i, sp):
+                _lib.check("cq_bench_read_best", bench_lib.cq_bench_read_best(rot.weights[i % pool].data_ptr(), read_bytes, sink.data_ptr(), sp))
+
             read_us = rot.event_us(rot.capture(plain_read), args.steps, args.warmup)
-            extra.update({"plain_read_us": round(read_us, 3), "plain_read_GBps": round(read_bytes / (read_us * 1e-6) / 1e9, 1)})
+            best_us = rot.event_us(rot.capture(plain_read_best), args.steps, args.warmup)
+            # plain_read: 256 x 1024 threads like the matvec, four loads in flight; plain_read_best: the fastest shape of a sweep
+            extra.update({"plain_read_us": round(read_us, 3), "plain_read_GBps": round(read_bytes / (read_us * 1e-6) / 1e9, 1),
+                          "plain_read_best_shape_us": round(best_us, 3),
+                          "plain_read_best_shape_GBps": round(read_bytes / (best_us * 1e-6) / 1e9, 1)})
 
     traffic, traffic_commit = committed_traffic() if headline else (None, None)
     out = {

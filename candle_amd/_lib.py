@@ -112,6 +112,8 @@ def bench_lib():
         B = ctypes.CDLL(BENCH_LIB_PATH)
         B.cq_bench_read.restype = _int
         B.cq_bench_read.argtypes = [_vp, _i64, _vp, _vp]
+        B.cq_bench_read_best.restype = _int
+        B.cq_bench_read_best.argtypes = [_vp, _i64, _vp, _vp]
         _bench = B
     return _bench
 
