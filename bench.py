@@ -614,7 +614,8 @@ def main():
                    "n": n, "k": k, "batch": m},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "kernel": "%s<%s, %d row%s, fused f32 activations>" % (
-                         "qms_kernel" if args.wdtype in ("q4k", "q5k") and m == 1 else "qmv_kernel", fmt, m, "" if m == 1 else "s"),
+                         ("qms_kernel_dw" if m == 1 else "qms_rows2_kernel") if args.wdtype in ("q4k", "q5k", "q6k", "q4_0", "q8_0") and m <= 2
+                         else "qmv_kernel", fmt, m, "" if m == 1 else "s"),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_commit": traffic_commit, "avg_kernel_us": round(kern_us, 3), "median_us": stats["median_us"],
                      "p10_us": stats["p10_us"], "p90_us": stats["p90_us"], "timed_launches": stats["replays"] * pool,
