@@ -149,6 +149,22 @@ def test_prefill_k_not_multiple_of_256(dtype):
     assert rel_l2(forward(qmm, x), oracle.matmul(dtype, x, blocks, 48)) <= TIGHT
 
 
+@pytest.mark.parametrize("dtype", WDTYPES, ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("k", [6144, 8192, 14336, 16384])
+@pytest.mark.parametrize("n", [67, 203, 1031])
+def test_long_rows_ragged_on_the_streaming_kernel(dtype, k, n):
+    """One and two f32 rows of 24 / 32 / 56 / 64 super-blocks: the long-row launches of the streaming kernel (a producer wave asks
+    for the first step of every wave and tells each one when it has landed) with fewer steps than waves, steps that are not
+    whole cache lines (Q6_K rows of 24 or 56 blocks) and a last step that ends inside the tensor's last row."""
+    blocks, qmm = make_weight(dtype, n, k, seed=500 + dtype)
+    for batch in (1, 2):
+        x = normal(600 + batch, (batch, k), 1.0)
+        got = forward(qmm, x)
+        err = rel_l2(got, oracle.matmul(dtype, x, blocks, n))
+        assert err <= TOL and err <= TIGHT, f"batch {batch}: rel-L2 {err}"
+        assert np.array_equal(got, forward(qmm, x))          # and the same bits on a second call
+
+
 def test_batching_invariance_on_gpu():
     # quantized_tests.rs:224-259: stacking the same rows must not change their results
     blocks, qmm = make_weight(oracle.Q4K, 24, 512, seed=71)
