@@ -34,6 +34,8 @@ fn main() {
         let child = Command::new(&hipcc)
             .args(["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off"])
             .args(["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"])
+            // the first fourteen dwords of scalar kernel arguments arrive in SGPRs at wave launch
+            .args(["-mllvm", "-amdgpu-kernarg-preload-count=14"])
             .arg("-c")
             .arg(csrc.join(format!("{s}.hip")))
             .arg("-o")
