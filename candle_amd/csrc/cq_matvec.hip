@@ -639,27 +639,10 @@ __device__ __forceinline__ void qs_quantize(const float (&v)[NS][4], int span0, 
     }
 }
 
-// The producer wave tells working wave WQ, WQ + 1, ... that their first steps have landed: vector loads complete in order, so
-// wave WQ's copies are done once no more than the copies of the waves after it are outstanding (a wave never has more than
-// 63 outstanding: a larger bound is already met).
-template <int NLD, int NW, int WQ> struct QsLanded {
-    static __device__ __forceinline__ void tell(volatile uint32_t *flags, int lane) {
-        constexpr int after = NLD * (NW - 1 - WQ) > 63 ? 63 : NLD * (NW - 1 - WQ);
-        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(after) : "memory");
-        if (lane == 0) flags[WQ] = 1u;
-        if constexpr (WQ + 1 < NW) QsLanded<NLD, NW, WQ + 1>::tell(flags, lane);
-    }
-};
-
-// PROD: the workgroup has one more wave, a producer, that requests the first step of all NW working waves at once and does
-// nothing else.  A wave that has asked for more than the memory pipeline takes is stopped at its next copy, so a working
-// wave can only ask for a few copies before its activation prologue; with rows of several spans per wave that prologue is
-// long, and the weights would wait for it.  The producer can be stopped: nobody queues behind it.
-template <int DT, int NW, int XS, int MAXB, int PRO, int EPI, int MSP = MAXS, bool PROD = false>
+template <int DT, int NW, int XS, int MAXB, int PRO, int EPI, int MSP = MAXS>
 __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const float *__restrict__ x, void *__restrict__ dst, const StreamGeom &g,
                                          const Fuse &fz, const int block, const int nblocks) {
     typedef StreamFmt<DT> SF;
-    static_assert(!PROD || (PRO != PRO_MERGE && EPI != EPI_SWIGLU), "the producer wave serves the long-row launches only");
     typedef StreamAct<MAXB> SA;
     constexpr bool RESID = epi_is_resid(EPI);
     constexpr bool PAIR = EPI == EPI_SWIGLU;               // two weight rows per output row: a step is two sub-steps, gate rows then up rows
@@ -679,7 +662,6 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     __shared__ __align__(16) uint8_t act[SA::BYTES];
     __shared__ __align__(16) float red[32];                // [0, 16): sum(x^2) of the prologue, [16, 32): residual^2 of the epilogue
     static_assert(NW == 8 || NW == 16, "the fixed-order sums below read 8 or 16 slots");
-    static_assert(!PROD || NW == 8, "the producer's flags live in the sum slots that only sixteen waves use");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int k = g.k, n = g.n, bpr = g.bpr;
@@ -700,23 +682,6 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         for (int j = 0; j < SF::NLD; j++)
             if (j >= j0 && j < j1) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(slots + wq * SLOT + j * 1024), 16, lane * 16, j * 1024, 0, 0);
     };
-    // red[8, 16) (unused with eight working waves): one flag per working wave, set by the producer when the wave's first
-    // step has landed.  The producer clears them before the barrier that opens the steps and sets them after it.
-    volatile uint32_t *landed = (volatile uint32_t *)&red[8];
-    if (PROD && wv == NW) {
-        // the producer wave: every working wave's first step, the workgroup's barriers (one with PRO_NORM_SPLIT, the one
-        // that opens the steps, one with the residual epilogues), and between them a word to each wave as its step lands,
-        // so that the first waves ask for their second step while the first steps of the last ones are still arriving
-        if (lane < NW) landed[lane] = 0u;
-#pragma unroll 1
-        for (int wq = 0; wq < NW; wq++) issue_for(wq, 0, 0, SF::NLD);
-        if (PRO == PRO_NORM_SPLIT) asm volatile("s_barrier" ::: "memory");
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        QsLanded<SF::NLD, NW, 0>::tell(landed, lane);
-        if (RESID) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        return;
-    }
-
     // 0. activation loads first (vector loads complete in order: what is asked for after the weights waits for them)
     f32x4 xt[XS], at[XS];
     float pp[NPART / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -745,12 +710,12 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     }
     asm volatile("" ::: "memory");
 
-    // 1. the wave's first step on its way into LDS (with a producer wave that is the producer's part)
+    // 1. the wave's first step on its way into LDS
     uint8_t *slot = slots + wv * SLOT;
     const int step0 = wv * nblocks + block;
     const int my = step0 < g.total_steps ? (g.total_steps - step0 + sstride - 1) / sstride : 0;
     auto issue = [&](int t, int j0, int j1) { issue_for(wv, t, j0, j1); };
-    if (!PROD) issue(0, 0, PRE);
+    issue(0, 0, PRE);
     asm volatile("" ::: "memory");
 
     // 2. activations -> LDS
@@ -801,7 +766,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     }
     qs_quantize<DT, XS>(xv, wv, NW, bpr, MAXB, lane, act, SA::AUX_OFF);
     asm volatile("" ::: "memory");
-    if (!PROD) issue(0, PRE, SF::NLD);
+    issue(0, PRE, SF::NLD);
     // a barrier without the fence of __syncthreads(): the fence would wait for the LDS copies in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
@@ -827,11 +792,6 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     float ssq = 0.0f;
 
     float gate = 0.0f;
-    if (PROD) {
-        // the wave's first step is the producer's: wait for its word (every wave of the workgroup is resident, and the
-        // producer waits for nothing but its own copies)
-        while (landed[wv] == 0u) __builtin_amdgcn_s_sleep(1);
-    }
     for (int t = 0; t < SUBS * my; t++) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's copies have landed
         const int step = step0 + (PAIR ? t >> 1 : t) * sstride;
@@ -967,13 +927,13 @@ __device__ __forceinline__ void qs_unpack(const QsArgs<PRO, EPI> &a, const uint8
     g.w_bytes = (int64_t)n * (bpr * StreamFmt<DT>::BB);
 }
 
-template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP, bool PROD>
-__global__ __launch_bounds__((QS_NW + (PROD ? 1 : 0)) * 64) void qms_kernel(QsArgs<PRO, EPI> a) {
+template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP>
+__global__ __launch_bounds__(QS_NW * 64) void qms_kernel(QsArgs<PRO, EPI> a) {
     const uint8_t *w; const float *x; void *dst; StreamGeom g; Fuse fz;
     qs_unpack<DT, PRO, EPI>(a, w, x, dst, g, fz);
     // the grid size is derived, not read: gridDim comes from the hidden arguments behind the explicit ones, and every
     // argument byte a kernel reads beyond the first 64 costs a second trip at its start
-    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP, PROD>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
+    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
 }
 
 // The same kernel with its argument block handed over as fourteen 32-bit scalars (every block of at most 56 bytes): scalar
@@ -995,12 +955,12 @@ template <typename A> __device__ __forceinline__ A from_dwords14(CQ_DW14_PARAMS)
     __builtin_memcpy(&a, d, sizeof(A));
     return a;
 }
-template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP, bool PROD>
-__global__ __launch_bounds__((QS_NW + (PROD ? 1 : 0)) * 64) void qms_kernel_dw(CQ_DW14_PARAMS) {
+template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP>
+__global__ __launch_bounds__(QS_NW * 64) void qms_kernel_dw(CQ_DW14_PARAMS) {
     const QsArgs<PRO, EPI> a = from_dwords14<QsArgs<PRO, EPI>>(CQ_DW14_LIST);
     const uint8_t *w; const float *x; void *dst; StreamGeom g; Fuse fz;
     qs_unpack<DT, PRO, EPI>(a, w, x, dst, g, fz);
-    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP, PROD>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
+    qms_body<DT, QS_NW, XS, MAXB, PRO, EPI, MSP>(w, x, dst, g, fz, blockIdx.x, qs_groups(g.total_steps));
 }
 
 // ---- two activation rows on the streaming kernel -------------------------------------------------------------
@@ -1185,14 +1145,12 @@ template <int DT, int XS, int MAXB, int PRO, int EPI, int MSP = 1>
 int launch_stream_xs(const void *w, const float *x, void *dst, const StreamGeom &g, hipStream_t s, const Fuse &fz) {
     const size_t lds_bytes = (size_t)QS_NW * StreamFmt<DT>::NLD * 1024;
     if (lds_bytes + StreamAct<MAXB>::BYTES + 256 > (size_t)LDS_BUDGET) return CQ_ERR_RANGE;
-    // rows of more than two spans per wave get the producer wave
-    constexpr bool PROD = XS > 2;
     const int groups = qs_groups(g.total_steps);
     if (fz.pair_off % 16 || fz.n_planes > 15 || fz.splits > 63 || g.dst_dtype > 255) return CQ_ERR_RANGE;
-    const dim3 grid((unsigned)groups), block(64 * (QS_NW + (PROD ? 1 : 0)));
+    const dim3 grid((unsigned)groups), block(64 * QS_NW);
     const QsArgs<PRO, EPI> a = qs_pack<DT, PRO, EPI>(w, x, dst, g, fz);
     if constexpr (sizeof(QsArgs<PRO, EPI>) <= 56) {
-        auto kern = qms_kernel_dw<DT, XS, MAXB, PRO, EPI, MSP, PROD>;
+        auto kern = qms_kernel_dw<DT, XS, MAXB, PRO, EPI, MSP>;
         if (lds_bytes > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
             if (e != hipSuccess) return (int)e;
@@ -1201,7 +1159,7 @@ int launch_stream_xs(const void *w, const float *x, void *dst, const StreamGeom 
         hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, r.d[0], r.d[1], r.d[2], r.d[3], r.d[4], r.d[5], r.d[6], r.d[7], r.d[8], r.d[9], r.d[10], r.d[11],
                            r.d[12], r.d[13]);
     } else {
-        auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI, MSP, PROD>;
+        auto kern = qms_kernel<DT, XS, MAXB, PRO, EPI, MSP>;
         if (lds_bytes > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
             if (e != hipSuccess) return (int)e;

@@ -153,8 +153,8 @@ def test_prefill_k_not_multiple_of_256(dtype):
 @pytest.mark.parametrize("k", [6144, 8192, 14336, 16384])
 @pytest.mark.parametrize("n", [67, 203, 1031])
 def test_long_rows_ragged_on_the_streaming_kernel(dtype, k, n):
-    """One and two f32 rows of 24 / 32 / 56 / 64 super-blocks: the long-row launches of the streaming kernel (a producer wave asks
-    for the first step of every wave and tells each one when it has landed) with fewer steps than waves, steps that are not
+    """One and two f32 rows of 24 / 32 / 56 / 64 super-blocks: the long-row launches of the streaming kernel (three to eight
+    activation spans per wave) with fewer steps than waves, steps that are not
     whole cache lines (Q6_K rows of 24 or 56 blocks) and a last step that ends inside the tensor's last row."""
     blocks, qmm = make_weight(dtype, n, k, seed=500 + dtype)
     for batch in (1, 2):
