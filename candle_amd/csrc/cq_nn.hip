@@ -620,13 +620,14 @@ __host__ __device__ inline int64_t attd_splits(int64_t max_kv_len) { const int64
 
 template <int HD, int G, int NW, int SPLIT>
 __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__restrict__ pos_dev, const float *__restrict__ q, float *k_cache,
-                                                                      float *v_cache, const float *__restrict__ cos_t,
-                                                                      const float *__restrict__ sin_t, int pos0, int splits,
+                                                                      const float *__restrict__ cos_t, const float *__restrict__ sin_t, int pos0,
+                                                                      int splits, int ctx, float scale, float *v_cache,
                                                                       const float *__restrict__ k_new, const float *__restrict__ v_new,
-                                                                      float *__restrict__ part, int ctx, float scale, const u32x4 *__restrict__ pf,
+                                                                      float *__restrict__ part, const u32x4 *__restrict__ pf,
                                                                       int64_t pf_chunks, uint32_t *__restrict__ pf_sink, float *__restrict__ out,
                                                                       int *__restrict__ counters) {
-    // (parameter order: the fourteen dwords that sit in SGPRs when the wave starts are what the first loads need)
+    // (parameter order: the fourteen dwords that sit in SGPRs when the wave starts are all that the key and query loads
+    // need, so that those go out without waiting for a scalar load: neither for further arguments nor for the position)
     if ((int)blockIdx.y >= splits) {
         // Workgroups beyond the attention splits only read: they pull the weights the following kernels will stream
         // (attention_wo, feed_forward_w1 / w3) through the memory-side cache while this latency-bound kernel leaves
@@ -645,49 +646,48 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
         if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
         return;
     }
-    constexpr int DPL = HD / 64, EPL = HD / 16, IT = SPLIT / (4 * NW), VU = SPLIT / NW;
-    __shared__ float sc[G * SPLIT];
-    __shared__ float red[NW * G * HD];
+    constexpr int DPL = HD / 64, EPL = HD / 16, IT = SPLIT / (4 * NW), VU = SPLIT / NW, QR = (G + 3) / 4;
+    __shared__ __align__(16) float sc[SPLIT * G];          // [key][query head]
+    __shared__ __align__(16) float red[NW * G * HD];
     __shared__ float ml[2 * G];
     const int kvh = blockIdx.x, sp = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const int p = min(pos0 + (pos_dev ? pos_dev[0] : 0), ctx - 1);
-    const int kv_len = p + 1;
+    const int p_raw = pos_dev ? pos_dev[0] : 0;             // on its way while the loads below go out
     const int j0 = sp * SPLIT;
-    const int cnt = min(kv_len - j0, SPLIT);
-    const int last = max(cnt - 1, 0);
     float *kb = k_cache + (int64_t)kvh * ctx * HD, *vb = v_cache + (int64_t)kvh * ctx * HD;
     const int sub = lane & 15, kq = lane >> 4;
 
     // ---- every load of the kernel, issued before any use ----
+    // What scoring needs goes first, and of that first what does not depend on the position: the split's key rows as they
+    // lie in the cache (rows beyond the position are read and masked later; the row of the position itself is replaced by
+    // the new key below) and the query heads.  A lane fetches its 16-dimension slice of one query head only (head kq of
+    // every four); the wave exchanges the rotated slices through LDS, a quarter of the load instructions of every lane
+    // fetching every head.
     f32x4 kd[IT][EPL / 4];
 #pragma unroll
     for (int it = 0; it < IT; it++) {
-        const int key = min((it * NW + wv) * 4 + kq, last);
-        const float *src = (j0 + key == p) ? k_new + kvh * HD + EPL * sub : kb + (int64_t)(j0 + key) * HD + EPL * sub;
+        const int row = min(j0 + (it * NW + wv) * 4 + kq, ctx - 1);
+        const float *src = kb + (int64_t)row * HD + EPL * sub;
 #pragma unroll
         for (int c = 0; c < EPL / 4; c++) kd[it][c] = reinterpret_cast<const f32x4 *>(src)[c];
     }
-    float vv[VU][DPL];
+    f32x4 qv[QR][EPL / 4];
 #pragma unroll
-    for (int u = 0; u < VU; u++) {
-        const int j = min(wv + NW * u, last);
-        const float *src = (j0 + j == p) ? v_new + kvh * HD + DPL * lane : vb + (int64_t)(j0 + j) * HD + DPL * lane;
-        if (DPL == 2) {
-            const float2 t = *reinterpret_cast<const float2 *>(src);
-            vv[u][0] = t.x; vv[u][DPL - 1] = t.y;
-        } else {
-#pragma unroll
-            for (int e = 0; e < DPL; e++) vv[u][e] = src[e];
-        }
-    }
-    f32x4 qf[G][EPL / 4];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
+    for (int r = 0; r < QR; r++) {
+        const int g = min(4 * r + kq, G - 1);
         const f32x4 *qr = reinterpret_cast<const f32x4 *>(q + (int64_t)(kvh * G + g) * HD + EPL * sub);
 #pragma unroll
-        for (int c = 0; c < EPL / 4; c++) qf[g][c] = qr[c];
+        for (int c = 0; c < EPL / 4; c++) qv[r][c] = qr[c];
     }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    // the arguments that did not arrive in registers, asked for here in one go (and waited for together with the position)
+    asm volatile("" ::"s"(v_cache), "s"(k_new), "s"(v_new), "s"(part));
+    const int p = min(pos0 + p_raw, ctx - 1);
+    const int kv_len = p + 1;
+    const int cnt = min(kv_len - j0, SPLIT);
+    const int last = max(cnt - 1, 0);
+    const bool has_p = p >= j0 && p < j0 + SPLIT;           // this split holds the new token (the same in every wave)
     // cos / sin of position p for this lane's EPL/2 pairs
     float cs[EPL / 2], sn[EPL / 2];
     if constexpr (EPL / 2 == 4) {
@@ -702,23 +702,67 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
             sn[c] = sin_t[(int64_t)p * (HD / 2) + (EPL / 2) * sub + c];
         }
     }
+    f32x4 kn[EPL / 4];
+#pragma unroll
+    for (int c = 0; c < EPL / 4; c++) kn[c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (has_p) {
+#pragma unroll
+        for (int c = 0; c < EPL / 4; c++) kn[c] = reinterpret_cast<const f32x4 *>(k_new + kvh * HD + EPL * sub)[c];
+    }
+    asm volatile("" ::: "memory");
+    // the values last: they are used after the softmax
+    float vv[VU][DPL];
+#pragma unroll
+    for (int u = 0; u < VU; u++) {
+        const int j = min(wv + NW * u, last);
+        const float *src = (j0 + j == p) ? v_new + kvh * HD + DPL * lane : vb + (int64_t)(j0 + j) * HD + DPL * lane;
+        if (DPL == 2) {
+            const float2 t = *reinterpret_cast<const float2 *>(src);
+            vv[u][0] = t.x; vv[u][DPL - 1] = t.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < DPL; e++) vv[u][e] = src[e];
+        }
+    }
+    // nothing that waits for data may be scheduled between the loads above: every one is requested before the first wait
+    __builtin_amdgcn_sched_barrier(0);
     auto rope4 = [&](f32x4 &v, int c) {       // two interleaved pairs (rotary_emb.rs:52-70)
         const float a = v.x * cs[2 * c] - v.y * sn[2 * c], b = v.x * sn[2 * c] + v.y * cs[2 * c];
         const float e = v.z * cs[2 * c + 1] - v.w * sn[2 * c + 1], f = v.z * sn[2 * c + 1] + v.w * cs[2 * c + 1];
         v = f32x4{a, b, e, f};
     };
+    // the lane's query slice rotated, then every head's slice back from the wave's own part of `red` (free until phase 3)
+    f32x4 qf[G][EPL / 4];
+    {
+        float *qx = red + wv * G * HD + EPL * sub;
 #pragma unroll
-    for (int g = 0; g < G; g++)
+        for (int r = 0; r < QR; r++) {
+            const int g = min(4 * r + kq, G - 1);         // G not a multiple of four: several lanes write the same head, the same values
 #pragma unroll
-        for (int c = 0; c < EPL / 4; c++) rope4(qf[g][c], c);
+            for (int c = 0; c < EPL / 4; c++) {
+                rope4(qv[r][c], c);
+                reinterpret_cast<f32x4 *>(qx + g * HD)[c] = qv[r][c];
+            }
+        }
+        // the wave reads what its own lanes wrote: LDS operations of a wave complete in order, the fences keep the compiler
+        // from moving the reads up
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int c = 0; c < EPL / 4; c++) qf[g][c] = reinterpret_cast<const f32x4 *>(qx + g * HD)[c];
+    }
 
-    // ---- phase 1: scores; the lanes holding the new key rotate it and append it to the cache ----
+    // ---- phase 1: scores; the lanes holding the new key take it from the projection, rotate it and append it to the cache ----
 #pragma unroll
     for (int it = 0; it < IT; it++) {
         const int key = (it * NW + wv) * 4 + kq;
         if (j0 + key == p) {
 #pragma unroll
             for (int c = 0; c < EPL / 4; c++) {
+                kd[it][c] = kn[c];
                 rope4(kd[it][c], c);
                 reinterpret_cast<f32x4 *>(kb + (int64_t)p * HD + EPL * sub)[c] = kd[it][c];
             }
@@ -734,7 +778,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
                 a += qf[g][c].w * kd[it][c].w;
             }
             a = row16_sum(a);
-            if (sub == 0) sc[g * SPLIT + key] = key < cnt ? a * scale : -INFINITY;
+            if (sub == 0) sc[key * G + g] = key < cnt ? a * scale : -INFINITY;
         }
     }
     __syncthreads();
@@ -745,7 +789,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
         float s[SPLIT / 64], m = -INFINITY;
 #pragma unroll
         for (int i = 0; i < SPLIT / 64; i++) {
-            s[i] = sc[g * SPLIT + lane + 64 * i];
+            s[i] = sc[(lane + 64 * i) * G + g];
             m = fmaxf(m, s[i]);
         }
         m = wave_max(m);
@@ -753,7 +797,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
 #pragma unroll
         for (int i = 0; i < SPLIT / 64; i++) {
             const float pr = (cnt > 0 && s[i] > -INFINITY) ? __expf(s[i] - m) : 0.0f;
-            sc[g * SPLIT + lane + 64 * i] = pr;
+            sc[(lane + 64 * i) * G + g] = pr;
             l += pr;
         }
         l = wave_sum(l);
@@ -762,6 +806,13 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
     __syncthreads();
 
     // ---- phase 3: p . v from registers; the wave holding the new value appends it ----
+    // every probability of the wave's keys read first (one LDS round trip), and no branch around the sums: the value of a
+    // key at or beyond cnt is replaced by zero (its probability is zero too, but what lies in the cache there need not be finite)
+    float pr[VU][G];
+#pragma unroll
+    for (int u = 0; u < VU; u++)
+#pragma unroll
+        for (int g = 0; g < G; g++) pr[u][g] = sc[(wv + NW * u) * G + g];
     float o[G][DPL];
 #pragma unroll
     for (int g = 0; g < G; g++)
@@ -769,18 +820,17 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
         for (int e = 0; e < DPL; e++) o[g][e] = 0.0f;
 #pragma unroll
     for (int u = 0; u < VU; u++) {
-        const int j = wv + NW * u;                    // < SPLIT; entries at or beyond cnt hold p = 0
+        const int j = wv + NW * u;                    // < SPLIT
         if (j0 + j == p) {
 #pragma unroll
             for (int e = 0; e < DPL; e++) vb[(int64_t)p * HD + DPL * lane + e] = vv[u][e];
         }
-        if (j < cnt) {                                // wave-uniform
+        const bool live = j < cnt;                    // wave-uniform
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                const float pr = sc[g * SPLIT + j];
+        for (int e = 0; e < DPL; e++) {
+            const float v = live ? vv[u][e] : 0.0f;
 #pragma unroll
-                for (int e = 0; e < DPL; e++) o[g][e] += pr * vv[u][e];
-            }
+            for (int g = 0; g < G; g++) o[g][e] += (live ? pr[u][g] : 0.0f) * v;
         }
     }
 #pragma unroll
@@ -1389,12 +1439,12 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     hipStream_t s = (hipStream_t)stream;
 #define CQ_ATTD(HH, GG)                                                                                                                   \
     if (fine)                                                                                                                             \
-        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 8, 64>), grid, dim3(64 * 8), 0, s, pos_dev, q_dev, k_cache_dev, v_cache_dev, cos_dev, sin_dev, \
-                           (int)pos, (int)splits, k_new_dev, v_new_dev, part, (int)ctx, scale, (const u32x4 *)prefetch_dev, pf_chunks,       \
+        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 8, 64>), grid, dim3(64 * 8), 0, s, pos_dev, q_dev, k_cache_dev, cos_dev, sin_dev, (int)pos, \
+                           (int)splits, (int)ctx, scale, v_cache_dev, k_new_dev, v_new_dev, part, (const u32x4 *)prefetch_dev, pf_chunks,   \
                            (uint32_t *)nullptr, out_dev, counters);                                                                       \
     else                                                                                                                                  \
-        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 16, 128>), grid, dim3(64 * 16), 0, s, pos_dev, q_dev, k_cache_dev, v_cache_dev, cos_dev,    \
-                           sin_dev, (int)pos, (int)splits, k_new_dev, v_new_dev, part, (int)ctx, scale, (const u32x4 *)prefetch_dev,          \
+        hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 16, 128>), grid, dim3(64 * 16), 0, s, pos_dev, q_dev, k_cache_dev, cos_dev, sin_dev,       \
+                           (int)pos, (int)splits, (int)ctx, scale, v_cache_dev, k_new_dev, v_new_dev, part, (const u32x4 *)prefetch_dev,     \
                            pf_chunks, (uint32_t *)nullptr, out_dev, counters)
     if (head_dim == 128) {
         switch (G) {
