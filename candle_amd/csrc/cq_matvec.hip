@@ -767,6 +767,12 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     qs_quantize<DT, XS>(xv, wv, NW, bpr, MAXB, lane, act, SA::AUX_OFF);
     asm volatile("" ::: "memory");
     issue(0, PRE, SF::NLD);
+    // The residual value of the wave's first row is asked for right behind its first step's copies (vector loads complete
+    // in order: it is there when they are); every later one travels in front of the next step's copies.  Asked for when
+    // its step begins, the last one of a wave would be waited for at the very end of the kernel, a memory trip long.
+    float rv_next = 0.0f;
+    if (RESID) rv_next = fz.resid[min(step0 * g.step_rows + (lane >> g.lp_shift), n - 1)];
+    asm volatile("" ::: "memory");
     // a barrier without the fence of __syncthreads(): the fence would wait for the LDS copies in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
@@ -797,19 +803,17 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
         const int step = step0 + (PAIR ? t >> 1 : t) * sstride;
         const int row = step * g.step_rows + rin;
         const bool store = last && row < n;
-        // the residual value (and the planes to add to it) travels in front of the next step's copies
-        float rv = 0.0f, pv[ME];
-        if (RESID) {
+        // the residual value was asked for a step ahead; the planes to add to it travel in front of the next step's copies
+        float rv = rv_next, pv[ME];
+        if (EPI == EPI_RESID_SPLIT) {
             const int rc = min(row, n - 1);
-            rv = fz.resid[rc];
-            if (EPI == EPI_RESID_SPLIT) {
 #pragma unroll
-                for (int sI = 0; sI < ME; sI++) pv[sI] = fz.planes[(int64_t)min(sI, fz.n_planes - 1) * n + rc];
-            }
+            for (int sI = 0; sI < ME; sI++) pv[sI] = fz.planes[(int64_t)min(sI, fz.n_planes - 1) * n + rc];
         }
         typename SF::Blk b0;
         SF::read(b0, slot + boff);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // every lane has its block in registers: the slot is free
+        if (RESID && t + 1 < my) rv_next = fz.resid[min(row + sstride * g.step_rows, n - 1)];
         issue(t + 1, 0, SF::NLD);
         asm volatile("" ::: "memory");
         float r = SF::dot(b0, areg, d8, aux1);
@@ -1593,7 +1597,9 @@ int launch_pair_stream_xs(const void *wa, float *dsta, const void *wb, int64_t n
         hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, a.wa, a.x, a.aux, a.extra, a.na, a.nb, a.meta, a.wb_off16, a.eps, a.dstb_off, a.dsta);
         return (int)hipGetLastError();
     };
-    if constexpr (qs_streams(DTB)) {
+    // (the sixteen-wave launch exists for a tensor B that does not stream)
+    if (sb && NW != QS_NW) return CQ_ERR_RANGE;
+    if constexpr (qs_streams(DTB) && NW == QS_NW) {
         if (sb) return go(qms2_kernel<DTA, DTB, NW, XS, MAXB, true, PRO, true>);
     }
     if (single) return go(qms2_kernel<DTA, DTB, NW, XS, MAXB, true, PRO, false>);
