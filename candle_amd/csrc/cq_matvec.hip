@@ -902,21 +902,31 @@ QsArgs<PRO, EPI> qs_pack(const void *w, const float *x, void *dst, const StreamG
     return a;
 }
 
+// A pointer rebuilt from integers (the fourteen-dword argument block) has no address space the compiler knows, and through
+// a plain pointer every access is a flat instruction.  Flat loads cannot be waited for by count: the wait for an
+// activation load becomes vmcnt(0), which also waits for every weight copy requested before it.  A round trip through
+// the global address space that the optimizer cannot see through (the empty asm) tells the compiler where the memory is.
+template <typename T> __device__ __forceinline__ T *qs_global(const void *p) {
+    auto gp = (__attribute__((address_space(1))) T *)p;
+    asm("" : "+s"(gp));
+    return (T *)gp;
+}
+
 template <int DT, int PRO, int EPI>
 __device__ __forceinline__ void qs_unpack(const QsArgs<PRO, EPI> &a, const uint8_t *&w, const float *&x, void *&dst, StreamGeom &g, Fuse &fz) {
     int np = 0;
-    w = (const uint8_t *)a.p[np++];
-    x = PRO != PRO_MERGE ? (const float *)a.p[np++] : nullptr;
-    fz.aux = PRO != PRO_NONE ? (const float *)a.p[np++] : nullptr;
-    fz.part_in = PRO == PRO_NORM ? (const float *)a.p[np++] : nullptr;
-    fz.planes = PRO == PRO_NORM_SPLIT ? (const float *)a.p[np++] : nullptr;
+    w = qs_global<const uint8_t>(a.p[np++]);
+    x = PRO != PRO_MERGE ? qs_global<const float>(a.p[np++]) : nullptr;
+    fz.aux = PRO != PRO_NONE ? qs_global<const float>(a.p[np++]) : nullptr;
+    fz.part_in = PRO == PRO_NORM ? qs_global<const float>(a.p[np++]) : nullptr;
+    fz.planes = PRO == PRO_NORM_SPLIT ? qs_global<const float>(a.p[np++]) : nullptr;
     dst = nullptr; fz.resid = nullptr; fz.part_out = nullptr;
     if (epi_is_resid(EPI)) {
-        fz.resid = (float *)a.p[np++];
-        fz.part_out = (float *)a.p[np++];
-        if (EPI == EPI_RESID_SPLIT) fz.planes = (const float *)a.p[np++];
+        fz.resid = qs_global<float>(a.p[np++]);
+        fz.part_out = qs_global<float>(a.p[np++]);
+        if (EPI == EPI_RESID_SPLIT) fz.planes = qs_global<const float>(a.p[np++]);
     } else {
-        dst = (void *)a.p[np++];
+        dst = qs_global<void>(a.p[np++]);
     }
     int ni = 0;
     const int n = a.i[ni++];
