@@ -719,7 +719,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     asm volatile("" ::: "memory");
     // With a norm prologue nothing of it may be scheduled in front of these copies: left to itself the compiler places the
     // whole sum of squares (which waits for the partial sums) before them, and the weights start a memory trip late.
-    // Without one the compiler's own order is the faster (Q6_K 4096 x 14336: 12.0 us, with the barrier 12.8).
+    // Without one the barrier gains nothing (measured: the same to slightly slower), so the compiler keeps its freedom there.
     if constexpr (PRO == PRO_NORM || PRO == PRO_NORM_SPLIT) __builtin_amdgcn_sched_barrier(0);
 
     // 2. activations -> LDS

@@ -1,7 +1,10 @@
 """CPU-only checks of the gfx950 code objects inside the built library: the kernels of the single-token decode step
 must not use a private segment.  A kernel with one starts 1.5-2 us later per launch on this hardware (the segment is
 set up before the first wave runs), which is a fifth of a 7 us matvec; the compiler creates one silently for register
-spills and for small arrays it decides to index in memory (a select chain over a lane-dependent index did)."""
+spills and for small arrays it decides to index in memory (a select chain over a lane-dependent index did).
+Nor may the streaming matvec access memory with flat instructions: the compiler cannot wait for a flat load by count,
+so the wait for the activation row also waits for every weight copy requested before it (pointers rebuilt from the
+integer argument block were flat until they were marked global)."""
 import os
 import re
 import shutil
@@ -17,8 +20,12 @@ READELF = os.path.join(LLVM, "llvm-readelf")
 MAGIC = b"__CLANG_OFFLOAD_BUNDLE__"
 
 
-def kernel_private_segments(so_path, tmp):
-    """{kernel symbol: private_segment_fixed_size} over every gfx950 code object bundled into the library."""
+OBJDUMP = os.path.join(LLVM, "llvm-objdump")
+
+
+def kernel_private_segments(so_path, tmp, objects=None):
+    """{kernel symbol: private_segment_fixed_size} over every gfx950 code object bundled into the library; `objects`, when
+    given, receives {kernel symbol: path of the code object that holds it}."""
     fat = os.path.join(tmp, "fat.bin")
     subprocess.run(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", so_path, fat], check=True)
     data = open(fat, "rb").read()
@@ -41,6 +48,8 @@ def kernel_private_segments(so_path, tmp):
             m = re.match(r"\s*\.symbol:\s*(\S+)", line)      # the last key of a kernel's record
             if m and size is not None:
                 out[m.group(1)] = size
+                if objects is not None:
+                    objects[m.group(1)] = co
                 size = None
     return out
 
@@ -64,3 +73,21 @@ def test_decode_step_kernels_have_no_private_segment(tmp_path):
     assert len(hot_syms) > 50, hot_syms[:5]
     bad = {s: v for s, v in segs.items() if hot(s) and v}
     assert not bad, f"decode kernels with a private segment: {bad}"
+
+
+@pytest.mark.skipif(not (os.path.exists(BUNDLER) and os.path.exists(READELF) and os.path.exists(OBJDUMP) and shutil.which("objcopy")),
+                    reason="needs objcopy and ROCm's llvm tools")
+def test_streaming_matvec_has_no_flat_memory_instructions(tmp_path):
+    objects = {}
+    kernel_private_segments(_lib.LIB_PATH, str(tmp_path), objects)
+    # the one-row streaming kernels of the 8B-shape decode step: Q4_K rows of 4096 (two spans per wave) and Q6_K rows of
+    # 14336 (seven), every prologue / epilogue pair
+    syms = [s for s in objects if re.search(r"13qms_kernel_dwILi12ELi2ELi16E|13qms_kernel_dwILi14ELi7ELi64E", s)]
+    assert len(syms) >= 8, syms
+    co = objects[syms[0]]
+    assert all(objects[s] == co for s in syms)
+    names = ",".join(s[:-3] if s.endswith(".kd") else s for s in syms)
+    text = subprocess.run([OBJDUMP, "-d", f"--disassemble-symbols={names}", co], capture_output=True, text=True, check=True).stdout
+    assert text.count("s_endpgm") >= len(syms), "kernels not found in the disassembly"
+    flat = [line.strip() for line in text.splitlines() if re.search(r"\bflat_(load|store|atomic)", line)]
+    assert not flat, flat[:5]
