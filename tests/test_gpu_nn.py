@@ -165,13 +165,13 @@ def test_attention_single_key_returns_value():
 @pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (32, 8, 128)])
 @pytest.mark.parametrize("pos,ctx,max_kv", [(0, 16, 1), (5, 64, 64), (127, 256, 200), (128, 256, 256), (300, 1024, 301), (600, 1024, 1024)])
 def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
-    """rope + cache append + attention over 128-key splits (+ merge kernel) == the separate calls == the CPU ops;
-    called twice in a row on fresh caches."""
+    """rope + cache append + attention over 64- or 128-key splits with the in-kernel merge == the CPU ops; called twice in a
+    row on fresh caches."""
     lib = L()
     cos, sin = lo.precomput_freqs_cis(D, 500000.0, ctx)
     q, k, v = normal(30, (1, H * D), 1.0), normal(31, (1, KV * D), 1.0), normal(32, (1, KV * D), 1.0)
     kc0, vc0 = normal(33, (KV, ctx, D), 1.0), normal(34, (KV, ctx, D), 1.0)
-    kc0[:, pos:], vc0[:, pos:] = np.nan, np.nan          # nothing at or beyond the new position may be read
+    kc0[:, pos:], vc0[:, pos:] = np.nan, np.nan          # nothing at or beyond the new position may reach the result (key rows there are read, and masked)
     wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
     # 64-key splits while at most 16 of them cover max_kv, else 128-key splits; more than 16 splits: not available
     want_splits = (max_kv + 63) // 64 if (max_kv + 63) // 64 <= 16 else (max_kv + 127) // 128
