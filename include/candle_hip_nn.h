@@ -69,6 +69,8 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
  * launch, same arithmetic as a separate merge); with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn.
  * The last 256 bytes of partials_dev are the arrival counters of that merge: they must be zero before the first call
  * with a buffer, and every call leaves them zero.
+ * Key rows of the cache beyond p, up to the end of the last split of max_kv_len (never beyond ctx), are read before the
+ * position is known and masked afterwards: whatever they hold, NaN included, does not reach the result.
  * prefetch_dev / prefetch_bytes (optional, 16-byte aligned): a byte range that extra read-only workgroups of this
  * otherwise latency-bound launch pull through the memory-side cache, e.g. the weights of the kernels that follow.
  * No counterpart in the reference, which runs these as separate tensor ops (quantized_llama.rs:217-261). */
