@@ -609,14 +609,56 @@ __global__ __launch_bounds__(HD) void attn_combine_kernel(const float *__restric
 //     every K and V row is requested before anything is consumed (one memory round trip);
 //   * the result is left as per-split partials { acc[HD], m, l, 0, 0 } (stride HD + 4 floats, 16-byte aligned
 //     rows); the last workgroup of each kv head, or the prologue of the attention_wo matvec, merges them.
-constexpr int ATTD_MAX_SPLITS = 16;
-constexpr int ATTD_COUNTER_BYTES = 256;       // arrival counters of the in-kernel merge, one int per kv head, behind the partials
-// Keys per split: 64 (workgroups of 8 waves) while that gives at most ATTD_MAX_SPLITS splits, else 128 (16 waves).  The
+constexpr int ATTD_MAX_SPLITS = 32;           // 4096 keys in splits of 128 (MAX_SEQ_LEN, quantized_llama.rs:27)
+constexpr int ATTD_FINE_SPLITS = 16;          // up to this many splits they are 64 keys long
+constexpr int ATTD_COUNTER_BYTES = CQ_NN_ATTD_HEADER_BYTES;      // arrival counters of the in-kernel merge, one int per kv head, in front of the partials
+// Keys per split: 64 (workgroups of 8 waves) while that gives at most ATTD_FINE_SPLITS splits, else 128 (16 waves).  The
 // vector memory pipeline of a CU takes one instruction of a wave per 16 cycles whatever it loads, and a split asks for
 // about 28 of them per wave: with 128-key splits of 16 waves the 48 workgroups of a 768-key step spent 3 us getting
 // their loads accepted; twice the workgroups of half the size halve that.
-__host__ __device__ inline int64_t attd_split_keys(int64_t max_kv_len) { return (max_kv_len + 63) / 64 <= ATTD_MAX_SPLITS ? 64 : 128; }
+__host__ __device__ inline int64_t attd_split_keys(int64_t max_kv_len) { return (max_kv_len + 63) / 64 <= ATTD_FINE_SPLITS ? 64 : 128; }
 __host__ __device__ inline int64_t attd_splits(int64_t max_kv_len) { const int64_t sk = attd_split_keys(max_kv_len); return (max_kv_len + sk - 1) / sk; }
+
+// The merge of a kv head's splits by the workgroup that arrived last: out = sum_s e^{m_s - M} acc_s / sum_s e^{m_s - M} l_s,
+// split by split, in order (the arithmetic of attn_combine_kernel and of the merge prologue of the attention_wo matvec).
+// MS: the number of splits the registers hold (16 or 32).
+template <int HD, int G, int NW, int MS>
+__device__ __forceinline__ void attd_merge(const float *__restrict__ part, float *__restrict__ out, int kvh, int splits, int tid) {
+    const int lane = tid & 63;
+    auto ld = [](const float *q) { return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    for (int i = tid; i < G * HD; i += 64 * NW) {
+        const int g = i / HD, d = i - g * HD;                 // g is the same in all lanes of a wave
+        const float *pp = part + (int64_t)(kvh * G + g) * splits * (HD + 4);
+        // Every load first (these bypass the caches: one after the other they would be a trip to memory each), and as few
+        // load instructions as possible, they are what the last workgroup's time goes into: one instruction fetches
+        // the (m, l) of all splits of the head (lane s: m of split s, lane MS + s: l), one per existing split the
+        // accumulators.  A split that does not exist re-reads the last one and is left out of the sums.
+        const float mlv = ld(pp + min(lane & (MS - 1), splits - 1) * (HD + 4) + HD + ((lane / MS) & 1));
+        float av[MS];
+#pragma unroll
+        for (int sI = 0; sI < MS; sI++) av[sI] = sI < splits ? ld(pp + sI * (HD + 4) + d) : 0.0f;
+        float mv[MS], lv[MS];
+#pragma unroll
+        for (int sI = 0; sI < MS; sI++) {
+            mv[sI] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mlv), sI));
+            lv[sI] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mlv), MS + sI));
+        }
+        float M = -INFINITY;
+#pragma unroll
+        for (int sI = 0; sI < MS; sI++)
+            if (sI < splits) M = fmaxf(M, lv[sI] > 0.0f ? mv[sI] : -INFINITY);
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int sI = 0; sI < MS; sI++) {
+            if (sI < splits && lv[sI] > 0.0f) {
+                const float wgt = __expf(mv[sI] - M);
+                num += wgt * av[sI];
+                den += wgt * lv[sI];
+            }
+        }
+        out[(int64_t)(kvh * G + g) * HD + d] = num / den;
+    }
+}
 
 template <int HD, int G, int NW, int SPLIT>
 __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__restrict__ pos_dev, const float *__restrict__ q, float *k_cache,
@@ -862,40 +904,11 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
     if (tid == 0) s_last = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == splits - 1;
     __syncthreads();
     if (!s_last) return;
-    auto ld = [](const float *q) { return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-    static_assert(HD % 64 == 0 && ATTD_MAX_SPLITS <= 16, "a wave stays inside one query head; lanes 0..31 fetch the (m, l) pairs");
-    for (int i = tid; i < G * HD; i += 64 * NW) {
-        const int g = i / HD, d = i - g * HD;                 // g is the same in all lanes of a wave
-        const float *pp = part + (int64_t)(kvh * G + g) * splits * (HD + 4);
-        // Every load first (these bypass the caches: one after the other they would be a trip to memory each), and as few
-        // load instructions as possible, they are what the last workgroup's time goes into: one instruction fetches
-        // the (m, l) of all splits of the head (lane s: m of split s, lane 16 + s: l), one per existing split the
-        // accumulators.  A split that does not exist re-reads the last one and is left out of the sums.
-        const float mlv = ld(pp + min(lane & 15, splits - 1) * (HD + 4) + HD + ((lane >> 4) & 1));
-        float av[ATTD_MAX_SPLITS];
-#pragma unroll
-        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++) av[sI] = sI < splits ? ld(pp + sI * (HD + 4) + d) : 0.0f;
-        float mv[ATTD_MAX_SPLITS], lv[ATTD_MAX_SPLITS];
-#pragma unroll
-        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++) {
-            mv[sI] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mlv), sI));
-            lv[sI] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mlv), 16 + sI));
-        }
-        float M = -INFINITY;
-#pragma unroll
-        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++)
-            if (sI < splits) M = fmaxf(M, lv[sI] > 0.0f ? mv[sI] : -INFINITY);
-        float num = 0.0f, den = 0.0f;
-#pragma unroll
-        for (int sI = 0; sI < ATTD_MAX_SPLITS; sI++) {
-            if (sI < splits && lv[sI] > 0.0f) {
-                const float wgt = __expf(mv[sI] - M);
-                num += wgt * av[sI];
-                den += wgt * lv[sI];
-            }
-        }
-        out[(int64_t)(kvh * G + g) * HD + d] = num / den;
-    }
+    static_assert(HD % 64 == 0 && ATTD_MAX_SPLITS <= 32, "a wave stays inside one query head; the lanes of a wave fetch the (m, l) pairs");
+    if (splits <= ATTD_FINE_SPLITS)
+        attd_merge<HD, G, NW, ATTD_FINE_SPLITS>(part, out, kvh, splits, tid);
+    else
+        attd_merge<HD, G, NW, ATTD_MAX_SPLITS>(part, out, kvh, splits, tid);
     if (tid == 0) __hip_atomic_store(&counters[kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -1400,7 +1413,7 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
 
 int64_t cq_nn_attention_decode_workspace_bytes(int64_t n_head, int64_t head_dim, int64_t max_kv_len) {
     if (n_head <= 0 || head_dim <= 0 || max_kv_len <= 0) return -1;
-    return n_head * attd_splits(max_kv_len) * (head_dim + 4) * 4 + ATTD_COUNTER_BYTES;
+    return ATTD_COUNTER_BYTES + n_head * attd_splits(max_kv_len) * (head_dim + 4) * 4;
 }
 
 int64_t cq_nn_attention_decode_splits(int64_t max_kv_len) {
@@ -1425,9 +1438,10 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     const int64_t splits = attd_splits(max_kv_len);
     if (splits > ATTD_MAX_SPLITS || ctx > 0x7fffffffLL || n_kv_head > ATTD_COUNTER_BYTES / 4) return CQ_ERR_RANGE;
     const bool fine = attd_split_keys(max_kv_len) == 64;
-    int *counters = (int *)((uint8_t *)partials_dev + n_head * splits * (head_dim + 4) * 4);
+    // the counters lie in front of the records: their place does not move with max_kv_len, so one buffer serves every length
+    int *counters = (int *)partials_dev;
     const int G = (int)(n_head / n_kv_head);
-    float *part = (float *)partials_dev;
+    float *part = (float *)((uint8_t *)partials_dev + ATTD_COUNTER_BYTES);
     // read-only workgroups for the prefetch range: enough, with the attention ones, for one per CU
     const int64_t pf_chunks = prefetch_bytes / 16;
     int64_t pf_rows = 0;

@@ -113,6 +113,7 @@ class ModelWeights:
         # would pull through the memory-side cache ahead of the kernels that stream them.  Measured on the 8B shape:
         # no gain at 4-24 MB and a loss beyond (the time moves into the attention launch), so it is off.
         self.prefetch_bytes = 0
+        self.tap = None                    # tests: called as tap(stage, layer) after each launch of an eager forward
 
     # ------------------------------------------------------------------------------------------ construction
     def _alloc(self, dtypes: Dict[str, GgmlDType]):
@@ -185,7 +186,7 @@ class ModelWeights:
         att_ws = L.cq_nn_attention_workspace_bytes(max_rows, cfg.n_head, cfg.head_dim, cfg.ctx)
         self.att_ws = torch.empty(max(att_ws, 256), dtype=torch.uint8, device=self.device)
         # single-token attention: per-split partials
-        attd = L.cq_nn_attention_decode_workspace_bytes(cfg.n_head, cfg.head_dim, min(cfg.ctx, 2048))
+        attd = L.cq_nn_attention_decode_workspace_bytes(cfg.n_head, cfg.head_dim, min(cfg.ctx, 4096))
         self.attd_ws = torch.zeros(attd, dtype=torch.uint8, device=self.device)
 
     @classmethod
@@ -336,12 +337,15 @@ class ModelWeights:
             return self._enqueue_decode_fused(ids_ptr, pos, pos_dev_ptr, max_kv_len, sp)
         if ids_ptr is None:
             raise ValueError("a step without token ids needs the fused single-token path")
+        tap = self.tap if self.tap is not None else (lambda stage, li: None)
         ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, x.data_ptr(), rows, cfg.hidden, cfg.vocab, None, sp))
+        tap("embedding", -1)
         for li, lw in enumerate(self.layers):
             w = lw.w
             # x (+= mlp output of the previous layer); xn = attention_norm(x)          :579-583, :590-592
             ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr(), delta.data_ptr() if li else None, lw.attention_norm.data_ptr(),
                                                  x.data_ptr() if li else None, xn.data_ptr(), rows, cfg.hidden, cfg.rms_eps, sp))
+            tap("attention_norm", li)
             # q, k, v projections                                                         :200-202
             wq, wk, wv = w["attention_wq"], w["attention_wk"], w["attention_wv"]
             if wq.dtype == wk.dtype and wk.ptr == wq.ptr + wq.nbytes:
@@ -352,18 +356,23 @@ class ModelWeights:
                 self._mm(wk, kvd, xn, qk.data_ptr() + 4 * rows * qd, rows, sp)
                 q_ptr, k_ptr, qs, ks = qk.data_ptr(), qk.data_ptr() + 4 * rows * qd, qd, kvd
             self._mm(wv, kvd, xn, v.data_ptr(), rows, sp)
+            tap("qkv", li)
             # rope on q and k, append k and v to the cache                                :217-233
             ck("cq_nn_rope_i_kv", L.cq_nn_rope_i_kv(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
                                                    self.cos.data_ptr(), self.sin.data_ptr(), pos_dev_ptr, pos, rows, cfg.n_head, cfg.n_kv_head,
                                                    cfg.head_dim, cfg.ctx, qs, ks, kvd, sp))
+            tap("rope", li)
             # softmax(q k^T / sqrt(d) + causal mask) v                                    :246-261
             ck("cq_nn_attention", L.cq_nn_attention(q_ptr, qs, lw.k_cache.data_ptr(), lw.v_cache.data_ptr(), att.data_ptr(), pos_dev_ptr, pos,
                                                    rows, cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
                                                    self.att_ws.data_ptr(), self.att_ws.numel(), sp))
+            tap("attention", li)
             self._mm(w["attention_wo"], cfg.hidden, att, delta.data_ptr(), rows, sp)    # :264
+            tap("attention_wo", li)
             # x += attn; xn = ffn_norm(x)                                                 :584-589
             ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr(), delta.data_ptr(), lw.ffn_norm.data_ptr(), x.data_ptr(), xn.data_ptr(), rows,
                                                  cfg.hidden, cfg.rms_eps, sp))
+            tap("ffn_norm", li)
             # w2(silu(w1 x) * w3 x)                                                       :56-63
             w1, w3 = w["feed_forward_w1"], w["feed_forward_w3"]
             if w1.dtype == w3.dtype and w3.ptr == w1.ptr + w1.nbytes:
@@ -373,6 +382,7 @@ class ModelWeights:
                 self._mm(w1, cfg.ffn, xn, gu.data_ptr(), rows, sp)
                 self._mm(w3, cfg.ffn, xn, gu.data_ptr() + 4 * rows * cfg.ffn, rows, sp)
                 g_ptr, u_ptr, gs = gu.data_ptr(), gu.data_ptr() + 4 * rows * cfg.ffn, cfg.ffn
+            tap("w13", li)
             w2 = w["feed_forward_w2"]
             if rows > 2 and cfg.ffn % 256 == 0:
                 # silu(w1 x) * w3 x goes straight into the activation quantizer of w2
@@ -381,11 +391,13 @@ class ModelWeights:
             else:
                 ck("cq_nn_silu_mul", L.cq_nn_silu_mul(g_ptr, u_ptr, h.data_ptr(), rows, cfg.ffn, gs, gs, sp))
                 self._mm(w2, cfg.hidden, h, delta.data_ptr(), rows, sp)
+            tap("w2", li)
         # last token only: x += mlp; final norm; output head                              :593-596
         last = 4 * (rows - 1) * cfg.hidden
         ck("cq_nn_rms_norm", L.cq_nn_rms_norm(x.data_ptr() + last, delta.data_ptr() + last, self.norm.data_ptr(), None, xn.data_ptr(), 1,
                                              cfg.hidden, cfg.rms_eps, sp))
         self._mm(self.output, cfg.vocab, xn, self.logits.data_ptr(), 1, sp)
+        tap("head", -1)
 
     def _enqueue_decode_fused(self, ids_ptr: Optional[int], pos: int, pos_dev_ptr: Optional[int], max_kv_len: int, sp) -> None:
         """The same single-token step with the glue folded into the matvec kernels: the residual add is the
@@ -405,8 +417,10 @@ class ModelWeights:
         all_full = all(w.dtype in full for lw in self.layers for w in lw.w.values()) and self.output.dtype in full
         cur = self.x.data_ptr()                                    # the residual row
         pending = 0                                                # planes of the previous feed_forward_w2 not yet added to it
+        tap = self.tap if self.tap is not None else (lambda stage, li: None)
         if ids_ptr is not None:
             ck("cq_nn_embedding", L.cq_nn_embedding(self.tok_embeddings.data_ptr(), ids_ptr, cur, 1, cfg.hidden, cfg.vocab, part.data_ptr(), sp))
+        tap("embedding", -1)
 
         def one_step(w: _W) -> bool:
             return w.k <= (4096 if w.dtype in kq + (GgmlDType.Q2K, GgmlDType.Q3K) else 2048)
@@ -444,13 +458,14 @@ class ModelWeights:
                 norm_mm(wq, qd, lw.attention_norm, qk.data_ptr())
                 norm_mm(wk, kvd, lw.attention_norm, qk.data_ptr() + 4 * qd)
                 norm_mm(wv, kvd, lw.attention_norm, v.data_ptr())
+            tap("qkv", li)
             q_ptr, k_ptr = qk.data_ptr(), qk.data_ptr() + 4 * qd
             # rope, cache append, attention and the merge of the key splits in one kernel          :217-261
             wo = w["attention_wo"]
             # the attention kernel merges its key splits itself (the last workgroup of a kv head does it once); merging in
             # the prologue of attention_wo instead makes every workgroup of that matvec read every partial
             merge_in_wo = self.merge_in_wo and wo.dtype in full and qd <= (4096 if wo.dtype in kq else 2048) and \
-                (cfg.head_dim & (cfg.head_dim - 1)) == 0
+                (cfg.head_dim & (cfg.head_dim - 1)) == 0 and L.cq_nn_attention_decode_splits(max_kv_len) <= 16
             ck("cq_nn_attention_decode", L.cq_nn_attention_decode(q_ptr, k_ptr, v.data_ptr(), lw.k_cache.data_ptr(), lw.v_cache.data_ptr(),
                                                                   self.cos.data_ptr(), self.sin.data_ptr(),
                                                                   None if merge_in_wo else att.data_ptr(), pos_dev_ptr, pos,
@@ -458,14 +473,16 @@ class ModelWeights:
                                                                   self.attd_ws.data_ptr(), self.attd_ws.numel(),
                                                                   wo.ptr if self.prefetch_bytes else None,
                                                                   min(self.prefetch_bytes, lw.prefetch_span), sp))
+            tap("attention", li)
             # attention_wo adds to the residual row, and folds the pending planes into it
             if merge_in_wo:
                 ck("cq_nn_qmatmul_residual_attn_merge", L.cq_nn_qmatmul_residual_attn_merge(
-                    int(wo.dtype), wo.ptr, self.attd_ws.data_ptr(), L.cq_nn_attention_decode_splits(max_kv_len), cfg.head_dim, cur,
+                    int(wo.dtype), wo.ptr, self.attd_ws.data_ptr() + 256, L.cq_nn_attention_decode_splits(max_kv_len), cfg.head_dim, cur,
                     part.data_ptr(), planes.data_ptr() if pending else None, pending, wo.k, cfg.hidden, sp))
             else:
                 resid_mm(wo, att.data_ptr(), None)
             pending = 0
+            tap("attention_wo", li)
             w1, w3, w2 = w["feed_forward_w1"], w["feed_forward_w3"], w["feed_forward_w2"]
             # the consumers of this layer's residual row: the next layer's q / k / v projections, or the output head
             nxt = self.layers[li + 1].w if li + 1 < len(self.layers) else None
@@ -482,12 +499,15 @@ class ModelWeights:
                 norm_mm(w1, cfg.ffn, lw.ffn_norm, gu.data_ptr())
                 norm_mm(w3, cfg.ffn, lw.ffn_norm, gu.data_ptr() + 4 * cfg.ffn)
                 src_ptr, up_ptr = gu.data_ptr(), gu.data_ptr() + 4 * cfg.ffn
+            tap("w13", li)
             if n_split:
                 ck("cq_nn_qmatmul_split", L.cq_nn_qmatmul_split(int(w2.dtype), w2.ptr, src_ptr, up_ptr, planes.data_ptr(), w2.k, cfg.hidden, sp))
                 pending = n_split
             else:
                 resid_mm(w2, src_ptr, up_ptr)
+            tap("w2", li)
         norm_mm(self.output, cfg.vocab, self.norm, self.logits.data_ptr())
+        tap("head", -1)
 
     def forward(self, x: torch.Tensor, index_pos: int) -> torch.Tensor:
         """ModelWeights::forward: token ids [1, seq_len] at positions index_pos.. -> logits [1, vocab] of the last token."""

@@ -62,18 +62,21 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
 /* One decode step (a single new token at position p = pos + *pos_dev) of the three calls above:
  * rope_i on q and on the new k, append of the new k and v to the cache at p, attention of the rotated q over keys
  * [0, p].  q [n_head*head_dim], k_new / v_new [n_kv_head*head_dim] are the raw projection outputs (16-byte aligned;
- * q is not modified).  The result is left in partials_dev as per-split records { acc[head_dim], m, l, 0, 0 } for
- * every head ([n_head][splits][head_dim + 4] floats, splits = cq_nn_attention_decode_splits(max_kv_len): splits of 64
- * keys while 16 of them cover max_kv_len, else of 128 keys; at most 16, i.e. max_kv_len <= 2048; -1 beyond).  When out_dev != NULL the
+ * q is not modified).  partials_dev is CQ_NN_ATTD_HEADER_BYTES of arrival counters followed by per-split records
+ * { acc[head_dim], m, l, 0, 0 } for every head ([n_head][splits][head_dim + 4] floats, splits =
+ * cq_nn_attention_decode_splits(max_kv_len): splits of 64 keys while 16 of them cover max_kv_len, else of 128 keys; at
+ * most 32, i.e. max_kv_len <= 4096, MAX_SEQ_LEN of quantized_llama.rs:27; -1 beyond).  When out_dev != NULL the
  * workgroup of each kv head that finishes last merges that head group's splits into out_dev [n_head*head_dim] (same
- * launch, same arithmetic as a separate merge); with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn.
- * The last 256 bytes of partials_dev are the arrival counters of that merge: they must be zero before the first call
- * with a buffer, and every call leaves them zero.
+ * launch, same arithmetic as a separate merge); with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn,
+ * which takes the address of the records (partials_dev + CQ_NN_ATTD_HEADER_BYTES).
+ * The counters (one int per kv head, n_kv_head <= 64) must be zero before the first call with a buffer, and every call
+ * leaves them zero; they sit in front of the records so that one buffer serves calls of any max_kv_len.
  * Key rows of the cache beyond p, up to the end of the last split of max_kv_len (never beyond ctx), are read before the
  * position is known and masked afterwards: whatever they hold, NaN included, does not reach the result.
  * prefetch_dev / prefetch_bytes (optional, 16-byte aligned): a byte range that extra read-only workgroups of this
  * otherwise latency-bound launch pull through the memory-side cache, e.g. the weights of the kernels that follow.
  * No counterpart in the reference, which runs these as separate tensor ops (quantized_llama.rs:217-261). */
+#define CQ_NN_ATTD_HEADER_BYTES 256
 int64_t cq_nn_attention_decode_workspace_bytes(int64_t n_head, int64_t head_dim, int64_t max_kv_len);
 int64_t cq_nn_attention_decode_splits(int64_t max_kv_len);
 int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const float *v_new_dev, float *k_cache_dev, float *v_cache_dev,
@@ -117,7 +120,8 @@ int cq_nn_qmatmul_norm_pair(int w_dtype_a, const void *w_a_dev, int64_t n_a, flo
                             float *dst_b_dev, const float *x_dev, const float *sumsq_partials_dev, const float *norm_weight_dev, float eps,
                             int64_t k, void *stream);
 /* cq_nn_qmatmul_residual whose input row is the attention output still in the per-split partials of
- * cq_nn_attention_decode (out_dev == NULL there): the merge of the splits is the matvec's prologue.
+ * cq_nn_attention_decode (out_dev == NULL there; attn_partials_dev = that call's partials_dev + CQ_NN_ATTD_HEADER_BYTES,
+ * the first record): the merge of the splits is the matvec's prologue.
  * CQ_ERR_RANGE (use the merge kernel + cq_nn_qmatmul_residual instead) when k = n_head*head_dim is longer than one
  * wave step per row (k > 4096 for K-quants, > 2048 for Q4_0 / Q8_0), splits > 16, or head_dim is not a power of 2. */
 int cq_nn_qmatmul_residual_attn(int w_dtype, const void *w_dev, const float *attn_partials_dev, int64_t splits, int64_t head_dim,

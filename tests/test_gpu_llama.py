@@ -134,8 +134,16 @@ def test_8b_shape_two_layers_prefill_16_then_decode_4():
         assert want[0, int(np.argmax(got))] >= want.max() - 4.0 * bound * float(np.abs(want).max()), pos
         return int(np.argmax(want))
 
-    tok = check(model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy(), prompt, 0)
-    for step in range(4):
+    # the wiring of the real-width model, op by op: every launch of the 16-row forward and of a single-token step (one kernel
+    # per op, then the fused step) against the CPU op on the GPU's own input: glue 1e-5, matmuls 2e-6
+    from tests.teacher import check_forward_ops
+    got16, flips16 = check_forward_ops(model, t, cfg, prompt, 0, fused=False)
+    tok = check(got16, prompt, 0)
+    _, flips_a = check_forward_ops(model, t, cfg, [tok], 16, fused=False)
+    got1, flips_b = check_forward_ops(model, t, cfg, [tok], 16, fused=True)
+    assert flips16 + flips_a + flips_b <= 6, (flips16, flips_a, flips_b)      # rows accepted through a boundary element of their quantizer
+    tok = check(got1, [tok], 16)
+    for step in range(1, 4):
         tok = check(model.forward(torch.tensor([[tok]], dtype=torch.int32), 16 + step).cpu().numpy(), [tok], 16 + step)
     # the same four steps replayed from a HIP graph give the same tokens as eager single-token forwards
     a = model.generate_greedy(prompt, 4, use_graph=False)["tokens"]
@@ -260,6 +268,56 @@ def test_long_context_decode_uses_split_attention():
         want_toks.append(tok)
         logits = ref.forward([tok], 300 + i)
     assert out["tokens"] == want_toks
+
+
+LONG_CTX = dict(n_layer=1, hidden=512, n_head=8, n_kv_head=2, head_dim=64, ffn=768, vocab=512, rope_theta=500000.0, rms_eps=1e-5, ctx=2048)
+
+
+def test_split_count_changes_on_one_model():
+    """The single-token attention takes 64-key splits up to 1024 keys and 128-key splits beyond; one model (one partials
+    buffer) walks across those boundaries token by token, and runs a short sequence after a long one."""
+    cfg, t, model = make(LONG_CTX, MIX, seed=27)
+    ref = lo.LlamaOracle(cfg, t, threads=8)
+    rng = np.random.default_rng(28)
+    prompt = rng.integers(0, cfg.vocab, size=1022).tolist()
+    got = model.forward(torch.tensor([prompt], dtype=torch.int32), 0).cpu().numpy()
+    want = ref.forward(prompt, 0)
+    assert rel_l2(got, want) <= TOL
+    tok = int(np.argmax(want))
+    from tests.teacher import check_forward_ops
+    # End to end, two correct evaluations of a step drift apart through the activation quantizers (a flipped element of the
+    # 1022-row prompt moves a cache row by 3e-3), so the steps are checked op by op on the GPU's own inputs instead.
+    for pos in range(1022, 1027):                         # max_kv_len 1023 .. 1027: 16 splits of 64, then 9 of 128
+        fused, _ = check_forward_ops(model, t, cfg, [tok], pos, fused=True)
+        unfused, _ = check_forward_ops(model, t, cfg, [tok], pos, fused=False)
+        assert rel_l2(fused, unfused) <= 1e-4, pos
+        tok = int(np.argmax(fused))
+    # a short sequence on the same model: one split, then two
+    rng2 = np.random.default_rng(29)
+    prompt2 = rng2.integers(0, cfg.vocab, size=62).tolist()
+    ref2 = lo.LlamaOracle(cfg, t, threads=8)
+    got = model.forward(torch.tensor([prompt2], dtype=torch.int32), 0).cpu().numpy()
+    want = ref2.forward(prompt2, 0)
+    assert rel_l2(got, want) <= TOL
+    tok = int(np.argmax(want))
+    for pos in range(62, 67):
+        got, _ = check_forward_ops(model, t, cfg, [tok], pos, fused=True)
+        want = ref2.forward([tok], pos)
+        assert rel_l2(got, want) <= TOL, pos
+        tok = int(np.argmax(want))
+    # greedy decoding, long (9 splits of 128 keys) then short (one split), graph replay against the eager loop and the oracle
+    short_p = prompt2[:20]
+    a = model.generate_greedy(prompt, 6, use_graph=True)["tokens"]
+    b = model.generate_greedy(short_p, 6, use_graph=True)["tokens"]
+    assert a == model.generate_greedy(prompt, 6, use_graph=False)["tokens"]
+    assert b == model.generate_greedy(short_p, 6, use_graph=False)["tokens"]
+    ref3 = lo.LlamaOracle(cfg, t, threads=8)
+    logits, want_toks = ref3.forward(short_p, 0), []
+    for i in range(6):
+        tk = int(np.argmax(logits))
+        want_toks.append(tk)
+        logits = ref3.forward([tk], len(short_p) + i)
+    assert b == want_toks
 
 
 def test_forward_argument_errors():

@@ -175,9 +175,10 @@ def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
     wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
     # 64-key splits while at most 16 of them cover max_kv, else 128-key splits; more than 16 splits: not available
     want_splits = (max_kv + 63) // 64 if (max_kv + 63) // 64 <= 16 else (max_kv + 127) // 128
-    assert lib.cq_nn_attention_decode_splits(max_kv) == want_splits and lib.cq_nn_attention_decode_splits(2049) == -1
+    assert lib.cq_nn_attention_decode_splits(max_kv) == want_splits
+    assert lib.cq_nn_attention_decode_splits(2049) == 17 and lib.cq_nn_attention_decode_splits(4096) == 32 and lib.cq_nn_attention_decode_splits(4097) == -1
     ws = torch.full((wsb,), 0xff, dtype=torch.uint8, device="cuda")
-    ws[-256:] = 0                                        # the arrival counters of the in-kernel merge start at zero
+    ws[:256] = 0                                         # the arrival counters of the in-kernel merge start at zero
     posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
     c, s = cos[pos:pos + 1], sin[pos:pos + 1]
     want_q = lo.rope_i(q.reshape(1, H, D).transpose(1, 0, 2)[None], c, s)[0].transpose(1, 0, 2).reshape(1, H * D)
@@ -198,6 +199,98 @@ def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
         assert np.allclose(kc.cpu().numpy()[:, pos], want_k[:, 0], rtol=1e-6, atol=1e-6)
         assert np.array_equal(vc.cpu().numpy()[:, pos], vc_ref[:, pos])
         assert np.array_equal(kc.cpu().numpy()[:, :pos], kc0[:, :pos])
+
+
+def _attention_decode_case(lib, ws, wsb, H, KV, D, pos, ctx, max_kv, seed):
+    """One fused decode-attention call on a given workspace against the CPU ops."""
+    cos, sin = lo.precomput_freqs_cis(D, 500000.0, ctx)
+    q, k, v = normal(seed, (1, H * D), 1.0), normal(seed + 1, (1, KV * D), 1.0), normal(seed + 2, (1, KV * D), 1.0)
+    kc0, vc0 = normal(seed + 3, (KV, ctx, D), 1.0), normal(seed + 4, (KV, ctx, D), 1.0)
+    kc0[:, pos:], vc0[:, pos:] = np.nan, np.nan
+    c, s = cos[pos:pos + 1], sin[pos:pos + 1]
+    want_q = lo.rope_i(q.reshape(1, H, D).transpose(1, 0, 2)[None], c, s)[0].transpose(1, 0, 2).reshape(1, H * D)
+    want_k = lo.rope_i(k.reshape(1, KV, D).transpose(1, 0, 2)[None], c, s)[0]
+    kc_ref, vc_ref = kc0.copy(), vc0.copy()
+    kc_ref[:, pos:pos + 1], vc_ref[:, pos:pos + 1] = want_k, v.reshape(1, KV, D).transpose(1, 0, 2)
+    want = attention_oracle(want_q, kc_ref, vc_ref, pos, H, KV, D)
+    kc, vc, out = dev(kc0), dev(vc0), torch.zeros((1, H * D), device="cuda")
+    posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    ok(lib.cq_nn_attention_decode(dev(q).data_ptr(), dev(k).data_ptr(), dev(v).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(),
+                                  dev(sin).data_ptr(), out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv,
+                                  float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None, 0, None))
+    torch.cuda.synchronize()
+    assert rel_l2(out.cpu().numpy(), want) <= TOL, (pos, max_kv)
+    assert np.array_equal(vc.cpu().numpy()[:, pos], vc_ref[:, pos])
+
+
+def test_attention_decode_one_workspace_across_split_counts():
+    """One partials buffer, sized for the longest context, serves calls whose split count rises and falls: the arrival
+    counters sit in front of the records, where no call's records reach them."""
+    lib = L()
+    H, KV, D, ctx = 32, 8, 128, 4096
+    wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, ctx)
+    ws = torch.zeros(wsb, dtype=torch.uint8, device="cuda")
+    # 16 splits of 64 keys, 9 of 128, one split, 32 splits, and back
+    for i, (pos, max_kv) in enumerate([(1000, 1024), (1024, 1025), (40, 64), (3000, 4096), (63, 64), (64, 65), (1023, 1024), (3000, 3001)]):
+        _attention_decode_case(lib, ws, wsb, H, KV, D, pos, ctx, max_kv, 300 + 10 * i)
+        assert int(ws[:256].to(torch.int32).sum()) == 0           # every call leaves its counters at zero
+
+
+@pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (32, 8, 128)])
+def test_attention_decode_beyond_2048_keys(H, KV, D):
+    """MAX_SEQ_LEN of quantized_llama.rs:27 is 4096: position 3000 of a 4096-key context, 32 splits of 128 keys."""
+    lib = L()
+    wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, 4096)
+    ws = torch.zeros(wsb, dtype=torch.uint8, device="cuda")
+    assert lib.cq_nn_attention_decode_splits(4096) == 32
+    _attention_decode_case(lib, ws, wsb, H, KV, D, 3000, 4096, 4096, 500)
+    _attention_decode_case(lib, ws, wsb, H, KV, D, 4095, 4096, 4096, 510)
+
+
+@pytest.mark.parametrize("pos,max_kv", [(760, 768), (1000, 1024)], ids=["12-splits", "16-splits"])
+def test_attention_decode_in_kernel_merge_soak(pos, max_kv):
+    """The in-kernel merge reads the partials of workgroups on other XCDs after one relaxed device-scope counter increment,
+    with no fence.  20 000 launches at the 8B head shape, the records poisoned with NaN before each: every launch must
+    reproduce, bit for bit, the merged output that the first launch produced (which is checked against the CPU ops, and whose
+    arithmetic test_attention_merge_as_matvec_prologue ties to the merge across a kernel boundary).  A partial read before it
+    was visible would come out as NaN."""
+    lib = L()
+    H, KV, D, ctx = 32, 8, 128, 2048
+    cos, sin = lo.precomput_freqs_cis(D, 500000.0, ctx)
+    q, k, v = normal(70, (1, H * D), 1.0), normal(71, (1, KV * D), 1.0), normal(72, (1, KV * D), 1.0)
+    kc0, vc0 = normal(73, (KV, ctx, D), 1.0), normal(74, (KV, ctx, D), 1.0)
+    c, s = cos[pos:pos + 1], sin[pos:pos + 1]
+    want_q = lo.rope_i(q.reshape(1, H, D).transpose(1, 0, 2)[None], c, s)[0].transpose(1, 0, 2).reshape(1, H * D)
+    kc_ref, vc_ref = kc0.copy(), vc0.copy()
+    kc_ref[:, pos:pos + 1] = lo.rope_i(k.reshape(1, KV, D).transpose(1, 0, 2)[None], c, s)[0]
+    vc_ref[:, pos:pos + 1] = v.reshape(1, KV, D).transpose(1, 0, 2)
+    want = attention_oracle(want_q, kc_ref, vc_ref, pos, H, KV, D)
+    wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
+    assert lib.cq_nn_attention_decode_splits(max_kv) == (12 if max_kv == 768 else 16)
+    ws = torch.zeros(wsb // 4, dtype=torch.float32, device="cuda")
+    records = ws[64:]                                     # behind the 256 bytes of counters
+    kc, vc, out = dev(kc0), dev(vc0), torch.zeros((1, H * D), device="cuda")
+    qd, kd, vd, cd, sd = dev(q), dev(k), dev(v), dev(cos), dev(sin)
+    posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    scale = float(np.float32(1.0 / math.sqrt(D)))
+
+    def launch():
+        ok(lib.cq_nn_attention_decode(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), kc.data_ptr(), vc.data_ptr(), cd.data_ptr(), sd.data_ptr(),
+                                      out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv, scale, ws.data_ptr(), wsb, None, 0, None))
+
+    launch()
+    torch.cuda.synchronize()
+    assert rel_l2(out.cpu().numpy(), want) <= TOL
+    first = out.clone().view(torch.int32)
+    bad = torch.zeros((), dtype=torch.int64, device="cuda")
+    for i in range(20000):
+        records.fill_(float("nan"))
+        out.fill_(float("nan"))
+        launch()
+        bad += (out.view(torch.int32) != first).sum()
+        if i % 2000 == 1999:
+            assert int(bad) == 0, i                       # stop at the first block of launches with a mismatch
+    assert int(ws[:64].view(torch.int32).abs().sum()) == 0
 
 
 @pytest.mark.parametrize("dtype", [12, 14, 2])
@@ -223,7 +316,7 @@ def test_attention_merge_as_matvec_prologue(dtype, pos, max_kv):
     p1, p2 = torch.empty(256, device="cuda"), torch.empty(256, device="cuda")
     ok(lib.cq_nn_qmatmul_residual(dtype, w.data_ptr(), att.data_ptr(), None, r1.data_ptr(), p1.data_ptr(), k, hidden, None))
     ok(lib.cq_nn_attention_decode(*args, None, *tail))
-    ok(lib.cq_nn_qmatmul_residual_attn(dtype, w.data_ptr(), ws.data_ptr(), lib.cq_nn_attention_decode_splits(max_kv), D, r2.data_ptr(),
+    ok(lib.cq_nn_qmatmul_residual_attn(dtype, w.data_ptr(), ws.data_ptr() + 256, lib.cq_nn_attention_decode_splits(max_kv), D, r2.data_ptr(),
                                        p2.data_ptr(), k, hidden, None))
     torch.cuda.synchronize()
     assert np.array_equal(r1.cpu().numpy(), r2.cpu().numpy()) and np.array_equal(p1.cpu().numpy(), p2.cpu().numpy())
