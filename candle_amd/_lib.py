@@ -65,6 +65,8 @@ SIGNATURES = {
     "cq_nn_attention_decode_splits": (_i64, [_i64]),
     "cq_nn_attention_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64,
                                       _vp]),
+    "cq_nn_coop_sync_bytes": (_i64, []),
+    "cq_nn_decode_mlp": (_int, [_int, _vp, _vp, _int, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp, _vp]),
     "cq_nn_silu_mul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "cq_nn_qmatmul_swiglu_rows": (_int, [_int, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_nn_argmax": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),

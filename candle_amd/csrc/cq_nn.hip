@@ -6,6 +6,8 @@
 // decode position can be read from device memory so that a whole decode step (including "pick the next
 // token, advance the position") can be captured in a HIP graph and replayed without host round trips.
 #include "cq_device.h"
+#include <stdlib.h>
+
 #include "../../include/candle_hip_nn.h"
 
 namespace {
@@ -667,16 +669,41 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
                                                                       const float *__restrict__ k_new, const float *__restrict__ v_new,
                                                                       float *__restrict__ part, const u32x4 *__restrict__ pf,
                                                                       int64_t pf_chunks, uint32_t *__restrict__ pf_sink, float *__restrict__ out,
-                                                                      int *__restrict__ counters) {
+                                                                      int *__restrict__ counters, int pf_piece16) {
     // (parameter order: the fourteen dwords that sit in SGPRs when the wave starts are all that the key and query loads
     // need, so that those go out without waiting for a scalar load: neither for further arguments nor for the position)
     if ((int)blockIdx.y >= splits) {
         // Workgroups beyond the attention splits only read: they pull the weights the following kernels will stream
         // (attention_wo, feed_forward_w1 / w3) through the memory-side cache while this latency-bound kernel leaves
         // the HBM idle.  Nothing is computed from the data; the store below never executes for real weights.
+        uint32_t acc = 0;
+        if (pf_piece16 > 0) {
+            // Piece p of the range (pf_piece16 chunks: one wave step of the matvec that will stream it) is read later by a workgroup
+            // on XCD p % 8; workgroups are dealt to the XCDs round-robin by their linear index, so this one reads pieces of its own
+            // XCD only and they land in the L2 that the consumer will look in.
+            const int lin = (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x;
+            const int xcd = lin & 7;
+            // rank of this workgroup among the read-only workgroups of its XCD, and their number (grids of 8 columns)
+            const int rank = (int)blockIdx.y - splits, count = (int)gridDim.y - splits;
+            const int64_t npieces = pf_chunks / pf_piece16;
+            const int64_t mine = (npieces - xcd + 7) / 8;                       // pieces of this XCD
+            const int64_t vtotal = mine * pf_piece16, T = (int64_t)count * (64 * NW);
+            for (int64_t v = (int64_t)rank * (64 * NW) + threadIdx.x; v < vtotal; v += 2 * T) {
+                const int64_t v2 = v + T;
+                const int64_t q = v / pf_piece16, o = v - q * pf_piece16;
+                const u32x4 a = pf[(xcd + 8 * q) * pf_piece16 + o];
+                u32x4 b = {0, 0, 0, 0};
+                if (v2 < vtotal) {
+                    const int64_t q2 = v2 / pf_piece16, o2 = v2 - q2 * pf_piece16;
+                    b = pf[(xcd + 8 * q2) * pf_piece16 + o2];
+                }
+                acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
+            }
+            if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
+            return;
+        }
         const int64_t nthreads = (int64_t)gridDim.x * ((int)gridDim.y - splits) * (64 * NW);
         int64_t i = ((int64_t)((int)blockIdx.y - splits) * gridDim.x + blockIdx.x) * (64 * NW) + threadIdx.x;
-        uint32_t acc = 0;
         for (; i + 3 * nthreads < pf_chunks; i += 4 * nthreads) {
             const u32x4 a = pf[i], b = pf[i + nthreads], c = pf[i + 2 * nthreads], d = pf[i + 3 * nthreads];
             acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
@@ -1451,15 +1478,17 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     }
     dim3 grid((unsigned)n_kv_head, (unsigned)(splits + pf_rows));
     hipStream_t s = (hipStream_t)stream;
+    static const int pf_piece_env = getenv("CQ_PF_PIECE") ? atoi(getenv("CQ_PF_PIECE")) : 0;
+    const int pf_piece16 = n_kv_head == 8 ? pf_piece_env / 16 : 0;
 #define CQ_ATTD(HH, GG)                                                                                                                   \
     if (fine)                                                                                                                             \
         hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 8, 64>), grid, dim3(64 * 8), 0, s, pos_dev, q_dev, k_cache_dev, cos_dev, sin_dev, (int)pos, \
                            (int)splits, (int)ctx, scale, v_cache_dev, k_new_dev, v_new_dev, part, (const u32x4 *)prefetch_dev, pf_chunks,   \
-                           (uint32_t *)nullptr, out_dev, counters);                                                                       \
+                           (uint32_t *)nullptr, out_dev, counters, pf_piece16);                                                           \
     else                                                                                                                                  \
         hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 16, 128>), grid, dim3(64 * 16), 0, s, pos_dev, q_dev, k_cache_dev, cos_dev, sin_dev,       \
                            (int)pos, (int)splits, (int)ctx, scale, v_cache_dev, k_new_dev, v_new_dev, part, (const u32x4 *)prefetch_dev,     \
-                           pf_chunks, (uint32_t *)nullptr, out_dev, counters)
+                           pf_chunks, (uint32_t *)nullptr, out_dev, counters, pf_piece16)
     if (head_dim == 128) {
         switch (G) {
             case 1: CQ_ATTD(128, 1); break;

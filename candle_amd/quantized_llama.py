@@ -113,6 +113,13 @@ class ModelWeights:
         # would pull through the memory-side cache ahead of the kernels that stream them.  Measured on the 8B shape:
         # no gain at 4-24 MB and a loss beyond (the time moves into the attention launch), so it is off.
         self.prefetch_bytes = 0
+        # Single-token steps can run the two matvecs of the feed-forward as one cooperative launch (cq_nn_decode_mlp) where a kernel
+        # exists for the formats and shapes; every such step is valid only while coop_error() is False (checked by forward and
+        # generate_greedy).  Off: measured on the 8B shape the launch takes 26.4 us against 24.2 us for the two launches it replaces
+        # (672 against 705 tok/s): the barrier and the acknowledged stores cost more than the kernel boundary they replace, and the
+        # weights requested ahead of the barrier do not make up for it.
+        self.coop = False
+        self.coop_sync = None
         self.tap = None                    # tests: called as tap(stage, layer) after each launch of an eager forward
 
     # ------------------------------------------------------------------------------------------ construction
@@ -489,6 +496,14 @@ class ModelWeights:
             consumers = [nxt["attention_wq"], nxt["attention_wk"], nxt["attention_wv"]] if nxt else [self.output]
             n_split = L.cq_nn_qmatmul_split_planes(int(w2.dtype), w2.k) if self.split_w2 and all_full and cfg.hidden <= 4096 and \
                 all(one_step(c) for c in consumers) else 0
+            if self.coop and not n_split and w1.dtype == w3.dtype and self.tap is None:
+                # both matvecs of the feed-forward in one cooperative launch (CQ_ERR_RANGE: no kernel for these formats / shapes)
+                rc = L.cq_nn_decode_mlp(int(w1.dtype), w1.ptr, w3.ptr, int(w2.dtype), w2.ptr, cur, part.data_ptr(), lw.ffn_norm.data_ptr(),
+                                        cfg.rms_eps, self.h.data_ptr(), cfg.hidden, cfg.ffn, self._coop_sync().data_ptr(), sp)
+                if rc == 0:
+                    continue
+                if rc != -6:
+                    ck("cq_nn_decode_mlp", rc)
             if w1.dtype == w3.dtype and w1.dtype in full and one_step(w1):
                 # h = silu(w1 xn) * (w3 xn) straight out of the paired-row matvec                    :56-63
                 ck("cq_nn_qmatmul_norm_swiglu", L.cq_nn_qmatmul_norm_swiglu(int(w1.dtype), w1.ptr, w3.ptr, cur, part.data_ptr(),
@@ -509,6 +524,22 @@ class ModelWeights:
         norm_mm(self.output, cfg.vocab, self.norm, self.logits.data_ptr())
         tap("head", -1)
 
+    def _coop_sync(self) -> torch.Tensor:
+        if self.coop_sync is None:
+            self.coop_sync = torch.zeros(self.L.cq_nn_coop_sync_bytes() // 4, dtype=torch.int32, device=self.device)
+        return self.coop_sync
+
+    def coop_error(self) -> bool:
+        """Whether a cooperative launch since the last call gave up waiting (synchronizes).  The steps enqueued since then are
+        invalid; the sync words are cleared so that cooperative launches can be used again."""
+        if self.coop_sync is None:
+            return False
+        bad = bool(int(self.coop_sync[1056]) != 0)          # CQ_NN_COOP_ERR_WORD
+        if bad:
+            self.coop_sync.zero_()
+            torch.cuda.synchronize(self.device)
+        return bad
+
     def forward(self, x: torch.Tensor, index_pos: int) -> torch.Tensor:
         """ModelWeights::forward: token ids [1, seq_len] at positions index_pos.. -> logits [1, vocab] of the last token."""
         if x.dim() != 2 or x.shape[0] != 1:
@@ -521,6 +552,14 @@ class ModelWeights:
         ids = x.to(device=self.device, dtype=torch.int32).contiguous()
         sp = torch.cuda.current_stream(self.device).cuda_stream
         self._enqueue(ids.data_ptr(), rows, index_pos, None, index_pos + rows, sp)
+        if rows == 1 and self.coop and self.coop_sync is not None and self.coop_error():
+            # a cooperative launch gave up waiting (the GPU is shared, or fewer compute units than workgroups were free):
+            # the same step through the chain of launches
+            self.coop = False
+            try:
+                self._enqueue(ids.data_ptr(), rows, index_pos, None, index_pos + rows, sp)
+            finally:
+                self.coop = True
         return self.logits.clone()
 
     # ------------------------------------------------------------------------------------------ greedy decode
@@ -595,5 +634,13 @@ class ModelWeights:
                     self._decode_step_dev(max_kv, stream.cuda_stream)
         torch.cuda.synchronize(dev)
         t2 = time.perf_counter()
+        if self.coop and self.coop_error():
+            # a cooperative launch gave up waiting for workgroups that were not running (a shared GPU): its tokens are invalid.
+            # The whole generation again through the chains of launches, which this model then keeps to.
+            import warnings
+            warnings.warn("a cooperative decode launch timed out; falling back to one launch per matvec")
+            self.coop = False
+            self._graph = None
+            return self.generate_greedy(prompt, n_new, use_graph)
         tokens = self.history_dev[:n_new].cpu().tolist()
         return {"tokens": tokens, "prompt_seconds": prompt_seconds, "decode_seconds": t2 - t1, "decode_steps": steps}

@@ -156,6 +156,32 @@ int cq_nn_qmatmul_residual_attn_merge(int w_dtype, const void *w_dev, const floa
                                       float *residual_dev, float *sumsq_partials_out_dev, const float *planes_dev, int64_t n_planes, int64_t k,
                                       int64_t n, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Cooperative decode launches: several of the dependent single-row calls above as ONE launch of 256 workgroups whose phases
+ * are separated by a barrier across the launch instead of a kernel boundary; a workgroup that waits has already requested
+ * the first weight steps of the next phase, so the HBM keeps streaming across the hand-over.  Results are bit-identical to
+ * the chain of calls they replace.  No counterpart in the reference (quantized_llama.rs:56-63, 191-266, 584-591 are tensor ops).
+ *
+ * sync_dev: cq_nn_coop_sync_bytes() bytes, 128-byte aligned, zero before the first use and owned by these calls afterwards
+ * (counters that only grow).  Word CQ_NN_COOP_ERR_WORD is the error word: every wait inside the kernels is bounded (4 ms), and a
+ * workgroup that gives up sets it, stops waiting and finishes; the step's results are then invalid.  A caller checks the word
+ * when it next synchronizes (at the latest before it uses a sampled token), and after an error clears all of sync_dev and
+ * repeats the step through the chain of calls.
+ * The launch needs all of its workgroups resident at once: CQ_ERR_RANGE on a device with fewer than 256 compute units, and for
+ * formats or shapes without a cooperative kernel (use the chain of calls).  Another process computing on the same GPU can make
+ * the waits expire.
+ *
+ * cq_nn_decode_mlp   residual[hidden] += W2 . q(silu(W1 . xn) * (W3 . xn)), xn = q(rms_norm(residual) * norm_weight)
+ *                    = cq_nn_qmatmul_norm_swiglu followed by cq_nn_qmatmul_residual (Mlp::forward and the add of :590-591).
+ *                    sumsq_partials_dev: sum(residual^2) in, and of the updated row out; h_dev [ffn]: scratch for the activation.
+ *                    W1 / W3 Q4_K, W2 Q4_K or Q6_K; hidden <= 4096.
+ * ------------------------------------------------------------------------------------------- */
+#define CQ_NN_COOP_ERR_WORD 1056
+int64_t cq_nn_coop_sync_bytes(void);
+int cq_nn_decode_mlp(int w13_dtype, const void *w1_dev, const void *w3_dev, int w2_dtype, const void *w2_dev, float *residual_dev,
+                     float *sumsq_partials_dev, const float *norm_weight_dev, float eps, float *h_dev, int64_t hidden, int64_t ffn, void *sync_dev,
+                     void *stream);
+
 /* Greedy sampling (LogitsProcessor with Sampling::ArgMax, candle-examples/examples/quantized/main.rs:603-604):
  * token_out[0] = index of the largest logit (lowest index on ties).  Optional bookkeeping for graph replay:
  * history_dev[*counter_dev] = token; *counter_dev += 1; *pos_dev += 1.
