@@ -31,6 +31,7 @@ SIGNATURES = {
     "cq_matvec": (_int, [_int, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
     "cq_matmul": (_int, [_int, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "cq_qmatmul_workspace_bytes": (_i64, [_int, _i64, _i64, _i64]),
+    "cq_qmatmul_stream_step_bytes": (_i64, [_int, _i64, _i64]),
     "cq_qmatmul_forward": (_int, [_int, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_static_workspace_bytes": (_i64, []),
     "cq_qmatmul_forward_static": (_int, [_int, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
@@ -64,7 +65,7 @@ SIGNATURES = {
     "cq_nn_attention_decode_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "cq_nn_attention_decode_splits": (_i64, [_i64]),
     "cq_nn_attention_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64,
-                                      _vp]),
+                                      _i64, _vp]),
     "cq_nn_coop_sync_bytes": (_i64, []),
     "cq_nn_decode_mlp": (_int, [_int, _vp, _vp, _int, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp, _vp]),
     "cq_nn_silu_mul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),

@@ -24,7 +24,7 @@ LIB = os.path.join(HERE, "libcandle_hip_quant.so")
 
 LIB_BENCH = os.path.join(HERE, "libcq_bench.so")
 
-SOURCES = ["cq_api.hip", "cq_dequant.hip", "cq_actquant.hip", "cq_matvec.hip", "cq_matmul.hip", "cq_moe.hip", "cq_quantize.hip", "cq_nn.hip", "cq_layer.hip"]
+SOURCES = ["cq_api.hip", "cq_dequant.hip", "cq_actquant.hip", "cq_matvec.hip", "cq_matmul.hip", "cq_moe.hip", "cq_quantize.hip", "cq_nn.hip", "cq_layer.hip", "cq_matvec_batch.hip"]
 # the benchmark's plain-read yardstick kernel: a library of its own, not part of the C ABI
 BENCH_SOURCES = ["cq_bench.hip"]
 

@@ -119,3 +119,13 @@ __device__ __forceinline__ void cq_quantize_q80_span(const void *x, int64_t span
     if (valid) cq_load4<XDT>(x, base, v);
     cq_quantize_q80_vals(v, valid, base, lane, qs, ds);
 }
+
+// silu(gate) * up computed on the fly (the expression of silu_mul_kernel) and quantized: the f32 product never exists in
+// memory.  Row r of the product is gate[r * gate_stride + i] , up[r * up_stride + i], i < 256 kb.
+__device__ __forceinline__ void cq_load_swiglu4(const float *gate, const float *up, int64_t gi, int64_t ui, float v[4]) {
+    const f32x4 g = *reinterpret_cast<const f32x4 *>(gate + gi), u = *reinterpret_cast<const f32x4 *>(up + ui);
+    v[0] = g.x / (1.0f + expf(-g.x)) * u.x;
+    v[1] = g.y / (1.0f + expf(-g.y)) * u.y;
+    v[2] = g.z / (1.0f + expf(-g.z)) * u.z;
+    v[3] = g.w / (1.0f + expf(-g.w)) * u.w;
+}

@@ -43,15 +43,6 @@ __global__ __launch_bounds__(256) void quantize_q80_gather_kernel(const float *_
     cq_quantize_q80_vals(v, true, span * 256 + lane * 4, lane, qs, ds);
 }
 
-// silu(gate) * up computed on the fly (the expression of silu_mul_kernel) and quantized: the f32 product never exists in
-// memory.  Row r of the product is gate[r * gate_stride + i] , up[r * up_stride + i], i < 256 kb.
-__device__ __forceinline__ void load_swiglu4(const float *gate, const float *up, int64_t gi, int64_t ui, float v[4]) {
-    const f32x4 g = *reinterpret_cast<const f32x4 *>(gate + gi), u = *reinterpret_cast<const f32x4 *>(up + ui);
-    v[0] = g.x / (1.0f + expf(-g.x)) * u.x;
-    v[1] = g.y / (1.0f + expf(-g.y)) * u.y;
-    v[2] = g.z / (1.0f + expf(-g.z)) * u.z;
-    v[3] = g.w / (1.0f + expf(-g.w)) * u.w;
-}
 __global__ __launch_bounds__(256) void quantize_q8k_swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up, int64_t gate_stride,
                                                                   int64_t up_stride, int kb, int8_t *__restrict__ qs, float *__restrict__ dout,
                                                                   int16_t *__restrict__ bsums, int64_t n_blocks) {
@@ -60,7 +51,7 @@ __global__ __launch_bounds__(256) void quantize_q8k_swiglu_kernel(const float *_
     const int lane = threadIdx.x & 63;
     const int64_t row = blk / kb, off = (blk - row * kb) * 256 + lane * 4;
     float v[4];
-    load_swiglu4(gate, up, row * gate_stride + off, row * up_stride + off, v);
+    cq_load_swiglu4(gate, up, row * gate_stride + off, row * up_stride + off, v);
     cq_quantize_q8k_vals(v, blk, lane, qs, dout, bsums);
 }
 __global__ __launch_bounds__(256) void quantize_q80_swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up, int64_t gate_stride,
@@ -71,7 +62,7 @@ __global__ __launch_bounds__(256) void quantize_q80_swiglu_kernel(const float *_
     const int lane = threadIdx.x & 63;
     const int64_t row = span / kb, off = (span - row * kb) * 256 + lane * 4;
     float v[4];
-    load_swiglu4(gate, up, row * gate_stride + off, row * up_stride + off, v);
+    cq_load_swiglu4(gate, up, row * gate_stride + off, row * up_stride + off, v);
     cq_quantize_q80_vals(v, true, span * 256 + lane * 4, lane, qs, ds);
 }
 

@@ -196,6 +196,9 @@ int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float
 int64_t cq_qmatmul_workspace_bytes(int w_dtype, int64_t m, int64_t k, int64_t n) {
     if (check_mm_shape(w_dtype, k, n, m)) return -1;
     int64_t bytes = cq_act_layout(w_dtype, k, m).total;
+    // the batched matvec lays the rows out as matrix operands, 16 row slots whatever the batch
+    const int64_t batch_ws = cq_matvec_batch_workspace(w_dtype, k, m);
+    if (batch_ws > bytes) bytes = batch_ws;
     // the MFMA path writes f32 and converts afterwards when the caller wants f16 / bf16; small grids split K into
     // partial planes that a second kernel adds up
     if (m > CQ_MATVEC_MAX_ROWS || cq_use_mfma(w_dtype, m, k)) {
@@ -221,6 +224,10 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     // (Q4_1, Q5_0, Q5_1, Q2K, Q3K have the fused instance for f32 activations only)
     if (m <= 2 && (cq_full_matvec(w_dtype) || x_dtype == CQ_F32))
         return cq_matvec_fused_launch(w_dtype, w_dev, x_dev, x_dtype, dst_dev, dst_dtype, k, n, m, n, s);
+    // 3..16 rows of Q4_K: one small kernel quantizes the rows, then the weights are read once at streaming speed with the rows
+    // as the second operand of the int8 matrix cores
+    if (m >= 3 && cq_matvec_batch_takes(w_dtype, w_dev, k, n, m))
+        return cq_matvec_batch_launch(w_dtype, w_dev, x_dev, x_dtype, workspace_dev, dst_dev, dst_dtype, k, n, m, n, s);
     // 3..8 rows: every workgroup re-quantizing all rows costs more than one small kernel that does it once
     if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) {
         if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
@@ -235,7 +242,13 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
     return cq_convert_f32_launch(tmp, dst_dev, dst_dtype, m * n, s);
 }
 
-int64_t cq_static_workspace_bytes(void) { return CQ_STATIC_WORKSPACE_BYTES; }
+int64_t cq_static_workspace_bytes(void) {
+    // also looks the array's address up for the current device (when one can be used), so that a caller who asks for the
+    // size before capturing a graph has the one-time lookup, which may load the code object, behind it
+    void *ws = nullptr;
+    (void)static_workspace(&ws);
+    return CQ_STATIC_WORKSPACE_BYTES;
+}
 
 int cq_qmatmul_forward_static(int w_dtype, const void *w_dev, const void *x_dev, int x_dtype, void *dst_dev, int dst_dtype,
                               int64_t m, int64_t k, int64_t n, void *stream) {
@@ -263,6 +276,8 @@ int cq_nn_qmatmul_swiglu_rows(int w_dtype, const void *w_dev, const float *gate_
     if (!aligned(gate_dev, 16) || !aligned(up_dev, 16) || !aligned(workspace_dev, 256) || !aligned(dst_dev, 4)) return CQ_ERR_ALIGN;
     if (workspace_bytes < cq_qmatmul_workspace_bytes(w_dtype, m, k, n)) return CQ_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
+    if (m >= 3 && cq_matvec_batch_takes(w_dtype, w_dev, k, n, m))          // the kernel cq_qmatmul_forward takes for these shapes
+        return cq_matvec_batch_swiglu_launch(w_dtype, w_dev, gate_dev, up_dev, gate_stride, up_stride, workspace_dev, dst_dev, CQ_F32, k, n, m, n, s);
     if ((rc = cq_quantize_act_swiglu_launch(w_dtype, gate_dev, up_dev, gate_stride, up_stride, workspace_dev, k, m, s))) return rc;
     if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, CQ_F32, k, n, m, n, s);
     float *tmp = (float *)((uint8_t *)workspace_dev + cq_act_layout(w_dtype, k, m).total);

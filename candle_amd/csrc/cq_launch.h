@@ -13,6 +13,14 @@ int cq_matvec_launch(int w_dtype, const void *w, const void *scratch, void *dst,
 // same, over an already resolved (possibly row-offset) view of the activation scratch
 int cq_matvec_launch_av(int w_dtype, const void *w, const ActView &av, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows,
                         int64_t stride_dst, hipStream_t s);
+// 3 .. 16 rows on the int8 matrix cores (quantized into `workspace` by a kernel of its own), the weights read once (cq_matvec_batch.hip); CQ_ERR_RANGE: not a call it takes
+bool cq_matvec_batch_takes(int w_dtype, const void *w, int64_t k, int64_t n, int64_t rows);
+int64_t cq_matvec_batch_workspace(int w_dtype, int64_t k, int64_t rows);
+int cq_matvec_batch_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *workspace, void *dst, int dst_dtype, int64_t k, int64_t n,
+                           int64_t rows, int64_t stride_dst, hipStream_t s);
+// the same over rows silu(gate[r]) * up[r] (f32, row strides in floats)
+int cq_matvec_batch_swiglu_launch(int w_dtype, const void *w, const float *gate, const float *up, int64_t gate_stride, int64_t up_stride, void *workspace,
+                                  void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s);
 // QMatMul::forward for <= CQ_MATVEC_MAX_ROWS rows with the activation quantization fused into the matvec kernel
 int cq_matvec_fused_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *dst, int dst_dtype, int64_t k, int64_t n,
                            int64_t rows, int64_t stride_dst, hipStream_t s);

@@ -7,6 +7,7 @@
 //
 // candle runs these as separate tensor ops (candle-transformers/src/models/quantized_llama.rs:56-63, 191-266, 584-591).
 #include "../../include/candle_hip_nn.h"
+#include "../../include/candle_hip_quant.h"
 #include "cq_coop.h"
 #include "cq_stream_body.h"
 
@@ -113,6 +114,22 @@ extern "C" void cl_set_stamps(uint32_t *p) { cl_stamps_dev = p; }
 #endif
 
 extern "C" {
+
+// bytes of one wave step of the streaming decode matvec over this weight (the unit in which its workgroups, and so the
+// XCDs, take turns along the tensor); 0 when the (format, k, n) does not take the streaming kernel
+int64_t cq_qmatmul_stream_step_bytes(int w_dtype, int64_t k, int64_t n) {
+    StreamGeom g;
+    bool okk = false;
+    switch (w_dtype) {
+        case CQ_Q4_0: okk = stream_geom<CQ_Q4_0>(g, k, n, CQ_F32); break;
+        case CQ_Q8_0: okk = stream_geom<CQ_Q8_0>(g, k, n, CQ_F32); break;
+        case CQ_Q4K: okk = stream_geom<CQ_Q4K>(g, k, n, CQ_F32); break;
+        case CQ_Q5K: okk = stream_geom<CQ_Q5K>(g, k, n, CQ_F32); break;
+        case CQ_Q6K: okk = stream_geom<CQ_Q6K>(g, k, n, CQ_F32); break;
+        default: break;
+    }
+    return okk ? g.step_bytes : 0;
+}
 
 int64_t cq_nn_coop_sync_bytes(void) { return COOP_SYNC_BYTES; }
 

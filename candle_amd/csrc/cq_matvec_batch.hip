@@ -1,0 +1,338 @@
+// Batched decode matvec on the int8 matrix cores:  dst[b, row] = sum_k W[row, k] * x^[b, k]  for 3 .. 16 activation rows,
+// Q4_K weights, the weights read once at streaming speed.
+//
+// The single-row kernels pay per activation row for every dot product (v_dot4 on the vector ALU), and the prefill tiles pay
+// per WEIGHT for folding the sub-block scales into the matrix operands — worth it when hundreds of rows share a weight tile,
+// not for a handful.  With at most 16 rows the cheap side is the OUTPUT: one v_mfma_i32_16x16x32_i8 is exactly one
+// 32-element sub-block of 16 weight rows against 16 activation rows, its int32 result is the sub-block dot the CPU forms
+// (k_quants.rs:1460-1540, BlockQ4K x BlockQ8K), and the 6-bit sub-block scale is applied to the 4 results a lane holds
+// (two vector instructions per result).  A weight costs a quarter of a vector instruction per nibble (one AND per four),
+// whatever the number of rows.
+//
+// Work split.  A workgroup takes blocks of 16 weight rows (block m = blockIdx.x, + gridDim.x, ...).  Its 8 waves split K:
+// wave w owns the super-block columns [w * CPW, (w + 1) * CPW) of every row, and keeps the int8 activations of those columns,
+// for all rows of the batch, in registers as matrix operands for the whole kernel (lane (c, kg): 8 consecutive values of
+// batch row c per sub-block), so the only stream is the weights: a block of 16 rows is one contiguous piece of the tensor,
+// which the waves copy HBM -> LDS together, one KB per instruction (buffer loads that write LDS directly; each wave copying
+// only its own columns, 16 short runs per tile, was tried first: those instructions take five times as long to issue), into
+// a ring of tiles, two blocks ahead.  The partial sums of the 8 waves meet in LDS once per block and are added in wave order.
+//
+// The activations are quantized exactly like BlockQ8K::from_float by a small kernel of this file, which leaves them laid out
+// as the matrix operands the waves load.
+#include "cq_actquant.h"
+#include "cq_device.h"
+#include "cq_fmt.h"
+#include "cq_launch.h"
+#include "cq_stream.h"
+
+#ifdef CL_STAMPS
+#define QB_STAMP(i) do { if ((threadIdx.x & 63) == 0) qb_stamp_lds[threadIdx.x >> 6][(i)] = (uint32_t)__builtin_amdgcn_s_memrealtime(); } while (0)
+static uint32_t *qb_stamps_dev = nullptr;
+extern "C" void qb_set_stamps(uint32_t *p) { qb_stamps_dev = p; }
+#else
+#define QB_STAMP(i) do { } while (0)
+#endif
+
+namespace {
+
+#ifdef CL_STAMPS
+__shared__ uint32_t qb_stamp_lds[8][16];
+#endif
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int QB_NW = 8;
+constexpr int QB_BB = 144;                        // bytes of a Q4_K super-block
+constexpr int QB_RED_BYTES = QB_NW * 64 * 16;     // the waves' partial results of one block of rows
+constexpr int QB_LDS_BYTES = 160 * 1024;
+// A tile (16 rows of up to 8 * CPW super-blocks) is copied by whole instructions of 64 lanes x 16 bytes, each wave the same number:
+// it occupies a multiple of 8 KB.
+constexpr int qb_tile_instr(int cpw) { return (16 * 8 * cpw * QB_BB + 8 * 1024 - 1) / (8 * 1024); }       // copy instructions per wave and tile
+// In LDS every KB of a tile is followed by 16 unused bytes: a row is 9 * 16 * (super-blocks per row) bytes, for rows of 16
+// super-blocks a multiple of all 64 banks, and the 16 lanes that read the same bytes of 16 different rows would meet on one bank.
+constexpr int QB_KB = 1024 + 16;
+// a tile of a block of `block_bytes`: its KBs, and one more that takes the zeros of the copy instructions beyond the block
+__host__ __device__ constexpr int qb_tile_bytes(int block_bytes) { return ((block_bytes + 1023) / 1024 + 1) * QB_KB; }
+
+// ---- the activations, quantized like BlockQ8K::from_float and laid out as this kernel's matrix operands ----
+// For super-block column s of the row length, 16 batch slots (rows beyond the batch are zeros):
+//   operands [s][sub-block j < 8][kg < 4][batch slot c < 16][8 bytes]   values 32 j + 8 kg .. + 7 of column s of row c: what lane
+//                                                                      (c, kg) feeds the matrix core for sub-block j, 512
+//                                                                      contiguous bytes per wave load;
+//   records  [s][c] { u8 bl[8], i8 bh[8] (sum of sub-block j = 128 * bh_j + bl_j), f32 d, 12 bytes unused }
+constexpr int QB_OP_COL_BYTES = 8 * 4 * 16 * 8;       // 4096
+constexpr int QB_REC_BYTES = 32;
+__host__ __device__ inline int64_t qb_operand_bytes(int64_t bpr) { return bpr * (QB_OP_COL_BYTES + 16 * QB_REC_BYTES); }
+
+// XDT < 0: the rows are silu(x[c]) * up[c], rows of f32 with strides of their own (a feed-forward's w2 over several rows)
+template <int XDT>
+__global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict__ x, const float *__restrict__ up, int64_t x_stride, int64_t up_stride,
+                                                          uint8_t *__restrict__ op, int bpr, int rows) {
+    const int span = (int)blockIdx.x * 4 + ((int)threadIdx.x >> 6);          // span = s * 16 + c
+    if (span >= bpr * 16) return;
+    const int lane = threadIdx.x & 63, s = span >> 4, c = span & 15;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (c < rows) {
+        if constexpr (XDT < 0) cq_load_swiglu4((const float *)x, up, c * x_stride + s * 256 + lane * 4, c * up_stride + s * 256 + lane * 4, v);
+        else cq_load4<XDT>(x, c * x_stride + s * 256 + lane * 4, v);
+    }
+    // the arithmetic of cq_quantize_q8k_vals (cq_actquant.h): the first element of largest magnitude sets the scale
+    float amax = 0.0f;
+    int idx = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float a = fabsf(v[i]);
+        if (amax < a) { amax = a; idx = i; }
+    }
+    const float wmax = wave_max_nonneg(amax);
+    const int cand = wave_min_int((amax == wmax && wmax != 0.0f) ? lane * 4 + idx : 256);
+    const float mine = idx == 0 ? v[0] : idx == 1 ? v[1] : idx == 2 ? v[2] : v[3];
+    const float maxv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), (cand >> 2) & 63));
+    uint32_t packed = 0;
+    int lsum = 0;
+    float d = 0.0f;
+    if (wmax != 0.0f) {
+        const float iscale = -127.0f / maxv;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int q = cq_round_sat_i8(iscale * v[i]);
+            lsum += q;
+            packed |= (uint32_t)(q & 0xff) << (8 * i);
+        }
+        d = 1.0f / iscale;
+    }
+    // elements 4 lane .. + 3: sub-block lane / 8, values 4 (lane % 8) .. + 3 of it: lane group kg = (lane % 8) / 2, dword lane % 2
+    uint8_t *colp = op + (int64_t)s * QB_OP_COL_BYTES;
+    *(uint32_t *)(colp + (((lane >> 3) * 4 + ((lane & 7) >> 1)) * 16 + c) * 8 + 4 * (lane & 1)) = packed;
+    const int s32 = oct_sum(lsum);                        // the sum of the 32-element sub-block, in its eight lanes
+    uint32_t bl[2] = {0, 0}, bh[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int sj = __builtin_amdgcn_readlane(s32, 8 * j);
+        bl[j >> 2] |= (uint32_t)(sj & 127) << (8 * (j & 3));
+        bh[j >> 2] |= (uint32_t)((sj >> 7) & 255) << (8 * (j & 3));
+    }
+    if (lane == 0) {
+        uint8_t *rec = op + (int64_t)bpr * QB_OP_COL_BYTES + (int64_t)span * QB_REC_BYTES;
+        *(u32x4 *)rec = u32x4{bl[0], bl[1], bh[0], bh[1]};
+        *(float *)(rec + 16) = d;
+    }
+}
+
+template <int CPW, int DEPTH>
+__global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ op, void *__restrict__ dst, int n, int bpr,
+                                                              int rows, int dst_dtype, int64_t stride_dst
+#ifdef CL_STAMPS
+                                                              , uint32_t *stamps
+#endif
+                                                              ) {
+    constexpr int NIW = qb_tile_instr(CPW);       // copy instructions per wave and tile (those beyond the block copy nothing)
+    static_assert((DEPTH - 1) * NIW <= 63 && DEPTH >= 2, "counted waits");
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int bx = blockIdx.x, gx = gridDim.x;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, kg = lane >> 4;
+    const int col0 = wv * CPW;
+    const int ncols = max(0, min(CPW, bpr - col0));
+    const int RS = bpr * QB_BB;                   // bytes of a row, in memory and in a tile
+    const int block_bytes = 16 * RS;
+    const int nkb = (block_bytes + 1023) >> 10;   // KBs of a tile
+    const int TILE = qb_tile_bytes(block_bytes);
+    float *red = (float *)(lds + DEPTH * TILE);                              // [8 waves][64 lanes][4]
+
+    // ---- the weight stream ----
+    const int nsteps = (n + 15) >> 4;
+    const int64_t w_bytes = (int64_t)n * RS;
+    // instruction t of wave w copies KB number t * 8 + w of the block
+    auto issue = [&](int i) {
+        const int m = bx + i * gx;
+        const bool live = m < nsteps;
+        const int64_t off = live ? (int64_t)m * block_bytes : 0;
+        const int64_t left = w_bytes - off;
+        const int bytes = live ? (int)(left < block_bytes ? left : block_bytes) : 0;      // an absent block: a descriptor of zero bytes
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(w + off), 0, bytes, 0x00020000);
+        uint8_t *tile = lds + (i % DEPTH) * TILE;
+#pragma unroll
+        for (int t = 0; t < NIW; t++) {
+            const int kb = min(t * QB_NW + wv, nkb);             // KB number nkb: beyond the block, nothing read, zeros into the spare KB
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(tile + kb * QB_KB), 16, lane * 16, kb * 1024, 0, 0);
+        }
+    };
+    issue(0);                                     // the first tile is on its way before anything else is asked for
+    asm volatile("" ::: "memory");
+
+    // ---- the wave's activations, in registers for the whole kernel ----
+    // The activations are the FIRST matrix operand (lane (c, kg): values 8 kg .. 8 kg + 7 of each sub-block of batch row c) and
+    // the weights the second, so a lane's four results belong to ONE weight row (row c of the block: one header to decode per
+    // column) and to the batch rows 4 kg + r, whose block sums and scales it keeps as well.
+    QB_STAMP(0);
+    long A[CPW][8];
+    u32x4 aux[CPW][4];                            // {bl 0-3, bl 4-7, bh 0-3, bh 4-7} of batch row 4 kg + r: sub-block sum j = 128 * bh_j + bl_j
+    float d8[CPW][4];
+    // (a wave's load of one operand is 512 contiguous bytes; the four lane groups read four records)
+#pragma unroll
+    for (int ci = 0; ci < CPW; ci++) {
+        const int col = min(col0 + ci, bpr - 1);
+        const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 8;          // lane = kg * 16 + c
+#pragma unroll
+        for (int j = 0; j < 8; j++) A[ci][j] = *(const long *)(colp + j * 512);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint8_t *rec = op + (int64_t)bpr * QB_OP_COL_BYTES + (int64_t)(col * 16 + 4 * kg + r) * QB_REC_BYTES;
+            aux[ci][r] = *(const u32x4 *)rec;
+            d8[ci][r] = *(const float *)(rec + 16);
+        }
+    }
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 1; i < DEPTH - 1; i++) issue(i);
+    const int my = bx < nsteps ? (nsteps - bx + gx - 1) / gx : 0;
+    QB_STAMP(1);
+    for (int i = 0; i < my; i++) {
+        // tile i has landed when this wave's copies of it have (at most the later tiles' outstanding) and every other wave's too
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * NIW) : "memory");
+        asm volatile("s_barrier" ::: "memory");
+        // (behind this barrier every wave has also finished the sums of block i - 1: `red` may be written again, and tile
+        // i - 1 is free, which is where tile i + 2 goes)
+        issue(i + DEPTH - 1);
+        const uint8_t *tile = lds + (i % DEPTH) * TILE;
+        if (i < 4) QB_STAMP(2 + 3 * i);
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ci = 0; ci < CPW; ci++) {
+            if (ci < ncols) {
+                const int o = c * RS + (col0 + ci) * QB_BB;                  // weight row c of the block, this column's super-block
+                auto at = [&](int off) { return tile + off + (off >> 10) * 16; };      // byte `off` of the block in the padded tile
+                const u32x4 hdr = *(const u32x4 *)at(o);
+                i32x4 cl[4], ch[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    // bytes 32g + 8kg .. + 7 of qs: low nibbles = sub-block 2g, high nibbles = sub-block 2g + 1
+                    const long qa = *(const long *)at(o + 16 + 32 * g + 8 * kg);
+                    const long lo = qa & 0x0f0f0f0f0f0f0f0fl, hi = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                    const i32x4 z = {0, 0, 0, 0};
+                    cl[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[ci][2 * g], lo, z, 0, 0, 0);
+                    ch[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[ci][2 * g + 1], hi, z, 0, 0, 0);
+                }
+                const QsScales s = qs_scales_k4(hdr.y, hdr.z, hdr.w);
+                int sc[8];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    sc[j] = (int)((s.scA >> (8 * j)) & 0xff);
+                    sc[4 + j] = (int)((s.scB >> (8 * j)) & 0xff);
+                }
+                const float dw = h2f(hdr.x), dm = h2f(hdr.x >> 16);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    int S = 0;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
+                    const int M = qs_dot_sums(s.mA, s.mB, aux[ci][r]);
+                    acc[r] += d8[ci][r] * (dw * (float)S - dm * (float)M);
+                }
+            }
+        }
+        if (i < 4) QB_STAMP(3 + 3 * i);
+        // ---- the eight K-slices of the block meet in LDS and are added in wave order ----
+        *(f32x4 *)(red + (wv * 64 + lane) * 4) = f32x4{acc[0], acc[1], acc[2], acc[3]};
+        // (barriers without the fence of __syncthreads(): the fence would wait for the copies in flight)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (tid < 256) {
+            const int l2 = tid & 63, r = tid >> 6;
+            float v = 0.0f;
+#pragma unroll
+            for (int w2 = 0; w2 < QB_NW; w2++) v += red[(w2 * 64 + l2) * 4 + r];
+            const int m = bx + i * gx;
+            const int row = m * 16 + (l2 & 15), br = 4 * (l2 >> 4) + r;
+            if (row < n && br < rows) store_out(dst, dst_dtype, (int64_t)br * stride_dst + row, v);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");          // the sums have left LDS before this wave reaches the next barrier
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");               // no copy may land in LDS after the workgroup has left
+#ifdef CL_STAMPS
+    QB_STAMP(15);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (tid < 128 && stamps) stamps[(bx * 8 + tid / 16) * 16 + tid % 16] = qb_stamp_lds[tid / 16][tid % 16];
+#endif
+}
+
+template <int CPW, int DEPTH>
+int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
+                 hipStream_t s) {
+    auto kern = qmb_q4k_kernel<CPW, DEPTH>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    const int64_t nsteps = (n + 15) / 16;
+    const unsigned grid = (unsigned)(nsteps < 256 ? nsteps : 256);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(QB_NW * 64), lds_bytes, s, (const uint8_t *)w, op, dst, (int)n, (int)(k / 256), (int)rows, dst_dtype,
+                       stride_dst
+#ifdef CL_STAMPS
+                       , qb_stamps_dev
+#endif
+    );
+    return (int)hipGetLastError();
+}
+// Three tiles where LDS holds them (the one being worked on and two on their way), else two.  (Four were measured slower:
+// with three tiles asked for at the start the first one lands 1 us later, and the steady state gains nothing.)
+template <int CPW>
+int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+    const int tile = qb_tile_bytes((int)(16 * (k / 256) * QB_BB));
+    const int fit = (QB_LDS_BYTES - QB_RED_BYTES - 1024) / tile;
+    if (fit >= 3) return launch_qmb_d<CPW, 3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)3 * tile + QB_RED_BYTES, s);
+    if (fit == 2) return launch_qmb_d<CPW, 2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)2 * tile + QB_RED_BYTES, s);
+    return CQ_ERR_RANGE;
+}
+
+}  // namespace
+
+// Does the batched matrix-core matvec take this call?  Q4_K, 3 .. 16 rows, rows of up to 24 super-blocks (three columns per wave:
+// beyond that the activations of a wave's columns no longer fit its registers).
+bool cq_matvec_batch_takes(int w_dtype, const void *w, int64_t k, int64_t n, int64_t rows) {
+    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= 24 && n >= 1 && n <= 0x7ffffff0 / 16 &&
+           n * (k / 256) * QB_BB < 0x7fffffffLL && ((uintptr_t)w & 15) == 0;
+}
+// bytes of workspace the call needs (the activations as matrix operands); 0 when the shape can never take this path
+int64_t cq_matvec_batch_workspace(int w_dtype, int64_t k, int64_t rows) {
+    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= 24 ? cq_align256(qb_operand_bytes(k / 256)) : 0;
+}
+
+// QMatMul::forward for 3 .. 16 rows of x: one small kernel quantizes them into `workspace`, then the weights are read once.
+// x_dtype < 0: the rows are silu(x) * up, f32, with row strides in floats (multiples of 4).
+static int qb_launch(int w_dtype, const void *w, const void *x, const float *up, int64_t x_stride, int64_t up_stride, int x_dtype, void *workspace,
+                     void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+    if (!cq_matvec_batch_takes(w_dtype, w, k, n, rows)) return CQ_ERR_RANGE;
+    const int bpr = (int)(k / 256);
+    const unsigned qgrid = (unsigned)((bpr * 16 + 3) / 4);
+    uint8_t *op = (uint8_t *)workspace;
+    switch (x_dtype) {
+        case -1: hipLaunchKernelGGL(qb_quantize_kernel<-1>, dim3(qgrid), dim3(256), 0, s, x, up, x_stride, up_stride, op, bpr, (int)rows); break;
+        case CQ_F32: hipLaunchKernelGGL(qb_quantize_kernel<CQ_F32>, dim3(qgrid), dim3(256), 0, s, x, up, x_stride, up_stride, op, bpr, (int)rows); break;
+        case CQ_F16: hipLaunchKernelGGL(qb_quantize_kernel<CQ_F16>, dim3(qgrid), dim3(256), 0, s, x, up, x_stride, up_stride, op, bpr, (int)rows); break;
+        case CQ_BF16: hipLaunchKernelGGL(qb_quantize_kernel<CQ_BF16>, dim3(qgrid), dim3(256), 0, s, x, up, x_stride, up_stride, op, bpr, (int)rows); break;
+        default: return CQ_ERR_DTYPE;
+    }
+    const int64_t cpw = (k / 256 + QB_NW - 1) / QB_NW;
+    switch (cpw) {
+        case 1: return launch_qmb<1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case 2: return launch_qmb<2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case 3: return launch_qmb<3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, s);
+        default: return CQ_ERR_RANGE;
+    }
+}
+int cq_matvec_batch_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *workspace, void *dst, int dst_dtype, int64_t k, int64_t n,
+                           int64_t rows, int64_t stride_dst, hipStream_t s) {
+    return qb_launch(w_dtype, w, x, nullptr, k, 0, x_dtype, workspace, dst, dst_dtype, k, n, rows, stride_dst, s);
+}
+int cq_matvec_batch_swiglu_launch(int w_dtype, const void *w, const float *gate, const float *up, int64_t gate_stride, int64_t up_stride, void *workspace,
+                                  void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+    return qb_launch(w_dtype, w, gate, up, gate_stride, up_stride, -1, workspace, dst, dst_dtype, k, n, rows, stride_dst, s);
+}
+
+#ifdef CL_STAMPS
+extern "C" int qb_debug_launch(const void *w, const void *x, void *workspace, void *dst, int64_t k, int64_t n, int64_t rows, void *stream) {
+    return cq_matvec_batch_launch(CQ_Q4K, w, x, CQ_F32, workspace, dst, CQ_F32, k, n, rows, n, (hipStream_t)stream);
+}
+#endif

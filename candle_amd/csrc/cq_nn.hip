@@ -6,8 +6,6 @@
 // decode position can be read from device memory so that a whole decode step (including "pick the next
 // token, advance the position") can be captured in a HIP graph and replayed without host round trips.
 #include "cq_device.h"
-#include <stdlib.h>
-
 #include "../../include/candle_hip_nn.h"
 
 namespace {
@@ -1452,9 +1450,10 @@ int64_t cq_nn_attention_decode_splits(int64_t max_kv_len) {
 int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const float *v_new_dev, float *k_cache_dev, float *v_cache_dev,
                            const float *cos_dev, const float *sin_dev, float *out_dev, const int32_t *pos_dev, int64_t pos, int64_t n_head,
                            int64_t n_kv_head, int64_t head_dim, int64_t ctx, int64_t max_kv_len, float scale, void *partials_dev,
-                           int64_t partials_bytes, const void *prefetch_dev, int64_t prefetch_bytes, void *stream) {
+                           int64_t partials_bytes, const void *prefetch_dev, int64_t prefetch_bytes, int64_t prefetch_piece_bytes, void *stream) {
     if (n_head <= 0 || n_kv_head <= 0 || n_head % n_kv_head || ctx <= 0 || pos < 0 || max_kv_len <= 0 || max_kv_len > ctx) return CQ_ERR_SHAPE;
     if (prefetch_bytes < 0 || (prefetch_bytes > 0 && (!prefetch_dev || misaligned(prefetch_dev, 16)))) return CQ_ERR_ALIGN;
+    if (prefetch_piece_bytes < 0 || prefetch_piece_bytes % 16 || prefetch_piece_bytes > 0x7fffffffLL) return CQ_ERR_ALIGN;
     if (head_dim != 64 && head_dim != 128) return CQ_ERR_RANGE;
     if (!q_dev || !k_new_dev || !v_new_dev || !k_cache_dev || !v_cache_dev || !cos_dev || !sin_dev || !partials_dev) return CQ_ERR_NULL;
     if (misaligned(q_dev, 16) || misaligned(k_new_dev, 16) || misaligned(v_new_dev, 16) || misaligned(k_cache_dev, 16) ||
@@ -1478,8 +1477,9 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     }
     dim3 grid((unsigned)n_kv_head, (unsigned)(splits + pf_rows));
     hipStream_t s = (hipStream_t)stream;
-    static const int pf_piece_env = getenv("CQ_PF_PIECE") ? atoi(getenv("CQ_PF_PIECE")) : 0;
-    const int pf_piece16 = n_kv_head == 8 ? pf_piece_env / 16 : 0;
+    // pieces go to the XCD of their consumer only where the grid's columns are the XCDs (workgroups are dealt to the 8 XCDs
+    // round-robin by linear index); other head counts read the range linearly
+    const int pf_piece16 = n_kv_head == 8 ? (int)(prefetch_piece_bytes / 16) : 0;
 #define CQ_ATTD(HH, GG)                                                                                                                   \
     if (fine)                                                                                                                             \
         hipLaunchKernelGGL((attn_decode_kernel<HH, GG, 8, 64>), grid, dim3(64 * 8), 0, s, pos_dev, q_dev, k_cache_dev, cos_dev, sin_dev, (int)pos, \

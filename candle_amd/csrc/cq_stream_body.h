@@ -197,7 +197,7 @@ __device__ __forceinline__ void qms_body(const uint8_t *__restrict__ w, const fl
     typedef StreamFmt<DT> SF;
     typedef StreamAct<MAXB> SA;
     constexpr bool RESID = epi_is_resid(EPI);
-    constexpr int SB = (COOP & CO_PRE) ? 8 : 0;            // (instrumented builds: where this phase's stamps go)
+    [[maybe_unused]] constexpr int SB = (COOP & CO_PRE) ? 8 : 0;            // (instrumented builds: where this phase's stamps go)
     constexpr bool PAIR = EPI == EPI_SWIGLU;               // two weight rows per output row: a step is two sub-steps, gate rows then up rows
     constexpr int SUBS = PAIR ? 2 : 1;
     // 16-byte-per-lane copies of the first step requested before the activation prologue; the rest follows it.
@@ -439,6 +439,9 @@ bool stream_geom(StreamGeom &g, int64_t k, int64_t n, int dst_dtype) {
     const int64_t bb = BlockInfo<DT>::bytes * (256 / BlockInfo<DT>::elems);       // bytes of 256 elements: a super-block, or eight blocks
     // every wave step must start on 16 bytes of the stream (Q6_K blocks are 210 bytes: steps of a multiple of 8 blocks)
     if (((64 >> sh) * bpr * bb) % 16) return false;
+    // the copies move whole dwords and their range check is per dword: a tensor of 2 (mod 4) bytes (Q6_K, odd block count)
+    // would lose the dword that holds its last two bytes, the f16 scale of the last block
+    if ((n * bpr * bb) % 4) return false;
     g.k = (int)k; g.n = (int)n; g.bpr = (int)bpr; g.lp_shift = sh;
     g.step_rows = 64 >> sh;
     g.step_bytes = (int)(g.step_rows * bpr * bb);

@@ -109,10 +109,12 @@ class ModelWeights:
         self.split_w2 = False              # ... and feed_forward_w2 as a K-split matvec (planes merged by its consumers) where the shapes allow it;
                                            # off: with every format of a Q4_K_M file on the streaming kernel the unsplit step is as fast (8B shape: 608 vs 603 tok/s)
         self.merge_in_wo = False           # merge the attention key splits in the prologue of attention_wo (else: in the attention kernel)
-        # bytes of the weights behind attention (wo, w1, w3, w2 are contiguous) that the attention launch's idle CUs
-        # would pull through the memory-side cache ahead of the kernels that stream them.  Measured on the 8B shape:
-        # no gain at 4-24 MB and a loss beyond (the time moves into the attention launch), so it is off.
-        self.prefetch_bytes = 0
+        # Bytes of the weights behind attention (wo, w1, w3, w2 are contiguous) that the attention launch's idle CUs read ahead of
+        # the kernels that stream them, each piece on the XCD whose L2 its consumer will look in.  Measured on the 8B shape
+        # (tok/s at 0 / 4 / 9.4 / 14 / 18 / 28 / 40 MB): 672 / 676 / 680 / 684 / 682 / 649 / 605, read linearly 672 / - / 675 / - / 677 /
+        # 673 / 656: all of attention_wo and the head of feed_forward_w1 pay, beyond what the L2s hold (8 x 4 MB) the time moves
+        # into the attention launch.
+        self.prefetch_bytes = 14 << 20
         # Single-token steps can run the two matvecs of the feed-forward as one cooperative launch (cq_nn_decode_mlp) where a kernel
         # exists for the formats and shapes; every such step is valid only while coop_error() is False (checked by forward and
         # generate_greedy).  Off: measured on the 8B shape the launch takes 26.4 us against 24.2 us for the two launches it replaces
@@ -479,7 +481,8 @@ class ModelWeights:
                                                                   cfg.n_head, cfg.n_kv_head, cfg.head_dim, cfg.ctx, max_kv_len, scale,
                                                                   self.attd_ws.data_ptr(), self.attd_ws.numel(),
                                                                   wo.ptr if self.prefetch_bytes else None,
-                                                                  min(self.prefetch_bytes, lw.prefetch_span), sp))
+                                                                  min(self.prefetch_bytes, lw.prefetch_span) // 16 * 16,
+                                                                  L.cq_qmatmul_stream_step_bytes(int(wo.dtype), wo.k, wo.n), sp))
             tap("attention", li)
             # attention_wo adds to the residual row, and folds the pending planes into it
             if merge_in_wo:

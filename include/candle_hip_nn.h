@@ -74,7 +74,11 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
  * Key rows of the cache beyond p, up to the end of the last split of max_kv_len (never beyond ctx), are read before the
  * position is known and masked afterwards: whatever they hold, NaN included, does not reach the result.
  * prefetch_dev / prefetch_bytes (optional, 16-byte aligned): a byte range that extra read-only workgroups of this
- * otherwise latency-bound launch pull through the memory-side cache, e.g. the weights of the kernels that follow.
+ * otherwise latency-bound launch pull into the caches, e.g. the weights of the kernels that follow.  With
+ * prefetch_piece_bytes > 0 (a multiple of 16; n_kv_head == 8) the range is taken as pieces of that size and piece p is read by
+ * a workgroup on XCD p % 8: with the piece = cq_qmatmul_stream_step_bytes() of the weight that starts at prefetch_dev, every
+ * piece lands in the L2 of the XCD whose workgroup will stream it (the L2s of the eight XCDs are separate, and what one holds
+ * survives the kernel boundary).
  * No counterpart in the reference, which runs these as separate tensor ops (quantized_llama.rs:217-261). */
 #define CQ_NN_ATTD_HEADER_BYTES 256
 int64_t cq_nn_attention_decode_workspace_bytes(int64_t n_head, int64_t head_dim, int64_t max_kv_len);
@@ -82,7 +86,7 @@ int64_t cq_nn_attention_decode_splits(int64_t max_kv_len);
 int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const float *v_new_dev, float *k_cache_dev, float *v_cache_dev,
                            const float *cos_dev, const float *sin_dev, float *out_dev, const int32_t *pos_dev, int64_t pos, int64_t n_head,
                            int64_t n_kv_head, int64_t head_dim, int64_t ctx, int64_t max_kv_len, float scale, void *partials_dev,
-                           int64_t partials_bytes, const void *prefetch_dev, int64_t prefetch_bytes, void *stream);
+                           int64_t partials_bytes, const void *prefetch_dev, int64_t prefetch_bytes, int64_t prefetch_piece_bytes, void *stream);
 
 /* out = silu(gate) * up with silu(v) = v / (1 + exp(-v)): Mlp::forward, quantized_llama.rs:56-63
  * (candle_nn::ops::silu, candle-core/src/op.rs Silu::f32).  gate/up rows may be strided views of one buffer. */

@@ -136,6 +136,11 @@ int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float
  * at least cq_qmatmul_workspace_bytes(w_dtype, m, k, n) bytes.
  * ------------------------------------------------------------------------------------------- */
 int64_t cq_qmatmul_workspace_bytes(int w_dtype, int64_t m, int64_t k, int64_t n);
+/* Bytes of one wave step of the single-row decode kernel over a [n, k] weight of this format, or 0 when the shape does not take
+ * the streaming kernel.  Workgroup b of that launch reads steps b, b + 256, ...; workgroups are dealt to the eight XCDs round-robin,
+ * so step s is read through the L2 of XCD s % 8 (what cq_nn_attention_decode's prefetch_piece_bytes wants to know).
+ * No counterpart in the reference. */
+int64_t cq_qmatmul_stream_step_bytes(int w_dtype, int64_t k, int64_t n);
 int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_dtype, void *dst_dev, int dst_dtype,
                        int64_t m, int64_t k, int64_t n, void *workspace_dev, int64_t workspace_bytes, void *stream);
 
@@ -144,7 +149,9 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
  * scratch is a grow-only buffer that the host allocates, fast_mmvq.rs:44-81): this entry point is for callers that
  * cannot allocate device memory — code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * The workspace is a fixed array of CQ_STATIC_WORKSPACE_BYTES inside the library's device code (one copy per GPU, held
- * until the process ends; its address is looked up on the first call made with a device current).  Results are those
+ * until the process ends; its address is looked up on the first call made with a device current, by this entry point or by
+ * cq_static_workspace_bytes(): the lookup may load the library's code object, so make one of the two calls on every device
+ * eagerly before the entry point is used under stream capture).  Results are those
  * of cq_qmatmul_forward bit for bit (same kernels).  A call whose cq_qmatmul_workspace_bytes() exceeds the array
  * returns CQ_ERR_RANGE and enqueues nothing.  All calls on one GPU share the array: calls that may overlap on one GPU
  * (different streams, different threads) race; serialize them or use cq_qmatmul_forward with separate workspaces.

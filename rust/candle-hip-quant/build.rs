@@ -4,8 +4,8 @@
 use std::path::PathBuf;
 use std::process::Command;
 
-const SOURCES: [&str; 9] =
-    ["cq_api", "cq_dequant", "cq_actquant", "cq_matvec", "cq_matmul", "cq_moe", "cq_quantize", "cq_nn", "cq_layer"];
+const SOURCES: [&str; 10] =
+    ["cq_api", "cq_dequant", "cq_actquant", "cq_matvec", "cq_matmul", "cq_moe", "cq_quantize", "cq_nn", "cq_layer", "cq_matvec_batch"];
 
 fn main() {
     let rocm = std::env::var("ROCM_PATH").unwrap_or_else(|_| "/opt/rocm".to_string());

@@ -64,3 +64,30 @@ def test_result_depends_on_tensor_bytes_only(fmt, base_mod4, n, k):
             alone = _forward(L, code, own.data_ptr(), x_dev, m, k, n)
             assert np.array_equal(outs[0].view(np.uint32), alone.view(np.uint32)), m
         assert rel_l2(outs[0], oracle.matmul(odt, x, blocks, n)) <= 1e-5, m
+
+
+@pytest.mark.parametrize("n,k", [(65, 256), (67, 768), (203, 1792), (64, 256), (129, 4096)])
+def test_q6k_tensor_of_2_mod_4_bytes_on_the_streaming_kernel(n, k):
+    """Q6_K super-blocks are 210 bytes: a tensor with an odd block count has a size of 2 (mod 4), and its last bytes are
+    the f16 scale of the last block.  One and two f32 rows take the streaming kernel, whose buffer descriptor ends inside
+    the dword that holds that scale: the last row must come out right and nothing beyond the tensor may be used."""
+    print(f"case q6k n={n} k={k}", flush=True)
+    L = _lib.lib()
+    blocks = oracle.from_float(oracle.Q6K, normal(6, (n, k), 0.02).reshape(-1))
+    raw = np.frombuffer(blocks, dtype=np.uint8)
+    assert raw.size == n * (k // 256) * 210
+    own = torch.from_numpy(raw.copy()).to("cuda:0")
+    buf = torch.empty(CANARY + raw.size + CANARY, dtype=torch.uint8, device="cuda:0")
+    w_ptr = buf.data_ptr() + CANARY                      # 16-byte aligned: the streaming kernel takes it
+    for m in (1, 2):
+        x = normal(40 + m, (m, k))
+        x_dev = torch.from_numpy(x).to("cuda:0")
+        outs = []
+        for fill in (0x00, 0xFF):
+            buf.fill_(fill)
+            buf[CANARY: CANARY + raw.size] = own
+            outs.append(_forward(L, 14, w_ptr, x_dev, m, k, n))
+        assert not np.isnan(outs[0]).any() and not np.isnan(outs[1]).any(), m
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), m
+        assert rel_l2(outs[0], oracle.matmul(oracle.Q6K, x, blocks, n)) <= 1e-5, m
+        assert rel_l2(outs[0][:, -1], oracle.matmul(oracle.Q6K, x, blocks, n)[:, -1]) <= 1e-5, m     # the row whose scale ends the tensor

@@ -88,6 +88,22 @@ def test_matvec_k_sweep(dtype, k):
     assert rel_l2(got, want) <= TIGHT
 
 
+@pytest.mark.parametrize("k", [256, 768, 2560, 4096, 6144, 8192, 11008, 14336])
+@pytest.mark.parametrize("n,batch", [(203, 3), (203, 16), (5, 4), (16, 11), (17, 13), (1024, 9)])
+def test_q4k_batched_rows_vs_oracle(k, n, batch):
+    """3 .. 16 rows of Q4_K take the batched matrix-core matvec (16 weight rows per block, K split over the waves in
+    1 .. 7 super-block columns each): ragged n, fewer rows than a block, every column count, idle waves (k = 256, 768)."""
+    blocks, qmm = make_weight(oracle.Q4K, n, k, seed=131)
+    x = normal(132 + batch, (batch, k), 1.0)
+    got = forward(qmm, x)
+    want = oracle.matmul_fast(oracle.Q4K, x, blocks, n, 8)
+    err = rel_l2(got, want)
+    assert err <= TOL and err <= TIGHT, f"rel-L2 {err}"
+    # row by row as well: a wrong batch column would hide in the norm of 16 rows
+    for r in range(batch):
+        assert rel_l2(got[r], want[r]) <= TIGHT, r
+
+
 def test_cfg1_q8_0_4096x4096():
     # BASELINE configs[0]: Q8_0 weight [4096 x 4096], activation 1 x 4096
     blocks, qmm = make_weight(oracle.Q8_0, 4096, 4096, seed=1)
@@ -210,7 +226,7 @@ def test_half_activations_keep_dtype(tdt):
 @pytest.mark.parametrize("dtype,n,k", [(oracle.Q4K, 14336, 4096), (oracle.Q4K, 4096, 14336), (oracle.Q6K, 4096, 14336),
                                        (oracle.Q5K, 14336, 4096), (oracle.Q4_0, 14336, 4096), (oracle.Q8_0, 4096, 4096)],
                          ids=lambda v: NAMES.get(v, str(v)))
-@pytest.mark.parametrize("batch", [1, 8, 16, 128])
+@pytest.mark.parametrize("batch", [1, 2, 4, 8, 16, 128])
 def test_full_size_equals_dot_of_dequantized(dtype, n, k, batch):
     """The quantized dot equals the dot of the two dequantized operands (up to f32 summation error):
     y = dequant(W) @ dequant(x^) in f64.  dequant(W) is the bit-exact GPU dequantizer checked

@@ -193,7 +193,7 @@ def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
         ok(lib.cq_nn_attention_decode(dev(q).data_ptr(), dev(k).data_ptr(), dev(v).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(),
                                       dev(sin).data_ptr(), out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv,
                                       float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, pf.data_ptr() if attempt else None,
-                                      pf.numel() if attempt else 0, None))
+                                      pf.numel() // 16 * 16 if attempt else 0, 9216 if attempt and KV == 8 else 0, None))
         torch.cuda.synchronize()
         assert rel_l2(out.cpu().numpy(), want) <= TOL, attempt
         assert np.allclose(kc.cpu().numpy()[:, pos], want_k[:, 0], rtol=1e-6, atol=1e-6)
@@ -217,7 +217,7 @@ def _attention_decode_case(lib, ws, wsb, H, KV, D, pos, ctx, max_kv, seed):
     posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
     ok(lib.cq_nn_attention_decode(dev(q).data_ptr(), dev(k).data_ptr(), dev(v).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(),
                                   dev(sin).data_ptr(), out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv,
-                                  float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None, 0, None))
+                                  float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None, 0, 0, None))
     torch.cuda.synchronize()
     assert rel_l2(out.cpu().numpy(), want) <= TOL, (pos, max_kv)
     assert np.array_equal(vc.cpu().numpy()[:, pos], vc_ref[:, pos])
@@ -276,7 +276,7 @@ def test_attention_decode_in_kernel_merge_soak(pos, max_kv):
 
     def launch():
         ok(lib.cq_nn_attention_decode(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), kc.data_ptr(), vc.data_ptr(), cd.data_ptr(), sd.data_ptr(),
-                                      out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv, scale, ws.data_ptr(), wsb, None, 0, None))
+                                      out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv, scale, ws.data_ptr(), wsb, None, 0, 0, None))
 
     launch()
     torch.cuda.synchronize()
@@ -309,7 +309,7 @@ def test_attention_merge_as_matvec_prologue(dtype, pos, max_kv):
     ws = torch.zeros(wsb, dtype=torch.uint8, device="cuda")
     att = torch.empty((1, k), device="cuda")
     args = (dev(q).data_ptr(), dev(kn).data_ptr(), dev(vn).data_ptr(), kc.data_ptr(), vc.data_ptr(), dev(cos).data_ptr(), dev(sin).data_ptr())
-    tail = (None, pos, H, KV, D, ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None, 0, None)
+    tail = (None, pos, H, KV, D, ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))), ws.data_ptr(), wsb, None, 0, 0, None)
     ok(lib.cq_nn_attention_decode(*args, att.data_ptr(), *tail))
     res0 = normal(46, (1, hidden), 1.0)
     r1, r2 = dev(res0), dev(res0)

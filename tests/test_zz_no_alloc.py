@@ -72,3 +72,34 @@ def test_static_workspace_rejects_oversized_calls():
     dummy = torch.zeros(64, dtype=torch.uint8, device="cuda:0")
     rc = L.cq_qmatmul_forward_static(12, _vp(dummy), _vp(dummy), 0, _vp(dummy), 0, m, k, n, None)
     assert rc == -6 and "exceeds" in _lib.status_string(rc)
+
+
+def test_static_workspace_under_graph_capture():
+    """The entry point is meant for callers under stream capture: after cq_static_workspace_bytes() has been called eagerly on
+    the device (the one-time address lookup), a captured call replays bit-equal to the eager result, several times, with eager
+    work between the replays."""
+    L = _lib.lib()
+    code, odt = CQ["q4k"]
+    n, k, m = 512, 1024, 5
+    blocks = oracle.from_float(odt, normal(21, (n, k), 0.02).reshape(-1))
+    w_dev = torch.from_numpy(np.frombuffer(blocks, dtype=np.uint8).copy()).to("cuda:0")
+    x_dev = torch.from_numpy(normal(22, (m, k))).to("cuda:0")
+    assert L.cq_static_workspace_bytes() == 32 << 20            # eager, before any capture
+    eager, want = _forward_pair(L, code, w_dev, x_dev, m, k, n, 0)
+    assert np.array_equal(eager.view(np.uint32), want.view(np.uint32))
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            _lib.check("cq_qmatmul_forward_static", L.cq_qmatmul_forward_static(code, _vp(w_dev), _vp(x_dev), 0, _vp(out), 0, m, k, n, s))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        out.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32)), rep
+        # eager work on the shared workspace between the replays
+        other, _ = _forward_pair(L, code, w_dev, torch.from_numpy(normal(30 + rep, (m, k))).to("cuda:0"), m, k, n, 0)
+        assert not np.isnan(other).any()
