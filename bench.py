@@ -202,8 +202,12 @@ def prefill_record(L, torch, fmt, n, k, m, steps=20, warmup=5, pmc=False):
         _lib.check("cq_qmatmul_forward", L.cq_qmatmul_forward(dt, wq.data_ptr(), x.data_ptr(), 0, dst.data_ptr(), 0, m, k, n,
                                                               ws.data_ptr(), ws_bytes, sp))
 
-    def matmul_only():
-        _lib.check("cq_matmul", L.cq_matmul(dt, wq.data_ptr(), ws.data_ptr(), dst.data_ptr(), k, n, m, n, sp))
+    def quantize_only():
+        _lib.check("cq_quantize_act", L.cq_quantize_act(dt, x.data_ptr(), 0, ws.data_ptr(), k, m, sp))
+
+    # small grids split K into partial planes that a second kernel adds up (the workspace then holds those planes too)
+    act_bytes = L.cq_act_scratch_bytes(dt, k, m)
+    split_k = ws_bytes > act_bytes + ((m * n * 4 + 255) // 256) * 256
 
     if pmc:
         with torch.cuda.stream(stream):
@@ -235,13 +239,19 @@ def prefill_record(L, torch, fmt, n, k, m, steps=20, warmup=5, pmc=False):
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / steps
     flops = 2.0 * m * n * k
-    kern_us, kst = event_us(matmul_only, steps)
+    # the matrix-core part of what the forward launches (the split-K kernel and its reduction where K is split): the
+    # forward's launches timed on the stream minus the activation quantization timed alone
+    fwd_us, fst = event_us(forward, steps)
+    q_us, _ = event_us(quantize_only, steps)
+    kern_us = fwd_us - q_us
+    kst = {key: fst[key] - q_us for key in ("median", "p10", "p90")}
     # the roofline is priced in algorithmic flop against the dense peak of the matrix-core type the kernel uses
     i8 = fmt in I8_PREFILL
     peak = MFMA_I8_PEAK_TOPS if i8 else MFMA_F16_PEAK_TFLOPS
     achieved = flops / (kern_us * 1e-6) / 1e12
     return {"fmt": fmt, "n": n, "k": k, "m": m, "steps": steps, "warmup": warmup, "forward_ms": round(ms, 5),
             "forward_TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1), "kernel": "qmm_q4k_i8_kernel" if fmt == "q4k" else ("qmm_q0_i8_kernel<%s>" if i8 else "qmm_kernel<%s>") % fmt,
+            "split_k": bool(split_k), "quantize_us": round(q_us, 2),
             "kernel_us": round(kern_us, 2), "kernel_median_us": round(kst["median"], 2), "kernel_p10_us": round(kst["p10"], 2),
             "kernel_p90_us": round(kst["p90"], 2), "kernel_TFLOPs": round(achieved, 1), "mfma": "i8" if i8 else "f16", "peak": peak,
             "frac": round(achieved / peak, 4)}
@@ -286,6 +296,11 @@ def decode8b(args):
     n_new = args.steps if args.steps else 256
     model.generate_greedy(prompt, min(n_new, 8))                      # warm-up: code paths, graph capture
     res = model.generate_greedy(prompt, n_new)
+    # the same run from a step captured once for the whole context (more, shorter attention splits per head)
+    model.generate_greedy(prompt, min(n_new, 8), max_kv=cfg.ctx)
+    res_ctx = model.generate_greedy(prompt, n_new, max_kv=cfg.ctx)
+    # (another split count sums the attention in another order: on random weights the greedy tokens may part ways at a near tie)
+    same = next((i for i, (a, b) in enumerate(zip(res["tokens"], res_ctx["tokens"])) if a != b), len(res["tokens"]))
     wbytes = model.weight_bytes_per_token()
     steps = res["decode_steps"]
     tok_s = steps / res["decode_seconds"]
@@ -303,6 +318,8 @@ def decode8b(args):
                                % (cfg.n_layer, args.prompt, steps),
                    "ctx": cfg.ctx, "prompt_tokens": args.prompt},
         "prompt_tok_s": round(args.prompt / res["prompt_seconds"], 1),
+        "captured_for_kv": args.prompt + n_new, "tok_s_captured_for_ctx": round(res_ctx["decode_steps"] / res_ctx["decode_seconds"], 1),
+        "captured_for_ctx_equal_leading_tokens": same,
         "weight_bytes_per_token": wbytes, "kv_bytes_per_token_mean": int(kv_bytes),
         "roofline": {"bound": "hbm", "kernel": "whole decode step (weights streamed once per token)",
                      "achieved": round((wbytes + kv_bytes) * tok_s / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -680,6 +697,7 @@ def other_configurations(L, torch, args):
     # cfg4: the 8B-shape decoder (same protocol as --workload decode8b)
     r = decode8b(argparse.Namespace(layers=32, prompt=512, steps=256))
     out["decode_8b"] = {"tok_s": r["value"], "ms_per_token": r["ms_per_step"], "prompt_tok_s": r["prompt_tok_s"],
+                        "captured_for_kv": r["captured_for_kv"], "tok_s_captured_for_ctx": r["tok_s_captured_for_ctx"],
                         "frac_of_roofline_tok_s": r["roofline"]["frac_of_roofline_tok_s"],
                         "roofline_tok_s": r["roofline"]["roofline_tok_s_weights_only"],
                         "weight_bytes_per_token": r["weight_bytes_per_token"], "workload": r["config"]["workload"]}

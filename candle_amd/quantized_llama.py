@@ -590,14 +590,18 @@ class ModelWeights:
         self._enqueue(None if chain else self.token_dev.data_ptr(), 1, 0, self.pos_dev.data_ptr(), max_kv_len, sp)
         self._argmax_dev(self.logits.data_ptr(), chain, sp)
 
-    def generate_greedy(self, prompt: Sequence[int], n_new: int, use_graph: bool = True) -> dict:
+    def generate_greedy(self, prompt: Sequence[int], n_new: int, use_graph: bool = True, max_kv: Optional[int] = None) -> dict:
         """The loop of candle-examples/examples/quantized/main.rs:616-690 with temperature <= 0 (Sampling::ArgMax):
         prefill the prompt in one forward, pick the arg-max token, then n_new - 1 single-token steps.
-        Returns the generated tokens and the wall-clock split prompt / decode, as the example prints them."""
+        Returns the generated tokens and the wall-clock split prompt / decode, as the example prints them.
+        max_kv: the number of cache positions the captured step is laid out for (its attention split count follows from
+        it); by default exactly prompt + n_new, a server that captures one step for every request passes the context."""
         cfg = self.cfg
         prompt = [int(t) for t in prompt]
         if len(prompt) + n_new > cfg.ctx:
             raise ValueError("prompt + generated tokens exceed the context")
+        if max_kv is not None and not len(prompt) + n_new <= max_kv <= cfg.ctx:
+            raise ValueError("max_kv must cover prompt + generated tokens and fit the context")
         dev = self.device
         torch.cuda.synchronize(dev)
         t0 = time.perf_counter()
@@ -606,7 +610,8 @@ class ModelWeights:
         self.counter_dev.zero_()
         self.pos_dev.fill_(len(prompt) - 1)       # argmax advances it to the position of the token it emits
         steps = n_new - 1
-        max_kv = len(prompt) + n_new
+        if max_kv is None:
+            max_kv = len(prompt) + n_new
         self._argmax_dev(logits.data_ptr(), steps > 0 and self._chain_embedding(max_kv), stream.cuda_stream)
         torch.cuda.synchronize(dev)
         t1 = time.perf_counter()
