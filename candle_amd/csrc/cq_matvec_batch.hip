@@ -40,6 +40,7 @@ __shared__ uint32_t qb_stamp_lds[8][16];
 #endif
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef long i64x2 __attribute__((ext_vector_type(2)));
 
 constexpr int QB_NW = 8;
 constexpr int QB_BB = 144;                        // bytes of a Q4_K super-block
@@ -56,9 +57,10 @@ __host__ __device__ constexpr int qb_tile_bytes(int block_bytes) { return ((bloc
 
 // ---- the activations, quantized like BlockQ8K::from_float and laid out as this kernel's matrix operands ----
 // For super-block column s of the row length, 16 batch slots (rows beyond the batch are zeros):
-//   operands [s][sub-block j < 8][kg < 4][batch slot c < 16][8 bytes]   values 32 j + 8 kg .. + 7 of column s of row c: what lane
-//                                                                      (c, kg) feeds the matrix core for sub-block j, 512
-//                                                                      contiguous bytes per wave load;
+//   operands [s][g < 4][kg < 4][batch slot c < 16][16 bytes]   values 8 kg .. 8 kg + 7 of sub-blocks 2 g and 2 g + 1 of column s of
+//                                                              row c: what lane (c, kg) feeds the matrix core against the low and
+//                                                              the high nibbles of weight bytes 32 g + 8 kg .. + 7; one 16-byte
+//                                                              load per lane, 1 KB contiguous per wave;
 //   records  [s][c] { u8 bl[8], i8 bh[8] (sum of sub-block j = 128 * bh_j + bl_j), f32 d, 12 bytes unused }
 constexpr int QB_OP_COL_BYTES = 8 * 4 * 16 * 8;       // 4096
 constexpr int QB_REC_BYTES = 32;
@@ -103,7 +105,7 @@ __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict
     }
     // elements 4 lane .. + 3: sub-block lane / 8, values 4 (lane % 8) .. + 3 of it: lane group kg = (lane % 8) / 2, dword lane % 2
     uint8_t *colp = op + (int64_t)s * QB_OP_COL_BYTES;
-    *(uint32_t *)(colp + (((lane >> 3) * 4 + ((lane & 7) >> 1)) * 16 + c) * 8 + 4 * (lane & 1)) = packed;
+    *(uint32_t *)(colp + (((lane >> 4) * 4 + ((lane & 7) >> 1)) * 16 + c) * 16 + 8 * ((lane >> 3) & 1) + 4 * (lane & 1)) = packed;
     const int s32 = oct_sum(lsum);                        // the sum of the 32-element sub-block, in its eight lanes
     uint32_t bl[2] = {0, 0}, bh[2] = {0, 0};
 #pragma unroll
@@ -174,9 +176,12 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
 #pragma unroll
     for (int ci = 0; ci < CPW; ci++) {
         const int col = min(col0 + ci, bpr - 1);
-        const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 8;          // lane = kg * 16 + c
+        const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 16;         // lane = kg * 16 + c
 #pragma unroll
-        for (int j = 0; j < 8; j++) A[ci][j] = *(const long *)(colp + j * 512);
+        for (int g = 0; g < 4; g++) {
+            const i64x2 v = c < rows ? *(const i64x2 *)(colp + g * 1024) : i64x2{0, 0};    // (batch slots beyond the rows hold zeros)
+            A[ci][2 * g] = v.x; A[ci][2 * g + 1] = v.y;
+        }
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const uint8_t *rec = op + (int64_t)bpr * QB_OP_COL_BYTES + (int64_t)(col * 16 + 4 * kg + r) * QB_REC_BYTES;
@@ -257,6 +262,199 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
 #endif
 }
 
+// ---- rows of more than 24 super-blocks ------------------------------------------------------------------------------------
+// The activations of a whole row no longer fit the registers of eight waves next to their block sums, and a block of 16 such
+// rows no longer fits LDS three times.  So a row block is taken in Q column chunks of cpp <= 16 super-blocks (tile = 16 rows x
+// one chunk, gathered by the copy instructions from 16 row segments), wave w owns columns 2 w, 2 w + 1 of EVERY chunk and
+// keeps their int8 operands in registers (Q x 2 x 16 registers), and the per-row records (block sums, scale) wait in LDS.
+// The accumulators run across the chunks of a block; everything else is the kernel above.
+template <int Q>
+__global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ op, void *__restrict__ dst, int n,
+                                                                   int bpr, int rows, int dst_dtype, int64_t stride_dst, int cpp
+#ifdef CL_STAMPS
+                                                                   , uint32_t *stamps
+#endif
+                                                                   ) {
+    constexpr int CPW = 2, DEPTH = 3;
+    constexpr int NIW = qb_tile_instr(CPW);
+    static_assert((DEPTH - 1) * NIW <= 63, "counted waits");
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int bx = blockIdx.x, gx = gridDim.x;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, kg = lane >> 4;
+    const int col0 = wv * CPW;                    // the wave's first column inside a chunk
+    const int RS = bpr * QB_BB;                   // bytes of a row in memory
+    const int block_bytes = 16 * RS;
+    const int TILE = qb_tile_bytes(16 * cpp * QB_BB);
+    const int last_cols = bpr - (Q - 1) * cpp;    // columns of the last chunk (1 .. cpp)
+    float *red = (float *)(lds + DEPTH * TILE);                              // [8 waves][64 lanes][4]
+    uint8_t *recs = (uint8_t *)red + QB_RED_BYTES;                           // [bpr][16 batch slots] records
+
+    const int nsteps = (n + 15) >> 4;
+    const int64_t w_bytes = (int64_t)n * RS;
+    const int my = bx < nsteps ? (nsteps - bx + gx - 1) / gx : 0;
+    const int ntiles = my * Q;
+    // instruction t of wave w copies KB number t * 8 + w of the tile; where in the block (less the chunk's first column) its
+    // lane's 16 bytes come from, for a full chunk and for the last one:
+    int voff_full[NIW], voff_last[NIW];
+#pragma unroll
+    for (int t = 0; t < NIW; t++) {
+        const int tb = (t * QB_NW + wv) * 1024 + lane * 16;
+        const int rf = tb / (cpp * QB_BB), rl = tb / (last_cols * QB_BB);
+        voff_full[t] = rf < 16 ? rf * RS + (tb - rf * cpp * QB_BB) : block_bytes;            // beyond the tile: out of range, zeros
+        voff_last[t] = rl < 16 ? rl * RS + (tb - rl * last_cols * QB_BB) : block_bytes;
+    }
+    // (Every workgroup takes the chunks in the same order.  Rotating the order by workgroup, so that the launch reads all column
+    // ranges of the tensor at any moment instead of the same quarter of every row, was measured a third slower.)
+    auto issue = [&](int tau) {
+        const int i = tau / Q, q = tau - i * Q;
+        const int m = bx + i * gx;
+        const bool live = tau < ntiles;
+        const int pc = q == Q - 1 ? last_cols : cpp;
+        const int64_t off = live ? (int64_t)m * block_bytes + q * cpp * QB_BB : 0;
+        const int64_t left = w_bytes - off;
+        const int bytes = live ? (int)(left < block_bytes ? left : block_bytes) : 0;      // an absent tile: a descriptor of zero bytes
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(w + off), 0, bytes, 0x00020000);
+        uint8_t *tile = lds + (tau % DEPTH) * TILE;
+        const int nkb = (16 * pc * QB_BB + 1023) >> 10;
+#pragma unroll
+        for (int t = 0; t < NIW; t++) {
+            const int kb = min(t * QB_NW + wv, nkb);             // KB number nkb: beyond the tile, nothing read, zeros into the spare KB
+            const int vo = q == Q - 1 ? voff_last[t] : voff_full[t];
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(tile + kb * QB_KB), 16, vo, 0, 0, 0);
+        }
+    };
+    issue(0);
+    asm volatile("" ::: "memory");
+    QB_STAMP(0);
+    // the operands into registers, the records (32 bytes per (column, batch slot), at most 4 pieces of 16 bytes per thread)
+    // through registers into LDS; the second tile is asked for before anything here is waited for
+    // (of the first chunk only: the operands of chunk q + 1 are asked for while chunk q of the first block is worked on --
+    // all of them up front would keep the load path busy for 6 us before the second tile could be asked for)
+    long A[Q][CPW][8];
+    auto load_operands = [&](int q) {
+#pragma unroll
+        for (int ci = 0; ci < CPW; ci++) {
+            const int col = min(q * cpp + col0 + ci, bpr - 1);
+            const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 16;     // lane = kg * 16 + c
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const i64x2 v = c < rows ? *(const i64x2 *)(colp + g * 1024) : i64x2{0, 0};    // (batch slots beyond the rows hold zeros)
+                A[q][ci][2 * g] = v.x; A[q][ci][2 * g + 1] = v.y;
+            }
+        }
+    };
+    load_operands(0);
+    const int npieces = bpr * 16 * (QB_REC_BYTES / 16);
+    u32x4 rv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        rv[j] = *(const u32x4 *)(op + (int64_t)bpr * QB_OP_COL_BYTES + (int64_t)min(tid + j * QB_NW * 64, npieces - 1) * 16);
+    asm volatile("" ::: "memory");
+    issue(1);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        if (tid + j * QB_NW * 64 < npieces) *(u32x4 *)(recs + (tid + j * QB_NW * 64) * 16) = rv[j];
+    QB_STAMP(1);
+    for (int i = 0; i < my; i++) {
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const int tau = i * Q + q;
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * NIW) : "memory");
+            // (lgkmcnt: the first time round, this wave's records are in LDS before anyone passes the barrier)
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            // (in front of the copies: waiting for these operands, one chunk on, then waits for nothing younger than tile tau + 1)
+            if (q + 1 < Q && i == 0) load_operands(q + 1 < Q ? q + 1 : 0);
+            asm volatile("" ::: "memory");
+            issue(tau + DEPTH - 1);
+            const uint8_t *tile = lds + (tau % DEPTH) * TILE;
+            if (tau < 4) QB_STAMP(2 + 3 * tau);
+            const int pc = q == Q - 1 ? last_cols : cpp;
+            const int TRS = pc * QB_BB;
+#pragma unroll
+            for (int ci = 0; ci < CPW; ci++) {
+                if (col0 + ci < pc) {
+                    const int o = c * TRS + (col0 + ci) * QB_BB;                 // weight row c of the block, this column's super-block
+                    auto at = [&](int off) { return tile + off + (off >> 10) * 16; };      // byte `off` of the tile in its padded form
+                    const u32x4 hdr = *(const u32x4 *)at(o);
+                    i32x4 cl[4], ch[4];
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const long qa = *(const long *)at(o + 16 + 32 * g + 8 * kg);
+                        const long lo = qa & 0x0f0f0f0f0f0f0f0fl, hi = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                        const i32x4 z = {0, 0, 0, 0};
+                        cl[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[q][ci][2 * g], lo, z, 0, 0, 0);
+                        ch[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[q][ci][2 * g + 1], hi, z, 0, 0, 0);
+                    }
+                    const QsScales s = qs_scales_k4(hdr.y, hdr.z, hdr.w);
+                    int sc[8];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        sc[j] = (int)((s.scA >> (8 * j)) & 0xff);
+                        sc[4 + j] = (int)((s.scB >> (8 * j)) & 0xff);
+                    }
+                    const float dw = h2f(hdr.x), dm = h2f(hdr.x >> 16);
+                    const uint8_t *rec = recs + ((q * cpp + col0 + ci) * 16 + 4 * kg) * QB_REC_BYTES;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        int S = 0;
+#pragma unroll
+                        for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
+                        const u32x4 aux = *(const u32x4 *)(rec + r * QB_REC_BYTES);
+                        const float d8 = *(const float *)(rec + r * QB_REC_BYTES + 16);
+                        const int M = qs_dot_sums(s.mA, s.mB, aux);
+                        acc[r] += d8 * (dw * (float)S - dm * (float)M);
+                    }
+                }
+            }
+            if (tau < 4) QB_STAMP(3 + 3 * tau);
+        }
+        // ---- the eight K-slices of the block meet in LDS and are added in wave order ----
+        *(f32x4 *)(red + (wv * 64 + lane) * 4) = f32x4{acc[0], acc[1], acc[2], acc[3]};
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (tid < 256) {
+            const int l2 = tid & 63, r = tid >> 6;
+            float v = 0.0f;
+#pragma unroll
+            for (int w2 = 0; w2 < QB_NW; w2++) v += red[(w2 * 64 + l2) * 4 + r];
+            const int m = bx + i * gx;
+            const int row = m * 16 + (l2 & 15), br = 4 * (l2 >> 4) + r;
+            if (row < n && br < rows) store_out(dst, dst_dtype, (int64_t)br * stride_dst + row, v);
+        }
+        // (the sums have left LDS before this wave passes the next barrier, behind which `red` is written again only after
+        // a whole block's chunks: the barrier at the top of the next chunk orders the reads above before those writes)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");               // no copy may land in LDS after the workgroup has left
+#ifdef CL_STAMPS
+    QB_STAMP(15);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (tid < 128 && stamps) stamps[(bx * 8 + tid / 16) * 16 + tid % 16] = qb_stamp_lds[tid / 16][tid % 16];
+#endif
+}
+
+template <int Q>
+int launch_qmb_long(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int cpp,
+                    hipStream_t s) {
+    const int64_t bpr = k / 256;
+    const size_t lds_bytes = (size_t)3 * qb_tile_bytes(16 * cpp * QB_BB) + QB_RED_BYTES + (size_t)bpr * 16 * QB_REC_BYTES;
+    if (lds_bytes > (size_t)QB_LDS_BYTES - 1024) return CQ_ERR_RANGE;
+    auto kern = qmb_q4k_long_kernel<Q>;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    const int64_t nsteps = (n + 15) / 16;
+    const unsigned grid = (unsigned)(nsteps < 256 ? nsteps : 256);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(QB_NW * 64), lds_bytes, s, (const uint8_t *)w, op, dst, (int)n, (int)bpr, (int)rows, dst_dtype, stride_dst,
+                       cpp
+#ifdef CL_STAMPS
+                       , qb_stamps_dev
+#endif
+    );
+    return (int)hipGetLastError();
+}
+
 template <int CPW, int DEPTH>
 int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
                  hipStream_t s) {
@@ -288,15 +486,18 @@ int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64
 
 }  // namespace
 
-// Does the batched matrix-core matvec take this call?  Q4_K, 3 .. 16 rows, rows of up to 24 super-blocks (three columns per wave:
-// beyond that the activations of a wave's columns no longer fit its registers).
+// Does the batched matrix-core matvec take this call?  Q4_K, 3 .. 16 rows, rows of up to 64 super-blocks (k <= 16384: up to 24
+// with three columns per wave, beyond that in up to four column chunks, which is what a wave's registers hold of a row).
+constexpr int QB_MAX_BPR = 64;        // (and 64 x 16 records of 32 bytes are 4 pieces of 16 bytes per thread)
 bool cq_matvec_batch_takes(int w_dtype, const void *w, int64_t k, int64_t n, int64_t rows) {
-    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= 24 && n >= 1 && n <= 0x7ffffff0 / 16 &&
+    // (three rows over chunked rows: the register-blocked matvec is still ahead there, 15.1 against 16.8 us on [4096 x 14336])
+    if (k / 256 > 3 * QB_NW && rows < 4) return false;
+    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= QB_MAX_BPR && n >= 1 && n <= 0x7ffffff0 / 16 &&
            n * (k / 256) * QB_BB < 0x7fffffffLL && ((uintptr_t)w & 15) == 0;
 }
 // bytes of workspace the call needs (the activations as matrix operands); 0 when the shape can never take this path
 int64_t cq_matvec_batch_workspace(int w_dtype, int64_t k, int64_t rows) {
-    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= 24 ? cq_align256(qb_operand_bytes(k / 256)) : 0;
+    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= QB_MAX_BPR ? cq_align256(qb_operand_bytes(k / 256)) : 0;
 }
 
 // QMatMul::forward for 3 .. 16 rows of x: one small kernel quantizes them into `workspace`, then the weights are read once.
@@ -313,6 +514,15 @@ static int qb_launch(int w_dtype, const void *w, const void *x, const float *up,
         case CQ_F16: hipLaunchKernelGGL(qb_quantize_kernel<CQ_F16>, dim3(qgrid), dim3(256), 0, s, x, up, x_stride, up_stride, op, bpr, (int)rows); break;
         case CQ_BF16: hipLaunchKernelGGL(qb_quantize_kernel<CQ_BF16>, dim3(qgrid), dim3(256), 0, s, x, up, x_stride, up_stride, op, bpr, (int)rows); break;
         default: return CQ_ERR_DTYPE;
+    }
+    if (bpr > 3 * QB_NW) {
+        const int chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW), cpp = (bpr + chunks - 1) / chunks;
+        switch (chunks) {
+            case 2: return launch_qmb_long<2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+            case 3: return launch_qmb_long<3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+            case 4: return launch_qmb_long<4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+            default: return CQ_ERR_RANGE;
+        }
     }
     const int64_t cpw = (k / 256 + QB_NW - 1) / QB_NW;
     switch (cpw) {
