@@ -774,10 +774,11 @@ template <> struct Q0Info<CQ_Q8_0> { static constexpr int QS = 2, QH = -1, MIN =
 template <> struct Q0Info<CQ_Q4_1> { static constexpr int QS = 4, QH = -1, MIN = 2; static constexpr uint32_t BIAS = 0; };
 template <> struct Q0Info<CQ_Q5_0> { static constexpr int QS = 6, QH = 2, MIN = -1; static constexpr uint32_t BIAS = 0x70707070u; };
 template <> struct Q0Info<CQ_Q5_1> { static constexpr int QS = 8, QH = 4, MIN = 2; static constexpr uint32_t BIAS = 0; };
-template <int DT, int NJ, bool SM = false>
+// MOE: blockIdx.x is a tile of the chunk table, as in the kernels above.
+template <int DT, int NJ, bool MOE = false, bool SM = false>
 __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const uint8_t *__restrict__ w, ActView av, float *__restrict__ dst,
-                                                                           int k, int n, int rows, int64_t stride_dst, MoeChunks,
-                                                                           int64_t, int64_t split_stride) {
+                                                                           int k, int n, int rows, int64_t stride_dst, MoeChunks mc,
+                                                                           int64_t expert_bytes, int64_t split_stride) {
     typedef Q0Info<DT> QI;                                      // byte offsets of qs / qh / the block minimum (-1: none)
     static_assert(!SM || NJ == 1, "the small-m tile has one 32-column MFMA tile per wave");
     constexpr int BB = BlockInfo<DT>::bytes;
@@ -794,7 +795,14 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = SM ? 0 : wv >> 1, wn = SM ? wv : wv & 1;
-    const int m0 = blockIdx.x * BMT, n0 = blockIdx.y * BN;
+    int m0 = blockIdx.x * BMT;
+    const int n0 = blockIdx.y * BN;
+    if (MOE) {
+        if ((int)blockIdx.x >= mc.n_chunks[0]) return;           // uniform over the workgroup
+        m0 = mc.first[blockIdx.x];
+        rows = m0 + mc.count[blockIdx.x];
+        w += (int64_t)mc.expert[blockIdx.x] * expert_bytes;
+    }
     // split-K over spans of 256 elements, like the other kernels; a stage is half a span
     const int nsb_all = k >> 8;
     const int st0 = 2 * (int)(((int64_t)nsb_all * blockIdx.z) / gridDim.z), st1 = 2 * (int)(((int64_t)nsb_all * (blockIdx.z + 1)) / gridDim.z);
@@ -923,7 +931,10 @@ __global__ __launch_bounds__(256, NJ == 1 ? 2 : 1) void qmm_q0_i8_kernel(const u
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int mm = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * kg + (e & 3);
-                if (mm < rows && nn < n) dst[(int64_t)mm * stride_dst + nn] = acc[i][j][e];
+                if (mm < rows && nn < n) {
+                    if (MOE) dst[(int64_t)mc.pair_out[mm] * stride_dst + nn] = acc[i][j][e] * mc.pair_scale[mm];
+                    else dst[(int64_t)mm * stride_dst + nn] = acc[i][j][e];
+                }
             }
         }
 }
@@ -948,10 +959,9 @@ typedef void (*QmmFn)(const uint8_t *, ActView, float *, int, int, int, int64_t,
 template <int DT, int NJ, bool MOE, bool SM>
 QmmFn qmm_fn() {
     if constexpr (DT == CQ_Q4K) return qmm_q4k_i8_kernel<NJ, MOE, SM>;
-    else if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0 || DT == CQ_Q4_1 || DT == CQ_Q5_0 || DT == CQ_Q5_1) {
-        static_assert(!MOE, "expert-grouped rows of the 32-element formats take the matvec kernels");
-        return qmm_q0_i8_kernel<DT, NJ, SM>;
-    } else return qmm_kernel<DT, NJ, MOE, SM>;
+    else if constexpr (DT == CQ_Q4_0 || DT == CQ_Q8_0 || DT == CQ_Q4_1 || DT == CQ_Q5_0 || DT == CQ_Q5_1)
+        return qmm_q0_i8_kernel<DT, NJ, MOE, SM>;
+    else return qmm_kernel<DT, NJ, MOE, SM>;
 }
 
 template <int DT>
@@ -1040,6 +1050,8 @@ int cq_matmul_moe_launch(int w_dtype, const void *w, const void *scratch, int64_
     if (tile_rows != CQ_MOE_TILE_SMALL && tile_rows != CQ_MOE_TILE_LARGE) return CQ_ERR_RANGE;
     ActView av = cq_act_view(scratch, w_dtype, k, rows_alloc);
     switch (w_dtype) {
+        case CQ_Q4_0: return launch_qmm_moe<CQ_Q4_0>(w, av, out, mc, k, n, tile_rows, s);
+        case CQ_Q8_0: return launch_qmm_moe<CQ_Q8_0>(w, av, out, mc, k, n, tile_rows, s);
         case CQ_Q4K: return launch_qmm_moe<CQ_Q4K>(w, av, out, mc, k, n, tile_rows, s);
         case CQ_Q5K: return launch_qmm_moe<CQ_Q5K>(w, av, out, mc, k, n, tile_rows, s);
         case CQ_Q6K: return launch_qmm_moe<CQ_Q6K>(w, av, out, mc, k, n, tile_rows, s);

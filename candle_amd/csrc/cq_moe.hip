@@ -192,7 +192,10 @@ int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_
 
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
-    const bool mfma = a.k % 256 == 0 && cq_is_kquant(a.w_dtype) && cq_has_mfma(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
+    // (the matrix-core kernel of the 32-element formats copies weight rows in 8-byte pieces: experts at another alignment take
+    // the matvec passes)
+    const bool q0_ok = (a.w_dtype == CQ_Q4_0 || a.w_dtype == CQ_Q8_0) && ((uintptr_t)a.w & 7) == 0 && (!a.w_b || ((uintptr_t)a.w_b & 7) == 0);
+    const bool mfma = a.k % 256 == 0 && (cq_is_kquant(a.w_dtype) || q0_ok) && cq_has_mfma(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
     if (a.w_b && !mfma) {
         // only the MFMA path shares its grouping pass and quantized activations between two weight tensors
         MoeArgs one = a;
@@ -219,8 +222,8 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     int *pin = (int *)(b + ws.pin_off), *pout = (int *)(b + ws.pout_off);
     float *pscale = (float *)(b + ws.pscale_off);
     int *chunks = (int *)(b + ws.chunk_off);
-    // Hundreds of pairs per call on K-quant experts: the expert-sorted rows go through the MFMA prefill kernel in tiles
-    // of up to 128 rows of one expert (integer-exact like the other K-quant paths).  Otherwise 8 pairs per matvec pass.
+    // Hundreds of pairs per call: the expert-sorted rows go through the MFMA prefill kernel of the format in tiles of up to
+    // 128 rows of one expert (integer-exact like the dense paths).  Otherwise 8 pairs per matvec pass.
     const int tile_rows = a.n_pairs < 40 * a.num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE;
     if (a.num_experts <= GROUP_LDS_EXPERTS)
         hipLaunchKernelGGL(moe_group_kernel<true>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,

@@ -251,6 +251,32 @@ def test_moe_qwen3_shape_token_batches(n, k, tokens, is_prefill):
     assert max(rel_l2(got[r], want[r]) for r in range(tokens * topk)) <= 4 * TIGHT
 
 
+@pytest.mark.parametrize("dtype", [oracle.Q8_0, oracle.Q4_0], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("tokens,E,topk", [(300, 16, 4), (330, 128, 8), (1100, 8, 2)])
+def test_grouped_matrix_core_tiles_of_the_32_element_formats(dtype, tokens, E, topk):
+    """Hundreds of pairs on Q8_0 / Q4_0 experts: the expert-sorted rows go through the int8 matrix-core kernel of the format
+    in tiles of one expert (32-row tiles while an expert sees few rows, 128-row tiles beyond), both call shapes, every
+    pair row held to the bound on its own; candle's prefill MoE takes these formats on the tensor cores as well
+    (candle-nn/src/moe.rs:208-221)."""
+    import candle_amd as ca
+    n, k = 203, 512
+    blocks, qt = make_experts(dtype, E, n, k, seed=160)
+    ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=161 + tokens)
+    sti, eid = torch.from_numpy(sorted_token_ids).cuda(), torch.from_numpy(expert_ids).cuda()
+    x = normal(162, (tokens, k), 1.0)
+    got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, None, sti, eid, topk, True).cpu().numpy()
+    want = oracle.moe_gemm_gguf(dtype, x, blocks, (E, n, k), sorted_token_ids, expert_ids, None, topk)
+    assert got.shape == want.shape == (tokens * topk, n)
+    assert rel_l2(got, want) <= TIGHT
+    assert max(rel_l2(got[r], want[r]) for r in range(tokens * topk)) <= 4 * TIGHT
+    xp = normal(163, (tokens * topk, k), 1.0)
+    twf = tw.reshape(-1)
+    got = ca.moe_gemm_gguf(torch.from_numpy(xp).cuda(), qt, torch.from_numpy(twf).cuda(), sti, eid, topk, True).cpu().numpy()
+    want = oracle.moe_gemm_gguf(dtype, xp, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
+    assert rel_l2(got, want) <= TIGHT
+    assert max(rel_l2(got[r], want[r]) for r in range(tokens * topk)) <= 4 * TIGHT
+
+
 @pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q6K, oracle.Q8_0, oracle.Q3K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("n,k", [(5, 256), (1, 768), (77, 1024), (130, 2048), (9, 4096)])
 def test_short_expert_rows_ragged(dtype, n, k):
