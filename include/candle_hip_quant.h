@@ -118,9 +118,11 @@ int cq_matvec(int w_dtype, const void *w_dev, const void *act_scratch_dev, void 
               int64_t k, int64_t n, int64_t rows, int64_t stride_dst, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
- * Prefill matmul over pre-quantized activations (any rows >= 1): more than CQ_MATVEC_MAX_ROWS rows with k a
- * multiple of 256 (Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K) run on the matrix cores with the converted operand tiles staged in LDS (K-quant operands are
- * exact integers there, Q4_0 / Q8_0 operands are rounded to f16); other shapes take 8 rows per matvec pass.
+ * Prefill matmul over pre-quantized activations (any rows >= 1): more than CQ_MATVEC_MAX_ROWS rows (Q4K: from 6 rows) with k a
+ * multiple of 256 run on the matrix cores, every format integer-exact: Q4K, Q4_0, Q8_0, Q4_1, Q5_0, Q5_1 on the int8 cores (the
+ * 32-element formats as one int8 MFMA per block, whose int32 result is the block sum the CPU forms; their weights must be 8-byte
+ * aligned), Q2K, Q3K, Q5K, Q6K on the f16 cores with operands that are exact small integers.  Other shapes take 8 rows per
+ * matvec pass.
  * Counterpart of launch_mmq_gguf_<t> (candle-core/src/quantized/fast_mmq.rs:71-111, candle-kernels/src/mmq_gguf/).
  * Same buffers as cq_matvec; dst is f32.
  * ------------------------------------------------------------------------------------------- */
@@ -130,8 +132,9 @@ int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float
 /* ---------------------------------------------------------------------------------------------
  * QCudaStorage::fwd (cuda.rs:846-878), the body of CustomOp1::cuda_fwd for QTensor
  * (mod.rs:1007-1017): quantize the m activation rows, then matvec (m <= CQ_MATVEC_MAX_ROWS; for m <= 2 the
- * quantization happens inside the matvec kernel) or MFMA matmul (split over k with an ordered reduction when the
- * grid would be small).  x is [m, k] contiguous (f32 / f16 / bf16), dst is [m, n] contiguous in dst_dtype
+ * quantization happens inside the matvec kernel; Q4K with 3 <= m <= 16, k a multiple of 256 up to 16384 and 16-byte
+ * aligned weights: one pass over the weights on the int8 matrix cores with the rows as register operands) or MFMA matmul
+ * (split over k with an ordered reduction when the grid would be small).  x is [m, k] contiguous (f32 / f16 / bf16), dst is [m, n] contiguous in dst_dtype
  * (CUDA keeps the input dtype: fast_mmvq.rs:161-323).  workspace_dev: 256-byte aligned,
  * at least cq_qmatmul_workspace_bytes(w_dtype, m, k, n) bytes.
  * ------------------------------------------------------------------------------------------- */
