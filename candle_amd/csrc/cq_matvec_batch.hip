@@ -445,7 +445,8 @@ int launch_qmb_long(const void *w, const uint8_t *op, void *dst, int dst_dtype, 
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     const int64_t nsteps = (n + 15) / 16;
-    const unsigned grid = (unsigned)(nsteps < 256 ? nsteps : 256);
+    // every workgroup the same number of blocks where that is possible with at most one workgroup per CU (896 blocks: 224 x 4)
+    const unsigned grid = (unsigned)(nsteps < 256 ? nsteps : (nsteps + (nsteps + 255) / 256 - 1) / ((nsteps + 255) / 256));
     hipLaunchKernelGGL(kern, dim3(grid), dim3(QB_NW * 64), lds_bytes, s, (const uint8_t *)w, op, dst, (int)n, (int)bpr, (int)rows, dst_dtype, stride_dst,
                        cpp
 #ifdef CL_STAMPS
@@ -464,7 +465,8 @@ int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int
         if (e != hipSuccess) return (int)e;
     }
     const int64_t nsteps = (n + 15) / 16;
-    const unsigned grid = (unsigned)(nsteps < 256 ? nsteps : 256);
+    // every workgroup the same number of blocks where that is possible with at most one workgroup per CU (896 blocks: 224 x 4)
+    const unsigned grid = (unsigned)(nsteps < 256 ? nsteps : (nsteps + (nsteps + 255) / 256 - 1) / ((nsteps + 255) / 256));
     hipLaunchKernelGGL(kern, dim3(grid), dim3(QB_NW * 64), lds_bytes, s, (const uint8_t *)w, op, dst, (int)n, (int)(k / 256), (int)rows, dst_dtype,
                        stride_dst
 #ifdef CL_STAMPS
