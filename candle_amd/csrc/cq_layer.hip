@@ -5,6 +5,8 @@
 // activation prologue of every kernel.  Each phase is the body of the streaming matvec kernel (cq_stream_body.h) with the
 // same step -> (workgroup, wave) assignment as the stand-alone launch, so results are bit-identical to the chain of launches.
 //
+// (-DCL_STAMPS compiles per-wave s_memrealtime stamps into the kernel for a timeline of the launch; the library is built without.)
+//
 // candle runs these as separate tensor ops (candle-transformers/src/models/quantized_llama.rs:56-63, 191-266, 584-591).
 #include "../../include/candle_hip_nn.h"
 #include "../../include/candle_hip_quant.h"

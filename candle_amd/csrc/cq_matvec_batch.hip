@@ -19,6 +19,9 @@
 //
 // The activations are quantized exactly like BlockQ8K::from_float by a small kernel of this file, which leaves them laid out
 // as the matrix operands the waves load.
+//
+// (-DCL_STAMPS compiles this file with per-wave s_memrealtime stamps and two extra entry points for a timeline of the launch;
+// the library is built without it.)
 #include "cq_actquant.h"
 #include "cq_device.h"
 #include "cq_fmt.h"
