@@ -209,11 +209,13 @@ def test_rank3_input_and_shape_errors():
         qmm.forward(torch.zeros((256, 2), device="cuda").t())
 
 
+@pytest.mark.parametrize("rows,k", [(3, 512), (5, 8192), (2, 512), (12, 2048)])
 @pytest.mark.parametrize("tdt", [torch.float16, torch.bfloat16])
-def test_half_activations_keep_dtype(tdt):
+def test_half_activations_keep_dtype(tdt, rows, k):
     # CPU f16 path: widen, quantize, dot, round the result to f16 (k_quants.rs:2652-2686); the GPU keeps the input dtype
-    blocks, qmm = make_weight(oracle.Q4K, 40, 512, seed=75)
-    x = torch.from_numpy(normal(76, (3, 512), 1.0)).to(tdt)
+    # (two rows: the streaming kernel; 3 .. 16 rows: the batched matrix-core kernel, rows of 8192 elements in column chunks)
+    blocks, qmm = make_weight(oracle.Q4K, 40, k, seed=75)
+    x = torch.from_numpy(normal(76, (rows, k), 1.0)).to(tdt)
     y = qmm.forward(x.cuda())
     torch.cuda.synchronize()
     assert y.dtype == tdt

@@ -336,7 +336,7 @@ def test_silu_mul_strided_views():
 
 
 @pytest.mark.parametrize("dtype", [12, 14, 13, 2, 8])
-@pytest.mark.parametrize("m,k,n", [(3, 512, 96), (8, 1024, 200), (40, 2048, 130), (130, 768, 64)])
+@pytest.mark.parametrize("m,k,n", [(3, 512, 96), (8, 1024, 200), (40, 2048, 130), (130, 768, 64), (5, 8192, 70)])
 def test_silu_mul_folded_into_the_quantizer_of_a_matmul(dtype, m, k, n):
     """feed_forward_w2 over several rows: equal to cq_nn_silu_mul + cq_qmatmul_forward (same arithmetic, bit for bit), and to
     the CPU sequence within what the device's expf may move through the quantizer."""
