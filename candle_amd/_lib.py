@@ -39,6 +39,7 @@ SIGNATURES = {
     "cq_indexed_moe_forward": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_moe_gemm_workspace_bytes": (_i64, [_int, _i64, _i64, _i64, _i64, _i64, _int]),
     "cq_moe_gemm_gguf_swiglu": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "cq_moe_gemm_gguf_down_after_pair": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "cq_moe_direct_pairs": (_int, [_int, _i64, _i64, _i64]),
     "cq_moe_gemm_gguf_pair": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),
     "cq_moe_gemm_gguf": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _vp]),

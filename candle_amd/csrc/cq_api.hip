@@ -375,6 +375,24 @@ int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, 
     return cq_moe_launch(a, workspace_dev, (hipStream_t)stream);
 }
 
+int cq_moe_gemm_gguf_down_after_pair(int w_dtype, const float *gate_dev, const float *up_dev, const void *w_down_dev, const float *topk_weights_dev,
+                                     float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int64_t k_pair,
+                                     void *workspace_dev, int64_t workspace_bytes, void *stream) {
+    int rc = moe_weight_dtype(w_dtype) ? check_mm_shape(w_dtype, k, n, size_m) : (int)CQ_ERR_DTYPE;
+    if (rc) return rc;
+    if (num_experts <= 0 || topk <= 0 || size_m % topk != 0 || k_pair <= 0) return CQ_ERR_SHAPE;
+    if (num_experts > (1 << 20)) return CQ_ERR_RANGE;
+    if (size_m == 0 || n == 0) return CQ_OK;
+    if ((rc = check_weight_ptr(w_dtype, w_down_dev))) return rc;
+    if (!gate_dev || !up_dev || !topk_weights_dev || !out_dev || !workspace_dev) return CQ_ERR_NULL;
+    if (!aligned(gate_dev, 16) || !aligned(up_dev, 16) || !aligned(topk_weights_dev, 4) || !aligned(out_dev, 4) || !aligned(workspace_dev, 256))
+        return CQ_ERR_ALIGN;
+    // the workspace is the one the gate / up call was given: at least what that call asked for
+    if (workspace_bytes < cq_moe_gemm_workspace_bytes(w_dtype, num_experts, topk, size_m, k, k_pair, 0)) return CQ_ERR_WORKSPACE;
+    return cq_moe_down_after_pair_launch(w_dtype, w_down_dev, gate_dev, up_dev, topk_weights_dev, out_dev, num_experts, topk, size_m, n, k, k_pair,
+                                         workspace_dev, (hipStream_t)stream);
+}
+
 int cq_moe_direct_pairs(int w_dtype, int64_t num_experts, int64_t size_m, int64_t k) {
     if (!moe_weight_dtype(w_dtype) || num_experts <= 0 || size_m < 0 || k <= 0) return 0;
     return cq_moe_direct(w_dtype, num_experts, size_m, k) ? 1 : 0;

@@ -74,6 +74,13 @@ struct MoeArgs {
 };
 int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k);
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s);
+// The down projection of an expert MLP right after a grouped gate / up call (cq_moe_launch with w_b, more pairs than the per-pair
+// kernels take) on the same workspace and pair list: out[pair] = topk_weights[pair] * W_down[e] . quantize(silu(gate[pair]) * up[pair]),
+// with the grouping that call left in the workspace.  CQ_ERR_RANGE when that call did not group on the matrix-core path or the
+// quantized rows of this one do not fit in front of its tables.
+int cq_moe_down_after_pair_launch(int w_dtype, const void *w_down, const float *gate, const float *up, const float *topk_weights, float *out,
+                                  int64_t num_experts, int64_t topk, int64_t n_pairs, int64_t n, int64_t k, int64_t k_pair, void *workspace,
+                                  hipStream_t s);
 
 // One (expert, activation row, output row, scale) pair of either MoE entry point.
 struct PairSource {
@@ -127,6 +134,8 @@ int cq_moe_pairs_swiglu_launch(int w_dtype, const void *w_gate, const void *w_up
 
 int cq_quantize_act_gather_launch(int w_dtype, const float *x, const int *row_map, void *scratch, int64_t k, int64_t rows, int64_t rows_alloc,
                                   hipStream_t s);
+int cq_quantize_act_swiglu_gather_launch(int w_dtype, const float *gate, const float *up, const int *row_map, const int *n_valid, const float *scale_in,
+                                         float *scale_out, void *scratch, int64_t k, int64_t rows, int64_t rows_alloc, hipStream_t s);
 // Expert-grouped MoE, 8 pairs per weight pass.  Chunk c (c < *n_chunks) covers sorted pairs [first[c], first[c] + count[c]) of expert[c];
 // the activation scratch holds the quantized rows in sorted-pair order (layout of rows_alloc rows).
 #define CQ_MOE_CHUNK 8

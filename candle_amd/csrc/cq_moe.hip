@@ -190,12 +190,42 @@ int64_t cq_moe_workspace_bytes_impl(int w_dtype, int64_t num_experts, int64_t n_
     return moe_workspace(w_dtype, num_experts, n_pairs, x_rows, k).total;
 }
 
-int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
-    if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
+// Does a call with this many pairs group them by expert and run the matrix-core kernel of the format over expert tiles?
+static bool moe_takes_mfma(int w_dtype, const void *w, const void *w_b, int64_t n_pairs, int64_t k) {
     // (the matrix-core kernel of the 32-element formats copies weight rows in 8-byte pieces: experts at another alignment take
     // the matvec passes)
-    const bool q0_ok = (a.w_dtype == CQ_Q4_0 || a.w_dtype == CQ_Q8_0) && ((uintptr_t)a.w & 7) == 0 && (!a.w_b || ((uintptr_t)a.w_b & 7) == 0);
-    const bool mfma = a.k % 256 == 0 && (cq_is_kquant(a.w_dtype) || q0_ok) && cq_has_mfma(a.w_dtype) && a.n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
+    const bool q0_ok = (w_dtype == CQ_Q4_0 || w_dtype == CQ_Q8_0) && ((uintptr_t)w & 7) == 0 && (!w_b || ((uintptr_t)w_b & 7) == 0);
+    return k % 256 == 0 && (cq_is_kquant(w_dtype) || q0_ok) && cq_has_mfma(w_dtype) && n_pairs >= CQ_MOE_MFMA_MIN_PAIRS;
+}
+static int moe_tile_rows(int64_t n_pairs, int64_t num_experts) { return n_pairs < 40 * num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE; }
+
+int cq_moe_down_after_pair_launch(int w_dtype, const void *w_down, const float *gate, const float *up, const float *topk_weights, float *out,
+                                  int64_t num_experts, int64_t topk, int64_t n_pairs, int64_t n, int64_t k, int64_t k_pair, void *workspace,
+                                  hipStream_t s) {
+    if (n_pairs > 0x7fffffffLL || topk <= 0 || n_pairs % topk) return CQ_ERR_RANGE;
+    // what the gate / up call did with these pairs, and what this one needs
+    // (K-quants only: whether Q4_0 / Q8_0 experts were grouped for the matrix cores also depended on that call's weight addresses)
+    if (!cq_is_kquant(w_dtype)) return CQ_ERR_RANGE;
+    if (cq_moe_direct(w_dtype, num_experts, n_pairs, k_pair) || !moe_takes_mfma(w_dtype, nullptr, nullptr, n_pairs, k_pair)) return CQ_ERR_RANGE;
+    if (!moe_takes_mfma(w_dtype, w_down, nullptr, n_pairs, k)) return CQ_ERR_RANGE;
+    const MoeWorkspace ws = moe_workspace(w_dtype, num_experts, n_pairs, n_pairs / topk, k_pair);
+    // the rows of this call are quantized into the front of the workspace: they must end before that call's tables begin
+    if (cq_act_layout(w_dtype, k, ws.rows_alloc).total > ws.offsets_off) return CQ_ERR_RANGE;
+    uint8_t *b = (uint8_t *)workspace;
+    const int *pout = (const int *)(b + ws.pout_off);
+    float *pscale = (float *)(b + ws.pscale_off);
+    const int *chunks = (const int *)(b + ws.chunk_off);
+    // pair i of the expert-sorted list reads row pair_out[i] (one row per pair here) and is scaled by that pair's routing weight
+    const int *n_valid = (const int *)(b + ws.offsets_off) + num_experts;          // the end of the last expert's segment
+    int rc = cq_quantize_act_swiglu_gather_launch(w_dtype, gate, up, pout, n_valid, topk_weights, pscale, b + ws.act_off, k, n_pairs, ws.rows_alloc, s);
+    if (rc) return rc;
+    MoeChunks mc{chunks, chunks + 1, chunks + 1 + ws.max_chunks, chunks + 1 + 2 * ws.max_chunks, pout, pscale, (int)ws.max_chunks};
+    return cq_matmul_moe_launch(w_dtype, w_down, b + ws.act_off, ws.rows_alloc, out, mc, k, n, moe_tile_rows(n_pairs, num_experts), s);
+}
+
+int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
+    if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
+    const bool mfma = moe_takes_mfma(a.w_dtype, a.w, a.w_b, a.n_pairs, a.k);
     if (a.w_b && !mfma) {
         // only the MFMA path shares its grouping pass and quantized activations between two weight tensors
         MoeArgs one = a;
@@ -224,7 +254,7 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     int *chunks = (int *)(b + ws.chunk_off);
     // Hundreds of pairs per call: the expert-sorted rows go through the MFMA prefill kernel of the format in tiles of up to
     // 128 rows of one expert (integer-exact like the dense paths).  Otherwise 8 pairs per matvec pass.
-    const int tile_rows = a.n_pairs < 40 * a.num_experts ? CQ_MOE_TILE_SMALL : CQ_MOE_TILE_LARGE;
+    const int tile_rows = moe_tile_rows(a.n_pairs, a.num_experts);
     if (a.num_experts <= GROUP_LDS_EXPERTS)
         hipLaunchKernelGGL(moe_group_kernel<true>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
                            (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);

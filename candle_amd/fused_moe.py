@@ -42,6 +42,9 @@ class FusedMoeGGUF:
         self.w_dtype = gate_experts.dtype()
         self.L = _lib.lib()
         self._cap = 0
+        # hundreds of pairs: the down projection reuses the grouping of the gate / up call and folds up * silu(gate) into its
+        # activation quantizer (False: silu_mul and a moe_gemm_gguf call of its own; the same bits)
+        self.share_grouping = True
 
     def _reserve(self, tokens: int) -> None:
         if tokens <= self._cap:
@@ -112,18 +115,28 @@ class FusedMoeGGUF:
                                               self.down_in.data_ptr(), E, topk, pairs, self.inter, hidden, sp)
             if fused != -6:
                 ck("cq_moe_gemm_gguf_swiglu", fused)
+        down_done = False
         if fused == -6:                                          # CQ_ERR_RANGE: not a shape of the fused launch
             # gate and up share x and the pairs: one grouping pass and one activation quantization for both
             ck("cq_moe_gemm_gguf_pair", L.cq_moe_gemm_gguf_pair(dt, x2.data_ptr(), self.gate_experts.device_ptr(), self.up_experts.device_ptr(),
                                                                 sti_ptr, eid_ptr, self.gate_out.data_ptr(), self.up_out.data_ptr(), E, topk, pairs,
                                                                 self.inter, hidden, 1 if is_prefill else 0, self.ws.data_ptr(), self.ws.numel(), sp))
-            # up * silu(gate), in chunks of rows the elementwise launch takes
-            for r0 in range(0, pairs, 65535):
-                r = min(65535, pairs - r0)
-                off = 4 * r0 * self.inter
-                ck("cq_nn_silu_mul", L.cq_nn_silu_mul(self.gate_out.data_ptr() + off, self.up_out.data_ptr() + off, self.down_in.data_ptr() + off,
-                                                      r, self.inter, self.inter, self.inter, sp))
-        gemm(self.down_in.data_ptr(), self.down_experts, self.topk_weights.data_ptr(), self.down_out, hidden, self.inter)
+            # the down projection on the grouping that call left in the workspace, up * silu(gate) inside its activation quantizer
+            rc = -6 if not self.share_grouping else L.cq_moe_gemm_gguf_down_after_pair(dt, self.gate_out.data_ptr(), self.up_out.data_ptr(), self.down_experts.device_ptr(),
+                                                    self.topk_weights.data_ptr(), self.down_out.data_ptr(), E, topk, pairs, hidden, self.inter,
+                                                    hidden, self.ws.data_ptr(), self.ws.numel(), sp)
+            if rc != -6:
+                ck("cq_moe_gemm_gguf_down_after_pair", rc)
+                down_done = True
+            else:
+                # up * silu(gate), in chunks of rows the elementwise launch takes
+                for r0 in range(0, pairs, 65535):
+                    r = min(65535, pairs - r0)
+                    off = 4 * r0 * self.inter
+                    ck("cq_nn_silu_mul", L.cq_nn_silu_mul(self.gate_out.data_ptr() + off, self.up_out.data_ptr() + off, self.down_in.data_ptr() + off,
+                                                          r, self.inter, self.inter, self.inter, sp))
+        if not down_done:
+            gemm(self.down_in.data_ptr(), self.down_experts, self.topk_weights.data_ptr(), self.down_out, hidden, self.inter)
         for t0 in range(0, tokens, 65535):
             t = min(65535, tokens - t0)
             ck("cq_nn_moe_sum", L.cq_nn_moe_sum(self.down_out.data_ptr() + 4 * t0 * topk * hidden, ys.data_ptr() + 4 * t0 * hidden, t, topk, hidden, sp))

@@ -216,6 +216,20 @@ int cq_moe_gemm_gguf_swiglu(int w_dtype, const float *x_dev, const void *w_gate_
                             const int32_t *expert_ids_dev, float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n,
                             int64_t k, void *stream);
 
+/* The down projection of an expert MLP (fused_moe.rs:281-294: silu(gate) * up, then moe_gemm_gguf with the routing weights)
+ * right after cq_moe_gemm_gguf_pair on the SAME workspace, pair list and expert count, for calls that bucket their pairs by
+ * expert (more pairs than cq_moe_direct_pairs takes; K-quant experts; k and k_pair multiples of 256): the grouping the pair
+ * call left in the workspace is used again (no second grouping pass), and silu(gate) * up is evaluated inside the activation
+ * quantizer (the f32 product is never written).  out[p, :] = topk_weights[p] * W_down[e_p] . quantize(silu(gate[p]) * up[p]) for
+ * pair p; gate / up: [size_m, k] f32 as the pair call wrote them (k = its n), k_pair = the pair call's k.  Bit-identical to
+ * cq_nn_silu_mul + cq_moe_gemm_gguf.  CQ_ERR_RANGE (nothing enqueued) when the pair call did not bucket its pairs for the
+ * matrix-core kernels or this call's quantized rows do not fit in front of that call's tables: the caller then takes the two
+ * separate calls.  Nothing else may use the workspace between the two calls.  No counterpart in the reference, which sorts the
+ * pairs once on the host side (fused_moe.rs:249-260) and passes the sorted list to all three calls. */
+int cq_moe_gemm_gguf_down_after_pair(int w_dtype, const float *gate_dev, const float *up_dev, const void *w_down_dev, const float *topk_weights_dev,
+                                     float *out_dev, int64_t num_experts, int64_t topk, int64_t size_m, int64_t n, int64_t k, int64_t k_pair,
+                                     void *workspace_dev, int64_t workspace_bytes, void *stream);
+
 /* 1 when a MoE call of size_m pairs runs every pair as its own fused matvec (no grouping by expert, so the order of the
  * pairs does not matter and a caller may skip its sort): up to 256 pairs always, up to 512 for rows of at most 32 units
  * (k <= 2048 for K-quants, 1024 otherwise) while size_m <= 3 * num_experts.  No counterpart in the reference, which always

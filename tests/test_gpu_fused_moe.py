@@ -202,6 +202,37 @@ def test_fused_moe_layer_qwen3_shape_token_batches(tokens, is_prefill):
     assert worst <= 1e-3, worst
 
 
+@pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q6K, oracle.Q5K])
+@pytest.mark.parametrize("tokens,E,topk", [(70, 16, 4), (300, 16, 4), (1000, 8, 2)])
+def test_down_projection_on_the_grouping_of_gate_and_up(dtype, tokens, E, topk):
+    """Hundreds of pairs: the down projection run on the grouping the gate / up call left in the workspace, with
+    up * silu(gate) inside its activation quantizer, gives the bits of silu_mul + a moe_gemm_gguf call of its own."""
+    hidden, inter = 512, 256
+    layer, ref = build_layer(dtype, E, hidden, inter, topk, True, seed=120)
+    x = normal(121 + tokens, (1, tokens, hidden), 1.0)
+    xd = torch.from_numpy(x).cuda()
+    layer.share_grouping = False
+    apart = layer.forward(xd, True).cpu().numpy()
+    layer.share_grouping = True
+    shared = layer.forward(xd, True).cpu().numpy()
+    assert np.array_equal(shared, apart)
+    assert rel_l2(shared, ref.forward(x)) <= 1e-3
+
+
+def test_down_after_pair_refuses_what_it_cannot_reuse():
+    lib = L()
+    p = 256          # an aligned non-null address: the calls below return before anything is enqueued
+    big = 1 << 40
+    # 16 pairs: the gate / up call ran every pair as a matvec of its own, there is no grouping to reuse
+    assert lib.cq_moe_gemm_gguf_down_after_pair(12, p, p, p, p, p, 128, 8, 16, 2048, 768, 2048, p, big, None) == -6
+    # Q8_0 experts: whether they were grouped for the matrix cores depended on the other call's weight addresses
+    assert lib.cq_moe_gemm_gguf_down_after_pair(8, p, p, p, p, p, 128, 8, 2048, 2048, 768, 2048, p, big, None) == -6
+    # this call's rows (k = 4096) would not fit in front of the tables of a call with k = 256
+    assert lib.cq_moe_gemm_gguf_down_after_pair(12, p, p, p, p, p, 128, 8, 2048, 2048, 4096, 256, p, big, None) == -6
+    assert lib.cq_moe_gemm_gguf_down_after_pair(12, p, p, p, p, p, 128, 8, 2048, 2048, 768, 2048, p, 1024, None) == -5   # CQ_ERR_WORKSPACE
+    assert lib.cq_moe_gemm_gguf_down_after_pair(12, None, p, p, p, p, 128, 8, 2048, 2048, 768, 2048, p, big, None) == -4
+
+
 def test_fused_moe_argument_errors():
     from candle_amd.fused_moe import FusedMoeGGUF
     layer, _ = build_layer(oracle.Q4K, 4, 256, 512, 2, True, seed=60)
