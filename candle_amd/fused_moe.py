@@ -45,6 +45,7 @@ class FusedMoeGGUF:
         # hundreds of pairs: the down projection reuses the grouping of the gate / up call and folds up * silu(gate) into its
         # activation quantizer (False: silu_mul and a moe_gemm_gguf call of its own; the same bits)
         self.share_grouping = True
+        self.sort_pairs = False
 
     def _reserve(self, tokens: int) -> None:
         if tokens <= self._cap:
@@ -92,12 +93,13 @@ class FusedMoeGGUF:
             ck("cq_nn_moe_route", L.cq_nn_moe_route(x2.data_ptr() + 4 * t0 * hidden, self.gate.data_ptr(), self.topk_ids.data_ptr() + 4 * t0 * topk,
                                                     self.topk_weights.data_ptr() + 4 * t0 * topk, self.router_logits.data_ptr() + 4 * t0 * E,
                                                     t, hidden, E, topk, 1 if self.norm_topk_prob else 0, sp))
-        # (expert_ids, sorted_token_ids) of fused_moe.rs:249-260.  The grouped matmuls give every pair its own row whatever
-        # the order of the pairs, and decode-sized calls (cq_moe_direct_pairs: up to 256 pairs, 512 for short expert rows) run
-        # each pair as its own matvec launch block, so the sort is skipped there: the pairs are taken in token order
-        # (expert_ids = topk_ids, sorted_token_ids = 0, 1, 2, ...).
+        # (expert_ids, sorted_token_ids) of fused_moe.rs:249-260.  Every path of the expert matmuls gives each pair a row of its
+        # own whatever the order of the pair list (decode-sized calls run each pair as its own matvec launch block, larger ones
+        # bucket the pairs by expert themselves), so the layer does not sort: the pairs are taken in token order
+        # (expert_ids = topk_ids, sorted_token_ids = 0, 1, 2, ...).  sort_pairs = True runs candle's sort (cq_nn_moe_sort) anyway;
+        # the results are the same bits.
         direct = bool(L.cq_moe_direct_pairs(dt, E, pairs, max(hidden, self.inter)))
-        if direct:
+        if not self.sort_pairs:
             eid_ptr, sti_ptr = self.topk_ids.data_ptr(), self.pair_iota.data_ptr()
         else:
             ck("cq_nn_moe_sort", L.cq_nn_moe_sort(self.topk_ids.data_ptr(), self.expert_ids.data_ptr(), self.sorted_token_ids.data_ptr(), pairs, E,

@@ -212,8 +212,10 @@ def test_down_projection_on_the_grouping_of_gate_and_up(dtype, tokens, E, topk):
     x = normal(121 + tokens, (1, tokens, hidden), 1.0)
     xd = torch.from_numpy(x).cuda()
     layer.share_grouping = False
+    layer.sort_pairs = True                    # the reference's sequence: sort, three grouped matmuls, silu_mul between them
     apart = layer.forward(xd, True).cpu().numpy()
     layer.share_grouping = True
+    layer.sort_pairs = False
     shared = layer.forward(xd, True).cpu().numpy()
     assert np.array_equal(shared, apart)
     assert rel_l2(shared, ref.forward(x)) <= 1e-3
