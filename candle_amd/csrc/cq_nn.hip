@@ -610,7 +610,7 @@ __global__ __launch_bounds__(HD) void attn_combine_kernel(const float *__restric
 //   * the result is left as per-split partials { acc[HD], m, l, 0, 0 } (stride HD + 4 floats, 16-byte aligned
 //     rows); the last workgroup of each kv head, or the prologue of the attention_wo matvec, merges them.
 constexpr int ATTD_MAX_SPLITS = 32;           // 4096 keys in splits of 128 (MAX_SEQ_LEN, quantized_llama.rs:27)
-constexpr int ATTD_FINE_SPLITS = 16;          // up to this many splits they are 64 keys long
+constexpr int ATTD_FINE_SPLITS = 32;          // up to this many splits they are 64 keys long
 constexpr int ATTD_COUNTER_BYTES = CQ_NN_ATTD_HEADER_BYTES;      // arrival counters of the in-kernel merge, one int per kv head, in front of the partials
 // Keys per split: 64 (workgroups of 8 waves) while that gives at most ATTD_FINE_SPLITS splits, else 128 (16 waves).  The
 // vector memory pipeline of a CU takes one instruction of a wave per 16 cycles whatever it loads, and a split asks for
@@ -623,12 +623,12 @@ __host__ __device__ inline int64_t attd_splits(int64_t max_kv_len) { const int64
 // split by split, in order (the arithmetic of attn_combine_kernel and of the merge prologue of the attention_wo matvec).
 // MS: the number of splits the registers hold (16 or 32).
 template <int HD, int G, int NW, int MS>
-__device__ __forceinline__ void attd_merge(const float *__restrict__ part, float *__restrict__ out, int kvh, int splits, int tid) {
+__device__ __forceinline__ void attd_merge(const float *__restrict__ part, float *__restrict__ out, int kvh, int stride, int splits, int tid) {
     const int lane = tid & 63;
     auto ld = [](const float *q) { return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
     for (int i = tid; i < G * HD; i += 64 * NW) {
         const int g = i / HD, d = i - g * HD;                 // g is the same in all lanes of a wave
-        const float *pp = part + (int64_t)(kvh * G + g) * splits * (HD + 4);
+        const float *pp = part + (int64_t)(kvh * G + g) * stride * (HD + 4);           // `stride` records per head, the first `splits` in use
         // Every load first (these bypass the caches: one after the other they would be a trip to memory each), and as few
         // load instructions as possible, they are what the last workgroup's time goes into: one instruction fetches
         // the (m, l) of all splits of the head (lane s: m of split s, lane MS + s: l), one per existing split the
@@ -660,6 +660,56 @@ __device__ __forceinline__ void attd_merge(const float *__restrict__ part, float
     }
 }
 
+// The read-only work of the single-token attention launch: workgroup `rank` of `count` read-only workgroups per grid column
+// pulls its share of the weights the following kernels will stream (attention_wo, feed_forward_w1 / w3) towards the caches
+// while this latency-bound kernel leaves the HBM idle.  Nothing is computed from the data; the store never executes for real weights.
+template <int NW>
+__device__ __forceinline__ void attd_prefetch(const u32x4 *__restrict__ pf, int64_t pf_chunks, int pf_piece16, uint32_t *__restrict__ pf_sink, int rank,
+                                              int count) {
+    uint32_t acc = 0;
+    if (pf_piece16 > 0) {
+        // Piece p of the range (pf_piece16 chunks: one wave step of the matvec that will stream it) is read later by a workgroup
+        // on XCD p % 8; workgroups are dealt to the XCDs round-robin by their linear index, so this one reads pieces of its own
+        // XCD only and they land in the L2 that the consumer will look in (grids of 8 columns).
+        const int lin = (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x;
+        const int xcd = lin & 7;
+        const int64_t npieces = pf_chunks / pf_piece16;
+        const int64_t mine = (npieces - xcd + 7) / 8;                       // pieces of this XCD
+        const int64_t vtotal = mine * pf_piece16, T = (int64_t)count * (64 * NW);
+        for (int64_t v = (int64_t)rank * (64 * NW) + threadIdx.x; v < vtotal; v += 2 * T) {
+            const int64_t v2 = v + T;
+            const int64_t q = v / pf_piece16, o = v - q * pf_piece16;
+            const u32x4 a = pf[(xcd + 8 * q) * pf_piece16 + o];
+            u32x4 b = {0, 0, 0, 0};
+            if (v2 < vtotal) {
+                const int64_t q2 = v2 / pf_piece16, o2 = v2 - q2 * pf_piece16;
+                b = pf[(xcd + 8 * q2) * pf_piece16 + o2];
+            }
+            acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
+        }
+        if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
+        return;
+    }
+    const int64_t nthreads = (int64_t)gridDim.x * count * (64 * NW);
+    int64_t i = ((int64_t)rank * gridDim.x + blockIdx.x) * (64 * NW) + threadIdx.x;
+    for (; i + 3 * nthreads < pf_chunks; i += 4 * nthreads) {
+        const u32x4 a = pf[i], b = pf[i + nthreads], c = pf[i + 2 * nthreads], d = pf[i + 3 * nthreads];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < pf_chunks; i += nthreads) {
+        const u32x4 a = pf[i];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w;
+    }
+    if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
+}
+
+// Splits that hold keys at this position: with the merge inside the kernel (out != NULL) only those take part -- a launch laid
+// out for a long context costs what the keys that exist cost -- and the workgroups of the others leave at once.
+template <int SPLIT>
+__device__ __forceinline__ int attd_active(int splits, int kv_len, bool merged) {
+    return merged ? min(splits, (kv_len + SPLIT - 1) / SPLIT) : splits;
+}
+
 template <int HD, int G, int NW, int SPLIT>
 __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__restrict__ pos_dev, const float *__restrict__ q, float *k_cache,
                                                                       const float *__restrict__ cos_t, const float *__restrict__ sin_t, int pos0,
@@ -671,46 +721,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
     // (parameter order: the fourteen dwords that sit in SGPRs when the wave starts are all that the key and query loads
     // need, so that those go out without waiting for a scalar load: neither for further arguments nor for the position)
     if ((int)blockIdx.y >= splits) {
-        // Workgroups beyond the attention splits only read: they pull the weights the following kernels will stream
-        // (attention_wo, feed_forward_w1 / w3) through the memory-side cache while this latency-bound kernel leaves
-        // the HBM idle.  Nothing is computed from the data; the store below never executes for real weights.
-        uint32_t acc = 0;
-        if (pf_piece16 > 0) {
-            // Piece p of the range (pf_piece16 chunks: one wave step of the matvec that will stream it) is read later by a workgroup
-            // on XCD p % 8; workgroups are dealt to the XCDs round-robin by their linear index, so this one reads pieces of its own
-            // XCD only and they land in the L2 that the consumer will look in.
-            const int lin = (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x;
-            const int xcd = lin & 7;
-            // rank of this workgroup among the read-only workgroups of its XCD, and their number (grids of 8 columns)
-            const int rank = (int)blockIdx.y - splits, count = (int)gridDim.y - splits;
-            const int64_t npieces = pf_chunks / pf_piece16;
-            const int64_t mine = (npieces - xcd + 7) / 8;                       // pieces of this XCD
-            const int64_t vtotal = mine * pf_piece16, T = (int64_t)count * (64 * NW);
-            for (int64_t v = (int64_t)rank * (64 * NW) + threadIdx.x; v < vtotal; v += 2 * T) {
-                const int64_t v2 = v + T;
-                const int64_t q = v / pf_piece16, o = v - q * pf_piece16;
-                const u32x4 a = pf[(xcd + 8 * q) * pf_piece16 + o];
-                u32x4 b = {0, 0, 0, 0};
-                if (v2 < vtotal) {
-                    const int64_t q2 = v2 / pf_piece16, o2 = v2 - q2 * pf_piece16;
-                    b = pf[(xcd + 8 * q2) * pf_piece16 + o2];
-                }
-                acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
-            }
-            if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
-            return;
-        }
-        const int64_t nthreads = (int64_t)gridDim.x * ((int)gridDim.y - splits) * (64 * NW);
-        int64_t i = ((int64_t)((int)blockIdx.y - splits) * gridDim.x + blockIdx.x) * (64 * NW) + threadIdx.x;
-        for (; i + 3 * nthreads < pf_chunks; i += 4 * nthreads) {
-            const u32x4 a = pf[i], b = pf[i + nthreads], c = pf[i + 2 * nthreads], d = pf[i + 3 * nthreads];
-            acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
-        }
-        for (; i < pf_chunks; i += nthreads) {
-            const u32x4 a = pf[i];
-            acc ^= a.x ^ a.y ^ a.z ^ a.w;
-        }
-        if (acc == 0x9e3779b9u && pf_sink) pf_sink[0] = acc;
+        // workgroups beyond the attention splits only read (they do not wait for the position: their share is fixed by the grid)
+        if (pf_chunks > 0) attd_prefetch<NW>(pf, pf_chunks, pf_piece16, pf_sink, (int)blockIdx.y - splits, (int)gridDim.y - splits);
         return;
     }
     constexpr int DPL = HD / 64, EPL = HD / 16, IT = SPLIT / (4 * NW), VU = SPLIT / NW, QR = (G + 3) / 4;
@@ -752,6 +764,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
     asm volatile("" ::"s"(v_cache), "s"(k_new), "s"(v_new), "s"(part));
     const int p = min(pos0 + p_raw, ctx - 1);
     const int kv_len = p + 1;
+    const int active = attd_active<SPLIT>(splits, kv_len, out != nullptr);
+    if (sp >= active) return;                     // uniform over the workgroup: no key of this split exists yet
     const int cnt = min(kv_len - j0, SPLIT);
     const int last = max(cnt - 1, 0);
     const bool has_p = p >= j0 && p < j0 + SPLIT;           // this split holds the new token (the same in every wave)
@@ -926,14 +940,14 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_kernel(const int32_t *__r
     __shared__ int s_last;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (tid == 0) s_last = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == splits - 1;
+    if (tid == 0) s_last = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == active - 1;
     __syncthreads();
     if (!s_last) return;
     static_assert(HD % 64 == 0 && ATTD_MAX_SPLITS <= 32, "a wave stays inside one query head; the lanes of a wave fetch the (m, l) pairs");
-    if (splits <= ATTD_FINE_SPLITS)
-        attd_merge<HD, G, NW, ATTD_FINE_SPLITS>(part, out, kvh, splits, tid);
+    if (active <= 16)
+        attd_merge<HD, G, NW, 16>(part, out, kvh, splits, active, tid);
     else
-        attd_merge<HD, G, NW, ATTD_MAX_SPLITS>(part, out, kvh, splits, tid);
+        attd_merge<HD, G, NW, ATTD_MAX_SPLITS>(part, out, kvh, splits, active, tid);
     if (tid == 0) __hip_atomic_store(&counters[kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -1484,7 +1498,9 @@ int cq_nn_attention_decode(const float *q_dev, const float *k_new_dev, const flo
     int64_t pf_rows = 0;
     if (pf_chunks > 0) {
         pf_rows = (256 - n_kv_head * splits + n_kv_head - 1) / n_kv_head;
-        if (pf_rows < 1) pf_rows = 1;
+        // ... and at least 160 of them (the splits beyond the position leave at once and make room): fewer would still be
+        // reading when the attention itself has finished
+        if (pf_rows < (160 + n_kv_head - 1) / n_kv_head) pf_rows = (160 + n_kv_head - 1) / n_kv_head;
     }
     dim3 grid((unsigned)n_kv_head, (unsigned)(splits + pf_rows));
     hipStream_t s = (hipStream_t)stream;

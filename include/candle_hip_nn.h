@@ -64,11 +64,14 @@ int cq_nn_attention(const float *q_dev, int64_t q_stride, const float *k_cache_d
  * [0, p].  q [n_head*head_dim], k_new / v_new [n_kv_head*head_dim] are the raw projection outputs (16-byte aligned;
  * q is not modified).  partials_dev is CQ_NN_ATTD_HEADER_BYTES of arrival counters followed by per-split records
  * { acc[head_dim], m, l, 0, 0 } for every head ([n_head][splits][head_dim + 4] floats, splits =
- * cq_nn_attention_decode_splits(max_kv_len): splits of 64 keys while 16 of them cover max_kv_len, else of 128 keys; at
- * most 32, i.e. max_kv_len <= 4096, MAX_SEQ_LEN of quantized_llama.rs:27; -1 beyond).  When out_dev != NULL the
+ * cq_nn_attention_decode_splits(max_kv_len): splits of 64 keys while 32 of them cover max_kv_len, i.e. up to 2048 keys, else
+ * of 128 keys; at most 32, i.e. max_kv_len <= 4096, MAX_SEQ_LEN of quantized_llama.rs:27; -1 beyond).  When out_dev != NULL the
  * workgroup of each kv head that finishes last merges that head group's splits into out_dev [n_head*head_dim] (same
- * launch, same arithmetic as a separate merge); with out_dev == NULL the merge is left to cq_nn_qmatmul_residual_attn,
- * which takes the address of the records (partials_dev + CQ_NN_ATTD_HEADER_BYTES).
+ * launch, same arithmetic as a separate merge), and only the splits that hold keys at position p take part: a launch laid
+ * out for a long context costs what the existing keys cost, the result does not depend on max_kv_len (splits of one length),
+ * and the records of the other splits are left untouched.  With out_dev == NULL every split writes its record (empty ones
+ * included) and the merge is left to cq_nn_qmatmul_residual_attn (up to 16 splits), which takes the address of the records
+ * (partials_dev + CQ_NN_ATTD_HEADER_BYTES).
  * The counters (one int per kv head, n_kv_head <= 64) must be zero before the first call with a buffer, and every call
  * leaves them zero; they sit in front of the records so that one buffer serves calls of any max_kv_len.
  * Key rows of the cache beyond p, up to the end of the last split of max_kv_len (never beyond ctx), are read before the

@@ -163,7 +163,8 @@ def test_attention_single_key_returns_value():
 
 
 @pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (8, 1, 128), (32, 8, 128)])
-@pytest.mark.parametrize("pos,ctx,max_kv", [(0, 16, 1), (5, 64, 64), (127, 256, 200), (128, 256, 256), (300, 1024, 301), (600, 1024, 1024)])
+@pytest.mark.parametrize("pos,ctx,max_kv", [(0, 16, 1), (5, 64, 64), (127, 256, 200), (128, 256, 256), (300, 1024, 301), (600, 1024, 1024),
+                                            (700, 2048, 2048), (1500, 2048, 2048), (1100, 4096, 4096)])
 def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
     """rope + cache append + attention over 64- or 128-key splits with the in-kernel merge == the CPU ops; called twice in a
     row on fresh caches."""
@@ -173,10 +174,11 @@ def test_attention_decode_fused_step(H, KV, D, pos, ctx, max_kv):
     kc0, vc0 = normal(33, (KV, ctx, D), 1.0), normal(34, (KV, ctx, D), 1.0)
     kc0[:, pos:], vc0[:, pos:] = np.nan, np.nan          # nothing at or beyond the new position may reach the result (key rows there are read, and masked)
     wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
-    # 64-key splits while at most 16 of them cover max_kv, else 128-key splits; more than 16 splits: not available
-    want_splits = (max_kv + 63) // 64 if (max_kv + 63) // 64 <= 16 else (max_kv + 127) // 128
+    # 64-key splits while at most 32 of them cover max_kv, else 128-key splits; more than 32 splits: not available
+    want_splits = (max_kv + 63) // 64 if (max_kv + 63) // 64 <= 32 else (max_kv + 127) // 128
     assert lib.cq_nn_attention_decode_splits(max_kv) == want_splits
-    assert lib.cq_nn_attention_decode_splits(2049) == 17 and lib.cq_nn_attention_decode_splits(4096) == 32 and lib.cq_nn_attention_decode_splits(4097) == -1
+    assert lib.cq_nn_attention_decode_splits(2048) == 32 and lib.cq_nn_attention_decode_splits(2049) == 17
+    assert lib.cq_nn_attention_decode_splits(4096) == 32 and lib.cq_nn_attention_decode_splits(4097) == -1
     ws = torch.full((wsb,), 0xff, dtype=torch.uint8, device="cuda")
     ws[:256] = 0                                         # the arrival counters of the in-kernel merge start at zero
     posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
@@ -236,6 +238,37 @@ def test_attention_decode_one_workspace_across_split_counts():
         assert int(ws[:256].to(torch.int32).sum()) == 0           # every call leaves its counters at zero
 
 
+def test_attention_decode_result_does_not_depend_on_the_layout_length():
+    """With the merge inside the kernel only the splits that hold keys take part, and up to 2048 keys all splits are 64 keys long:
+    a step laid out for 704, 768, 1024 or 2048 keys gives the same bits at position 700 (a server may capture one step for its
+    whole context), the splits beyond the position leave their (poisoned) records alone, and the counters end at zero."""
+    lib = L()
+    H, KV, D, ctx, pos = 32, 8, 128, 2048, 700
+    cos, sin = lo.precomput_freqs_cis(D, 500000.0, ctx)
+    q, k, v = dev(normal(80, (1, H * D), 1.0)), dev(normal(81, (1, KV * D), 1.0)), dev(normal(82, (1, KV * D), 1.0))
+    kc0, vc0 = normal(83, (KV, ctx, D), 1.0), normal(84, (KV, ctx, D), 1.0)
+    cd, sd = dev(cos), dev(sin)
+    posd = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    outs = []
+    for max_kv in (704, 768, 1024, 2048):
+        wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
+        ws = torch.zeros(wsb // 4, dtype=torch.float32, device="cuda")
+        ws[64:] = float("nan")
+        kc, vc, out = dev(kc0), dev(vc0), torch.zeros((1, H * D), device="cuda")
+        ok(lib.cq_nn_attention_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), kc.data_ptr(), vc.data_ptr(), cd.data_ptr(), sd.data_ptr(),
+                                      out.data_ptr(), posd.data_ptr(), 0, H, KV, D, ctx, max_kv, float(np.float32(1.0 / math.sqrt(D))),
+                                      ws.data_ptr(), wsb, None, 0, 0, None))
+        torch.cuda.synchronize()
+        assert int(ws[:64].view(torch.int32).abs().sum()) == 0
+        splits = lib.cq_nn_attention_decode_splits(max_kv)
+        rec = ws[64:].view(H, splits, D + 4)
+        assert not torch.isnan(rec[:, :11]).any() and torch.isnan(rec[:, 11:]).all()      # 701 keys: 11 splits of 64
+        outs.append(out.cpu().numpy())
+    assert not np.isnan(outs[0]).any()
+    for o in outs[1:]:
+        assert np.array_equal(o, outs[0])
+
+
 @pytest.mark.parametrize("H,KV,D", [(4, 2, 64), (32, 8, 128)])
 def test_attention_decode_beyond_2048_keys(H, KV, D):
     """MAX_SEQ_LEN of quantized_llama.rs:27 is 4096: position 3000 of a 4096-key context, 32 splits of 128 keys."""
@@ -247,7 +280,8 @@ def test_attention_decode_beyond_2048_keys(H, KV, D):
     _attention_decode_case(lib, ws, wsb, H, KV, D, 4095, 4096, 4096, 510)
 
 
-@pytest.mark.parametrize("pos,max_kv", [(760, 768), (1000, 1024)], ids=["12-splits", "16-splits"])
+@pytest.mark.parametrize("pos,max_kv", [(760, 768), (1000, 1024), (700, 2048), (2040, 2048)],
+                         ids=["12-splits", "16-splits", "11-of-32-splits", "32-splits"])
 def test_attention_decode_in_kernel_merge_soak(pos, max_kv):
     """The in-kernel merge reads the partials of workgroups on other XCDs after one relaxed device-scope counter increment,
     with no fence.  20 000 launches at the 8B head shape, the records poisoned with NaN before each: every launch must
@@ -266,7 +300,7 @@ def test_attention_decode_in_kernel_merge_soak(pos, max_kv):
     vc_ref[:, pos:pos + 1] = v.reshape(1, KV, D).transpose(1, 0, 2)
     want = attention_oracle(want_q, kc_ref, vc_ref, pos, H, KV, D)
     wsb = lib.cq_nn_attention_decode_workspace_bytes(H, D, max_kv)
-    assert lib.cq_nn_attention_decode_splits(max_kv) == (12 if max_kv == 768 else 16)
+    assert lib.cq_nn_attention_decode_splits(max_kv) == (12 if max_kv == 768 else 16 if max_kv == 1024 else 32)
     ws = torch.zeros(wsb // 4, dtype=torch.float32, device="cuda")
     records = ws[64:]                                     # behind the 256 bytes of counters
     kc, vc, out = dev(kc0), dev(vc0), torch.zeros((1, H * D), device="cuda")
@@ -294,7 +328,7 @@ def test_attention_decode_in_kernel_merge_soak(pos, max_kv):
 
 
 @pytest.mark.parametrize("dtype", [12, 14, 2])
-@pytest.mark.parametrize("pos,max_kv", [(3, 128), (700, 701), (700, 2048)])
+@pytest.mark.parametrize("pos,max_kv", [(3, 128), (700, 701), (700, 1024)])
 def test_attention_merge_as_matvec_prologue(dtype, pos, max_kv):
     """attention partials merged inside the attention_wo matvec == merge kernel followed by the plain fused matvec, bit for bit."""
     import oracle
