@@ -69,6 +69,41 @@ constexpr int QB_OP_COL_BYTES = 8 * 4 * 16 * 8;       // 4096
 constexpr int QB_REC_BYTES = 32;
 __host__ __device__ inline int64_t qb_operand_bytes(int64_t bpr) { return bpr * (QB_OP_COL_BYTES + 16 * QB_REC_BYTES); }
 
+// The arithmetic of cq_quantize_q8k_vals (cq_actquant.h) on the four values a lane holds of a 256-element span (elements
+// 4 lane .. 4 lane + 3): the first element of largest magnitude sets the scale.  packed: the lane's four int8 values;
+// lsum: their sum; d: the span's scale.
+__device__ __forceinline__ void qb_quantize_span(const float (&v)[4], int lane, uint32_t &packed, int &lsum, float &d) {
+    float amax = 0.0f;
+    int idx = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float a = fabsf(v[i]);
+        if (amax < a) { amax = a; idx = i; }
+    }
+    const float wmax = wave_max_nonneg(amax);
+    const int cand = wave_min_int((amax == wmax && wmax != 0.0f) ? lane * 4 + idx : 256);
+    const float mine = idx == 0 ? v[0] : idx == 1 ? v[1] : idx == 2 ? v[2] : v[3];
+    const float maxv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), (cand >> 2) & 63));
+    packed = 0;
+    lsum = 0;
+    d = 0.0f;
+    if (wmax != 0.0f) {
+        const float iscale = -127.0f / maxv;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int q = cq_round_sat_i8(iscale * v[i]);
+            lsum += q;
+            packed |= (uint32_t)(q & 0xff) << (8 * i);
+        }
+        d = 1.0f / iscale;
+    }
+}
+// where the lane's dword of a span goes inside one column of operands laid out [g < 4][kg < 4][slot < SLOTS][16 bytes]:
+// elements 4 lane .. + 3 are values 4 (lane % 8) .. + 3 of sub-block lane / 8: lane group kg = (lane % 8) / 2, dword lane % 2
+__device__ __forceinline__ int qb_operand_dword(int lane, int c, int slots) {
+    return (((lane >> 4) * 4 + ((lane & 7) >> 1)) * slots + c) * 16 + 8 * ((lane >> 3) & 1) + 4 * (lane & 1);
+}
+
 // XDT < 0: the rows are silu(x[c]) * up[c], rows of f32 with strides of their own (a feed-forward's w2 over several rows)
 template <int XDT>
 __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict__ x, const float *__restrict__ up, int64_t x_stride, int64_t up_stride,
@@ -81,34 +116,12 @@ __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict
         if constexpr (XDT < 0) cq_load_swiglu4((const float *)x, up, c * x_stride + s * 256 + lane * 4, c * up_stride + s * 256 + lane * 4, v);
         else cq_load4<XDT>(x, c * x_stride + s * 256 + lane * 4, v);
     }
-    // the arithmetic of cq_quantize_q8k_vals (cq_actquant.h): the first element of largest magnitude sets the scale
-    float amax = 0.0f;
-    int idx = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float a = fabsf(v[i]);
-        if (amax < a) { amax = a; idx = i; }
-    }
-    const float wmax = wave_max_nonneg(amax);
-    const int cand = wave_min_int((amax == wmax && wmax != 0.0f) ? lane * 4 + idx : 256);
-    const float mine = idx == 0 ? v[0] : idx == 1 ? v[1] : idx == 2 ? v[2] : v[3];
-    const float maxv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), (cand >> 2) & 63));
-    uint32_t packed = 0;
-    int lsum = 0;
-    float d = 0.0f;
-    if (wmax != 0.0f) {
-        const float iscale = -127.0f / maxv;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int q = cq_round_sat_i8(iscale * v[i]);
-            lsum += q;
-            packed |= (uint32_t)(q & 0xff) << (8 * i);
-        }
-        d = 1.0f / iscale;
-    }
-    // elements 4 lane .. + 3: sub-block lane / 8, values 4 (lane % 8) .. + 3 of it: lane group kg = (lane % 8) / 2, dword lane % 2
+    uint32_t packed;
+    int lsum;
+    float d;
+    qb_quantize_span(v, lane, packed, lsum, d);
     uint8_t *colp = op + (int64_t)s * QB_OP_COL_BYTES;
-    *(uint32_t *)(colp + (((lane >> 4) * 4 + ((lane & 7) >> 1)) * 16 + c) * 16 + 8 * ((lane >> 3) & 1) + 4 * (lane & 1)) = packed;
+    *(uint32_t *)(colp + qb_operand_dword(lane, c, 16)) = packed;
     const int s32 = oct_sum(lsum);                        // the sum of the 32-element sub-block, in its eight lanes
     uint32_t bl[2] = {0, 0}, bh[2] = {0, 0};
 #pragma unroll
@@ -124,7 +137,17 @@ __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict
     }
 }
 
-template <int CPW, int DEPTH>
+// FQ > 0: `op` is not the operand buffer but the f32 activations themselves, [rows == FQ][256 bpr], and every wave quantizes
+// the spans of its own columns while the first tiles are on their way (all 64 lanes on one span at a time, the int8 values
+// turned into matrix operands through the LDS of the last tile of the ring, which the weights need only later).  The same
+// results as from qb_quantize_kernel's operands, bit for bit (where the first largest magnitude of a span is negative the
+// int8 values and the scale both come out with the other sign, as in the streaming kernel, and their products are the same).  Every workgroup repeats the work, which pays while it hides behind the
+// first tile's latency: up to 8 rows.  (The row count is a template parameter: with the spans behind run-time conditions
+// the compiler cannot interleave their dependent chains, and a span costs 0.67 us instead of a third of that.)
+constexpr int QB_FQ_MAX_SPANS = 16;                // spans (columns x rows) a wave quantizes itself at most; beyond, the separate kernel is ahead
+constexpr int QB_FQ_REC = 32;                      // bytes of a staged record {u8 bl[8], u8 bh[8], f32 d, unused}
+__host__ __device__ constexpr int qb_fq_col_bytes(int fq) { return fq * 256 + fq * QB_FQ_REC; }      // operands + records of one column
+template <int CPW, int DEPTH, int FQ>
 __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ op, void *__restrict__ dst, int n, int bpr,
                                                               int rows, int dst_dtype, int64_t stride_dst
 #ifdef CL_STAMPS
@@ -164,6 +187,93 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(tile + kb * QB_KB), 16, lane * 16, kb * 1024, 0, 0);
         }
     };
+    long A[CPW][8];
+    u32x4 aux[CPW][4];                            // {bl 0-3, bl 4-7, bh 0-3, bh 4-7} of batch row 4 kg + r: sub-block sum j = 128 * bh_j + bl_j
+    float d8[CPW][4];
+    if constexpr (FQ > 0) {
+        // ---- the wave quantizes the activations of its columns itself ----
+        // Vector loads complete in order: the activations are asked for before the weights, or they would wait for them.
+        const float *x = (const float *)op;
+        constexpr int NSP = CPW * FQ;              // the wave's spans: (column ci, batch row r) = span ci * FQ + r
+        float xv[NSP][4];
+#pragma unroll
+        for (int ci = 0; ci < CPW; ci++) {
+            const int col = min(col0 + ci, bpr - 1);
+#pragma unroll
+            for (int r = 0; r < FQ; r++) {
+                const f32x4 t = *(const f32x4 *)(x + ((int64_t)r * bpr + col) * 256 + lane * 4);
+                xv[ci * FQ + r][0] = t.x; xv[ci * FQ + r][1] = t.y; xv[ci * FQ + r][2] = t.z; xv[ci * FQ + r][3] = t.w;
+            }
+        }
+        asm volatile("" ::: "memory");
+        issue(0);
+        asm volatile("" ::: "memory");
+        QB_STAMP(0);
+        uint8_t *stage = lds + (DEPTH - 1) * TILE + wv * (CPW * qb_fq_col_bytes(FQ));        // this wave's part of the ring's last tile
+        // the streaming kernel's span quantizer (cq_stream.h): the largest magnitudes, one division sequence for all spans, the values
+        uint32_t wmax[NSP];
+        float iscale[NSP], dsp[NSP];
+        // (the six cross-lane steps of all spans side by side: a span's chain alone waits two cycles between steps)
+#pragma unroll
+        for (int j = 0; j < NSP; j++) {
+            float amax = fmaxf(fmaxf(fabsf(xv[j][0]), fabsf(xv[j][1])), fmaxf(fabsf(xv[j][2]), fabsf(xv[j][3])));
+            amax = amax == amax ? amax : 0.0f;
+            wmax[j] = __float_as_uint(amax);
+        }
+#define QB_S(ctrl, rm, bc)                                                                                                    \
+    _Pragma("unroll") for (int j = 0; j < NSP; j++)                                                                           \
+        wmax[j] = max(wmax[j], (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wmax[j], ctrl, rm, 0xf, bc));                    \
+    __builtin_amdgcn_sched_barrier(0);
+        QB_S(0x111, 0xf, true) QB_S(0x112, 0xf, true) QB_S(0x114, 0xf, true) QB_S(0x118, 0xf, true) QB_S(0x142, 0xa, false) QB_S(0x143, 0xc, false)
+#undef QB_S
+#pragma unroll
+        for (int j = 0; j < NSP; j++) wmax[j] = (uint32_t)__builtin_amdgcn_readlane((int)wmax[j], 63);
+        qs_span_scales<NSP>(wmax, lane, iscale, dsp);
+        QB_STAMP(14);
+        // (the second tile is asked for a little after the first, as in the kernel without the quantizer: asked for together, the
+        // first tiles of the late workgroups queue behind the second tiles of the early ones and the launch starts 0.5 us later)
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int i = 1; i < DEPTH - 1; i++) issue(i);
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int ci = 0; ci < CPW; ci++) {
+            uint8_t *colp = stage + ci * qb_fq_col_bytes(FQ), *recs = colp + FQ * 256;
+#pragma unroll
+            for (int r = 0; r < FQ; r++) {
+                const int j = ci * FQ + r;
+                int q[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) q[i] = qs_round_i8(iscale[j] * xv[j][i]);
+                const uint32_t packed = qs_pack4(q);
+                *(uint32_t *)(colp + qb_operand_dword(lane, r, FQ)) = packed;
+                const int s32 = oct_sum(sdot4(packed, 0x01010101u, 0));       // the sum of the 32-element sub-block, in its eight lanes
+                uint8_t *rec = recs + r * QB_FQ_REC;
+                // (the eight lanes of a sub-block write the same bytes, every lane the same scale: cheaper than masking lanes off)
+                rec[lane >> 3] = (uint8_t)(s32 & 127);
+                rec[8 + (lane >> 3)] = (uint8_t)(s32 >> 7);
+                *(float *)(rec + 16) = dsp[j];
+            }
+        }
+        // (the wave reads back what it wrote itself: LDS takes a wave's accesses in order)
+#pragma unroll
+        for (int ci = 0; ci < CPW; ci++) {
+            const uint8_t *colp = stage + ci * qb_fq_col_bytes(FQ), *recs = colp + FQ * 256;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const i64x2 v = c < FQ ? *(const i64x2 *)(colp + ((g * 4 + kg) * FQ + c) * 16) : i64x2{0, 0};
+                A[ci][2 * g] = v.x; A[ci][2 * g + 1] = v.y;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint8_t *rec = recs + min(4 * kg + r, FQ - 1) * QB_FQ_REC;         // (results of batch rows beyond the last are not stored)
+                aux[ci][r] = *(const u32x4 *)rec;
+                d8[ci][r] = *(const float *)(rec + 16);
+            }
+        }
+        // everything is in registers before the wave passes the first barrier, behind which the last tile is asked for
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    } else {
     issue(0);                                     // the first tile is on its way before anything else is asked for
     asm volatile("" ::: "memory");
 
@@ -172,9 +282,6 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
     // the weights the second, so a lane's four results belong to ONE weight row (row c of the block: one header to decode per
     // column) and to the batch rows 4 kg + r, whose block sums and scales it keeps as well.
     QB_STAMP(0);
-    long A[CPW][8];
-    u32x4 aux[CPW][4];                            // {bl 0-3, bl 4-7, bh 0-3, bh 4-7} of batch row 4 kg + r: sub-block sum j = 128 * bh_j + bl_j
-    float d8[CPW][4];
     // (a wave's load of one operand is 512 contiguous bytes; the four lane groups read four records)
 #pragma unroll
     for (int ci = 0; ci < CPW; ci++) {
@@ -195,6 +302,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int i = 1; i < DEPTH - 1; i++) issue(i);
+    }
     const int my = bx < nsteps ? (nsteps - bx + gx - 1) / gx : 0;
     QB_STAMP(1);
     for (int i = 0; i < my; i++) {
@@ -459,10 +567,10 @@ int launch_qmb_long(const void *w, const uint8_t *op, void *dst, int dst_dtype, 
     return (int)hipGetLastError();
 }
 
-template <int CPW, int DEPTH>
+template <int CPW, int DEPTH, int FQ = 0>
 int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
                  hipStream_t s) {
-    auto kern = qmb_q4k_kernel<CPW, DEPTH>;
+    auto kern = qmb_q4k_kernel<CPW, DEPTH, FQ>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
@@ -480,10 +588,23 @@ int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int
 }
 // Three tiles where LDS holds them (the one being worked on and two on their way), else two.  (Four were measured slower:
 // with three tiles asked for at the start the first one lands 1 us later, and the steady state gains nothing.)
+// fq: `op` holds the f32 activations (see the kernel); the caller has checked qb_fused_rows
 template <int CPW>
-int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int fq, hipStream_t s) {
     const int tile = qb_tile_bytes((int)(16 * (k / 256) * QB_BB));
     const int fit = (QB_LDS_BYTES - QB_RED_BYTES - 1024) / tile;
+#define QB_FQ_CASE(R)                                                                                                                           \
+    case R:                                                                                                                                    \
+        if constexpr (CPW * R <= QB_FQ_MAX_SPANS) {                                                                                            \
+            if (fit >= 3) return launch_qmb_d<CPW, 3, R>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)3 * tile + QB_RED_BYTES, s);  \
+            if (fit == 2) return launch_qmb_d<CPW, 2, R>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)2 * tile + QB_RED_BYTES, s);  \
+        }                                                                                                                                      \
+        return CQ_ERR_RANGE;
+    switch (fq) {
+        QB_FQ_CASE(3) QB_FQ_CASE(4) QB_FQ_CASE(5) QB_FQ_CASE(6) QB_FQ_CASE(7) QB_FQ_CASE(8)
+        default: break;
+    }
+#undef QB_FQ_CASE
     if (fit >= 3) return launch_qmb_d<CPW, 3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)3 * tile + QB_RED_BYTES, s);
     if (fit == 2) return launch_qmb_d<CPW, 2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)2 * tile + QB_RED_BYTES, s);
     return CQ_ERR_RANGE;
@@ -505,12 +626,33 @@ int64_t cq_matvec_batch_workspace(int w_dtype, int64_t k, int64_t rows) {
     return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= QB_MAX_BPR ? cq_align256(qb_operand_bytes(k / 256)) : 0;
 }
 
+// Rows the main kernel quantizes itself (= rows), 0: the quantize kernel runs first.  Contiguous f32 rows of up to
+// 24 super-blocks, at most 8 of them and at most QB_FQ_MAX_SPANS spans per wave, and the staged operands of the eight waves
+// must fit one tile of the ring.
+static int qb_fused_rows(int x_dtype, const void *x, int64_t x_stride, int64_t k, int64_t rows) {
+    const int64_t bpr = k / 256, cpw = (bpr + QB_NW - 1) / QB_NW;
+    if (x_dtype != CQ_F32 || x_stride != k || bpr > 3 * QB_NW || rows > 8 || cpw * rows > QB_FQ_MAX_SPANS || ((uintptr_t)x & 15)) return 0;
+    const int fq = (int)rows;
+    const int tile = qb_tile_bytes((int)(16 * bpr * QB_BB));
+    if ((QB_LDS_BYTES - QB_RED_BYTES - 1024) / tile < 2) return 0;
+    return QB_NW * cpw * qb_fq_col_bytes(fq) <= tile ? fq : 0;
+}
+
 // QMatMul::forward for 3 .. 16 rows of x: one small kernel quantizes them into `workspace`, then the weights are read once.
 // x_dtype < 0: the rows are silu(x) * up, f32, with row strides in floats (multiples of 4).
 static int qb_launch(int w_dtype, const void *w, const void *x, const float *up, int64_t x_stride, int64_t up_stride, int x_dtype, void *workspace,
                      void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
     if (!cq_matvec_batch_takes(w_dtype, w, k, n, rows)) return CQ_ERR_RANGE;
     const int bpr = (int)(k / 256);
+    const int64_t cpw = (k / 256 + QB_NW - 1) / QB_NW;
+    if (const int fq = qb_fused_rows(x_dtype, x, x_stride, k, rows)) {
+        switch (cpw) {
+            case 1: return launch_qmb<1>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
+            case 2: return launch_qmb<2>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
+            case 3: return launch_qmb<3>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
+            default: return CQ_ERR_RANGE;
+        }
+    }
     const unsigned qgrid = (unsigned)((bpr * 16 + 3) / 4);
     uint8_t *op = (uint8_t *)workspace;
     switch (x_dtype) {
@@ -529,11 +671,10 @@ static int qb_launch(int w_dtype, const void *w, const void *x, const float *up,
             default: return CQ_ERR_RANGE;
         }
     }
-    const int64_t cpw = (k / 256 + QB_NW - 1) / QB_NW;
     switch (cpw) {
-        case 1: return launch_qmb<1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, s);
-        case 2: return launch_qmb<2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, s);
-        case 3: return launch_qmb<3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, s);
+        case 1: return launch_qmb<1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
+        case 2: return launch_qmb<2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
+        case 3: return launch_qmb<3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
         default: return CQ_ERR_RANGE;
     }
 }

@@ -104,6 +104,29 @@ def test_q4k_batched_rows_vs_oracle(k, n, batch):
         assert rel_l2(got[r], want[r]) <= TIGHT, r
 
 
+@pytest.mark.parametrize("k", [256, 2048, 4096, 6144])
+@pytest.mark.parametrize("rows", [3, 4, 5, 6, 8])
+def test_q4k_batched_rows_quantized_inside_the_kernel(k, rows):
+    """Few f32 rows are quantized by the waves of the matvec kernel itself (up to 16 spans per wave), more rows by a kernel
+    of their own: a row gives the same bits either way, and both agree with the oracle.  The rows hold what the two
+    quantizers treat differently inside: a largest value that is negative, a tie between +max and -max, an all-zero span."""
+    n = 203
+    blocks, qmm = make_weight(oracle.Q4K, n, k, seed=171)
+    x = normal(172 + rows, (rows, k), 1.0)
+    x[0, :256] = 0.0
+    x[1, 5] = -9.0
+    x[2, 7] = 6.0
+    x[2, 9] = -6.0
+    x[rows - 1, k - 3] = -7.5
+    big = np.concatenate([x, normal(173, (16 - rows, k), 1.0)])
+    got = forward(qmm, x)
+    ref = forward(qmm, big)[:rows]
+    assert np.array_equal(got, ref)
+    want = oracle.matmul_fast(oracle.Q4K, x, blocks, n, 8)
+    for r in range(rows):
+        assert rel_l2(got[r], want[r]) <= TIGHT, r
+
+
 def test_cfg1_q8_0_4096x4096():
     # BASELINE configs[0]: Q8_0 weight [4096 x 4096], activation 1 x 4096
     blocks, qmm = make_weight(oracle.Q8_0, 4096, 4096, seed=1)
