@@ -148,6 +148,17 @@ struct MoeChunks {
 int cq_moe_chunks_launch(int w_dtype, const void *w, const void *scratch, int64_t rows_alloc, float *out, const MoeChunks &mc, int64_t k,
                          int64_t n, hipStream_t s);
 
+// Q4_K experts hit by a few dozen pairs each as batched matvecs (cq_matvec_batch.hip): the expert-sorted pairs of an expert are the
+// batch rows, in sets of 16 whose quantized rows sit in operand tiles.
+bool cq_moe_stream_shape(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n);      // ... by shape alone
+bool cq_moe_stream_takes(int w_dtype, const void *w, const void *w_b, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n);
+int64_t cq_moe_stream_operand_bytes(int64_t num_experts, int64_t n_pairs, int64_t k);
+#define CQ_MOE_STREAM_CHUNK 16
+int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *row_map, const float *scale_in, float *scale_out, const int *chunks,
+                                  int64_t max_chunks, const int *offsets, void *op, int64_t k, hipStream_t s);
+int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
+                         const float *pair_scale, int64_t num_experts, int64_t k, int64_t n, hipStream_t s);
+
 // Pairs from which a K-quant MoE call goes through the MFMA kernel (tiles of expert-sorted rows): everything the
 // per-pair kernels do not take.  Measured on 128 experts of 768 x 2048: 264-1016 pairs take 211-229 us per layer on
 // 32-row tiles against 427-644 us on the 8-pairs-per-pass matvec.

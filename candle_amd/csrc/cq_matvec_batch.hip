@@ -20,6 +20,9 @@
 // The activations are quantized exactly like BlockQ8K::from_float by a small kernel of this file, which leaves them laid out
 // as the matrix operands the waves load.
 //
+// The same formulation serves MoE calls with hundreds of pairs: every expert a batched matvec over its own pairs
+// (qme_q4k_kernel at the end of this file).
+//
 // (-DCL_STAMPS compiles this file with per-wave s_memrealtime stamps and two extra entry points for a timeline of the launch;
 // the library is built without it.)
 #include "cq_actquant.h"
@@ -610,6 +613,302 @@ int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64
     return CQ_ERR_RANGE;
 }
 
+
+// ---- the expert-grouped form (MoE with hundreds of pairs) -----------------------------------------------------------------
+// Every expert hit by at most a few dozen pairs is a batched matvec of its own: its pairs are the batch rows (sets of 16, two
+// sets held in registers per pass over the weights), its matrix the weight stream.  What bounds such a launch is how evenly the
+// experts' bytes are spread over the CUs (a CU streams about 20 KB per us through the copy-to-LDS path): workgroup
+// (part, expert, tensor) takes a contiguous range of the expert's row tiles, with parts x experts x tensors a multiple of the
+// CU count where the shape allows, and leaves at once when the expert has no pair.
+//
+// Short rows.  With fewer than eight super-blocks per row the waves do not all get a column: CW waves (a power of two) share a
+// block of 16 rows, wave w taking columns (w % CW) * CPW .. of row block w / CW of a tile of 8 / CW row blocks.
+//
+// Operands.  Tile (expert e, set s) — pairs offsets[e] + 16 s .. of the expert-sorted pair list — lives at tile index
+// offsets[e] / 16 + e + s (unique and below n_pairs / 16 + experts without a scan over the experts), laid out like one column
+// set of the dense kernel: [column][g][kg][slot][16 bytes], then [column][slot] records.
+// Pair b of a set sits in operand slot 4 (b % 4) + b / 4: a lane's result r of lane group kg then belongs to pair 4 r + kg, and a
+// set of `cnt` pairs needs only the first ceil(cnt / 4) of a lane's four results worked out (the scaling of a result is most of
+// the kernel's vector work, and most sets are far from full).
+__host__ __device__ constexpr int qme_slot(int b) { return 4 * (b & 3) + (b >> 2); }
+constexpr int QME_TILE_COL_BYTES = QB_OP_COL_BYTES + 16 * QB_REC_BYTES;          // 4608 bytes of a tile per super-block column
+__host__ __device__ inline int64_t qme_operand_tiles(int64_t n_pairs, int64_t num_experts) { return n_pairs / 16 + num_experts + 1; }
+
+// workgroup (chunk of the grouping pass, column): one wave per pair of the chunk (16 sorted pairs of one expert at most) quantizes
+// the pair's 256 values of the column, gathered through row_map, into the chunk's operand tile — the streaming kernel's span
+// quantizer (cq_stream.h: where the first largest magnitude is negative the int8 values and the scale come out with the other
+// sign than BlockQ8K::from_float gives them, and every product is the same).  SW: the rows are silu(x[row]) * up[row], and the
+// pair's scale is scale_in[row] (the down projection after gate / up: one row per pair)
+template <bool SW>
+__global__ __launch_bounds__(1024) void qme_quantize_kernel(const float *__restrict__ x, const float *__restrict__ up, const int *__restrict__ row_map,
+                                                            const float *__restrict__ scale_in, float *__restrict__ scale_out,
+                                                            const int *__restrict__ chunks, int max_chunks, const int *__restrict__ offsets,
+                                                            uint8_t *__restrict__ op, int bpr) {
+    const int ci = blockIdx.x, col = blockIdx.y;
+    if (ci >= chunks[0]) return;
+    const int count = chunks[1 + 2 * max_chunks + ci];
+    const int lane = threadIdx.x & 63, c = threadIdx.x >> 6;
+    if (c >= count) return;
+    const int e = chunks[1 + ci], first = chunks[1 + max_chunks + ci];
+    const int seg0 = offsets[e];
+    const int tile = (seg0 >> 4) + e + ((first - seg0) >> 4);
+    uint8_t *tp = op + (int64_t)tile * bpr * QME_TILE_COL_BYTES;
+    const int64_t row = row_map[first + c];
+    if (SW && col == 0 && lane == 0) scale_out[first + c] = scale_in[row];
+    float v[1][4];
+    if constexpr (SW) cq_load_swiglu4(x, up, (row * bpr + col) * 256 + lane * 4, (row * bpr + col) * 256 + lane * 4, v[0]);
+    else cq_load4<CQ_F32>(x, (row * bpr + col) * 256 + lane * 4, v[0]);
+    const uint32_t wmax[1] = {qs_span_umax(v[0])};
+    float iscale[1], d[1];
+    qs_span_scales<1>(wmax, lane, iscale, d);
+    int q[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) q[i] = qs_round_i8(iscale[0] * v[0][i]);
+    const uint32_t packed = qs_pack4(q);
+    const int slot = qme_slot(c);
+    *(uint32_t *)(tp + col * QB_OP_COL_BYTES + qb_operand_dword(lane, slot, 16)) = packed;
+    const int s32 = oct_sum(sdot4(packed, 0x01010101u, 0));
+    uint8_t *rec = tp + bpr * QB_OP_COL_BYTES + (col * 16 + slot) * QB_REC_BYTES;
+    if ((lane & 7) == 0) { rec[lane >> 3] = (uint8_t)(s32 & 127); rec[8 + (lane >> 3)] = (uint8_t)(s32 >> 7); }
+    if (lane == 0) *(float *)(rec + 16) = d[0];
+}
+
+#ifdef CL_STAMPS
+__device__ uint32_t *qme_stamps;
+#endif
+struct QmeArgs {
+    const uint8_t *w[2];          // [experts][n][bpr] super-blocks each
+    float *out[2];                // [pairs][n]
+    const uint8_t *op;
+    const int *offsets;           // [experts + 1]: expert e's pairs are offsets[e] .. offsets[e + 1] of the sorted list
+    const int *pair_out;          // output row of a sorted pair
+    const float *pair_scale;      // and the factor on its results
+    int n, bpr, parts;
+};
+constexpr int QME_NS = 2;         // sets of 16 pairs per pass over the weights
+constexpr int QME_DEPTH = 4;      // tiles of the ring where LDS holds them
+
+template <int CW, int CPW, int DEPTH>
+__global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
+    constexpr int NRB = QB_NW / CW;                                        // row blocks of a tile
+    constexpr int NIW = (16 * NRB * CW * CPW * QB_BB + 8 * 1024 - 1) / (8 * 1024);      // copy instructions per wave and tile
+    static_assert((DEPTH - 1) * NIW <= 63 && DEPTH >= 2, "counted waits");
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int e = blockIdx.y;
+    const int seg0 = a.offsets[e], seg1 = a.offsets[e + 1];
+    if (seg0 >= seg1) return;
+    QB_STAMP(0);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, kg = lane >> 4;
+    const int rb = wv / CW, col0 = (wv % CW) * CPW;
+    const int n = a.n, bpr = a.bpr;
+    const int ncols = max(0, min(CPW, bpr - col0));
+    const int RS = bpr * QB_BB;
+    const int block_bytes = 16 * NRB * RS;
+    const int nkb = (block_bytes + 1023) >> 10;
+    const int TILE = qb_tile_bytes(block_bytes);
+    float *red = (float *)(lds + DEPTH * TILE);                            // [2][sets][8 waves][64 lanes][4]
+    constexpr int REC_KB = (CW * CPW * 16 * QB_REC_BYTES + 1023) / 1024;   // KBs of the records of one set (at most CW * CPW columns)
+    uint8_t *recs = lds + DEPTH * TILE + 2 * QME_NS * QB_RED_BYTES;        // [sets][REC_KB KB], one spare KB
+    const uint8_t *w = a.w[blockIdx.z] + (int64_t)e * n * RS;
+    float *out = a.out[blockIdx.z];
+    const int ntiles = (n + 16 * NRB - 1) / (16 * NRB);
+    const int t0 = (int)((int64_t)blockIdx.x * ntiles / a.parts), t1 = (int)((int64_t)(blockIdx.x + 1) * ntiles / a.parts);
+    const int my = t1 - t0;
+    const int64_t w_bytes = (int64_t)n * RS;
+    int seq = 0;                                                           // tiles asked for so far, over all passes: the ring slot
+    auto issue = [&](int i) {                                              // tile t0 + i of this pass (nothing beyond the range)
+        const bool live = i < my;
+        const int64_t off = live ? (int64_t)(t0 + i) * block_bytes : 0;
+        const int64_t left = w_bytes - off;
+        const int bytes = live ? (int)(left < block_bytes ? left : block_bytes) : 0;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(w + off), 0, bytes, 0x00020000);
+        uint8_t *tile = lds + (seq % DEPTH) * TILE;
+        seq++;
+#pragma unroll
+        for (int t = 0; t < NIW; t++) {
+            const int kb = min(t * QB_NW + wv, nkb);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(tile + kb * QB_KB), 16, lane * 16, kb * 1024, 0, 0);
+        }
+    };
+    const int nsets = (seg1 - seg0 + 15) >> 4;
+    for (int sg = 0; sg < nsets; sg += QME_NS) {
+        // (a second pass starts behind the barrier that ended the first: every tile of the ring is free)
+        const int sets_here = min(QME_NS, nsets - sg);
+        // The records of the pass (block sums and scales of every pair and column) go to LDS by copy instructions ahead of the
+        // first tile, whose wait covers them: loaded by every lane from memory they were 2/3 of the wave's operand requests,
+        // sixteen lanes asking for the same 20 bytes, and the waves took 4 us to get their requests out.
+#pragma unroll
+        for (int t = 0; t < (QME_NS * REC_KB + QB_NW - 1) / QB_NW; t++) {
+            const int j = t * QB_NW + wv, st = j / REC_KB, piece = j - st * REC_KB;
+            const bool live = st < sets_here;
+            const int tile = (seg0 >> 4) + e + sg + (live ? st : 0);
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(a.op + (int64_t)tile * bpr * QME_TILE_COL_BYTES + bpr * QB_OP_COL_BYTES), 0, live ? bpr * 16 * QB_REC_BYTES : 0, 0x00020000);
+            // (a copy for a set that does not exist carries no bytes and writes zeros: into a spare KB behind the records)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(recs + (live ? st * REC_KB + piece : QME_NS * REC_KB) * 1024), 16, lane * 16,
+                                                     piece * 1024, 0, 0);
+        }
+        issue(0);
+        asm volatile("" ::: "memory");
+        int rounds[QME_NS];                                                // results per lane a set needs: ceil(pairs / 4)
+#pragma unroll
+        for (int st = 0; st < QME_NS; st++) rounds[st] = (min(16, max(0, seg1 - seg0 - (sg + st) * 16)) + 3) >> 2;
+        long A[QME_NS][CPW][8];
+        u32x4 aux[QME_NS][CPW][4];
+        float d8[QME_NS][CPW][4];
+#pragma unroll
+        for (int st = 0; st < QME_NS; st++) {
+            const int cnt = min(16, seg1 - seg0 - (sg + st) * 16);         // pairs of this set (<= 0: the set does not exist)
+            const int tile = (seg0 >> 4) + e + min(sg + st, nsets - 1);
+            const uint8_t *tp = a.op + (int64_t)tile * bpr * QME_TILE_COL_BYTES;
+#pragma unroll
+            for (int ci = 0; ci < CPW; ci++) {
+                const int col = min(col0 + ci, bpr - 1);
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const i64x2 v = qme_slot(c) < cnt ? *(const i64x2 *)(tp + col * QB_OP_COL_BYTES + g * 1024 + lane * 16) : i64x2{0, 0};
+                    A[st][ci][2 * g] = v.x; A[st][ci][2 * g + 1] = v.y;
+                }
+            }
+        }
+        // the pair this thread stores at the end of every tile: set tid / 256, result r of lane group l2 / 16 = pair 4 r + l2 / 16
+        const int oset = tid >> 8, ol2 = tid & 63, orr = (tid >> 6) & 3;
+        const int opos = seg0 + (sg + oset) * 16 + 4 * orr + (ol2 >> 4);
+        const bool ovalid = opos < seg1;
+        const int64_t orow = ovalid ? a.pair_out[opos] : 0;
+        const float oscale = ovalid ? a.pair_scale[opos] : 0.0f;
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int i = 1; i < DEPTH - 1; i++) issue(i);
+        // One barrier per tile: behind it tile i has landed for every wave, and every wave has left its partial results of tile
+        // i - 1 in red[(i - 1) % 2], which 8 threads per result add up and store while the waves go on with tile i.
+        QB_STAMP(1);
+        for (int i = 0; i <= my; i++) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * NIW) : "memory");
+            if (i < 4) QB_STAMP(2 + 3 * i);
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            if (i < 4) QB_STAMP(3 + 3 * i);
+            if (i == 0) {
+                // the lane's records, now in LDS: slot 4 kg + r holds pair 4 r + kg
+#pragma unroll
+                for (int st = 0; st < QME_NS; st++) {
+                    const int cnt = min(16, seg1 - seg0 - (sg + st) * 16);
+#pragma unroll
+                    for (int ci = 0; ci < CPW; ci++) {
+                        const int col = min(col0 + ci, bpr - 1);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const uint8_t *rec = recs + min(st, sets_here - 1) * (REC_KB * 1024) + (col * 16 + 4 * kg + r) * QB_REC_BYTES;
+                            const bool on = 4 * r + kg < cnt;
+                            const u32x4 t4 = *(const u32x4 *)rec;
+                            const float td = *(const float *)(rec + 16);
+                            aux[st][ci][r] = on ? t4 : u32x4{0, 0, 0, 0};
+                            d8[st][ci][r] = on ? td : 0.0f;
+                        }
+                    }
+                }
+            }
+            if (i > 0 && ovalid) {
+                const float *rd = red + ((i - 1) & 1) * (QME_NS * QB_NW * 64 * 4);
+#pragma unroll
+                for (int g = 0; g < NRB; g++) {
+                    float v = 0.0f;
+#pragma unroll
+                    for (int w2 = 0; w2 < CW; w2++) v += rd[((oset * QB_NW + g * CW + w2) * 64 + ol2) * 4 + orr];
+                    const int row = ((t0 + i - 1) * NRB + g) * 16 + (ol2 & 15);
+                    if (row < n) out[orow * n + row] = v * oscale;
+                }
+            }
+            if (i == my) break;
+            const uint8_t *tile = lds + ((seq - (DEPTH - 1)) % DEPTH) * TILE;       // tile i of this pass
+            issue(i + DEPTH - 1);
+            float acc[QME_NS][4];
+#pragma unroll
+            for (int st = 0; st < QME_NS; st++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[st][r] = 0.0f;
+#pragma unroll
+            for (int ci = 0; ci < CPW; ci++) {
+                if (ci < ncols) {
+                    const int o = (rb * 16 + c) * RS + (col0 + ci) * QB_BB;
+                    auto at = [&](int off) { return tile + off + (off >> 10) * 16; };
+                    const u32x4 hdr = *(const u32x4 *)at(o);
+                    long lo[4], hi[4];
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const long qa = *(const long *)at(o + 16 + 32 * g + 8 * kg);
+                        lo[g] = qa & 0x0f0f0f0f0f0f0f0fl; hi[g] = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                    }
+                    const QsScales s = qs_scales_k4(hdr.y, hdr.z, hdr.w);
+                    int sc[8];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        sc[j] = (int)((s.scA >> (8 * j)) & 0xff);
+                        sc[4 + j] = (int)((s.scB >> (8 * j)) & 0xff);
+                    }
+                    const float dw = h2f(hdr.x), dm = h2f(hdr.x >> 16);
+#pragma unroll
+                    for (int st = 0; st < QME_NS; st++) {
+                        if (st >= sets_here) continue;
+                        i32x4 cl[4], ch[4];
+                        const i32x4 z = {0, 0, 0, 0};
+#pragma unroll
+                        for (int g = 0; g < 4; g++) {
+                            cl[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[st][ci][2 * g], lo[g], z, 0, 0, 0);
+                            ch[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[st][ci][2 * g + 1], hi[g], z, 0, 0, 0);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            if (r < rounds[st]) {
+                                int S = 0;
+#pragma unroll
+                                for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
+                                const int M = qs_dot_sums(s.mA, s.mB, aux[st][ci][r]);
+                                acc[st][r] += d8[st][ci][r] * (dw * (float)S - dm * (float)M);
+                            }
+                        }
+                    }
+                }
+            }
+            if (i < 4) QB_STAMP(4 + 3 * i);
+            float *rw = red + (i & 1) * (QME_NS * QB_NW * 64 * 4);
+#pragma unroll
+            for (int st = 0; st < QME_NS; st++)
+                *(f32x4 *)(rw + ((st * QB_NW + wv) * 64 + lane) * 4) = f32x4{acc[st][0], acc[st][1], acc[st][2], acc[st][3]};
+        }
+        // the copies beyond the range carried no bytes, but they count: nothing may be outstanding when the next pass counts again
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+#ifdef CL_STAMPS
+    QB_STAMP(15);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (tid < 128 && qme_stamps) qme_stamps[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + tid / 16) * 16 + tid % 16] = qb_stamp_lds[tid / 16][tid % 16];
+#endif
+}
+
+template <int CW, int CPW, int DEPTH>
+int launch_qme_d(const QmeArgs &a, int64_t num_experts, int tensors, size_t lds_bytes, hipStream_t s) {
+    auto kern = qme_q4k_kernel<CW, CPW, DEPTH>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)a.parts, (unsigned)num_experts, (unsigned)tensors), dim3(QB_NW * 64), lds_bytes, s, a);
+    return (int)hipGetLastError();
+}
+template <int CW, int CPW>
+int launch_qme(const QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s) {
+    const int tile = qb_tile_bytes(16 * (QB_NW / CW) * a.bpr * QB_BB);
+    const int red = 2 * QME_NS * QB_RED_BYTES + (QME_NS * ((CW * CPW * 16 * QB_REC_BYTES + 1023) / 1024) + 1) * 1024;      // partial results, records
+    const int fit = (QB_LDS_BYTES - red - 1024) / tile;
+    if (fit >= QME_DEPTH) return launch_qme_d<CW, CPW, QME_DEPTH>(a, num_experts, tensors, (size_t)QME_DEPTH * tile + red, s);
+    if (fit >= 3) return launch_qme_d<CW, CPW, 3>(a, num_experts, tensors, (size_t)3 * tile + red, s);
+    if (fit == 2) return launch_qme_d<CW, CPW, 2>(a, num_experts, tensors, (size_t)2 * tile + red, s);
+    return CQ_ERR_RANGE;
+}
+
 }  // namespace
 
 // Does the batched matrix-core matvec take this call?  Q4_K, 3 .. 16 rows, rows of up to 64 super-blocks (k <= 16384: up to 24
@@ -687,7 +986,61 @@ int cq_matvec_batch_swiglu_launch(int w_dtype, const void *w, const float *gate,
     return qb_launch(w_dtype, w, gate, up, gate_stride, up_stride, -1, workspace, dst, dst_dtype, k, n, rows, stride_dst, s);
 }
 
+// ---- MoE: experts as batched matvecs (see qme_q4k_kernel) ----
+// Q4_K experts of rows up to 16 super-blocks (two columns per wave: three do not fit the registers next to two operand sets),
+// 16-byte aligned, and on average at most 32 pairs per expert: beyond that a pass over the weights per 32 pairs loses to the
+// tiles that reuse a weight 32 or 128 times.
+bool cq_moe_stream_shape(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n) {
+    return w_dtype == CQ_Q4K && k % 256 == 0 && k / 256 <= 2 * QB_NW && n >= 1 && n <= 0x7ffffff0 / 16 && num_experts >= 1 && num_experts <= 65535 &&
+           n_pairs <= 32 * num_experts && n * (k / 256) * QB_BB < 0x7fffffffLL;
+}
+bool cq_moe_stream_takes(int w_dtype, const void *w, const void *w_b, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n) {
+    return cq_moe_stream_shape(w_dtype, num_experts, n_pairs, k, n) && ((uintptr_t)w & 15) == 0 && ((uintptr_t)w_b & 15) == 0;
+}
+int64_t cq_moe_stream_operand_bytes(int64_t num_experts, int64_t n_pairs, int64_t k) {
+    return qme_operand_tiles(n_pairs, num_experts) * (k / 256) * QME_TILE_COL_BYTES;
+}
+// chunks: the grouping pass's table for chunks of 16 pairs (n | expert[max_chunks] | first[] | count[]).  up != nullptr: the rows are
+// silu(x[row]) * up[row] and scale_out[i] = scale_in[row_map[i]].
+int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *row_map, const float *scale_in, float *scale_out, const int *chunks,
+                                  int64_t max_chunks, const int *offsets, void *op, int64_t k, hipStream_t s) {
+    if (up)
+        hipLaunchKernelGGL(qme_quantize_kernel<true>, dim3((unsigned)max_chunks, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
+                           (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256));
+    else
+        hipLaunchKernelGGL(qme_quantize_kernel<false>, dim3((unsigned)max_chunks, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
+                           (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256));
+    return (int)hipGetLastError();
+}
+// out_a[pair_out[p]][:] = (W_a[expert of p] . x^[p]) * pair_scale[p] for every sorted pair p; the same for (w_b, out_b) when given
+int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
+                         const float *pair_scale, int64_t num_experts, int64_t k, int64_t n, hipStream_t s) {
+    const int bpr = (int)(k / 256), tensors = w_b ? 2 : 1;
+    QmeArgs a;
+    a.w[0] = (const uint8_t *)w_a; a.w[1] = (const uint8_t *)w_b; a.out[0] = out_a; a.out[1] = out_b;
+    a.op = (const uint8_t *)op; a.offsets = offsets; a.pair_out = pair_out; a.pair_scale = pair_scale; a.n = (int)n; a.bpr = bpr;
+    // waves that share a row block: the fewest (a power of two) with at most two columns each — large tiles: a tile costs about
+    // a microsecond of barriers and latencies whatever it holds
+    const int cw = bpr > 8 ? 8 : bpr > 4 ? 4 : bpr > 2 ? 2 : 1;
+    const int64_t ntiles = (n + 16 * (QB_NW / cw) - 1) / (16 * (QB_NW / cw));
+    // parts: experts x tensors x parts fills the CUs once or twice (all experts hit: the same bytes everywhere)
+    int64_t parts = (256 + num_experts * tensors - 1) / (num_experts * tensors);
+    if (parts > ntiles) parts = ntiles;
+    a.parts = (int)parts;
+    switch (cw) {
+        case 8: return launch_qme<8, 2>(a, num_experts, tensors, s);
+        case 4: return launch_qme<4, 2>(a, num_experts, tensors, s);
+        case 2: return launch_qme<2, 2>(a, num_experts, tensors, s);
+        default: return bpr == 2 ? launch_qme<1, 2>(a, num_experts, tensors, s) : launch_qme<1, 1>(a, num_experts, tensors, s);
+    }
+}
+
 #ifdef CL_STAMPS
+extern "C" int qme_debug_launch(const void *w, float *out, const void *op, const int *offsets, const int *pout, const float *pscale, int64_t experts,
+                                int64_t k, int64_t n, uint32_t *stamps, void *stream) {
+    hipMemcpyToSymbol(HIP_SYMBOL(qme_stamps), &stamps, sizeof(stamps));
+    return cq_moe_stream_launch(w, nullptr, out, nullptr, op, offsets, pout, pscale, experts, k, n, (hipStream_t)stream);
+}
 extern "C" int qb_debug_launch(const void *w, const void *x, void *workspace, void *dst, int64_t k, int64_t n, int64_t rows, void *stream) {
     return cq_matvec_batch_launch(CQ_Q4K, w, x, CQ_F32, workspace, dst, CQ_F32, k, n, rows, n, (hipStream_t)stream);
 }

@@ -13,7 +13,10 @@
 // reference sorts with an unstable sort, candle-core/src/sort.rs:282-297).  Step 3 streams every
 // hit expert's rows once: workgroup (row tile, expert) keeps the decoded weight registers and loops
 // over that expert's pairs — unlike the reference kernels, which re-read the expert's weights for
-// every pair routed to it.
+// every pair routed to it.  (Few pairs skip steps 1 and 2: a fused matvec per pair.  Hundreds of pairs take step 3 on the matrix
+// cores: Q4_K experts with up to 32 pairs each as batched matvecs over their pairs, cq_matvec_batch.hip, the rest as tiles of
+// expert-sorted rows through the prefill kernel of the format.)
+#include <algorithm>
 #include "cq_device.h"
 #include "cq_fmt.h"
 #include "cq_launch.h"
@@ -32,6 +35,8 @@ inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pa
     w.rows_alloc = n_pairs + CQ_MOE_CHUNK;
     w.max_chunks = n_pairs / CQ_MOE_CHUNK + (num_experts < n_pairs ? num_experts : n_pairs) + 1;
     w.offsets_off = cq_act_layout(w_dtype, k, w.rows_alloc > x_rows ? w.rows_alloc : x_rows).total;
+    // (experts run as batched matvecs keep their pairs' rows as operand tiles instead)
+    if (w_dtype == CQ_Q4K && k % 256 == 0) w.offsets_off = std::max<int64_t>(w.offsets_off, cq_align256(cq_moe_stream_operand_bytes(num_experts, n_pairs, k)));
     w.cursor_off = w.offsets_off + cq_align256((num_experts + 1) * 4);
     w.pin_off = w.cursor_off + cq_align256(num_experts * 4);
     w.pout_off = w.pin_off + cq_align256(n_pairs * 4);
@@ -209,6 +214,20 @@ int cq_moe_down_after_pair_launch(int w_dtype, const void *w_down, const float *
     if (cq_moe_direct(w_dtype, num_experts, n_pairs, k_pair) || !moe_takes_mfma(w_dtype, nullptr, nullptr, n_pairs, k_pair)) return CQ_ERR_RANGE;
     if (!moe_takes_mfma(w_dtype, w_down, nullptr, n_pairs, k)) return CQ_ERR_RANGE;
     const MoeWorkspace ws = moe_workspace(w_dtype, num_experts, n_pairs, n_pairs / topk, k_pair);
+    // the pair call ran its experts as batched matvecs (chunks of 16 pairs): this one must be able to as well
+    // (n of the pair call = this call's k; its expert tensors were 16-byte aligned or it returned CQ_ERR_ALIGN)
+    if (cq_moe_stream_shape(w_dtype, num_experts, n_pairs, k_pair, k)) {
+        if (!cq_moe_stream_takes(w_dtype, w_down, nullptr, num_experts, n_pairs, k, n)) return CQ_ERR_RANGE;
+        if (cq_align256(cq_moe_stream_operand_bytes(num_experts, n_pairs, k)) > ws.offsets_off) return CQ_ERR_RANGE;
+        uint8_t *b = (uint8_t *)workspace;
+        const int *offsets = (const int *)(b + ws.offsets_off);
+        const int *pout = (const int *)(b + ws.pout_off);
+        float *pscale = (float *)(b + ws.pscale_off);
+        const int *chunks = (const int *)(b + ws.chunk_off);
+        int rc = cq_moe_stream_quantize_launch(gate, up, pout, topk_weights, pscale, chunks, ws.max_chunks, offsets, b + ws.act_off, k, s);
+        if (rc) return rc;
+        return cq_moe_stream_launch(w_down, nullptr, out, nullptr, b + ws.act_off, offsets, pout, pscale, num_experts, k, n, s);
+    }
     // the rows of this call are quantized into the front of the workspace: they must end before that call's tables begin
     if (cq_act_layout(w_dtype, k, ws.rows_alloc).total > ws.offsets_off) return CQ_ERR_RANGE;
     uint8_t *b = (uint8_t *)workspace;
@@ -226,6 +245,10 @@ int cq_moe_down_after_pair_launch(int w_dtype, const void *w_down, const float *
 int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if (a.n_pairs > 0x7fffffffLL || a.x_rows > 0x7fffffffLL) return CQ_ERR_RANGE;
     const bool mfma = moe_takes_mfma(a.w_dtype, a.w, a.w_b, a.n_pairs, a.k);
+    const bool stream_shape = mfma && !cq_moe_direct(a.w_dtype, a.num_experts, a.n_pairs, a.k) && cq_moe_stream_shape(a.w_dtype, a.num_experts, a.n_pairs, a.k, a.n);
+    const bool stream = stream_shape && cq_moe_stream_takes(a.w_dtype, a.w, a.w_b, a.num_experts, a.n_pairs, a.k, a.n);
+    // (a later cq_moe_down_after_pair_launch tells from the shape alone how this call chunked its pairs)
+    if (a.w_b && stream_shape && !stream) return CQ_ERR_ALIGN;
     if (a.w_b && !mfma) {
         // only the MFMA path shares its grouping pass and quantized activations between two weight tensors
         MoeArgs one = a;
@@ -257,11 +280,16 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     const int tile_rows = moe_tile_rows(a.n_pairs, a.num_experts);
     if (a.num_experts <= GROUP_LDS_EXPERTS)
         hipLaunchKernelGGL(moe_group_kernel<true>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
-                           (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);
+                           (int)ws.max_chunks, stream ? CQ_MOE_STREAM_CHUNK : mfma ? tile_rows : CQ_MOE_CHUNK);
     else
         hipLaunchKernelGGL(moe_group_kernel<false>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
-                           (int)ws.max_chunks, mfma ? tile_rows : CQ_MOE_CHUNK);
+                           (int)ws.max_chunks, stream ? CQ_MOE_STREAM_CHUNK : mfma ? tile_rows : CQ_MOE_CHUNK);
     if ((rc = (int)hipGetLastError())) return rc;
+    if (stream) {
+        // every expert a batched matvec over its own pairs: the weights of an expert are streamed once per 32 pairs
+        if ((rc = cq_moe_stream_quantize_launch(a.x, nullptr, pin, nullptr, nullptr, chunks, ws.max_chunks, offsets, b + ws.act_off, a.k, s))) return rc;
+        return cq_moe_stream_launch(a.w, a.w_b, a.out, a.out_b, b + ws.act_off, offsets, pout, pscale, a.num_experts, a.k, a.n, s);
+    }
     if (mfma) {
         if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;
         MoeChunks mc{chunks, chunks + 1, chunks + 1 + ws.max_chunks, chunks + 1 + 2 * ws.max_chunks, pout, pscale, (int)ws.max_chunks};

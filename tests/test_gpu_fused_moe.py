@@ -233,6 +233,10 @@ def test_down_after_pair_refuses_what_it_cannot_reuse():
     assert lib.cq_moe_gemm_gguf_down_after_pair(12, p, p, p, p, p, 128, 8, 2048, 2048, 4096, 256, p, big, None) == -6
     assert lib.cq_moe_gemm_gguf_down_after_pair(12, p, p, p, p, p, 128, 8, 2048, 2048, 768, 2048, p, 1024, None) == -5   # CQ_ERR_WORKSPACE
     assert lib.cq_moe_gemm_gguf_down_after_pair(12, None, p, p, p, p, 128, 8, 2048, 2048, 768, 2048, p, big, None) == -4
+    # Q4_K experts that would run as batched matvecs must be 16-byte aligned in the gate / up call (the down call tells from the
+    # shape alone how that call grouped its pairs): CQ_ERR_ALIGN, nothing enqueued
+    assert lib.cq_moe_gemm_gguf_pair(12, p, p + 8, p, p, p, p, p, 128, 8, 2048, 768, 2048, 1, p, big, None) == -3
+    assert lib.cq_moe_gemm_gguf_pair(12, p, p, p + 8, p, p, p, p, 128, 8, 2048, 768, 2048, 1, p, big, None) == -3
 
 
 def test_fused_moe_argument_errors():

@@ -87,6 +87,43 @@ def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     assert err2 <= TOL and err2 <= TIGHT, err2
 
 
+@pytest.mark.parametrize("k,n", [(256, 64), (512, 40), (768, 203), (1024, 130), (1792, 50), (2048, 96), (2304, 33), (4096, 72)])
+@pytest.mark.parametrize("with_weights", [False, True])
+def test_moe_gemm_gguf_experts_as_batched_matvecs(k, n, with_weights):
+    """Q4_K experts hit by at most 32 pairs on average run as batched matvecs over their own pairs (sets of 16, two sets per pass
+    over the weights).  Expert loads on every edge: none, one pair, 15 / 16 / 17, 31 / 32 / 33 (a second pass), 47 .. 49, 65 (a
+    third pass); rows of 1 .. 16 super-blocks (one to eight waves per row block, columns without a wave's second column), ragged
+    n, several workgroups per expert."""
+    import candle_amd as ca
+    counts = [0, 1, 15, 16, 17, 31, 32, 33, 47, 48, 49, 65, 0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13]
+    E, topk = len(counts), 2
+    n_pairs = sum(counts)
+    assert n_pairs % topk == 0 and 257 <= n_pairs <= 32 * E
+    tokens = n_pairs // topk
+    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=91)
+    rng = np.random.Generator(np.random.PCG64(92))
+    expert_ids = np.repeat(np.arange(E, dtype=np.int32), counts)
+    sorted_token_ids = rng.permutation(n_pairs).astype(np.int32)
+    sti, eid = torch.from_numpy(sorted_token_ids).cuda(), torch.from_numpy(expert_ids).cuda()
+    if with_weights:
+        x = normal(93, (n_pairs, k), 1.0)
+        tw = rng.uniform(0.1, 1.0, n_pairs).astype(np.float32)
+        got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, torch.from_numpy(tw).cuda(), sti, eid, topk, True)
+    else:
+        x = normal(94, (tokens, k), 1.0)
+        tw = None
+        got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, None, sti, eid, topk, True)
+    torch.cuda.synchronize()
+    want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, tw, topk)
+    got = got.cpu().numpy()
+    assert got.shape == (n_pairs, n)
+    err = rel_l2(got, want)
+    assert err <= TOL and err <= TIGHT, err
+    # pair by pair as well: a pair in the wrong slot of its set would hide in the norm of hundreds of rows
+    for p in range(n_pairs):
+        assert rel_l2(got[p], want[p]) <= 1e-5, (p, int(expert_ids[np.where(sorted_token_ids == p)[0][0]]))
+
+
 @pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q5K, oracle.Q6K, oracle.Q2K, oracle.Q3K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("E,n", [(64, 160), (8, 160)])      # 1200 pairs: about 19 rows per expert (32-row tiles of the MFMA
                                                             # kernel, 128 weight rows wide) or 150 (128-row tiles); n is ragged
