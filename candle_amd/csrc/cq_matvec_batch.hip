@@ -686,6 +686,7 @@ struct QmeArgs {
     int n, bpr, parts;
 };
 constexpr int QME_NS = 2;         // sets of 16 pairs per pass over the weights
+constexpr int QME_MAX_AVG_PAIRS = 64;   // pairs per expert on average up to which a call takes this form
 constexpr int QME_DEPTH = 4;      // tiles of the ring where LDS holds them
 
 template <int CW, int CPW, int DEPTH>
@@ -756,7 +757,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
 #pragma unroll
         for (int st = 0; st < QME_NS; st++) rounds[st] = (min(16, max(0, seg1 - seg0 - (sg + st) * 16)) + 3) >> 2;
         long A[QME_NS][CPW][8];
-        u32x4 aux[QME_NS][CPW][4];
+        long Abl[QME_NS][CPW], Abh[QME_NS][CPW];          // the block sums of slot c (sum j = 128 * bh_j + bl_j) as matrix operands: lane group 0 only
         float d8[QME_NS][CPW][4];
 #pragma unroll
         for (int st = 0; st < QME_NS; st++) {
@@ -801,12 +802,13 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
                             const uint8_t *rec = recs + min(st, sets_here - 1) * (REC_KB * 1024) + (col * 16 + 4 * kg + r) * QB_REC_BYTES;
-                            const bool on = 4 * r + kg < cnt;
-                            const u32x4 t4 = *(const u32x4 *)rec;
                             const float td = *(const float *)(rec + 16);
-                            aux[st][ci][r] = on ? t4 : u32x4{0, 0, 0, 0};
-                            d8[st][ci][r] = on ? td : 0.0f;
+                            d8[st][ci][r] = 4 * r + kg < cnt ? td : 0.0f;
                         }
+                        const i64x2 sums = *(const i64x2 *)(recs + min(st, sets_here - 1) * (REC_KB * 1024) + (col * 16 + c) * QB_REC_BYTES);
+                        const bool mine = kg == 0 && qme_slot(c) < cnt;
+                        Abl[st][ci] = mine ? sums.x : 0;
+                        Abh[st][ci] = mine ? sums.y : 0;
                     }
                 }
             }
@@ -849,6 +851,10 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
                         sc[4 + j] = (int)((s.scB >> (8 * j)) & 0xff);
                     }
                     const float dw = h2f(hdr.x), dm = h2f(hdr.x >> 16);
+                    // The minimum term sum_j m_j * (sub-block sum j of the pair) is a product of its own — the row's eight 6-bit
+                    // minima against the pair's eight sums, split 128 * bh + bl into bytes — and goes to the matrix cores as
+                    // well: two instructions per set and column instead of six vector instructions per result.
+                    const long mins = kg == 0 ? (long)(((uint64_t)s.mB << 32) | s.mA) : 0;
 #pragma unroll
                     for (int st = 0; st < QME_NS; st++) {
                         if (st >= sets_here) continue;
@@ -859,13 +865,19 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
                             cl[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[st][ci][2 * g], lo[g], z, 0, 0, 0);
                             ch[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[st][ci][2 * g + 1], hi[g], z, 0, 0, 0);
                         }
+                        const i32x4 ml = __builtin_amdgcn_mfma_i32_16x16x32_i8(Abl[st][ci], mins, z, 0, 0, 0);
+                        const i32x4 mh = __builtin_amdgcn_mfma_i32_16x16x32_i8(Abh[st][ci], mins, z, 0, 0, 0);
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
                             if (r < rounds[st]) {
-                                int S = 0;
+                                int S = __mul24(sc[0], cl[0][r]);
+                                S = __mul24(sc[1], ch[0][r]) + S;
 #pragma unroll
-                                for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
-                                const int M = qs_dot_sums(s.mA, s.mB, aux[st][ci][r]);
+                                for (int g = 1; g < 4; g++) {
+                                    S = __mul24(sc[2 * g], cl[g][r]) + S;
+                                    S = __mul24(sc[2 * g + 1], ch[g][r]) + S;
+                                }
+                                const int M = (mh[r] << 7) + ml[r];
                                 acc[st][r] += d8[st][ci][r] * (dw * (float)S - dm * (float)M);
                             }
                         }
@@ -988,11 +1000,11 @@ int cq_matvec_batch_swiglu_launch(int w_dtype, const void *w, const float *gate,
 
 // ---- MoE: experts as batched matvecs (see qme_q4k_kernel) ----
 // Q4_K experts of rows up to 16 super-blocks (two columns per wave: three do not fit the registers next to two operand sets),
-// 16-byte aligned, and on average at most 32 pairs per expert: beyond that a pass over the weights per 32 pairs loses to the
+// 16-byte aligned, and on average at most 64 pairs per expert: beyond that a pass over the weights per 32 pairs loses to the
 // tiles that reuse a weight 32 or 128 times.
 bool cq_moe_stream_shape(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n) {
     return w_dtype == CQ_Q4K && k % 256 == 0 && k / 256 <= 2 * QB_NW && n >= 1 && n <= 0x7ffffff0 / 16 && num_experts >= 1 && num_experts <= 65535 &&
-           n_pairs <= 32 * num_experts && n * (k / 256) * QB_BB < 0x7fffffffLL;
+           n_pairs <= QME_MAX_AVG_PAIRS * num_experts && n * (k / 256) * QB_BB < 0x7fffffffLL;
 }
 bool cq_moe_stream_takes(int w_dtype, const void *w, const void *w_b, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n) {
     return cq_moe_stream_shape(w_dtype, num_experts, n_pairs, k, n) && ((uintptr_t)w & 15) == 0 && ((uintptr_t)w_b & 15) == 0;

@@ -14,7 +14,7 @@
 // hit expert's rows once: workgroup (row tile, expert) keeps the decoded weight registers and loops
 // over that expert's pairs — unlike the reference kernels, which re-read the expert's weights for
 // every pair routed to it.  (Few pairs skip steps 1 and 2: a fused matvec per pair.  Hundreds of pairs take step 3 on the matrix
-// cores: Q4_K experts with up to 32 pairs each as batched matvecs over their pairs, cq_matvec_batch.hip, the rest as tiles of
+// cores: Q4_K experts with up to 64 pairs each as batched matvecs over their pairs, cq_matvec_batch.hip, the rest as tiles of
 // expert-sorted rows through the prefill kernel of the format.)
 #include <algorithm>
 #include "cq_device.h"

@@ -200,7 +200,7 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
 /* Two moe_gemm_gguf calls without topk_weights over the same x and the same pairs — the gate and up matmuls of
  * FusedMoeGGUF::forward (candle-transformers/src/fused_moe.rs:263-276) — as one call: out_a = x W_a^T, out_b = x W_b^T per
  * pair, results identical to two cq_moe_gemm_gguf calls.  With more than 256 pairs on K-quant experts the pairs are
- * grouped by expert and the activations quantized once for both (Q4_K experts that see at most 32 pairs each on average, rows
+ * grouped by expert and the activations quantized once for both (Q4_K experts that see at most 64 pairs each on average, rows
  * up to 4096 elements: both tensors in one launch, every expert a batched matvec over its own pairs); otherwise it is the two
  * calls.  w_a / w_b [num_experts, n, k] of one format; workspace as cq_moe_gemm_workspace_bytes(..., has_topk_weights = 0).
  * CQ_ERR_ALIGN when such Q4_K experts are not 16-byte aligned (a later cq_moe_gemm_gguf_down_after_pair tells from the shape

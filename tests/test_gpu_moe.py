@@ -90,7 +90,7 @@ def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
 @pytest.mark.parametrize("k,n", [(256, 64), (512, 40), (768, 203), (1024, 130), (1792, 50), (2048, 96), (2304, 33), (4096, 72)])
 @pytest.mark.parametrize("with_weights", [False, True])
 def test_moe_gemm_gguf_experts_as_batched_matvecs(k, n, with_weights):
-    """Q4_K experts hit by at most 32 pairs on average run as batched matvecs over their own pairs (sets of 16, two sets per pass
+    """Q4_K experts hit by at most 64 pairs on average run as batched matvecs over their own pairs (sets of 16, two sets per pass
     over the weights).  Expert loads on every edge: none, one pair, 15 / 16 / 17, 31 / 32 / 33 (a second pass), 47 .. 49, 65 (a
     third pass); rows of 1 .. 16 super-blocks (one to eight waves per row block, columns without a wave's second column), ragged
     n, several workgroups per expert."""
@@ -98,7 +98,7 @@ def test_moe_gemm_gguf_experts_as_batched_matvecs(k, n, with_weights):
     counts = [0, 1, 15, 16, 17, 31, 32, 33, 47, 48, 49, 65, 0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13]
     E, topk = len(counts), 2
     n_pairs = sum(counts)
-    assert n_pairs % topk == 0 and 257 <= n_pairs <= 32 * E
+    assert n_pairs % topk == 0 and 257 <= n_pairs <= 64 * E
     tokens = n_pairs // topk
     blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=91)
     rng = np.random.Generator(np.random.PCG64(92))
@@ -138,6 +138,23 @@ def test_moe_gemm_gguf_mfma_tile_sizes(dtype, E, n):
     got = ca.moe_gemm_gguf(torch.from_numpy(x2).cuda(), qt, torch.from_numpy(twf).cuda(), sti, eid, topk, True)
     torch.cuda.synchronize()
     want = oracle.moe_gemm_gguf(dtype, x2, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
+    err = rel_l2(got.cpu().numpy(), want)
+    assert err <= TIGHT, err
+
+
+def test_moe_gemm_gguf_q4k_rows_too_long_for_the_batched_form():
+    """Q4_K experts with rows of more than 16 super-blocks do not run as batched matvecs: 25 pairs per expert go through the
+    32-row tiles of the Q4_K matrix-core kernel."""
+    import candle_amd as ca
+    E, n, k, topk, tokens = 16, 96, 4352, 4, 100
+    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=75)
+    ids, tw, expert_ids, sorted_token_ids = route(tokens, E, topk, seed=76)
+    sti, eid = torch.from_numpy(sorted_token_ids).cuda(), torch.from_numpy(expert_ids).cuda()
+    x2 = normal(77, (tokens * topk, k), 1.0)
+    twf = tw.reshape(-1)
+    got = ca.moe_gemm_gguf(torch.from_numpy(x2).cuda(), qt, torch.from_numpy(twf).cuda(), sti, eid, topk, True)
+    torch.cuda.synchronize()
+    want = oracle.moe_gemm_gguf(oracle.Q4K, x2, blocks, (E, n, k), sorted_token_ids, expert_ids, twf, topk)
     err = rel_l2(got.cpu().numpy(), want)
     assert err <= TIGHT, err
 
