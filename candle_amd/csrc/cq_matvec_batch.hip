@@ -696,8 +696,6 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
     static_assert((DEPTH - 1) * NIW <= 63 && DEPTH >= 2, "counted waits");
     extern __shared__ __align__(16) uint8_t lds[];
     const int e = blockIdx.y;
-    const int seg0 = a.offsets[e], seg1 = a.offsets[e + 1];
-    if (seg0 >= seg1) return;
     QB_STAMP(0);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -733,6 +731,15 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(tile + kb * QB_KB), 16, lane * 16, kb * 1024, 0, 0);
         }
     };
+    // The first tile is asked for before the expert's pair range is known (a memory trip): where the weights are does not
+    // depend on it.  An expert without pairs waits for those copies and leaves.
+    issue(0);
+    asm volatile("" ::: "memory");
+    const int seg0 = a.offsets[e], seg1 = a.offsets[e + 1];
+    if (seg0 >= seg1) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        return;
+    }
     const int nsets = (seg1 - seg0 + 15) >> 4;
     for (int sg = 0; sg < nsets; sg += QME_NS) {
         // (a second pass starts behind the barrier that ended the first: every tile of the ring is free)
@@ -751,7 +758,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(recs + (live ? st * REC_KB + piece : QME_NS * REC_KB) * 1024), 16, lane * 16,
                                                      piece * 1024, 0, 0);
         }
-        issue(0);
+        if (sg > 0) issue(0);
         asm volatile("" ::: "memory");
         int rounds[QME_NS];                                                // results per lane a set needs: ceil(pairs / 4)
 #pragma unroll

@@ -188,18 +188,24 @@ def _qwen3_layer():
     return _QWEN3["v"]
 
 
-@pytest.mark.parametrize("tokens,is_prefill", [(16, False), (16, True), (256, True), (256, False)])
+@pytest.mark.parametrize("tokens,is_prefill", [(16, False), (16, True), (40, True), (256, True), (256, False), (600, True)])
 def test_fused_moe_layer_qwen3_shape_token_batches(tokens, is_prefill):
-    """16 and 256 tokens through the Qwen3-30B-A3B-shape layer: 128 and 2048 (token, expert) pairs, i.e. the per-pair
-    kernels and the expert-grouped matrix-core tiles, against the CPU restatement of FusedMoeGGUF::forward."""
+    """16 to 600 tokens through the Qwen3-30B-A3B-shape layer: 128 (token, expert) pairs on the per-pair kernels; 320, 2048 and
+    4800 pairs with every expert as a batched matvec over its own pairs (2.5, 16 and 37.5 pairs per expert on average: one
+    sparse set, two sets, a second pass over the weights), against the CPU restatement of FusedMoeGGUF::forward."""
     layer, ref = _qwen3_layer()
     x = normal(70 + tokens, (1, tokens, 2048), 1.0)
     got = layer.forward(torch.from_numpy(x).cuda(), is_prefill).cpu().numpy()
     want = ref.forward(x)
     assert got.shape == want.shape == (1, tokens, 2048)
     assert rel_l2(got, want) <= 1e-3
-    worst = max(rel_l2(got[0, r], want[0, r]) for r in range(tokens))
-    assert worst <= 1e-3, worst
+    # Row by row: the matmuls agree with the CPU to 2e-6 on the same quantized rows (tests/test_gpu_moe.py), and so does the typical
+    # row here.  A few rows in hundreds lie further off: gate and up differ from the CPU's in the last bit, so one value of
+    # silu(gate) * up now and then falls on the other side of a rounding boundary of the int8 quantizer of the down projection, a
+    # step of 1 / 127 of the row's largest value on one of 768 products.
+    errs = np.array([rel_l2(got[0, r], want[0, r]) for r in range(tokens)])
+    assert np.median(errs) <= 5e-6, float(np.median(errs))
+    assert errs.max() <= 5e-3, float(errs.max())
 
 
 @pytest.mark.parametrize("dtype", [oracle.Q4K, oracle.Q6K, oracle.Q5K])
