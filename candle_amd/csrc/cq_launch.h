@@ -155,7 +155,7 @@ bool cq_moe_stream_takes(int w_dtype, const void *w, const void *w_b, int64_t nu
 int64_t cq_moe_stream_operand_bytes(int64_t num_experts, int64_t n_pairs, int64_t k);
 #define CQ_MOE_STREAM_CHUNK 16
 int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *row_map, const float *scale_in, float *scale_out, const int *chunks,
-                                  int64_t max_chunks, const int *offsets, void *op, int64_t k, hipStream_t s);
+                                  int64_t max_chunks, int64_t num_experts, int64_t n_pairs, const int *offsets, void *op, int64_t k, hipStream_t s);
 int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
                          const float *pair_scale, int64_t num_experts, int64_t k, int64_t n, hipStream_t s);
 

@@ -25,6 +25,7 @@
 //
 // (-DCL_STAMPS compiles this file with per-wave s_memrealtime stamps and two extra entry points for a timeline of the launch;
 // the library is built without it.)
+#include <algorithm>
 #include "cq_actquant.h"
 #include "cq_device.h"
 #include "cq_fmt.h"
@@ -638,18 +639,18 @@ __host__ __device__ inline int64_t qme_operand_tiles(int64_t n_pairs, int64_t nu
 // the pair's 256 values of the column, gathered through row_map, into the chunk's operand tile — the streaming kernel's span
 // quantizer (cq_stream.h: where the first largest magnitude is negative the int8 values and the scale come out with the other
 // sign than BlockQ8K::from_float gives them, and every product is the same).  SW: the rows are silu(x[row]) * up[row], and the
-// pair's scale is scale_in[row] (the down projection after gate / up: one row per pair)
+// pair's scale is scale_in[row] (the down projection after gate / up: one row per pair).  The kernel is a chain of four memory
+// trips (chunk, row index, values, store); a wave that takes several columns in turn makes it longer, not shorter.
 template <bool SW>
 __global__ __launch_bounds__(1024) void qme_quantize_kernel(const float *__restrict__ x, const float *__restrict__ up, const int *__restrict__ row_map,
                                                             const float *__restrict__ scale_in, float *__restrict__ scale_out,
                                                             const int *__restrict__ chunks, int max_chunks, const int *__restrict__ offsets,
                                                             uint8_t *__restrict__ op, int bpr) {
     const int ci = blockIdx.x, col = blockIdx.y;
-    if (ci >= chunks[0]) return;
-    const int count = chunks[1 + 2 * max_chunks + ci];
+    // (the four words of the chunk in one trip: entries behind the last chunk hold anything and are not used)
+    const int n_chunks = chunks[0], e = chunks[1 + ci], first = chunks[1 + max_chunks + ci], count = chunks[1 + 2 * max_chunks + ci];
     const int lane = threadIdx.x & 63, c = threadIdx.x >> 6;
-    if (c >= count) return;
-    const int e = chunks[1 + ci], first = chunks[1 + max_chunks + ci];
+    if (ci >= n_chunks || c >= count) return;
     const int seg0 = offsets[e];
     const int tile = (seg0 >> 4) + e + ((first - seg0) >> 4);
     uint8_t *tp = op + (int64_t)tile * bpr * QME_TILE_COL_BYTES;
@@ -1022,12 +1023,14 @@ int64_t cq_moe_stream_operand_bytes(int64_t num_experts, int64_t n_pairs, int64_
 // chunks: the grouping pass's table for chunks of 16 pairs (n | expert[max_chunks] | first[] | count[]).  up != nullptr: the rows are
 // silu(x[row]) * up[row] and scale_out[i] = scale_in[row_map[i]].
 int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *row_map, const float *scale_in, float *scale_out, const int *chunks,
-                                  int64_t max_chunks, const int *offsets, void *op, int64_t k, hipStream_t s) {
+                                  int64_t max_chunks, int64_t num_experts, int64_t n_pairs, const int *offsets, void *op, int64_t k, hipStream_t s) {
+    // chunks of 16 pairs: at most one partly filled chunk per expert (the table has room for chunks of 8)
+    const int64_t grid = std::min<int64_t>(max_chunks, n_pairs / 16 + std::min(num_experts, n_pairs));
     if (up)
-        hipLaunchKernelGGL(qme_quantize_kernel<true>, dim3((unsigned)max_chunks, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
+        hipLaunchKernelGGL(qme_quantize_kernel<true>, dim3((unsigned)grid, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
                            (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256));
     else
-        hipLaunchKernelGGL(qme_quantize_kernel<false>, dim3((unsigned)max_chunks, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
+        hipLaunchKernelGGL(qme_quantize_kernel<false>, dim3((unsigned)grid, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
                            (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256));
     return (int)hipGetLastError();
 }

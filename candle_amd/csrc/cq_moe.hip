@@ -63,7 +63,18 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
     const int E = ps.num_experts;
     for (int e = tid; e < E; e += 1024) cur[e] = 0;
     __syncthreads();
-    for (int p = tid; p < ps.n_pairs; p += 1024) {
+    // the first KEEP pairs of every thread stay in registers between the two sweeps (decoding a pair is two dependent loads)
+    constexpr int KEEP = 4;
+    int ke[KEEP], kin[KEEP], kout[KEEP];
+    float ksc[KEEP];
+    bool kok[KEEP];
+#pragma unroll
+    for (int i = 0; i < KEEP; i++) {
+        const int p = tid + i * 1024;
+        kok[i] = p < ps.n_pairs && pair_decode(ps, p, ke[i], kin[i], kout[i], ksc[i]);
+        if (kok[i]) atomicAdd(&cur[ke[i]], 1);
+    }
+    for (int p = tid + KEEP * 1024; p < ps.n_pairs; p += 1024) {
         int e, in_row, out_row;
         float scale;
         if (pair_decode(ps, p, e, in_row, out_row, scale)) atomicAdd(&cur[e], 1);
@@ -106,10 +117,8 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
     // positions behind the last valid pair are never part of a chunk, but the gathering quantizer walks all n_pairs
     // rows: give them a valid source row
     for (int p = carry + tid; p < ps.n_pairs; p += 1024) pair_in[p] = 0;
-    for (int p = tid; p < ps.n_pairs; p += 1024) {
-        int e, in_row, out_row;
-        float scale;
-        if (pair_decode(ps, p, e, in_row, out_row, scale)) {
+    auto place = [&](int p, bool ok, int e, int in_row, int out_row, float scale) {
+        if (ok) {
             int pos = atomicAdd(&cur[e], 1);
             pair_in[pos] = in_row;
             pair_out[pos] = out_row;
@@ -117,6 +126,15 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
         } else if (ps.mode == MOE_INDEXED) {
             for (int c = 0; c < n; c++) out[(int64_t)p * n + c] = 0.0f;   // id out of range: defined output
         }
+    };
+#pragma unroll
+    for (int i = 0; i < KEEP; i++)
+        if (tid + i * 1024 < ps.n_pairs) place(tid + i * 1024, kok[i], ke[i], kin[i], kout[i], ksc[i]);
+    for (int p = tid + KEEP * 1024; p < ps.n_pairs; p += 1024) {
+        int e, in_row, out_row;
+        float scale;
+        const bool ok = pair_decode(ps, p, e, in_row, out_row, scale);
+        place(p, ok, e, in_row, out_row, scale);
     }
 }
 
@@ -224,7 +242,7 @@ int cq_moe_down_after_pair_launch(int w_dtype, const void *w_down, const float *
         const int *pout = (const int *)(b + ws.pout_off);
         float *pscale = (float *)(b + ws.pscale_off);
         const int *chunks = (const int *)(b + ws.chunk_off);
-        int rc = cq_moe_stream_quantize_launch(gate, up, pout, topk_weights, pscale, chunks, ws.max_chunks, offsets, b + ws.act_off, k, s);
+        int rc = cq_moe_stream_quantize_launch(gate, up, pout, topk_weights, pscale, chunks, ws.max_chunks, num_experts, n_pairs, offsets, b + ws.act_off, k, s);
         if (rc) return rc;
         return cq_moe_stream_launch(w_down, nullptr, out, nullptr, b + ws.act_off, offsets, pout, pscale, num_experts, k, n, s);
     }
@@ -287,7 +305,7 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if ((rc = (int)hipGetLastError())) return rc;
     if (stream) {
         // every expert a batched matvec over its own pairs: the weights of an expert are streamed once per 32 pairs
-        if ((rc = cq_moe_stream_quantize_launch(a.x, nullptr, pin, nullptr, nullptr, chunks, ws.max_chunks, offsets, b + ws.act_off, a.k, s))) return rc;
+        if ((rc = cq_moe_stream_quantize_launch(a.x, nullptr, pin, nullptr, nullptr, chunks, ws.max_chunks, a.num_experts, a.n_pairs, offsets, b + ws.act_off, a.k, s))) return rc;
         return cq_moe_stream_launch(a.w, a.w_b, a.out, a.out_b, b + ws.act_off, offsets, pout, pscale, a.num_experts, a.k, a.n, s);
     }
     if (mfma) {
