@@ -17,7 +17,8 @@
 // only its own columns, 16 short runs per tile, was tried first: those instructions take five times as long to issue), into
 // a ring of tiles, two blocks ahead.  The partial sums of the 8 waves meet in LDS once per block and are added in wave order.
 //
-// The activations are quantized exactly like BlockQ8K::from_float by a small kernel of this file, which leaves them laid out
+// The activations are quantized like BlockQ8K::from_float (up to a common sign of a span's values and scale, which no product
+// sees) by a small kernel of this file, or by the waves of the main kernel for up to 8 rows, which leaves them laid out
 // as the matrix operands the waves load.
 //
 // The same formulation serves MoE calls with hundreds of pairs: every expert a batched matvec over its own pairs
@@ -73,35 +74,6 @@ constexpr int QB_OP_COL_BYTES = 8 * 4 * 16 * 8;       // 4096
 constexpr int QB_REC_BYTES = 32;
 __host__ __device__ inline int64_t qb_operand_bytes(int64_t bpr) { return bpr * (QB_OP_COL_BYTES + 16 * QB_REC_BYTES); }
 
-// The arithmetic of cq_quantize_q8k_vals (cq_actquant.h) on the four values a lane holds of a 256-element span (elements
-// 4 lane .. 4 lane + 3): the first element of largest magnitude sets the scale.  packed: the lane's four int8 values;
-// lsum: their sum; d: the span's scale.
-__device__ __forceinline__ void qb_quantize_span(const float (&v)[4], int lane, uint32_t &packed, int &lsum, float &d) {
-    float amax = 0.0f;
-    int idx = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float a = fabsf(v[i]);
-        if (amax < a) { amax = a; idx = i; }
-    }
-    const float wmax = wave_max_nonneg(amax);
-    const int cand = wave_min_int((amax == wmax && wmax != 0.0f) ? lane * 4 + idx : 256);
-    const float mine = idx == 0 ? v[0] : idx == 1 ? v[1] : idx == 2 ? v[2] : v[3];
-    const float maxv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), (cand >> 2) & 63));
-    packed = 0;
-    lsum = 0;
-    d = 0.0f;
-    if (wmax != 0.0f) {
-        const float iscale = -127.0f / maxv;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int q = cq_round_sat_i8(iscale * v[i]);
-            lsum += q;
-            packed |= (uint32_t)(q & 0xff) << (8 * i);
-        }
-        d = 1.0f / iscale;
-    }
-}
 // where the lane's dword of a span goes inside one column of operands laid out [g < 4][kg < 4][slot < SLOTS][16 bytes]:
 // elements 4 lane .. + 3 are values 4 (lane % 8) .. + 3 of sub-block lane / 8: lane group kg = (lane % 8) / 2, dword lane % 2
 __device__ __forceinline__ int qb_operand_dword(int lane, int c, int slots) {
@@ -120,25 +92,22 @@ __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict
         if constexpr (XDT < 0) cq_load_swiglu4((const float *)x, up, c * x_stride + s * 256 + lane * 4, c * up_stride + s * 256 + lane * 4, v);
         else cq_load4<XDT>(x, c * x_stride + s * 256 + lane * 4, v);
     }
-    uint32_t packed;
-    int lsum;
-    float d;
-    qb_quantize_span(v, lane, packed, lsum, d);
+    // the streaming kernel's span quantizer (cq_stream.h: where the first largest magnitude is negative the int8 values and the scale
+    // come out with the other sign than BlockQ8K::from_float gives them, and every product is the same)
+    const float vv[1][4] = {{v[0], v[1], v[2], v[3]}};
+    const uint32_t wmax[1] = {qs_span_umax(vv[0])};
+    float iscale[1], d[1];
+    qs_span_scales<1>(wmax, lane, iscale, d);
+    int q[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) q[i] = qs_round_i8(iscale[0] * v[i]);
+    const uint32_t packed = qs_pack4(q);
     uint8_t *colp = op + (int64_t)s * QB_OP_COL_BYTES;
     *(uint32_t *)(colp + qb_operand_dword(lane, c, 16)) = packed;
-    const int s32 = oct_sum(lsum);                        // the sum of the 32-element sub-block, in its eight lanes
-    uint32_t bl[2] = {0, 0}, bh[2] = {0, 0};
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const int sj = __builtin_amdgcn_readlane(s32, 8 * j);
-        bl[j >> 2] |= (uint32_t)(sj & 127) << (8 * (j & 3));
-        bh[j >> 2] |= (uint32_t)((sj >> 7) & 255) << (8 * (j & 3));
-    }
-    if (lane == 0) {
-        uint8_t *rec = op + (int64_t)bpr * QB_OP_COL_BYTES + (int64_t)span * QB_REC_BYTES;
-        *(u32x4 *)rec = u32x4{bl[0], bl[1], bh[0], bh[1]};
-        *(float *)(rec + 16) = d;
-    }
+    const int s32 = oct_sum(sdot4(packed, 0x01010101u, 0));       // the sum of the 32-element sub-block, in its eight lanes
+    uint8_t *rec = op + (int64_t)bpr * QB_OP_COL_BYTES + (int64_t)span * QB_REC_BYTES;
+    if ((lane & 7) == 0) { rec[lane >> 3] = (uint8_t)(s32 & 127); rec[8 + (lane >> 3)] = (uint8_t)(s32 >> 7); }
+    if (lane == 0) *(float *)(rec + 16) = d[0];
 }
 
 // FQ > 0: `op` is not the operand buffer but the f32 activations themselves, [rows == FQ][256 bpr], and every wave quantizes
