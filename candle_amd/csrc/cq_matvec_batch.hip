@@ -65,11 +65,15 @@ __host__ __device__ constexpr int qb_tile_bytes(int block_bytes) { return ((bloc
 
 // ---- the activations, quantized like BlockQ8K::from_float and laid out as this kernel's matrix operands ----
 // For super-block column s of the row length, 16 batch slots (rows beyond the batch are zeros):
-//   operands [s][g < 4][kg < 4][batch slot c < 16][16 bytes]   values 8 kg .. 8 kg + 7 of sub-blocks 2 g and 2 g + 1 of column s of
+//   operands [s][g < 4][kg < 4][slot c < 16][16 bytes]         values 8 kg .. 8 kg + 7 of sub-blocks 2 g and 2 g + 1 of column s of
 //                                                              row c: what lane (c, kg) feeds the matrix core against the low and
 //                                                              the high nibbles of weight bytes 32 g + 8 kg .. + 7; one 16-byte
 //                                                              load per lane, 1 KB contiguous per wave;
 //   records  [s][c] { u8 bl[8], i8 bh[8] (sum of sub-block j = 128 * bh_j + bl_j), f32 d, 12 bytes unused }
+// Batch row b sits in operand slot 4 (b % 4) + b / 4 (the map is its own inverse): a lane's result r of lane group kg then belongs
+// to batch row 4 r + kg, and a batch of `rows` rows needs only the first ceil(rows / 4) of a lane's four results worked out (the
+// scaling of a result is most of the kernels' vector work).
+__host__ __device__ constexpr int qb_slot(int b) { return 4 * (b & 3) + (b >> 2); }
 constexpr int QB_OP_COL_BYTES = 8 * 4 * 16 * 8;       // 4096
 constexpr int QB_REC_BYTES = 32;
 __host__ __device__ inline int64_t qb_operand_bytes(int64_t bpr) { return bpr * (QB_OP_COL_BYTES + 16 * QB_REC_BYTES); }
@@ -86,7 +90,7 @@ __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict
                                                           uint8_t *__restrict__ op, int bpr, int rows) {
     const int span = (int)blockIdx.x * 4 + ((int)threadIdx.x >> 6);          // span = s * 16 + c
     if (span >= bpr * 16) return;
-    const int lane = threadIdx.x & 63, s = span >> 4, c = span & 15;
+    const int lane = threadIdx.x & 63, s = span >> 4, slot = span & 15, c = qb_slot(slot);      // c: the batch row of this slot
     float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (c < rows) {
         if constexpr (XDT < 0) cq_load_swiglu4((const float *)x, up, c * x_stride + s * 256 + lane * 4, c * up_stride + s * 256 + lane * 4, v);
@@ -103,7 +107,7 @@ __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict
     for (int i = 0; i < 4; i++) q[i] = qs_round_i8(iscale[0] * v[i]);
     const uint32_t packed = qs_pack4(q);
     uint8_t *colp = op + (int64_t)s * QB_OP_COL_BYTES;
-    *(uint32_t *)(colp + qb_operand_dword(lane, c, 16)) = packed;
+    *(uint32_t *)(colp + qb_operand_dword(lane, slot, 16)) = packed;
     const int s32 = oct_sum(sdot4(packed, 0x01010101u, 0));       // the sum of the 32-element sub-block, in its eight lanes
     uint8_t *rec = op + (int64_t)bpr * QB_OP_COL_BYTES + (int64_t)span * QB_REC_BYTES;
     if ((lane & 7) == 0) { rec[lane >> 3] = (uint8_t)(s32 & 127); rec[8 + (lane >> 3)] = (uint8_t)(s32 >> 7); }
@@ -120,7 +124,9 @@ __global__ __launch_bounds__(256) void qb_quantize_kernel(const void *__restrict
 constexpr int QB_FQ_MAX_SPANS = 16;                // spans (columns x rows) a wave quantizes itself at most; beyond, the separate kernel is ahead
 constexpr int QB_FQ_REC = 32;                      // bytes of a staged record {u8 bl[8], u8 bh[8], f32 d, unused}
 __host__ __device__ constexpr int qb_fq_col_bytes(int fq) { return fq * 256 + fq * QB_FQ_REC; }      // operands + records of one column
-template <int CPW, int DEPTH, int FQ>
+// NR: results per lane that the batch needs, ceil(rows / 4) (a template parameter: behind a run-time bound every result is a basic
+// block of its own, and 16 rows lose 0.7 us)
+template <int CPW, int DEPTH, int FQ, int NR = (FQ + 3) / 4>
 __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ op, void *__restrict__ dst, int n, int bpr,
                                                               int rows, int dst_dtype, int64_t stride_dst
 #ifdef CL_STAMPS
@@ -161,7 +167,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
         }
     };
     long A[CPW][8];
-    u32x4 aux[CPW][4];                            // {bl 0-3, bl 4-7, bh 0-3, bh 4-7} of batch row 4 kg + r: sub-block sum j = 128 * bh_j + bl_j
+    u32x4 aux[CPW][4];                            // {bl 0-3, bl 4-7, bh 0-3, bh 4-7} of slot 4 kg + r (batch row 4 r + kg): sub-block sum j = 128 * bh_j + bl_j
     float d8[CPW][4];
     if constexpr (FQ > 0) {
         // ---- the wave quantizes the activations of its columns itself ----
@@ -234,12 +240,13 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
             const uint8_t *colp = stage + ci * qb_fq_col_bytes(FQ), *recs = colp + FQ * 256;
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const i64x2 v = c < FQ ? *(const i64x2 *)(colp + ((g * 4 + kg) * FQ + c) * 16) : i64x2{0, 0};
+                // (staged by batch row; slot c of the operand is batch row qb_slot(c))
+                const i64x2 v = qb_slot(c) < FQ ? *(const i64x2 *)(colp + ((g * 4 + kg) * FQ + qb_slot(c)) * 16) : i64x2{0, 0};
                 A[ci][2 * g] = v.x; A[ci][2 * g + 1] = v.y;
             }
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const uint8_t *rec = recs + min(4 * kg + r, FQ - 1) * QB_FQ_REC;         // (results of batch rows beyond the last are not stored)
+                const uint8_t *rec = recs + min(4 * r + kg, FQ - 1) * QB_FQ_REC;         // (results of batch rows beyond the last are not stored)
                 aux[ci][r] = *(const u32x4 *)rec;
                 d8[ci][r] = *(const float *)(rec + 16);
             }
@@ -253,7 +260,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
     // ---- the wave's activations, in registers for the whole kernel ----
     // The activations are the FIRST matrix operand (lane (c, kg): values 8 kg .. 8 kg + 7 of each sub-block of batch row c) and
     // the weights the second, so a lane's four results belong to ONE weight row (row c of the block: one header to decode per
-    // column) and to the batch rows 4 kg + r, whose block sums and scales it keeps as well.
+    // column) and to the slots 4 kg + r (batch rows 4 r + kg), whose block sums and scales it keeps as well.
     QB_STAMP(0);
     // (a wave's load of one operand is 512 contiguous bytes; the four lane groups read four records)
 #pragma unroll
@@ -262,7 +269,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
         const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 16;         // lane = kg * 16 + c
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            const i64x2 v = c < rows ? *(const i64x2 *)(colp + g * 1024) : i64x2{0, 0};    // (batch slots beyond the rows hold zeros)
+            const i64x2 v = qb_slot(c) < rows ? *(const i64x2 *)(colp + g * 1024) : i64x2{0, 0};    // (slots beyond the batch hold zeros)
             A[ci][2 * g] = v.x; A[ci][2 * g + 1] = v.y;
         }
 #pragma unroll
@@ -314,11 +321,13 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
                 const float dw = h2f(hdr.x), dm = h2f(hdr.x >> 16);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    int S = 0;
+                    if (r < NR) {                                     // result r belongs to batch rows 4 r .. 4 r + 3
+                        int S = 0;
 #pragma unroll
-                    for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
-                    const int M = qs_dot_sums(s.mA, s.mB, aux[ci][r]);
-                    acc[r] += d8[ci][r] * (dw * (float)S - dm * (float)M);
+                        for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
+                        const int M = qs_dot_sums(s.mA, s.mB, aux[ci][r]);
+                        acc[r] += d8[ci][r] * (dw * (float)S - dm * (float)M);
+                    }
                 }
             }
         }
@@ -333,7 +342,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
 #pragma unroll
             for (int w2 = 0; w2 < QB_NW; w2++) v += red[(w2 * 64 + l2) * 4 + r];
             const int m = bx + i * gx;
-            const int row = m * 16 + (l2 & 15), br = 4 * (l2 >> 4) + r;
+            const int row = m * 16 + (l2 & 15), br = 4 * r + (l2 >> 4);
             if (row < n && br < rows) store_out(dst, dst_dtype, (int64_t)br * stride_dst + row, v);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");          // the sums have left LDS before this wave reaches the next barrier
@@ -352,7 +361,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
 // one chunk, gathered by the copy instructions from 16 row segments), wave w owns columns 2 w, 2 w + 1 of EVERY chunk and
 // keeps their int8 operands in registers (Q x 2 x 16 registers), and the per-row records (block sums, scale) wait in LDS.
 // The accumulators run across the chunks of a block; everything else is the kernel above.
-template <int Q>
+template <int Q, int NR>
 __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ op, void *__restrict__ dst, int n,
                                                                    int bpr, int rows, int dst_dtype, int64_t stride_dst, int cpp
 #ifdef CL_STAMPS
@@ -424,7 +433,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
             const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 16;     // lane = kg * 16 + c
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const i64x2 v = c < rows ? *(const i64x2 *)(colp + g * 1024) : i64x2{0, 0};    // (batch slots beyond the rows hold zeros)
+                const i64x2 v = qb_slot(c) < rows ? *(const i64x2 *)(colp + g * 1024) : i64x2{0, 0};    // (slots beyond the batch hold zeros)
                 A[q][ci][2 * g] = v.x; A[q][ci][2 * g + 1] = v.y;
             }
         }
@@ -483,13 +492,15 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
                     const uint8_t *rec = recs + ((q * cpp + col0 + ci) * 16 + 4 * kg) * QB_REC_BYTES;
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        int S = 0;
+                        if (r < NR) {                                     // result r belongs to batch rows 4 r .. 4 r + 3
+                            int S = 0;
 #pragma unroll
-                        for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
-                        const u32x4 aux = *(const u32x4 *)(rec + r * QB_REC_BYTES);
-                        const float d8 = *(const float *)(rec + r * QB_REC_BYTES + 16);
-                        const int M = qs_dot_sums(s.mA, s.mB, aux);
-                        acc[r] += d8 * (dw * (float)S - dm * (float)M);
+                            for (int g = 0; g < 4; g++) S += __mul24(sc[2 * g], cl[g][r]) + __mul24(sc[2 * g + 1], ch[g][r]);
+                            const u32x4 aux = *(const u32x4 *)(rec + r * QB_REC_BYTES);
+                            const float d8 = *(const float *)(rec + r * QB_REC_BYTES + 16);
+                            const int M = qs_dot_sums(s.mA, s.mB, aux);
+                            acc[r] += d8 * (dw * (float)S - dm * (float)M);
+                        }
                     }
                 }
             }
@@ -504,7 +515,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
 #pragma unroll
             for (int w2 = 0; w2 < QB_NW; w2++) v += red[(w2 * 64 + l2) * 4 + r];
             const int m = bx + i * gx;
-            const int row = m * 16 + (l2 & 15), br = 4 * (l2 >> 4) + r;
+            const int row = m * 16 + (l2 & 15), br = 4 * r + (l2 >> 4);
             if (row < n && br < rows) store_out(dst, dst_dtype, (int64_t)br * stride_dst + row, v);
         }
         // (the sums have left LDS before this wave passes the next barrier, behind which `red` is written again only after
@@ -519,13 +530,13 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
 #endif
 }
 
-template <int Q>
-int launch_qmb_long(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int cpp,
-                    hipStream_t s) {
+template <int Q, int NR>
+int launch_qmb_long_r(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int cpp,
+                      hipStream_t s) {
     const int64_t bpr = k / 256;
     const size_t lds_bytes = (size_t)3 * qb_tile_bytes(16 * cpp * QB_BB) + QB_RED_BYTES + (size_t)bpr * 16 * QB_REC_BYTES;
     if (lds_bytes > (size_t)QB_LDS_BYTES - 1024) return CQ_ERR_RANGE;
-    auto kern = qmb_q4k_long_kernel<Q>;
+    auto kern = qmb_q4k_long_kernel<Q, NR>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     const int64_t nsteps = (n + 15) / 16;
@@ -540,10 +551,21 @@ int launch_qmb_long(const void *w, const uint8_t *op, void *dst, int dst_dtype, 
     return (int)hipGetLastError();
 }
 
-template <int CPW, int DEPTH, int FQ = 0>
-int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
-                 hipStream_t s) {
-    auto kern = qmb_q4k_kernel<CPW, DEPTH, FQ>;
+template <int Q>
+int launch_qmb_long(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int cpp,
+                    hipStream_t s) {
+    switch ((rows + 3) / 4) {
+        case 1: return launch_qmb_long_r<Q, 1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+        case 2: return launch_qmb_long_r<Q, 2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+        case 3: return launch_qmb_long_r<Q, 3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+        default: return launch_qmb_long_r<Q, 4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+    }
+}
+
+template <int CPW, int DEPTH, int FQ, int NR>
+int launch_qmb_dr(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
+                  hipStream_t s) {
+    auto kern = qmb_q4k_kernel<CPW, DEPTH, FQ, NR>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
@@ -558,6 +580,17 @@ int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int
 #endif
     );
     return (int)hipGetLastError();
+}
+template <int CPW, int DEPTH, int FQ = 0>
+int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
+                 hipStream_t s) {
+    if constexpr (FQ > 0) return launch_qmb_dr<CPW, DEPTH, FQ, (FQ + 3) / 4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+    switch ((rows + 3) / 4) {
+        case 1: return launch_qmb_dr<CPW, DEPTH, 0, 1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+        case 2: return launch_qmb_dr<CPW, DEPTH, 0, 2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+        case 3: return launch_qmb_dr<CPW, DEPTH, 0, 3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+        default: return launch_qmb_dr<CPW, DEPTH, 0, 4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+    }
 }
 // Three tiles where LDS holds them (the one being worked on and two on their way), else two.  (Four were measured slower:
 // with three tiles asked for at the start the first one lands 1 us later, and the steady state gains nothing.)
@@ -600,7 +633,7 @@ int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64
 // Pair b of a set sits in operand slot 4 (b % 4) + b / 4: a lane's result r of lane group kg then belongs to pair 4 r + kg, and a
 // set of `cnt` pairs needs only the first ceil(cnt / 4) of a lane's four results worked out (the scaling of a result is most of
 // the kernel's vector work, and most sets are far from full).
-__host__ __device__ constexpr int qme_slot(int b) { return 4 * (b & 3) + (b >> 2); }
+__host__ __device__ constexpr int qme_slot(int b) { return qb_slot(b); }
 constexpr int QME_TILE_COL_BYTES = QB_OP_COL_BYTES + 16 * QB_REC_BYTES;          // 4608 bytes of a tile per super-block column
 __host__ __device__ inline int64_t qme_operand_tiles(int64_t n_pairs, int64_t num_experts) { return n_pairs / 16 + num_experts + 1; }
 
