@@ -19,6 +19,11 @@ int64_t cq_matvec_batch_workspace(int w_dtype, int64_t k, int64_t rows);
 int cq_matvec_batch_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *workspace, void *dst, int dst_dtype, int64_t k, int64_t n,
                            int64_t rows, int64_t stride_dst, hipStream_t s);
 // the same over rows silu(gate[r]) * up[r] (f32, row strides in floats)
+// 17 .. 64 f32 rows of Q4_K with rows of up to 16 super-blocks: the rows in sets of 16, two sets per pass over the weights
+bool cq_matvec_batch_mid_takes(int w_dtype, const void *w, const void *x, int x_dtype, int dst_dtype, int64_t k, int64_t n, int64_t rows);
+int64_t cq_matvec_batch_mid_workspace(int w_dtype, int64_t k, int64_t rows);
+int cq_matvec_batch_mid_launch(const void *w, const float *x, const float *up, int64_t x_stride, int64_t up_stride, void *workspace, float *dst,
+                               int64_t k, int64_t n, int64_t rows, hipStream_t s);      // up != nullptr: rows silu(x[r]) * up[r]
 int cq_matvec_batch_swiglu_launch(int w_dtype, const void *w, const float *gate, const float *up, int64_t gate_stride, int64_t up_stride, void *workspace,
                                   void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s);
 // QMatMul::forward for <= CQ_MATVEC_MAX_ROWS rows with the activation quantization fused into the matvec kernel

@@ -647,20 +647,31 @@ template <bool SW>
 __global__ __launch_bounds__(1024) void qme_quantize_kernel(const float *__restrict__ x, const float *__restrict__ up, const int *__restrict__ row_map,
                                                             const float *__restrict__ scale_in, float *__restrict__ scale_out,
                                                             const int *__restrict__ chunks, int max_chunks, const int *__restrict__ offsets,
-                                                            uint8_t *__restrict__ op, int bpr) {
+                                                            uint8_t *__restrict__ op, int bpr, int64_t x_stride, int64_t up_stride) {
     const int ci = blockIdx.x, col = blockIdx.y;
-    // (the four words of the chunk in one trip: entries behind the last chunk hold anything and are not used)
-    const int n_chunks = chunks[0], e = chunks[1 + ci], first = chunks[1 + max_chunks + ci], count = chunks[1 + 2 * max_chunks + ci];
     const int lane = threadIdx.x & 63, c = threadIdx.x >> 6;
-    if (ci >= n_chunks || c >= count) return;
-    const int seg0 = offsets[e];
-    const int tile = (seg0 >> 4) + e + ((first - seg0) >> 4);
+    int tile;
+    int64_t row;
+    int first = 16 * ci;
+    if (chunks) {
+        // (the four words of the chunk in one trip: entries behind the last chunk hold anything and are not used)
+        const int n_chunks = chunks[0], e = chunks[1 + ci], count = chunks[1 + 2 * max_chunks + ci];
+        first = chunks[1 + max_chunks + ci];
+        if (ci >= n_chunks || c >= count) return;
+        const int seg0 = offsets[e];
+        tile = (seg0 >> 4) + e + ((first - seg0) >> 4);
+        row = row_map[first + c];
+    } else {
+        // one matrix, the rows as they are (max_chunks: the number of rows): chunk ci is rows 16 ci .. of tile ci
+        if (first + c >= max_chunks) return;
+        tile = ci;
+        row = first + c;
+    }
     uint8_t *tp = op + (int64_t)tile * bpr * QME_TILE_COL_BYTES;
-    const int64_t row = row_map[first + c];
-    if (SW && col == 0 && lane == 0) scale_out[first + c] = scale_in[row];
+    if (SW && scale_out && col == 0 && lane == 0) scale_out[first + c] = scale_in[row];
     float v[1][4];
-    if constexpr (SW) cq_load_swiglu4(x, up, (row * bpr + col) * 256 + lane * 4, (row * bpr + col) * 256 + lane * 4, v[0]);
-    else cq_load4<CQ_F32>(x, (row * bpr + col) * 256 + lane * 4, v[0]);
+    if constexpr (SW) cq_load_swiglu4(x, up, row * x_stride + col * 256 + lane * 4, row * up_stride + col * 256 + lane * 4, v[0]);
+    else cq_load4<CQ_F32>(x, row * x_stride + col * 256 + lane * 4, v[0]);
     const uint32_t wmax[1] = {qs_span_umax(v[0])};
     float iscale[1], d[1];
     qs_span_scales<1>(wmax, lane, iscale, d);
@@ -687,6 +698,7 @@ struct QmeArgs {
     const int *pair_out;          // output row of a sorted pair
     const float *pair_scale;      // and the factor on its results
     int n, bpr, parts;
+    int dense_rows;               // > 0: one matrix and rows 0 .. dense_rows - 1 as its pairs (no offsets, output row = pair, factor 1)
 };
 constexpr int QME_NS = 2;         // sets of 16 pairs per pass over the weights
 constexpr int QME_MAX_AVG_PAIRS = 64;   // pairs per expert on average up to which a call takes this form
@@ -738,7 +750,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
     // depend on it.  An expert without pairs waits for those copies and leaves.
     issue(0);
     asm volatile("" ::: "memory");
-    const int seg0 = a.offsets[e], seg1 = a.offsets[e + 1];
+    const int seg0 = a.dense_rows ? 0 : a.offsets[e], seg1 = a.dense_rows ? a.dense_rows : a.offsets[e + 1];
     if (seg0 >= seg1) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         return;
@@ -788,8 +800,8 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
         const int oset = tid >> 8, ol2 = tid & 63, orr = (tid >> 6) & 3;
         const int opos = seg0 + (sg + oset) * 16 + 4 * orr + (ol2 >> 4);
         const bool ovalid = opos < seg1;
-        const int64_t orow = ovalid ? a.pair_out[opos] : 0;
-        const float oscale = ovalid ? a.pair_scale[opos] : 0.0f;
+        const int64_t orow = !ovalid ? 0 : a.dense_rows ? opos : a.pair_out[opos];
+        const float oscale = !ovalid ? 0.0f : a.dense_rows ? 1.0f : a.pair_scale[opos];
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int i = 1; i < DEPTH - 1; i++) issue(i);
@@ -1030,12 +1042,13 @@ int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *ro
     const int64_t grid = std::min<int64_t>(max_chunks, n_pairs / 16 + std::min(num_experts, n_pairs));
     if (up)
         hipLaunchKernelGGL(qme_quantize_kernel<true>, dim3((unsigned)grid, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
-                           (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256));
+                           (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256), k, k);
     else
         hipLaunchKernelGGL(qme_quantize_kernel<false>, dim3((unsigned)grid, (unsigned)(k / 256)), dim3(1024), 0, s, x, up, row_map, scale_in, scale_out, chunks,
-                           (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256));
+                           (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256), k, k);
     return (int)hipGetLastError();
 }
+static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s);
 // out_a[pair_out[p]][:] = (W_a[expert of p] . x^[p]) * pair_scale[p] for every sorted pair p; the same for (w_b, out_b) when given
 int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
                          const float *pair_scale, int64_t num_experts, int64_t k, int64_t n, hipStream_t s) {
@@ -1043,6 +1056,14 @@ int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *
     QmeArgs a;
     a.w[0] = (const uint8_t *)w_a; a.w[1] = (const uint8_t *)w_b; a.out[0] = out_a; a.out[1] = out_b;
     a.op = (const uint8_t *)op; a.offsets = offsets; a.pair_out = pair_out; a.pair_scale = pair_scale; a.n = (int)n; a.bpr = bpr;
+    a.dense_rows = 0;
+    return qme_launch(a, num_experts, tensors, s);
+}
+
+// the launch geometry of the expert kernel: waves per row block, parts per expert and tensor
+static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s) {
+    const int bpr = a.bpr;
+    const int64_t n = a.n;
     // waves that share a row block: the fewest (a power of two) with at most two columns each — large tiles: a tile costs about
     // a microsecond of barriers and latencies whatever it holds
     const int cw = bpr > 8 ? 8 : bpr > 4 ? 4 : bpr > 2 ? 2 : 1;
@@ -1050,6 +1071,8 @@ int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *
     // parts: experts x tensors x parts fills the CUs once or twice (all experts hit: the same bytes everywhere)
     int64_t parts = (256 + num_experts * tensors - 1) / (num_experts * tensors);
     if (parts > ntiles) parts = ntiles;
+    // (every part the same number of tiles where that is possible: 896 tiles are 224 parts of 4, not 256 of 3 or 4)
+    if (parts > 1) parts = (ntiles + (ntiles + parts - 1) / parts - 1) / ((ntiles + parts - 1) / parts);
     a.parts = (int)parts;
     switch (cw) {
         case 8: return launch_qme<8, 2>(a, num_experts, tensors, s);
@@ -1057,6 +1080,37 @@ int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *
         case 2: return launch_qme<2, 2>(a, num_experts, tensors, s);
         default: return bpr == 2 ? launch_qme<1, 2>(a, num_experts, tensors, s) : launch_qme<1, 1>(a, num_experts, tensors, s);
     }
+}
+
+// ---- QMatMul::forward for 17 .. 64 rows: the matrix as the one expert of the kernel above, the rows as its pairs (two sets of 16
+// per pass over the weights) ----
+// (the 32-row / 128-row matrix-core tiles convert every weight for the rows of a tile: at these row counts that costs more than
+// scaling the results)
+bool cq_matvec_batch_mid_takes(int w_dtype, const void *w, const void *x, int x_dtype, int dst_dtype, int64_t k, int64_t n, int64_t rows) {
+    return w_dtype == CQ_Q4K && x_dtype == CQ_F32 && dst_dtype == CQ_F32 && rows > 16 && rows <= 64 &&
+           cq_moe_stream_takes(w_dtype, w, nullptr, 1, rows, k, n) && ((uintptr_t)x & 15) == 0;
+}
+int64_t cq_matvec_batch_mid_workspace(int w_dtype, int64_t k, int64_t rows) {
+    return w_dtype == CQ_Q4K && rows > 16 && rows <= 64 && k % 256 == 0 && k / 256 <= 2 * QB_NW ? cq_align256(((rows + 15) / 16) * (k / 256) * QME_TILE_COL_BYTES) : 0;
+}
+// up != nullptr: the rows are silu(x[r]) * up[r], with row strides in floats
+int cq_matvec_batch_mid_launch(const void *w, const float *x, const float *up, int64_t x_stride, int64_t up_stride, void *workspace, float *dst,
+                               int64_t k, int64_t n, int64_t rows, hipStream_t s) {
+    const int bpr = (int)(k / 256);
+    const dim3 grid((unsigned)((rows + 15) / 16), (unsigned)bpr);
+    if (up)
+        hipLaunchKernelGGL(qme_quantize_kernel<true>, grid, dim3(1024), 0, s, x, up, (const int *)nullptr, (const float *)nullptr, (float *)nullptr,
+                           (const int *)nullptr, (int)rows, (const int *)nullptr, (uint8_t *)workspace, bpr, x_stride, up_stride);
+    else
+        hipLaunchKernelGGL(qme_quantize_kernel<false>, grid, dim3(1024), 0, s, x, up, (const int *)nullptr, (const float *)nullptr, (float *)nullptr,
+                           (const int *)nullptr, (int)rows, (const int *)nullptr, (uint8_t *)workspace, bpr, x_stride, up_stride);
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    QmeArgs a;
+    a.w[0] = (const uint8_t *)w; a.w[1] = nullptr; a.out[0] = dst; a.out[1] = nullptr;
+    a.op = (const uint8_t *)workspace; a.offsets = nullptr; a.pair_out = nullptr; a.pair_scale = nullptr; a.n = (int)n; a.bpr = bpr;
+    a.dense_rows = (int)rows;
+    return qme_launch(a, 1, 1, s);
 }
 
 #ifdef CL_STAMPS

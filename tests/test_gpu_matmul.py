@@ -127,6 +127,23 @@ def test_q4k_batched_rows_quantized_inside_the_kernel(k, rows):
         assert rel_l2(got[r], want[r]) <= TIGHT, r
 
 
+@pytest.mark.parametrize("k", [256, 768, 2048, 4096])
+@pytest.mark.parametrize("n,rows", [(203, 17), (203, 32), (96, 33), (50, 47), (130, 64)])
+def test_q4k_rows_in_sets_of_16_vs_oracle(k, n, rows):
+    """17 .. 64 f32 rows of Q4_K (rows of up to 4096 elements) run as sets of 16 rows, two sets per pass over the weights: a
+    partly filled second set, a second pass with one set and with two, ragged n, one to eight waves per row block."""
+    blocks, qmm = make_weight(oracle.Q4K, n, k, seed=181)
+    x = normal(182 + rows, (rows, k), 1.0)
+    x[0, :256] = 0.0
+    x[rows - 1, k - 3] = -7.5
+    got = forward(qmm, x)
+    want = oracle.matmul_fast(oracle.Q4K, x, blocks, n, 8)
+    err = rel_l2(got, want)
+    assert err <= TOL and err <= TIGHT, f"rel-L2 {err}"
+    for r in range(rows):
+        assert rel_l2(got[r], want[r]) <= TIGHT, r
+
+
 def test_cfg1_q8_0_4096x4096():
     # BASELINE configs[0]: Q8_0 weight [4096 x 4096], activation 1 x 4096
     blocks, qmm = make_weight(oracle.Q8_0, 4096, 4096, seed=1)
