@@ -133,7 +133,9 @@ int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float
  * QCudaStorage::fwd (cuda.rs:846-878), the body of CustomOp1::cuda_fwd for QTensor
  * (mod.rs:1007-1017): quantize the m activation rows, then matvec (m <= CQ_MATVEC_MAX_ROWS; for m <= 2 the
  * quantization happens inside the matvec kernel; Q4K with 3 <= m <= 16, k a multiple of 256 up to 16384 and 16-byte
- * aligned weights: one pass over the weights on the int8 matrix cores with the rows as register operands) or MFMA matmul
+ * aligned weights: one pass over the weights on the int8 matrix cores with the rows as register operands, up to 8 f32 rows of
+ * up to 6144 elements quantized inside that kernel; Q4K with 17 <= m <= 64 f32 rows of up to 4096 elements to an f32 dst: the
+ * same with the rows in sets of 16, one pass over the weights per 32 rows) or MFMA matmul
  * (split over k with an ordered reduction when the grid would be small).  x is [m, k] contiguous (f32 / f16 / bf16), dst is [m, n] contiguous in dst_dtype
  * (CUDA keeps the input dtype: fast_mmvq.rs:161-323).  workspace_dev: 256-byte aligned,
  * at least cq_qmatmul_workspace_bytes(w_dtype, m, k, n) bytes.
@@ -171,7 +173,8 @@ int cq_qmatmul_forward_static(int w_dtype, const void *w_dev, const void *x_dev,
  *   ids [batch, topk] u32  ->  out [batch, topk, n] f32,
  *   out[b, t, :] = W[ids[b, t]] . x[b, input_dim1 == 1 ? 0 : t, :].
  * Up to 256 pairs (512 for short rows, see cq_moe_direct_pairs) each pair is its own fused matvec; beyond, pairs are grouped by expert on the device and an expert's
- * rows are streamed once per tile of 32 or 128 pairs on the matrix cores (K-quant experts; integer-exact) or once per
+ * rows are streamed once per 32 of its pairs as a batched matvec (Q4K experts with rows of up to 4096 elements that see at
+ * most 64 pairs each on average), once per tile of 32 or 128 pairs on the matrix cores (K-quant experts; integer-exact) or once per
  * 8 pairs by the matvec kernel (the other formats).  The reference takes Q2K-Q6K and Q8_0 experts (cuda.rs:543-548).
  * An id >= num_experts leaves its output row zero-filled.
  * ------------------------------------------------------------------------------------------- */
