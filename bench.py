@@ -674,10 +674,11 @@ def other_configurations(L, torch, args):
                    "frac_of_hbm_peak": round(rot.alg_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
     del rot, g
     torch.cuda.empty_cache()
-    # cfg2: the Q4_K batch sweep on both FFN shapes (batch 16 takes the matrix-core kernel: two kernels per step)
+    # cfg2: the Q4_K batch sweep on both FFN shapes (3 .. 16 rows: the batched matrix-core matvec; the first shape also at 32 and 64
+    # rows, which run as sets of 16 rows through the same formulation)
     sweep = []
     for (n, k) in ((14336, 4096), (4096, 14336)):
-        for b in (1, 2, 4, 8, 16):
+        for b in (1, 2, 4, 8, 16) + ((32, 64) if k <= 4096 else ()):
             rot = Rotation(L, torch, "q4k", n, k, b, 600)
             g = rot.capture(rot.step)
             us = rot.event_us(g, 1000, 100)
