@@ -161,8 +161,11 @@ int64_t cq_moe_stream_operand_bytes(int64_t num_experts, int64_t n_pairs, int64_
 #define CQ_MOE_STREAM_CHUNK 16
 int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *row_map, const float *scale_in, float *scale_out, const int *chunks,
                                   int64_t max_chunks, int64_t num_experts, int64_t n_pairs, const int *offsets, void *op, int64_t k, hipStream_t s);
+// extra: n | counter of launch 0 | counter of launch 1 | (expert, pass)[n]: the passes beyond the first of the experts with more than
+// 32 pairs, written (counters zero) by the grouping pass; launch_slot: which counter this launch counts with
+#define CQ_MOE_EXTRA_HEADER 3
 int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
-                         const float *pair_scale, int64_t num_experts, int64_t k, int64_t n, hipStream_t s);
+                         const float *pair_scale, int *extra, int launch_slot, int64_t num_experts, int64_t k, int64_t n, hipStream_t s);
 
 // Pairs from which a K-quant MoE call goes through the MFMA kernel (tiles of expert-sorted rows): everything the
 // per-pair kernels do not take.  Measured on 128 experts of 768 x 2048: 264-1016 pairs take 211-229 us per layer on

@@ -699,6 +699,9 @@ struct QmeArgs {
     const float *pair_scale;      // and the factor on its results
     int n, bpr, parts;
     int dense_rows;               // > 0: one matrix and rows 0 .. dense_rows - 1 as its pairs (no offsets, output row = pair, factor 1)
+    int *extra;                   // n | two counters | (expert, pass)[n]: the passes beyond an expert's first; NULL: every workgroup runs all passes of its expert
+    int extra_slot;               // which of the two counters this launch counts with
+    int extra_parts;              // parts per expert and tensor that a listed pass is cut into (a multiple of parts: finer than a workgroup's own share)
 };
 constexpr int QME_NS = 2;         // sets of 16 pairs per pass over the weights
 constexpr int QME_MAX_AVG_PAIRS = 64;   // pairs per expert on average up to which a call takes this form
@@ -710,7 +713,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
     constexpr int NIW = (16 * NRB * CW * CPW * QB_BB + 8 * 1024 - 1) / (8 * 1024);      // copy instructions per wave and tile
     static_assert((DEPTH - 1) * NIW <= 63 && DEPTH >= 2, "counted waits");
     extern __shared__ __align__(16) uint8_t lds[];
-    const int e = blockIdx.y;
+    int e = blockIdx.y;
     QB_STAMP(0);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -725,12 +728,22 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
     float *red = (float *)(lds + DEPTH * TILE);                            // [2][sets][8 waves][64 lanes][4]
     constexpr int REC_KB = (CW * CPW * 16 * QB_REC_BYTES + 1023) / 1024;   // KBs of the records of one set (at most CW * CPW columns)
     uint8_t *recs = lds + DEPTH * TILE + 2 * QME_NS * QB_RED_BYTES;        // [sets][REC_KB KB], one spare KB
-    const uint8_t *w = a.w[blockIdx.z] + (int64_t)e * n * RS;
-    float *out = a.out[blockIdx.z];
     const int ntiles = (n + 16 * NRB - 1) / (16 * NRB);
-    const int t0 = (int)((int64_t)blockIdx.x * ntiles / a.parts), t1 = (int)((int64_t)(blockIdx.x + 1) * ntiles / a.parts);
-    const int my = t1 - t0;
     const int64_t w_bytes = (int64_t)n * RS;
+    // what the workgroup works on: expert e, tensor, tiles t0 .. t0 + my - 1 of the expert's matrix (its own share first; then, where
+    // a list of further passes exists, whatever it draws from that list)
+    const uint8_t *w;
+    float *out;
+    int t0, my;
+    auto place = [&](int ee, int tensor, int part, int nparts) {
+        e = ee;
+        w = a.w[tensor] + (int64_t)ee * n * RS;
+        out = a.out[tensor];
+        t0 = (int)((int64_t)part * ntiles / nparts);
+        my = (int)((int64_t)(part + 1) * ntiles / nparts) - t0;
+    };
+    place(blockIdx.y, blockIdx.z, blockIdx.x, a.parts);
+    __shared__ int drawn;
     int seq = 0;                                                           // tiles asked for so far, over all passes: the ring slot
     auto issue = [&](int i) {                                              // tile t0 + i of this pass (nothing beyond the range)
         const bool live = i < my;
@@ -750,14 +763,12 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
     // depend on it.  An expert without pairs waits for those copies and leaves.
     issue(0);
     asm volatile("" ::: "memory");
-    const int seg0 = a.dense_rows ? 0 : a.offsets[e], seg1 = a.dense_rows ? a.dense_rows : a.offsets[e + 1];
-    if (seg0 >= seg1) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        return;
-    }
-    const int nsets = (seg1 - seg0 + 15) >> 4;
-    for (int sg = 0; sg < nsets; sg += QME_NS) {
-        // (a second pass starts behind the barrier that ended the first: every tile of the ring is free)
+    int seg0 = a.dense_rows ? 0 : a.offsets[e], seg1 = a.dense_rows ? a.dense_rows : a.offsets[e + 1];
+    const int n_extra = a.extra ? a.extra[0] : 0;
+    // one pass over tiles t0 .. of expert e's matrix against sets sg, sg + 1 of its pairs; issued0: the first tile is on its way
+    auto run_pass = [&](const int sg, const bool issued0) {
+        const int nsets = (seg1 - seg0 + 15) >> 4;
+        // (a pass starts behind the barrier that ended the one before: every tile of the ring is free)
         const int sets_here = min(QME_NS, nsets - sg);
         // The records of the pass (block sums and scales of every pair and column) go to LDS by copy instructions ahead of the
         // first tile, whose wait covers them: loaded by every lane from memory they were 2/3 of the wave's operand requests,
@@ -773,7 +784,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (cq_lds_void *)(recs + (live ? st * REC_KB + piece : QME_NS * REC_KB) * 1024), 16, lane * 16,
                                                      piece * 1024, 0, 0);
         }
-        if (sg > 0) issue(0);
+        if (!issued0) issue(0);
         asm volatile("" ::: "memory");
         int rounds[QME_NS];                                                // results per lane a set needs: ceil(pairs / 4)
 #pragma unroll
@@ -914,6 +925,32 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
         }
         // the copies beyond the range carried no bytes, but they count: nothing may be outstanding when the next pass counts again
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+    if (seg0 >= seg1) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // (the first tile of an expert without pairs: wait, then nothing)
+    } else if (a.extra) {
+        run_pass(0, true);
+    } else {
+        for (int sg = 0; 16 * sg < seg1 - seg0; sg += QME_NS) run_pass(sg, sg == 0);
+    }
+    // Further passes of experts with more than 32 pairs: (expert, pass) items x tensors x parts, drawn from a counter by whichever
+    // workgroup has finished what it had, in pieces finer than a workgroup's own share (a router is rarely balanced: with a static
+    // split the launch would wait for the workgroups of its most loaded expert).  Every draw is one atomic; the loop ends with the first draw beyond the list.
+    if (n_extra > 0) {
+        const int per_item = a.extra_parts * (int)gridDim.z, total = n_extra * per_item;
+        for (;;) {
+            if (tid == 0) drawn = __hip_atomic_fetch_add(a.extra + 1 + a.extra_slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            const int idx = drawn;
+            if (idx >= total) break;
+            const int item = idx / per_item, rem = idx - item * per_item;
+            place(a.extra[CQ_MOE_EXTRA_HEADER + 2 * item], rem / a.extra_parts, rem % a.extra_parts, a.extra_parts);
+            seg0 = a.offsets[e];
+            seg1 = a.offsets[e + 1];
+            // (every wave has read `drawn` before any of them passes the first barrier of the pass, and thread 0 writes it again
+            // only behind the last one)
+            run_pass(a.extra[CQ_MOE_EXTRA_HEADER + 2 * item + 1] * QME_NS, false);
+        }
     }
 #ifdef CL_STAMPS
     QB_STAMP(15);
@@ -1051,12 +1088,12 @@ int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *ro
 static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s);
 // out_a[pair_out[p]][:] = (W_a[expert of p] . x^[p]) * pair_scale[p] for every sorted pair p; the same for (w_b, out_b) when given
 int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
-                         const float *pair_scale, int64_t num_experts, int64_t k, int64_t n, hipStream_t s) {
+                         const float *pair_scale, int *extra, int launch_slot, int64_t num_experts, int64_t k, int64_t n, hipStream_t s) {
     const int bpr = (int)(k / 256), tensors = w_b ? 2 : 1;
     QmeArgs a;
     a.w[0] = (const uint8_t *)w_a; a.w[1] = (const uint8_t *)w_b; a.out[0] = out_a; a.out[1] = out_b;
     a.op = (const uint8_t *)op; a.offsets = offsets; a.pair_out = pair_out; a.pair_scale = pair_scale; a.n = (int)n; a.bpr = bpr;
-    a.dense_rows = 0;
+    a.dense_rows = 0; a.extra = extra; a.extra_slot = launch_slot;
     return qme_launch(a, num_experts, tensors, s);
 }
 
@@ -1074,6 +1111,10 @@ static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t 
     // (every part the same number of tiles where that is possible: 896 tiles are 224 parts of 4, not 256 of 3 or 4)
     if (parts > 1) parts = (ntiles + (ntiles + parts - 1) / parts - 1) / ((ntiles + parts - 1) / parts);
     a.parts = (int)parts;
+    // a listed pass in pieces of about eight tiles: short enough to spread over the workgroups that have finished, long enough for
+    // the five microseconds until a piece's first tile is there
+    const int64_t tiles_per_part = (ntiles + parts - 1) / parts;
+    a.extra_parts = (int)(parts * std::max<int64_t>(1, tiles_per_part / 8));
     switch (cw) {
         case 8: return launch_qme<8, 2>(a, num_experts, tensors, s);
         case 4: return launch_qme<4, 2>(a, num_experts, tensors, s);
@@ -1109,7 +1150,7 @@ int cq_matvec_batch_mid_launch(const void *w, const float *x, const float *up, i
     QmeArgs a;
     a.w[0] = (const uint8_t *)w; a.w[1] = nullptr; a.out[0] = dst; a.out[1] = nullptr;
     a.op = (const uint8_t *)workspace; a.offsets = nullptr; a.pair_out = nullptr; a.pair_scale = nullptr; a.n = (int)n; a.bpr = bpr;
-    a.dense_rows = (int)rows;
+    a.dense_rows = (int)rows; a.extra = nullptr; a.extra_slot = 0;
     return qme_launch(a, 1, 1, s);
 }
 
@@ -1117,7 +1158,7 @@ int cq_matvec_batch_mid_launch(const void *w, const float *x, const float *up, i
 extern "C" int qme_debug_launch(const void *w, float *out, const void *op, const int *offsets, const int *pout, const float *pscale, int64_t experts,
                                 int64_t k, int64_t n, uint32_t *stamps, void *stream) {
     hipMemcpyToSymbol(HIP_SYMBOL(qme_stamps), &stamps, sizeof(stamps));
-    return cq_moe_stream_launch(w, nullptr, out, nullptr, op, offsets, pout, pscale, experts, k, n, (hipStream_t)stream);
+    return cq_moe_stream_launch(w, nullptr, out, nullptr, op, offsets, pout, pscale, nullptr, 0, experts, k, n, (hipStream_t)stream);
 }
 extern "C" int qb_debug_launch(const void *w, const void *x, void *workspace, void *dst, int64_t k, int64_t n, int64_t rows, void *stream) {
     return cq_matvec_batch_launch(CQ_Q4K, w, x, CQ_F32, workspace, dst, CQ_F32, k, n, rows, n, (hipStream_t)stream);

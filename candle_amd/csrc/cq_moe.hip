@@ -24,7 +24,7 @@
 namespace {
 
 struct MoeWorkspace {
-    int64_t act_off, offsets_off, cursor_off, pin_off, pout_off, pscale_off, chunk_off, max_chunks, rows_alloc, total;
+    int64_t act_off, offsets_off, cursor_off, pin_off, pout_off, pscale_off, chunk_off, max_chunks, rows_alloc, extra_off, total;
 };
 
 inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t x_rows, int64_t k) {
@@ -42,7 +42,9 @@ inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pa
     w.pout_off = w.pin_off + cq_align256(n_pairs * 4);
     w.pscale_off = w.pout_off + cq_align256(n_pairs * 4);
     w.chunk_off = w.pscale_off + cq_align256(n_pairs * 4);
-    w.total = w.chunk_off + cq_align256((3 * w.max_chunks + 1) * 4);      // n_chunks | expert[] | first[] | count[]
+    w.extra_off = w.chunk_off + cq_align256((3 * w.max_chunks + 1) * 4);  // n_chunks | expert[] | first[] | count[]
+    // further passes of the experts with more than 32 pairs, for the batched-matvec form: n | two counters | (expert, pass)[]
+    w.total = w.extra_off + cq_align256((CQ_MOE_EXTRA_HEADER + 2 * (n_pairs / 32 + 1)) * 4);
     return w;
 }
 
@@ -54,8 +56,8 @@ template <bool LC>
 __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__restrict__ offsets, int *__restrict__ cursor,
                                                          int *__restrict__ pair_in, int *__restrict__ pair_out,
                                                          float *__restrict__ pair_scale, float *__restrict__ out, int n, int *__restrict__ chunks,
-                                                         int max_chunks, int chunk) {
-    __shared__ int carry, n_chunks;
+                                                         int max_chunks, int chunk, int *__restrict__ extra) {
+    __shared__ int carry, n_chunks, n_extra;
     __shared__ int buf[1024];
     __shared__ int lcur[LC ? GROUP_LDS_EXPERTS : 1];
     int *cur = LC ? lcur : cursor;
@@ -79,7 +81,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
         float scale;
         if (pair_decode(ps, p, e, in_row, out_row, scale)) atomicAdd(&cur[e], 1);
     }
-    if (tid == 0) { carry = 0; n_chunks = 0; }
+    if (tid == 0) { carry = 0; n_chunks = 0; n_extra = 0; }
     __syncthreads();
     // exclusive scan of the counts, 1024 experts per sweep (only as many doubling steps as the sweep is wide)
     for (int base = 0; base < E; base += 1024) {
@@ -99,6 +101,16 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
             offsets[e] = start;
             cur[e] = start;
             // chunk table: expert e's segment in pieces of `chunk` pairs (any order: chunks are independent)
+            // (the batched-matvec form takes 32 pairs of an expert per pass over its weights: every further pass is an item of a
+            // list that the workgroups of that launch share out among themselves once their own pass is done)
+            if (extra && c > 32) {
+                const int np = (c + 31) / 32 - 1;
+                const int eb = atomicAdd(&n_extra, np);
+                for (int i = 0; i < np; i++) {
+                    extra[CQ_MOE_EXTRA_HEADER + 2 * (eb + i)] = e;
+                    extra[CQ_MOE_EXTRA_HEADER + 2 * (eb + i) + 1] = i + 1;
+                }
+            }
             const int cc = (c + chunk - 1) / chunk;
             if (cc > 0) {
                 const int cb = atomicAdd(&n_chunks, cc);
@@ -113,7 +125,11 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(PairSource ps, int *__r
         if (tid == width - 1) carry += buf[tid];              // the inclusive sum of the sweep
         __syncthreads();
     }
-    if (tid == 0) { offsets[E] = carry; chunks[0] = n_chunks; }
+    if (tid == 0) {
+        offsets[E] = carry;
+        chunks[0] = n_chunks;
+        if (extra) { extra[0] = n_extra; extra[1] = 0; extra[2] = 0; }         // the list's length, and the two launches' counters
+    }
     // positions behind the last valid pair are never part of a chunk, but the gathering quantizer walks all n_pairs
     // rows: give them a valid source row
     for (int p = carry + tid; p < ps.n_pairs; p += 1024) pair_in[p] = 0;
@@ -244,7 +260,8 @@ int cq_moe_down_after_pair_launch(int w_dtype, const void *w_down, const float *
         const int *chunks = (const int *)(b + ws.chunk_off);
         int rc = cq_moe_stream_quantize_launch(gate, up, pout, topk_weights, pscale, chunks, ws.max_chunks, num_experts, n_pairs, offsets, b + ws.act_off, k, s);
         if (rc) return rc;
-        return cq_moe_stream_launch(w_down, nullptr, out, nullptr, b + ws.act_off, offsets, pout, pscale, num_experts, k, n, s);
+        return cq_moe_stream_launch(w_down, nullptr, out, nullptr, b + ws.act_off, offsets, pout, pscale, (int *)(b + ws.extra_off), 1,
+                                    num_experts, k, n, s);
     }
     // the rows of this call are quantized into the front of the workspace: they must end before that call's tables begin
     if (cq_act_layout(w_dtype, k, ws.rows_alloc).total > ws.offsets_off) return CQ_ERR_RANGE;
@@ -293,20 +310,21 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     int *pin = (int *)(b + ws.pin_off), *pout = (int *)(b + ws.pout_off);
     float *pscale = (float *)(b + ws.pscale_off);
     int *chunks = (int *)(b + ws.chunk_off);
+    int *extra = (int *)(b + ws.extra_off);
     // Hundreds of pairs per call: the expert-sorted rows go through the MFMA prefill kernel of the format in tiles of up to
     // 128 rows of one expert (integer-exact like the dense paths).  Otherwise 8 pairs per matvec pass.
     const int tile_rows = moe_tile_rows(a.n_pairs, a.num_experts);
     if (a.num_experts <= GROUP_LDS_EXPERTS)
         hipLaunchKernelGGL(moe_group_kernel<true>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
-                           (int)ws.max_chunks, stream ? CQ_MOE_STREAM_CHUNK : mfma ? tile_rows : CQ_MOE_CHUNK);
+                           (int)ws.max_chunks, stream ? CQ_MOE_STREAM_CHUNK : mfma ? tile_rows : CQ_MOE_CHUNK, stream ? extra : nullptr);
     else
         hipLaunchKernelGGL(moe_group_kernel<false>, dim3(1), dim3(1024), 0, s, ps, offsets, cursor, pin, pout, pscale, a.out, (int)a.n, chunks,
-                           (int)ws.max_chunks, stream ? CQ_MOE_STREAM_CHUNK : mfma ? tile_rows : CQ_MOE_CHUNK);
+                           (int)ws.max_chunks, stream ? CQ_MOE_STREAM_CHUNK : mfma ? tile_rows : CQ_MOE_CHUNK, stream ? extra : nullptr);
     if ((rc = (int)hipGetLastError())) return rc;
     if (stream) {
         // every expert a batched matvec over its own pairs: the weights of an expert are streamed once per 32 pairs
         if ((rc = cq_moe_stream_quantize_launch(a.x, nullptr, pin, nullptr, nullptr, chunks, ws.max_chunks, a.num_experts, a.n_pairs, offsets, b + ws.act_off, a.k, s))) return rc;
-        return cq_moe_stream_launch(a.w, a.w_b, a.out, a.out_b, b + ws.act_off, offsets, pout, pscale, a.num_experts, a.k, a.n, s);
+        return cq_moe_stream_launch(a.w, a.w_b, a.out, a.out_b, b + ws.act_off, offsets, pout, pscale, extra, 0, a.num_experts, a.k, a.n, s);
     }
     if (mfma) {
         if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;

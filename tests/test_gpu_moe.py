@@ -142,6 +142,34 @@ def test_moe_gemm_gguf_mfma_tile_sizes(dtype, E, n):
     assert err <= TIGHT, err
 
 
+@pytest.mark.parametrize("k,n", [(2048, 96), (768, 203)])
+def test_moe_gemm_gguf_one_expert_draws_most_pairs(k, n):
+    """A router far from balanced: one expert with 300 of 432 pairs (ten passes over its weights, of which nine are shared out
+    among the workgroups of the launch as they finish), two with 40, the rest with none or a few."""
+    import candle_amd as ca
+    counts = [300, 40, 40, 0, 0, 7, 0, 1, 0, 12, 0, 0, 0, 3, 0, 29]
+    E, topk = len(counts), 2
+    n_pairs = sum(counts)
+    assert n_pairs % topk == 0 and 257 <= n_pairs <= 64 * E
+    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=95)
+    rng = np.random.Generator(np.random.PCG64(96))
+    expert_ids = np.repeat(np.arange(E, dtype=np.int32), counts)
+    sorted_token_ids = rng.permutation(n_pairs).astype(np.int32)
+    x = normal(97, (n_pairs, k), 1.0)
+    tw = rng.uniform(0.1, 1.0, n_pairs).astype(np.float32)
+    got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, torch.from_numpy(tw).cuda(), torch.from_numpy(sorted_token_ids).cuda(),
+                           torch.from_numpy(expert_ids).cuda(), topk, True)
+    torch.cuda.synchronize()
+    want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, tw, topk)
+    got = got.cpu().numpy()
+    for p in range(n_pairs):
+        assert rel_l2(got[p], want[p]) <= 1e-5, p
+    # a second call on the same workspace draws from counters that the grouping pass has set back to zero
+    got2 = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, torch.from_numpy(tw).cuda(), torch.from_numpy(sorted_token_ids).cuda(),
+                            torch.from_numpy(expert_ids).cuda(), topk, True).cpu().numpy()
+    assert np.array_equal(got, got2)
+
+
 def test_moe_gemm_gguf_q4k_rows_too_long_for_the_batched_form():
     """Q4_K experts with rows of more than 16 super-blocks do not run as batched matvecs: 25 pairs per expert go through the
     32-row tiles of the Q4_K matrix-core kernel."""
