@@ -346,15 +346,16 @@ def moe(args):
     L = _lib.lib()
     dev = torch.device("cuda:0")
     E, H, F, TOPK, NL = 128, 2048, 768, 8, args.moe_layers
+    wdt, block_bytes, _ = WDTYPES[args.wdtype]              # (--wdtype: the experts' format, Q4_K unless given)
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
-    gate = [quantized_weight(L, torch, Q4K, E * F, H, gen, dev) for _ in range(NL)]
-    up = [quantized_weight(L, torch, Q4K, E * F, H, gen, dev) for _ in range(NL)]
-    down = [quantized_weight(L, torch, Q4K, E * H, F, gen, dev) for _ in range(NL)]
+    gate = [quantized_weight(L, torch, wdt, E * F, H, gen, dev) for _ in range(NL)]
+    up = [quantized_weight(L, torch, wdt, E * F, H, gen, dev) for _ in range(NL)]
+    down = [quantized_weight(L, torch, wdt, E * H, F, gen, dev) for _ in range(NL)]
     router = torch.randn((E, H), generator=gen, device=dev)
 
     def qt(buf, n, k):
-        return QTensor.new(QStorage(buf, GgmlDType.Q4K), (E, n, k))
+        return QTensor.new(QStorage(buf, GgmlDType(wdt)), (E, n, k))
 
     fused = [FusedMoeGGUF(router, qt(gate[i], F, H), qt(up[i], F, H), qt(down[i], H, F), True, TOPK) for i in range(NL)]
     reps, warm = max(1, (MIN_TIMED_LAUNCHES + NL - 1) // NL), max(1, (MIN_WARMUP_LAUNCHES + NL - 1) // NL)
@@ -368,12 +369,12 @@ def moe(args):
         h = torch.randn((tokens, TOPK, F), generator=gen, device=dev)
         o1, o2 = torch.empty((tokens, TOPK, F), device=dev), torch.empty((tokens, TOPK, F), device=dev)
         o3 = torch.empty((tokens, TOPK, H), device=dev)
-        nws = max(L.cq_indexed_moe_workspace_bytes(Q4K, E, F, H, tokens, TOPK, 1), L.cq_indexed_moe_workspace_bytes(Q4K, E, H, F, tokens, TOPK, TOPK))
+        nws = max(L.cq_indexed_moe_workspace_bytes(wdt, E, F, H, tokens, TOPK, 1), L.cq_indexed_moe_workspace_bytes(wdt, E, H, F, tokens, TOPK, TOPK))
         ws = torch.empty(nws, dtype=torch.uint8, device=dev)
 
         def layer(i, sp):
             for w, src, dst, n, k, d1 in ((gate[i], xg, o1, F, H, 1), (up[i], xg, o2, F, H, 1), (down[i], h, o3, H, F, TOPK)):
-                _lib.check("cq_indexed_moe_forward", L.cq_indexed_moe_forward(Q4K, w.data_ptr(), src.data_ptr(), ids32.data_ptr(), dst.data_ptr(),
+                _lib.check("cq_indexed_moe_forward", L.cq_indexed_moe_forward(wdt, w.data_ptr(), src.data_ptr(), ids32.data_ptr(), dst.data_ptr(),
                                                                               E, n, k, tokens, TOPK, d1, ws.data_ptr(), nws, sp))
 
         st = torch.cuda.Stream(device=dev)
@@ -405,17 +406,17 @@ def moe(args):
         # the whole layer as FusedMoeGGUF::forward runs it: router + softmax + top-k, sort by expert, three grouped
         # matmuls (moe_gemm_gguf), silu(gate) * up, sum over top-k
         fused_us, fst = timed(lambda i: fused[i].forward(x3, tokens > 1, out=y))
-        alg = distinct * 3 * 884736
+        alg = distinct * 3 * (F * H // 256) * block_bytes
         results.append({"tokens": tokens, "distinct_experts": distinct, "layer_us": round(us, 1), "layer_median_us": round(ust["median"], 1),
                         "layer_p10_us": round(ust["p10"], 1), "layer_p90_us": round(ust["p90"], 1), "algorithmic_MB": round(alg / 1e6, 1),
                         "GBps": round(alg / us / 1e3, 1), "frac_of_hbm_peak": round(alg / us / 1e3 / HBM_PEAK_GBPS, 4),
                         "fused_moe_layer_us": round(fused_us, 1), "fused_moe_layer_median_us": round(fst["median"], 1),
                         "tok_s_%d_layers_fused" % NL: round(tokens / (NL * fused_us * 1e-6), 1), "timed_layer_launches": reps * NL})
-    out = {"metric": "Qwen3-30B-A3B-shape MoE layer, expert matmuls (Q4_K, 128 experts, top-8)", "unit": "us per layer", "n_gpus": 1,
+    out = {"metric": "Qwen3-30B-A3B-shape MoE layer, expert matmuls (%s, 128 experts, top-8)" % FMT_NAMES[args.wdtype], "unit": "us per layer", "n_gpus": 1,
            "data": "synthetic", "config": {"workload": "gate + up [tokens, 2048] -> 768 and down [tokens*8, 768] -> 2048 via indexed_moe_forward, "
                                                        "%d layers with distinct weights (%.1f GB) in one HIP graph; fused_moe_layer_us: the same "
                                                        "layers through FusedMoeGGUF::forward (router, top-k, sort, moe_gemm_gguf x3, "
-                                                       "silu*up, sum over top-k)" % (NL, NL * 3 * E * F * H * 0.5625 / 1e9), "layers": NL},
+                                                       "silu*up, sum over top-k)" % (NL, NL * 3 * E * (F * H // 256) * block_bytes / 1e9), "layers": NL},
            "results": results}
     del gate, up, down, fused
     torch.cuda.empty_cache()
@@ -703,7 +704,7 @@ def other_configurations(L, torch, args):
                         "roofline_tok_s": r["roofline"]["roofline_tok_s_weights_only"],
                         "weight_bytes_per_token": r["weight_bytes_per_token"], "workload": r["config"]["workload"]}
     # cfg5: the 48-layer MoE stack
-    mo = moe(argparse.Namespace(moe_layers=48, moe_tokens="1,16,256"))
+    mo = moe(argparse.Namespace(moe_layers=48, moe_tokens="1,16,256", wdtype="q4k"))
     out["moe"] = {"workload": mo["config"]["workload"], "results": mo["results"]}
     return out
 

@@ -232,7 +232,7 @@ int cq_qmatmul_forward(int w_dtype, const void *w_dev, const void *x_dev, int x_
         return cq_matvec_batch_launch(w_dtype, w_dev, x_dev, x_dtype, workspace_dev, dst_dev, dst_dtype, k, n, m, n, s);
     // 17..64 rows of Q4_K (rows of up to 4096 elements): the same formulation, the rows in sets of 16
     if (m > 16 && cq_matvec_batch_mid_takes(w_dtype, w_dev, x_dev, x_dtype, dst_dtype, k, n, m))
-        return cq_matvec_batch_mid_launch(w_dev, (const float *)x_dev, nullptr, k, 0, workspace_dev, (float *)dst_dev, k, n, m, s);
+        return cq_matvec_batch_mid_launch(w_dtype, w_dev, (const float *)x_dev, nullptr, k, 0, workspace_dev, (float *)dst_dev, k, n, m, s);
     // 3..8 rows: every workgroup re-quantizing all rows costs more than one small kernel that does it once
     if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) {
         if ((rc = cq_quantize_act_launch(w_dtype, x_dev, x_dtype, workspace_dev, k, m, s))) return rc;
@@ -284,7 +284,7 @@ int cq_nn_qmatmul_swiglu_rows(int w_dtype, const void *w_dev, const float *gate_
     if (m >= 3 && cq_matvec_batch_takes(w_dtype, w_dev, k, n, m))          // the kernel cq_qmatmul_forward takes for these shapes
         return cq_matvec_batch_swiglu_launch(w_dtype, w_dev, gate_dev, up_dev, gate_stride, up_stride, workspace_dev, dst_dev, CQ_F32, k, n, m, n, s);
     if (m > 16 && cq_matvec_batch_mid_takes(w_dtype, w_dev, gate_dev, CQ_F32, CQ_F32, k, n, m))
-        return cq_matvec_batch_mid_launch(w_dev, gate_dev, up_dev, gate_stride, up_stride, workspace_dev, dst_dev, k, n, m, s);
+        return cq_matvec_batch_mid_launch(w_dtype, w_dev, gate_dev, up_dev, gate_stride, up_stride, workspace_dev, dst_dev, k, n, m, s);
     if ((rc = cq_quantize_act_swiglu_launch(w_dtype, gate_dev, up_dev, gate_stride, up_stride, workspace_dev, k, m, s))) return rc;
     if (m <= CQ_MATVEC_MAX_ROWS && !cq_use_mfma(w_dtype, m, k)) return cq_matvec_launch(w_dtype, w_dev, workspace_dev, dst_dev, CQ_F32, k, n, m, n, s);
     float *tmp = (float *)((uint8_t *)workspace_dev + cq_act_layout(w_dtype, k, m).total);

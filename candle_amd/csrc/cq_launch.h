@@ -22,7 +22,7 @@ int cq_matvec_batch_launch(int w_dtype, const void *w, const void *x, int x_dtyp
 // 17 .. 64 f32 rows of Q4_K with rows of up to 16 super-blocks: the rows in sets of 16, two sets per pass over the weights
 bool cq_matvec_batch_mid_takes(int w_dtype, const void *w, const void *x, int x_dtype, int dst_dtype, int64_t k, int64_t n, int64_t rows);
 int64_t cq_matvec_batch_mid_workspace(int w_dtype, int64_t k, int64_t rows);
-int cq_matvec_batch_mid_launch(const void *w, const float *x, const float *up, int64_t x_stride, int64_t up_stride, void *workspace, float *dst,
+int cq_matvec_batch_mid_launch(int w_dtype, const void *w, const float *x, const float *up, int64_t x_stride, int64_t up_stride, void *workspace, float *dst,
                                int64_t k, int64_t n, int64_t rows, hipStream_t s);      // up != nullptr: rows silu(x[r]) * up[r]
 int cq_matvec_batch_swiglu_launch(int w_dtype, const void *w, const float *gate, const float *up, int64_t gate_stride, int64_t up_stride, void *workspace,
                                   void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s);
@@ -164,7 +164,7 @@ int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *ro
 // extra: n | counter of launch 0 | counter of launch 1 | (expert, pass)[n]: the passes beyond the first of the experts with more than
 // 32 pairs, written (counters zero) by the grouping pass; launch_slot: which counter this launch counts with
 #define CQ_MOE_EXTRA_HEADER 3
-int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
+int cq_moe_stream_launch(int w_dtype, const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
                          const float *pair_scale, int *extra, int launch_slot, int64_t num_experts, int64_t k, int64_t n, hipStream_t s);
 
 // Pairs from which a K-quant MoE call goes through the MFMA kernel (tiles of expert-sorted rows): everything the

@@ -52,11 +52,17 @@ typedef long i64x2 __attribute__((ext_vector_type(2)));
 
 constexpr int QB_NW = 8;
 constexpr int QB_BB = 144;                        // bytes of a Q4_K super-block
+// Q5_K is Q4_K with a fifth bit per weight: the same 16-byte header (d, dmin, 6-bit scales and minima), then qh[32] (bit j of
+// byte l: the fifth bit of element l of sub-block j), then the nibbles.  The kernels of this file take both (template flag Q5):
+// the fifth bits of a lane's eight elements of all eight sub-blocks are one 8-byte read, and a sub-block's operand is
+// nibbles | (bits << 4), values 0 .. 31.
+template <bool Q5> struct QbW { static constexpr int BB = Q5 ? 176 : 144, QS = Q5 ? 48 : 16; };
+__host__ __device__ constexpr int qb_bb(bool q5) { return q5 ? 176 : 144; }
 constexpr int QB_RED_BYTES = QB_NW * 64 * 16;     // the waves' partial results of one block of rows
 constexpr int QB_LDS_BYTES = 160 * 1024;
 // A tile (16 rows of up to 8 * CPW super-blocks) is copied by whole instructions of 64 lanes x 16 bytes, each wave the same number:
 // it occupies a multiple of 8 KB.
-constexpr int qb_tile_instr(int cpw) { return (16 * 8 * cpw * QB_BB + 8 * 1024 - 1) / (8 * 1024); }       // copy instructions per wave and tile
+constexpr int qb_tile_instr(int cpw, int bb = QB_BB) { return (16 * 8 * cpw * bb + 8 * 1024 - 1) / (8 * 1024); }       // copy instructions per wave and tile
 // In LDS every KB of a tile is followed by 16 unused bytes: a row is 9 * 16 * (super-blocks per row) bytes, for rows of 16
 // super-blocks a multiple of all 64 banks, and the 16 lanes that read the same bytes of 16 different rows would meet on one bank.
 constexpr int QB_KB = 1024 + 16;
@@ -126,14 +132,15 @@ constexpr int QB_FQ_REC = 32;                      // bytes of a staged record {
 __host__ __device__ constexpr int qb_fq_col_bytes(int fq) { return fq * 256 + fq * QB_FQ_REC; }      // operands + records of one column
 // NR: results per lane that the batch needs, ceil(rows / 4) (a template parameter: behind a run-time bound every result is a basic
 // block of its own, and 16 rows lose 0.7 us)
-template <int CPW, int DEPTH, int FQ, int NR = (FQ + 3) / 4>
+template <int CPW, int DEPTH, int FQ, int NR = (FQ + 3) / 4, bool Q5 = false>
 __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ op, void *__restrict__ dst, int n, int bpr,
                                                               int rows, int dst_dtype, int64_t stride_dst
 #ifdef CL_STAMPS
                                                               , uint32_t *stamps
 #endif
                                                               ) {
-    constexpr int NIW = qb_tile_instr(CPW);       // copy instructions per wave and tile (those beyond the block copy nothing)
+    constexpr int BB = QbW<Q5>::BB, QS = QbW<Q5>::QS;
+    constexpr int NIW = qb_tile_instr(CPW, BB);   // copy instructions per wave and tile (those beyond the block copy nothing)
     static_assert((DEPTH - 1) * NIW <= 63 && DEPTH >= 2, "counted waits");
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -142,7 +149,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
     const int c = lane & 15, kg = lane >> 4;
     const int col0 = wv * CPW;
     const int ncols = max(0, min(CPW, bpr - col0));
-    const int RS = bpr * QB_BB;                   // bytes of a row, in memory and in a tile
+    const int RS = bpr * BB;                   // bytes of a row, in memory and in a tile
     const int block_bytes = 16 * RS;
     const int nkb = (block_bytes + 1023) >> 10;   // KBs of a tile
     const int TILE = qb_tile_bytes(block_bytes);
@@ -298,15 +305,21 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
 #pragma unroll
         for (int ci = 0; ci < CPW; ci++) {
             if (ci < ncols) {
-                const int o = c * RS + (col0 + ci) * QB_BB;                  // weight row c of the block, this column's super-block
+                const int o = c * RS + (col0 + ci) * BB;                  // weight row c of the block, this column's super-block
                 auto at = [&](int off) { return tile + off + (off >> 10) * 16; };      // byte `off` of the block in the padded tile
                 const u32x4 hdr = *(const u32x4 *)at(o);
                 i32x4 cl[4], ch[4];
+                long qh = 0;
+                if constexpr (Q5) qh = *(const long *)at(o + 16 + 8 * kg);       // fifth bits of elements 8kg .. 8kg + 7, bit j: sub-block j
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     // bytes 32g + 8kg .. + 7 of qs: low nibbles = sub-block 2g, high nibbles = sub-block 2g + 1
-                    const long qa = *(const long *)at(o + 16 + 32 * g + 8 * kg);
-                    const long lo = qa & 0x0f0f0f0f0f0f0f0fl, hi = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                    const long qa = *(const long *)at(o + QS + 32 * g + 8 * kg);
+                    long lo = qa & 0x0f0f0f0f0f0f0f0fl, hi = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                    if constexpr (Q5) {
+                        lo |= ((qh >> (2 * g)) & 0x0101010101010101l) << 4;
+                        hi |= ((qh >> (2 * g + 1)) & 0x0101010101010101l) << 4;
+                    }
                     const i32x4 z = {0, 0, 0, 0};
                     cl[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[ci][2 * g], lo, z, 0, 0, 0);
                     ch[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[ci][2 * g + 1], hi, z, 0, 0, 0);
@@ -361,7 +374,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
 // one chunk, gathered by the copy instructions from 16 row segments), wave w owns columns 2 w, 2 w + 1 of EVERY chunk and
 // keeps their int8 operands in registers (Q x 2 x 16 registers), and the per-row records (block sums, scale) wait in LDS.
 // The accumulators run across the chunks of a block; everything else is the kernel above.
-template <int Q, int NR>
+template <int Q, int NR, bool Q5 = false>
 __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ op, void *__restrict__ dst, int n,
                                                                    int bpr, int rows, int dst_dtype, int64_t stride_dst, int cpp
 #ifdef CL_STAMPS
@@ -369,7 +382,8 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
 #endif
                                                                    ) {
     constexpr int CPW = 2, DEPTH = 3;
-    constexpr int NIW = qb_tile_instr(CPW);
+    constexpr int BB = QbW<Q5>::BB, QS = QbW<Q5>::QS;
+    constexpr int NIW = qb_tile_instr(CPW, BB);
     static_assert((DEPTH - 1) * NIW <= 63, "counted waits");
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -377,9 +391,9 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, kg = lane >> 4;
     const int col0 = wv * CPW;                    // the wave's first column inside a chunk
-    const int RS = bpr * QB_BB;                   // bytes of a row in memory
+    const int RS = bpr * BB;                   // bytes of a row in memory
     const int block_bytes = 16 * RS;
-    const int TILE = qb_tile_bytes(16 * cpp * QB_BB);
+    const int TILE = qb_tile_bytes(16 * cpp * BB);
     const int last_cols = bpr - (Q - 1) * cpp;    // columns of the last chunk (1 .. cpp)
     float *red = (float *)(lds + DEPTH * TILE);                              // [8 waves][64 lanes][4]
     uint8_t *recs = (uint8_t *)red + QB_RED_BYTES;                           // [bpr][16 batch slots] records
@@ -394,9 +408,9 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
 #pragma unroll
     for (int t = 0; t < NIW; t++) {
         const int tb = (t * QB_NW + wv) * 1024 + lane * 16;
-        const int rf = tb / (cpp * QB_BB), rl = tb / (last_cols * QB_BB);
-        voff_full[t] = rf < 16 ? rf * RS + (tb - rf * cpp * QB_BB) : block_bytes;            // beyond the tile: out of range, zeros
-        voff_last[t] = rl < 16 ? rl * RS + (tb - rl * last_cols * QB_BB) : block_bytes;
+        const int rf = tb / (cpp * BB), rl = tb / (last_cols * BB);
+        voff_full[t] = rf < 16 ? rf * RS + (tb - rf * cpp * BB) : block_bytes;            // beyond the tile: out of range, zeros
+        voff_last[t] = rl < 16 ? rl * RS + (tb - rl * last_cols * BB) : block_bytes;
     }
     // (Every workgroup takes the chunks in the same order.  Rotating the order by workgroup, so that the launch reads all column
     // ranges of the tensor at any moment instead of the same quarter of every row, was measured a third slower.)
@@ -405,12 +419,12 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
         const int m = bx + i * gx;
         const bool live = tau < ntiles;
         const int pc = q == Q - 1 ? last_cols : cpp;
-        const int64_t off = live ? (int64_t)m * block_bytes + q * cpp * QB_BB : 0;
+        const int64_t off = live ? (int64_t)m * block_bytes + q * cpp * BB : 0;
         const int64_t left = w_bytes - off;
         const int bytes = live ? (int)(left < block_bytes ? left : block_bytes) : 0;      // an absent tile: a descriptor of zero bytes
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(w + off), 0, bytes, 0x00020000);
         uint8_t *tile = lds + (tau % DEPTH) * TILE;
-        const int nkb = (16 * pc * QB_BB + 1023) >> 10;
+        const int nkb = (16 * pc * BB + 1023) >> 10;
 #pragma unroll
         for (int t = 0; t < NIW; t++) {
             const int kb = min(t * QB_NW + wv, nkb);             // KB number nkb: beyond the tile, nothing read, zeros into the spare KB
@@ -465,18 +479,24 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
             const uint8_t *tile = lds + (tau % DEPTH) * TILE;
             if (tau < 4) QB_STAMP(2 + 3 * tau);
             const int pc = q == Q - 1 ? last_cols : cpp;
-            const int TRS = pc * QB_BB;
+            const int TRS = pc * BB;
 #pragma unroll
             for (int ci = 0; ci < CPW; ci++) {
                 if (col0 + ci < pc) {
-                    const int o = c * TRS + (col0 + ci) * QB_BB;                 // weight row c of the block, this column's super-block
+                    const int o = c * TRS + (col0 + ci) * BB;                 // weight row c of the block, this column's super-block
                     auto at = [&](int off) { return tile + off + (off >> 10) * 16; };      // byte `off` of the tile in its padded form
                     const u32x4 hdr = *(const u32x4 *)at(o);
                     i32x4 cl[4], ch[4];
+                    long qh = 0;
+                    if constexpr (Q5) qh = *(const long *)at(o + 16 + 8 * kg);
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const long qa = *(const long *)at(o + 16 + 32 * g + 8 * kg);
-                        const long lo = qa & 0x0f0f0f0f0f0f0f0fl, hi = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                        const long qa = *(const long *)at(o + QS + 32 * g + 8 * kg);
+                        long lo = qa & 0x0f0f0f0f0f0f0f0fl, hi = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                        if constexpr (Q5) {
+                            lo |= ((qh >> (2 * g)) & 0x0101010101010101l) << 4;
+                            hi |= ((qh >> (2 * g + 1)) & 0x0101010101010101l) << 4;
+                        }
                         const i32x4 z = {0, 0, 0, 0};
                         cl[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[q][ci][2 * g], lo, z, 0, 0, 0);
                         ch[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(A[q][ci][2 * g + 1], hi, z, 0, 0, 0);
@@ -530,13 +550,15 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
 #endif
 }
 
-template <int Q, int NR>
+// LDS of the chunked-row kernel: three tiles of a chunk, the partial results, the records of a whole row of operands
+constexpr size_t qb_long_lds(int64_t bpr, int cpp, int bb) { return (size_t)3 * qb_tile_bytes(16 * cpp * bb) + QB_RED_BYTES + (size_t)bpr * 16 * QB_REC_BYTES; }
+template <int Q, int NR, bool Q5>
 int launch_qmb_long_r(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int cpp,
                       hipStream_t s) {
     const int64_t bpr = k / 256;
-    const size_t lds_bytes = (size_t)3 * qb_tile_bytes(16 * cpp * QB_BB) + QB_RED_BYTES + (size_t)bpr * 16 * QB_REC_BYTES;
+    const size_t lds_bytes = qb_long_lds(bpr, cpp, qb_bb(Q5));
     if (lds_bytes > (size_t)QB_LDS_BYTES - 1024) return CQ_ERR_RANGE;
-    auto kern = qmb_q4k_long_kernel<Q, NR>;
+    auto kern = qmb_q4k_long_kernel<Q, NR, Q5>;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     const int64_t nsteps = (n + 15) / 16;
@@ -551,21 +573,21 @@ int launch_qmb_long_r(const void *w, const uint8_t *op, void *dst, int dst_dtype
     return (int)hipGetLastError();
 }
 
-template <int Q>
+template <int Q, bool Q5>
 int launch_qmb_long(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int cpp,
                     hipStream_t s) {
     switch ((rows + 3) / 4) {
-        case 1: return launch_qmb_long_r<Q, 1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
-        case 2: return launch_qmb_long_r<Q, 2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
-        case 3: return launch_qmb_long_r<Q, 3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
-        default: return launch_qmb_long_r<Q, 4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+        case 1: return launch_qmb_long_r<Q, 1, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+        case 2: return launch_qmb_long_r<Q, 2, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+        case 3: return launch_qmb_long_r<Q, 3, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+        default: return launch_qmb_long_r<Q, 4, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
     }
 }
 
-template <int CPW, int DEPTH, int FQ, int NR>
+template <int CPW, int DEPTH, int FQ, int NR, bool Q5>
 int launch_qmb_dr(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
                   hipStream_t s) {
-    auto kern = qmb_q4k_kernel<CPW, DEPTH, FQ, NR>;
+    auto kern = qmb_q4k_kernel<CPW, DEPTH, FQ, NR, Q5>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
@@ -581,29 +603,29 @@ int launch_qmb_dr(const void *w, const uint8_t *op, void *dst, int dst_dtype, in
     );
     return (int)hipGetLastError();
 }
-template <int CPW, int DEPTH, int FQ = 0>
+template <int CPW, int DEPTH, bool Q5, int FQ = 0>
 int launch_qmb_d(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, size_t lds_bytes,
                  hipStream_t s) {
-    if constexpr (FQ > 0) return launch_qmb_dr<CPW, DEPTH, FQ, (FQ + 3) / 4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+    if constexpr (FQ > 0) return launch_qmb_dr<CPW, DEPTH, FQ, (FQ + 3) / 4, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
     switch ((rows + 3) / 4) {
-        case 1: return launch_qmb_dr<CPW, DEPTH, 0, 1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
-        case 2: return launch_qmb_dr<CPW, DEPTH, 0, 2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
-        case 3: return launch_qmb_dr<CPW, DEPTH, 0, 3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
-        default: return launch_qmb_dr<CPW, DEPTH, 0, 4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+        case 1: return launch_qmb_dr<CPW, DEPTH, 0, 1, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+        case 2: return launch_qmb_dr<CPW, DEPTH, 0, 2, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+        case 3: return launch_qmb_dr<CPW, DEPTH, 0, 3, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
+        default: return launch_qmb_dr<CPW, DEPTH, 0, 4, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, lds_bytes, s);
     }
 }
 // Three tiles where LDS holds them (the one being worked on and two on their way), else two.  (Four were measured slower:
 // with three tiles asked for at the start the first one lands 1 us later, and the steady state gains nothing.)
 // fq: `op` holds the f32 activations (see the kernel); the caller has checked qb_fused_rows
-template <int CPW>
+template <int CPW, bool Q5>
 int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, int fq, hipStream_t s) {
-    const int tile = qb_tile_bytes((int)(16 * (k / 256) * QB_BB));
+    const int tile = qb_tile_bytes((int)(16 * (k / 256) * qb_bb(Q5)));
     const int fit = (QB_LDS_BYTES - QB_RED_BYTES - 1024) / tile;
 #define QB_FQ_CASE(R)                                                                                                                           \
     case R:                                                                                                                                    \
         if constexpr (CPW * R <= QB_FQ_MAX_SPANS) {                                                                                            \
-            if (fit >= 3) return launch_qmb_d<CPW, 3, R>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)3 * tile + QB_RED_BYTES, s);  \
-            if (fit == 2) return launch_qmb_d<CPW, 2, R>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)2 * tile + QB_RED_BYTES, s);  \
+            if (fit >= 3) return launch_qmb_d<CPW, 3, Q5, R>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)3 * tile + QB_RED_BYTES, s);  \
+            if (fit == 2) return launch_qmb_d<CPW, 2, Q5, R>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)2 * tile + QB_RED_BYTES, s);  \
         }                                                                                                                                      \
         return CQ_ERR_RANGE;
     switch (fq) {
@@ -611,8 +633,8 @@ int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64
         default: break;
     }
 #undef QB_FQ_CASE
-    if (fit >= 3) return launch_qmb_d<CPW, 3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)3 * tile + QB_RED_BYTES, s);
-    if (fit == 2) return launch_qmb_d<CPW, 2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)2 * tile + QB_RED_BYTES, s);
+    if (fit >= 3) return launch_qmb_d<CPW, 3, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)3 * tile + QB_RED_BYTES, s);
+    if (fit == 2) return launch_qmb_d<CPW, 2, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, (size_t)2 * tile + QB_RED_BYTES, s);
     return CQ_ERR_RANGE;
 }
 
@@ -707,10 +729,11 @@ constexpr int QME_NS = 2;         // sets of 16 pairs per pass over the weights
 constexpr int QME_MAX_AVG_PAIRS = 64;   // pairs per expert on average up to which a call takes this form
 constexpr int QME_DEPTH = 4;      // tiles of the ring where LDS holds them
 
-template <int CW, int CPW, int DEPTH>
+template <int CW, int CPW, int DEPTH, bool Q5 = false>
 __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
+    constexpr int BB = QbW<Q5>::BB, QS = QbW<Q5>::QS;
     constexpr int NRB = QB_NW / CW;                                        // row blocks of a tile
-    constexpr int NIW = (16 * NRB * CW * CPW * QB_BB + 8 * 1024 - 1) / (8 * 1024);      // copy instructions per wave and tile
+    constexpr int NIW = (16 * NRB * CW * CPW * BB + 8 * 1024 - 1) / (8 * 1024);      // copy instructions per wave and tile
     static_assert((DEPTH - 1) * NIW <= 63 && DEPTH >= 2, "counted waits");
     extern __shared__ __align__(16) uint8_t lds[];
     int e = blockIdx.y;
@@ -721,7 +744,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
     const int rb = wv / CW, col0 = (wv % CW) * CPW;
     const int n = a.n, bpr = a.bpr;
     const int ncols = max(0, min(CPW, bpr - col0));
-    const int RS = bpr * QB_BB;
+    const int RS = bpr * BB;
     const int block_bytes = 16 * NRB * RS;
     const int nkb = (block_bytes + 1023) >> 10;
     const int TILE = qb_tile_bytes(block_bytes);
@@ -867,14 +890,20 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
 #pragma unroll
             for (int ci = 0; ci < CPW; ci++) {
                 if (ci < ncols) {
-                    const int o = (rb * 16 + c) * RS + (col0 + ci) * QB_BB;
+                    const int o = (rb * 16 + c) * RS + (col0 + ci) * BB;
                     auto at = [&](int off) { return tile + off + (off >> 10) * 16; };
                     const u32x4 hdr = *(const u32x4 *)at(o);
                     long lo[4], hi[4];
+                    long qh = 0;
+                    if constexpr (Q5) qh = *(const long *)at(o + 16 + 8 * kg);       // fifth bits of elements 8kg .. 8kg + 7, bit j: sub-block j
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const long qa = *(const long *)at(o + 16 + 32 * g + 8 * kg);
+                        const long qa = *(const long *)at(o + QS + 32 * g + 8 * kg);
                         lo[g] = qa & 0x0f0f0f0f0f0f0f0fl; hi[g] = (qa >> 4) & 0x0f0f0f0f0f0f0f0fl;
+                        if constexpr (Q5) {
+                            lo[g] |= ((qh >> (2 * g)) & 0x0101010101010101l) << 4;
+                            hi[g] |= ((qh >> (2 * g + 1)) & 0x0101010101010101l) << 4;
+                        }
                     }
                     const QsScales s = qs_scales_k4(hdr.y, hdr.z, hdr.w);
                     int sc[8];
@@ -959,9 +988,9 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
 #endif
 }
 
-template <int CW, int CPW, int DEPTH>
+template <int CW, int CPW, int DEPTH, bool Q5>
 int launch_qme_d(const QmeArgs &a, int64_t num_experts, int tensors, size_t lds_bytes, hipStream_t s) {
-    auto kern = qme_q4k_kernel<CW, CPW, DEPTH>;
+    auto kern = qme_q4k_kernel<CW, CPW, DEPTH, Q5>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
@@ -969,57 +998,65 @@ int launch_qme_d(const QmeArgs &a, int64_t num_experts, int tensors, size_t lds_
     hipLaunchKernelGGL(kern, dim3((unsigned)a.parts, (unsigned)num_experts, (unsigned)tensors), dim3(QB_NW * 64), lds_bytes, s, a);
     return (int)hipGetLastError();
 }
-template <int CW, int CPW>
+template <int CW, int CPW, bool Q5>
 int launch_qme(const QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s) {
-    const int tile = qb_tile_bytes(16 * (QB_NW / CW) * a.bpr * QB_BB);
+    const int tile = qb_tile_bytes(16 * (QB_NW / CW) * a.bpr * qb_bb(Q5));
     const int red = 2 * QME_NS * QB_RED_BYTES + (QME_NS * ((CW * CPW * 16 * QB_REC_BYTES + 1023) / 1024) + 1) * 1024;      // partial results, records
     const int fit = (QB_LDS_BYTES - red - 1024) / tile;
-    if (fit >= QME_DEPTH) return launch_qme_d<CW, CPW, QME_DEPTH>(a, num_experts, tensors, (size_t)QME_DEPTH * tile + red, s);
-    if (fit >= 3) return launch_qme_d<CW, CPW, 3>(a, num_experts, tensors, (size_t)3 * tile + red, s);
-    if (fit == 2) return launch_qme_d<CW, CPW, 2>(a, num_experts, tensors, (size_t)2 * tile + red, s);
+    if (fit >= QME_DEPTH) return launch_qme_d<CW, CPW, QME_DEPTH, Q5>(a, num_experts, tensors, (size_t)QME_DEPTH * tile + red, s);
+    if (fit >= 3) return launch_qme_d<CW, CPW, 3, Q5>(a, num_experts, tensors, (size_t)3 * tile + red, s);
+    if (fit == 2) return launch_qme_d<CW, CPW, 2, Q5>(a, num_experts, tensors, (size_t)2 * tile + red, s);
     return CQ_ERR_RANGE;
 }
 
 }  // namespace
 
-// Does the batched matrix-core matvec take this call?  Q4_K, 3 .. 16 rows, rows of up to 64 super-blocks (k <= 16384: up to 24
-// with three columns per wave, beyond that in up to four column chunks, which is what a wave's registers hold of a row).
+// Does the batched matrix-core matvec take this call?  Q4_K or Q5_K, 3 .. 16 rows, rows of up to 64 super-blocks (k <= 16384:
+// up to 24 with three columns per wave, beyond that in up to four column chunks, which is what a wave's registers hold of a
+// row; Q5_K's larger tiles leave room for the records of up to 56 super-blocks beside them).
 constexpr int QB_MAX_BPR = 64;        // (and 64 x 16 records of 32 bytes are 4 pieces of 16 bytes per thread)
+static bool qb_weights(int w_dtype) { return w_dtype == CQ_Q4K || w_dtype == CQ_Q5K; }
+// the chunked-row kernel's split of a row: chunks of at most 16 super-blocks, all about the same size
+static int qb_long_cpp(int64_t bpr) { const int64_t chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW); return (int)((bpr + chunks - 1) / chunks); }
+static bool qb_row_fits(int w_dtype, int64_t bpr) {
+    return bpr >= 1 && bpr <= QB_MAX_BPR && (bpr <= 3 * QB_NW || qb_long_lds(bpr, qb_long_cpp(bpr), qb_bb(w_dtype == CQ_Q5K)) <= (size_t)QB_LDS_BYTES - 1024);
+}
 bool cq_matvec_batch_takes(int w_dtype, const void *w, int64_t k, int64_t n, int64_t rows) {
     // (three rows over chunked rows: the register-blocked matvec is still ahead there, 15.1 against 16.8 us on [4096 x 14336])
     if (k / 256 > 3 * QB_NW && rows < 4) return false;
-    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= QB_MAX_BPR && n >= 1 && n <= 0x7ffffff0 / 16 &&
-           n * (k / 256) * QB_BB < 0x7fffffffLL && ((uintptr_t)w & 15) == 0;
+    return qb_weights(w_dtype) && rows >= 3 && rows <= 16 && k % 256 == 0 && qb_row_fits(w_dtype, k / 256) && n >= 1 && n <= 0x7ffffff0 / 16 &&
+           n * (k / 256) * qb_bb(w_dtype == CQ_Q5K) < 0x7fffffffLL && ((uintptr_t)w & 15) == 0;
 }
 // bytes of workspace the call needs (the activations as matrix operands); 0 when the shape can never take this path
 int64_t cq_matvec_batch_workspace(int w_dtype, int64_t k, int64_t rows) {
-    return w_dtype == CQ_Q4K && rows >= 3 && rows <= 16 && k % 256 == 0 && k / 256 <= QB_MAX_BPR ? cq_align256(qb_operand_bytes(k / 256)) : 0;
+    return qb_weights(w_dtype) && rows >= 3 && rows <= 16 && k % 256 == 0 && qb_row_fits(w_dtype, k / 256) ? cq_align256(qb_operand_bytes(k / 256)) : 0;
 }
 
 // Rows the main kernel quantizes itself (= rows), 0: the quantize kernel runs first.  Contiguous f32 rows of up to
 // 24 super-blocks, at most 8 of them and at most QB_FQ_MAX_SPANS spans per wave, and the staged operands of the eight waves
 // must fit one tile of the ring.
-static int qb_fused_rows(int x_dtype, const void *x, int64_t x_stride, int64_t k, int64_t rows) {
+static int qb_fused_rows(int w_dtype, int x_dtype, const void *x, int64_t x_stride, int64_t k, int64_t rows) {
     const int64_t bpr = k / 256, cpw = (bpr + QB_NW - 1) / QB_NW;
     if (x_dtype != CQ_F32 || x_stride != k || bpr > 3 * QB_NW || rows > 8 || cpw * rows > QB_FQ_MAX_SPANS || ((uintptr_t)x & 15)) return 0;
     const int fq = (int)rows;
-    const int tile = qb_tile_bytes((int)(16 * bpr * QB_BB));
+    const int tile = qb_tile_bytes((int)(16 * bpr * qb_bb(w_dtype == CQ_Q5K)));
     if ((QB_LDS_BYTES - QB_RED_BYTES - 1024) / tile < 2) return 0;
     return QB_NW * cpw * qb_fq_col_bytes(fq) <= tile ? fq : 0;
 }
 
 // QMatMul::forward for 3 .. 16 rows of x: one small kernel quantizes them into `workspace`, then the weights are read once.
 // x_dtype < 0: the rows are silu(x) * up, f32, with row strides in floats (multiples of 4).
-static int qb_launch(int w_dtype, const void *w, const void *x, const float *up, int64_t x_stride, int64_t up_stride, int x_dtype, void *workspace,
-                     void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+template <bool Q5>
+static int qb_launch_w(int w_dtype, const void *w, const void *x, const float *up, int64_t x_stride, int64_t up_stride, int x_dtype, void *workspace,
+                       void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
     if (!cq_matvec_batch_takes(w_dtype, w, k, n, rows)) return CQ_ERR_RANGE;
     const int bpr = (int)(k / 256);
     const int64_t cpw = (k / 256 + QB_NW - 1) / QB_NW;
-    if (const int fq = qb_fused_rows(x_dtype, x, x_stride, k, rows)) {
+    if (const int fq = qb_fused_rows(w_dtype, x_dtype, x, x_stride, k, rows)) {
         switch (cpw) {
-            case 1: return launch_qmb<1>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
-            case 2: return launch_qmb<2>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
-            case 3: return launch_qmb<3>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
+            case 1: return launch_qmb<1, Q5>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
+            case 2: return launch_qmb<2, Q5>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
+            case 3: return launch_qmb<3, Q5>(w, (const uint8_t *)x, dst, dst_dtype, k, n, rows, stride_dst, fq, s);
             default: return CQ_ERR_RANGE;
         }
     }
@@ -1033,20 +1070,25 @@ static int qb_launch(int w_dtype, const void *w, const void *x, const float *up,
         default: return CQ_ERR_DTYPE;
     }
     if (bpr > 3 * QB_NW) {
-        const int chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW), cpp = (bpr + chunks - 1) / chunks;
+        const int chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW), cpp = qb_long_cpp(bpr);
         switch (chunks) {
-            case 2: return launch_qmb_long<2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
-            case 3: return launch_qmb_long<3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
-            case 4: return launch_qmb_long<4>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+            case 2: return launch_qmb_long<2, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+            case 3: return launch_qmb_long<3, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
+            case 4: return launch_qmb_long<4, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
             default: return CQ_ERR_RANGE;
         }
     }
     switch (cpw) {
-        case 1: return launch_qmb<1>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
-        case 2: return launch_qmb<2>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
-        case 3: return launch_qmb<3>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
+        case 1: return launch_qmb<1, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
+        case 2: return launch_qmb<2, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
+        case 3: return launch_qmb<3, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, 0, s);
         default: return CQ_ERR_RANGE;
     }
+}
+static int qb_launch(int w_dtype, const void *w, const void *x, const float *up, int64_t x_stride, int64_t up_stride, int x_dtype, void *workspace,
+                     void *dst, int dst_dtype, int64_t k, int64_t n, int64_t rows, int64_t stride_dst, hipStream_t s) {
+    return w_dtype == CQ_Q5K ? qb_launch_w<true>(w_dtype, w, x, up, x_stride, up_stride, x_dtype, workspace, dst, dst_dtype, k, n, rows, stride_dst, s)
+                             : qb_launch_w<false>(w_dtype, w, x, up, x_stride, up_stride, x_dtype, workspace, dst, dst_dtype, k, n, rows, stride_dst, s);
 }
 int cq_matvec_batch_launch(int w_dtype, const void *w, const void *x, int x_dtype, void *workspace, void *dst, int dst_dtype, int64_t k, int64_t n,
                            int64_t rows, int64_t stride_dst, hipStream_t s) {
@@ -1058,12 +1100,12 @@ int cq_matvec_batch_swiglu_launch(int w_dtype, const void *w, const float *gate,
 }
 
 // ---- MoE: experts as batched matvecs (see qme_q4k_kernel) ----
-// Q4_K experts of rows up to 16 super-blocks (two columns per wave: three do not fit the registers next to two operand sets),
+// Q4_K or Q5_K experts of rows up to 16 super-blocks (two columns per wave: three do not fit the registers next to two operand sets),
 // 16-byte aligned, and on average at most 64 pairs per expert: beyond that a pass over the weights per 32 pairs loses to the
 // tiles that reuse a weight 32 or 128 times.
 bool cq_moe_stream_shape(int w_dtype, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n) {
-    return w_dtype == CQ_Q4K && k % 256 == 0 && k / 256 <= 2 * QB_NW && n >= 1 && n <= 0x7ffffff0 / 16 && num_experts >= 1 && num_experts <= 65535 &&
-           n_pairs <= QME_MAX_AVG_PAIRS * num_experts && n * (k / 256) * QB_BB < 0x7fffffffLL;
+    return qb_weights(w_dtype) && k % 256 == 0 && k / 256 <= 2 * QB_NW && n >= 1 && n <= 0x7ffffff0 / 16 && num_experts >= 1 && num_experts <= 65535 &&
+           n_pairs <= QME_MAX_AVG_PAIRS * num_experts && n * (k / 256) * qb_bb(w_dtype == CQ_Q5K) < 0x7fffffffLL;
 }
 bool cq_moe_stream_takes(int w_dtype, const void *w, const void *w_b, int64_t num_experts, int64_t n_pairs, int64_t k, int64_t n) {
     return cq_moe_stream_shape(w_dtype, num_experts, n_pairs, k, n) && ((uintptr_t)w & 15) == 0 && ((uintptr_t)w_b & 15) == 0;
@@ -1085,20 +1127,21 @@ int cq_moe_stream_quantize_launch(const float *x, const float *up, const int *ro
                            (int)max_chunks, offsets, (uint8_t *)op, (int)(k / 256), k, k);
     return (int)hipGetLastError();
 }
-static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s);
+static int qme_launch(QmeArgs &a, int w_dtype, int64_t num_experts, int tensors, hipStream_t s);
 // out_a[pair_out[p]][:] = (W_a[expert of p] . x^[p]) * pair_scale[p] for every sorted pair p; the same for (w_b, out_b) when given
-int cq_moe_stream_launch(const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
+int cq_moe_stream_launch(int w_dtype, const void *w_a, const void *w_b, float *out_a, float *out_b, const void *op, const int *offsets, const int *pair_out,
                          const float *pair_scale, int *extra, int launch_slot, int64_t num_experts, int64_t k, int64_t n, hipStream_t s) {
     const int bpr = (int)(k / 256), tensors = w_b ? 2 : 1;
     QmeArgs a;
     a.w[0] = (const uint8_t *)w_a; a.w[1] = (const uint8_t *)w_b; a.out[0] = out_a; a.out[1] = out_b;
     a.op = (const uint8_t *)op; a.offsets = offsets; a.pair_out = pair_out; a.pair_scale = pair_scale; a.n = (int)n; a.bpr = bpr;
     a.dense_rows = 0; a.extra = extra; a.extra_slot = launch_slot;
-    return qme_launch(a, num_experts, tensors, s);
+    return qme_launch(a, w_dtype, num_experts, tensors, s);
 }
 
 // the launch geometry of the expert kernel: waves per row block, parts per expert and tensor
-static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s) {
+template <bool Q5>
+static int qme_launch_w(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s) {
     const int bpr = a.bpr;
     const int64_t n = a.n;
     // waves that share a row block: the fewest (a power of two) with at most two columns each — large tiles: a tile costs about
@@ -1116,11 +1159,14 @@ static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t 
     const int64_t tiles_per_part = (ntiles + parts - 1) / parts;
     a.extra_parts = (int)(parts * std::max<int64_t>(1, tiles_per_part / 8));
     switch (cw) {
-        case 8: return launch_qme<8, 2>(a, num_experts, tensors, s);
-        case 4: return launch_qme<4, 2>(a, num_experts, tensors, s);
-        case 2: return launch_qme<2, 2>(a, num_experts, tensors, s);
-        default: return bpr == 2 ? launch_qme<1, 2>(a, num_experts, tensors, s) : launch_qme<1, 1>(a, num_experts, tensors, s);
+        case 8: return launch_qme<8, 2, Q5>(a, num_experts, tensors, s);
+        case 4: return launch_qme<4, 2, Q5>(a, num_experts, tensors, s);
+        case 2: return launch_qme<2, 2, Q5>(a, num_experts, tensors, s);
+        default: return bpr == 2 ? launch_qme<1, 2, Q5>(a, num_experts, tensors, s) : launch_qme<1, 1, Q5>(a, num_experts, tensors, s);
     }
+}
+static int qme_launch(QmeArgs &a, int w_dtype, int64_t num_experts, int tensors, hipStream_t s) {
+    return w_dtype == CQ_Q5K ? qme_launch_w<true>(a, num_experts, tensors, s) : qme_launch_w<false>(a, num_experts, tensors, s);
 }
 
 // ---- QMatMul::forward for 17 .. 64 rows: the matrix as the one expert of the kernel above, the rows as its pairs (two sets of 16
@@ -1128,14 +1174,14 @@ static int qme_launch(QmeArgs &a, int64_t num_experts, int tensors, hipStream_t 
 // (the 32-row / 128-row matrix-core tiles convert every weight for the rows of a tile: at these row counts that costs more than
 // scaling the results)
 bool cq_matvec_batch_mid_takes(int w_dtype, const void *w, const void *x, int x_dtype, int dst_dtype, int64_t k, int64_t n, int64_t rows) {
-    return w_dtype == CQ_Q4K && x_dtype == CQ_F32 && dst_dtype == CQ_F32 && rows > 16 && rows <= 64 &&
+    return qb_weights(w_dtype) && x_dtype == CQ_F32 && dst_dtype == CQ_F32 && rows > 16 && rows <= 64 &&
            cq_moe_stream_takes(w_dtype, w, nullptr, 1, rows, k, n) && ((uintptr_t)x & 15) == 0;
 }
 int64_t cq_matvec_batch_mid_workspace(int w_dtype, int64_t k, int64_t rows) {
-    return w_dtype == CQ_Q4K && rows > 16 && rows <= 64 && k % 256 == 0 && k / 256 <= 2 * QB_NW ? cq_align256(((rows + 15) / 16) * (k / 256) * QME_TILE_COL_BYTES) : 0;
+    return qb_weights(w_dtype) && rows > 16 && rows <= 64 && k % 256 == 0 && k / 256 <= 2 * QB_NW ? cq_align256(((rows + 15) / 16) * (k / 256) * QME_TILE_COL_BYTES) : 0;
 }
 // up != nullptr: the rows are silu(x[r]) * up[r], with row strides in floats
-int cq_matvec_batch_mid_launch(const void *w, const float *x, const float *up, int64_t x_stride, int64_t up_stride, void *workspace, float *dst,
+int cq_matvec_batch_mid_launch(int w_dtype, const void *w, const float *x, const float *up, int64_t x_stride, int64_t up_stride, void *workspace, float *dst,
                                int64_t k, int64_t n, int64_t rows, hipStream_t s) {
     const int bpr = (int)(k / 256);
     const dim3 grid((unsigned)((rows + 15) / 16), (unsigned)bpr);
@@ -1151,14 +1197,14 @@ int cq_matvec_batch_mid_launch(const void *w, const float *x, const float *up, i
     a.w[0] = (const uint8_t *)w; a.w[1] = nullptr; a.out[0] = dst; a.out[1] = nullptr;
     a.op = (const uint8_t *)workspace; a.offsets = nullptr; a.pair_out = nullptr; a.pair_scale = nullptr; a.n = (int)n; a.bpr = bpr;
     a.dense_rows = (int)rows; a.extra = nullptr; a.extra_slot = 0;
-    return qme_launch(a, 1, 1, s);
+    return qme_launch(a, w_dtype, 1, 1, s);
 }
 
 #ifdef CL_STAMPS
 extern "C" int qme_debug_launch(const void *w, float *out, const void *op, const int *offsets, const int *pout, const float *pscale, int64_t experts,
                                 int64_t k, int64_t n, uint32_t *stamps, void *stream) {
     hipMemcpyToSymbol(HIP_SYMBOL(qme_stamps), &stamps, sizeof(stamps));
-    return cq_moe_stream_launch(w, nullptr, out, nullptr, op, offsets, pout, pscale, nullptr, 0, experts, k, n, (hipStream_t)stream);
+    return cq_moe_stream_launch(CQ_Q4K, w, nullptr, out, nullptr, op, offsets, pout, pscale, nullptr, 0, experts, k, n, (hipStream_t)stream);
 }
 extern "C" int qb_debug_launch(const void *w, const void *x, void *workspace, void *dst, int64_t k, int64_t n, int64_t rows, void *stream) {
     return cq_matvec_batch_launch(CQ_Q4K, w, x, CQ_F32, workspace, dst, CQ_F32, k, n, rows, n, (hipStream_t)stream);

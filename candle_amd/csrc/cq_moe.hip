@@ -36,7 +36,7 @@ inline MoeWorkspace moe_workspace(int w_dtype, int64_t num_experts, int64_t n_pa
     w.max_chunks = n_pairs / CQ_MOE_CHUNK + (num_experts < n_pairs ? num_experts : n_pairs) + 1;
     w.offsets_off = cq_act_layout(w_dtype, k, w.rows_alloc > x_rows ? w.rows_alloc : x_rows).total;
     // (experts run as batched matvecs keep their pairs' rows as operand tiles instead)
-    if (w_dtype == CQ_Q4K && k % 256 == 0) w.offsets_off = std::max<int64_t>(w.offsets_off, cq_align256(cq_moe_stream_operand_bytes(num_experts, n_pairs, k)));
+    if ((w_dtype == CQ_Q4K || w_dtype == CQ_Q5K) && k % 256 == 0) w.offsets_off = std::max<int64_t>(w.offsets_off, cq_align256(cq_moe_stream_operand_bytes(num_experts, n_pairs, k)));
     w.cursor_off = w.offsets_off + cq_align256((num_experts + 1) * 4);
     w.pin_off = w.cursor_off + cq_align256(num_experts * 4);
     w.pout_off = w.pin_off + cq_align256(n_pairs * 4);
@@ -260,7 +260,7 @@ int cq_moe_down_after_pair_launch(int w_dtype, const void *w_down, const float *
         const int *chunks = (const int *)(b + ws.chunk_off);
         int rc = cq_moe_stream_quantize_launch(gate, up, pout, topk_weights, pscale, chunks, ws.max_chunks, num_experts, n_pairs, offsets, b + ws.act_off, k, s);
         if (rc) return rc;
-        return cq_moe_stream_launch(w_down, nullptr, out, nullptr, b + ws.act_off, offsets, pout, pscale, (int *)(b + ws.extra_off), 1,
+        return cq_moe_stream_launch(w_dtype, w_down, nullptr, out, nullptr, b + ws.act_off, offsets, pout, pscale, (int *)(b + ws.extra_off), 1,
                                     num_experts, k, n, s);
     }
     // the rows of this call are quantized into the front of the workspace: they must end before that call's tables begin
@@ -323,8 +323,9 @@ int cq_moe_launch(const MoeArgs &a, void *workspace, hipStream_t s) {
     if ((rc = (int)hipGetLastError())) return rc;
     if (stream) {
         // every expert a batched matvec over its own pairs: the weights of an expert are streamed once per 32 pairs
+        if (cq_align256(cq_moe_stream_operand_bytes(a.num_experts, a.n_pairs, a.k)) > ws.offsets_off) return CQ_ERR_RANGE;      // (the workspace layout above reserves it)
         if ((rc = cq_moe_stream_quantize_launch(a.x, nullptr, pin, nullptr, nullptr, chunks, ws.max_chunks, a.num_experts, a.n_pairs, offsets, b + ws.act_off, a.k, s))) return rc;
-        return cq_moe_stream_launch(a.w, a.w_b, a.out, a.out_b, b + ws.act_off, offsets, pout, pscale, extra, 0, a.num_experts, a.k, a.n, s);
+        return cq_moe_stream_launch(a.w_dtype, a.w, a.w_b, a.out, a.out_b, b + ws.act_off, offsets, pout, pscale, extra, 0, a.num_experts, a.k, a.n, s);
     }
     if (mfma) {
         if ((rc = cq_quantize_act_gather_launch(a.w_dtype, a.x, pin, b + ws.act_off, a.k, a.n_pairs, ws.rows_alloc, s))) return rc;

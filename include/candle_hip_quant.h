@@ -132,9 +132,9 @@ int cq_matmul(int w_dtype, const void *w_dev, const void *act_scratch_dev, float
 /* ---------------------------------------------------------------------------------------------
  * QCudaStorage::fwd (cuda.rs:846-878), the body of CustomOp1::cuda_fwd for QTensor
  * (mod.rs:1007-1017): quantize the m activation rows, then matvec (m <= CQ_MATVEC_MAX_ROWS; for m <= 2 the
- * quantization happens inside the matvec kernel; Q4K with 3 <= m <= 16, k a multiple of 256 up to 16384 and 16-byte
+ * quantization happens inside the matvec kernel; Q4K / Q5K with 3 <= m <= 16, k a multiple of 256 up to 16384 (Q5K: 14336) and 16-byte
  * aligned weights: one pass over the weights on the int8 matrix cores with the rows as register operands, up to 8 f32 rows of
- * up to 6144 elements quantized inside that kernel; Q4K with 17 <= m <= 64 f32 rows of up to 4096 elements to an f32 dst: the
+ * up to 6144 elements quantized inside that kernel; Q4K / Q5K with 17 <= m <= 64 f32 rows of up to 4096 elements to an f32 dst: the
  * same with the rows in sets of 16, one pass over the weights per 32 rows) or MFMA matmul
  * (split over k with an ordered reduction when the grid would be small).  x is [m, k] contiguous (f32 / f16 / bf16), dst is [m, n] contiguous in dst_dtype
  * (CUDA keeps the input dtype: fast_mmvq.rs:161-323).  workspace_dev: 256-byte aligned,
@@ -173,7 +173,7 @@ int cq_qmatmul_forward_static(int w_dtype, const void *w_dev, const void *x_dev,
  *   ids [batch, topk] u32  ->  out [batch, topk, n] f32,
  *   out[b, t, :] = W[ids[b, t]] . x[b, input_dim1 == 1 ? 0 : t, :].
  * Up to 256 pairs (512 for short rows, see cq_moe_direct_pairs) each pair is its own fused matvec; beyond, pairs are grouped by expert on the device and an expert's
- * rows are streamed once per 32 of its pairs as a batched matvec (Q4K experts with rows of up to 4096 elements that see at
+ * rows are streamed once per 32 of its pairs as a batched matvec (Q4K / Q5K experts with rows of up to 4096 elements that see at
  * most 64 pairs each on average), once per tile of 32 or 128 pairs on the matrix cores (K-quant experts; integer-exact) or once per
  * 8 pairs by the matvec kernel (the other formats).  The reference takes Q2K-Q6K and Q8_0 experts (cuda.rs:543-548).
  * An id >= num_experts leaves its output row zero-filled.
@@ -203,10 +203,10 @@ int cq_moe_gemm_gguf(int w_dtype, const float *x_dev, const void *w_dev, const i
 /* Two moe_gemm_gguf calls without topk_weights over the same x and the same pairs — the gate and up matmuls of
  * FusedMoeGGUF::forward (candle-transformers/src/fused_moe.rs:263-276) — as one call: out_a = x W_a^T, out_b = x W_b^T per
  * pair, results identical to two cq_moe_gemm_gguf calls.  With more than 256 pairs on K-quant experts the pairs are
- * grouped by expert and the activations quantized once for both (Q4_K experts that see at most 64 pairs each on average, rows
+ * grouped by expert and the activations quantized once for both (Q4_K / Q5_K experts that see at most 64 pairs each on average, rows
  * up to 4096 elements: both tensors in one launch, every expert a batched matvec over its own pairs); otherwise it is the two
  * calls.  w_a / w_b [num_experts, n, k] of one format; workspace as cq_moe_gemm_workspace_bytes(..., has_topk_weights = 0).
- * CQ_ERR_ALIGN when such Q4_K experts are not 16-byte aligned (a later cq_moe_gemm_gguf_down_after_pair tells from the shape
+ * CQ_ERR_ALIGN when such experts are not 16-byte aligned (a later cq_moe_gemm_gguf_down_after_pair tells from the shape
  * alone how this call grouped its pairs). */
 int cq_moe_gemm_gguf_pair(int w_dtype, const float *x_dev, const void *w_a_dev, const void *w_b_dev, const int32_t *sorted_token_ids_dev,
                           const int32_t *expert_ids_dev, float *out_a_dev, float *out_b_dev, int64_t num_experts, int64_t topk, int64_t size_m,

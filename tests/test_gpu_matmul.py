@@ -88,15 +88,16 @@ def test_matvec_k_sweep(dtype, k):
     assert rel_l2(got, want) <= TIGHT
 
 
+@pytest.mark.parametrize("wdt", [oracle.Q4K, oracle.Q5K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("k", [256, 768, 2560, 4096, 6144, 8192, 11008, 14336])
 @pytest.mark.parametrize("n,batch", [(203, 3), (203, 16), (5, 4), (16, 11), (17, 13), (1024, 9)])
-def test_q4k_batched_rows_vs_oracle(k, n, batch):
-    """3 .. 16 rows of Q4_K take the batched matrix-core matvec (16 weight rows per block, K split over the waves in
+def test_q4k_batched_rows_vs_oracle(wdt, k, n, batch):
+    """3 .. 16 rows of Q4_K or Q5_K take the batched matrix-core matvec (16 weight rows per block, K split over the waves in
     1 .. 7 super-block columns each): ragged n, fewer rows than a block, every column count, idle waves (k = 256, 768)."""
-    blocks, qmm = make_weight(oracle.Q4K, n, k, seed=131)
+    blocks, qmm = make_weight(wdt, n, k, seed=131)
     x = normal(132 + batch, (batch, k), 1.0)
     got = forward(qmm, x)
-    want = oracle.matmul_fast(oracle.Q4K, x, blocks, n, 8)
+    want = oracle.matmul_fast(wdt, x, blocks, n, 8)
     err = rel_l2(got, want)
     assert err <= TOL and err <= TIGHT, f"rel-L2 {err}"
     # row by row as well: a wrong batch column would hide in the norm of 16 rows
@@ -104,14 +105,15 @@ def test_q4k_batched_rows_vs_oracle(k, n, batch):
         assert rel_l2(got[r], want[r]) <= TIGHT, r
 
 
+@pytest.mark.parametrize("wdt", [oracle.Q4K, oracle.Q5K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("k", [256, 2048, 4096, 6144])
 @pytest.mark.parametrize("rows", [3, 4, 5, 6, 8])
-def test_q4k_batched_rows_quantized_inside_the_kernel(k, rows):
+def test_q4k_batched_rows_quantized_inside_the_kernel(wdt, k, rows):
     """Few f32 rows are quantized by the waves of the matvec kernel itself (up to 16 spans per wave), more rows by a kernel
     of their own: a row gives the same bits either way, and both agree with the oracle.  The rows hold what the two
     quantizers treat differently inside: a largest value that is negative, a tie between +max and -max, an all-zero span."""
     n = 203
-    blocks, qmm = make_weight(oracle.Q4K, n, k, seed=171)
+    blocks, qmm = make_weight(wdt, n, k, seed=171)
     x = normal(172 + rows, (rows, k), 1.0)
     x[0, :256] = 0.0
     x[1, 5] = -9.0
@@ -122,22 +124,23 @@ def test_q4k_batched_rows_quantized_inside_the_kernel(k, rows):
     got = forward(qmm, x)
     ref = forward(qmm, big)[:rows]
     assert np.array_equal(got, ref)
-    want = oracle.matmul_fast(oracle.Q4K, x, blocks, n, 8)
+    want = oracle.matmul_fast(wdt, x, blocks, n, 8)
     for r in range(rows):
         assert rel_l2(got[r], want[r]) <= TIGHT, r
 
 
+@pytest.mark.parametrize("wdt", [oracle.Q4K, oracle.Q5K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("k", [256, 768, 2048, 4096])
 @pytest.mark.parametrize("n,rows", [(203, 17), (203, 32), (96, 33), (50, 47), (130, 64)])
-def test_q4k_rows_in_sets_of_16_vs_oracle(k, n, rows):
-    """17 .. 64 f32 rows of Q4_K (rows of up to 4096 elements) run as sets of 16 rows, two sets per pass over the weights: a
+def test_q4k_rows_in_sets_of_16_vs_oracle(wdt, k, n, rows):
+    """17 .. 64 f32 rows of Q4_K or Q5_K (rows of up to 4096 elements) run as sets of 16 rows, two sets per pass over the weights: a
     partly filled second set, a second pass with one set and with two, ragged n, one to eight waves per row block."""
-    blocks, qmm = make_weight(oracle.Q4K, n, k, seed=181)
+    blocks, qmm = make_weight(wdt, n, k, seed=181)
     x = normal(182 + rows, (rows, k), 1.0)
     x[0, :256] = 0.0
     x[rows - 1, k - 3] = -7.5
     got = forward(qmm, x)
-    want = oracle.matmul_fast(oracle.Q4K, x, blocks, n, 8)
+    want = oracle.matmul_fast(wdt, x, blocks, n, 8)
     err = rel_l2(got, want)
     assert err <= TOL and err <= TIGHT, f"rel-L2 {err}"
     for r in range(rows):

@@ -87,10 +87,11 @@ def test_moe_gemm_gguf_gate_and_down(dtype, tokens, is_prefill):
     assert err2 <= TOL and err2 <= TIGHT, err2
 
 
+@pytest.mark.parametrize("wdt", [oracle.Q4K, oracle.Q5K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("k,n", [(256, 64), (512, 40), (768, 203), (1024, 130), (1792, 50), (2048, 96), (2304, 33), (4096, 72)])
 @pytest.mark.parametrize("with_weights", [False, True])
-def test_moe_gemm_gguf_experts_as_batched_matvecs(k, n, with_weights):
-    """Q4_K experts hit by at most 64 pairs on average run as batched matvecs over their own pairs (sets of 16, two sets per pass
+def test_moe_gemm_gguf_experts_as_batched_matvecs(wdt, k, n, with_weights):
+    """Q4_K or Q5_K experts hit by at most 64 pairs on average run as batched matvecs over their own pairs (sets of 16, two sets per pass
     over the weights).  Expert loads on every edge: none, one pair, 15 / 16 / 17, 31 / 32 / 33 (a second pass), 47 .. 49, 65 (a
     third pass); rows of 1 .. 16 super-blocks (one to eight waves per row block, columns without a wave's second column), ragged
     n, several workgroups per expert."""
@@ -100,7 +101,7 @@ def test_moe_gemm_gguf_experts_as_batched_matvecs(k, n, with_weights):
     n_pairs = sum(counts)
     assert n_pairs % topk == 0 and 257 <= n_pairs <= 64 * E
     tokens = n_pairs // topk
-    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=91)
+    blocks, qt = make_experts(wdt, E, n, k, seed=91)
     rng = np.random.Generator(np.random.PCG64(92))
     expert_ids = np.repeat(np.arange(E, dtype=np.int32), counts)
     sorted_token_ids = rng.permutation(n_pairs).astype(np.int32)
@@ -114,7 +115,7 @@ def test_moe_gemm_gguf_experts_as_batched_matvecs(k, n, with_weights):
         tw = None
         got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, None, sti, eid, topk, True)
     torch.cuda.synchronize()
-    want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, tw, topk)
+    want = oracle.moe_gemm_gguf(wdt, x, blocks, (E, n, k), sorted_token_ids, expert_ids, tw, topk)
     got = got.cpu().numpy()
     assert got.shape == (n_pairs, n)
     err = rel_l2(got, want)
@@ -142,8 +143,9 @@ def test_moe_gemm_gguf_mfma_tile_sizes(dtype, E, n):
     assert err <= TIGHT, err
 
 
+@pytest.mark.parametrize("wdt", [oracle.Q4K, oracle.Q5K], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("k,n", [(2048, 96), (768, 203)])
-def test_moe_gemm_gguf_one_expert_draws_most_pairs(k, n):
+def test_moe_gemm_gguf_one_expert_draws_most_pairs(wdt, k, n):
     """A router far from balanced: one expert with 300 of 432 pairs (ten passes over its weights, of which nine are shared out
     among the workgroups of the launch as they finish), two with 40, the rest with none or a few."""
     import candle_amd as ca
@@ -151,7 +153,7 @@ def test_moe_gemm_gguf_one_expert_draws_most_pairs(k, n):
     E, topk = len(counts), 2
     n_pairs = sum(counts)
     assert n_pairs % topk == 0 and 257 <= n_pairs <= 64 * E
-    blocks, qt = make_experts(oracle.Q4K, E, n, k, seed=95)
+    blocks, qt = make_experts(wdt, E, n, k, seed=95)
     rng = np.random.Generator(np.random.PCG64(96))
     expert_ids = np.repeat(np.arange(E, dtype=np.int32), counts)
     sorted_token_ids = rng.permutation(n_pairs).astype(np.int32)
@@ -160,7 +162,7 @@ def test_moe_gemm_gguf_one_expert_draws_most_pairs(k, n):
     got = ca.moe_gemm_gguf(torch.from_numpy(x).cuda(), qt, torch.from_numpy(tw).cuda(), torch.from_numpy(sorted_token_ids).cuda(),
                            torch.from_numpy(expert_ids).cuda(), topk, True)
     torch.cuda.synchronize()
-    want = oracle.moe_gemm_gguf(oracle.Q4K, x, blocks, (E, n, k), sorted_token_ids, expert_ids, tw, topk)
+    want = oracle.moe_gemm_gguf(wdt, x, blocks, (E, n, k), sorted_token_ids, expert_ids, tw, topk)
     got = got.cpu().numpy()
     for p in range(n_pairs):
         assert rel_l2(got[p], want[p]) <= 1e-5, p
