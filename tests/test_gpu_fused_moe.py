@@ -22,7 +22,8 @@ def L():
 
 
 @pytest.mark.parametrize("tokens,E,hidden,topk,norm", [(1, 128, 2048, 8, True), (7, 16, 256, 4, False), (300, 64, 512, 6, True), (3, 5, 64, 5, True),
-                                                            (9, 256, 128, 8, True), (5, 300, 128, 8, True), (2, 1000, 64, 60, False)])   # > 256 experts: the LDS kernel
+                                                            (9, 256, 128, 8, True), (5, 300, 128, 8, True), (2, 1000, 64, 60, False),   # > 256 experts: the LDS kernel
+                                                            (256, 128, 2048, 8, True), (130, 40, 256, 4, True), (517, 100, 768, 8, False)])  # token tiles in LDS
 def test_route_kernel(tokens, E, hidden, topk, norm):
     x, router = normal(1, (tokens, hidden), 1.0), normal(2, (E, hidden), 0.1)
     xd, rd = torch.from_numpy(x).cuda(), torch.from_numpy(router).cuda()
@@ -35,6 +36,12 @@ def test_route_kernel(tokens, E, hidden, topk, norm):
     want_ids, want_w = fm.route(x, router, topk, norm)
     assert np.array_equal(ids.cpu().numpy().astype(np.uint32), want_ids)
     assert np.allclose(w.cpu().numpy(), want_w, rtol=2e-5, atol=1e-8)
+    if tokens >= 128:
+        # the logits do not depend on how many tokens a call holds (the kernels differ, the order of a lane's additions does not)
+        few = torch.empty((5, E), dtype=torch.float32, device="cuda")
+        assert L().cq_nn_moe_route(xd.data_ptr() + 4 * 3 * hidden, rd.data_ptr(), ids.data_ptr(), w.data_ptr(), few.data_ptr(), 5, hidden, E, topk,
+                                   1 if norm else 0, None) == 0
+        assert np.array_equal(few.cpu().numpy(), lg.cpu().numpy()[3:8])
 
 
 def test_route_kernel_ties_take_the_lower_expert():
