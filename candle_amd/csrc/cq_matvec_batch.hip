@@ -647,7 +647,7 @@ int launch_qmb(const void *w, const uint8_t *op, void *dst, int dst_dtype, int64
 // CU count where the shape allows, and leaves at once when the expert has no pair.
 //
 // Short rows.  With fewer than eight super-blocks per row the waves do not all get a column: CW waves (a power of two) share a
-// block of 16 rows, wave w taking columns (w % CW) * CPW .. of row block w / CW of a tile of 8 / CW row blocks.
+// block of 16 rows, wave w taking columns (w / NRB) * CPW .. of row block w % NRB of a tile of NRB = 8 / CW row blocks.
 //
 // Operands.  Tile (expert e, set s) — pairs offsets[e] + 16 s .. of the expert-sorted pair list — lives at tile index
 // offsets[e] / 16 + e + s (unique and below n_pairs / 16 + experts without a scan over the experts), laid out like one column
@@ -741,7 +741,9 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, kg = lane >> 4;
-    const int rb = wv / CW, col0 = (wv % CW) * CPW;
+    // wave w: row block w % NRB, column group w / NRB.  Waves w and w + 4 share a SIMD, and where the last column group holds fewer
+    // columns (rows of 3 super-blocks: two columns and one) every SIMD then gets a heavy and a light wave instead of two of a kind.
+    const int rb = wv % NRB, col0 = (wv / NRB) * CPW;
     const int n = a.n, bpr = a.bpr;
     const int ncols = max(0, min(CPW, bpr - col0));
     const int RS = bpr * BB;
@@ -874,7 +876,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qme_q4k_kernel(const QmeArgs a) {
                 for (int g = 0; g < NRB; g++) {
                     float v = 0.0f;
 #pragma unroll
-                    for (int w2 = 0; w2 < CW; w2++) v += rd[((oset * QB_NW + g * CW + w2) * 64 + ol2) * 4 + orr];
+                    for (int w2 = 0; w2 < CW; w2++) v += rd[((oset * QB_NW + w2 * NRB + g) * 64 + ol2) * 4 + orr];
                     const int row = ((t0 + i - 1) * NRB + g) * 16 + (ol2 & 15);
                     if (row < n) out[orow * n + row] = v * oscale;
                 }
