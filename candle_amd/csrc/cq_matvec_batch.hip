@@ -1019,9 +1019,16 @@ int launch_qme(const QmeArgs &a, int64_t num_experts, int tensors, hipStream_t s
 constexpr int QB_MAX_BPR = 64;        // (and 64 x 16 records of 32 bytes are 4 pieces of 16 bytes per thread)
 static bool qb_weights(int w_dtype) { return w_dtype == CQ_Q4K || w_dtype == CQ_Q5K; }
 // the chunked-row kernel's split of a row: chunks of at most 16 super-blocks, all about the same size
-static int qb_long_cpp(int64_t bpr) { const int64_t chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW); return (int)((bpr + chunks - 1) / chunks); }
+// Full chunks of 16 super-blocks and a shorter last one where LDS holds three such tiles beside the records (every wave then has two
+// columns in all chunks but the last: with chunks of equal size, 14 for rows of 56 super-blocks, the eighth wave has none and its
+// SIMD half the work of the others); else chunks of about the same size.
+static int qb_long_cpp(int64_t bpr, int bb) {
+    const int64_t chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW);
+    if (qb_long_lds(bpr, 2 * QB_NW, bb) <= (size_t)QB_LDS_BYTES - 1024) return 2 * QB_NW;
+    return (int)((bpr + chunks - 1) / chunks);
+}
 static bool qb_row_fits(int w_dtype, int64_t bpr) {
-    return bpr >= 1 && bpr <= QB_MAX_BPR && (bpr <= 3 * QB_NW || qb_long_lds(bpr, qb_long_cpp(bpr), qb_bb(w_dtype == CQ_Q5K)) <= (size_t)QB_LDS_BYTES - 1024);
+    return bpr >= 1 && bpr <= QB_MAX_BPR && (bpr <= 3 * QB_NW || qb_long_lds(bpr, qb_long_cpp(bpr, qb_bb(w_dtype == CQ_Q5K)), qb_bb(w_dtype == CQ_Q5K)) <= (size_t)QB_LDS_BYTES - 1024);
 }
 bool cq_matvec_batch_takes(int w_dtype, const void *w, int64_t k, int64_t n, int64_t rows) {
     // (three rows over chunked rows: the register-blocked matvec is still ahead there, 15.1 against 16.8 us on [4096 x 14336])
@@ -1072,7 +1079,7 @@ static int qb_launch_w(int w_dtype, const void *w, const void *x, const float *u
         default: return CQ_ERR_DTYPE;
     }
     if (bpr > 3 * QB_NW) {
-        const int chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW), cpp = qb_long_cpp(bpr);
+        const int chunks = (bpr + 2 * QB_NW - 1) / (2 * QB_NW), cpp = qb_long_cpp(bpr, qb_bb(Q5));
         switch (chunks) {
             case 2: return launch_qmb_long<2, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
             case 3: return launch_qmb_long<3, Q5>(w, op, dst, dst_dtype, k, n, rows, stride_dst, cpp, s);
