@@ -147,8 +147,9 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
     const int bx = blockIdx.x, gx = gridDim.x;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, kg = lane >> 4;
-    const int col0 = wv * CPW;
-    const int ncols = max(0, min(CPW, bpr - col0));
+    // wave w takes columns w, w + 8, w + 16: waves w and w + 4 share a SIMD, and where the columns do not fill all waves evenly (12 or 20
+    // super-blocks per row) every SIMD gets the same number of them, which contiguous columns per wave do not give
+    const int ncols = max(0, min(CPW, (bpr - wv + QB_NW - 1) / QB_NW));
     const int RS = bpr * BB;                   // bytes of a row, in memory and in a tile
     const int block_bytes = 16 * RS;
     const int nkb = (block_bytes + 1023) >> 10;   // KBs of a tile
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
         float xv[NSP][4];
 #pragma unroll
         for (int ci = 0; ci < CPW; ci++) {
-            const int col = min(col0 + ci, bpr - 1);
+            const int col = min(wv + QB_NW * ci, bpr - 1);
 #pragma unroll
             for (int r = 0; r < FQ; r++) {
                 const f32x4 t = *(const f32x4 *)(x + ((int64_t)r * bpr + col) * 256 + lane * 4);
@@ -272,7 +273,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
     // (a wave's load of one operand is 512 contiguous bytes; the four lane groups read four records)
 #pragma unroll
     for (int ci = 0; ci < CPW; ci++) {
-        const int col = min(col0 + ci, bpr - 1);
+        const int col = min(wv + QB_NW * ci, bpr - 1);
         const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 16;         // lane = kg * 16 + c
 #pragma unroll
         for (int g = 0; g < 4; g++) {
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_kernel(const uint8_t *__re
 #pragma unroll
         for (int ci = 0; ci < CPW; ci++) {
             if (ci < ncols) {
-                const int o = c * RS + (col0 + ci) * BB;                  // weight row c of the block, this column's super-block
+                const int o = c * RS + (wv + QB_NW * ci) * BB;                  // weight row c of the block, this column's super-block
                 auto at = [&](int off) { return tile + off + (off >> 10) * 16; };      // byte `off` of the block in the padded tile
                 const u32x4 hdr = *(const u32x4 *)at(o);
                 i32x4 cl[4], ch[4];
