@@ -391,7 +391,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
     const int bx = blockIdx.x, gx = gridDim.x;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, kg = lane >> 4;
-    const int col0 = wv * CPW;                    // the wave's first column inside a chunk
+    // inside a chunk wave w takes columns w and w + 8 (a short last chunk is spread over all waves, and over the SIMDs evenly)
     const int RS = bpr * BB;                   // bytes of a row in memory
     const int block_bytes = 16 * RS;
     const int TILE = qb_tile_bytes(16 * cpp * BB);
@@ -444,7 +444,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
     auto load_operands = [&](int q) {
 #pragma unroll
         for (int ci = 0; ci < CPW; ci++) {
-            const int col = min(q * cpp + col0 + ci, bpr - 1);
+            const int col = min(q * cpp + wv + QB_NW * ci, bpr - 1);
             const uint8_t *colp = op + (int64_t)col * QB_OP_COL_BYTES + lane * 16;     // lane = kg * 16 + c
 #pragma unroll
             for (int g = 0; g < 4; g++) {
@@ -483,8 +483,8 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
             const int TRS = pc * BB;
 #pragma unroll
             for (int ci = 0; ci < CPW; ci++) {
-                if (col0 + ci < pc) {
-                    const int o = c * TRS + (col0 + ci) * BB;                 // weight row c of the block, this column's super-block
+                if (wv + QB_NW * ci < pc) {
+                    const int o = c * TRS + (wv + QB_NW * ci) * BB;                 // weight row c of the block, this column's super-block
                     auto at = [&](int off) { return tile + off + (off >> 10) * 16; };      // byte `off` of the tile in its padded form
                     const u32x4 hdr = *(const u32x4 *)at(o);
                     i32x4 cl[4], ch[4];
@@ -510,7 +510,7 @@ __global__ __launch_bounds__(QB_NW * 64) void qmb_q4k_long_kernel(const uint8_t 
                         sc[4 + j] = (int)((s.scB >> (8 * j)) & 0xff);
                     }
                     const float dw = h2f(hdr.x), dm = h2f(hdr.x >> 16);
-                    const uint8_t *rec = recs + ((q * cpp + col0 + ci) * 16 + 4 * kg) * QB_REC_BYTES;
+                    const uint8_t *rec = recs + ((q * cpp + wv + QB_NW * ci) * 16 + 4 * kg) * QB_REC_BYTES;
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         if (r < NR) {                                     // result r belongs to batch rows 4 r .. 4 r + 3
