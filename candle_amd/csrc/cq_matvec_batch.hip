@@ -1032,8 +1032,6 @@ static bool qb_row_fits(int w_dtype, int64_t bpr) {
     return bpr >= 1 && bpr <= QB_MAX_BPR && (bpr <= 3 * QB_NW || qb_long_lds(bpr, qb_long_cpp(bpr, qb_bb(w_dtype == CQ_Q5K)), qb_bb(w_dtype == CQ_Q5K)) <= (size_t)QB_LDS_BYTES - 1024);
 }
 bool cq_matvec_batch_takes(int w_dtype, const void *w, int64_t k, int64_t n, int64_t rows) {
-    // (three rows over chunked rows: the register-blocked matvec is still ahead there, 15.1 against 16.8 us on [4096 x 14336])
-    if (k / 256 > 3 * QB_NW && rows < 4) return false;
     return qb_weights(w_dtype) && rows >= 3 && rows <= 16 && k % 256 == 0 && qb_row_fits(w_dtype, k / 256) && n >= 1 && n <= 0x7ffffff0 / 16 &&
            n * (k / 256) * qb_bb(w_dtype == CQ_Q5K) < 0x7fffffffLL && ((uintptr_t)w & 15) == 0;
 }
