@@ -252,17 +252,18 @@ def test_rank3_input_and_shape_errors():
         qmm.forward(torch.zeros((256, 2), device="cuda").t())
 
 
-@pytest.mark.parametrize("rows,k", [(3, 512), (5, 8192), (2, 512), (12, 2048)])
+@pytest.mark.parametrize("wdt", [oracle.Q4K, oracle.Q5K], ids=lambda d: NAMES[d])
+@pytest.mark.parametrize("rows,k", [(3, 512), (5, 8192), (2, 512), (12, 2048), (16, 3072), (9, 5120)])   # 3072, 5120: columns that do not fill the waves evenly
 @pytest.mark.parametrize("tdt", [torch.float16, torch.bfloat16])
-def test_half_activations_keep_dtype(tdt, rows, k):
+def test_half_activations_keep_dtype(tdt, rows, k, wdt):
     # CPU f16 path: widen, quantize, dot, round the result to f16 (k_quants.rs:2652-2686); the GPU keeps the input dtype
     # (two rows: the streaming kernel; 3 .. 16 rows: the batched matrix-core kernel, rows of 8192 elements in column chunks)
-    blocks, qmm = make_weight(oracle.Q4K, 40, k, seed=75)
+    blocks, qmm = make_weight(wdt, 40, k, seed=75)
     x = torch.from_numpy(normal(76, (rows, k), 1.0)).to(tdt)
     y = qmm.forward(x.cuda())
     torch.cuda.synchronize()
     assert y.dtype == tdt
-    want = torch.from_numpy(oracle.matmul(oracle.Q4K, x.float().numpy(), blocks, 40)).to(tdt)
+    want = torch.from_numpy(oracle.matmul(wdt, x.float().numpy(), blocks, 40)).to(tdt)
     # identical up to one rounding step of the output type
     assert rel_l2(y.float().cpu().numpy(), want.float().numpy()) <= (2e-3 if tdt == torch.float16 else 1e-2)
 
