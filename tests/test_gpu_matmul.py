@@ -106,7 +106,7 @@ def test_q4k_batched_rows_vs_oracle(wdt, k, n, batch):
 
 
 @pytest.mark.parametrize("wdt", [oracle.Q4K, oracle.Q5K], ids=lambda d: NAMES[d])
-@pytest.mark.parametrize("k", [256, 2048, 4096, 6144])
+@pytest.mark.parametrize("k", [256, 2048, 3072, 4096, 5120, 6144])     # 3072, 5120: some waves hold one column fewer than others
 @pytest.mark.parametrize("rows", [3, 4, 5, 6, 8])
 def test_q4k_batched_rows_quantized_inside_the_kernel(wdt, k, rows):
     """Few f32 rows are quantized by the waves of the matvec kernel itself (up to 16 spans per wave), more rows by a kernel
