@@ -680,7 +680,7 @@ def other_configurations(L, torch, args):
     sweep = []
     for (n, k) in ((14336, 4096), (4096, 14336)):
         for b in (1, 2, 4, 8, 16) + ((32, 64) if k <= 4096 else ()):
-            rot = Rotation(L, torch, "q4k", n, k, b, 600)
+            rot = Rotation(L, torch, "q4k", n, k, b, args.pool_mb)          # the headline's pool: 39 launches per graph replay
             g = rot.capture(rot.step)
             us = rot.event_us(g, 1000, 100)
             st = rot.replay_stats(g, 1000, 100)
